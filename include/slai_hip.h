@@ -1,0 +1,239 @@
+/*
+ * slai_hip.h -- C ABI of libslai_hip.so, the MI355X (gfx950) implementation of slai's
+ * per-token decode path.
+ *
+ * Every entry point names the reference interface it stands in for
+ * (paths relative to the dimforge/slai tree).  All functions return 0 on success or a
+ * negative SLAI_E_* code; slai_last_error() gives the message (the reference's
+ * `Result<(), B::Error>`).  Shape violations return SLAI_E_SHAPE instead of panicking.
+ *
+ * A context owns one HIP stream; every launch goes to it.  A context is not thread
+ * safe (the reference serialises forwards with three RwLock write guards,
+ * crates/slai-chat/src/chat_llama2.rs:170-172); distinct contexts are independent.
+ */
+#ifndef SLAI_HIP_H
+#define SLAI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SLAI_OK 0
+#define SLAI_E_HIP (-1)       /* a HIP runtime call failed */
+#define SLAI_E_SHAPE (-2)     /* dimension / stride / alignment mismatch */
+#define SLAI_E_TYPE (-3)      /* unsupported ggml type tag */
+#define SLAI_E_ARG (-4)       /* null or out-of-range argument */
+#define SLAI_E_PARSE (-5)     /* malformed GGUF */
+#define SLAI_E_MISSING (-6)   /* missing tensor / metadata key */
+#define SLAI_E_STATE (-7)     /* call not valid in the current state */
+
+typedef struct slai_ctx slai_ctx;
+typedef struct slai_buffer slai_buffer;
+typedef struct slai_qmat slai_qmat;
+typedef struct slai_graph slai_graph;
+typedef struct slai_gguf slai_gguf;
+typedef struct slai_llama2 slai_llama2;
+typedef struct slai_gpt2 slai_gpt2;
+
+/* stensor `GpuTensorView` = buffer slice + `ViewShape{size, strides, offset}` (used
+ * throughout crates/slai/src/context.rs).  Offsets and strides are in ELEMENTS of
+ * the buffer's scalar type; element (i,j,k,l) lives at
+ * offset + i*stride[0] + j*stride[1] + k*stride[2] + l*stride[3].
+ * size = [nrows, ncols, nmats, ncubes]. */
+typedef struct {
+    slai_buffer *buf;
+    uint64_t offset;
+    uint32_t size[4];
+    uint32_t stride[4];
+} slai_view;
+
+/* crates/slai/src/ops/rms_norm.rs:15-21 */
+typedef struct { float nudge_factor; uint32_t _padding[3]; } slai_rms_norm_config;
+/* crates/slai/src/ops/rope.rs:24-33 */
+typedef struct { uint32_t head_size, kv_dim, pos; float base_freq; } slai_rope_config;
+/* crates/slai/src/ops/batched_multiquery_attention.rs:17-29 */
+typedef struct { uint32_t seq_len, kv_dim, kv_mul, n_heads, head_size, pos; uint32_t _padding[2]; } slai_attn_params;
+
+/* wgpu BufferUsages bits accepted by the constructors (crates/slai/src/models/llama2/transformer.rs:49-137);
+ * only MAP_READ changes behaviour (pinned host staging for slai_read_buffer). */
+#define SLAI_USAGE_MAP_READ 0x1u
+#define SLAI_USAGE_COPY_SRC 0x4u
+#define SLAI_USAGE_COPY_DST 0x8u
+#define SLAI_USAGE_UNIFORM 0x40u
+#define SLAI_USAGE_STORAGE 0x80u
+
+/* Buffer scalar types. */
+#define SLAI_DT_F32 0
+#define SLAI_DT_F16 1
+#define SLAI_DT_U8 2
+#define SLAI_DT_I32 3
+
+/* crates/slai/src/ops/rope.rs:8-14 `RoPEVariant` */
+#define SLAI_ROPE_ORIGINAL 0
+#define SLAI_ROPE_NEOX 1
+/* stensor `MatrixMode` N / T (crates/slai/src/context.rs:298-317) */
+#define SLAI_MODE_N 0
+#define SLAI_MODE_T 1
+
+/* ---- context / backend -------------------------------------------------
+ * slang_hal `Backend` + `LlmOps::new` (crates/slai/src/context.rs:48-66): creating the
+ * context loads the one code object that holds every kernel. */
+int slai_ctx_create(int device, slai_ctx **out);
+void slai_ctx_destroy(slai_ctx *ctx);
+const char *slai_last_error(slai_ctx *ctx);
+/* The HIP stream every launch of this context goes to (as a `hipStream_t`). */
+void *slai_ctx_stream(slai_ctx *ctx);
+
+/* `LlmContext::begin_submission` / `submit` (crates/slai/src/context.rs:79-95) and
+ * `Backend::synchronize` (crates/slai-chat/src/chat_llama2.rs:219). */
+int slai_begin_submission(slai_ctx *ctx);
+int slai_submit(slai_ctx *ctx);
+int slai_synchronize(slai_ctx *ctx);
+
+/* ---- buffers ------------------------------------------------------------
+ * `GpuTensor::{vector,matrix,scalar}(_uninit)` allocations
+ * (crates/slai/src/models/llama2/transformer.rs:54-137); buffers are zero-filled. */
+int slai_buffer_create(slai_ctx *ctx, size_t bytes, int dtype, uint32_t usage, slai_buffer **out);
+void slai_buffer_destroy(slai_ctx *ctx, slai_buffer *buf);
+size_t slai_buffer_size(const slai_buffer *buf);
+void *slai_buffer_device_ptr(const slai_buffer *buf);
+/* `Backend::write_buffer` (crates/slai-chat/src/chat_llama2.rs:180-185); byte offsets. */
+int slai_write_buffer(slai_ctx *ctx, slai_buffer *buf, size_t offset, const void *src, size_t bytes);
+/* `Backend::read_buffer` (crates/slai-chat/src/chat_llama2.rs:225-227); synchronises. */
+int slai_read_buffer(slai_ctx *ctx, const slai_buffer *buf, size_t offset, void *dst, size_t bytes);
+/* `GpuTensor::copy_from_view` (crates/slai-chat/src/chat_llama2.rs:186-188,207). */
+int slai_copy_buffer(slai_ctx *ctx, slai_buffer *dst, size_t dst_offset, const slai_buffer *src,
+                     size_t src_offset, size_t bytes);
+
+/* ---- quantized matrices ---------------------------------------------------
+ * `GpuQuantMatrix` (crates/slai/src/quantized_matrix.rs:11-22) built by
+ * `GgufTensorData::to_gpu_matrix` (crates/slai/src/gguf.rs:133-194).  `packed` holds
+ * nrows rows of verbatim GGUF blocks (ggml type tag as in gguf.rs:75-107:
+ * 0 F32, 1 F16, 2 Q4_0, 8 Q8_0, 12 Q4_K, 13 Q5_K, 14 Q6_K).  Any block count is
+ * accepted (no pairing constraint), F16 stays 16-bit. */
+int slai_qmat_create(slai_ctx *ctx, uint32_t ggml_type, uint32_t nrows, uint32_t ncols, const void *packed,
+                     slai_qmat **out);
+void slai_qmat_destroy(slai_ctx *ctx, slai_qmat *m);
+/* `GpuQuantMatrix::shape` (quantized_matrix.rs:72-86): [nrows, ncols] in elements, and the type tag. */
+int slai_qmat_shape(const slai_qmat *m, uint32_t *nrows, uint32_t *ncols, uint32_t *ggml_type);
+/* Bytes the matrix occupies in device memory. */
+size_t slai_qmat_device_bytes(const slai_qmat *m);
+/* `GgufTensorData::dequantize` (crates/slai/src/gguf.rs:116-131, block math
+ * crates/slai/src/quantization.rs) evaluated on the device from the device layout:
+ * rows [row0, row0+nrows) to a dense row-major f32 view.  Bit-exact. */
+int slai_qmat_dequantize(slai_ctx *ctx, const slai_qmat *m, uint32_t row0, uint32_t nrows, slai_view out);
+
+/* ---- ops: the `LlmContext` facade (crates/slai/src/context.rs) -------------
+ * Out-parameter first, then inputs, as in the reference. */
+/* context.rs:230-246 -> ops/rms_norm.rs:35-66, shader rms_norm.slang:48-67 */
+int slai_rms_norm_assign(slai_ctx *ctx, const slai_buffer *config, slai_view out, slai_view value, slai_view weight);
+/* context.rs:205-217 -> ops/layernorm.rs:60-98 (rows of a vector = one group), no affine;
+ * eps is explicit (the shader hard-codes 1e-6, the CPU path 1e-5: layernorm.slang:6, ops/layernorm.rs:105). */
+int slai_layernorm_assign(slai_ctx *ctx, slai_view out, slai_view value, float eps);
+/* context.rs:355-369 -> ops/gemv_quant.rs:206-312: out = m * v */
+int slai_matmul_quant_assign(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view v);
+/* context.rs:298-317 (stensor f32 Gemv): out = op(a) * op(b), batched over dims 2,3 */
+int slai_matmul_assign(slai_ctx *ctx, slai_view out, slai_view a, slai_view b, int a_mode, int b_mode);
+/* context.rs:428-441 / 456-469 / 660-672 (stensor OpAssign Add / Mul / Copy) */
+int slai_add_assign(slai_ctx *ctx, slai_view in_out_a, slai_view b);
+int slai_mul_assign(slai_ctx *ctx, slai_view in_out_a, slai_view b);
+int slai_copy(slai_ctx *ctx, slai_view in, slai_view out);
+/* context.rs:471-487 -> ops/rope.rs:45-85, rope.slang:27-84 */
+int slai_rope(slai_ctx *ctx, int variant, const slai_buffer *config, slai_view in_out_q, slai_view in_out_k);
+/* context.rs:489-501 -> ops/silu.rs:24-48, silu.slang:11-27 */
+int slai_silu(slai_ctx *ctx, slai_view in_out_h1, slai_view in_h2);
+/* context.rs:565-570 -> ops/unary.rs:159-223 (UnaryOp::Gelu), unary.slang:67-74 */
+int slai_gelu_inplace(slai_ctx *ctx, slai_view x);
+/* context.rs:760-785, batched_multiquery_attention.slang:18-32 */
+int slai_attn_mask(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_buffer *attn);
+/* context.rs:787-797 -> ops/softmax.rs:22-40, softmax.slang:26-96 */
+int slai_softmax_cols(slai_ctx *ctx, slai_view in_out_mat);
+/* `BatchedMultiqueryAttention::launch` (ops/batched_multiquery_attention.rs:32-100): one fused
+ * kernel pair (QK^T, softmax, .V with split-K) instead of the reference's four launches.
+ * Caches are [kv_dim x seq_len] column-major, f32 or f16 by the buffer's dtype.  `att` is
+ * accepted for signature parity and not written. */
+int slai_attention(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q,
+                   slai_view key_cache, slai_view value_cache, slai_view att, slai_view xb);
+/* `Sampler::sample_argmax` (crates/slai/src/models/sampler.rs:55-57; first strict maximum),
+ * on the device; out_index is a 1-element I32 buffer. */
+int slai_argmax(slai_ctx *ctx, slai_view logits, slai_buffer *out_index);
+
+/* ---- HIP graph capture of a submission (no reference counterpart: the reference
+ * re-encodes ~550 dispatches per token, crates/slai-chat/src/chat_llama2.rs:179-230) */
+int slai_graph_begin_capture(slai_ctx *ctx);
+int slai_graph_end_capture(slai_ctx *ctx, slai_graph **out);
+int slai_graph_launch(slai_ctx *ctx, slai_graph *g);
+void slai_graph_destroy(slai_ctx *ctx, slai_graph *g);
+
+/* ---- GGUF (crates/slai/src/gguf.rs) -----------------------------------------
+ * `Gguf::from_bytes` (gguf.rs:504-524).  The bytes must outlive the handle. */
+int slai_gguf_parse(const void *bytes, size_t len, slai_gguf **out, char *err, size_t err_len);
+void slai_gguf_free(slai_gguf *g);
+uint32_t slai_gguf_version(const slai_gguf *g);
+uint64_t slai_gguf_tensor_count(const slai_gguf *g);
+uint64_t slai_gguf_metadata_count(const slai_gguf *g);
+uint64_t slai_gguf_data_start(const slai_gguf *g);
+/* tensor i: name, dims [nrows, ncols, nmats, ncubes] (gguf.rs:579-581), ggml type, absolute offset */
+int slai_gguf_tensor_info(const slai_gguf *g, uint64_t i, const char **name, uint64_t dims[4], uint32_t *ggml_type,
+                          uint64_t *offset);
+int slai_gguf_find_tensor(const slai_gguf *g, const char *name, uint64_t *index);
+/* metadata lookups (gguf.rs:283-331 `unwrap_u32`, `as_f32`, `as_string`, `unwrap_array_len`) */
+int slai_gguf_meta_u32(const slai_gguf *g, const char *key, uint32_t *out);
+int slai_gguf_meta_f32(const slai_gguf *g, const char *key, float *out);
+int slai_gguf_meta_str(const slai_gguf *g, const char *key, const char **out);
+int slai_gguf_meta_array_len(const slai_gguf *g, const char *key, uint64_t *out);
+/* `GgufTensor::to_gpu_matrix` (gguf.rs:357-366) */
+int slai_gguf_tensor_to_qmat(slai_ctx *ctx, const slai_gguf *g, const char *name, slai_qmat **out);
+
+/* ---- Llama-2 / Qwen2 model assembly ------------------------------------------
+ * `ChatLlama2::from_gguf_with_model_type` (crates/slai-chat/src/chat_llama2.rs:39-62):
+ * `Llama2Config::from_gguf_with_model_type` (models/llama2/cpu.rs:79-109),
+ * `Llama2Weights::from_gguf` (models/llama2/transformer.rs:202-297),
+ * `Llama2State::new` (transformer.rs:47-140). */
+#define SLAI_MODEL_LLAMA 0
+#define SLAI_MODEL_QWEN2 1
+#define SLAI_KV_F32 0   /* the reference's cache type (transformer.rs:87-106) */
+#define SLAI_KV_F16 1
+typedef struct {
+    uint32_t dim, hidden_dim, n_layers, n_q_heads, n_kv_heads, vocab_size, seq_len;
+    float rope_base_freq, rms_norm_eps;
+} slai_llama2_config;   /* models/llama2/cpu.rs:46-67 */
+
+int slai_llama2_from_gguf(slai_ctx *ctx, const slai_gguf *g, int model_type, int kv_dtype, slai_llama2 **out);
+void slai_llama2_destroy(slai_llama2 *m);
+int slai_llama2_get_config(const slai_llama2 *m, slai_llama2_config *out);
+/* Bytes of packed weights resident in device memory (roofline denominator). */
+size_t slai_llama2_weight_bytes(const slai_llama2 *m);
+/* `ChatLlama2::forward_logits` (chat_llama2.rs:163-240): one position through
+ * `Llama2::launch` (transformer.rs:316-381); logits (vocab floats) copied to `logits_out` when
+ * not NULL.  fused = 0 issues the reference's op sequence one kernel per op; fused = 1 uses the
+ * fused kernels (norm-in-GEMV, gate/up+SiLU, residual epilogues, RoPE-in-attention). */
+int slai_llama2_forward_logits(slai_llama2 *m, uint32_t pos, uint32_t token, int fused, float *logits_out);
+/* The per-token loop of `ChatLlama2::forward` (chat_llama2.rs:105-158) with greedy sampling and
+ * the forced-token rule (crates/slai-chat/src/sampler.rs:100-105): runs positions
+ * start_pos .. start_pos+n_steps-1 entirely on the device (one captured graph replayed per
+ * token, argmax and token feedback on the device); out_tokens[i] = token chosen after step i.
+ * elapsed_ms (optional) = stream time of the n_steps replays measured with HIP events. */
+int slai_llama2_generate(slai_llama2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
+                         uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms);
+/* Device access for set-up and inspection: layer l's caches ([kv_dim x seq_len]) and the state vectors. */
+int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache);
+int slai_llama2_logits_buffer(slai_llama2 *m, slai_buffer **logits);
+
+/* ---- GPT-2 model assembly (crates/slai/src/models/gpt2/cpu.rs:19-48,113-217,224-383) */
+typedef struct { uint32_t n_vocab, n_seq, n_embd, n_head, n_layer, ff_len, attn_b; } slai_gpt2_params;
+int slai_gpt2_from_gguf(slai_ctx *ctx, const slai_gguf *g, int kv_dtype, slai_gpt2 **out);
+void slai_gpt2_destroy(slai_gpt2 *m);
+int slai_gpt2_get_params(const slai_gpt2 *m, slai_gpt2_params *out);
+size_t slai_gpt2_weight_bytes(const slai_gpt2 *m);
+int slai_gpt2_forward_logits(slai_gpt2 *m, uint32_t pos, uint32_t token, float *logits_out);
+int slai_gpt2_generate(slai_gpt2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
+                       uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SLAI_HIP_H */

@@ -54,6 +54,8 @@ def build_hip(jobs=8):
         flags = list(HIP_FLAGS)
         if s.endswith(".cpp"):
             flags = ["-x", "hip"] + flags
+        if s.endswith("_exact.hip"):
+            flags = flags + ["-ffp-contract=off"]   # bit-exact dequantisation: no FMA contraction
         _run([HIPCC] + flags + ["-c", s, "-o", o])
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:

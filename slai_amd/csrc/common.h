@@ -1,0 +1,143 @@
+// Internal definitions shared by the runtime and the kernel launchers of libslai_hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string>
+#include <vector>
+
+#include "slai_hip.h"
+
+#define SLAI_EXPORT extern "C" __attribute__((visibility("default")))
+
+struct slai_buffer {
+    void *dptr = nullptr;
+    size_t bytes = 0;
+    int dtype = SLAI_DT_F32;
+    uint32_t usage = 0;
+    void *host_staging = nullptr;  // pinned, when created with SLAI_USAGE_MAP_READ
+};
+
+struct slai_qmat {
+    int type = 0;
+    uint32_t nrows = 0, ncols = 0, nb = 0;  // nb = blocks per row
+    size_t row_stride = 0;                  // bytes between rows in device memory
+    uint8_t *dptr = nullptr;
+    size_t bytes = 0;
+};
+
+struct slai_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+struct slai_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::string err;
+    bool capturing = false;
+    // attention split-K partials (grown on demand, never inside a capture)
+    float *attn_scratch = nullptr;
+    size_t attn_scratch_floats = 0;
+    // tuning knobs (environment overridable, see runtime.cpp)
+    int gemv_rows_per_wg = 8;
+    int gemv_max_threads = 1024;
+    int attn_splits = 0;  // 0 = automatic
+};
+
+namespace slai {
+
+int set_error(slai_ctx *ctx, int code, const std::string &msg);
+int hip_fail(slai_ctx *ctx, hipError_t e, const char *what);
+
+#define SLAI_HIP_TRY(ctx, call)                                         \
+    do {                                                                \
+        hipError_t e__ = (call);                                        \
+        if (e__ != hipSuccess) return ::slai::hip_fail(ctx, e__, #call); \
+    } while (0)
+
+// ---- GEMV -------------------------------------------------------------------
+enum : uint32_t {
+    GEMV_BIAS = 1u,      // val += bias[row]
+    GEMV_ACCUM = 2u,     // out[row] += val
+    GEMV_SILU_GATE = 4u, // dual: val = up * gate/(1+exp(-gate))   (W = gate, W2 = up)
+    GEMV_GELU = 8u,      // val = gelu(val)
+};
+enum : int { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_LAYERNORM = 2 };
+
+struct GemvSeg {
+    const uint8_t *W = nullptr;
+    const uint8_t *W2 = nullptr;
+    size_t row_stride = 0;
+    uint32_t nrows = 0;
+    uint32_t nblocks = 0;  // filled by the launcher
+    float *out = nullptr;
+    const float *bias = nullptr;
+    uint32_t flags = 0;
+};
+struct GemvParams {
+    GemvSeg seg[3];
+    int nseg = 1;
+    uint32_t ncols = 0, nb = 0;
+    const float *x = nullptr;
+    int prologue = PRO_NONE;
+    const float *norm_w = nullptr, *norm_b = nullptr;
+    float eps = 0.0f;
+    const float *eps_ptr = nullptr;  // when set, eps is read from device memory
+    uint32_t rows_per_wg = 8;
+};
+// All segments share the ggml type `type`, the input x and the prologue.
+hipError_t launch_gemv(slai_ctx *ctx, int type, GemvParams p);
+bool gemv_supports(int type, uint32_t ncols);
+
+// ---- dequantisation / repack ---------------------------------------------------
+hipError_t launch_repack(hipStream_t s, int type, const uint8_t *src, uint8_t *dst, uint32_t nrows, uint32_t ncols);
+// rows [row0,row0+nrows) of a device-layout matrix to f32, out[(r)*out_stride + c]
+hipError_t launch_dequant_rows(hipStream_t s, int type, const uint8_t *dev, size_t row_stride, uint32_t nb,
+                               uint32_t row0, uint32_t nrows, uint32_t ncols, float *out, size_t out_stride);
+// out[c] = deq(A[row_a][c]) (+ deq(B[row_b][c]) when B != null); row indices read from device memory
+hipError_t launch_embed(hipStream_t s, int type_a, const uint8_t *a, size_t stride_a, uint32_t nb_a, const int *row_a,
+                        int type_b, const uint8_t *b, size_t stride_b, uint32_t nb_b, const int *row_b,
+                        uint32_t ncols, float *out);
+
+// ---- element-wise / normalisation ops -------------------------------------------------
+struct VecView { float *p; uint32_t n; uint32_t stride; };  // element i at p[i*stride]
+hipError_t launch_rms_norm(hipStream_t s, VecView out, VecView v, VecView w, const float *eps_ptr, float eps);
+hipError_t launch_layernorm(hipStream_t s, VecView out, VecView v, float eps);
+hipError_t launch_binop(hipStream_t s, int op /*0 add,1 mul,2 copy(a<-b)*/, VecView a, VecView b);
+hipError_t launch_silu(hipStream_t s, VecView a, VecView b);
+hipError_t launch_gelu(hipStream_t s, VecView a);
+hipError_t launch_rope(hipStream_t s, int variant, const slai_rope_config *cfg_dev, VecView q, VecView k);
+hipError_t launch_attn_mask(hipStream_t s, const slai_attn_params *params_dev, float *attn, uint32_t nthreads);
+struct View4 { float *p; uint32_t size[4]; uint32_t stride[4]; };
+hipError_t launch_softmax_cols(hipStream_t s, View4 m);
+hipError_t launch_matmul_f32(hipStream_t s, View4 out, View4 a, View4 b, int a_mode, int b_mode);
+// first strict maximum over n floats -> *out_index.  When `decode` is set the kernel also applies the
+// forced-token rule and advances the device-side decode state (see DecodeState).
+struct DecodeState {      // lives in device memory; the whole greedy loop runs without the host
+    int pos;              // position of the token being processed
+    int token;            // token fed at `pos`
+    int n_prompt;         // prompt length (forced tokens while pos < n_prompt-1)
+    int step;             // index into out_tokens
+};
+hipError_t launch_argmax(hipStream_t s, const float *v, uint32_t n, int *out_index, DecodeState *decode,
+                         const int *prompt, int *out_tokens);
+
+// ---- attention ---------------------------------------------------------------------
+struct AttnLaunch {
+    const float *q;          // [n_heads*head_size] (pre-RoPE when rope != -1)
+    void *kcache, *vcache;   // [seq_len][kv_dim] (position major), f32 or f16
+    int kv_f16;
+    uint32_t n_heads, kv_mul, head_size, kv_dim, seq_len;
+    const uint32_t *pos_ptr; // device; the attended range is [0, *pos_ptr]
+    // fused RoPE + cache write of the current position (model path): the fresh k/v columns
+    const float *knew, *vnew;  // null: caches already hold position pos and q is already rotated
+    const float *qbias, *kbias, *vbias;  // optional (Qwen2), added before RoPE
+    int rope_variant; float rope_base;
+    float *out;              // [n_heads*head_size]
+    float *scratch;          // n_heads*n_splits*(head_size+2) floats when n_splits > 1
+    uint32_t n_splits;
+};
+hipError_t launch_attention(hipStream_t s, const AttnLaunch &a);
+size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n_splits);
+
+}  // namespace slai

@@ -1,0 +1,692 @@
+// Llama-2 / Qwen2 and GPT-2 model assembly on top of the op facade.
+//
+// Mirrors crates/slai/src/models/llama2/transformer.rs (`Llama2State` :16-140, `Llama2Weights` :179-297,
+// `Llama2::launch` :316-381), models/llama2/cpu.rs (`Llama2Config` :46-143), the per-token driver
+// crates/slai-chat/src/chat_llama2.rs:64-240 and, for GPT-2, models/gpt2/cpu.rs:19-48,113-217,224-383.
+#include "common.h"
+#include "host_gguf.h"
+#include "llm_context.h"
+#include "quant_formats.h"
+
+#include <cstring>
+#include <memory>
+
+namespace slai {
+uint32_t pick_attn_splits(const slai_ctx *ctx, uint32_t n_heads, uint32_t seq_len);
+int ensure_attn_scratch(slai_ctx *ctx, size_t floats);
+hipError_t launch_store_kv(hipStream_t s, const float *src, void *dst, uint32_t n, int f16);
+}  // namespace slai
+
+using namespace slai;
+
+#define TRY(call) do { int rc__ = (call); if (rc__) return rc__; } while (0)
+
+namespace {
+const uint32_t STORAGE = SLAI_USAGE_STORAGE, UNIFORM = SLAI_USAGE_UNIFORM, COPY_DST = SLAI_USAGE_COPY_DST,
+               COPY_SRC = SLAI_USAGE_COPY_SRC, MAP_READ = SLAI_USAGE_MAP_READ;
+
+// `gguf.tensors[name].data().as_f32().unwrap()` + `GpuTensor::vector` (transformer.rs:250-263)
+int f32_vector_from_gguf(slai_ctx *ctx, const Gguf &g, const std::string &name, bool required, GpuTensor *out) {
+    const GgufTensorInfo *t = g.find(name);
+    if (!t) return required ? set_error(ctx, SLAI_E_MISSING, "missing tensor '" + name + "'") : SLAI_OK;
+    if (t->type != 0) return set_error(ctx, SLAI_E_TYPE, "tensor '" + name + "' must be F32");
+    uint64_t n = t->dims[0] * t->dims[1] * t->dims[2] * t->dims[3];
+    return GpuTensor::vector_from(ctx, reinterpret_cast<const float *>(g.bytes + t->offset), (uint32_t)n, STORAGE, out);
+}
+int qmat_from_gguf(slai_ctx *ctx, const slai_gguf *g, const std::string &name, slai_qmat **out) {
+    return slai_gguf_tensor_to_qmat(ctx, g, name.c_str(), out);
+}
+int meta_u32(slai_ctx *ctx, const Gguf &g, const std::string &key, uint32_t *out) {
+    const GgufMetaValue *v = g.meta(key);
+    if (!v) return set_error(ctx, SLAI_E_MISSING, "missing metadata key '" + key + "'");
+    if (v->type != 4) return set_error(ctx, SLAI_E_TYPE, "unwrap: unexpected GGUF attribute type for '" + key + "'");
+    *out = (uint32_t)v->u;
+    return SLAI_OK;
+}
+
+struct DeviceLoop {           // device-resident state of the greedy loop
+    slai_buffer *state = nullptr;       // DecodeState
+    slai_buffer *prompt = nullptr;      // int32[capacity]
+    slai_buffer *out_tokens = nullptr;  // int32[capacity]
+    uint32_t capacity = 0;
+    slai_graph *graph = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+};
+int loop_init(slai_ctx *ctx, DeviceLoop &L, uint32_t capacity) {
+    L.capacity = capacity;
+    TRY(slai_buffer_create(ctx, sizeof(DecodeState), SLAI_DT_I32, STORAGE | COPY_DST, &L.state));
+    TRY(slai_buffer_create(ctx, (size_t)capacity * 4, SLAI_DT_I32, STORAGE | COPY_DST, &L.prompt));
+    TRY(slai_buffer_create(ctx, (size_t)capacity * 4, SLAI_DT_I32, STORAGE | COPY_SRC, &L.out_tokens));
+    SLAI_HIP_TRY(ctx, hipEventCreate(&L.ev0));
+    SLAI_HIP_TRY(ctx, hipEventCreate(&L.ev1));
+    return SLAI_OK;
+}
+void loop_destroy(slai_ctx *ctx, DeviceLoop &L) {
+    if (L.graph) slai_graph_destroy(ctx, L.graph);
+    if (L.state) slai_buffer_destroy(ctx, L.state);
+    if (L.prompt) slai_buffer_destroy(ctx, L.prompt);
+    if (L.out_tokens) slai_buffer_destroy(ctx, L.out_tokens);
+    if (L.ev0) hipEventDestroy(L.ev0);
+    if (L.ev1) hipEventDestroy(L.ev1);
+}
+}  // namespace
+
+// =================================================================================================
+// Llama-2
+// =================================================================================================
+struct Llama2LayerWeights {          // transformer.rs:179-192
+    GpuTensor attn_norm;
+    slai_qmat *attn_k = nullptr, *attn_q = nullptr, *attn_v = nullptr;
+    GpuTensor attn_k_bias, attn_q_bias, attn_v_bias;   // optional
+    slai_qmat *ffn_down = nullptr, *ffn_gate = nullptr;
+    GpuTensor ffn_norm;
+    slai_qmat *ffn_up = nullptr, *attn_output = nullptr;
+};
+struct Llama2Weights {               // transformer.rs:194-199
+    std::vector<Llama2LayerWeights> layers;
+    slai_qmat *token_embd = nullptr;   // kept packed; one row is dequantised on the device per token
+    slai_qmat *output = nullptr;       // aliases token_embd when the file has no output.weight
+    GpuTensor output_norm;
+};
+struct Llama2State {                 // transformer.rs:16-44
+    GpuTensor x, xb, xb2, hb, hb2, q, att, logits;
+    GpuTensor kcol, vcol;            // fresh K/V of the current position (fused path, and staging for f16 caches)
+    std::vector<GpuTensor> key_cache, value_cache;
+    slai_buffer *rope_config = nullptr, *rms_norm_config = nullptr, *attn_params = nullptr;
+};
+
+struct slai_llama2 {
+    slai_ctx *ctx = nullptr;
+    int model_type = SLAI_MODEL_LLAMA;
+    int kv_dtype = SLAI_KV_F32;
+    slai_llama2_config config{};
+    Llama2Weights weights;
+    Llama2State state;
+    DeviceLoop loop;
+    size_t weight_bytes = 0;
+    uint32_t attn_splits = 1;
+
+    uint32_t kv_dim() const { return config.dim * config.n_kv_heads / config.n_q_heads; }
+    uint32_t head_size() const { return config.dim / config.n_q_heads; }
+    int rope_variant() const { return model_type == SLAI_MODEL_QWEN2 ? SLAI_ROPE_NEOX : SLAI_ROPE_ORIGINAL; }  // llama2/mod.rs:27-32
+
+    int load(const slai_gguf *g);
+    int launch(LlmContext &ctxt, const slai_attn_params &attn_params, uint32_t pos);   // transformer.rs:316-381
+    int enqueue_fused(bool with_sampler);
+    int gemv_fused(int type, GemvParams &p);
+};
+
+// models/llama2/cpu.rs:79-109
+static int llama2_config_from_gguf(slai_ctx *ctx, const Gguf &g, int model_type, slai_llama2_config *c) {
+    const std::string m = model_type == SLAI_MODEL_QWEN2 ? "qwen2" : "llama";   // llama2/mod.rs:19-25
+    TRY(meta_u32(ctx, g, m + ".embedding_length", &c->dim));
+    TRY(meta_u32(ctx, g, m + ".feed_forward_length", &c->hidden_dim));
+    TRY(meta_u32(ctx, g, m + ".block_count", &c->n_layers));
+    TRY(meta_u32(ctx, g, m + ".attention.head_count", &c->n_q_heads));
+    TRY(meta_u32(ctx, g, m + ".attention.head_count_kv", &c->n_kv_heads));
+    TRY(meta_u32(ctx, g, m + ".context_length", &c->seq_len));
+    const GgufMetaValue *tok = g.meta("tokenizer.ggml.tokens");
+    if (!tok) return set_error(ctx, SLAI_E_MISSING, "missing metadata key 'tokenizer.ggml.tokens'");
+    if (tok->type != 9) return set_error(ctx, SLAI_E_TYPE, "unwrap: unexpected GGUF attribute type for 'tokenizer.ggml.tokens'");
+    c->vocab_size = (uint32_t)tok->arr_len;
+    const GgufMetaValue *fb = g.meta(m + ".rope.freq_base");
+    if (fb && fb->type != 6) return set_error(ctx, SLAI_E_TYPE, "unwrap: unexpected GGUF attribute type for rope.freq_base");
+    c->rope_base_freq = fb ? (float)fb->f : 10000.0f;
+    const GgufMetaValue *ep = g.meta(m + ".attention.layer_norm_rms_epsilon");
+    if (ep && ep->type != 6) return set_error(ctx, SLAI_E_TYPE, "unwrap: unexpected GGUF attribute type for layer_norm_rms_epsilon");
+    c->rms_norm_eps = ep ? (float)ep->f : 1.0e-6f;
+    if (!c->dim || !c->n_q_heads || !c->n_kv_heads || c->dim % c->n_q_heads || c->n_q_heads % c->n_kv_heads || !c->seq_len || !c->vocab_size)
+        return set_error(ctx, SLAI_E_SHAPE, "inconsistent model hyper-parameters");
+    return SLAI_OK;
+}
+
+int slai_llama2::load(const slai_gguf *gg) {
+    const Gguf &g = gg->g;
+    TRY(llama2_config_from_gguf(ctx, g, model_type, &config));
+    const uint32_t dim = config.dim, kvd = kv_dim();
+    if (head_size() % 2 || head_size() > 256) return set_error(ctx, SLAI_E_SHAPE, "head size must be even and <= 256");
+    // ---- Llama2Weights::from_gguf (transformer.rs:202-297)
+    weights.layers.resize(config.n_layers);
+    for (uint32_t l = 0; l < config.n_layers; ++l) {
+        Llama2LayerWeights &w = weights.layers[l];
+        const std::string p = "blk." + std::to_string(l) + ".";
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_q.weight", &w.attn_q));
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_k.weight", &w.attn_k));
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_v.weight", &w.attn_v));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_q.bias", false, &w.attn_q_bias));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_k.bias", false, &w.attn_k_bias));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_v.bias", false, &w.attn_v_bias));
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_output.weight", &w.attn_output));
+        TRY(qmat_from_gguf(ctx, gg, p + "ffn_down.weight", &w.ffn_down));
+        TRY(qmat_from_gguf(ctx, gg, p + "ffn_gate.weight", &w.ffn_gate));
+        TRY(qmat_from_gguf(ctx, gg, p + "ffn_up.weight", &w.ffn_up));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.weight", true, &w.ffn_norm));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.weight", true, &w.attn_norm));
+        struct { slai_qmat *m; uint32_t r, c; } chk[] = {{w.attn_q, dim, dim}, {w.attn_k, kvd, dim}, {w.attn_v, kvd, dim},
+            {w.attn_output, dim, dim}, {w.ffn_down, dim, config.hidden_dim}, {w.ffn_gate, config.hidden_dim, dim}, {w.ffn_up, config.hidden_dim, dim}};
+        for (auto &c : chk)
+            if (c.m->nrows != c.r || c.m->ncols != c.c) return set_error(ctx, SLAI_E_SHAPE, "layer " + std::to_string(l) + ": weight shape does not match the config");
+        for (slai_qmat *m : {w.attn_q, w.attn_k, w.attn_v, w.attn_output, w.ffn_down, w.ffn_gate, w.ffn_up}) weight_bytes += m->bytes;
+        weight_bytes += 2 * (size_t)dim * 4;
+    }
+    TRY(qmat_from_gguf(ctx, gg, "token_embd.weight", &weights.token_embd));
+    if (g.find("output.weight")) TRY(qmat_from_gguf(ctx, gg, "output.weight", &weights.output));
+    else weights.output = weights.token_embd;                                       // transformer.rs:279-285
+    TRY(f32_vector_from_gguf(ctx, g, "output_norm.weight", true, &weights.output_norm));
+    if (weights.token_embd->nrows != config.vocab_size || weights.token_embd->ncols != dim || weights.output->nrows != config.vocab_size ||
+        weights.output->ncols != dim)
+        return set_error(ctx, SLAI_E_SHAPE, "embedding / output shape does not match the config");
+    weight_bytes += weights.output->bytes + (size_t)dim * 4;
+
+    // ---- Llama2State::new (transformer.rs:47-140); buffers are zero-initialised
+    Llama2State &s = state;
+    TRY(GpuTensor::vector(ctx, dim, STORAGE | COPY_DST | COPY_SRC, &s.x));
+    TRY(GpuTensor::vector(ctx, dim, STORAGE | COPY_SRC, &s.xb));
+    TRY(GpuTensor::vector(ctx, dim, STORAGE, &s.xb2));
+    TRY(GpuTensor::vector(ctx, config.hidden_dim, STORAGE, &s.hb));
+    TRY(GpuTensor::vector(ctx, config.hidden_dim, STORAGE, &s.hb2));
+    TRY(GpuTensor::vector(ctx, dim, STORAGE | COPY_SRC, &s.q));
+    TRY(GpuTensor::vector(ctx, kvd, STORAGE, &s.kcol));
+    TRY(GpuTensor::vector(ctx, kvd, STORAGE, &s.vcol));
+    const int cdt = kv_dtype == SLAI_KV_F16 ? SLAI_DT_F16 : SLAI_DT_F32;
+    s.key_cache.resize(config.n_layers); s.value_cache.resize(config.n_layers);
+    for (uint32_t l = 0; l < config.n_layers; ++l) {
+        TRY(GpuTensor::matrix(ctx, kvd, config.seq_len, STORAGE, &s.key_cache[l], cdt));
+        TRY(GpuTensor::matrix(ctx, kvd, config.seq_len, STORAGE, &s.value_cache[l], cdt));
+    }
+    TRY(GpuTensor::matrix(ctx, config.seq_len, config.n_q_heads, STORAGE, &s.att));
+    TRY(GpuTensor::vector(ctx, config.vocab_size, STORAGE | COPY_SRC | MAP_READ, &s.logits));
+    TRY(slai_buffer_create(ctx, sizeof(slai_rope_config), SLAI_DT_U8, UNIFORM | COPY_DST, &s.rope_config));
+    TRY(slai_buffer_create(ctx, sizeof(slai_rms_norm_config), SLAI_DT_U8, UNIFORM | COPY_DST, &s.rms_norm_config));
+    TRY(slai_buffer_create(ctx, sizeof(slai_attn_params), SLAI_DT_U8, UNIFORM | COPY_DST, &s.attn_params));
+
+    attn_splits = pick_attn_splits(ctx, config.n_q_heads, config.seq_len);
+    TRY(ensure_attn_scratch(ctx, attention_scratch_floats(config.n_q_heads, head_size(), attn_splits)));
+    TRY(loop_init(ctx, loop, config.seq_len + 1));
+    return slai_synchronize(ctx);
+}
+
+// `Llama2::launch` (transformer.rs:316-381), one kernel per op in the reference's order.
+int slai_llama2::launch(LlmContext &ctxt, const slai_attn_params &attn_params, uint32_t pos) {
+    Llama2State &s = state;
+    const bool f16 = kv_dtype == SLAI_KV_F16;
+    for (uint32_t l = 0; l < config.n_layers; ++l) {
+        const Llama2LayerWeights &wl = weights.layers[l];
+        TRY(ctxt.rms_norm_assign(s.rms_norm_config, s.xb.view(), s.x.view(), wl.attn_norm.view()));             // :327
+        // :329-334 -- the GEMVs write straight into the cache column; an f16 cache goes through kcol/vcol
+        slai_view k_cache = f16 ? s.kcol.view() : s.key_cache[l].column(pos);
+        slai_view v_cache = f16 ? s.vcol.view() : s.value_cache[l].column(pos);
+        TRY(ctxt.matmul_quant_assign(s.q.view(), wl.attn_q, s.xb.view()));
+        TRY(ctxt.matmul_quant_assign(k_cache, wl.attn_k, s.xb.view()));
+        TRY(ctxt.matmul_quant_assign(v_cache, wl.attn_v, s.xb.view()));
+        if (wl.attn_q_bias.buf) TRY(ctxt.add_assign(s.q.view(), wl.attn_q_bias.view()));                        // :336-344
+        if (wl.attn_k_bias.buf) TRY(ctxt.add_assign(k_cache, wl.attn_k_bias.view()));
+        if (wl.attn_v_bias.buf) TRY(ctxt.add_assign(v_cache, wl.attn_v_bias.view()));
+        TRY(ctxt.rope(rope_variant(), s.rope_config, s.q.view(), k_cache));                                      // :346-347
+        if (f16) {
+            const size_t off = (size_t)pos * kv_dim() * 2;
+            SLAI_HIP_TRY(ctx, launch_store_kv(ctx->stream, (const float *)s.kcol.buf->dptr, (char *)s.key_cache[l].buf->dptr + off, kv_dim(), 1));
+            SLAI_HIP_TRY(ctx, launch_store_kv(ctx->stream, (const float *)s.vcol.buf->dptr, (char *)s.value_cache[l].buf->dptr + off, kv_dim(), 1));
+        }
+        TRY(slai_attention(ctx, &attn_params, s.attn_params, s.q.view(), s.key_cache[l].view(), s.value_cache[l].view(),
+                           s.att.view(), s.xb.view()));                                                          // :350, :383-400
+        TRY(ctxt.matmul_quant_assign(s.xb2.view(), wl.attn_output, s.xb.view()));                                // :352
+        TRY(ctxt.add_assign(s.x.view(), s.xb2.view()));                                                          // :355
+        TRY(ctxt.rms_norm_assign(s.rms_norm_config, s.xb.view(), s.x.view(), wl.ffn_norm.view()));               // :356
+        TRY(ctxt.matmul_quant_assign(s.hb.view(), wl.ffn_gate, s.xb.view()));                                    // :359
+        TRY(ctxt.matmul_quant_assign(s.hb2.view(), wl.ffn_up, s.xb.view()));                                     // :360
+        TRY(ctxt.silu(s.hb.view(), s.hb2.view()));                                                               // :361
+        TRY(ctxt.matmul_quant_assign(s.xb2.view(), wl.ffn_down, s.hb.view()));                                   // :362
+        TRY(ctxt.add_assign(s.x.view(), s.xb2.view()));                                                          // :365
+    }
+    TRY(ctxt.rms_norm_assign(s.rms_norm_config, s.xb.view(), s.x.view(), weights.output_norm.view()));           // :368-373
+    TRY(ctxt.matmul_quant_assign(s.logits.view(), weights.output, s.xb.view()));                                 // :375
+    return SLAI_OK;
+}
+
+int slai_llama2::gemv_fused(int type, GemvParams &p) {
+    p.rows_per_wg = ctx->gemv_rows_per_wg;
+    hipError_t e = launch_gemv(ctx, type, p);
+    if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "fused GEMV: unsupported shape for this format");
+    SLAI_HIP_TRY(ctx, e);
+    return SLAI_OK;
+}
+
+// The same computation as `launch`, as fused kernels whose per-token scalars (position, token) live
+// in device memory, so the sequence can be captured once and replayed for every token:
+//   embedding-row gather | per layer: [RMSNorm+QKV GEMV] [RoPE+cache write+attention] [Wo GEMV+residual]
+//   [RMSNorm+gate/up GEMV+SiLU] [down GEMV+residual] | [RMSNorm+logits GEMV] [argmax + loop state]
+int slai_llama2::enqueue_fused(bool with_sampler) {
+    Llama2State &s = state;
+    DecodeState *ds = (DecodeState *)loop.state->dptr;
+    float *x = (float *)s.x.buf->dptr, *xb = (float *)s.xb.buf->dptr, *hb = (float *)s.hb.buf->dptr, *hb2 = (float *)s.hb2.buf->dptr;
+    float *q = (float *)s.q.buf->dptr, *kcol = (float *)s.kcol.buf->dptr, *vcol = (float *)s.vcol.buf->dptr;
+    const uint32_t dim = config.dim, kvd = kv_dim();
+    const slai_qmat *te = weights.token_embd;
+    SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, te->type, te->dptr, te->row_stride, te->nb, &ds->token, 0, nullptr, 0, 0, nullptr, dim, x));
+    for (uint32_t l = 0; l < config.n_layers; ++l) {
+        const Llama2LayerWeights &wl = weights.layers[l];
+        // ---- RMSNorm + Q/K/V projections: matrices of one format share a launch
+        {
+            const slai_qmat *mats[3] = {wl.attn_q, wl.attn_k, wl.attn_v};
+            float *outs[3] = {q, kcol, vcol};
+            bool done[3] = {false, false, false};
+            for (int i = 0; i < 3; ++i) {
+                if (done[i]) continue;
+                GemvParams p;
+                p.nseg = 0; p.ncols = dim; p.nb = mats[i]->nb; p.x = x;
+                p.prologue = PRO_RMSNORM; p.norm_w = (const float *)wl.attn_norm.buf->dptr; p.eps = config.rms_norm_eps;
+                for (int j = i; j < 3; ++j) {
+                    if (done[j] || mats[j]->type != mats[i]->type) continue;
+                    GemvSeg &sg = p.seg[p.nseg++];
+                    sg.W = mats[j]->dptr; sg.row_stride = mats[j]->row_stride; sg.nrows = mats[j]->nrows; sg.out = outs[j];
+                    done[j] = true;
+                }
+                TRY(gemv_fused(mats[i]->type, p));
+            }
+        }
+        // ---- bias + RoPE + cache write + attention
+        {
+            AttnLaunch a{};
+            a.q = q; a.kcache = s.key_cache[l].buf->dptr; a.vcache = s.value_cache[l].buf->dptr;
+            a.kv_f16 = kv_dtype == SLAI_KV_F16;
+            a.n_heads = config.n_q_heads; a.kv_mul = config.n_q_heads / config.n_kv_heads; a.head_size = head_size();
+            a.kv_dim = kvd; a.seq_len = config.seq_len;
+            a.pos_ptr = (const uint32_t *)&ds->pos;
+            a.knew = kcol; a.vnew = vcol;
+            a.qbias = wl.attn_q_bias.buf ? (const float *)wl.attn_q_bias.buf->dptr : nullptr;
+            a.kbias = wl.attn_k_bias.buf ? (const float *)wl.attn_k_bias.buf->dptr : nullptr;
+            a.vbias = wl.attn_v_bias.buf ? (const float *)wl.attn_v_bias.buf->dptr : nullptr;
+            a.rope_variant = rope_variant(); a.rope_base = config.rope_base_freq;
+            a.out = xb; a.scratch = ctx->attn_scratch; a.n_splits = attn_splits;
+            hipError_t e = launch_attention(ctx->stream, a);
+            if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "attention: unsupported head size or context length");
+            SLAI_HIP_TRY(ctx, e);
+        }
+        // ---- attention output projection, residual in the epilogue
+        {
+            GemvParams p;
+            p.nseg = 1; p.ncols = dim; p.nb = wl.attn_output->nb; p.x = xb;
+            p.seg[0].W = wl.attn_output->dptr; p.seg[0].row_stride = wl.attn_output->row_stride; p.seg[0].nrows = dim;
+            p.seg[0].out = x; p.seg[0].flags = GEMV_ACCUM;
+            TRY(gemv_fused(wl.attn_output->type, p));
+        }
+        // ---- RMSNorm + gate/up + SiLU
+        if (wl.ffn_gate->type == wl.ffn_up->type) {
+            GemvParams p;
+            p.nseg = 1; p.ncols = dim; p.nb = wl.ffn_gate->nb; p.x = x;
+            p.prologue = PRO_RMSNORM; p.norm_w = (const float *)wl.ffn_norm.buf->dptr; p.eps = config.rms_norm_eps;
+            p.seg[0].W = wl.ffn_gate->dptr; p.seg[0].W2 = wl.ffn_up->dptr; p.seg[0].row_stride = wl.ffn_gate->row_stride;
+            p.seg[0].nrows = config.hidden_dim; p.seg[0].out = hb; p.seg[0].flags = GEMV_SILU_GATE;
+            TRY(gemv_fused(wl.ffn_gate->type, p));
+        } else {
+            const slai_qmat *mats[2] = {wl.ffn_gate, wl.ffn_up};
+            float *outs[2] = {hb, hb2};
+            for (int i = 0; i < 2; ++i) {
+                GemvParams p;
+                p.nseg = 1; p.ncols = dim; p.nb = mats[i]->nb; p.x = x;
+                p.prologue = PRO_RMSNORM; p.norm_w = (const float *)wl.ffn_norm.buf->dptr; p.eps = config.rms_norm_eps;
+                p.seg[0].W = mats[i]->dptr; p.seg[0].row_stride = mats[i]->row_stride; p.seg[0].nrows = config.hidden_dim; p.seg[0].out = outs[i];
+                TRY(gemv_fused(mats[i]->type, p));
+            }
+            SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, config.hidden_dim, 1}, VecView{hb2, config.hidden_dim, 1}));
+        }
+        // ---- down projection, residual in the epilogue
+        {
+            GemvParams p;
+            p.nseg = 1; p.ncols = config.hidden_dim; p.nb = wl.ffn_down->nb; p.x = hb;
+            p.seg[0].W = wl.ffn_down->dptr; p.seg[0].row_stride = wl.ffn_down->row_stride; p.seg[0].nrows = dim;
+            p.seg[0].out = x; p.seg[0].flags = GEMV_ACCUM;
+            TRY(gemv_fused(wl.ffn_down->type, p));
+        }
+    }
+    {
+        GemvParams p;
+        p.nseg = 1; p.ncols = dim; p.nb = weights.output->nb; p.x = x;
+        p.prologue = PRO_RMSNORM; p.norm_w = (const float *)weights.output_norm.buf->dptr; p.eps = config.rms_norm_eps;
+        p.seg[0].W = weights.output->dptr; p.seg[0].row_stride = weights.output->row_stride; p.seg[0].nrows = config.vocab_size;
+        p.seg[0].out = (float *)s.logits.buf->dptr;
+        TRY(gemv_fused(weights.output->type, p));
+    }
+    if (with_sampler)
+        SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, nullptr, ds,
+                                        (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_llama2_from_gguf(slai_ctx *ctx, const slai_gguf *g, int model_type, int kv_dtype, slai_llama2 **out) {
+    if (!ctx || !g || !out) return SLAI_E_ARG;
+    *out = nullptr;
+    if ((model_type != SLAI_MODEL_LLAMA && model_type != SLAI_MODEL_QWEN2) || (kv_dtype != SLAI_KV_F32 && kv_dtype != SLAI_KV_F16))
+        return set_error(ctx, SLAI_E_ARG, "slai_llama2_from_gguf: bad model type or kv dtype");
+    std::unique_ptr<slai_llama2> m(new slai_llama2());
+    m->ctx = ctx; m->model_type = model_type; m->kv_dtype = kv_dtype;
+    int rc = m->load(g);
+    if (rc) { std::string keep = ctx->err; slai_llama2_destroy(m.release()); ctx->err = keep; return rc; }
+    *out = m.release();
+    return SLAI_OK;
+}
+
+SLAI_EXPORT void slai_llama2_destroy(slai_llama2 *m) {
+    if (!m) return;
+    slai_ctx *ctx = m->ctx;
+    slai_synchronize(ctx);
+    loop_destroy(ctx, m->loop);
+    for (auto &w : m->weights.layers) {
+        for (slai_qmat *q : {w.attn_k, w.attn_q, w.attn_v, w.ffn_down, w.ffn_gate, w.ffn_up, w.attn_output}) slai_qmat_destroy(ctx, q);
+        for (GpuTensor *t : {&w.attn_norm, &w.attn_k_bias, &w.attn_q_bias, &w.attn_v_bias, &w.ffn_norm}) t->destroy(ctx);
+    }
+    if (m->weights.output != m->weights.token_embd) slai_qmat_destroy(ctx, m->weights.output);
+    slai_qmat_destroy(ctx, m->weights.token_embd);
+    m->weights.output_norm.destroy(ctx);
+    Llama2State &s = m->state;
+    for (GpuTensor *t : {&s.x, &s.xb, &s.xb2, &s.hb, &s.hb2, &s.q, &s.att, &s.logits, &s.kcol, &s.vcol}) t->destroy(ctx);
+    for (auto &t : s.key_cache) t.destroy(ctx);
+    for (auto &t : s.value_cache) t.destroy(ctx);
+    for (slai_buffer *b : {s.rope_config, s.rms_norm_config, s.attn_params}) if (b) slai_buffer_destroy(ctx, b);
+    delete m;
+}
+
+SLAI_EXPORT int slai_llama2_get_config(const slai_llama2 *m, slai_llama2_config *out) {
+    if (!m || !out) return SLAI_E_ARG;
+    *out = m->config;
+    return SLAI_OK;
+}
+SLAI_EXPORT size_t slai_llama2_weight_bytes(const slai_llama2 *m) { return m ? m->weight_bytes : 0; }
+
+// `Llama2Config::derived_configs` (models/llama2/cpu.rs:111-143)
+static void derived_configs(const slai_llama2 *m, uint32_t pos, slai_rope_config *rope, slai_rms_norm_config *rms, slai_attn_params *attn) {
+    const slai_llama2_config &c = m->config;
+    *rope = slai_rope_config{m->head_size(), m->kv_dim(), pos, c.rope_base_freq};
+    *rms = slai_rms_norm_config{c.rms_norm_eps, {0, 0, 0}};
+    *attn = slai_attn_params{c.seq_len, m->kv_dim(), c.n_q_heads / c.n_kv_heads, c.n_q_heads, m->head_size(), pos, {0, 0}};
+}
+
+SLAI_EXPORT int slai_llama2_forward_logits(slai_llama2 *m, uint32_t pos, uint32_t token, int fused, float *logits_out) {
+    if (!m) return SLAI_E_ARG;
+    slai_ctx *ctx = m->ctx;
+    if (pos >= m->config.seq_len || token >= m->config.vocab_size) return set_error(ctx, SLAI_E_ARG, "slai_llama2_forward_logits: position or token out of range");
+    Llama2State &s = m->state;
+    if (!fused) {
+        // chat_llama2.rs:176-189: per-token uniforms, then the embedding column into x
+        slai_rope_config rope; slai_rms_norm_config rms; slai_attn_params attn;
+        derived_configs(m, pos, &rope, &rms, &attn);
+        TRY(slai_write_buffer(ctx, s.rope_config, 0, &rope, sizeof rope));
+        TRY(slai_write_buffer(ctx, s.rms_norm_config, 0, &rms, sizeof rms));
+        TRY(slai_write_buffer(ctx, s.attn_params, 0, &attn, sizeof attn));
+        const slai_qmat *te = m->weights.token_embd;
+        TRY(slai_qmat_dequantize(ctx, te, token, 1, slai_view{s.x.buf, 0, {1, m->config.dim, 1, 1}, {m->config.dim, 1, m->config.dim, m->config.dim}}));
+        LlmContext ctxt(ctx);
+        TRY(ctxt.begin_submission());                                   // :199
+        TRY(m->launch(ctxt, attn, pos));                                 // :200-207
+        TRY(ctxt.submit());                                              // :218
+    } else {
+        DecodeState ds{(int)pos, (int)token, 0, 0};
+        TRY(slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds));
+        TRY(m->enqueue_fused(false));
+    }
+    TRY(slai_synchronize(ctx));                                          // :219
+    if (logits_out) TRY(slai_read_buffer(ctx, s.logits.buf, 0, logits_out, (size_t)m->config.vocab_size * 4));   // :225-227
+    return SLAI_OK;
+}
+
+template <class Model>
+static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_len, uint32_t vocab, const int32_t *prompt, uint32_t n_prompt,
+                         uint32_t start_pos, uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms) {
+    if (!prompt || !out_tokens || n_prompt == 0 || start_pos >= n_prompt) return set_error(ctx, SLAI_E_ARG, "generate: bad prompt / start position");
+    if (n_steps == 0) return SLAI_OK;
+    if (start_pos + n_steps > seq_len) return set_error(ctx, SLAI_E_SHAPE, "generate: would run past the context length");
+    if (n_prompt > L.capacity || n_steps > L.capacity) return set_error(ctx, SLAI_E_SHAPE, "generate: prompt longer than the context length");
+    for (uint32_t i = 0; i < n_prompt; ++i)
+        if (prompt[i] < 0 || (uint32_t)prompt[i] >= vocab) return set_error(ctx, SLAI_E_ARG, "generate: prompt token out of range");
+    DecodeState ds{(int)start_pos, prompt[start_pos], (int)n_prompt, 0};     // chat_llama2.rs:105
+    TRY(slai_write_buffer(ctx, L.state, 0, &ds, sizeof ds));
+    TRY(slai_write_buffer(ctx, L.prompt, 0, prompt, (size_t)n_prompt * 4));
+    if (!L.graph) {
+        TRY(slai_graph_begin_capture(ctx));
+        int rc = m->enqueue_fused(true);
+        slai_graph *g = nullptr;
+        int rc2 = slai_graph_end_capture(ctx, &g);
+        if (rc) { if (g) slai_graph_destroy(ctx, g); return rc; }
+        if (rc2) return rc2;
+        L.graph = g;
+    }
+    SLAI_HIP_TRY(ctx, hipEventRecord(L.ev0, ctx->stream));
+    for (uint32_t i = 0; i < n_steps; ++i) TRY(slai_graph_launch(ctx, L.graph));       // chat_llama2.rs:109 loop
+    SLAI_HIP_TRY(ctx, hipEventRecord(L.ev1, ctx->stream));
+    TRY(slai_synchronize(ctx));
+    if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, L.ev0, L.ev1));
+    return slai_read_buffer(ctx, L.out_tokens, 0, out_tokens, (size_t)n_steps * 4);
+}
+
+SLAI_EXPORT int slai_llama2_generate(slai_llama2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos, uint32_t n_steps,
+                                     int32_t *out_tokens, float *elapsed_ms) {
+    if (!m) return SLAI_E_ARG;
+    return generate_impl(m, m->ctx, m->loop, m->config.seq_len, m->config.vocab_size, prompt, n_prompt, start_pos, n_steps, out_tokens, elapsed_ms);
+}
+
+SLAI_EXPORT int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache) {
+    if (!m || layer >= m->config.n_layers) return SLAI_E_ARG;
+    if (key_cache) *key_cache = m->state.key_cache[layer].buf;
+    if (value_cache) *value_cache = m->state.value_cache[layer].buf;
+    return SLAI_OK;
+}
+SLAI_EXPORT int slai_llama2_logits_buffer(slai_llama2 *m, slai_buffer **logits) {
+    if (!m || !logits) return SLAI_E_ARG;
+    *logits = m->state.logits.buf;
+    return SLAI_OK;
+}
+
+// =================================================================================================
+// GPT-2 (models/gpt2/cpu.rs)
+// =================================================================================================
+struct Gpt2Layer {                   // gpt2/cpu.rs:67-89
+    GpuTensor ln_1_g, ln_1_b, ln_2_g, ln_2_b;
+    slai_qmat *c_attn_attn_w = nullptr; GpuTensor c_attn_attn_b;
+    slai_qmat *c_attn_proj_w = nullptr; GpuTensor c_attn_proj_b;
+    GpuTensor key_cache, value_cache;
+    slai_qmat *c_mlp_fc_w = nullptr; GpuTensor c_mlp_fc_b;
+    slai_qmat *c_mlp_proj_w = nullptr; GpuTensor c_mlp_proj_b;
+};
+
+struct slai_gpt2 {
+    slai_ctx *ctx = nullptr;
+    int kv_dtype = SLAI_KV_F32;
+    slai_gpt2_params params{};
+    std::vector<Gpt2Layer> layers;
+    GpuTensor ln_f_g, ln_f_b;
+    slai_qmat *wte = nullptr, *wpe = nullptr;   // lm_head is wte (gpt2/cpu.rs:196-197)
+    GpuTensor layer_input, curr_768, curr_2304, curr_3072, curr_vocab;   // gpt2/cpu.rs:102-110
+    DeviceLoop loop;
+    size_t weight_bytes = 0;
+    uint32_t attn_splits = 1;
+
+    int load(const slai_gguf *g);
+    int enqueue_fused(bool with_sampler);
+    int gemv(int type, GemvParams &p) {
+        p.rows_per_wg = ctx->gemv_rows_per_wg;
+        hipError_t e = launch_gemv(ctx, type, p);
+        if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "GEMV: unsupported shape for this format");
+        SLAI_HIP_TRY(ctx, e);
+        return SLAI_OK;
+    }
+};
+
+int slai_gpt2::load(const slai_gguf *gg) {
+    const Gguf &g = gg->g;
+    // Gpt2Params::from_gguf (gpt2/cpu.rs:37-48)
+    const GgufMetaValue *tok = g.meta("tokenizer.ggml.tokens");
+    if (!tok) return set_error(ctx, SLAI_E_MISSING, "missing metadata key 'tokenizer.ggml.tokens'");
+    if (tok->type != 9) return set_error(ctx, SLAI_E_TYPE, "unwrap: unexpected GGUF attribute type for 'tokenizer.ggml.tokens'");
+    params.n_vocab = (uint32_t)tok->arr_len;
+    TRY(meta_u32(ctx, g, "gpt2.context_length", &params.n_seq));
+    TRY(meta_u32(ctx, g, "gpt2.embedding_length", &params.n_embd));
+    TRY(meta_u32(ctx, g, "gpt2.attention.head_count", &params.n_head));
+    TRY(meta_u32(ctx, g, "gpt2.block_count", &params.n_layer));
+    TRY(meta_u32(ctx, g, "gpt2.feed_forward_length", &params.ff_len));
+    // The reference reads attn_b from dimensions()[0] of a 1-D bias, which is 1 after the dim swap
+    // (gpt2/cpu.rs:46 + gguf.rs:581); the forward needs 3*n_embd (:252-270).
+    params.attn_b = 3 * params.n_embd;
+    const uint32_t E = params.n_embd;
+    if (!E || !params.n_head || E % params.n_head || (E / params.n_head) % 2 || E / params.n_head > 256) return set_error(ctx, SLAI_E_SHAPE, "inconsistent GPT-2 hyper-parameters");
+    const int cdt = kv_dtype == SLAI_KV_F16 ? SLAI_DT_F16 : SLAI_DT_F32;
+    layers.resize(params.n_layer);
+    for (uint32_t l = 0; l < params.n_layer; ++l) {       // gpt2/cpu.rs:118-179
+        Gpt2Layer &w = layers[l];
+        const std::string p = "blk." + std::to_string(l) + ".";
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.weight", true, &w.ln_1_g));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.bias", true, &w.ln_1_b));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.weight", true, &w.ln_2_g));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.bias", true, &w.ln_2_b));
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_qkv.weight", &w.c_attn_attn_w));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_qkv.bias", true, &w.c_attn_attn_b));
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_output.weight", &w.c_attn_proj_w));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_output.bias", true, &w.c_attn_proj_b));
+        TRY(qmat_from_gguf(ctx, gg, p + "ffn_up.weight", &w.c_mlp_fc_w));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_up.bias", true, &w.c_mlp_fc_b));
+        TRY(qmat_from_gguf(ctx, gg, p + "ffn_down.weight", &w.c_mlp_proj_w));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_down.bias", true, &w.c_mlp_proj_b));
+        struct { slai_qmat *m; uint32_t r, c; } chk[] = {{w.c_attn_attn_w, 3 * E, E}, {w.c_attn_proj_w, E, E}, {w.c_mlp_fc_w, params.ff_len, E}, {w.c_mlp_proj_w, E, params.ff_len}};
+        for (auto &c : chk)
+            if (c.m->nrows != c.r || c.m->ncols != c.c) return set_error(ctx, SLAI_E_SHAPE, "layer " + std::to_string(l) + ": weight shape does not match the parameters");
+        TRY(GpuTensor::matrix(ctx, E, params.n_seq, STORAGE, &w.key_cache, cdt));
+        TRY(GpuTensor::matrix(ctx, E, params.n_seq, STORAGE, &w.value_cache, cdt));
+        for (slai_qmat *m : {w.c_attn_attn_w, w.c_attn_proj_w, w.c_mlp_fc_w, w.c_mlp_proj_w}) weight_bytes += m->bytes;
+        weight_bytes += (size_t)(4 * E + 3 * E + E + params.ff_len + E) * 4;
+    }
+    TRY(f32_vector_from_gguf(ctx, g, "output_norm.weight", true, &ln_f_g));
+    TRY(f32_vector_from_gguf(ctx, g, "output_norm.bias", true, &ln_f_b));
+    TRY(qmat_from_gguf(ctx, gg, "token_embd.weight", &wte));
+    TRY(qmat_from_gguf(ctx, gg, "position_embd.weight", &wpe));
+    if (wte->nrows != params.n_vocab || wte->ncols != E || wpe->ncols != E || wpe->nrows < params.n_seq)
+        return set_error(ctx, SLAI_E_SHAPE, "embedding shapes do not match the parameters");
+    weight_bytes += wte->bytes + 2 * (size_t)E * 4;
+    TRY(GpuTensor::vector(ctx, E, STORAGE, &layer_input));
+    TRY(GpuTensor::vector(ctx, E, STORAGE, &curr_768));
+    TRY(GpuTensor::vector(ctx, params.attn_b, STORAGE, &curr_2304));
+    TRY(GpuTensor::vector(ctx, params.ff_len, STORAGE, &curr_3072));
+    TRY(GpuTensor::vector(ctx, params.n_vocab, STORAGE | COPY_SRC | MAP_READ, &curr_vocab));
+    attn_splits = pick_attn_splits(ctx, params.n_head, params.n_seq);
+    TRY(ensure_attn_scratch(ctx, attention_scratch_floats(params.n_head, E / params.n_head, attn_splits)));
+    TRY(loop_init(ctx, loop, params.n_seq + 1));
+    return slai_synchronize(ctx);
+}
+
+// gpt2/cpu.rs:224-383 as fused kernels (LayerNorm eps 1e-5: ops/layernorm.rs:105)
+int slai_gpt2::enqueue_fused(bool with_sampler) {
+    DecodeState *ds = (DecodeState *)loop.state->dptr;
+    const uint32_t E = params.n_embd;
+    float *x = (float *)layer_input.buf->dptr, *att_out = (float *)curr_768.buf->dptr, *qkv = (float *)curr_2304.buf->dptr,
+          *h = (float *)curr_3072.buf->dptr, *logits = (float *)curr_vocab.buf->dptr;
+    const float eps = 1.0e-5f;
+    // :227-228 wte[:,tok] + wpe[:,pos]
+    SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, wte->type, wte->dptr, wte->row_stride, wte->nb, &ds->token, wpe->type, wpe->dptr,
+                                   wpe->row_stride, wpe->nb, &ds->pos, E, x));
+    for (uint32_t l = 0; l < params.n_layer; ++l) {
+        Gpt2Layer &w = layers[l];
+        {   // :235-255 LayerNorm*g+b, qkv GEMV + bias
+            GemvParams p;
+            p.nseg = 1; p.ncols = E; p.nb = w.c_attn_attn_w->nb; p.x = x;
+            p.prologue = PRO_LAYERNORM; p.norm_w = (const float *)w.ln_1_g.buf->dptr; p.norm_b = (const float *)w.ln_1_b.buf->dptr; p.eps = eps;
+            p.seg[0].W = w.c_attn_attn_w->dptr; p.seg[0].row_stride = w.c_attn_attn_w->row_stride; p.seg[0].nrows = 3 * E;
+            p.seg[0].out = qkv; p.seg[0].bias = (const float *)w.c_attn_attn_b.buf->dptr; p.seg[0].flags = GEMV_BIAS;
+            TRY(gemv(w.c_attn_attn_w->type, p));
+        }
+        {   // :263-290 split q/k/v, cache write, attention with kv_mul = 1
+            AttnLaunch a{};
+            a.q = qkv; a.knew = qkv + E; a.vnew = qkv + 2 * E;
+            a.kcache = w.key_cache.buf->dptr; a.vcache = w.value_cache.buf->dptr; a.kv_f16 = kv_dtype == SLAI_KV_F16;
+            a.n_heads = params.n_head; a.kv_mul = 1; a.head_size = E / params.n_head; a.kv_dim = E; a.seq_len = params.n_seq;
+            a.pos_ptr = (const uint32_t *)&ds->pos;
+            a.rope_variant = -1; a.rope_base = 0.0f;
+            a.out = att_out; a.scratch = ctx->attn_scratch; a.n_splits = attn_splits;
+            hipError_t e = launch_attention(ctx->stream, a);
+            if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "attention: unsupported head size or context length");
+            SLAI_HIP_TRY(ctx, e);
+        }
+        {   // :302-312 projection + bias + residual
+            GemvParams p;
+            p.nseg = 1; p.ncols = E; p.nb = w.c_attn_proj_w->nb; p.x = att_out;
+            p.seg[0].W = w.c_attn_proj_w->dptr; p.seg[0].row_stride = w.c_attn_proj_w->row_stride; p.seg[0].nrows = E;
+            p.seg[0].out = x; p.seg[0].bias = (const float *)w.c_attn_proj_b.buf->dptr; p.seg[0].flags = GEMV_BIAS | GEMV_ACCUM;
+            TRY(gemv(w.c_attn_proj_w->type, p));
+        }
+        {   // :318-343 LayerNorm*g+b, fc GEMV + bias, GELU
+            GemvParams p;
+            p.nseg = 1; p.ncols = E; p.nb = w.c_mlp_fc_w->nb; p.x = x;
+            p.prologue = PRO_LAYERNORM; p.norm_w = (const float *)w.ln_2_g.buf->dptr; p.norm_b = (const float *)w.ln_2_b.buf->dptr; p.eps = eps;
+            p.seg[0].W = w.c_mlp_fc_w->dptr; p.seg[0].row_stride = w.c_mlp_fc_w->row_stride; p.seg[0].nrows = params.ff_len;
+            p.seg[0].out = h; p.seg[0].bias = (const float *)w.c_mlp_fc_b.buf->dptr; p.seg[0].flags = GEMV_BIAS | GEMV_GELU;
+            TRY(gemv(w.c_mlp_fc_w->type, p));
+        }
+        {   // :353-360 projection + bias + residual
+            GemvParams p;
+            p.nseg = 1; p.ncols = params.ff_len; p.nb = w.c_mlp_proj_w->nb; p.x = h;
+            p.seg[0].W = w.c_mlp_proj_w->dptr; p.seg[0].row_stride = w.c_mlp_proj_w->row_stride; p.seg[0].nrows = E;
+            p.seg[0].out = x; p.seg[0].bias = (const float *)w.c_mlp_proj_b.buf->dptr; p.seg[0].flags = GEMV_BIAS | GEMV_ACCUM;
+            TRY(gemv(w.c_mlp_proj_w->type, p));
+        }
+    }
+    {   // :366-379 final LayerNorm*g+b, lm_head = wte
+        GemvParams p;
+        p.nseg = 1; p.ncols = E; p.nb = wte->nb; p.x = x;
+        p.prologue = PRO_LAYERNORM; p.norm_w = (const float *)ln_f_g.buf->dptr; p.norm_b = (const float *)ln_f_b.buf->dptr; p.eps = eps;
+        p.seg[0].W = wte->dptr; p.seg[0].row_stride = wte->row_stride; p.seg[0].nrows = params.n_vocab; p.seg[0].out = logits;
+        TRY(gemv(wte->type, p));
+    }
+    if (with_sampler)
+        SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, logits, params.n_vocab, nullptr, ds, (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_gpt2_from_gguf(slai_ctx *ctx, const slai_gguf *g, int kv_dtype, slai_gpt2 **out) {
+    if (!ctx || !g || !out) return SLAI_E_ARG;
+    *out = nullptr;
+    if (kv_dtype != SLAI_KV_F32 && kv_dtype != SLAI_KV_F16) return set_error(ctx, SLAI_E_ARG, "slai_gpt2_from_gguf: bad kv dtype");
+    std::unique_ptr<slai_gpt2> m(new slai_gpt2());
+    m->ctx = ctx; m->kv_dtype = kv_dtype;
+    int rc = m->load(g);
+    if (rc) { std::string keep = ctx->err; slai_gpt2_destroy(m.release()); ctx->err = keep; return rc; }
+    *out = m.release();
+    return SLAI_OK;
+}
+
+SLAI_EXPORT void slai_gpt2_destroy(slai_gpt2 *m) {
+    if (!m) return;
+    slai_ctx *ctx = m->ctx;
+    slai_synchronize(ctx);
+    loop_destroy(ctx, m->loop);
+    for (auto &w : m->layers) {
+        for (slai_qmat *q : {w.c_attn_attn_w, w.c_attn_proj_w, w.c_mlp_fc_w, w.c_mlp_proj_w}) slai_qmat_destroy(ctx, q);
+        for (GpuTensor *t : {&w.ln_1_g, &w.ln_1_b, &w.ln_2_g, &w.ln_2_b, &w.c_attn_attn_b, &w.c_attn_proj_b, &w.key_cache, &w.value_cache,
+                             &w.c_mlp_fc_b, &w.c_mlp_proj_b}) t->destroy(ctx);
+    }
+    slai_qmat_destroy(ctx, m->wte); slai_qmat_destroy(ctx, m->wpe);
+    for (GpuTensor *t : {&m->ln_f_g, &m->ln_f_b, &m->layer_input, &m->curr_768, &m->curr_2304, &m->curr_3072, &m->curr_vocab}) t->destroy(ctx);
+    delete m;
+}
+
+SLAI_EXPORT int slai_gpt2_get_params(const slai_gpt2 *m, slai_gpt2_params *out) {
+    if (!m || !out) return SLAI_E_ARG;
+    *out = m->params;
+    return SLAI_OK;
+}
+SLAI_EXPORT size_t slai_gpt2_weight_bytes(const slai_gpt2 *m) { return m ? m->weight_bytes : 0; }
+
+SLAI_EXPORT int slai_gpt2_forward_logits(slai_gpt2 *m, uint32_t pos, uint32_t token, float *logits_out) {
+    if (!m) return SLAI_E_ARG;
+    slai_ctx *ctx = m->ctx;
+    if (pos >= m->params.n_seq || token >= m->params.n_vocab) return set_error(ctx, SLAI_E_ARG, "slai_gpt2_forward_logits: position or token out of range");
+    DecodeState ds{(int)pos, (int)token, 0, 0};
+    TRY(slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds));
+    TRY(m->enqueue_fused(false));
+    TRY(slai_synchronize(ctx));
+    if (logits_out) TRY(slai_read_buffer(ctx, m->curr_vocab.buf, 0, logits_out, (size_t)m->params.n_vocab * 4));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_gpt2_generate(slai_gpt2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos, uint32_t n_steps,
+                                   int32_t *out_tokens, float *elapsed_ms) {
+    if (!m) return SLAI_E_ARG;
+    return generate_impl(m, m->ctx, m->loop, m->params.n_seq, m->params.n_vocab, prompt, n_prompt, start_pos, n_steps, out_tokens, elapsed_ms);
+}

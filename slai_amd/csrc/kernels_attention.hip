@@ -1,0 +1,230 @@
+// KV-cache attention for single-token decode: QK^T, softmax, .V in one kernel, split over the
+// sequence (flash-decoding) with a small combine kernel when more than one split is used.
+//
+// Reproduces `BatchedMultiqueryAttention` (crates/slai/src/ops/batched_multiquery_attention.rs:32-156,
+// CPU form models/llama2/cpu.rs:488-539): per query head h (kv head h / kv_mul)
+//   s_t = q_h . K[t]_h / sqrt(head_size), t <= pos;  p = softmax(s);  out_h = sum_t p_t V[t]_h
+// which the reference issues as four launches (gemv, mask/scale, softmax, gemv) with the score
+// matrix round-tripping through memory.  Exactly pos+1 positions are read (the reference rounds
+// up to a multiple of 4 and reads uninitialised cache columns).
+//
+// Cache layout is the reference's: [kv_dim x seq_len] column-major, i.e. one position = kv_dim
+// contiguous values (transformer.rs:87-106), f32 or f16.
+//
+// In the model path the kernel also performs RoPE (rope.slang:27-84) on q and on the fresh key
+// and writes the fresh key/value into the cache, so Q/K/V leave the projection GEMV exactly once.
+#include "common.h"
+#include "quant_formats.h"
+#include <float.h>
+
+namespace slai {
+namespace {
+
+constexpr int ATT_THREADS = 256;
+constexpr int MAX_HS = 256;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+    return v;
+}
+
+template <bool F16> struct KV;
+template <> struct KV<true> {
+    using T = uint16_t;
+    __device__ static float2 load2(const T *p) { uint32_t w = *reinterpret_cast<const uint32_t *>(p); return make_float2(decode_f16((uint16_t)(w & 0xffffu)), decode_f16((uint16_t)(w >> 16))); }
+    __device__ static float round(float v) { return decode_f16(encode_f16(v)); }
+    __device__ static void store(T *p, float v) { *p = encode_f16(v); }
+};
+template <> struct KV<false> {
+    using T = float;
+    __device__ static float2 load2(const T *p) { return *reinterpret_cast<const float2 *>(p); }
+    __device__ static float round(float v) { return v; }
+    __device__ static void store(T *p, float v) { *p = v; }
+};
+
+// grid = (n_heads, n_splits), block = ATT_THREADS.  Dynamic LDS: scores for one split.
+template <bool F16>
+__global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_t max_split_len) {
+    using C = KV<F16>;
+    using CT = typename C::T;
+    extern __shared__ float sscore[];             // [max_split_len]
+    __shared__ float sq[MAX_HS], sk[MAX_HS], sv[MAX_HS];
+    __shared__ float sred[ATT_THREADS / 64];
+    __shared__ float sacc[ATT_THREADS * 2];  // cross-group reduction of the output
+
+    const uint32_t h = blockIdx.x, split = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t hs = a.head_size, kvh = h / a.kv_mul;
+    const uint32_t pos = *a.pos_ptr;
+    const uint32_t T = pos + 1;
+    const uint32_t chunk = (T + a.n_splits - 1) / a.n_splits;
+    const uint32_t t0 = split * chunk;
+    const uint32_t t1 = min(T, t0 + chunk);
+    CT *kc = reinterpret_cast<CT *>(a.kcache), *vc = reinterpret_cast<CT *>(a.vcache);
+    const size_t hoff = (size_t)kvh * hs;
+    const bool fresh = a.knew != nullptr;
+    const bool own_new = fresh && t0 <= pos && pos < t1;   // this split covers the current position
+
+    // ---- q (and the fresh k/v) into LDS, with bias and RoPE when fused -----------------------
+    if (tid < hs / 2) {
+        const uint32_t i = tid;   // pair index inside the head
+        uint32_t e0, e1;
+        if (a.rope_variant == SLAI_ROPE_NEOX) { e0 = i; e1 = i + hs / 2; } else { e0 = 2 * i; e1 = 2 * i + 1; }
+        float q0 = a.q[(size_t)h * hs + e0], q1 = a.q[(size_t)h * hs + e1];
+        if (fresh) {
+            if (a.qbias) { q0 += a.qbias[(size_t)h * hs + e0]; q1 += a.qbias[(size_t)h * hs + e1]; }
+            const bool rot = a.rope_variant >= 0;   // GPT-2 has learned positions: no rotation
+            float c = 1.0f, s = 0.0f;
+            if (rot) {
+                // rope.slang:36-39: the angle depends on (2*i) mod head_size for both variants
+                const float head_dim = (float)((2 * i) % hs);
+                const float theta = powf(a.rope_base, -head_dim / (float)hs);
+                const float m_theta = (float)pos * theta;
+                c = cosf(m_theta); s = sinf(m_theta);
+                const float r0 = c * q0 - s * q1, r1 = s * q0 + c * q1;
+                q0 = r0; q1 = r1;
+            }
+            if (own_new) {
+                float k0 = a.knew[hoff + e0], k1 = a.knew[hoff + e1];
+                float v0 = a.vnew[hoff + e0], v1 = a.vnew[hoff + e1];
+                if (a.kbias) { k0 += a.kbias[hoff + e0]; k1 += a.kbias[hoff + e1]; }
+                if (a.vbias) { v0 += a.vbias[hoff + e0]; v1 += a.vbias[hoff + e1]; }
+                if (rot) {
+                    const float kr0 = c * k0 - s * k1, kr1 = s * k0 + c * k1;
+                    k0 = kr0; k1 = kr1;
+                }
+                sk[e0] = C::round(k0); sk[e1] = C::round(k1);
+                sv[e0] = C::round(v0); sv[e1] = C::round(v1);
+                // several query heads share a kv head: the first of the group writes the cache
+                if (h % a.kv_mul == 0) {
+                    CT *kd = kc + (size_t)pos * a.kv_dim + hoff, *vd = vc + (size_t)pos * a.kv_dim + hoff;
+                    C::store(kd + e0, k0); C::store(kd + e1, k1);
+                    C::store(vd + e0, v0); C::store(vd + e1, v1);
+                }
+            }
+        }
+        sq[e0] = q0; sq[e1] = q1;
+    }
+    __syncthreads();
+
+    // ---- scores: one wave per position, lanes over element pairs ----------------------------------
+    const float inv_sqrt = sqrtf((float)hs);
+    float lmax = -FLT_MAX;
+    for (uint32_t t = t0 + wave; t < t1; t += ATT_THREADS / 64) {
+        float part = 0.0f;
+        const bool use_new = own_new && t == pos;
+        for (uint32_t e = 2 * lane; e < hs; e += 128) {
+            float2 kv;
+            if (use_new) kv = make_float2(sk[e], sk[e + 1]);
+            else kv = C::load2(kc + (size_t)t * a.kv_dim + hoff + e);
+            part = fmaf(sq[e], kv.x, part);
+            part = fmaf(sq[e + 1], kv.y, part);
+        }
+        part = wave_sum(part);
+        const float sc = part / inv_sqrt;       // cpu.rs:521 `score /= sqrt(head_size)`
+        if (lane == 0) sscore[t - t0] = sc;
+        lmax = fmaxf(lmax, sc);
+    }
+    // block max
+    if (lane == 0) sred[wave] = lmax;
+    __syncthreads();
+    float m = sred[0];
+#pragma unroll
+    for (int w = 1; w < ATT_THREADS / 64; ++w) m = fmaxf(m, sred[w]);
+    __syncthreads();
+
+    // ---- exp and sum ------------------------------------------------------------------------------
+    float lsum = 0.0f;
+    for (uint32_t t = t0 + tid; t < t1; t += ATT_THREADS) {
+        const float e = expf(sscore[t - t0] - m);
+        sscore[t - t0] = e;
+        lsum += e;
+    }
+    lsum = wave_sum(lsum);
+    if (lane == 0) sred[wave] = lsum;
+    __syncthreads();
+    float l = 0.0f;
+#pragma unroll
+    for (int w = 0; w < ATT_THREADS / 64; ++w) l += sred[w];
+
+    // ---- weighted sum of values: thread = (position group g, element pair i) ------------------------
+    const uint32_t pairs = hs / 2;
+    const uint32_t groups = ATT_THREADS / pairs ? ATT_THREADS / pairs : 1;
+    const uint32_t g = tid / pairs, i2 = tid % pairs;
+    float o0 = 0.0f, o1 = 0.0f;
+    if (g < groups && pairs <= ATT_THREADS) {
+        for (uint32_t t = t0 + g; t < t1; t += groups) {
+            const float p = sscore[t - t0];
+            float2 vv;
+            if (own_new && t == pos) vv = make_float2(sv[2 * i2], sv[2 * i2 + 1]);
+            else vv = C::load2(vc + (size_t)t * a.kv_dim + hoff + 2 * i2);
+            o0 = fmaf(p, vv.x, o0);
+            o1 = fmaf(p, vv.y, o1);
+        }
+    }
+    sacc[2 * tid] = o0; sacc[2 * tid + 1] = o1;
+    __syncthreads();
+    if (tid < pairs) {
+        float r0 = 0.0f, r1 = 0.0f;
+        for (uint32_t gg = 0; gg < groups; ++gg) { r0 += sacc[2 * (gg * pairs + tid)]; r1 += sacc[2 * (gg * pairs + tid) + 1]; }
+        if (a.n_splits == 1) {
+            a.out[(size_t)h * hs + 2 * tid] = r0 / l;
+            a.out[(size_t)h * hs + 2 * tid + 1] = r1 / l;
+        } else {
+            float *po = a.scratch + ((size_t)h * a.n_splits + split) * (hs + 2);
+            po[2 * tid] = r0; po[2 * tid + 1] = r1;
+            if (tid == 0) { po[hs] = (t1 > t0) ? m : -FLT_MAX; po[hs + 1] = (t1 > t0) ? l : 0.0f; }
+        }
+    }
+}
+
+// grid = n_heads, block = 128: merge the per-split (max, sum, unnormalised output) triples
+__global__ void attn_combine_kernel(const float *scratch, float *out, uint32_t hs, uint32_t n_splits) {
+    const uint32_t h = blockIdx.x;
+    const float *base = scratch + (size_t)h * n_splits * (hs + 2);
+    float M = -FLT_MAX;
+    for (uint32_t s = 0; s < n_splits; ++s) M = fmaxf(M, base[(size_t)s * (hs + 2) + hs]);
+    float L = 0.0f;
+    for (uint32_t s = 0; s < n_splits; ++s) {
+        const float ms = base[(size_t)s * (hs + 2) + hs], ls = base[(size_t)s * (hs + 2) + hs + 1];
+        L += ls > 0.0f ? expf(ms - M) * ls : 0.0f;
+    }
+    for (uint32_t e = threadIdx.x; e < hs; e += blockDim.x) {
+        float acc = 0.0f;
+        for (uint32_t s = 0; s < n_splits; ++s) {
+            const float ms = base[(size_t)s * (hs + 2) + hs], ls = base[(size_t)s * (hs + 2) + hs + 1];
+            if (ls > 0.0f) acc = fmaf(expf(ms - M), base[(size_t)s * (hs + 2) + e], acc);
+        }
+        out[(size_t)h * hs + e] = acc / L;
+    }
+}
+
+}  // namespace
+
+size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n_splits) {
+    return n_splits > 1 ? (size_t)n_heads * n_splits * (head_size + 2) : 0;
+}
+
+hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
+    if (a.head_size > MAX_HS || a.head_size % 2 || a.head_size / 2 > ATT_THREADS || a.n_splits == 0) return hipErrorInvalidValue;
+    const uint32_t max_split_len = (a.seq_len + a.n_splits - 1) / a.n_splits;
+    const size_t smem = (size_t)max_split_len * sizeof(float);
+    if (smem > 48 * 1024) return hipErrorInvalidValue;
+    dim3 grid(a.n_heads, a.n_splits);
+    if (a.kv_f16) attn_kernel<true><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
+    else attn_kernel<false><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (a.n_splits > 1) {
+        attn_combine_kernel<<<a.n_heads, 128, 0, s>>>(a.scratch, a.out, a.head_size, a.n_splits);
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+}  // namespace slai

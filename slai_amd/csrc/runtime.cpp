@@ -1,0 +1,448 @@
+// C-ABI runtime of libslai_hip: context, buffers, quantized matrices, the LlmContext op
+// facade (crates/slai/src/context.rs) and HIP-graph capture.  Declarations and the reference
+// interfaces they replace are in include/slai_hip.h.
+#include "common.h"
+#include "quant_formats.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+namespace slai {
+
+int set_error(slai_ctx *ctx, int code, const std::string &msg) {
+    if (ctx) ctx->err = msg;
+    return code;
+}
+int hip_fail(slai_ctx *ctx, hipError_t e, const char *what) {
+    return set_error(ctx, SLAI_E_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+static int env_int(const char *name, int dflt) {
+    const char *v = getenv(name);
+    return v && *v ? atoi(v) : dflt;
+}
+
+static bool view_is_vector(const slai_view &v) { return v.size[1] == 1 && v.size[2] == 1 && v.size[3] == 1; }
+static uint32_t view_len(const slai_view &v) { return v.size[0] * v.size[1] * v.size[2] * v.size[3]; }
+
+// A view used as a flat vector: either a genuine vector, or any contiguous tensor.
+static bool as_vec(const slai_view &v, VecView *out) {
+    if (!v.buf || v.buf->dtype != SLAI_DT_F32) return false;
+    uint32_t n = view_len(v), stride;
+    if (view_is_vector(v)) stride = v.stride[0] ? v.stride[0] : 1;
+    else {
+        // contiguous column-major or row-major block
+        bool cm = v.stride[0] == 1 && (v.size[1] == 1 || v.stride[1] == v.size[0]);
+        bool rm = v.stride[1] == 1 && (v.size[0] == 1 || v.stride[0] == v.size[1]);
+        if (!(cm || rm) || v.size[2] != 1 || v.size[3] != 1) return false;
+        stride = 1;
+    }
+    if (n == 0) return false;
+    size_t last = v.offset + (size_t)(n - 1) * stride;
+    if ((last + 1) * sizeof(float) > v.buf->bytes) return false;
+    out->p = reinterpret_cast<float *>(v.buf->dptr) + v.offset;
+    out->n = n;
+    out->stride = stride;
+    return true;
+}
+
+static bool as_view4(const slai_view &v, View4 *out) {
+    if (!v.buf || v.buf->dtype != SLAI_DT_F32) return false;
+    size_t last = v.offset;
+    for (int d = 0; d < 4; ++d) {
+        if (v.size[d] == 0) return false;
+        last += (size_t)(v.size[d] - 1) * v.stride[d];
+    }
+    if ((last + 1) * sizeof(float) > v.buf->bytes) return false;
+    out->p = reinterpret_cast<float *>(v.buf->dptr) + v.offset;
+    for (int d = 0; d < 4; ++d) { out->size[d] = v.size[d]; out->stride[d] = v.stride[d]; }
+    return true;
+}
+
+}  // namespace slai
+
+using namespace slai;
+
+// ---- context ------------------------------------------------------------------
+SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
+    if (!out) return SLAI_E_ARG;
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) return SLAI_E_HIP;
+    if (hipSetDevice(device) != hipSuccess) return SLAI_E_HIP;
+    slai_ctx *ctx = new slai_ctx();
+    ctx->device = device;
+    if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) { delete ctx; return SLAI_E_HIP; }
+    ctx->gemv_rows_per_wg = env_int("SLAI_GEMV_ROWS_PER_WG", 8);
+    ctx->gemv_max_threads = env_int("SLAI_GEMV_MAX_THREADS", 512);
+    ctx->attn_splits = env_int("SLAI_ATTN_SPLITS", 0);
+    *out = ctx;
+    return SLAI_OK;
+}
+
+SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
+    if (!ctx) return;
+    hipSetDevice(ctx->device);
+    hipStreamSynchronize(ctx->stream);
+    if (ctx->attn_scratch) hipFree(ctx->attn_scratch);
+    hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+SLAI_EXPORT const char *slai_last_error(slai_ctx *ctx) { return ctx ? ctx->err.c_str() : "null context"; }
+SLAI_EXPORT void *slai_ctx_stream(slai_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+SLAI_EXPORT int slai_begin_submission(slai_ctx *ctx) { return ctx ? SLAI_OK : SLAI_E_ARG; }
+SLAI_EXPORT int slai_submit(slai_ctx *ctx) { return ctx ? SLAI_OK : SLAI_E_ARG; }
+SLAI_EXPORT int slai_synchronize(slai_ctx *ctx) {
+    if (!ctx) return SLAI_E_ARG;
+    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return SLAI_OK;
+}
+
+// ---- buffers --------------------------------------------------------------------
+SLAI_EXPORT int slai_buffer_create(slai_ctx *ctx, size_t bytes, int dtype, uint32_t usage, slai_buffer **out) {
+    if (!ctx || !out) return SLAI_E_ARG;
+    *out = nullptr;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_buffer_create during graph capture");
+    if (dtype < SLAI_DT_F32 || dtype > SLAI_DT_I32) return set_error(ctx, SLAI_E_ARG, "bad dtype");
+    slai_buffer *b = new slai_buffer();
+    b->bytes = bytes; b->dtype = dtype; b->usage = usage;
+    size_t alloc = bytes ? bytes : 16;
+    hipError_t e = hipMalloc(&b->dptr, alloc);
+    if (e == hipSuccess) e = hipMemsetAsync(b->dptr, 0, alloc, ctx->stream);
+    if (e == hipSuccess && (usage & SLAI_USAGE_MAP_READ)) e = hipHostMalloc(&b->host_staging, alloc, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        if (b->dptr) hipFree(b->dptr);
+        delete b;
+        return hip_fail(ctx, e, "slai_buffer_create");
+    }
+    *out = b;
+    return SLAI_OK;
+}
+
+SLAI_EXPORT void slai_buffer_destroy(slai_ctx *ctx, slai_buffer *b) {
+    if (!b) return;
+    if (ctx) hipStreamSynchronize(ctx->stream);
+    if (b->dptr) hipFree(b->dptr);
+    if (b->host_staging) hipHostFree(b->host_staging);
+    delete b;
+}
+SLAI_EXPORT size_t slai_buffer_size(const slai_buffer *b) { return b ? b->bytes : 0; }
+SLAI_EXPORT void *slai_buffer_device_ptr(const slai_buffer *b) { return b ? b->dptr : nullptr; }
+
+SLAI_EXPORT int slai_write_buffer(slai_ctx *ctx, slai_buffer *b, size_t offset, const void *src, size_t bytes) {
+    if (!ctx || !b || (!src && bytes)) return SLAI_E_ARG;
+    if (offset + bytes > b->bytes) return set_error(ctx, SLAI_E_SHAPE, "slai_write_buffer: out of range");
+    if (!bytes) return SLAI_OK;
+    SLAI_HIP_TRY(ctx, hipMemcpyAsync((char *)b->dptr + offset, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    // pageable source: the copy must have consumed `src` before the caller reuses it
+    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_read_buffer(slai_ctx *ctx, const slai_buffer *b, size_t offset, void *dst, size_t bytes) {
+    if (!ctx || !b || (!dst && bytes)) return SLAI_E_ARG;
+    if (offset + bytes > b->bytes) return set_error(ctx, SLAI_E_SHAPE, "slai_read_buffer: out of range");
+    if (!bytes) return SLAI_OK;
+    if (b->host_staging) {
+        SLAI_HIP_TRY(ctx, hipMemcpyAsync((char *)b->host_staging + offset, (const char *)b->dptr + offset, bytes,
+                                         hipMemcpyDeviceToHost, ctx->stream));
+        SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        memcpy(dst, (const char *)b->host_staging + offset, bytes);
+    } else {
+        SLAI_HIP_TRY(ctx, hipMemcpyAsync(dst, (const char *)b->dptr + offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
+        SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    }
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_copy_buffer(slai_ctx *ctx, slai_buffer *dst, size_t dst_offset, const slai_buffer *src,
+                                 size_t src_offset, size_t bytes) {
+    if (!ctx || !dst || !src) return SLAI_E_ARG;
+    if (dst_offset + bytes > dst->bytes || src_offset + bytes > src->bytes)
+        return set_error(ctx, SLAI_E_SHAPE, "slai_copy_buffer: out of range");
+    if (!bytes) return SLAI_OK;
+    SLAI_HIP_TRY(ctx, hipMemcpyAsync((char *)dst->dptr + dst_offset, (const char *)src->dptr + src_offset, bytes,
+                                     hipMemcpyDeviceToDevice, ctx->stream));
+    return SLAI_OK;
+}
+
+// ---- quantized matrices ---------------------------------------------------------
+SLAI_EXPORT int slai_qmat_create(slai_ctx *ctx, uint32_t ggml_type, uint32_t nrows, uint32_t ncols, const void *packed,
+                                 slai_qmat **out) {
+    if (!ctx || !out || !packed) return SLAI_E_ARG;
+    *out = nullptr;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_qmat_create during graph capture");
+    const int t = (int)ggml_type;
+    const int be = block_elems(t);
+    if (!be) return set_error(ctx, SLAI_E_TYPE, "slai_qmat_create: unsupported ggml type " + std::to_string(ggml_type));
+    if (nrows == 0 || ncols == 0 || ncols % be) return set_error(ctx, SLAI_E_SHAPE, "slai_qmat_create: ncols must be a multiple of the block length");
+    slai_qmat *m = new slai_qmat();
+    m->type = t; m->nrows = nrows; m->ncols = ncols; m->nb = ncols / be;
+    m->row_stride = device_row_stride(t, ncols);
+    m->bytes = m->row_stride * nrows;
+    const size_t src_bytes = gguf_row_bytes(t, ncols) * nrows;
+    uint8_t *staging = nullptr;
+    hipError_t e = hipMalloc((void **)&m->dptr, m->bytes);
+    const bool verbatim = (t == T_Q4_K || t == T_Q5_K || ((t == T_F32 || t == T_F16) && gguf_row_bytes(t, ncols) == m->row_stride));
+    if (e == hipSuccess) {
+        if (verbatim) {
+            e = hipMemcpyAsync(m->dptr, packed, src_bytes, hipMemcpyHostToDevice, ctx->stream);
+        } else {
+            e = hipMalloc((void **)&staging, src_bytes);
+            if (e == hipSuccess) e = hipMemsetAsync(m->dptr, 0, m->bytes, ctx->stream);
+            if (e == hipSuccess) e = hipMemcpyAsync(staging, packed, src_bytes, hipMemcpyHostToDevice, ctx->stream);
+            if (e == hipSuccess) e = launch_repack(ctx->stream, t, staging, m->dptr, nrows, ncols);
+        }
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (staging) hipFree(staging);
+    if (e != hipSuccess) {
+        if (m->dptr) hipFree(m->dptr);
+        delete m;
+        return hip_fail(ctx, e, "slai_qmat_create");
+    }
+    *out = m;
+    return SLAI_OK;
+}
+
+SLAI_EXPORT void slai_qmat_destroy(slai_ctx *ctx, slai_qmat *m) {
+    if (!m) return;
+    if (ctx) hipStreamSynchronize(ctx->stream);
+    if (m->dptr) hipFree(m->dptr);
+    delete m;
+}
+SLAI_EXPORT int slai_qmat_shape(const slai_qmat *m, uint32_t *nrows, uint32_t *ncols, uint32_t *ggml_type) {
+    if (!m) return SLAI_E_ARG;
+    if (nrows) *nrows = m->nrows;
+    if (ncols) *ncols = m->ncols;
+    if (ggml_type) *ggml_type = (uint32_t)m->type;
+    return SLAI_OK;
+}
+SLAI_EXPORT size_t slai_qmat_device_bytes(const slai_qmat *m) { return m ? m->bytes : 0; }
+
+SLAI_EXPORT int slai_qmat_dequantize(slai_ctx *ctx, const slai_qmat *m, uint32_t row0, uint32_t nrows, slai_view out) {
+    if (!ctx || !m || !out.buf) return SLAI_E_ARG;
+    if (row0 + nrows > m->nrows) return set_error(ctx, SLAI_E_SHAPE, "slai_qmat_dequantize: row range");
+    if (out.buf->dtype != SLAI_DT_F32) return set_error(ctx, SLAI_E_TYPE, "slai_qmat_dequantize: out must be f32");
+    if (out.size[0] != nrows || out.size[1] != m->ncols || out.stride[1] != 1 || out.stride[0] < m->ncols)
+        return set_error(ctx, SLAI_E_SHAPE, "slai_qmat_dequantize: out must be a row-major [nrows x ncols] view");
+    if (nrows == 0) return SLAI_OK;
+    size_t last = out.offset + (size_t)(nrows - 1) * out.stride[0] + m->ncols;
+    if (last * sizeof(float) > out.buf->bytes) return set_error(ctx, SLAI_E_SHAPE, "slai_qmat_dequantize: out too small");
+    SLAI_HIP_TRY(ctx, launch_dequant_rows(ctx->stream, m->type, m->dptr, m->row_stride, m->nb, row0, nrows, m->ncols,
+                                          (float *)out.buf->dptr + out.offset, out.stride[0]));
+    return SLAI_OK;
+}
+
+// ---- ops ---------------------------------------------------------------------------
+#define NEED_VEC(view, name, vv)                                                                           \
+    VecView vv;                                                                                            \
+    if (!as_vec(view, &vv)) return set_error(ctx, SLAI_E_SHAPE, std::string(__func__) + ": bad view '" name "'")
+
+SLAI_EXPORT int slai_rms_norm_assign(slai_ctx *ctx, const slai_buffer *config, slai_view out, slai_view value, slai_view weight) {
+    if (!ctx || !config) return SLAI_E_ARG;
+    if (config->bytes < sizeof(slai_rms_norm_config)) return set_error(ctx, SLAI_E_SHAPE, "slai_rms_norm_assign: config buffer too small");
+    NEED_VEC(out, "out", vo); NEED_VEC(value, "value", vv); NEED_VEC(weight, "weight", vw);
+    if (vo.n != vv.n || vw.n != vv.n) return set_error(ctx, SLAI_E_SHAPE, "slai_rms_norm_assign: length mismatch");
+    SLAI_HIP_TRY(ctx, launch_rms_norm(ctx->stream, vo, vv, vw, (const float *)config->dptr, 0.0f));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_layernorm_assign(slai_ctx *ctx, slai_view out, slai_view value, float eps) {
+    if (!ctx) return SLAI_E_ARG;
+    NEED_VEC(out, "out", vo); NEED_VEC(value, "value", vv);
+    if (vo.n != vv.n) return set_error(ctx, SLAI_E_SHAPE, "slai_layernorm_assign: length mismatch");
+    SLAI_HIP_TRY(ctx, launch_layernorm(ctx->stream, vo, vv, eps));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_matmul_quant_assign(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view v) {
+    if (!ctx || !m) return SLAI_E_ARG;
+    NEED_VEC(out, "out", vo); NEED_VEC(v, "v", vv);
+    if (vo.n != m->nrows || vv.n != m->ncols) return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_quant_assign: dimension mismatch");
+    if (vo.stride != 1 || vv.stride != 1 || (v.offset % 4) != 0)
+        return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_quant_assign: vectors must be contiguous, input offset a multiple of 4");
+    if (!gemv_supports(m->type, m->ncols)) return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_quant_assign: unsupported column count for this format");
+    GemvParams p;
+    p.nseg = 1;
+    p.seg[0].W = m->dptr; p.seg[0].row_stride = m->row_stride; p.seg[0].nrows = m->nrows; p.seg[0].out = vo.p;
+    p.ncols = m->ncols; p.nb = m->nb; p.x = vv.p; p.rows_per_wg = ctx->gemv_rows_per_wg;
+    SLAI_HIP_TRY(ctx, launch_gemv(ctx, m->type, p));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_matmul_assign(slai_ctx *ctx, slai_view out, slai_view a, slai_view b, int a_mode, int b_mode) {
+    if (!ctx) return SLAI_E_ARG;
+    View4 vo, va, vb;
+    if (!as_view4(out, &vo) || !as_view4(a, &va) || !as_view4(b, &vb)) return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_assign: bad view");
+    const uint32_t m = a_mode == SLAI_MODE_N ? va.size[0] : va.size[1], inner = a_mode == SLAI_MODE_N ? va.size[1] : va.size[0];
+    const uint32_t inner_b = b_mode == SLAI_MODE_N ? vb.size[0] : vb.size[1], n = b_mode == SLAI_MODE_N ? vb.size[1] : vb.size[0];
+    if (inner != inner_b || vo.size[0] != m || vo.size[1] != n) return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_assign: dimension mismatch");
+    for (int d = 2; d < 4; ++d)
+        if ((va.size[d] != 1 && va.size[d] != vo.size[d]) || (vb.size[d] != 1 && vb.size[d] != vo.size[d]))
+            return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_assign: batch dimension mismatch");
+    SLAI_HIP_TRY(ctx, launch_matmul_f32(ctx->stream, vo, va, vb, a_mode, b_mode));
+    return SLAI_OK;
+}
+
+static int binop(slai_ctx *ctx, int op, slai_view a, slai_view b, const char *fn) {
+    if (!ctx) return SLAI_E_ARG;
+    VecView va, vb;
+    if (!as_vec(a, &va) || !as_vec(b, &vb) || va.n != vb.n) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": bad views or length mismatch");
+    SLAI_HIP_TRY(ctx, launch_binop(ctx->stream, op, va, vb));
+    return SLAI_OK;
+}
+SLAI_EXPORT int slai_add_assign(slai_ctx *ctx, slai_view a, slai_view b) { return binop(ctx, 0, a, b, "slai_add_assign"); }
+SLAI_EXPORT int slai_mul_assign(slai_ctx *ctx, slai_view a, slai_view b) { return binop(ctx, 1, a, b, "slai_mul_assign"); }
+SLAI_EXPORT int slai_copy(slai_ctx *ctx, slai_view in, slai_view out) { return binop(ctx, 2, out, in, "slai_copy"); }
+
+SLAI_EXPORT int slai_rope(slai_ctx *ctx, int variant, const slai_buffer *config, slai_view in_out_q, slai_view in_out_k) {
+    if (!ctx || !config) return SLAI_E_ARG;
+    if (config->bytes < sizeof(slai_rope_config)) return set_error(ctx, SLAI_E_SHAPE, "slai_rope: config buffer too small");
+    if (variant != SLAI_ROPE_ORIGINAL && variant != SLAI_ROPE_NEOX) return set_error(ctx, SLAI_E_ARG, "slai_rope: bad variant");
+    NEED_VEC(in_out_q, "q", vq); NEED_VEC(in_out_k, "k", vk);
+    // ops/rope.rs:58-64
+    if (vq.n % 2 || vk.n % 2 || vq.n < vk.n) return set_error(ctx, SLAI_E_SHAPE, "slai_rope: q and k must have even lengths with len(q) >= len(k)");
+    SLAI_HIP_TRY(ctx, launch_rope(ctx->stream, variant, (const slai_rope_config *)config->dptr, vq, vk));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_silu(slai_ctx *ctx, slai_view h1, slai_view h2) {
+    if (!ctx) return SLAI_E_ARG;
+    NEED_VEC(h1, "h1", va); NEED_VEC(h2, "h2", vb);
+    if (va.n != vb.n) return set_error(ctx, SLAI_E_SHAPE, "slai_silu: length mismatch");
+    SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, va, vb));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_gelu_inplace(slai_ctx *ctx, slai_view x) {
+    if (!ctx) return SLAI_E_ARG;
+    NEED_VEC(x, "x", va);
+    SLAI_HIP_TRY(ctx, launch_gelu(ctx->stream, va));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_attn_mask(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_buffer *attn) {
+    if (!ctx || !params || !params_gpu || !attn) return SLAI_E_ARG;
+    if (params_gpu->bytes < sizeof(slai_attn_params)) return set_error(ctx, SLAI_E_SHAPE, "slai_attn_mask: params buffer too small");
+    const uint32_t rounded_pos = (params->pos + 1 + 3) / 4 * 4;          // context.rs:773
+    const size_t n = (size_t)params->n_heads * rounded_pos;             // context.rs:783
+    if (n * sizeof(float) > attn->bytes) return set_error(ctx, SLAI_E_SHAPE, "slai_attn_mask: attn buffer too small");
+    SLAI_HIP_TRY(ctx, launch_attn_mask(ctx->stream, (const slai_attn_params *)params_gpu->dptr, (float *)attn->dptr, (uint32_t)n));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_softmax_cols(slai_ctx *ctx, slai_view m) {
+    if (!ctx) return SLAI_E_ARG;
+    View4 v;
+    if (!as_view4(m, &v)) return set_error(ctx, SLAI_E_SHAPE, "slai_softmax_cols: bad view");
+    if (v.size[2] > 65535 || v.size[3] > 65535) return set_error(ctx, SLAI_E_SHAPE, "slai_softmax_cols: batch too large");
+    SLAI_HIP_TRY(ctx, launch_softmax_cols(ctx->stream, v));
+    return SLAI_OK;
+}
+
+namespace slai {
+uint32_t pick_attn_splits(const slai_ctx *ctx, uint32_t n_heads, uint32_t seq_len) {
+    if (ctx->attn_splits > 0) return (uint32_t)ctx->attn_splits;
+    // enough workgroups to cover the chip, at least ~32 positions per split at full context
+    uint32_t s = (512 + n_heads - 1) / n_heads;
+    uint32_t cap = seq_len / 32 ? seq_len / 32 : 1;
+    if (s > cap) s = cap;
+    if (s > 32) s = 32;
+    return s ? s : 1;
+}
+int ensure_attn_scratch(slai_ctx *ctx, size_t floats) {
+    if (floats <= ctx->attn_scratch_floats) return SLAI_OK;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "attention scratch must be sized before graph capture");
+    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->attn_scratch) hipFree(ctx->attn_scratch);
+    ctx->attn_scratch = nullptr; ctx->attn_scratch_floats = 0;
+    SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->attn_scratch, floats * sizeof(float)));
+    ctx->attn_scratch_floats = floats;
+    return SLAI_OK;
+}
+}  // namespace slai
+
+SLAI_EXPORT int slai_attention(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q,
+                               slai_view key_cache, slai_view value_cache, slai_view att, slai_view xb) {
+    (void)att;
+    if (!ctx || !params || !params_gpu || !key_cache.buf || !value_cache.buf) return SLAI_E_ARG;
+    if (params_gpu->bytes < sizeof(slai_attn_params)) return set_error(ctx, SLAI_E_SHAPE, "slai_attention: params buffer too small");
+    NEED_VEC(q, "q", vq); NEED_VEC(xb, "xb", vx);
+    const uint32_t hs = params->head_size, nh = params->n_heads;
+    if (!params->kv_mul || nh % params->kv_mul || vq.n != nh * hs || vx.n != nh * hs || vq.stride != 1 || vx.stride != 1 ||
+        params->kv_dim != nh / params->kv_mul * hs || params->pos >= params->seq_len)
+        return set_error(ctx, SLAI_E_SHAPE, "slai_attention: inconsistent parameters");
+    const int kdt = key_cache.buf->dtype;
+    if (kdt != value_cache.buf->dtype || (kdt != SLAI_DT_F32 && kdt != SLAI_DT_F16)) return set_error(ctx, SLAI_E_TYPE, "slai_attention: caches must both be f32 or f16");
+    const size_t esz = kdt == SLAI_DT_F16 ? 2 : 4;
+    for (const slai_view *c : {&key_cache, &value_cache}) {
+        if (c->size[0] != params->kv_dim || c->size[1] != params->seq_len || c->stride[0] != 1 || c->stride[1] != params->kv_dim ||
+            (c->offset + (size_t)params->kv_dim * params->seq_len) * esz > c->buf->bytes || (c->offset % 2))
+            return set_error(ctx, SLAI_E_SHAPE, "slai_attention: caches must be [kv_dim x seq_len] column-major");
+    }
+    AttnLaunch a{};
+    a.q = vq.p;
+    a.kcache = (char *)key_cache.buf->dptr + key_cache.offset * esz;
+    a.vcache = (char *)value_cache.buf->dptr + value_cache.offset * esz;
+    a.kv_f16 = kdt == SLAI_DT_F16;
+    a.n_heads = nh; a.kv_mul = params->kv_mul; a.head_size = hs; a.kv_dim = params->kv_dim; a.seq_len = params->seq_len;
+    a.pos_ptr = &((const slai_attn_params *)params_gpu->dptr)->pos;
+    a.rope_variant = SLAI_ROPE_ORIGINAL; a.rope_base = 0.0f;
+    a.out = vx.p;
+    a.n_splits = pick_attn_splits(ctx, nh, params->seq_len);
+    int rc = ensure_attn_scratch(ctx, attention_scratch_floats(nh, hs, a.n_splits));
+    if (rc) return rc;
+    a.scratch = ctx->attn_scratch;
+    hipError_t e = launch_attention(ctx->stream, a);
+    if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "slai_attention: unsupported head size or context length");
+    SLAI_HIP_TRY(ctx, e);
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_argmax(slai_ctx *ctx, slai_view logits, slai_buffer *out_index) {
+    if (!ctx || !out_index) return SLAI_E_ARG;
+    NEED_VEC(logits, "logits", vl);
+    if (vl.stride != 1 || out_index->dtype != SLAI_DT_I32 || out_index->bytes < 4) return set_error(ctx, SLAI_E_SHAPE, "slai_argmax: contiguous logits and an I32 output are required");
+    SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, vl.p, vl.n, (int *)out_index->dptr, nullptr, nullptr, nullptr));
+    return SLAI_OK;
+}
+
+// ---- graphs ---------------------------------------------------------------------------
+SLAI_EXPORT int slai_graph_begin_capture(slai_ctx *ctx) {
+    if (!ctx) return SLAI_E_ARG;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "capture already in progress");
+    SLAI_HIP_TRY(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return SLAI_OK;
+}
+SLAI_EXPORT int slai_graph_end_capture(slai_ctx *ctx, slai_graph **out) {
+    if (!ctx || !out) return SLAI_E_ARG;
+    if (!ctx->capturing) return set_error(ctx, SLAI_E_STATE, "no capture in progress");
+    ctx->capturing = false;
+    slai_graph *g = new slai_graph();
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        if (g->graph) hipGraphDestroy(g->graph);
+        delete g;
+        return hip_fail(ctx, e, "slai_graph_end_capture");
+    }
+    *out = g;
+    return SLAI_OK;
+}
+SLAI_EXPORT int slai_graph_launch(slai_ctx *ctx, slai_graph *g) {
+    if (!ctx || !g) return SLAI_E_ARG;
+    SLAI_HIP_TRY(ctx, hipGraphLaunch(g->exec, ctx->stream));
+    return SLAI_OK;
+}
+SLAI_EXPORT void slai_graph_destroy(slai_ctx *ctx, slai_graph *g) {
+    if (!g) return;
+    if (ctx) hipStreamSynchronize(ctx->stream);
+    if (g->exec) hipGraphExecDestroy(g->exec);
+    if (g->graph) hipGraphDestroy(g->graph);
+    delete g;
+}

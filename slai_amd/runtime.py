@@ -1,0 +1,355 @@
+"""Python face of the C ABI: contexts, tensors, quantized matrices, the ``LlmContext`` op
+facade and the Llama-2 / GPT-2 model handles.
+
+Class and method names follow the reference's Rust API for this path
+(crates/slai/src/context.rs ``LlmContext``, stensor ``GpuTensor`` / ``GpuTensorView``,
+crates/slai/src/quantized_matrix.rs ``GpuQuantMatrix``, crates/slai/src/gguf.rs ``Gguf``,
+crates/slai/src/models/llama2/transformer.rs ``Llama2``), so tests read like the reference's.
+Everything executes in libslai_hip.so; nothing here computes.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _ffi
+from ._ffi import AttnParams, RmsNormConfig, RopeConfig, View
+
+_NP = {_ffi.DT_F32: np.float32, _ffi.DT_F16: np.float16, _ffi.DT_U8: np.uint8, _ffi.DT_I32: np.int32}
+STORAGE = _ffi.USAGE_STORAGE | _ffi.USAGE_COPY_DST | _ffi.USAGE_COPY_SRC
+
+
+class SlaiError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("slai error %d: %s" % (code, msg))
+        self.code = code
+
+
+class Backend:
+    """One device + stream (slang_hal ``Backend``) with its kernels loaded (``LlmOps::new``)."""
+
+    def __init__(self, device=0):
+        self.L = _ffi.lib()
+        h = C.c_void_p()
+        rc = self.L.slai_ctx_create(device, C.byref(h))
+        if rc:
+            raise SlaiError(rc, "slai_ctx_create failed (is a GPU visible?)")
+        self.h = h
+
+    def check(self, rc):
+        if rc:
+            raise SlaiError(rc, self.L.slai_last_error(self.h).decode())
+
+    def synchronize(self):
+        self.check(self.L.slai_synchronize(self.h))
+
+    def close(self):
+        if self.h:
+            self.L.slai_ctx_destroy(self.h)
+            self.h = None
+
+
+class GpuTensor:
+    """stensor ``GpuTensor<T>``: an owned device buffer with a column-major [nrows, ncols] shape."""
+
+    def __init__(self, backend, nrows, ncols=1, dtype=_ffi.DT_F32, usage=STORAGE, data=None):
+        self.b, self.nrows, self.ncols, self.dtype = backend, int(nrows), int(ncols), dtype
+        esz = np.dtype(_NP[dtype]).itemsize
+        self.nbytes = self.nrows * self.ncols * esz
+        h = C.c_void_p()
+        backend.check(backend.L.slai_buffer_create(backend.h, self.nbytes, dtype, usage, C.byref(h)))
+        self.h = h
+        if data is not None:
+            self.write(data)
+
+    @classmethod
+    def vector(cls, backend, data, usage=STORAGE):
+        data = np.ascontiguousarray(data, dtype=np.float32)
+        return cls(backend, data.size, 1, _ffi.DT_F32, usage, data)
+
+    @classmethod
+    def matrix(cls, backend, data, usage=STORAGE):
+        """data: numpy [nrows, ncols]; stored column-major like stensor's default ordering."""
+        data = np.asarray(data, dtype=np.float32)
+        return cls(backend, data.shape[0], data.shape[1], _ffi.DT_F32, usage, np.asfortranarray(data).T.copy())
+
+    @classmethod
+    def scalar(cls, backend, struct, usage=_ffi.USAGE_UNIFORM | _ffi.USAGE_COPY_DST):
+        raw = np.frombuffer(bytes(struct), dtype=np.uint8)
+        return cls(backend, raw.size, 1, _ffi.DT_U8, usage, raw)
+
+    def write(self, data, offset_bytes=0):
+        data = np.ascontiguousarray(data)
+        self.b.check(self.b.L.slai_write_buffer(self.b.h, self.h, offset_bytes, data.ctypes.data, data.nbytes))
+
+    def write_struct(self, struct):
+        raw = np.frombuffer(bytes(struct), dtype=np.uint8)
+        self.write(raw)
+
+    def read(self):
+        out = np.empty(self.nrows * self.ncols, dtype=_NP[self.dtype])
+        self.b.check(self.b.L.slai_read_buffer(self.b.h, self.h, 0, out.ctypes.data, out.nbytes))
+        return out
+
+    def read_matrix(self):
+        return self.read().reshape(self.ncols, self.nrows).T
+
+    def view(self, offset=0, size=None, stride=None):
+        n, m = self.nrows, self.ncols
+        size = size or (n, m, 1, 1)
+        stride = stride or (1, n, n * m, n * m)
+        size = tuple(size) + (1,) * (4 - len(size))
+        stride = tuple(stride) + (stride[-1],) * (4 - len(stride))
+        return View(self.h, offset, (C.c_uint32 * 4)(*size), (C.c_uint32 * 4)(*stride))
+
+    def as_view(self):
+        return self.view()
+
+    def column(self, i):
+        return self.view(i * self.nrows, (self.nrows, 1, 1, 1), (1, self.nrows, self.nrows, self.nrows))
+
+    def rows(self, start, n):
+        return self.view(start, (n, 1, 1, 1), (1, n, n, n))
+
+    def destroy(self):
+        if self.h:
+            self.b.L.slai_buffer_destroy(self.b.h, self.h)
+            self.h = None
+
+
+def _v(t):
+    return t if isinstance(t, View) else t.as_view()
+
+
+class GpuQuantMatrix:
+    """crates/slai/src/quantized_matrix.rs ``GpuQuantMatrix``: packed GGUF rows resident on the device."""
+
+    def __init__(self, backend, ggml_type, nrows, ncols, packed):
+        self.b = backend
+        packed = np.ascontiguousarray(packed).view(np.uint8).reshape(-1)
+        h = C.c_void_p()
+        backend.check(backend.L.slai_qmat_create(backend.h, ggml_type, nrows, ncols, packed.ctypes.data, C.byref(h)))
+        self.h, self.ggml_type, self.nrows, self.ncols = h, ggml_type, nrows, ncols
+
+    def shape(self):
+        r, c, t = C.c_uint32(), C.c_uint32(), C.c_uint32()
+        self.b.check(self.b.L.slai_qmat_shape(self.h, C.byref(r), C.byref(c), C.byref(t)))
+        return r.value, c.value, t.value
+
+    def device_bytes(self):
+        return self.b.L.slai_qmat_device_bytes(self.h)
+
+    def dequantize(self, row0=0, nrows=None):
+        """``GgufTensorData::dequantize`` evaluated on the device; returns numpy [nrows, ncols]."""
+        nrows = self.nrows - row0 if nrows is None else nrows
+        out = GpuTensor(self.b, nrows * self.ncols)
+        v = out.view(0, (nrows, self.ncols, 1, 1), (self.ncols, 1, nrows * self.ncols, nrows * self.ncols))
+        self.b.check(self.b.L.slai_qmat_dequantize(self.b.h, self.h, row0, nrows, v))
+        res = out.read().reshape(nrows, self.ncols)
+        out.destroy()
+        return res
+
+    def destroy(self):
+        if self.h:
+            self.b.L.slai_qmat_destroy(self.b.h, self.h)
+            self.h = None
+
+
+class LlmContext:
+    """crates/slai/src/context.rs ``LlmContext``: same method names and argument order (out first)."""
+
+    def __init__(self, backend):
+        self.backend = backend
+        self.L, self.h = backend.L, backend.h
+
+    def begin_submission(self):
+        self.backend.check(self.L.slai_begin_submission(self.h))
+
+    def submit(self):
+        self.backend.check(self.L.slai_submit(self.h))
+
+    def rms_norm_assign(self, config, out, value, weight):
+        self.backend.check(self.L.slai_rms_norm_assign(self.h, config.h, _v(out), _v(value), _v(weight)))
+
+    def layernorm_assign(self, out, value, eps=1e-5):
+        self.backend.check(self.L.slai_layernorm_assign(self.h, _v(out), _v(value), eps))
+
+    def matmul_quant_assign(self, out, a, b):
+        self.backend.check(self.L.slai_matmul_quant_assign(self.h, _v(out), a.h, _v(b)))
+
+    def matmul_assign(self, out, a, b, a_mode, b_mode):
+        self.backend.check(self.L.slai_matmul_assign(self.h, _v(out), _v(a), _v(b), a_mode, b_mode))
+
+    def add_assign(self, in_out_a, b):
+        self.backend.check(self.L.slai_add_assign(self.h, _v(in_out_a), _v(b)))
+
+    def mul_assign(self, in_out_a, b):
+        self.backend.check(self.L.slai_mul_assign(self.h, _v(in_out_a), _v(b)))
+
+    def copy(self, in_, out):
+        self.backend.check(self.L.slai_copy(self.h, _v(in_), _v(out)))
+
+    def rope(self, variant, config, in_out_q, in_out_k):
+        self.backend.check(self.L.slai_rope(self.h, variant, config.h, _v(in_out_q), _v(in_out_k)))
+
+    def silu(self, in_out_h1, in_h2):
+        self.backend.check(self.L.slai_silu(self.h, _v(in_out_h1), _v(in_h2)))
+
+    def gelu_inplace(self, x):
+        self.backend.check(self.L.slai_gelu_inplace(self.h, _v(x)))
+
+    def attn_mask(self, params, params_gpu, attn):
+        self.backend.check(self.L.slai_attn_mask(self.h, C.byref(params), params_gpu.h, attn.h))
+
+    def softmax_cols(self, in_out_mat):
+        self.backend.check(self.L.slai_softmax_cols(self.h, _v(in_out_mat)))
+
+    def attention(self, params, params_gpu, q, key_cache, value_cache, att, xb):
+        """``BatchedMultiqueryAttention::launch`` (ops/batched_multiquery_attention.rs:32-100)."""
+        self.backend.check(self.L.slai_attention(self.h, C.byref(params), params_gpu.h, _v(q), _v(key_cache), _v(value_cache),
+                                                 _v(att), _v(xb)))
+
+    def argmax(self, logits, out_index):
+        self.backend.check(self.L.slai_argmax(self.h, _v(logits), out_index.h))
+
+
+class Gguf:
+    """crates/slai/src/gguf.rs ``Gguf::from_bytes``; keeps the bytes alive for the handle."""
+
+    def __init__(self, data):
+        self.L = _ffi.lib()
+        self.data = np.ascontiguousarray(data, dtype=np.uint8)
+        h = C.c_void_p()
+        err = C.create_string_buffer(512)
+        rc = self.L.slai_gguf_parse(self.data.ctypes.data, self.data.size, C.byref(h), err, 512)
+        if rc:
+            raise SlaiError(rc, err.value.decode(errors="replace"))
+        self.h = h
+
+    @property
+    def version(self):
+        return self.L.slai_gguf_version(self.h)
+
+    def tensors(self):
+        out = {}
+        for i in range(self.L.slai_gguf_tensor_count(self.h)):
+            name, dims, t, off = C.c_char_p(), (C.c_uint64 * 4)(), C.c_uint32(), C.c_uint64()
+            self.L.slai_gguf_tensor_info(self.h, i, C.byref(name), C.byref(dims), C.byref(t), C.byref(off))
+            out[name.value.decode()] = dict(dims=list(dims), type=t.value, offset=off.value)
+        return out
+
+    def meta_u32(self, key):
+        v = C.c_uint32()
+        rc = self.L.slai_gguf_meta_u32(self.h, key.encode(), C.byref(v))
+        if rc:
+            raise SlaiError(rc, "metadata u32 '%s'" % key)
+        return v.value
+
+    def meta_f32(self, key):
+        v = C.c_float()
+        rc = self.L.slai_gguf_meta_f32(self.h, key.encode(), C.byref(v))
+        if rc:
+            raise SlaiError(rc, "metadata f32 '%s'" % key)
+        return v.value
+
+    def meta_str(self, key):
+        v = C.c_char_p()
+        rc = self.L.slai_gguf_meta_str(self.h, key.encode(), C.byref(v))
+        if rc:
+            raise SlaiError(rc, "metadata string '%s'" % key)
+        return v.value.decode()
+
+    def meta_array_len(self, key):
+        v = C.c_uint64()
+        rc = self.L.slai_gguf_meta_array_len(self.h, key.encode(), C.byref(v))
+        if rc:
+            raise SlaiError(rc, "metadata array '%s'" % key)
+        return v.value
+
+    def to_gpu_matrix(self, backend, name):
+        h = C.c_void_p()
+        backend.check(self.L.slai_gguf_tensor_to_qmat(backend.h, self.h, name.encode(), C.byref(h)))
+        m = GpuQuantMatrix.__new__(GpuQuantMatrix)
+        m.b, m.h = backend, h
+        m.nrows, m.ncols, m.ggml_type = m.shape()
+        return m
+
+    def close(self):
+        if self.h:
+            self.L.slai_gguf_free(self.h)
+            self.h = None
+
+
+class Llama2:
+    """``ChatLlama2`` without the tokenizer: config + weights + state + the per-token driver."""
+
+    def __init__(self, backend, gguf, model_type=_ffi.MODEL_LLAMA, kv_dtype=_ffi.KV_F32):
+        self.b = backend
+        h = C.c_void_p()
+        backend.check(backend.L.slai_llama2_from_gguf(backend.h, gguf.h, model_type, kv_dtype, C.byref(h)))
+        self.h = h
+        cfg = _ffi.Llama2Config()
+        backend.check(backend.L.slai_llama2_get_config(h, C.byref(cfg)))
+        self.config = cfg
+
+    def weight_bytes(self):
+        return self.b.L.slai_llama2_weight_bytes(self.h)
+
+    def forward_logits(self, pos, token, fused=True):
+        out = np.empty(self.config.vocab_size, dtype=np.float32)
+        self.b.check(self.b.L.slai_llama2_forward_logits(self.h, pos, token, 1 if fused else 0, out.ctypes.data))
+        return out
+
+    def generate(self, prompt, n_steps, start_pos=0):
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        out = np.zeros(n_steps, dtype=np.int32)
+        ms = C.c_float()
+        self.b.check(self.b.L.slai_llama2_generate(self.h, prompt.ctypes.data, prompt.size, start_pos, n_steps, out.ctypes.data, C.byref(ms)))
+        return out, ms.value
+
+    def kv_buffers(self, layer):
+        k, v = C.c_void_p(), C.c_void_p()
+        self.b.check(self.b.L.slai_llama2_kv_buffers(self.h, layer, C.byref(k), C.byref(v)))
+        return k, v
+
+    def write_kv(self, layer, k, v):
+        """Fills positions [0, n) of layer `layer`'s caches from [n, kv_dim] arrays (cache dtype)."""
+        kb, vb = self.kv_buffers(layer)
+        for buf, arr in ((kb, k), (vb, v)):
+            arr = np.ascontiguousarray(arr)
+            self.b.check(self.b.L.slai_write_buffer(self.b.h, buf, 0, arr.ctypes.data, arr.nbytes))
+
+    def destroy(self):
+        if self.h:
+            self.b.L.slai_llama2_destroy(self.h)
+            self.h = None
+
+
+class Gpt2:
+    def __init__(self, backend, gguf, kv_dtype=_ffi.KV_F32):
+        self.b = backend
+        h = C.c_void_p()
+        backend.check(backend.L.slai_gpt2_from_gguf(backend.h, gguf.h, kv_dtype, C.byref(h)))
+        self.h = h
+        p = _ffi.Gpt2Params()
+        backend.check(backend.L.slai_gpt2_get_params(h, C.byref(p)))
+        self.params = p
+
+    def weight_bytes(self):
+        return self.b.L.slai_gpt2_weight_bytes(self.h)
+
+    def forward_logits(self, pos, token):
+        out = np.empty(self.params.n_vocab, dtype=np.float32)
+        self.b.check(self.b.L.slai_gpt2_forward_logits(self.h, pos, token, out.ctypes.data))
+        return out
+
+    def generate(self, prompt, n_steps, start_pos=0):
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        out = np.zeros(n_steps, dtype=np.int32)
+        ms = C.c_float()
+        self.b.check(self.b.L.slai_gpt2_generate(self.h, prompt.ctypes.data, prompt.size, start_pos, n_steps, out.ctypes.data, C.byref(ms)))
+        return out, ms.value
+
+    def destroy(self):
+        if self.h:
+            self.b.L.slai_gpt2_destroy(self.h)
+            self.h = None

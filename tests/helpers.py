@@ -15,6 +15,7 @@ class OracleGguf:
 
     def __init__(self, data):
         self.L = oracle.load()
+        self.L.slo_set_threads(min(8, os.cpu_count() or 1))   # row-parallel GEMV: same bits, less waiting
         self.data = np.ascontiguousarray(data, dtype=np.uint8)
         err = C.c_int(0)
         self.h = self.L.slo_gguf_parse(self.data.ctypes.data, self.data.size, C.byref(err))

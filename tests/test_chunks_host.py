@@ -1,0 +1,91 @@
+"""CPU checks of the device-side layout and lane-chunk decoders (slai_amd/csrc/quant_formats.h),
+built for the host: repack + element dequantisation must reproduce the oracle bit for bit, and
+the per-chunk dot products must add up to W.x."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from helpers import random_blocks
+from slai_amd import synth
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+TYPES = [0, 1, 2, 8, 12, 13, 14]
+
+
+@pytest.fixture(scope="module")
+def cc(tmp_path_factory):
+    out = str(tmp_path_factory.mktemp("cc") / "libchunk_check.so")
+    subprocess.check_call(["g++", "-O1", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+                           "-I", os.path.join(ROOT, "slai_amd", "csrc"),
+                           os.path.join(HERE, "native", "chunk_check.cpp"), "-o", out])
+    L = C.CDLL(out)
+    L.cc_row_stride.restype = C.c_size_t
+    L.cc_row_stride.argtypes = [C.c_int, C.c_uint32]
+    L.cc_repack.argtypes = [C.c_int, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
+    L.cc_dequant.argtypes = [C.c_int, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
+    L.cc_gemv.argtypes = [C.c_int, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+    L.cc_cover.restype = C.c_uint32
+    L.cc_cover.argtypes = [C.c_int, C.c_uint32]
+    L.cc_encode_f16.restype = C.c_uint16
+    L.cc_encode_f16.argtypes = [C.c_float]
+    L.cc_decode_f16.restype = C.c_float
+    L.cc_decode_f16.argtypes = [C.c_uint16]
+    return L
+
+
+def repack(cc, t, raw, nrows, ncols):
+    dev = np.zeros(nrows * cc.cc_row_stride(t, ncols), np.uint8)
+    cc.cc_repack(t, raw.ctypes.data, nrows, ncols, dev.ctypes.data)
+    return dev
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("ncols", [256, 768, 2816])
+def test_repack_dequant_bit_exact(cc, oracle_lib, t, ncols):
+    nrows = 5
+    be = oracle_lib.slo_block_elems(t)
+    raw = random_blocks(t, nrows * ncols // be, seed=7 * t + ncols)
+    ref = np.empty(nrows * ncols, np.float32)
+    assert oracle_lib.slo_dequantize(t, raw.ctypes.data, nrows * ncols, ref.ctypes.data) == 0
+    dev = repack(cc, t, raw, nrows, ncols)
+    got = np.empty(nrows * ncols, np.float32)
+    cc.cc_dequant(t, dev.ctypes.data, nrows, ncols, got.ctypes.data)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("ncols", [256, 2816, 11008])
+def test_chunk_column_cover(cc, t, ncols):
+    assert cc.cc_cover(t, ncols) == ncols
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_chunk_dots_sum_to_gemv(cc, oracle_lib, t):
+    nrows, ncols = 9, 1280
+    x = synth.normal(50 + t, nrows * ncols, 0.02).reshape(nrows, ncols)
+    raw = synth.quantize(t, x)
+    w = np.empty(nrows * ncols, np.float32)
+    oracle_lib.slo_dequantize(t, raw.ctypes.data, nrows * ncols, w.ctypes.data)
+    v = synth.normal(99, ncols, 1.0)
+    ref = w.reshape(nrows, ncols).astype(np.float64) @ v.astype(np.float64)
+    dev = repack(cc, t, raw, nrows, ncols)
+    got = np.empty(nrows, np.float32)
+    assert cc.cc_gemv(t, dev.ctypes.data, nrows, ncols, v.ctypes.data, got.ctypes.data) == 0
+    scale = np.abs(w.reshape(nrows, ncols)).astype(np.float64) @ np.abs(v).astype(np.float64)
+    assert np.all(np.abs(got - ref) <= 2e-5 * scale), np.abs(got - ref) / scale
+
+
+def test_f16_codec_host_side(cc):
+    u = np.arange(65536, dtype=np.uint16)
+    ref = u.view(np.float16).astype(np.float32)
+    got = np.array([cc.cc_decode_f16(int(h)) for h in u[::7]], np.float32)
+    r = ref[::7]
+    nan = np.isnan(r)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(got[~nan].view(np.uint32), r[~nan].view(np.uint32))
+    vals = np.random.Generator(np.random.PCG64(3)).normal(0, 1, 5000).astype(np.float32)
+    enc = np.array([cc.cc_encode_f16(float(v)) for v in vals], np.uint16)
+    assert np.array_equal(enc, vals.astype(np.float16).view(np.uint16))

@@ -1,0 +1,174 @@
+"""GPU parity of the LlmContext ops against the oracle.  LEN 1757 and the tolerances follow the
+reference's own op tests (ops/silu.rs:97-131 1e-5, ops/softmax.rs:98-131 1e-7, ops/rope.rs:160-228
+1e-5, ops/rms_norm.rs:117-168 1e-4, ops/layernorm.rs:150-190 1e-5, ops/unary.rs:293-408 1e-5)."""
+import numpy as np
+import pytest
+
+from gpu_common import backend, rel_err  # noqa: F401
+from slai_amd import _ffi
+from slai_amd._ffi import AttnParams, RmsNormConfig, RopeConfig
+
+pytestmark = pytest.mark.gpu
+LEN = 1757
+
+
+def rnd(seed, n, scale=1.0):
+    return np.random.Generator(np.random.PCG64(seed)).normal(0, scale, n).astype(np.float32)
+
+
+def uni(seed, n):
+    return np.random.Generator(np.random.PCG64(seed)).random(n, dtype=np.float32)   # DVector::new_random: U[0,1)
+
+
+def test_rms_norm(backend, oracle_lib):
+    from slai_amd.runtime import GpuTensor, LlmContext
+    for n, eps in ((LEN, 1e-5), (4096, 1e-6), (288, 1e-5)):
+        v, w = uni(1, n), uni(2, n)
+        ref = np.empty(n, np.float32)
+        oracle_lib.slo_rms_norm(ref.ctypes.data, v.ctypes.data, w.ctypes.data, n, eps)
+        cfg = GpuTensor.scalar(backend, RmsNormConfig(eps, (0, 0, 0)))
+        gv, gw, go = GpuTensor.vector(backend, v), GpuTensor.vector(backend, w), GpuTensor(backend, n)
+        LlmContext(backend).rms_norm_assign(cfg, go, gv, gw)
+        np.testing.assert_allclose(go.read(), ref, rtol=1e-4, atol=1e-6)
+        for o in (cfg, gv, gw, go):
+            o.destroy()
+
+
+def test_layernorm_and_gelu_and_silu(backend, oracle_lib):
+    from slai_amd.runtime import GpuTensor, LlmContext
+    ctxt = LlmContext(backend)
+    v = rnd(3, LEN, 2.0)
+    ref = np.empty(LEN, np.float32)
+    oracle_lib.slo_layernorm(ref.ctypes.data, v.ctypes.data, LEN, 1e-5)
+    gv, go = GpuTensor.vector(backend, v), GpuTensor(backend, LEN)
+    ctxt.layernorm_assign(go, gv, 1e-5)
+    np.testing.assert_allclose(go.read(), ref, rtol=1e-5, atol=1e-6)
+    g = v.copy(); oracle_lib.slo_gelu_n(g.ctypes.data, LEN)
+    ctxt.gelu_inplace(gv)
+    np.testing.assert_allclose(gv.read(), g, rtol=1e-5, atol=1e-6)
+    a, b = rnd(4, LEN, 3.0), rnd(5, LEN)
+    r = a.copy(); oracle_lib.slo_silu(r.ctypes.data, b.ctypes.data, LEN)
+    ga, gb = GpuTensor.vector(backend, a), GpuTensor.vector(backend, b)
+    ctxt.silu(ga, gb)
+    np.testing.assert_allclose(ga.read(), r, rtol=1e-5, atol=1e-7)
+    for o in (gv, go, ga, gb):
+        o.destroy()
+
+
+def test_add_mul_copy(backend):
+    from slai_amd.runtime import GpuTensor, LlmContext
+    ctxt = LlmContext(backend)
+    a, b = rnd(6, LEN), rnd(7, LEN)
+    ga, gb, gc = GpuTensor.vector(backend, a), GpuTensor.vector(backend, b), GpuTensor(backend, LEN)
+    ctxt.add_assign(ga, gb)
+    assert np.array_equal(ga.read(), a + b)
+    ctxt.mul_assign(ga, gb)
+    assert np.array_equal(ga.read(), (a + b) * b)
+    ctxt.copy(gb, gc)
+    assert np.array_equal(gc.read(), b)
+    # a strided / offset destination: column 2 of a [LEN x 4] matrix
+    gm = GpuTensor(backend, LEN, 4)
+    ctxt.copy(gb, gm.column(2))
+    m = gm.read_matrix()
+    assert np.array_equal(m[:, 2], b) and not m[:, [0, 1, 3]].any()
+    for o in (ga, gb, gc, gm):
+        o.destroy()
+
+
+@pytest.mark.parametrize("variant", [_ffi.ROPE_ORIGINAL, _ffi.ROPE_NEOX])
+def test_rope(backend, oracle_lib, variant):
+    from slai_amd.runtime import GpuTensor, LlmContext
+    hs, nq, nk, pos = 128, 13, 9, 10                       # ops/rope.rs:160-170
+    dim, kv_dim = hs * nq, hs * nk
+    q, k = uni(8, dim), uni(9, kv_dim)
+    rq, rk = q.copy(), k.copy()
+    oracle_lib.slo_rope(rq.ctypes.data, rk.ctypes.data, hs, dim, kv_dim, pos, 10000.0, variant)
+    cfg = GpuTensor.scalar(backend, RopeConfig(hs, kv_dim, pos, 10000.0))
+    gq, gk = GpuTensor.vector(backend, q), GpuTensor.vector(backend, k)
+    LlmContext(backend).rope(variant, cfg, gq, gk)
+    np.testing.assert_allclose(gq.read(), rq, rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(gk.read(), rk, rtol=1e-5, atol=2e-6)
+    for o in (cfg, gq, gk):
+        o.destroy()
+
+
+def test_softmax_cols(backend, oracle_lib):
+    from slai_amd.runtime import GpuTensor, LlmContext
+    m = rnd(10, LEN * 5, 3.0).reshape(LEN, 5)
+    ref = m.copy()
+    for j in range(5):
+        col = np.ascontiguousarray(ref[:, j]); oracle_lib.slo_softmax(col.ctypes.data, LEN); ref[:, j] = col
+    gm = GpuTensor.matrix(backend, m)
+    LlmContext(backend).softmax_cols(gm)
+    np.testing.assert_allclose(gm.read_matrix(), ref, rtol=2e-6, atol=1e-7)
+    gm.destroy()
+
+
+def test_argmax_first_maximum(backend):
+    from slai_amd.runtime import GpuTensor, LlmContext
+    ctxt = LlmContext(backend)
+    idx = GpuTensor(backend, 1, 1, _ffi.DT_I32)
+    for n, seed in ((32000, 1), (50257, 2), (7, 3)):
+        v = rnd(seed, n)
+        gv = GpuTensor.vector(backend, v)
+        ctxt.argmax(gv, idx)
+        assert int(idx.read()[0]) == int(np.argmax(v))
+        gv.destroy()
+    v = np.zeros(5000, np.float32); v[[4000, 17, 2999]] = 3.0
+    gv = GpuTensor.vector(backend, v)
+    ctxt.argmax(gv, idx)
+    assert int(idx.read()[0]) == 17
+    gv.destroy(); idx.destroy()
+
+
+@pytest.mark.parametrize("cfg", [dict(n_heads=6, kv_mul=1, hs=48, seq=256, pos=37),
+                                 dict(n_heads=12, kv_mul=3, hs=64, seq=96, pos=95),
+                                 dict(n_heads=32, kv_mul=1, hs=128, seq=512, pos=300),
+                                 dict(n_heads=8, kv_mul=2, hs=128, seq=64, pos=0)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_attention_fused_and_reference_sequence(backend, oracle_lib, cfg, f16):
+    """`BatchedMultiqueryAttention::launch`: the fused op and the reference's own four-launch
+    sequence (ops/batched_multiquery_attention.rs:46-98) both against `run_cpu` (:102-156)."""
+    from slai_amd.runtime import GpuTensor, LlmContext
+    nh, kv_mul, hs, seq, pos = cfg["n_heads"], cfg["kv_mul"], cfg["hs"], cfg["seq"], cfg["pos"]
+    print("case", cfg, f16, flush=True)
+    nkv = nh // kv_mul
+    kv_dim = nkv * hs
+    q = rnd(11, nh * hs)
+    kc = rnd(12, seq * kv_dim).reshape(seq, kv_dim); vc = rnd(13, seq * kv_dim).reshape(seq, kv_dim)
+    if f16:
+        kc = kc.astype(np.float16).astype(np.float32); vc = vc.astype(np.float16).astype(np.float32)
+    att = np.zeros(seq * nh, np.float32); ref = np.empty(nh * hs, np.float32)
+    oracle_lib.slo_attention(nh, kv_mul, hs, pos, seq, kv_dim, q.ctypes.data, kc.ctypes.data, vc.ctypes.data, att.ctypes.data, ref.ctypes.data)
+    ctxt = LlmContext(backend)
+    params = AttnParams(seq, kv_dim, kv_mul, nh, hs, pos, (0, 0))
+    gparams = GpuTensor.scalar(backend, params)
+    gq = GpuTensor.vector(backend, q)
+    dt = _ffi.DT_F16 if f16 else _ffi.DT_F32
+    npdt = np.float16 if f16 else np.float32
+    gk = GpuTensor(backend, kv_dim, seq, dt, data=kc.astype(npdt)); gv = GpuTensor(backend, kv_dim, seq, dt, data=vc.astype(npdt))
+    gatt = GpuTensor(backend, seq, nh); gxb = GpuTensor(backend, nh * hs)
+    ctxt.attention(params, gparams, gq, gk, gv, gatt, gxb)
+    got = gxb.read()
+    np.testing.assert_allclose(got, ref, rtol=2e-4, atol=2e-6)
+    if not f16:
+        # the reference's sequence with its padded views
+        rp = (pos + 1 + 3) // 4 * 4
+        if rp <= seq:
+            gxb2 = GpuTensor(backend, nh * hs)
+            k_view = gk.view(0, (hs, rp, nkv, 1), (1, kv_dim, hs, hs * nkv))
+            q_view = gq.view(0, (hs, kv_mul, nkv, 1), (1, hs, hs * kv_mul, hs * nh))
+            att_view = gatt.view(0, (rp, kv_mul, nkv, 1), (1, rp, rp * kv_mul, rp * nh))
+            ctxt.matmul_assign(att_view, k_view, q_view, _ffi.MODE_T, _ffi.MODE_N)
+            ctxt.attn_mask(params, gparams, gatt)
+            ctxt.softmax_cols(gatt.view(0, (pos + 1, nh, 1, 1), (1, rp, rp * nh, rp * nh)))
+            v_view = gv.view(0, (hs, rp, nkv, 1), (1, kv_dim, hs, hs * nkv))
+            xb_view = gxb2.view(0, (hs, kv_mul, nkv, 1), (1, hs, hs * kv_mul, hs * nh))
+            ctxt.matmul_assign(xb_view, v_view, att_view, _ffi.MODE_N, _ffi.MODE_N)
+            np.testing.assert_allclose(gxb2.read(), ref, rtol=2e-4, atol=2e-6)
+            probs = gatt.read()[:rp * nh].reshape(nh, rp)
+            np.testing.assert_allclose(probs[:, :pos + 1], att.reshape(nh, seq)[:, :pos + 1], rtol=2e-4, atol=1e-7)
+            assert not probs[:, pos + 1:].any()
+            gxb2.destroy()
+    for o in (gparams, gq, gk, gv, gatt, gxb):
+        o.destroy()
