@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Decode benchmark: Llama-2-7B-shape, Q4_K_M-style weights (Q4_K; Q6_K for v-proj and output),
+fp16 KV cache, batch 1 -- BASELINE configuration 4.
+
+One "step" = one token through the whole layer stack (greedy decode loop on the device).  The
+prompt (W = --warmup positions, processed token by token like the reference) is untimed; the next
+K = --steps generated tokens are timed with HIP events on the library's stream, with inputs and
+weights resident in HBM.  Prints ONE JSON line.
+
+Also measured here:
+  * roofline: the dominant kernel (fused RMSNorm + gate/up Q4_K GEMV + SiLU, 11008x4096 x2) timed
+    alone with HIP events while rotating over enough distinct weight copies to defeat the 256 MB
+    Infinity Cache; achieved = algorithmic bytes / mean launch time, peak = 8 TB/s.
+  * cpu_baseline: the CPU oracle (a C restatement of the reference's CPU path) on the host cores,
+    on a bounded sample of the same workload (the same layer shapes at depth 2 and 4, a few
+    tokens), extrapolated to 32 layers.  A reported baseline, not the target.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+CFG = dict(dim=4096, hidden_dim=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def token_bytes(cfg, weight_bytes, pos_lo, pos_hi, kv_bytes=2):
+    """Algorithmic HBM bytes per token: packed weights + norm vectors (both in weight_bytes) +
+    KV read 2*L*(pos+1)*kv_dim*kv_bytes averaged over the timed positions + KV write."""
+    kv_dim = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
+    mean_t = (pos_lo + pos_hi) / 2.0 + 1.0
+    kv_read = 2 * cfg["n_layers"] * mean_t * kv_dim * kv_bytes
+    kv_write = 2 * cfg["n_layers"] * kv_dim * kv_bytes
+    return weight_bytes + kv_read + kv_write
+
+
+def measure_dominant_kernel(backend, reps=20):
+    """Mean launch duration of the fused gate/up GEMV (Q4_K, 11008x4096 twice) over distinct copies."""
+    import torch
+    from slai_amd import synth
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
+    dim, hid, t = CFG["dim"], CFG["hidden_dim"], 12
+    ncopies = 8                                     # 8 x 50.7 MB = 406 MB > 256 MB Infinity Cache
+    base = synth.normal_quantized(4242, t, hid, dim, 0.02)
+    rb = base.size // hid
+    mats = []
+    for i in range(2 * ncopies):
+        mats.append(GpuQuantMatrix(backend, t, hid, dim, np.roll(base.reshape(hid, rb), i + 1, axis=0)))
+    x = GpuTensor.vector(backend, synth.normal(7, dim, 1.0))
+    w = GpuTensor.vector(backend, np.ones(dim, np.float32))
+    hb = GpuTensor(backend, hid)
+    ctxt = LlmContext(backend)
+    stream = torch.cuda.ExternalStream(backend.L.slai_ctx_stream(backend.h))
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(ncopies):
+        ctxt.ffn_gate_up_silu(hb, mats[2 * i], mats[2 * i + 1], x, w, 1e-5)
+    backend.synchronize()
+    ev0.record(stream)
+    for _ in range(reps):
+        for i in range(ncopies):
+            ctxt.ffn_gate_up_silu(hb, mats[2 * i], mats[2 * i + 1], x, w, 1e-5)
+    ev1.record(stream)
+    backend.synchronize()
+    ms = ev0.elapsed_time(ev1) / (reps * ncopies)
+    algo = 2 * mats[0].device_bytes() + dim * 4 * 2 + hid * 4     # 2 packed matrices + x + norm weight + out
+    for o in mats + [x, w, hb]:
+        o.destroy()
+    return ms, algo
+
+
+def cpu_baseline(seed, n_tokens=6):
+    """Oracle decode of the same layer shapes at depth 2 and 4 (pos 64..), extrapolated to 32 layers."""
+    import oracle
+    from slai_amd import gguf_writer as gw
+    L = oracle.load()
+    threads = min(16, os.cpu_count() or 1)
+    L.slo_set_threads(threads)
+    times = {}
+    for nl in (2, 4):
+        data = gw.llama_gguf(dim=CFG["dim"], hidden_dim=CFG["hidden_dim"], n_layers=nl, n_heads=CFG["n_heads"],
+                             n_kv_heads=CFG["n_kv_heads"], vocab=CFG["vocab"], seq_len=128, wtype=12, v_type=14,
+                             out_type=14, embd_type=12, seed=seed, with_output=True, distinct_layers=2)
+        err = C.c_int(0)
+        g = L.slo_gguf_parse(data.ctypes.data, data.size, C.byref(err))
+        m = L.slo_llama2_from_gguf(g, b"llama", 1, 0, 1)
+        prompt = np.random.Generator(np.random.PCG64(seed)).integers(0, CFG["vocab"], 2).astype(np.int32)
+        out = np.zeros(n_tokens + 2, np.int32)
+        L.slo_llama2_generate(m, prompt.ctypes.data, 2, 0, 2, -1, out.ctypes.data, None)       # untimed
+        t0 = time.perf_counter()
+        seq = np.concatenate([prompt, out[:2]]).astype(np.int32)
+        L.slo_llama2_generate(m, seq.ctypes.data, seq.size, 2, n_tokens, -1, out.ctypes.data, None)
+        times[nl] = (time.perf_counter() - t0) / n_tokens
+        L.slo_llama2_free(m); L.slo_gguf_free(g)
+        del data
+    per_layer = (times[4] - times[2]) / 2.0
+    head = max(times[2] - 2 * per_layer, 0.0)
+    full = head + CFG["n_layers"] * per_layer
+    return dict(value=1.0 / full, unit="tok/s", cores=threads, kind="port",
+                sample="oracle (C restatement of models/llama2/cpu.rs) at the same layer shapes, depth 2 and 4, "
+                       "%d tokens each; per-layer %.3f s + head %.3f s extrapolated to 32 layers" % (n_tokens, per_layer, head))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--layers", type=int, default=CFG["n_layers"], help="depth (32 = the benchmark configuration)")
+    ap.add_argument("--distinct-layers", type=int, default=4)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the decode path on ONE GPU (batch-1 decode does not shard usefully); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    K, W = args.steps, max(args.warmup, 1)
+    cfg = dict(CFG, n_layers=args.layers)
+    seq_len = max(512, ((W + K + 63) // 64) * 64)
+
+    from slai_amd import _ffi
+    from slai_amd import gguf_writer as gw
+    from slai_amd.runtime import Backend, Gguf, Llama2
+
+    t0 = time.perf_counter()
+    data = gw.llama_gguf(dim=cfg["dim"], hidden_dim=cfg["hidden_dim"], n_layers=cfg["n_layers"], n_heads=cfg["n_heads"],
+                         n_kv_heads=cfg["n_kv_heads"], vocab=cfg["vocab"], seq_len=seq_len, wtype=12, v_type=14, out_type=14,
+                         embd_type=12, seed=args.seed, distinct_layers=min(args.distinct_layers, cfg["n_layers"]))
+    log("model file: %.2f GB in %.1f s" % (data.size / 1e9, time.perf_counter() - t0))
+    backend = Backend(0)
+    t0 = time.perf_counter()
+    g = Gguf(data)
+    model = Llama2(backend, g, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+    log("upload: %.1f s, weights %.3f GB" % (time.perf_counter() - t0, model.weight_bytes() / 1e9))
+
+    prompt = np.random.Generator(np.random.PCG64(args.seed)).integers(0, cfg["vocab"], W).astype(np.int32)
+    # warmup: the W prompt positions (forced tokens), untimed; the last one yields the first generated token
+    warm, _ = model.generate(prompt, W, start_pos=0)
+    seq = np.concatenate([prompt, warm[W - 1:W]]).astype(np.int32)
+    # timed: K tokens at positions W .. W+K-1
+    wall0 = time.perf_counter()
+    toks, ms = model.generate(seq, K, start_pos=W)
+    wall = time.perf_counter() - wall0
+    ms_per_step = ms / K
+    tok_s = 1000.0 / ms_per_step
+    tb = token_bytes(cfg, model.weight_bytes(), W, W + K - 1)
+    log("decode: %.3f ms/token (events), wall %.3f ms/token, %.1f tok/s, %.2f GB/token -> %.1f GB/s"
+        % (ms_per_step, wall * 1000 / K, tok_s, tb / 1e9, tb / ms_per_step / 1e6))
+    model.destroy(); g.close(); del data
+
+    roof = None
+    if not args.no_roofline:
+        kms, kalgo = measure_dominant_kernel(backend)
+        ach = kalgo / (kms * 1e-3) / 1e9
+        roof = dict(bound="hbm", kernel="gemv_kernel<Q4_K, dual> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096)",
+                    achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
+                    traffic=None, launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
+        log("dominant kernel: %.2f us/launch, %.1f GB/s" % (kms * 1000, ach))
+    backend.close()
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        cpu = cpu_baseline(args.seed)
+        log("cpu baseline: %.3f tok/s on %d threads (%.1f s)" % (cpu["value"], cpu["cores"], time.perf_counter() - t0))
+
+    out = {
+        "metric": "decode tok/s & % of HBM roofline, Llama-2-7B-shape Q4_K, batch 1",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic: seeded N(0,0.02) weights quantized with ggml's reference algorithm "
+                                "(%d layers generated, the rest are row-rotated copies in distinct memory), seeded prompt ids"
+                                % min(args.distinct_layers, cfg["n_layers"]),
+        "config": {"workload": "BASELINE config 4: Llama-2-7B-shape greedy decode, dim 4096, %d layers, 32 heads, FFN 11008, "
+                               "vocab 32000, Q4_K weights (Q6_K v-proj/output), fp16 KV, %d prompt + %d generated tokens"
+                               % (cfg["n_layers"], W, K), "batch": 1, "kv_dtype": "f16", "context": seq_len},
+        "token_bytes": int(tb), "hbm_gbs": round(tb / ms_per_step / 1e6, 1),
+        "hbm_roofline_frac": round(tb / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
+        "roofline_tok_s": round(HBM_PEAK_GBS * 1e9 / tb, 1),
+        "roofline": roof, "cpu_baseline": cpu,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
