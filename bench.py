@@ -47,7 +47,6 @@ def token_bytes(cfg, weight_bytes, pos_lo, pos_hi, kv_bytes=2):
 
 def measure_dominant_kernel(backend, reps=20):
     """Mean launch duration of the fused gate/up GEMV (Q4_K, 11008x4096 twice) over distinct copies."""
-    import torch
     from slai_amd import synth
     from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
     dim, hid, t = CFG["dim"], CFG["hidden_dim"], 12
@@ -61,18 +60,14 @@ def measure_dominant_kernel(backend, reps=20):
     w = GpuTensor.vector(backend, np.ones(dim, np.float32))
     hb = GpuTensor(backend, hid)
     ctxt = LlmContext(backend)
-    stream = torch.cuda.ExternalStream(backend.L.slai_ctx_stream(backend.h))
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for i in range(ncopies):
         ctxt.ffn_gate_up_silu(hb, mats[2 * i], mats[2 * i + 1], x, w, 1e-5)
     backend.synchronize()
-    ev0.record(stream)
+    backend.timer_begin()
     for _ in range(reps):
         for i in range(ncopies):
             ctxt.ffn_gate_up_silu(hb, mats[2 * i], mats[2 * i + 1], x, w, 1e-5)
-    ev1.record(stream)
-    backend.synchronize()
-    ms = ev0.elapsed_time(ev1) / (reps * ncopies)
+    ms = backend.timer_end() / (reps * ncopies)
     algo = 2 * mats[0].device_bytes() + dim * 4 * 2 + hid * 4     # 2 packed matrices + x + norm weight + out
     for o in mats + [x, w, hb]:
         o.destroy()

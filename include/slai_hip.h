@@ -161,6 +161,24 @@ int slai_attention(slai_ctx *ctx, const slai_attn_params *params, const slai_buf
  * on the device; out_index is a 1-element I32 buffer. */
 int slai_argmax(slai_ctx *ctx, slai_view logits, slai_buffer *out_index);
 
+/* ---- fused forms of the call sequences `Llama2::launch` issues (no single reference counterpart;
+ * each replaces the listed context.rs calls with one kernel, same results up to summation order) */
+/* rms_norm_assign(xb, x, w) + matmul_quant_assign(out, m, xb)   (transformer.rs:327-334, 368-375) */
+int slai_rms_norm_matmul_quant_assign(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view norm_weight,
+                                      float eps);
+/* rms_norm_assign + matmul_quant_assign(hb, gate) + matmul_quant_assign(hb2, up) + silu(hb, hb2)
+ * (transformer.rs:356-361); gate and up must share a format */
+int slai_ffn_gate_up_silu(slai_ctx *ctx, slai_view out_hb, const slai_qmat *gate, const slai_qmat *up, slai_view x,
+                          slai_view norm_weight, float eps);
+/* matmul_quant_assign(xb2, m, v) + add_assign(x, xb2)   (transformer.rs:352-355, 362-365) */
+int slai_matmul_quant_add_assign(slai_ctx *ctx, slai_view in_out_x, const slai_qmat *m, slai_view v);
+
+/* ---- GPU timing on the context's stream with HIP events: the role of the GPU timestamp
+ * queries bracketing a pass in crates/slai-bench/src/main.rs:198,223-241.  slai_timer_end
+ * synchronises and returns the milliseconds since the matching slai_timer_begin. */
+int slai_timer_begin(slai_ctx *ctx);
+int slai_timer_end(slai_ctx *ctx, float *elapsed_ms);
+
 /* ---- HIP graph capture of a submission (no reference counterpart: the reference
  * re-encodes ~550 dispatches per token, crates/slai-chat/src/chat_llama2.rs:179-230) */
 int slai_graph_begin_capture(slai_ctx *ctx);

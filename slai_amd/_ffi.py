@@ -71,6 +71,9 @@ SIGNATURES = {
     "slai_layernorm_assign": (i32, [vp, View, View, C.c_float]),
     "slai_matmul_quant_assign": (i32, [vp, View, vp, View]),
     "slai_matmul_assign": (i32, [vp, View, View, View, i32, i32]),
+    "slai_rms_norm_matmul_quant_assign": (i32, [vp, View, vp, View, View, C.c_float]),
+    "slai_ffn_gate_up_silu": (i32, [vp, View, vp, vp, View, View, C.c_float]),
+    "slai_matmul_quant_add_assign": (i32, [vp, View, vp, View]),
     "slai_add_assign": (i32, [vp, View, View]),
     "slai_mul_assign": (i32, [vp, View, View]),
     "slai_copy": (i32, [vp, View, View]),
@@ -81,6 +84,8 @@ SIGNATURES = {
     "slai_softmax_cols": (i32, [vp, View]),
     "slai_attention": (i32, [vp, P(AttnParams), vp, View, View, View, View, View]),
     "slai_argmax": (i32, [vp, View, vp]),
+    "slai_timer_begin": (i32, [vp]),
+    "slai_timer_end": (i32, [vp, P(C.c_float)]),
     "slai_graph_begin_capture": (i32, [vp]),
     "slai_graph_end_capture": (i32, [vp, P(vp)]),
     "slai_graph_launch": (i32, [vp, vp]),

@@ -42,6 +42,7 @@ struct slai_ctx {
     int gemv_rows_per_wg = 8;
     int gemv_max_threads = 1024;
     int attn_splits = 0;  // 0 = automatic
+    hipEvent_t timer0 = nullptr, timer1 = nullptr;
 };
 
 namespace slai {

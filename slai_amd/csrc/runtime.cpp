@@ -86,6 +86,8 @@ SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     hipSetDevice(ctx->device);
     hipStreamSynchronize(ctx->stream);
     if (ctx->attn_scratch) hipFree(ctx->attn_scratch);
+    if (ctx->timer0) hipEventDestroy(ctx->timer0);
+    if (ctx->timer1) hipEventDestroy(ctx->timer1);
     hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -274,6 +276,41 @@ SLAI_EXPORT int slai_matmul_quant_assign(slai_ctx *ctx, slai_view out, const sla
     return SLAI_OK;
 }
 
+static int fused_gemv(slai_ctx *ctx, const char *fn, slai_view out, const slai_qmat *m, const slai_qmat *m2, slai_view v,
+                      const slai_view *norm_weight, float eps, uint32_t flags) {
+    if (!ctx || !m) return SLAI_E_ARG;
+    VecView vo, vv, vw{nullptr, 0, 1};
+    if (!as_vec(out, &vo) || !as_vec(v, &vv)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": bad view");
+    if (norm_weight && (!as_vec(*norm_weight, &vw) || vw.n != m->ncols || vw.stride != 1))
+        return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": bad norm weight");
+    if (vo.n != m->nrows || vv.n != m->ncols || vo.stride != 1 || vv.stride != 1 || (v.offset % 4) != 0)
+        return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": dimension mismatch or non-contiguous vectors");
+    if (m2 && (m2->type != m->type || m2->nrows != m->nrows || m2->ncols != m->ncols))
+        return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": gate and up must share format and shape");
+    if (!gemv_supports(m->type, m->ncols)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": unsupported column count for this format");
+    GemvParams p;
+    p.nseg = 1;
+    p.seg[0].W = m->dptr; p.seg[0].W2 = m2 ? m2->dptr : nullptr; p.seg[0].row_stride = m->row_stride; p.seg[0].nrows = m->nrows;
+    p.seg[0].out = vo.p; p.seg[0].flags = flags;
+    p.ncols = m->ncols; p.nb = m->nb; p.x = vv.p; p.rows_per_wg = ctx->gemv_rows_per_wg;
+    if (norm_weight) { p.prologue = PRO_RMSNORM; p.norm_w = vw.p; p.eps = eps; }
+    SLAI_HIP_TRY(ctx, launch_gemv(ctx, m->type, p));
+    return SLAI_OK;
+}
+
+SLAI_EXPORT int slai_rms_norm_matmul_quant_assign(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view norm_weight,
+                                                  float eps) {
+    return fused_gemv(ctx, "slai_rms_norm_matmul_quant_assign", out, m, nullptr, x, &norm_weight, eps, 0);
+}
+SLAI_EXPORT int slai_ffn_gate_up_silu(slai_ctx *ctx, slai_view out_hb, const slai_qmat *gate, const slai_qmat *up, slai_view x,
+                                      slai_view norm_weight, float eps) {
+    if (!up) return SLAI_E_ARG;
+    return fused_gemv(ctx, "slai_ffn_gate_up_silu", out_hb, gate, up, x, &norm_weight, eps, GEMV_SILU_GATE);
+}
+SLAI_EXPORT int slai_matmul_quant_add_assign(slai_ctx *ctx, slai_view in_out_x, const slai_qmat *m, slai_view v) {
+    return fused_gemv(ctx, "slai_matmul_quant_add_assign", in_out_x, m, nullptr, v, nullptr, 0.0f, GEMV_ACCUM);
+}
+
 SLAI_EXPORT int slai_matmul_assign(slai_ctx *ctx, slai_view out, slai_view a, slai_view b, int a_mode, int b_mode) {
     if (!ctx) return SLAI_E_ARG;
     View4 vo, va, vb;
@@ -408,6 +445,25 @@ SLAI_EXPORT int slai_argmax(slai_ctx *ctx, slai_view logits, slai_buffer *out_in
     NEED_VEC(logits, "logits", vl);
     if (vl.stride != 1 || out_index->dtype != SLAI_DT_I32 || out_index->bytes < 4) return set_error(ctx, SLAI_E_SHAPE, "slai_argmax: contiguous logits and an I32 output are required");
     SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, vl.p, vl.n, (int *)out_index->dptr, nullptr, nullptr, nullptr));
+    return SLAI_OK;
+}
+
+// ---- timing ---------------------------------------------------------------------------
+SLAI_EXPORT int slai_timer_begin(slai_ctx *ctx) {
+    if (!ctx) return SLAI_E_ARG;
+    if (!ctx->timer0) {
+        SLAI_HIP_TRY(ctx, hipEventCreate(&ctx->timer0));
+        SLAI_HIP_TRY(ctx, hipEventCreate(&ctx->timer1));
+    }
+    SLAI_HIP_TRY(ctx, hipEventRecord(ctx->timer0, ctx->stream));
+    return SLAI_OK;
+}
+SLAI_EXPORT int slai_timer_end(slai_ctx *ctx, float *elapsed_ms) {
+    if (!ctx || !elapsed_ms) return SLAI_E_ARG;
+    if (!ctx->timer0) return set_error(ctx, SLAI_E_STATE, "slai_timer_end without slai_timer_begin");
+    SLAI_HIP_TRY(ctx, hipEventRecord(ctx->timer1, ctx->stream));
+    SLAI_HIP_TRY(ctx, hipEventSynchronize(ctx->timer1));
+    SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, ctx->timer0, ctx->timer1));
     return SLAI_OK;
 }
 

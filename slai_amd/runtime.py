@@ -42,6 +42,14 @@ class Backend:
     def synchronize(self):
         self.check(self.L.slai_synchronize(self.h))
 
+    def timer_begin(self):
+        self.check(self.L.slai_timer_begin(self.h))
+
+    def timer_end(self):
+        ms = C.c_float()
+        self.check(self.L.slai_timer_end(self.h, C.byref(ms)))
+        return ms.value
+
     def close(self):
         if self.h:
             self.L.slai_ctx_destroy(self.h)
@@ -175,6 +183,16 @@ class LlmContext:
 
     def matmul_quant_assign(self, out, a, b):
         self.backend.check(self.L.slai_matmul_quant_assign(self.h, _v(out), a.h, _v(b)))
+
+    # fused forms (one kernel each) of the call sequences Llama2::launch issues
+    def rms_norm_matmul_quant_assign(self, out, m, x, norm_weight, eps):
+        self.backend.check(self.L.slai_rms_norm_matmul_quant_assign(self.h, _v(out), m.h, _v(x), _v(norm_weight), eps))
+
+    def ffn_gate_up_silu(self, out_hb, gate, up, x, norm_weight, eps):
+        self.backend.check(self.L.slai_ffn_gate_up_silu(self.h, _v(out_hb), gate.h, up.h, _v(x), _v(norm_weight), eps))
+
+    def matmul_quant_add_assign(self, in_out_x, m, v):
+        self.backend.check(self.L.slai_matmul_quant_add_assign(self.h, _v(in_out_x), m.h, _v(v)))
 
     def matmul_assign(self, out, a, b, a_mode, b_mode):
         self.backend.check(self.L.slai_matmul_assign(self.h, _v(out), _v(a), _v(b), a_mode, b_mode))

@@ -121,3 +121,39 @@ def test_shape_errors_are_reported_not_fatal(backend):
     assert e.value.code == _ffi.E_SHAPE
     for o in (m, v, out):
         o.destroy()
+
+
+@pytest.mark.parametrize("t", [8, 12, 14], ids=lambda t: NAMES[t])
+def test_fused_op_forms(backend, oracle_lib, t):
+    """rms-norm prologue, gate/up + SiLU, and residual-accumulate GEMV against the unfused oracle ops."""
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
+    dim, hid = 1024, 2816
+    ctxt = LlmContext(backend)
+    x, w = synth.normal(1, dim, 1.0), (1.0 + synth.normal(2, dim, 0.1)).astype(np.float32)
+    xn = np.empty(dim, np.float32)
+    oracle_lib.slo_rms_norm(xn.ctypes.data, x.ctypes.data, w.ctypes.data, dim, 1e-5)
+    raws = [synth.normal_quantized(10 + i, t, hid, dim, 0.05) for i in range(2)]
+    ws = [oracle_deq(oracle_lib, t, r, hid * dim).reshape(hid, dim) for r in raws]
+    g = np.empty(hid, np.float32); u = np.empty(hid, np.float32)
+    oracle_lib.slo_gemv(g.ctypes.data, ws[0].ctypes.data, xn.ctypes.data, hid, dim)
+    oracle_lib.slo_gemv(u.ctypes.data, ws[1].ctypes.data, xn.ctypes.data, hid, dim)
+    gate, up = [GpuQuantMatrix(backend, t, hid, dim, r) for r in raws]
+    gx, gw, ghb = GpuTensor.vector(backend, x), GpuTensor.vector(backend, w), GpuTensor(backend, hid)
+    ctxt.rms_norm_matmul_quant_assign(ghb, gate, gx, gw, 1e-5)
+    assert rel_err(ghb.read(), g) < 1e-4
+    h = g.copy(); oracle_lib.slo_silu(h.ctypes.data, u.ctypes.data, hid)
+    ctxt.ffn_gate_up_silu(ghb, gate, up, gx, gw, 1e-5)
+    assert rel_err(ghb.read(), h) < 1e-4
+    # residual accumulate: x += Wd . h   (Wd: [dim x hid2])
+    hid2 = 2816 if t == 8 else 3072
+    rawd = synth.normal_quantized(21, t, dim, hid2, 0.05)
+    wd = oracle_deq(oracle_lib, t, rawd, dim * hid2).reshape(dim, hid2)
+    hv = synth.normal(22, hid2, 1.0)
+    d = np.empty(dim, np.float32)
+    oracle_lib.slo_gemv(d.ctypes.data, wd.ctypes.data, hv.ctypes.data, dim, hid2)
+    down = GpuQuantMatrix(backend, t, dim, hid2, rawd)
+    gh = GpuTensor.vector(backend, hv)
+    ctxt.matmul_quant_add_assign(gx, down, gh)
+    assert rel_err(gx.read(), x + d) < 1e-4
+    for o in (gate, up, down, gx, gw, ghb, gh):
+        o.destroy()
