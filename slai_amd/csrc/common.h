@@ -19,8 +19,12 @@ struct slai_buffer {
 
 struct slai_qmat {
     int type = 0;
-    uint32_t nrows = 0, ncols = 0, nb = 0;  // nb = blocks per row
-    size_t row_stride = 0;                  // bytes between rows in device memory
+    uint32_t nrows = 0, ncols = 0, nb = 0;  // nb = GGUF blocks per row
+    // row layout (quant_formats.h): bytes between rows.  Unused when `tiled`.
+    size_t row_stride = 0;
+    // tiled layout (quant_tiled.h)
+    bool tiled = false;
+    uint32_t rows_log2 = 0, ncb = 0, ngroups = 0, ntiles = 0, unit_bytes = 0;
     uint8_t *dptr = nullptr;
     size_t bytes = 0;
 };
@@ -41,8 +45,11 @@ struct slai_ctx {
     // tuning knobs (environment overridable, see runtime.cpp)
     int gemv_rows_per_wg = 8;
     int gemv_max_threads = 1024;
+    int gemv_tiles_per_wg = 2;
+    bool tiled_layout = true;   // SLAI_TILED=0 keeps every matrix in the row layout
     int attn_splits = 0;  // 0 = automatic
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
+    bool use_graph = true;  // SLAI_NO_GRAPH=1 replays the token sequence eagerly (profilers that cannot trace graph launches)
 };
 
 namespace slai {
@@ -90,15 +97,59 @@ struct GemvParams {
 hipError_t launch_gemv(slai_ctx *ctx, int type, GemvParams p);
 bool gemv_supports(int type, uint32_t ncols);
 
+// GEMV over the tiled layout (kernels_gemv_tiled.hip); all segments share type and column geometry.
+struct GemvTiledSeg {
+    const uint8_t *W = nullptr;
+    const uint8_t *W2 = nullptr;
+    uint32_t nrows = 0;
+    uint32_t nblocks = 0;  // filled by the launcher
+    float *out = nullptr;
+    const float *bias = nullptr;
+    uint32_t flags = 0;
+};
+struct GemvTiledParams {
+    GemvTiledSeg seg[3];
+    int nseg = 1;
+    uint32_t ncols = 0, ncb = 0, ngroups = 0, rows_log2 = 4, unit_bytes = 0;
+    const float *x = nullptr;
+    int prologue = PRO_NONE;
+    const float *norm_w = nullptr, *norm_b = nullptr;
+    float eps = 0.0f;
+    const float *eps_ptr = nullptr;
+};
+hipError_t launch_gemv_tiled(slai_ctx *ctx, int type, GemvTiledParams p);
+
+// One GEMV launch over up to three matrices of one format and layout: out[i] = epilogue(m[i] . prologue(x)).
+struct GemvCall {
+    const slai_qmat *m[3] = {nullptr, nullptr, nullptr};
+    const slai_qmat *m2[3] = {nullptr, nullptr, nullptr};   // second matrix of a SiLU-gated pair
+    float *out[3] = {nullptr, nullptr, nullptr};
+    const float *bias[3] = {nullptr, nullptr, nullptr};
+    uint32_t flags[3] = {0, 0, 0};
+    int nseg = 1;
+    const float *x = nullptr;
+    int prologue = PRO_NONE;
+    const float *norm_w = nullptr, *norm_b = nullptr;
+    float eps = 0.0f;
+    const float *eps_ptr = nullptr;
+};
+// Returns SLAI_OK or an error code with the message set on ctx.
+int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who);
+
 // ---- dequantisation / repack ---------------------------------------------------
-hipError_t launch_repack(hipStream_t s, int type, const uint8_t *src, uint8_t *dst, uint32_t nrows, uint32_t ncols);
-// rows [row0,row0+nrows) of a device-layout matrix to f32, out[(r)*out_stride + c]
-hipError_t launch_dequant_rows(hipStream_t s, int type, const uint8_t *dev, size_t row_stride, uint32_t nb,
-                               uint32_t row0, uint32_t nrows, uint32_t ncols, float *out, size_t out_stride);
+// Device-side description of a quantized matrix in either layout.
+struct QMatDev {
+    int type; int tiled;
+    const uint8_t *dptr;
+    size_t row_stride; uint32_t nb;                                   // row layout
+    uint32_t nrows, ncols, rows_log2, ncb, ngroups, ntiles, unit_bytes;   // tiled layout
+};
+QMatDev qmat_dev(const slai_qmat *m);
+hipError_t launch_repack(hipStream_t s, const slai_qmat *m, const uint8_t *src_gguf_rows);
+// rows [row0,row0+nrows) to f32, out[r*out_stride + c]
+hipError_t launch_dequant_rows(hipStream_t s, const slai_qmat *m, uint32_t row0, uint32_t nrows, float *out, size_t out_stride);
 // out[c] = deq(A[row_a][c]) (+ deq(B[row_b][c]) when B != null); row indices read from device memory
-hipError_t launch_embed(hipStream_t s, int type_a, const uint8_t *a, size_t stride_a, uint32_t nb_a, const int *row_a,
-                        int type_b, const uint8_t *b, size_t stride_b, uint32_t nb_b, const int *row_b,
-                        uint32_t ncols, float *out);
+hipError_t launch_embed(hipStream_t s, const slai_qmat *a, const int *row_a, const slai_qmat *b, const int *row_b, uint32_t ncols, float *out);
 
 // ---- element-wise / normalisation ops -------------------------------------------------
 struct VecView { float *p; uint32_t n; uint32_t stride; };  // element i at p[i*stride]

@@ -113,7 +113,6 @@ struct slai_llama2 {
     int load(const slai_gguf *g);
     int launch(LlmContext &ctxt, const slai_attn_params &attn_params, uint32_t pos);   // transformer.rs:316-381
     int enqueue_fused(bool with_sampler);
-    int gemv_fused(int type, GemvParams &p);
 };
 
 // models/llama2/cpu.rs:79-109
@@ -244,14 +243,6 @@ int slai_llama2::launch(LlmContext &ctxt, const slai_attn_params &attn_params, u
     return SLAI_OK;
 }
 
-int slai_llama2::gemv_fused(int type, GemvParams &p) {
-    p.rows_per_wg = ctx->gemv_rows_per_wg;
-    hipError_t e = launch_gemv(ctx, type, p);
-    if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "fused GEMV: unsupported shape for this format");
-    SLAI_HIP_TRY(ctx, e);
-    return SLAI_OK;
-}
-
 // The same computation as `launch`, as fused kernels whose per-token scalars (position, token) live
 // in device memory, so the sequence can be captured once and replayed for every token:
 //   embedding-row gather | per layer: [RMSNorm+QKV GEMV] [RoPE+cache write+attention] [Wo GEMV+residual]
@@ -262,27 +253,25 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
     float *x = (float *)s.x.buf->dptr, *xb = (float *)s.xb.buf->dptr, *hb = (float *)s.hb.buf->dptr, *hb2 = (float *)s.hb2.buf->dptr;
     float *q = (float *)s.q.buf->dptr, *kcol = (float *)s.kcol.buf->dptr, *vcol = (float *)s.vcol.buf->dptr;
     const uint32_t dim = config.dim, kvd = kv_dim();
-    const slai_qmat *te = weights.token_embd;
-    SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, te->type, te->dptr, te->row_stride, te->nb, &ds->token, 0, nullptr, 0, 0, nullptr, dim, x));
+    SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, &ds->token, nullptr, nullptr, dim, x));
     for (uint32_t l = 0; l < config.n_layers; ++l) {
         const Llama2LayerWeights &wl = weights.layers[l];
-        // ---- RMSNorm + Q/K/V projections: matrices of one format share a launch
+        // ---- RMSNorm + Q/K/V projections: matrices of one format and layout share a launch
         {
             const slai_qmat *mats[3] = {wl.attn_q, wl.attn_k, wl.attn_v};
             float *outs[3] = {q, kcol, vcol};
             bool done[3] = {false, false, false};
             for (int i = 0; i < 3; ++i) {
                 if (done[i]) continue;
-                GemvParams p;
-                p.nseg = 0; p.ncols = dim; p.nb = mats[i]->nb; p.x = x;
-                p.prologue = PRO_RMSNORM; p.norm_w = (const float *)wl.attn_norm.buf->dptr; p.eps = config.rms_norm_eps;
+                GemvCall c;
+                c.nseg = 0; c.x = x;
+                c.prologue = PRO_RMSNORM; c.norm_w = (const float *)wl.attn_norm.buf->dptr; c.eps = config.rms_norm_eps;
                 for (int j = i; j < 3; ++j) {
-                    if (done[j] || mats[j]->type != mats[i]->type) continue;
-                    GemvSeg &sg = p.seg[p.nseg++];
-                    sg.W = mats[j]->dptr; sg.row_stride = mats[j]->row_stride; sg.nrows = mats[j]->nrows; sg.out = outs[j];
+                    if (done[j] || mats[j]->type != mats[i]->type || mats[j]->tiled != mats[i]->tiled) continue;
+                    c.m[c.nseg] = mats[j]; c.out[c.nseg] = outs[j]; ++c.nseg;
                     done[j] = true;
                 }
-                TRY(gemv_fused(mats[i]->type, p));
+                TRY(gemv_call(ctx, c, "llama2 qkv"));
             }
         }
         // ---- bias + RoPE + cache write + attention
@@ -305,48 +294,39 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
         }
         // ---- attention output projection, residual in the epilogue
         {
-            GemvParams p;
-            p.nseg = 1; p.ncols = dim; p.nb = wl.attn_output->nb; p.x = xb;
-            p.seg[0].W = wl.attn_output->dptr; p.seg[0].row_stride = wl.attn_output->row_stride; p.seg[0].nrows = dim;
-            p.seg[0].out = x; p.seg[0].flags = GEMV_ACCUM;
-            TRY(gemv_fused(wl.attn_output->type, p));
+            GemvCall c;
+            c.m[0] = wl.attn_output; c.out[0] = x; c.flags[0] = GEMV_ACCUM; c.x = xb;
+            TRY(gemv_call(ctx, c, "llama2 attn_output"));
         }
         // ---- RMSNorm + gate/up + SiLU
-        if (wl.ffn_gate->type == wl.ffn_up->type) {
-            GemvParams p;
-            p.nseg = 1; p.ncols = dim; p.nb = wl.ffn_gate->nb; p.x = x;
-            p.prologue = PRO_RMSNORM; p.norm_w = (const float *)wl.ffn_norm.buf->dptr; p.eps = config.rms_norm_eps;
-            p.seg[0].W = wl.ffn_gate->dptr; p.seg[0].W2 = wl.ffn_up->dptr; p.seg[0].row_stride = wl.ffn_gate->row_stride;
-            p.seg[0].nrows = config.hidden_dim; p.seg[0].out = hb; p.seg[0].flags = GEMV_SILU_GATE;
-            TRY(gemv_fused(wl.ffn_gate->type, p));
+        if (wl.ffn_gate->type == wl.ffn_up->type && wl.ffn_gate->tiled == wl.ffn_up->tiled) {
+            GemvCall c;
+            c.m[0] = wl.ffn_gate; c.m2[0] = wl.ffn_up; c.out[0] = hb; c.flags[0] = GEMV_SILU_GATE; c.x = x;
+            c.prologue = PRO_RMSNORM; c.norm_w = (const float *)wl.ffn_norm.buf->dptr; c.eps = config.rms_norm_eps;
+            TRY(gemv_call(ctx, c, "llama2 ffn gate/up"));
         } else {
             const slai_qmat *mats[2] = {wl.ffn_gate, wl.ffn_up};
             float *outs[2] = {hb, hb2};
             for (int i = 0; i < 2; ++i) {
-                GemvParams p;
-                p.nseg = 1; p.ncols = dim; p.nb = mats[i]->nb; p.x = x;
-                p.prologue = PRO_RMSNORM; p.norm_w = (const float *)wl.ffn_norm.buf->dptr; p.eps = config.rms_norm_eps;
-                p.seg[0].W = mats[i]->dptr; p.seg[0].row_stride = mats[i]->row_stride; p.seg[0].nrows = config.hidden_dim; p.seg[0].out = outs[i];
-                TRY(gemv_fused(mats[i]->type, p));
+                GemvCall c;
+                c.m[0] = mats[i]; c.out[0] = outs[i]; c.x = x;
+                c.prologue = PRO_RMSNORM; c.norm_w = (const float *)wl.ffn_norm.buf->dptr; c.eps = config.rms_norm_eps;
+                TRY(gemv_call(ctx, c, "llama2 ffn gate/up"));
             }
             SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, config.hidden_dim, 1}, VecView{hb2, config.hidden_dim, 1}));
         }
         // ---- down projection, residual in the epilogue
         {
-            GemvParams p;
-            p.nseg = 1; p.ncols = config.hidden_dim; p.nb = wl.ffn_down->nb; p.x = hb;
-            p.seg[0].W = wl.ffn_down->dptr; p.seg[0].row_stride = wl.ffn_down->row_stride; p.seg[0].nrows = dim;
-            p.seg[0].out = x; p.seg[0].flags = GEMV_ACCUM;
-            TRY(gemv_fused(wl.ffn_down->type, p));
+            GemvCall c;
+            c.m[0] = wl.ffn_down; c.out[0] = x; c.flags[0] = GEMV_ACCUM; c.x = hb;
+            TRY(gemv_call(ctx, c, "llama2 ffn_down"));
         }
     }
     {
-        GemvParams p;
-        p.nseg = 1; p.ncols = dim; p.nb = weights.output->nb; p.x = x;
-        p.prologue = PRO_RMSNORM; p.norm_w = (const float *)weights.output_norm.buf->dptr; p.eps = config.rms_norm_eps;
-        p.seg[0].W = weights.output->dptr; p.seg[0].row_stride = weights.output->row_stride; p.seg[0].nrows = config.vocab_size;
-        p.seg[0].out = (float *)s.logits.buf->dptr;
-        TRY(gemv_fused(weights.output->type, p));
+        GemvCall c;
+        c.m[0] = weights.output; c.out[0] = (float *)s.logits.buf->dptr; c.x = x;
+        c.prologue = PRO_RMSNORM; c.norm_w = (const float *)weights.output_norm.buf->dptr; c.eps = config.rms_norm_eps;
+        TRY(gemv_call(ctx, c, "llama2 output"));
     }
     if (with_sampler)
         SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, nullptr, ds,
@@ -442,6 +422,14 @@ static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_le
     DecodeState ds{(int)start_pos, prompt[start_pos], (int)n_prompt, 0};     // chat_llama2.rs:105
     TRY(slai_write_buffer(ctx, L.state, 0, &ds, sizeof ds));
     TRY(slai_write_buffer(ctx, L.prompt, 0, prompt, (size_t)n_prompt * 4));
+    if (!ctx->use_graph) {
+        SLAI_HIP_TRY(ctx, hipEventRecord(L.ev0, ctx->stream));
+        for (uint32_t i = 0; i < n_steps; ++i) TRY(m->enqueue_fused(true));
+        SLAI_HIP_TRY(ctx, hipEventRecord(L.ev1, ctx->stream));
+        TRY(slai_synchronize(ctx));
+        if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, L.ev0, L.ev1));
+        return slai_read_buffer(ctx, L.out_tokens, 0, out_tokens, (size_t)n_steps * 4);
+    }
     if (!L.graph) {
         TRY(slai_graph_begin_capture(ctx));
         int rc = m->enqueue_fused(true);
@@ -503,13 +491,6 @@ struct slai_gpt2 {
 
     int load(const slai_gguf *g);
     int enqueue_fused(bool with_sampler);
-    int gemv(int type, GemvParams &p) {
-        p.rows_per_wg = ctx->gemv_rows_per_wg;
-        hipError_t e = launch_gemv(ctx, type, p);
-        if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "GEMV: unsupported shape for this format");
-        SLAI_HIP_TRY(ctx, e);
-        return SLAI_OK;
-    }
 };
 
 int slai_gpt2::load(const slai_gguf *gg) {
@@ -580,17 +561,14 @@ int slai_gpt2::enqueue_fused(bool with_sampler) {
           *h = (float *)curr_3072.buf->dptr, *logits = (float *)curr_vocab.buf->dptr;
     const float eps = 1.0e-5f;
     // :227-228 wte[:,tok] + wpe[:,pos]
-    SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, wte->type, wte->dptr, wte->row_stride, wte->nb, &ds->token, wpe->type, wpe->dptr,
-                                   wpe->row_stride, wpe->nb, &ds->pos, E, x));
+    SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, wte, &ds->token, wpe, &ds->pos, E, x));
     for (uint32_t l = 0; l < params.n_layer; ++l) {
         Gpt2Layer &w = layers[l];
         {   // :235-255 LayerNorm*g+b, qkv GEMV + bias
-            GemvParams p;
-            p.nseg = 1; p.ncols = E; p.nb = w.c_attn_attn_w->nb; p.x = x;
-            p.prologue = PRO_LAYERNORM; p.norm_w = (const float *)w.ln_1_g.buf->dptr; p.norm_b = (const float *)w.ln_1_b.buf->dptr; p.eps = eps;
-            p.seg[0].W = w.c_attn_attn_w->dptr; p.seg[0].row_stride = w.c_attn_attn_w->row_stride; p.seg[0].nrows = 3 * E;
-            p.seg[0].out = qkv; p.seg[0].bias = (const float *)w.c_attn_attn_b.buf->dptr; p.seg[0].flags = GEMV_BIAS;
-            TRY(gemv(w.c_attn_attn_w->type, p));
+            GemvCall c;
+            c.m[0] = w.c_attn_attn_w; c.out[0] = qkv; c.bias[0] = (const float *)w.c_attn_attn_b.buf->dptr; c.flags[0] = GEMV_BIAS; c.x = x;
+            c.prologue = PRO_LAYERNORM; c.norm_w = (const float *)w.ln_1_g.buf->dptr; c.norm_b = (const float *)w.ln_1_b.buf->dptr; c.eps = eps;
+            TRY(gemv_call(ctx, c, "gpt2 qkv"));
         }
         {   // :263-290 split q/k/v, cache write, attention with kv_mul = 1
             AttnLaunch a{};
@@ -605,34 +583,27 @@ int slai_gpt2::enqueue_fused(bool with_sampler) {
             SLAI_HIP_TRY(ctx, e);
         }
         {   // :302-312 projection + bias + residual
-            GemvParams p;
-            p.nseg = 1; p.ncols = E; p.nb = w.c_attn_proj_w->nb; p.x = att_out;
-            p.seg[0].W = w.c_attn_proj_w->dptr; p.seg[0].row_stride = w.c_attn_proj_w->row_stride; p.seg[0].nrows = E;
-            p.seg[0].out = x; p.seg[0].bias = (const float *)w.c_attn_proj_b.buf->dptr; p.seg[0].flags = GEMV_BIAS | GEMV_ACCUM;
-            TRY(gemv(w.c_attn_proj_w->type, p));
+            GemvCall c;
+            c.m[0] = w.c_attn_proj_w; c.out[0] = x; c.bias[0] = (const float *)w.c_attn_proj_b.buf->dptr; c.flags[0] = GEMV_BIAS | GEMV_ACCUM; c.x = att_out;
+            TRY(gemv_call(ctx, c, "gpt2 attn proj"));
         }
         {   // :318-343 LayerNorm*g+b, fc GEMV + bias, GELU
-            GemvParams p;
-            p.nseg = 1; p.ncols = E; p.nb = w.c_mlp_fc_w->nb; p.x = x;
-            p.prologue = PRO_LAYERNORM; p.norm_w = (const float *)w.ln_2_g.buf->dptr; p.norm_b = (const float *)w.ln_2_b.buf->dptr; p.eps = eps;
-            p.seg[0].W = w.c_mlp_fc_w->dptr; p.seg[0].row_stride = w.c_mlp_fc_w->row_stride; p.seg[0].nrows = params.ff_len;
-            p.seg[0].out = h; p.seg[0].bias = (const float *)w.c_mlp_fc_b.buf->dptr; p.seg[0].flags = GEMV_BIAS | GEMV_GELU;
-            TRY(gemv(w.c_mlp_fc_w->type, p));
+            GemvCall c;
+            c.m[0] = w.c_mlp_fc_w; c.out[0] = h; c.bias[0] = (const float *)w.c_mlp_fc_b.buf->dptr; c.flags[0] = GEMV_BIAS | GEMV_GELU; c.x = x;
+            c.prologue = PRO_LAYERNORM; c.norm_w = (const float *)w.ln_2_g.buf->dptr; c.norm_b = (const float *)w.ln_2_b.buf->dptr; c.eps = eps;
+            TRY(gemv_call(ctx, c, "gpt2 mlp fc"));
         }
         {   // :353-360 projection + bias + residual
-            GemvParams p;
-            p.nseg = 1; p.ncols = params.ff_len; p.nb = w.c_mlp_proj_w->nb; p.x = h;
-            p.seg[0].W = w.c_mlp_proj_w->dptr; p.seg[0].row_stride = w.c_mlp_proj_w->row_stride; p.seg[0].nrows = E;
-            p.seg[0].out = x; p.seg[0].bias = (const float *)w.c_mlp_proj_b.buf->dptr; p.seg[0].flags = GEMV_BIAS | GEMV_ACCUM;
-            TRY(gemv(w.c_mlp_proj_w->type, p));
+            GemvCall c;
+            c.m[0] = w.c_mlp_proj_w; c.out[0] = x; c.bias[0] = (const float *)w.c_mlp_proj_b.buf->dptr; c.flags[0] = GEMV_BIAS | GEMV_ACCUM; c.x = h;
+            TRY(gemv_call(ctx, c, "gpt2 mlp proj"));
         }
     }
     {   // :366-379 final LayerNorm*g+b, lm_head = wte
-        GemvParams p;
-        p.nseg = 1; p.ncols = E; p.nb = wte->nb; p.x = x;
-        p.prologue = PRO_LAYERNORM; p.norm_w = (const float *)ln_f_g.buf->dptr; p.norm_b = (const float *)ln_f_b.buf->dptr; p.eps = eps;
-        p.seg[0].W = wte->dptr; p.seg[0].row_stride = wte->row_stride; p.seg[0].nrows = params.n_vocab; p.seg[0].out = logits;
-        TRY(gemv(wte->type, p));
+        GemvCall c;
+        c.m[0] = wte; c.out[0] = logits; c.x = x;
+        c.prologue = PRO_LAYERNORM; c.norm_w = (const float *)ln_f_g.buf->dptr; c.norm_b = (const float *)ln_f_b.buf->dptr; c.eps = eps;
+        TRY(gemv_call(ctx, c, "gpt2 lm_head"));
     }
     if (with_sampler)
         SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, logits, params.n_vocab, nullptr, ds, (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));

@@ -4,20 +4,43 @@
 // -ffp-contract=off so that `d * q - m` stays two roundings.
 #include "common.h"
 #include "quant_formats.h"
+#include "quant_tiled.h"
 
 namespace slai {
+
+QMatDev qmat_dev(const slai_qmat *m) {
+    QMatDev d{};
+    if (!m) return d;
+    d.type = m->type; d.tiled = m->tiled ? 1 : 0; d.dptr = m->dptr; d.row_stride = m->row_stride; d.nb = m->nb;
+    d.nrows = m->nrows; d.ncols = m->ncols; d.rows_log2 = m->rows_log2; d.ncb = m->ncb; d.ngroups = m->ngroups;
+    d.ntiles = m->ntiles; d.unit_bytes = m->unit_bytes;
+    return d;
+}
+
 namespace {
 
-__global__ void repack_kernel(int type, const uint8_t *src, uint8_t *dst, uint32_t nrows, uint32_t nb, size_t gguf_row,
-                              size_t dev_row, int bb) {
-    const size_t total = (size_t)nrows * nb;
+__device__ __forceinline__ TiledGeom geom_of(const QMatDev &m) {
+    TiledGeom g;
+    g.type = m.type; g.nrows = m.nrows; g.ncols = m.ncols; g.rows_log2 = m.rows_log2; g.ncb = m.ncb; g.ngroups = m.ngroups;
+    g.ntiles = m.ntiles; g.pieces = tiled_pieces(m.type); g.unit_bytes = m.unit_bytes;
+    return g;
+}
+__device__ __forceinline__ float qmat_elem(const QMatDev &m, uint32_t row, uint32_t col) {
+    if (m.tiled) return tiled_dequant_elem(geom_of(m), m.dptr, row, col);
+    return dequant_elem(m.type, m.dptr + (size_t)row * m.row_stride, m.nb, col);
+}
+
+__global__ void repack_kernel(QMatDev m, uint8_t *dst, const uint8_t *src, size_t gguf_row, int bb) {
+    const size_t total = (size_t)m.nrows * m.nb;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const uint32_t r = (uint32_t)(i / nb), b = (uint32_t)(i % nb);
-        repack_block(type, src + (size_t)r * gguf_row + (size_t)b * bb, dst + (size_t)r * dev_row, nb, b);
+        const uint32_t r = (uint32_t)(i / m.nb), b = (uint32_t)(i % m.nb);
+        const uint8_t *blk = src + (size_t)r * gguf_row + (size_t)b * bb;
+        if (m.tiled) tiled_repack_block(geom_of(m), blk, dst, r, b);
+        else repack_block(m.type, blk, dst + (size_t)r * m.row_stride, m.nb, b);
     }
 }
 
-// f32 / f16 rows: plain byte copy with the padded device stride
+// f32 / f16 rows: plain copy with the padded device stride
 __global__ void copy_rows_kernel(const uint8_t *src, uint8_t *dst, uint32_t nrows, size_t gguf_row, size_t dev_row) {
     const size_t words = gguf_row / 2;  // rows are multiples of 2 bytes
     const size_t total = (size_t)nrows * words;
@@ -27,55 +50,47 @@ __global__ void copy_rows_kernel(const uint8_t *src, uint8_t *dst, uint32_t nrow
     }
 }
 
-__global__ void dequant_rows_kernel(int type, const uint8_t *dev, size_t row_stride, uint32_t nb, uint32_t row0,
-                                    uint32_t nrows, uint32_t ncols, float *out, size_t out_stride) {
-    const size_t total = (size_t)nrows * ncols;
+__global__ void dequant_rows_kernel(QMatDev m, uint32_t row0, uint32_t nrows, float *out, size_t out_stride) {
+    const size_t total = (size_t)nrows * m.ncols;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const uint32_t r = (uint32_t)(i / ncols), c = (uint32_t)(i % ncols);
-        out[(size_t)r * out_stride + c] = dequant_elem(type, dev + (size_t)(row0 + r) * row_stride, nb, c);
+        const uint32_t r = (uint32_t)(i / m.ncols), c = (uint32_t)(i % m.ncols);
+        out[(size_t)r * out_stride + c] = qmat_elem(m, row0 + r, c);
     }
 }
 
-__global__ void embed_kernel(int type_a, const uint8_t *a, size_t stride_a, uint32_t nb_a, const int *row_a, int type_b,
-                             const uint8_t *b, size_t stride_b, uint32_t nb_b, const int *row_b, uint32_t ncols,
-                             float *out) {
+__global__ void embed_kernel(QMatDev a, const int *row_a, QMatDev b, const int *row_b, int has_b, uint32_t ncols, float *out) {
     const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= ncols) return;
-    float v = dequant_elem(type_a, a + (size_t)(*row_a) * stride_a, nb_a, c);
+    float v = qmat_elem(a, (uint32_t)*row_a, c);
     // gpt2/cpu.rs:227-228: token embedding first, then += position embedding
-    if (b) v = v + dequant_elem(type_b, b + (size_t)(*row_b) * stride_b, nb_b, c);
+    if (has_b) v = v + qmat_elem(b, (uint32_t)*row_b, c);
     out[c] = v;
 }
 
 }  // namespace
 
-hipError_t launch_repack(hipStream_t s, int type, const uint8_t *src, uint8_t *dst, uint32_t nrows, uint32_t ncols) {
-    const uint32_t nb = ncols / block_elems(type);
-    const size_t gr = gguf_row_bytes(type, ncols), dr = device_row_stride(type, ncols);
-    if (type == T_F32 || type == T_F16) {
-        if (gr == dr) return hipMemcpyAsync(dst, src, gr * nrows, hipMemcpyDeviceToDevice, s);
-        copy_rows_kernel<<<1024, 256, 0, s>>>(src, dst, nrows, gr, dr);
+hipError_t launch_repack(hipStream_t s, const slai_qmat *m, const uint8_t *src) {
+    const size_t gr = gguf_row_bytes(m->type, m->ncols);
+    if (!m->tiled && (m->type == T_F32 || m->type == T_F16)) {
+        if (gr == m->row_stride) return hipMemcpyAsync(m->dptr, src, gr * m->nrows, hipMemcpyDeviceToDevice, s);
+        copy_rows_kernel<<<1024, 256, 0, s>>>(src, m->dptr, m->nrows, gr, m->row_stride);
     } else {
-        repack_kernel<<<2048, 256, 0, s>>>(type, src, dst, nrows, nb, gr, dr, block_bytes(type));
+        repack_kernel<<<2048, 256, 0, s>>>(qmat_dev(m), m->dptr, src, gr, block_bytes(m->type));
     }
     return hipGetLastError();
 }
 
-hipError_t launch_dequant_rows(hipStream_t s, int type, const uint8_t *dev, size_t row_stride, uint32_t nb, uint32_t row0,
-                               uint32_t nrows, uint32_t ncols, float *out, size_t out_stride) {
-    size_t total = (size_t)nrows * ncols;
+hipError_t launch_dequant_rows(hipStream_t s, const slai_qmat *m, uint32_t row0, uint32_t nrows, float *out, size_t out_stride) {
+    size_t total = (size_t)nrows * m->ncols;
     uint32_t grid = (uint32_t)((total + 255) / 256);
     if (grid > 65536) grid = 65536;
     if (grid == 0) return hipSuccess;
-    dequant_rows_kernel<<<grid, 256, 0, s>>>(type, dev, row_stride, nb, row0, nrows, ncols, out, out_stride);
+    dequant_rows_kernel<<<grid, 256, 0, s>>>(qmat_dev(m), row0, nrows, out, out_stride);
     return hipGetLastError();
 }
 
-hipError_t launch_embed(hipStream_t s, int type_a, const uint8_t *a, size_t stride_a, uint32_t nb_a, const int *row_a,
-                        int type_b, const uint8_t *b, size_t stride_b, uint32_t nb_b, const int *row_b, uint32_t ncols,
-                        float *out) {
-    embed_kernel<<<(ncols + 255) / 256, 256, 0, s>>>(type_a, a, stride_a, nb_a, row_a, type_b, b, stride_b, nb_b, row_b,
-                                                      ncols, out);
+hipError_t launch_embed(hipStream_t s, const slai_qmat *a, const int *row_a, const slai_qmat *b, const int *row_b, uint32_t ncols, float *out) {
+    embed_kernel<<<(ncols + 255) / 256, 256, 0, s>>>(qmat_dev(a), row_a, qmat_dev(b), row_b, b ? 1 : 0, ncols, out);
     return hipGetLastError();
 }
 

@@ -3,6 +3,7 @@
 // interfaces they replace are in include/slai_hip.h.
 #include "common.h"
 #include "quant_formats.h"
+#include "quant_tiled.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -77,6 +78,9 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->gemv_rows_per_wg = env_int("SLAI_GEMV_ROWS_PER_WG", 8);
     ctx->gemv_max_threads = env_int("SLAI_GEMV_MAX_THREADS", 512);
     ctx->attn_splits = env_int("SLAI_ATTN_SPLITS", 0);
+    ctx->use_graph = env_int("SLAI_NO_GRAPH", 0) == 0;
+    ctx->gemv_tiles_per_wg = env_int("SLAI_GEMV_TILES_PER_WG", 2);
+    ctx->tiled_layout = env_int("SLAI_TILED", 1) != 0;
     *out = ctx;
     return SLAI_OK;
 }
@@ -185,10 +189,17 @@ SLAI_EXPORT int slai_qmat_create(slai_ctx *ctx, uint32_t ggml_type, uint32_t nro
     m->type = t; m->nrows = nrows; m->ncols = ncols; m->nb = ncols / be;
     m->row_stride = device_row_stride(t, ncols);
     m->bytes = m->row_stride * nrows;
+    if (ctx->tiled_layout && tiled_supported(t) && ncols % 256 == 0) {
+        const TiledGeom g = tiled_geom(t, nrows, ncols);
+        if (g.ngroups <= 16) {
+            m->tiled = true; m->rows_log2 = g.rows_log2; m->ncb = g.ncb; m->ngroups = g.ngroups; m->ntiles = g.ntiles;
+            m->unit_bytes = g.unit_bytes; m->bytes = tiled_bytes(g);
+        }
+    }
     const size_t src_bytes = gguf_row_bytes(t, ncols) * nrows;
     uint8_t *staging = nullptr;
     hipError_t e = hipMalloc((void **)&m->dptr, m->bytes);
-    const bool verbatim = (t == T_Q4_K || t == T_Q5_K || ((t == T_F32 || t == T_F16) && gguf_row_bytes(t, ncols) == m->row_stride));
+    const bool verbatim = !m->tiled && (t == T_Q4_K || t == T_Q5_K || ((t == T_F32 || t == T_F16) && gguf_row_bytes(t, ncols) == m->row_stride));
     if (e == hipSuccess) {
         if (verbatim) {
             e = hipMemcpyAsync(m->dptr, packed, src_bytes, hipMemcpyHostToDevice, ctx->stream);
@@ -196,7 +207,7 @@ SLAI_EXPORT int slai_qmat_create(slai_ctx *ctx, uint32_t ggml_type, uint32_t nro
             e = hipMalloc((void **)&staging, src_bytes);
             if (e == hipSuccess) e = hipMemsetAsync(m->dptr, 0, m->bytes, ctx->stream);
             if (e == hipSuccess) e = hipMemcpyAsync(staging, packed, src_bytes, hipMemcpyHostToDevice, ctx->stream);
-            if (e == hipSuccess) e = launch_repack(ctx->stream, t, staging, m->dptr, nrows, ncols);
+            if (e == hipSuccess) e = launch_repack(ctx->stream, m, staging);
         }
     }
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -234,10 +245,50 @@ SLAI_EXPORT int slai_qmat_dequantize(slai_ctx *ctx, const slai_qmat *m, uint32_t
     if (nrows == 0) return SLAI_OK;
     size_t last = out.offset + (size_t)(nrows - 1) * out.stride[0] + m->ncols;
     if (last * sizeof(float) > out.buf->bytes) return set_error(ctx, SLAI_E_SHAPE, "slai_qmat_dequantize: out too small");
-    SLAI_HIP_TRY(ctx, launch_dequant_rows(ctx->stream, m->type, m->dptr, m->row_stride, m->nb, row0, nrows, m->ncols,
-                                          (float *)out.buf->dptr + out.offset, out.stride[0]));
+    SLAI_HIP_TRY(ctx, launch_dequant_rows(ctx->stream, m, row0, nrows, (float *)out.buf->dptr + out.offset, out.stride[0]));
     return SLAI_OK;
 }
+
+// ---- GEMV dispatch over the two weight layouts ------------------------------------------------
+namespace slai {
+int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who) {
+    const slai_qmat *m0 = c.m[0];
+    if (!m0 || c.nseg < 1 || c.nseg > 3) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": bad GEMV call");
+    for (int i = 0; i < c.nseg; ++i) {
+        const slai_qmat *m = c.m[i], *m2 = c.m2[i];
+        if (!m || m->type != m0->type || m->ncols != m0->ncols || m->tiled != m0->tiled)
+            return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": matrices of one launch must share format, width and layout");
+        if (m2 && (m2->type != m->type || m2->ncols != m->ncols || m2->nrows != m->nrows || m2->tiled != m->tiled))
+            return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": gate and up must share format, shape and layout");
+        if ((c.flags[i] & GEMV_SILU_GATE) && !m2) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": gated GEMV without a second matrix");
+    }
+    hipError_t e;
+    if (m0->tiled) {
+        GemvTiledParams p;
+        p.nseg = c.nseg; p.ncols = m0->ncols; p.ncb = m0->ncb; p.ngroups = m0->ngroups; p.rows_log2 = m0->rows_log2;
+        p.unit_bytes = m0->unit_bytes; p.x = c.x; p.prologue = c.prologue; p.norm_w = c.norm_w; p.norm_b = c.norm_b;
+        p.eps = c.eps; p.eps_ptr = c.eps_ptr;
+        for (int i = 0; i < c.nseg; ++i) {
+            p.seg[i].W = c.m[i]->dptr; p.seg[i].W2 = c.m2[i] ? c.m2[i]->dptr : nullptr; p.seg[i].nrows = c.m[i]->nrows;
+            p.seg[i].out = c.out[i]; p.seg[i].bias = c.bias[i]; p.seg[i].flags = c.flags[i];
+        }
+        e = launch_gemv_tiled(ctx, m0->type, p);
+    } else {
+        if (!gemv_supports(m0->type, m0->ncols)) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported column count for this format");
+        GemvParams p;
+        p.nseg = c.nseg; p.ncols = m0->ncols; p.nb = m0->nb; p.x = c.x; p.prologue = c.prologue; p.norm_w = c.norm_w;
+        p.norm_b = c.norm_b; p.eps = c.eps; p.eps_ptr = c.eps_ptr; p.rows_per_wg = ctx->gemv_rows_per_wg;
+        for (int i = 0; i < c.nseg; ++i) {
+            p.seg[i].W = c.m[i]->dptr; p.seg[i].W2 = c.m2[i] ? c.m2[i]->dptr : nullptr; p.seg[i].row_stride = c.m[i]->row_stride;
+            p.seg[i].nrows = c.m[i]->nrows; p.seg[i].out = c.out[i]; p.seg[i].bias = c.bias[i]; p.seg[i].flags = c.flags[i];
+        }
+        e = launch_gemv(ctx, m0->type, p);
+    }
+    if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported shape for this format");
+    if (e != hipSuccess) return hip_fail(ctx, e, who);
+    return SLAI_OK;
+}
+}  // namespace slai
 
 // ---- ops ---------------------------------------------------------------------------
 #define NEED_VEC(view, name, vv)                                                                           \
@@ -267,13 +318,9 @@ SLAI_EXPORT int slai_matmul_quant_assign(slai_ctx *ctx, slai_view out, const sla
     if (vo.n != m->nrows || vv.n != m->ncols) return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_quant_assign: dimension mismatch");
     if (vo.stride != 1 || vv.stride != 1 || (v.offset % 4) != 0)
         return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_quant_assign: vectors must be contiguous, input offset a multiple of 4");
-    if (!gemv_supports(m->type, m->ncols)) return set_error(ctx, SLAI_E_SHAPE, "slai_matmul_quant_assign: unsupported column count for this format");
-    GemvParams p;
-    p.nseg = 1;
-    p.seg[0].W = m->dptr; p.seg[0].row_stride = m->row_stride; p.seg[0].nrows = m->nrows; p.seg[0].out = vo.p;
-    p.ncols = m->ncols; p.nb = m->nb; p.x = vv.p; p.rows_per_wg = ctx->gemv_rows_per_wg;
-    SLAI_HIP_TRY(ctx, launch_gemv(ctx, m->type, p));
-    return SLAI_OK;
+    GemvCall c;
+    c.m[0] = m; c.out[0] = vo.p; c.x = vv.p;
+    return gemv_call(ctx, c, "slai_matmul_quant_assign");
 }
 
 static int fused_gemv(slai_ctx *ctx, const char *fn, slai_view out, const slai_qmat *m, const slai_qmat *m2, slai_view v,
@@ -287,15 +334,10 @@ static int fused_gemv(slai_ctx *ctx, const char *fn, slai_view out, const slai_q
         return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": dimension mismatch or non-contiguous vectors");
     if (m2 && (m2->type != m->type || m2->nrows != m->nrows || m2->ncols != m->ncols))
         return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": gate and up must share format and shape");
-    if (!gemv_supports(m->type, m->ncols)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": unsupported column count for this format");
-    GemvParams p;
-    p.nseg = 1;
-    p.seg[0].W = m->dptr; p.seg[0].W2 = m2 ? m2->dptr : nullptr; p.seg[0].row_stride = m->row_stride; p.seg[0].nrows = m->nrows;
-    p.seg[0].out = vo.p; p.seg[0].flags = flags;
-    p.ncols = m->ncols; p.nb = m->nb; p.x = vv.p; p.rows_per_wg = ctx->gemv_rows_per_wg;
-    if (norm_weight) { p.prologue = PRO_RMSNORM; p.norm_w = vw.p; p.eps = eps; }
-    SLAI_HIP_TRY(ctx, launch_gemv(ctx, m->type, p));
-    return SLAI_OK;
+    GemvCall c;
+    c.m[0] = m; c.m2[0] = m2; c.out[0] = vo.p; c.flags[0] = flags; c.x = vv.p;
+    if (norm_weight) { c.prologue = PRO_RMSNORM; c.norm_w = vw.p; c.eps = eps; }
+    return gemv_call(ctx, c, fn);
 }
 
 SLAI_EXPORT int slai_rms_norm_matmul_quant_assign(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view norm_weight,
