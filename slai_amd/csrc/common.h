@@ -45,7 +45,7 @@ struct slai_ctx {
     // tuning knobs (environment overridable, see runtime.cpp)
     int gemv_rows_per_wg = 8;
     int gemv_max_threads = 1024;
-    int gemv_tiles_per_wg = 2;
+    int gemv_max_wgs = 512;     // workgroups per tiled GEMV launch (SLAI_GEMV_MAX_WGS)
     bool tiled_layout = true;   // SLAI_TILED=0 keeps every matrix in the row layout
     int attn_splits = 0;  // 0 = automatic
     hipEvent_t timer0 = nullptr, timer1 = nullptr;

@@ -183,24 +183,28 @@ __global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_
     }
 }
 
-// grid = n_heads, block = 128: merge the per-split (max, sum, unnormalised output) triples
-__global__ void attn_combine_kernel(const float *scratch, float *out, uint32_t hs, uint32_t n_splits) {
-    const uint32_t h = blockIdx.x;
+// grid = n_heads, block = 128: merge the per-split (max, sum, unnormalised output) triples.
+// n_splits <= 64: one lane per split computes its weight exp(m_s - M) / L, then every thread
+// accumulates its output elements with independent loads.
+__global__ void __launch_bounds__(128) attn_combine_kernel(const float *scratch, float *out, uint32_t hs, uint32_t n_splits) {
+    __shared__ float sw[64];
+    const uint32_t h = blockIdx.x, tid = threadIdx.x;
     const float *base = scratch + (size_t)h * n_splits * (hs + 2);
-    float M = -FLT_MAX;
-    for (uint32_t s = 0; s < n_splits; ++s) M = fmaxf(M, base[(size_t)s * (hs + 2) + hs]);
-    float L = 0.0f;
-    for (uint32_t s = 0; s < n_splits; ++s) {
-        const float ms = base[(size_t)s * (hs + 2) + hs], ls = base[(size_t)s * (hs + 2) + hs + 1];
-        L += ls > 0.0f ? expf(ms - M) * ls : 0.0f;
+    if (tid < 64) {
+        const bool on = tid < n_splits;
+        const float ms = on ? base[(size_t)tid * (hs + 2) + hs] : -FLT_MAX;
+        const float ls = on ? base[(size_t)tid * (hs + 2) + hs + 1] : 0.0f;
+        const float M = wave_max(ms);
+        const float w = ls > 0.0f ? expf(ms - M) : 0.0f;
+        const float L = wave_sum(w * ls);
+        sw[tid] = w / L;
     }
-    for (uint32_t e = threadIdx.x; e < hs; e += blockDim.x) {
+    __syncthreads();
+    for (uint32_t e = tid; e < hs; e += blockDim.x) {
         float acc = 0.0f;
-        for (uint32_t s = 0; s < n_splits; ++s) {
-            const float ms = base[(size_t)s * (hs + 2) + hs], ls = base[(size_t)s * (hs + 2) + hs + 1];
-            if (ls > 0.0f) acc = fmaf(expf(ms - M), base[(size_t)s * (hs + 2) + e], acc);
-        }
-        out[(size_t)h * hs + e] = acc / L;
+#pragma unroll 8
+        for (uint32_t s = 0; s < n_splits; ++s) acc = fmaf(sw[s], base[(size_t)s * (hs + 2) + e], acc);
+        out[(size_t)h * hs + e] = acc;
     }
 }
 
@@ -211,7 +215,7 @@ size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n
 }
 
 hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
-    if (a.head_size > MAX_HS || a.head_size % 2 || a.head_size / 2 > ATT_THREADS || a.n_splits == 0) return hipErrorInvalidValue;
+    if (a.head_size > MAX_HS || a.head_size % 2 || a.head_size / 2 > ATT_THREADS || a.n_splits == 0 || a.n_splits > 64) return hipErrorInvalidValue;
     const uint32_t max_split_len = (a.seq_len + a.n_splits - 1) / a.n_splits;
     const size_t smem = (size_t)max_split_len * sizeof(float);
     if (smem > 48 * 1024) return hipErrorInvalidValue;

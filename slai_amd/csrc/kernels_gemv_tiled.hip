@@ -20,9 +20,17 @@ __device__ __forceinline__ float gelu_f(float x) {
     return 0.5f * x * (1.0f + tanhf(SQRT_2_OVER_PI * x * (1.0f + GELU_COEF_A * x * x)));
 }
 
+// Sum over each 16-lane DPP row, result in every lane of the row: an inclusive scan with row_shr
+// (lanes shifted in from outside the row read 0), then lane 15 is broadcast to the row.
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float row16_sum(float v) {
-    v += __shfl_xor(v, 1, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 4, 64); v += __shfl_xor(v, 8, 64);
-    return v;
+    v += dpp_mov<0x111>(v);   // row_shr:1
+    v += dpp_mov<0x112>(v);   // row_shr:2
+    v += dpp_mov<0x114>(v);   // row_shr:4
+    v += dpp_mov<0x118>(v);   // row_shr:8
+    return dpp_mov<0x15F>(v); // row_newbcast:15
 }
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -63,8 +71,10 @@ template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, 
     else tail = 0;
 }
 
-// NU = tiles per workgroup whose loads are issued before any arithmetic (2 matrices when DUAL).
-template <int T, bool DUAL, int NU, int MAXT>
+// One workgroup = `ngroups` waves; wave w owns column group w of every tile the workgroup visits.  The
+// workgroup walks its tiles with a stride of the segment's workgroup count; the next tile's weights
+// are requested before the current tile is consumed.
+template <int T, bool DUAL, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams p) {
     using F = Tiled<T>;
     extern __shared__ float smem[];
@@ -72,35 +82,44 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     const int ROWS = 1 << p.rows_log2, KQ = 64 >> p.rows_log2;
     const int lane16 = lane & 15;
     const int kq = lane >> p.rows_log2;
-    float *partial = smem;                                          // [NU][DUAL?2:1][NW][64]
-    float *red = smem + (size_t)NU * (DUAL ? 2 : 1) * NW * 64;      // [NW]
+    float *partial = smem;                                   // [DUAL?2:1][NW][64]
+    float *red = smem + (size_t)(DUAL ? 2 : 1) * NW * 64;    // [NW]
 
     int s = 0;
     uint32_t blk = blockIdx.x;
     while (s < p.nseg - 1 && blk >= p.seg[s].nblocks) { blk -= p.seg[s].nblocks; ++s; }
     const GemvTiledSeg &seg = p.seg[s];
     const uint32_t ntiles = (seg.nrows + ROWS - 1) >> p.rows_log2;
+    const uint32_t step = seg.nblocks;
 
-    // ---- issue every weight load of this workgroup first: they do not depend on x ------------
-    const uint32_t g = wave;                                        // column group owned by this wave
-    typename F::Data d[NU];
-    typename F::Data d2[DUAL ? NU : 1];
-    uint16_t tail[NU], tail2[DUAL ? NU : 1];
-#pragma unroll
-    for (int u = 0; u < NU; ++u) {
-        const uint32_t tile = min(blk * NU + u, ntiles - 1);
-        const size_t off = ((size_t)tile * p.ngroups + g) * p.unit_bytes;
-        load_unit<T>(seg.W + off, lane, d[u], tail[u]);
-        if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, d2[u], tail2[u]);
-    }
-
-    // ---- activations of this wave's super-blocks ---------------------------------------------------
-    DevX X;
+    // ---- requests first: activations (small, cache resident), then the first tile's weights --------
+    const uint32_t g = wave;                                 // column group owned by this wave
     const uint32_t cb = g * KQ + kq;
     const bool valid = cb < p.ncb;
-    const float *xp = p.x + (size_t)(valid ? cb : 0) * 256 + lane16;
+    const size_t xoff = (size_t)(valid ? cb : 0) * 256 + lane16;
+    DevX X;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) X.x[i] = valid ? xp[16 * i] : 0.0f;
+    for (int i = 0; i < 16; ++i) X.x[i] = p.x[xoff + 16 * i];
+    float nw[16], nb[16];
+    if (p.prologue != PRO_NONE) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) nw[i] = p.norm_w[xoff + 16 * i];
+        if (p.norm_b) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) nb[i] = p.norm_b[xoff + 16 * i];
+        }
+    }
+    typename F::Data d, dn;
+    typename F::Data d2, d2n;
+    uint16_t tail = 0, tailn = 0, tail2 = 0, tail2n = 0;
+    uint32_t tile = blk;
+    {
+        const size_t off = ((size_t)min(tile, ntiles - 1) * p.ngroups + g) * p.unit_bytes;
+        load_unit<T>(seg.W + off, lane, d, tail);
+        if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, d2, tail2);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) X.x[i] = valid ? X.x[i] : 0.0f;
 
     if (p.prologue != PRO_NONE) {
         // every activation is held by ROWS/16 DPP rows; count it once
@@ -133,58 +152,70 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
         for (int w = 0; w < NW; ++w) t += red[w];
         const float eps = p.eps_ptr ? *p.eps_ptr : p.eps;
         const float scale = 1.0f / sqrtf(t / n + eps);    // rms_norm.slang:60-66 / ops/layernorm.rs:104-111
-        const float *wp = p.norm_w + (size_t)(valid ? cb : 0) * 256 + lane16;
-        const float *bp = p.norm_b ? p.norm_b + (size_t)(valid ? cb : 0) * 256 + lane16 : nullptr;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            float v = X.x[i] * scale;
-            if (valid) { v = v * wp[16 * i]; if (bp) v += bp[16 * i]; }
-            X.x[i] = v;
+            float v = (X.x[i] * scale) * nw[i];
+            if (p.norm_b) v += nb[i];
+            X.x[i] = valid ? v : 0.0f;
         }
     }
+    if constexpr (T == T_Q6_K) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) X.s[i] = row16_sum(X.x[i]);
+        for (int i = 0; i < 16; ++i) X.s[i] = row16_sum(X.x[i]);
+    } else {
+        // Q4_K and Q8_0 only use sums over 32 consecutive activations: reduce pairs, keep the odd slots 0
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) { X.s[i] = row16_sum(X.x[i] + X.x[i + 1]); X.s[i + 1] = 0.0f; }
+    }
 
-    // ---- per-lane row dot products ------------------------------------------------------------------
-#pragma unroll
-    for (int u = 0; u < NU; ++u) {
-        float v = F::dot(d[u], tail[u], X);
+    // ---- tiles ------------------------------------------------------------------------------------------
+    while (tile < ntiles) {
+        const uint32_t next = tile + step;
+        if (next < ntiles) {
+            const size_t off = ((size_t)next * p.ngroups + g) * p.unit_bytes;
+            load_unit<T>(seg.W + off, lane, dn, tailn);
+            if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, d2n, tail2n);
+        }
+        float v = F::dot(d, tail, X);
         for (int m = ROWS; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);     // across the KQ super-blocks of the wave
-        if (lane < ROWS) partial[((u * (DUAL ? 2 : 1)) * NW + wave) * 64 + lane] = v;
+        if (lane < ROWS) partial[wave * 64 + lane] = v;
         if constexpr (DUAL) {
-            float v2 = F::dot(d2[u], tail2[u], X);
+            float v2 = F::dot(d2, tail2, X);
             for (int m = ROWS; m < 64; m <<= 1) v2 += __shfl_xor(v2, m, 64);
-            if (lane < ROWS) partial[((u * 2 + 1) * NW + wave) * 64 + lane] = v2;
+            if (lane < ROWS) partial[(NW + wave) * 64 + lane] = v2;
         }
-    }
-    __syncthreads();
-
-    // ---- epilogue: one thread per output row ----------------------------------------------------------
-    if (tid < NU * ROWS) {
-        const int u = tid >> p.rows_log2, r = tid & (ROWS - 1);
-        const uint32_t tile = blk * NU + u;
-        const uint32_t row = tile * ROWS + r;
-        if (tile < ntiles && row < seg.nrows) {
-            float v = 0.0f;
-            for (int w = 0; w < NW; ++w) v += partial[((u * (DUAL ? 2 : 1)) * NW + w) * 64 + r];
-            if constexpr (DUAL) {
-                float up = 0.0f;
-                for (int w = 0; w < NW; ++w) up += partial[((u * 2 + 1) * NW + w) * 64 + r];
-                v = up * (v / (1.0f + expf(-v)));          // silu.slang:8-26
+        __syncthreads();
+        // epilogue: one thread per output row
+        if (tid < ROWS) {
+            const uint32_t row = tile * ROWS + tid;
+            if (row < seg.nrows) {
+                float o = 0.0f;
+                for (int w = 0; w < NW; ++w) o += partial[w * 64 + tid];
+                if constexpr (DUAL) {
+                    float up = 0.0f;
+                    for (int w = 0; w < NW; ++w) up += partial[(NW + w) * 64 + tid];
+                    o = up * (o / (1.0f + expf(-o)));          // silu.slang:8-26
+                }
+                if (seg.flags & GEMV_BIAS) o += seg.bias[row];
+                if (seg.flags & GEMV_GELU) o = gelu_f(o);
+                if (seg.flags & GEMV_ACCUM) o = seg.out[row] + o;
+                seg.out[row] = o;
             }
-            if (seg.flags & GEMV_BIAS) v += seg.bias[row];
-            if (seg.flags & GEMV_GELU) v = gelu_f(v);
-            if (seg.flags & GEMV_ACCUM) v = seg.out[row] + v;
-            seg.out[row] = v;
         }
+        if (next < ntiles) {
+            __syncthreads();                                   // partial[] is reused by the next tile
+            d = dn; tail = tailn;
+            if constexpr (DUAL) { d2 = d2n; tail2 = tail2n; }
+        }
+        tile = next;
     }
 }
 
-template <int T, bool DUAL, int NU>
+template <int T, bool DUAL>
 hipError_t go(hipStream_t s, const GemvTiledParams &p, dim3 grid, int NT, size_t smem) {
-    if (NT <= 256) gemv_tiled_kernel<T, DUAL, NU, 256><<<grid, NT, smem, s>>>(p);
-    else if (NT <= 512) gemv_tiled_kernel<T, DUAL, NU, 512><<<grid, NT, smem, s>>>(p);
-    else gemv_tiled_kernel<T, DUAL, NU, 1024><<<grid, NT, smem, s>>>(p);
+    if (NT <= 256) gemv_tiled_kernel<T, DUAL, 256><<<grid, NT, smem, s>>>(p);
+    else if (NT <= 512) gemv_tiled_kernel<T, DUAL, 512><<<grid, NT, smem, s>>>(p);
+    else gemv_tiled_kernel<T, DUAL, 1024><<<grid, NT, smem, s>>>(p);
     return hipGetLastError();
 }
 
@@ -198,21 +229,23 @@ template <int T> hipError_t launch_t(slai_ctx *ctx, GemvTiledParams &p) {
         total_tiles += (p.seg[i].nrows + rows - 1) / rows;
         if (p.seg[i].flags & GEMV_SILU_GATE) dual = true;
     }
-    // two tiles per workgroup once there are plenty of tiles and registers allow it
-    int NU = (!dual && NT <= 256 && total_tiles >= 1024 && ctx->gemv_tiles_per_wg >= 2) ? 2 : 1;
-    if (T == T_Q8_0 && NT > 256) NU = 1;
+    // workgroups: at most `gemv_max_wgs` in total (a small multiple of the CU count), shared between the
+    // segments in proportion to their tile counts
+    const uint32_t cap = (uint32_t)(ctx->gemv_max_wgs > 0 ? ctx->gemv_max_wgs : 512);
     uint32_t total = 0;
     for (int i = 0; i < p.nseg; ++i) {
         const uint32_t nt = (p.seg[i].nrows + rows - 1) / rows;
-        p.seg[i].nblocks = (nt + NU - 1) / NU;
-        total += p.seg[i].nblocks;
+        uint32_t nb = total_tiles <= cap ? nt : (uint32_t)(((uint64_t)nt * cap + total_tiles - 1) / total_tiles);
+        if (nb < 1) nb = 1;
+        if (nb > nt) nb = nt;
+        p.seg[i].nblocks = nb;
+        total += nb;
     }
     const int NW = NT / 64;
-    const size_t smem = ((size_t)NU * (dual ? 2 : 1) * NW * 64 + NW) * sizeof(float);
+    const size_t smem = ((size_t)(dual ? 2 : 1) * NW * 64 + NW) * sizeof(float);
     dim3 grid(total);
-    if (dual) return go<T, true, 1>(ctx->stream, p, grid, NT, smem);
-    if (NU == 2) return go<T, false, 2>(ctx->stream, p, grid, NT, smem);
-    return go<T, false, 1>(ctx->stream, p, grid, NT, smem);
+    if (dual) return go<T, true>(ctx->stream, p, grid, NT, smem);
+    return go<T, false>(ctx->stream, p, grid, NT, smem);
 }
 
 }  // namespace

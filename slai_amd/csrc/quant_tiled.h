@@ -137,7 +137,9 @@ SLAI_HD float tiled_dequant_elem(const TiledGeom &g, const uint8_t *base, uint32
 //   X.fma4<I,W>(w, acc) -> acc + sum_{b<4} byte_b(w) * x[16*I + 4*W + b]
 //        (device: four byte->float conversions and four v_fmac_f32 whose x operand is a
 //         row_newbcast DPP read of register I)
-//   X.sum16(I)   -> sum_k x[16*I + k]  (row sums, loop invariant, precomputed)
+//   X.sum16(I)   -> sum_k x[16*I + k]  (row sums, loop invariant, precomputed).  Q4_K and Q8_0 only
+//                   ever use sum16(2n) + sum16(2n+1); an accessor may keep that pair sum in the even
+//                   slot and 0 in the odd one.
 // ---------------------------------------------------------------------------
 template <int I, class X> SLAI_HD float piece_dot(const X &x, const U4 &q, float acc) {
     // q holds sixteen unsigned byte values; byte k pairs with x[16*I + k]:  acc += q_k * x[16*I + k]
@@ -146,6 +148,15 @@ template <int I, class X> SLAI_HD float piece_dot(const X &x, const U4 &q, float
     acc = x.template fma4<I, 2>(q.z, acc);
     acc = x.template fma4<I, 3>(q.w, acc);
     return acc;
+}
+
+// Two independent accumulation chains interleaved word by word (keeps the FMA pipeline fed when a
+// SIMD holds a single wave).
+template <int I1, int I2, class X> SLAI_HD void piece_dot2(const X &x, const U4 &q1, const U4 &q2, float &a1, float &a2) {
+    a1 = x.template fma4<I1, 0>(q1.x, a1); a2 = x.template fma4<I2, 0>(q2.x, a2);
+    a1 = x.template fma4<I1, 1>(q1.y, a1); a2 = x.template fma4<I2, 1>(q2.y, a2);
+    a1 = x.template fma4<I1, 2>(q1.z, a1); a2 = x.template fma4<I2, 2>(q2.z, a2);
+    a1 = x.template fma4<I1, 3>(q1.w, a1); a2 = x.template fma4<I2, 3>(q2.w, a2);
 }
 
 template <int T> struct Tiled;
@@ -157,10 +168,9 @@ template <> struct Tiled<T_Q4_K> {
     template <int J, class X> SLAI_HD static void pair(const Data &d, const X &x, uint32_t scw, uint32_t mw, float &accd, float &accm) {
         // sub-blocks 2J (low nibbles) and 2J+1 (high nibbles) of qs pieces 2J, 2J+1
         const U4 &a = d.p[1 + 2 * J], &b = d.p[2 + 2 * J];
-        float slo = piece_dot<4 * J>(x, and4(a, 0x0F0F0F0Fu), 0.0f);
-        slo = piece_dot<4 * J + 1>(x, and4(b, 0x0F0F0F0Fu), slo);
-        float shi = piece_dot<4 * J + 2>(x, and4(shr4(a, 4), 0x0F0F0F0Fu), 0.0f);
-        shi = piece_dot<4 * J + 3>(x, and4(shr4(b, 4), 0x0F0F0F0Fu), shi);
+        float slo = 0.0f, shi = 0.0f;
+        piece_dot2<4 * J, 4 * J + 2>(x, and4(a, 0x0F0F0F0Fu), and4(shr4(a, 4), 0x0F0F0F0Fu), slo, shi);
+        piece_dot2<4 * J + 1, 4 * J + 3>(x, and4(b, 0x0F0F0F0Fu), and4(shr4(b, 4), 0x0F0F0F0Fu), slo, shi);
         constexpr int sh = (J & 1) * 16;
         accd = fmaf((float)((scw >> sh) & 0xffu), slo, accd);
         accd = fmaf((float)((scw >> (sh + 8)) & 0xffu), shi, accd);
@@ -199,10 +209,13 @@ template <> struct Tiled<T_Q6_K> {
         const U4 q4 = or4(and4(shr4(ql32, 4), 0x0F0F0F0Fu), shl4(and4(shr4(qh, 6), 0x03030303u), 4));
         const float s0 = (float)(int8_t)((scw >> (8 * M)) & 0xff), s1 = (float)(int8_t)((scw >> (8 * (M + 2))) & 0xff);
         const float s2 = (float)(int8_t)((scw2 >> (8 * M)) & 0xff), s3 = (float)(int8_t)((scw2 >> (8 * (M + 2))) & 0xff);
-        acc = fmaf(s0, piece_dot<8 * I + M>(x, q1, 0.0f) - 32.0f * x.sum16(8 * I + M), acc);
-        acc = fmaf(s1, piece_dot<8 * I + 2 + M>(x, q2, 0.0f) - 32.0f * x.sum16(8 * I + 2 + M), acc);
-        acc = fmaf(s2, piece_dot<8 * I + 4 + M>(x, q3, 0.0f) - 32.0f * x.sum16(8 * I + 4 + M), acc);
-        acc = fmaf(s3, piece_dot<8 * I + 6 + M>(x, q4, 0.0f) - 32.0f * x.sum16(8 * I + 6 + M), acc);
+        float t1 = 0.0f, t2 = 0.0f, t3 = 0.0f, t4 = 0.0f;
+        piece_dot2<8 * I + M, 8 * I + 2 + M>(x, q1, q2, t1, t2);
+        piece_dot2<8 * I + 4 + M, 8 * I + 6 + M>(x, q3, q4, t3, t4);
+        acc = fmaf(s0, t1 - 32.0f * x.sum16(8 * I + M), acc);
+        acc = fmaf(s1, t2 - 32.0f * x.sum16(8 * I + 2 + M), acc);
+        acc = fmaf(s2, t3 - 32.0f * x.sum16(8 * I + 4 + M), acc);
+        acc = fmaf(s3, t4 - 32.0f * x.sum16(8 * I + 6 + M), acc);
         return acc;
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
@@ -221,9 +234,9 @@ template <> struct Tiled<T_Q8_0> {
     struct Data { U4 p[17]; };
     template <int B, class X> SLAI_HD static float blk(const Data &d, const X &x, uint32_t dword, float acc) {
         // block B of the cblock: qs pieces 2B, 2B+1; int8 -> unsigned via ^0x80, the 128 comes back through the sums
-        float s = piece_dot<2 * B>(x, xor4(d.p[2 * B], 0x80808080u), 0.0f);
-        s = piece_dot<2 * B + 1>(x, xor4(d.p[2 * B + 1], 0x80808080u), s);
-        s -= 128.0f * (x.sum16(2 * B) + x.sum16(2 * B + 1));
+        float s = 0.0f, s2 = 0.0f;
+        piece_dot2<2 * B, 2 * B + 1>(x, xor4(d.p[2 * B], 0x80808080u), xor4(d.p[2 * B + 1], 0x80808080u), s, s2);
+        s = (s + s2) - 128.0f * (x.sum16(2 * B) + x.sum16(2 * B + 1));
         const float dd = decode_f16((uint16_t)((B & 1) ? (dword >> 16) : (dword & 0xffffu)));
         return fmaf(dd, s, acc);
     }

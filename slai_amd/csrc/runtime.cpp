@@ -79,7 +79,7 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->gemv_max_threads = env_int("SLAI_GEMV_MAX_THREADS", 512);
     ctx->attn_splits = env_int("SLAI_ATTN_SPLITS", 0);
     ctx->use_graph = env_int("SLAI_NO_GRAPH", 0) == 0;
-    ctx->gemv_tiles_per_wg = env_int("SLAI_GEMV_TILES_PER_WG", 2);
+    ctx->gemv_max_wgs = env_int("SLAI_GEMV_MAX_WGS", 512);
     ctx->tiled_layout = env_int("SLAI_TILED", 1) != 0;
     *out = ctx;
     return SLAI_OK;
