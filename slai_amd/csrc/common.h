@@ -90,7 +90,6 @@ struct GemvParams {
     int prologue = PRO_NONE;
     const float *norm_w = nullptr, *norm_b = nullptr;
     float eps = 0.0f;
-    const float *eps_ptr = nullptr;  // when set, eps is read from device memory
     uint32_t rows_per_wg = 8;
 };
 // All segments share the ggml type `type`, the input x and the prologue.
@@ -115,7 +114,6 @@ struct GemvTiledParams {
     int prologue = PRO_NONE;
     const float *norm_w = nullptr, *norm_b = nullptr;
     float eps = 0.0f;
-    const float *eps_ptr = nullptr;
 };
 hipError_t launch_gemv_tiled(slai_ctx *ctx, int type, GemvTiledParams p);
 
@@ -131,7 +129,6 @@ struct GemvCall {
     int prologue = PRO_NONE;
     const float *norm_w = nullptr, *norm_b = nullptr;
     float eps = 0.0f;
-    const float *eps_ptr = nullptr;
 };
 // Returns SLAI_OK or an error code with the message set on ctx.
 int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who);

@@ -84,7 +84,7 @@ __global__ void __launch_bounds__(MAXT) gemv_kernel(const GemvParams p) {
 
     // ---- prologue: normalise x in registers ---------------------------------------
     if (p.prologue != PRO_NONE) {
-        const float eps = p.eps_ptr ? *p.eps_ptr : p.eps;
+        const float eps = p.eps;
         const float n = (float)p.ncols;
         float mean = 0.0f;
         if (p.prologue == PRO_LAYERNORM) {

@@ -15,6 +15,15 @@
 namespace slai {
 namespace {
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, which on
+// this target means waiting for every outstanding global load (vmcnt(0)) -- it would serialise the
+// weight stream behind each reduction step.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ float gelu_f(float x) {
     const float GELU_COEF_A = 0.044715f, SQRT_2_OVER_PI = 0.7978846f;   // ops/unary.rs:81-85
     return 0.5f * x * (1.0f + tanhf(SQRT_2_OVER_PI * x * (1.0f + GELU_COEF_A * x * x)));
@@ -109,14 +118,23 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
             for (int i = 0; i < 16; ++i) nb[i] = p.norm_b[xoff + 16 * i];
         }
     }
-    typename F::Data d, dn;
-    typename F::Data d2, d2n;
-    uint16_t tail = 0, tailn = 0, tail2 = 0, tail2n = 0;
+    // two register buffers used alternately: while one tile is consumed the other one's loads are in flight
+    typename F::Data dA, dB;
+    typename F::Data eA, eB;                                 // second matrix of a gated pair
+    uint16_t tA = 0, tB = 0, uA = 0, uB = 0;
     uint32_t tile = blk;
+    float old0 = 0.0f, bias0 = 0.0f;
+    {
+        const uint32_t row = tile * ROWS + tid;
+        if (tid < ROWS && tile < ntiles && row < seg.nrows) {
+            if (seg.flags & GEMV_ACCUM) old0 = seg.out[row];
+            if (seg.flags & GEMV_BIAS) bias0 = seg.bias[row];
+        }
+    }
     {
         const size_t off = ((size_t)min(tile, ntiles - 1) * p.ngroups + g) * p.unit_bytes;
-        load_unit<T>(seg.W + off, lane, d, tail);
-        if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, d2, tail2);
+        load_unit<T>(seg.W + off, lane, dA, tA);
+        if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, eA, uA);
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i) X.x[i] = valid ? X.x[i] : 0.0f;
@@ -132,11 +150,11 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
             for (int i = 0; i < 16; ++i) sm += X.x[i];
             sm = wave_sum(counted ? sm : 0.0f);
             if (lane == 0) red[wave] = sm;
-            __syncthreads();
+            lds_barrier();
             float t = 0.0f;
             for (int w = 0; w < NW; ++w) t += red[w];
             mean = t / n;
-            __syncthreads();
+            lds_barrier();
         }
         float ss = 0.0f;
 #pragma unroll
@@ -147,11 +165,10 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
         }
         ss = wave_sum(counted ? ss : 0.0f);
         if (lane == 0) red[wave] = ss;
-        __syncthreads();
+        lds_barrier();
         float t = 0.0f;
         for (int w = 0; w < NW; ++w) t += red[w];
-        const float eps = p.eps_ptr ? *p.eps_ptr : p.eps;
-        const float scale = 1.0f / sqrtf(t / n + eps);    // rms_norm.slang:60-66 / ops/layernorm.rs:104-111
+        const float scale = 1.0f / sqrtf(t / n + p.eps);    // rms_norm.slang:60-66 / ops/layernorm.rs:104-111
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             float v = (X.x[i] * scale) * nw[i];
@@ -169,25 +186,30 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     }
 
     // ---- tiles ------------------------------------------------------------------------------------------
-    while (tile < ntiles) {
-        const uint32_t next = tile + step;
-        if (next < ntiles) {
-            const size_t off = ((size_t)next * p.ngroups + g) * p.unit_bytes;
-            load_unit<T>(seg.W + off, lane, dn, tailn);
-            if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, d2n, tail2n);
+    // Loads are retired in issue order, so everything the epilogue reads from global memory (the value
+    // accumulated into, the bias) is requested BEFORE the next tile's weights; waiting for it then does
+    // not wait for the weight stream.
+    auto epi_request = [&](uint32_t t, float &old, float &bias) {
+        old = 0.0f; bias = 0.0f;
+        const uint32_t row = t * ROWS + tid;
+        if (tid < ROWS && row < seg.nrows) {
+            if (seg.flags & GEMV_ACCUM) old = seg.out[row];
+            if (seg.flags & GEMV_BIAS) bias = seg.bias[row];
         }
-        float v = F::dot(d, tail, X);
+    };
+    auto consume = [&](const typename F::Data &d, uint16_t dt, const typename F::Data &e, uint16_t et, uint32_t t, bool more,
+                       float old, float bias) {
+        float v = F::dot(d, dt, X);
         for (int m = ROWS; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);     // across the KQ super-blocks of the wave
         if (lane < ROWS) partial[wave * 64 + lane] = v;
         if constexpr (DUAL) {
-            float v2 = F::dot(d2, tail2, X);
+            float v2 = F::dot(e, et, X);
             for (int m = ROWS; m < 64; m <<= 1) v2 += __shfl_xor(v2, m, 64);
             if (lane < ROWS) partial[(NW + wave) * 64 + lane] = v2;
         }
-        __syncthreads();
-        // epilogue: one thread per output row
-        if (tid < ROWS) {
-            const uint32_t row = tile * ROWS + tid;
+        lds_barrier();
+        if (tid < ROWS) {                                      // epilogue: one thread per output row
+            const uint32_t row = t * ROWS + tid;
             if (row < seg.nrows) {
                 float o = 0.0f;
                 for (int w = 0; w < NW; ++w) o += partial[w * 64 + tid];
@@ -196,18 +218,33 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
                     for (int w = 0; w < NW; ++w) up += partial[(NW + w) * 64 + tid];
                     o = up * (o / (1.0f + expf(-o)));          // silu.slang:8-26
                 }
-                if (seg.flags & GEMV_BIAS) o += seg.bias[row];
+                if (seg.flags & GEMV_BIAS) o += bias;
                 if (seg.flags & GEMV_GELU) o = gelu_f(o);
-                if (seg.flags & GEMV_ACCUM) o = seg.out[row] + o;
+                if (seg.flags & GEMV_ACCUM) o = old + o;
                 seg.out[row] = o;
             }
         }
-        if (next < ntiles) {
-            __syncthreads();                                   // partial[] is reused by the next tile
-            d = dn; tail = tailn;
-            if constexpr (DUAL) { d2 = d2n; tail2 = tail2n; }
+        if (more) lds_barrier();                               // partial[] is reused by the next tile
+    };
+    auto request = [&](typename F::Data &d, uint16_t &dt, typename F::Data &e, uint16_t &et, uint32_t t) {
+        const size_t off = ((size_t)t * p.ngroups + g) * p.unit_bytes;
+        load_unit<T>(seg.W + off, lane, d, dt);
+        if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, e, et);
+    };
+    if (tile < ntiles) {
+        float old = old0, bias = bias0;
+        for (;;) {
+            uint32_t next = tile + step;
+            float oldn = 0.0f, biasn = 0.0f;
+            if (next < ntiles) { epi_request(next, oldn, biasn); request(dB, tB, eB, uB, next); }
+            consume(dA, tA, eA, uA, tile, next < ntiles, old, bias);
+            if (next >= ntiles) break;
+            tile = next; next = tile + step;
+            if (next < ntiles) { epi_request(next, old, bias); request(dA, tA, eA, uA, next); }
+            consume(dB, tB, eB, uB, tile, next < ntiles, oldn, biasn);
+            if (next >= ntiles) break;
+            tile = next;
         }
-        tile = next;
     }
 }
 

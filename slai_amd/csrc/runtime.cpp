@@ -267,7 +267,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who) {
         GemvTiledParams p;
         p.nseg = c.nseg; p.ncols = m0->ncols; p.ncb = m0->ncb; p.ngroups = m0->ngroups; p.rows_log2 = m0->rows_log2;
         p.unit_bytes = m0->unit_bytes; p.x = c.x; p.prologue = c.prologue; p.norm_w = c.norm_w; p.norm_b = c.norm_b;
-        p.eps = c.eps; p.eps_ptr = c.eps_ptr;
+        p.eps = c.eps;
         for (int i = 0; i < c.nseg; ++i) {
             p.seg[i].W = c.m[i]->dptr; p.seg[i].W2 = c.m2[i] ? c.m2[i]->dptr : nullptr; p.seg[i].nrows = c.m[i]->nrows;
             p.seg[i].out = c.out[i]; p.seg[i].bias = c.bias[i]; p.seg[i].flags = c.flags[i];
@@ -277,7 +277,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who) {
         if (!gemv_supports(m0->type, m0->ncols)) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported column count for this format");
         GemvParams p;
         p.nseg = c.nseg; p.ncols = m0->ncols; p.nb = m0->nb; p.x = c.x; p.prologue = c.prologue; p.norm_w = c.norm_w;
-        p.norm_b = c.norm_b; p.eps = c.eps; p.eps_ptr = c.eps_ptr; p.rows_per_wg = ctx->gemv_rows_per_wg;
+        p.norm_b = c.norm_b; p.eps = c.eps; p.rows_per_wg = ctx->gemv_rows_per_wg;
         for (int i = 0; i < c.nseg; ++i) {
             p.seg[i].W = c.m[i]->dptr; p.seg[i].W2 = c.m2[i] ? c.m2[i]->dptr : nullptr; p.seg[i].row_stride = c.m[i]->row_stride;
             p.seg[i].nrows = c.m[i]->nrows; p.seg[i].out = c.out[i]; p.seg[i].bias = c.bias[i]; p.seg[i].flags = c.flags[i];
