@@ -28,6 +28,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the dominant kernel moves: rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch (two counter
+# runs of `bench.py --probe`), each scaled by what the same counter reads for the 64 MiB copy kernel of that probe.
+# The summary of those runs is kept under profiles/.
+DOMINANT_KERNEL_TRAFFIC_BYTES = 51415470
 CFG = dict(dim=4096, hidden_dim=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000)
 
 
@@ -74,15 +78,34 @@ def measure_dominant_kernel(backend, reps=20):
     return ms, algo
 
 
-def cpu_baseline(seed, n_tokens=6):
-    """Oracle decode of the same layer shapes at depth 2 and 4 (pos 64..), extrapolated to 32 layers."""
+def counter_probe(backend):
+    """For hardware-counter runs: 64 launches of a plain copy kernel of known size (64 MiB read, 64 MiB
+    written) and the dominant-kernel loop, nothing else, so that per-dispatch FETCH_SIZE / WRITE_SIZE of
+    the GEMV can be scaled by what the same counter reads for the copy."""
+    from slai_amd.runtime import GpuTensor, LlmContext
+    n = 16 * 1024 * 1024
+    a = GpuTensor(backend, n)
+    b = GpuTensor(backend, n)
+    ctxt = LlmContext(backend)
+    for _ in range(64):
+        ctxt.copy(a, b)
+    backend.synchronize()
+    ms, algo = measure_dominant_kernel(backend, reps=8)
+    a.destroy(); b.destroy()
+    print(json.dumps({"probe": "copy kernel 67108864 B read + 67108864 B written per launch (64 launches); "
+                               "gate/up GEMV %d algorithmic bytes per launch" % algo,
+                      "gemv_launch_us": round(ms * 1000, 2)}))
+
+
+def cpu_baseline(seed, n_tokens=32):
+    """Oracle decode of the same layer shapes at depth 2 and 6, extrapolated linearly to 32 layers."""
     import oracle
     from slai_amd import gguf_writer as gw
     L = oracle.load()
     threads = min(16, os.cpu_count() or 1)
     L.slo_set_threads(threads)
     times = {}
-    for nl in (2, 4):
+    for nl in (2, 6):
         data = gw.llama_gguf(dim=CFG["dim"], hidden_dim=CFG["hidden_dim"], n_layers=nl, n_heads=CFG["n_heads"],
                              n_kv_heads=CFG["n_kv_heads"], vocab=CFG["vocab"], seq_len=128, wtype=12, v_type=14,
                              out_type=14, embd_type=12, seed=seed, with_output=True, distinct_layers=2)
@@ -98,12 +121,13 @@ def cpu_baseline(seed, n_tokens=6):
         times[nl] = (time.perf_counter() - t0) / n_tokens
         L.slo_llama2_free(m); L.slo_gguf_free(g)
         del data
-    per_layer = (times[4] - times[2]) / 2.0
+    per_layer = (times[6] - times[2]) / 4.0
     head = max(times[2] - 2 * per_layer, 0.0)
     full = head + CFG["n_layers"] * per_layer
     return dict(value=1.0 / full, unit="tok/s", cores=threads, kind="port",
-                sample="oracle (C restatement of models/llama2/cpu.rs) at the same layer shapes, depth 2 and 4, "
-                       "%d tokens each; per-layer %.3f s + head %.3f s extrapolated to 32 layers" % (n_tokens, per_layer, head))
+                sample="oracle (C restatement of models/llama2/cpu.rs, OpenMP over GEMV rows) on the same layer shapes and "
+                       "quantization at depth 2 and 6, %d tokens each; %.2f ms per layer + %.2f ms embedding/head per token, "
+                       "extrapolated to 32 layers" % (n_tokens, per_layer * 1e3, head * 1e3))
 
 
 def main():
@@ -116,11 +140,18 @@ def main():
     ap.add_argument("--distinct-layers", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--probe", action="store_true", help="counter probe: copy kernel + dominant GEMV only")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the decode path on ONE GPU (batch-1 decode does not shard usefully); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
+    if args.probe:
+        from slai_amd.runtime import Backend
+        backend = Backend(0)
+        counter_probe(backend)
+        backend.close()
+        return
     K, W = args.steps, max(args.warmup, 1)
     cfg = dict(CFG, n_layers=args.layers)
     seq_len = max(512, ((W + K + 63) // 64) * 64)
@@ -161,7 +192,7 @@ def main():
         ach = kalgo / (kms * 1e-3) / 1e9
         roof = dict(bound="hbm", kernel="gemv_kernel<Q4_K, dual> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096)",
                     achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
-                    traffic=None, launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
+                    traffic=DOMINANT_KERNEL_TRAFFIC_BYTES, launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
         log("dominant kernel: %.2f us/launch, %.1f GB/s" % (kms * 1000, ach))
     backend.close()
 

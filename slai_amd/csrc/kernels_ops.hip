@@ -66,11 +66,14 @@ __global__ void layernorm_kernel(VecView out, VecView v, float eps) {
 }
 
 // stensor OpAssign Add / Mul / Copy (context.rs:428-469,660-672)
-__global__ void binop_kernel(int op, VecView a, VecView b) {
+template <int OP>   // 0 add, 1 mul, 2 copy (a <- b; a is not read)
+__global__ void binop_kernel(VecView a, VecView b) {
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < a.n; i += gridDim.x * blockDim.x) {
         float *pa = a.p + (size_t)i * a.stride;
         const float vb = b.p[(size_t)i * b.stride];
-        *pa = op == 0 ? *pa + vb : (op == 1 ? *pa * vb : vb);
+        if constexpr (OP == 0) *pa = *pa + vb;
+        else if constexpr (OP == 1) *pa = *pa * vb;
+        else *pa = vb;
     }
 }
 
@@ -230,7 +233,10 @@ hipError_t launch_layernorm(hipStream_t s, VecView out, VecView v, float eps) {
     return hipGetLastError();
 }
 hipError_t launch_binop(hipStream_t s, int op, VecView a, VecView b) {
-    binop_kernel<<<grid_for(a.n, 256), 256, 0, s>>>(op, a, b);
+    const dim3 grid = grid_for(a.n, 256);
+    if (op == 0) binop_kernel<0><<<grid, 256, 0, s>>>(a, b);
+    else if (op == 1) binop_kernel<1><<<grid, 256, 0, s>>>(a, b);
+    else binop_kernel<2><<<grid, 256, 0, s>>>(a, b);
     return hipGetLastError();
 }
 hipError_t launch_silu(hipStream_t s, VecView a, VecView b) {
