@@ -116,6 +116,16 @@ int slai_copy_buffer(slai_ctx *ctx, slai_buffer *dst, size_t dst_offset, const s
  * accepted (no pairing constraint), F16 stays 16-bit. */
 int slai_qmat_create(slai_ctx *ctx, uint32_t ggml_type, uint32_t nrows, uint32_t ncols, const void *packed,
                      slai_qmat **out);
+/* The same with the device layout chosen by the caller.  Layouts are private regroupings of the packed GGUF
+ * bytes; every layout serves every op, they differ in speed.  AUTO picks by shape; ROWS keeps rows contiguous;
+ * TILE16 / TILE64 regroup 16..64-row tiles for the row-per-lane GEMVs (TILE64: matrices that are launched
+ * together over the same input and jointly have many rows, e.g. q/k/v or gate/up). */
+#define SLAI_LAYOUT_AUTO 0
+#define SLAI_LAYOUT_ROWS 1
+#define SLAI_LAYOUT_TILE16 2
+#define SLAI_LAYOUT_TILE64 3
+int slai_qmat_create_layout(slai_ctx *ctx, uint32_t ggml_type, uint32_t nrows, uint32_t ncols, const void *packed,
+                            int layout, slai_qmat **out);
 void slai_qmat_destroy(slai_ctx *ctx, slai_qmat *m);
 /* `GpuQuantMatrix::shape` (quantized_matrix.rs:72-86): [nrows, ncols] in elements, and the type tag. */
 int slai_qmat_shape(const slai_qmat *m, uint32_t *nrows, uint32_t *ncols, uint32_t *ggml_type);
@@ -172,6 +182,19 @@ int slai_ffn_gate_up_silu(slai_ctx *ctx, slai_view out_hb, const slai_qmat *gate
                           slai_view norm_weight, float eps);
 /* matmul_quant_assign(xb2, m, v) + add_assign(x, xb2)   (transformer.rs:352-355, 362-365) */
 int slai_matmul_quant_add_assign(slai_ctx *ctx, slai_view in_out_x, const slai_qmat *m, slai_view v);
+/* "Prepared" activations: for an input x and the weight w of the RMSNorm that follows it, the n products x[i]*w[i]
+ * followed by the n/16 sums of 16 consecutive products (n + n/16 contiguous floats, 64-byte aligned, n % 16 == 0).
+ * A GEMV over a TILE64 matrix that is handed this form reads its activations directly and only derives the norm's
+ * scale from x; it equals slai_rms_norm_assign + slai_matmul_quant_assign.  slai_rms_norm_prepare builds the form
+ * from x; slai_matmul_quant_add_assign_emit is slai_matmul_quant_add_assign that also leaves the form of its result
+ * (with the weight of the norm that comes next) for the GEMV after it, so that no separate pass is needed. */
+int slai_rms_norm_prepare(slai_ctx *ctx, slai_view out_prepared, slai_view x, slai_view norm_weight);
+int slai_rms_norm_matmul_quant_assign_prepared(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view prepared,
+                                               float eps);
+int slai_ffn_gate_up_silu_prepared(slai_ctx *ctx, slai_view out_hb, const slai_qmat *gate, const slai_qmat *up, slai_view x,
+                                   slai_view prepared, float eps);
+int slai_matmul_quant_add_assign_emit(slai_ctx *ctx, slai_view in_out_x, const slai_qmat *m, slai_view v, slai_view next_norm_weight,
+                                      slai_view out_prepared);
 
 /* ---- GPU timing on the context's stream with HIP events: the role of the GPU timestamp
  * queries bracketing a pass in crates/slai-bench/src/main.rs:198,223-241.  slai_timer_end
@@ -205,6 +228,7 @@ int slai_gguf_meta_str(const slai_gguf *g, const char *key, const char **out);
 int slai_gguf_meta_array_len(const slai_gguf *g, const char *key, uint64_t *out);
 /* `GgufTensor::to_gpu_matrix` (gguf.rs:357-366) */
 int slai_gguf_tensor_to_qmat(slai_ctx *ctx, const slai_gguf *g, const char *name, slai_qmat **out);
+int slai_gguf_tensor_to_qmat_layout(slai_ctx *ctx, const slai_gguf *g, const char *name, int layout, slai_qmat **out);
 
 /* ---- Llama-2 / Qwen2 model assembly ------------------------------------------
  * `ChatLlama2::from_gguf_with_model_type` (crates/slai-chat/src/chat_llama2.rs:39-62):

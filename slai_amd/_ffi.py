@@ -15,6 +15,7 @@ ROPE_ORIGINAL, ROPE_NEOX = 0, 1
 MODE_N, MODE_T = 0, 1
 MODEL_LLAMA, MODEL_QWEN2 = 0, 1
 KV_F32, KV_F16 = 0, 1
+LAYOUT_AUTO, LAYOUT_ROWS, LAYOUT_TILE16, LAYOUT_TILE64 = 0, 1, 2, 3
 
 
 class View(C.Structure):
@@ -63,6 +64,7 @@ SIGNATURES = {
     "slai_read_buffer": (i32, [vp, vp, sz, vp, sz]),
     "slai_copy_buffer": (i32, [vp, vp, sz, vp, sz, sz]),
     "slai_qmat_create": (i32, [vp, u32, u32, u32, vp, P(vp)]),
+    "slai_qmat_create_layout": (i32, [vp, u32, u32, u32, vp, i32, P(vp)]),
     "slai_qmat_destroy": (None, [vp, vp]),
     "slai_qmat_shape": (i32, [vp, P(u32), P(u32), P(u32)]),
     "slai_qmat_device_bytes": (sz, [vp]),
@@ -74,6 +76,10 @@ SIGNATURES = {
     "slai_rms_norm_matmul_quant_assign": (i32, [vp, View, vp, View, View, C.c_float]),
     "slai_ffn_gate_up_silu": (i32, [vp, View, vp, vp, View, View, C.c_float]),
     "slai_matmul_quant_add_assign": (i32, [vp, View, vp, View]),
+    "slai_rms_norm_prepare": (i32, [vp, View, View, View]),
+    "slai_rms_norm_matmul_quant_assign_prepared": (i32, [vp, View, vp, View, View, C.c_float]),
+    "slai_ffn_gate_up_silu_prepared": (i32, [vp, View, vp, vp, View, View, C.c_float]),
+    "slai_matmul_quant_add_assign_emit": (i32, [vp, View, vp, View, View, View]),
     "slai_add_assign": (i32, [vp, View, View]),
     "slai_mul_assign": (i32, [vp, View, View]),
     "slai_copy": (i32, [vp, View, View]),
@@ -103,6 +109,7 @@ SIGNATURES = {
     "slai_gguf_meta_str": (i32, [vp, C.c_char_p, P(C.c_char_p)]),
     "slai_gguf_meta_array_len": (i32, [vp, C.c_char_p, P(u64)]),
     "slai_gguf_tensor_to_qmat": (i32, [vp, vp, C.c_char_p, P(vp)]),
+    "slai_gguf_tensor_to_qmat_layout": (i32, [vp, vp, C.c_char_p, i32, P(vp)]),
     "slai_llama2_from_gguf": (i32, [vp, vp, i32, i32, P(vp)]),
     "slai_llama2_destroy": (None, [vp]),
     "slai_llama2_get_config": (i32, [vp, P(Llama2Config)]),

@@ -42,11 +42,15 @@ struct slai_ctx {
     // attention split-K partials (grown on demand, never inside a capture)
     float *attn_scratch = nullptr;
     size_t attn_scratch_floats = 0;
+    // per-workgroup activation slots of the row-tile GEMV (grown on demand, never inside a capture)
+    float *gemv_scratch = nullptr;
+    size_t gemv_scratch_floats = 0;
     // tuning knobs (environment overridable, see runtime.cpp)
     int gemv_rows_per_wg = 8;
     int gemv_max_threads = 1024;
     int gemv_max_wgs = 512;     // workgroups per tiled GEMV launch (SLAI_GEMV_MAX_WGS)
     bool tiled_layout = true;   // SLAI_TILED=0 keeps every matrix in the row layout
+    bool rowtile_gemv = true;   // SLAI_ROWTILE=0: no 64-row tiles / wave-uniform GEMV
     int attn_splits = 0;  // 0 = automatic
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
     bool use_graph = true;  // SLAI_NO_GRAPH=1 replays the token sequence eagerly (profilers that cannot trace graph launches)
@@ -69,6 +73,7 @@ enum : uint32_t {
     GEMV_ACCUM = 2u,     // out[row] += val
     GEMV_SILU_GATE = 4u, // dual: val = up * gate/(1+exp(-gate))   (W = gate, W2 = up)
     GEMV_GELU = 8u,      // val = gelu(val)
+    GEMV_EMIT = 16u,     // also write the weighted copy of the result for the next row-tile GEMV (tiled kernel only)
 };
 enum : int { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_LAYERNORM = 2 };
 
@@ -114,8 +119,39 @@ struct GemvTiledParams {
     int prologue = PRO_NONE;
     const float *norm_w = nullptr, *norm_b = nullptr;
     float eps = 0.0f;
+    const float *emit_w = nullptr;    // GEMV_EMIT (segment 0): weights of the next norm
+    float *emit_out = nullptr;        // [nrows + nrows/16]
 };
 hipError_t launch_gemv_tiled(slai_ctx *ctx, int type, GemvTiledParams p);
+
+// GEMV over 64-row tiles with wave-uniform activations (kernels_gemv_rowtile.hip).  Segments share the
+// input, the prologue and the column count; their block formats may differ.
+struct GemvRowtileSeg {
+    const uint8_t *W = nullptr;
+    const uint8_t *W2 = nullptr;
+    int type = 0;
+    uint32_t nrows = 0;
+    uint32_t ntiles = 0;   // filled by the launcher
+    float *out = nullptr;
+    const float *bias = nullptr;
+    uint32_t flags = 0;
+};
+struct GemvRowtileParams {
+    GemvRowtileSeg seg[3];
+    int nseg = 1;
+    uint32_t ncols = 0, ncb = 0;
+    const float *x = nullptr;
+    int prologue = PRO_NONE;          // PRO_NONE or PRO_RMSNORM
+    const float *norm_w = nullptr;
+    float eps = 0.0f;
+    // When set: the weighted activations followed by their ncols/16 sums of 16, left by the kernel that produced x
+    // (GEMV_EMIT); x itself is then only read for the RMSNorm sum of squares.
+    const float *prepared = nullptr;
+    float *scratch = nullptr;         // one slot of ncols + ncols/16 floats per workgroup (= per tile); unused with `prepared`
+    uint32_t scratch_stride = 0;      // filled by the launcher
+};
+size_t gemv_rowtile_scratch_floats(const GemvRowtileParams &p);
+hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p);
 
 // One GEMV launch over up to three matrices of one format and layout: out[i] = epilogue(m[i] . prologue(x)).
 struct GemvCall {
@@ -129,9 +165,21 @@ struct GemvCall {
     int prologue = PRO_NONE;
     const float *norm_w = nullptr, *norm_b = nullptr;
     float eps = 0.0f;
+    // Producer side (segment 0 only, needs GEMV_EMIT in flags[0]): besides out[0], write emit_out[row] = out[row] *
+    // emit_w[row] and, behind the nrows products, the nrows/16 sums of 16 consecutive products.
+    const float *emit_w = nullptr;
+    float *emit_out = nullptr;
+    // Consumer side: such a copy of norm_w-weighted x (see GemvRowtileParams::prepared); nullptr = none.
+    const float *prepared = nullptr;
 };
+// True when gemv_call would honour GEMV_EMIT for this matrix as segment 0.
+bool gemv_can_emit(const slai_qmat *m);
+// True when gemv_call takes the 64-row-tile path for this matrix (and so can use `prepared`).
+bool gemv_is_rowtile(const slai_ctx *ctx, const slai_qmat *m);
 // Returns SLAI_OK or an error code with the message set on ctx.
 int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who);
+// Makes sure the row-tile GEMV's scratch holds `floats` floats (call outside graph capture).
+int gemv_scratch_reserve(slai_ctx *ctx, size_t floats);
 
 // ---- dequantisation / repack ---------------------------------------------------
 // Device-side description of a quantized matrix in either layout.
@@ -154,6 +202,8 @@ hipError_t launch_rms_norm(hipStream_t s, VecView out, VecView v, VecView w, con
 hipError_t launch_layernorm(hipStream_t s, VecView out, VecView v, float eps);
 hipError_t launch_binop(hipStream_t s, int op /*0 add,1 mul,2 copy(a<-b)*/, VecView a, VecView b);
 hipError_t launch_silu(hipStream_t s, VecView a, VecView b);
+// out[i] = x[i]*w[i] (i < n), out[n + j] = sum of products 16j..16j+15; n % 16 == 0
+hipError_t launch_prepare(hipStream_t s, float *out, const float *x, const float *w, uint32_t n);
 hipError_t launch_gelu(hipStream_t s, VecView a);
 hipError_t launch_rope(hipStream_t s, int variant, const slai_rope_config *cfg_dev, VecView q, VecView k);
 hipError_t launch_attn_mask(hipStream_t s, const slai_attn_params *params_dev, float *attn, uint32_t nthreads);

@@ -222,10 +222,13 @@ SLAI_EXPORT int slai_gguf_meta_array_len(const slai_gguf *g, const char *key, ui
 // gguf.rs:357-366 `GgufTensor::to_gpu_matrix` -> gguf.rs:133-194: packed upload, row-major,
 // without the reference's even-block-count / ncols%{64,512} conditions and f32 fallbacks.
 SLAI_EXPORT int slai_gguf_tensor_to_qmat(slai_ctx *ctx, const slai_gguf *g, const char *name, slai_qmat **out) {
+    return slai_gguf_tensor_to_qmat_layout(ctx, g, name, SLAI_LAYOUT_AUTO, out);
+}
+SLAI_EXPORT int slai_gguf_tensor_to_qmat_layout(slai_ctx *ctx, const slai_gguf *g, const char *name, int layout, slai_qmat **out) {
     if (!ctx || !g || !name || !out) return SLAI_E_ARG;
     const GgufTensorInfo *t = g->g.find(name);
     if (!t) return set_error(ctx, SLAI_E_MISSING, std::string("missing tensor '") + name + "'");
     if (t->dims[2] != 1 || t->dims[3] != 1) return set_error(ctx, SLAI_E_SHAPE, std::string("tensor '") + name + "' is not a matrix");  // gguf.rs:362-363
     if (!block_elems((int)t->type)) return set_error(ctx, SLAI_E_TYPE, std::string("tensor '") + name + "' has ggml type " + std::to_string(t->type) + " which has no device kernel");
-    return slai_qmat_create(ctx, t->type, (uint32_t)t->dims[0], (uint32_t)t->dims[1], g->g.bytes + t->offset, out);
+    return slai_qmat_create_layout(ctx, t->type, (uint32_t)t->dims[0], (uint32_t)t->dims[1], g->g.bytes + t->offset, layout, out);
 }

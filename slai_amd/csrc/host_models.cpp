@@ -8,6 +8,7 @@
 #include "llm_context.h"
 #include "quant_formats.h"
 
+#include <algorithm>
 #include <cstring>
 #include <memory>
 
@@ -33,8 +34,8 @@ int f32_vector_from_gguf(slai_ctx *ctx, const Gguf &g, const std::string &name, 
     uint64_t n = t->dims[0] * t->dims[1] * t->dims[2] * t->dims[3];
     return GpuTensor::vector_from(ctx, reinterpret_cast<const float *>(g.bytes + t->offset), (uint32_t)n, STORAGE, out);
 }
-int qmat_from_gguf(slai_ctx *ctx, const slai_gguf *g, const std::string &name, slai_qmat **out) {
-    return slai_gguf_tensor_to_qmat(ctx, g, name.c_str(), out);
+int qmat_from_gguf(slai_ctx *ctx, const slai_gguf *g, const std::string &name, slai_qmat **out, int layout = SLAI_LAYOUT_AUTO) {
+    return slai_gguf_tensor_to_qmat_layout(ctx, g, name.c_str(), layout, out);
 }
 int meta_u32(slai_ctx *ctx, const Gguf &g, const std::string &key, uint32_t *out) {
     const GgufMetaValue *v = g.meta(key);
@@ -42,6 +43,13 @@ int meta_u32(slai_ctx *ctx, const Gguf &g, const std::string &key, uint32_t *out
     if (v->type != 4) return set_error(ctx, SLAI_E_TYPE, "unwrap: unexpected GGUF attribute type for '" + key + "'");
     *out = (uint32_t)v->u;
     return SLAI_OK;
+}
+
+// Two matrices over the same input can share a GEMV launch: any formats in 64-row tiles, otherwise one format and layout.
+bool same_launch(const slai_qmat *a, const slai_qmat *b) {
+    if (a->tiled && b->tiled && a->rows_log2 == 6 && b->rows_log2 == 6 && (a->type == b->type || (a->type != T_Q8_0 && b->type != T_Q8_0)))
+        return true;
+    return a->type == b->type && a->tiled == b->tiled && (!a->tiled || a->rows_log2 == b->rows_log2);
 }
 
 struct DeviceLoop {           // device-resident state of the greedy loop
@@ -91,6 +99,7 @@ struct Llama2Weights {               // transformer.rs:194-199
 struct Llama2State {                 // transformer.rs:16-44
     GpuTensor x, xb, xb2, hb, hb2, q, att, logits;
     GpuTensor kcol, vcol;            // fresh K/V of the current position (fused path, and staging for f16 caches)
+    GpuTensor xw;                    // fused path: norm-weighted copy of x (+ dim/16 sums of 16) left by the producer of x
     std::vector<GpuTensor> key_cache, value_cache;
     slai_buffer *rope_config = nullptr, *rms_norm_config = nullptr, *attn_params = nullptr;
 };
@@ -149,16 +158,16 @@ int slai_llama2::load(const slai_gguf *gg) {
     for (uint32_t l = 0; l < config.n_layers; ++l) {
         Llama2LayerWeights &w = weights.layers[l];
         const std::string p = "blk." + std::to_string(l) + ".";
-        TRY(qmat_from_gguf(ctx, gg, p + "attn_q.weight", &w.attn_q));
-        TRY(qmat_from_gguf(ctx, gg, p + "attn_k.weight", &w.attn_k));
-        TRY(qmat_from_gguf(ctx, gg, p + "attn_v.weight", &w.attn_v));
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_q.weight", &w.attn_q, SLAI_LAYOUT_TILE64));
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_k.weight", &w.attn_k, SLAI_LAYOUT_TILE64));
+        TRY(qmat_from_gguf(ctx, gg, p + "attn_v.weight", &w.attn_v, SLAI_LAYOUT_TILE64));
         TRY(f32_vector_from_gguf(ctx, g, p + "attn_q.bias", false, &w.attn_q_bias));
         TRY(f32_vector_from_gguf(ctx, g, p + "attn_k.bias", false, &w.attn_k_bias));
         TRY(f32_vector_from_gguf(ctx, g, p + "attn_v.bias", false, &w.attn_v_bias));
         TRY(qmat_from_gguf(ctx, gg, p + "attn_output.weight", &w.attn_output));
         TRY(qmat_from_gguf(ctx, gg, p + "ffn_down.weight", &w.ffn_down));
-        TRY(qmat_from_gguf(ctx, gg, p + "ffn_gate.weight", &w.ffn_gate));
-        TRY(qmat_from_gguf(ctx, gg, p + "ffn_up.weight", &w.ffn_up));
+        TRY(qmat_from_gguf(ctx, gg, p + "ffn_gate.weight", &w.ffn_gate, SLAI_LAYOUT_TILE64));
+        TRY(qmat_from_gguf(ctx, gg, p + "ffn_up.weight", &w.ffn_up, SLAI_LAYOUT_TILE64));
         TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.weight", true, &w.ffn_norm));
         TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.weight", true, &w.attn_norm));
         struct { slai_qmat *m; uint32_t r, c; } chk[] = {{w.attn_q, dim, dim}, {w.attn_k, kvd, dim}, {w.attn_v, kvd, dim},
@@ -168,8 +177,8 @@ int slai_llama2::load(const slai_gguf *gg) {
         for (slai_qmat *m : {w.attn_q, w.attn_k, w.attn_v, w.attn_output, w.ffn_down, w.ffn_gate, w.ffn_up}) weight_bytes += m->bytes;
         weight_bytes += 2 * (size_t)dim * 4;
     }
-    TRY(qmat_from_gguf(ctx, gg, "token_embd.weight", &weights.token_embd));
-    if (g.find("output.weight")) TRY(qmat_from_gguf(ctx, gg, "output.weight", &weights.output));
+    TRY(qmat_from_gguf(ctx, gg, "token_embd.weight", &weights.token_embd, SLAI_LAYOUT_TILE64));
+    if (g.find("output.weight")) TRY(qmat_from_gguf(ctx, gg, "output.weight", &weights.output, SLAI_LAYOUT_TILE64));
     else weights.output = weights.token_embd;                                       // transformer.rs:279-285
     TRY(f32_vector_from_gguf(ctx, g, "output_norm.weight", true, &weights.output_norm));
     if (weights.token_embd->nrows != config.vocab_size || weights.token_embd->ncols != dim || weights.output->nrows != config.vocab_size ||
@@ -177,6 +186,10 @@ int slai_llama2::load(const slai_gguf *gg) {
         return set_error(ctx, SLAI_E_SHAPE, "embedding / output shape does not match the config");
     weight_bytes += weights.output->bytes + (size_t)dim * 4;
 
+    {   // activation slots of the 64-row-tile GEMV: the largest launch is q/k/v together, gate/up, or the output matrix
+        const uint32_t t64 = std::max(std::max((dim + 63) / 64 + 2 * ((kvd + 63) / 64), (config.hidden_dim + 63) / 64), (config.vocab_size + 63) / 64);
+        TRY(gemv_scratch_reserve(ctx, (size_t)t64 * (dim + dim / 16 + 16)));
+    }
     // ---- Llama2State::new (transformer.rs:47-140); buffers are zero-initialised
     Llama2State &s = state;
     TRY(GpuTensor::vector(ctx, dim, STORAGE | COPY_DST | COPY_SRC, &s.x));
@@ -186,6 +199,7 @@ int slai_llama2::load(const slai_gguf *gg) {
     TRY(GpuTensor::vector(ctx, config.hidden_dim, STORAGE, &s.hb2));
     TRY(GpuTensor::vector(ctx, dim, STORAGE | COPY_SRC, &s.q));
     TRY(GpuTensor::vector(ctx, kvd, STORAGE, &s.kcol));
+    TRY(GpuTensor::vector(ctx, dim + dim / 16 + 16, STORAGE, &s.xw));
     TRY(GpuTensor::vector(ctx, kvd, STORAGE, &s.vcol));
     const int cdt = kv_dtype == SLAI_KV_F16 ? SLAI_DT_F16 : SLAI_DT_F32;
     s.key_cache.resize(config.n_layers); s.value_cache.resize(config.n_layers);
@@ -254,6 +268,10 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
     float *q = (float *)s.q.buf->dptr, *kcol = (float *)s.kcol.buf->dptr, *vcol = (float *)s.vcol.buf->dptr;
     const uint32_t dim = config.dim, kvd = kv_dim();
     SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, &ds->token, nullptr, nullptr, dim, x));
+    // When the GEMV that writes x can leave a norm-weighted copy for the 64-row-tile GEMV that reads it next, that
+    // consumer skips its own staging of the activations.
+    float *xw = (float *)s.xw.buf->dptr;
+    const float *prepared = nullptr;                           // valid copy for the next consumer of x, or none
     for (uint32_t l = 0; l < config.n_layers; ++l) {
         const Llama2LayerWeights &wl = weights.layers[l];
         // ---- RMSNorm + Q/K/V projections: matrices of one format and layout share a launch
@@ -266,8 +284,9 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
                 GemvCall c;
                 c.nseg = 0; c.x = x;
                 c.prologue = PRO_RMSNORM; c.norm_w = (const float *)wl.attn_norm.buf->dptr; c.eps = config.rms_norm_eps;
+                if (gemv_is_rowtile(ctx, mats[i])) c.prepared = prepared;
                 for (int j = i; j < 3; ++j) {
-                    if (done[j] || mats[j]->type != mats[i]->type || mats[j]->tiled != mats[i]->tiled) continue;
+                    if (done[j] || !same_launch(mats[i], mats[j])) continue;
                     c.m[c.nseg] = mats[j]; c.out[c.nseg] = outs[j]; ++c.nseg;
                     done[j] = true;
                 }
@@ -296,13 +315,19 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
         {
             GemvCall c;
             c.m[0] = wl.attn_output; c.out[0] = x; c.flags[0] = GEMV_ACCUM; c.x = xb;
+            prepared = nullptr;
+            if (gemv_can_emit(wl.attn_output) && gemv_is_rowtile(ctx, wl.ffn_gate) && gemv_is_rowtile(ctx, wl.ffn_up)) {
+                c.flags[0] |= GEMV_EMIT; c.emit_w = (const float *)wl.ffn_norm.buf->dptr; c.emit_out = xw;
+                prepared = xw;
+            }
             TRY(gemv_call(ctx, c, "llama2 attn_output"));
         }
         // ---- RMSNorm + gate/up + SiLU
-        if (wl.ffn_gate->type == wl.ffn_up->type && wl.ffn_gate->tiled == wl.ffn_up->tiled) {
+        if (wl.ffn_gate->type == wl.ffn_up->type && wl.ffn_gate->tiled == wl.ffn_up->tiled && wl.ffn_gate->rows_log2 == wl.ffn_up->rows_log2) {
             GemvCall c;
             c.m[0] = wl.ffn_gate; c.m2[0] = wl.ffn_up; c.out[0] = hb; c.flags[0] = GEMV_SILU_GATE; c.x = x;
             c.prologue = PRO_RMSNORM; c.norm_w = (const float *)wl.ffn_norm.buf->dptr; c.eps = config.rms_norm_eps;
+            c.prepared = prepared;
             TRY(gemv_call(ctx, c, "llama2 ffn gate/up"));
         } else {
             const slai_qmat *mats[2] = {wl.ffn_gate, wl.ffn_up};
@@ -311,6 +336,7 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
                 GemvCall c;
                 c.m[0] = mats[i]; c.out[0] = outs[i]; c.x = x;
                 c.prologue = PRO_RMSNORM; c.norm_w = (const float *)wl.ffn_norm.buf->dptr; c.eps = config.rms_norm_eps;
+                c.prepared = prepared;
                 TRY(gemv_call(ctx, c, "llama2 ffn gate/up"));
             }
             SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, config.hidden_dim, 1}, VecView{hb2, config.hidden_dim, 1}));
@@ -319,6 +345,20 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
         {
             GemvCall c;
             c.m[0] = wl.ffn_down; c.out[0] = x; c.flags[0] = GEMV_ACCUM; c.x = hb;
+            // the next reader of x: the next layer's q/k/v (all three must take the prepared copy) or the output matrix
+            const bool last = l + 1 == config.n_layers;
+            bool next_ok = gemv_can_emit(wl.ffn_down);
+            if (last) next_ok = next_ok && gemv_is_rowtile(ctx, weights.output);
+            else {
+                const Llama2LayerWeights &wn = weights.layers[l + 1];
+                next_ok = next_ok && gemv_is_rowtile(ctx, wn.attn_q) && gemv_is_rowtile(ctx, wn.attn_k) && gemv_is_rowtile(ctx, wn.attn_v);
+            }
+            prepared = nullptr;
+            if (next_ok) {
+                const GpuTensor &nw = last ? weights.output_norm : weights.layers[l + 1].attn_norm;
+                c.flags[0] |= GEMV_EMIT; c.emit_w = (const float *)nw.buf->dptr; c.emit_out = xw;
+                prepared = xw;
+            }
             TRY(gemv_call(ctx, c, "llama2 ffn_down"));
         }
     }
@@ -326,6 +366,7 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
         GemvCall c;
         c.m[0] = weights.output; c.out[0] = (float *)s.logits.buf->dptr; c.x = x;
         c.prologue = PRO_RMSNORM; c.norm_w = (const float *)weights.output_norm.buf->dptr; c.eps = config.rms_norm_eps;
+        c.prepared = prepared;
         TRY(gemv_call(ctx, c, "llama2 output"));
     }
     if (with_sampler)
@@ -360,7 +401,7 @@ SLAI_EXPORT void slai_llama2_destroy(slai_llama2 *m) {
     slai_qmat_destroy(ctx, m->weights.token_embd);
     m->weights.output_norm.destroy(ctx);
     Llama2State &s = m->state;
-    for (GpuTensor *t : {&s.x, &s.xb, &s.xb2, &s.hb, &s.hb2, &s.q, &s.att, &s.logits, &s.kcol, &s.vcol}) t->destroy(ctx);
+    for (GpuTensor *t : {&s.x, &s.xb, &s.xb2, &s.hb, &s.hb2, &s.q, &s.att, &s.logits, &s.kcol, &s.vcol, &s.xw}) t->destroy(ctx);
     for (auto &t : s.key_cache) t.destroy(ctx);
     for (auto &t : s.value_cache) t.destroy(ctx);
     for (slai_buffer *b : {s.rope_config, s.rms_norm_config, s.attn_params}) if (b) slai_buffer_destroy(ctx, b);

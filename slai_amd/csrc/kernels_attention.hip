@@ -14,6 +14,7 @@
 // In the model path the kernel also performs RoPE (rope.slang:27-84) on q and on the fresh key
 // and writes the fresh key/value into the cache, so Q/K/V leave the projection GEMV exactly once.
 #include "common.h"
+#include "device_util.h"
 #include "quant_formats.h"
 #include <float.h>
 
@@ -51,6 +52,7 @@ template <> struct KV<false> {
 // grid = (n_heads, n_splits), block = ATT_THREADS.  Dynamic LDS: scores for one split.
 template <bool F16>
 __global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_t max_split_len) {
+    touch_kernel_arguments<sizeof(AttnLaunch) + 8>();
     using C = KV<F16>;
     using CT = typename C::T;
     extern __shared__ float sscore[];             // [max_split_len]

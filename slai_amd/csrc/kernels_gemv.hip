@@ -16,6 +16,7 @@
 // residual accumulate, SiLU-gate of two matrices, and GELU as epilogues.  Up to three
 // matrices of the same format share one launch.
 #include "common.h"
+#include "device_util.h"
 #include "quant_formats.h"
 
 namespace slai {
@@ -48,6 +49,7 @@ __device__ __forceinline__ float gelu_f(float x) {
 
 template <int T, int K, bool DUAL, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemv_kernel(const GemvParams p) {
+    touch_kernel_arguments<sizeof(GemvParams)>();
     using F = Chunk<T>;
     extern __shared__ float smem[];
     const int tid = threadIdx.x, NT = blockDim.x, lane = tid & 63, wave = tid >> 6, NW = NT >> 6;

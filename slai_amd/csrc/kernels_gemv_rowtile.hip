@@ -1,0 +1,317 @@
+// Dequantisation-fused GEMV over 64-row tiles of the tiled weight layout (quant_tiled.h, ROWS = 64, KQ = 1)
+// with wave-uniform activations, gfx950.
+//
+// Same contract as kernels_gemv.hip / kernels_gemv_tiled.hip (the reference's gemv_quant_*.slang shaders
+// dispatched by crates/slai/src/ops/gemv_quant.rs:206-312).  A lane owns one row of a 64-row tile and a
+// wave consumes one 256-column super-block at a time, so all 64 lanes multiply by the SAME activation:
+// it is a scalar register operand of a plain v_fmac_f32 (full rate; a DPP-broadcast operand runs at half
+// rate on this target).  The activations therefore have to be readable through the scalar data cache:
+// the workgroup writes its normalised copy (and the per-16 sums the block formats need for their offset
+// terms) to a private slot of a scratch buffer with ordinary vector stores, waits for them, and every
+// wave then streams its 256 activations with s_load_dwordx8/16.  The slot is written before it is first
+// read in a dispatch and the scalar cache starts every dispatch empty, so no cache maintenance is needed.
+// When the kernel that produced the input already left such a copy (`prepared`: weighted activations followed
+// by their sums of 16, see GEMV_EMIT in kernels_gemv_tiled.hip) the waves read that directly, nothing is staged
+// and the only work left of the RMSNorm is the sum of squares, whose scale is applied in the epilogue.
+//
+// One workgroup = one tile = 64 complete output rows; wave w owns super-blocks w, w+NW, ...; partial
+// sums meet in LDS once.  Segments of one launch may differ in block format (Q4_K q/k with a Q6_K v).
+#include "common.h"
+#include "device_util.h"
+#include "quant_tiled.h"
+
+namespace slai {
+namespace {
+
+typedef const float __attribute__((address_space(4))) cfloat;   // constant address space: scalar loads
+
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+__device__ __forceinline__ float gelu_f(float x) {
+    const float GELU_COEF_A = 0.044715f, SQRT_2_OVER_PI = 0.7978846f;   // ops/unary.rs:81-85
+    return 0.5f * x * (1.0f + tanhf(SQRT_2_OVER_PI * x * (1.0f + GELU_COEF_A * x * x)));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
+typedef float fx16 __attribute__((ext_vector_type(16)));
+typedef const fx16 __attribute__((address_space(4))) cfx16;
+
+// Activations of one super-block, wave-uniform, fetched through the scalar cache one stage ahead of their use.
+struct ScalarX {
+    cfloat *x;   // 256 activations
+    cfloat *s;   // 16 sums of 16 consecutive activations
+    struct St { fx16 a, b; };
+    template <int I1, int I2> __device__ __forceinline__ St stage() const {
+        return St{*(cfx16 *)(x + 16 * I1), *(cfx16 *)(x + 16 * I2)};
+    }
+    // acc += sum_b byte_b(w) * x[16*I_SLOT + 4*W + b].  The conversions are spelled out because the compiler
+    // otherwise extracts bytes 1..3 with a bit-field instruction first.
+    template <int SLOT, int W> __device__ __forceinline__ float fma4(const St &st, uint32_t w, float acc) const {
+        float t0, t1, t2, t3;
+        asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(t0) : "v"(w));
+        asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(t1) : "v"(w));
+        asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(t2) : "v"(w));
+        asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(t3) : "v"(w));
+        const fx16 &c = SLOT ? st.b : st.a;
+        acc = fmaf(t0, c[4 * W], acc);
+        acc = fmaf(t1, c[4 * W + 1], acc);
+        acc = fmaf(t2, c[4 * W + 2], acc);
+        acc = fmaf(t3, c[4 * W + 3], acc);
+        return acc;
+    }
+    __device__ __forceinline__ float sum16(int i) const { return s[i]; }
+};
+
+template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, int lane, typename Tiled<T>::Data &d, uint16_t &tail) {
+    using F = Tiled<T>;
+#pragma unroll
+    for (int p = 0; p < F::PT; ++p) d.p[p] = ld128(unit + (size_t)p * 1024 + lane * 16);
+    if constexpr (F::TAIL) tail = ld16(unit + (size_t)F::PT * 1024 + lane * 2);
+    else tail = 0;
+}
+
+// The body for one block format.  `partial` = [DUAL?2:1][NW][64] floats, `red` = [NW] floats.
+template <int T, bool DUAL, bool PREP>
+__device__ __forceinline__ void tile_body(const GemvRowtileParams &p, const GemvRowtileSeg &seg, uint32_t tile, float *partial, float *red) {
+    using F = Tiled<T>;
+    const int tid = threadIdx.x, lane = tid & 63, NT = blockDim.x, NW = NT >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
+    // both matrices of a gated pair are requested together when their registers fit beside each other
+    constexpr bool BOTH = DUAL && F::PT <= 9;
+
+    // ---- requests.  Loads retire in issue order.  With prepared activations nothing before the epilogue needs x, so
+    // the weights go first; otherwise x is needed at once (the workgroup stages its copy) and goes first. ----------
+    constexpr int XMAX = 4;                                   // float4 per thread: ncols <= 16 * blockDim
+    float4 xv[XMAX], wv[XMAX];
+    const bool norm = p.prologue == PRO_RMSNORM;
+    auto request_x = [&]() {
+#pragma unroll
+        for (int j = 0; j < XMAX; ++j) {
+            // every thread loads (clamped to the last float4) so that the requests are branch-free; `live` says whether
+            // the value counts
+            const uint32_t i = min((uint32_t)(j * NT + tid) * 4, p.ncols - 4);
+            xv[j] = *(const float4 *)(p.x + i);
+            if (!PREP) wv[j] = norm ? *(const float4 *)(p.norm_w + i) : make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+        }
+    };
+    typename F::Data d, e;
+    uint16_t dt = 0, et = 0;
+    uint32_t cb = wave;
+    auto request_w = [&]() {
+        if (cb < p.ncb) {
+            const size_t off = ((size_t)tile * p.ncb + cb) * unit_bytes;
+            load_unit<T>(seg.W + off, lane, d, dt);
+            if constexpr (BOTH) load_unit<T>(seg.W2 + off, lane, e, et);
+        }
+    };
+    if constexpr (PREP) { request_w(); if (norm) request_x(); }
+    else { request_x(); request_w(); }
+    float old = 0.0f, bias = 0.0f;
+    const uint32_t row = tile * 64 + tid;
+    if (tid < 64 && row < seg.nrows) {
+        if (seg.flags & GEMV_ACCUM) old = seg.out[row];
+        if (seg.flags & GEMV_BIAS) bias = seg.bias[row];
+    }
+
+    float ss = 0.0f, scale = 1.0f;
+    cfloat *xs;
+    if constexpr (PREP) {
+        xs = (cfloat *)(uintptr_t)p.prepared;
+        // The copy was written by another kernel, possibly on another die: the first touch of each of its cache lines
+        // goes to memory.  Touch the 17 lines of this wave's first super-block at once (one word each) so that those
+        // misses overlap each other and the weight stream, instead of stalling the stages one after the other.
+        if (cb < p.ncb) {
+            typedef const uint32_t __attribute__((address_space(4))) cu32;
+            cu32 *wx = (cu32 *)(xs + (size_t)cb * 256), *ws = (cu32 *)(xs + p.ncols + (size_t)cb * 16);
+            uint32_t warm = ws[0];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) warm |= wx[16 * i];
+            asm volatile("" : : "s"(warm));
+        }
+    } else {
+        // ---- the workgroup's own copy of the (weighted) activations and their sums of 16 ----------------------
+        float *slot = p.scratch + (size_t)blockIdx.x * p.scratch_stride;
+#pragma unroll
+        for (int j = 0; j < XMAX; ++j) {
+            const uint32_t i = (uint32_t)(j * NT + tid) * 4;
+            if (i < p.ncols) {
+                float4 v = xv[j];
+                ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
+                v.x *= wv[j].x; v.y *= wv[j].y; v.z *= wv[j].z; v.w *= wv[j].w;
+                *(float4 *)(slot + i) = v;
+                float s4 = (v.x + v.y) + (v.z + v.w);
+                s4 += __shfl_xor(s4, 1, 64);
+                s4 += __shfl_xor(s4, 2, 64);                  // lanes 4q..4q+3 hold 16 consecutive activations
+                if ((lane & 3) == 0) slot[p.ncols + (i >> 4)] = s4;
+            }
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();  // also waits for this thread's stores (and, unavoidably, its weight loads) to complete
+        // The slot is read through the constant address space, whose loads the compiler may move freely; hand it
+        // the pointer only now, behind the barrier.
+        uint64_t slot_bits = (uint64_t)(uintptr_t)slot;
+        asm volatile("" : "+s"(slot_bits) : : "memory");
+        xs = (cfloat *)slot_bits;
+    }
+
+    // ---- super-blocks of this wave -------------------------------------------------------------------
+    float v = 0.0f, v2 = 0.0f;
+    // At most four super-blocks per wave (ncols <= 16384 with 16 waves).  Straight-line code: inside a real loop the
+    // compiler's scheduler requests all scalar loads of a super-block at once and runs out of registers.
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        if (cb < p.ncb) {
+            ScalarX X{xs + (size_t)cb * 256, xs + p.ncols + (size_t)cb * 16};
+            if constexpr (DUAL) {
+                if constexpr (!BOTH) load_unit<T>(seg.W2 + ((size_t)tile * p.ncb + cb) * unit_bytes, lane, e, et);
+                const typename F::Data *dp[2] = {&d, &e};
+                const uint16_t tails[2] = {dt, et};
+                float o2[2];
+                F::template dotn<2>(dp, tails, X, o2);        // both matrices in lockstep: one pass over the activations
+                v += o2[0]; v2 += o2[1];
+            } else {
+                v += F::dot(d, dt, X);
+            }
+            cb += NW;
+            if (it < 3 && cb < p.ncb) {
+                const size_t off = ((size_t)tile * p.ncb + cb) * unit_bytes;
+                load_unit<T>(seg.W + off, lane, d, dt);
+                if constexpr (BOTH) load_unit<T>(seg.W2 + off, lane, e, et);
+            }
+        }
+    }
+    if constexpr (PREP) {
+        if (norm) {                                           // the sum of squares is only needed by the epilogue
+#pragma unroll
+            for (int j = 0; j < XMAX; ++j) {
+                const float4 q = xv[j];
+                const float live = (uint32_t)(j * NT + tid) * 4 < p.ncols ? 1.0f : 0.0f;
+                ss = fmaf(live * q.x, q.x, ss); ss = fmaf(live * q.y, q.y, ss); ss = fmaf(live * q.z, q.z, ss); ss = fmaf(live * q.w, q.w, ss);
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+        }
+    }
+    partial[wave * 64 + lane] = v;
+    if constexpr (DUAL) partial[(NW + wave) * 64 + lane] = v2;
+    lds_barrier();
+    if (tid < 64 && row < seg.nrows) {                        // epilogue: one thread per output row
+        if (p.prologue == PRO_RMSNORM) {
+            float t = 0.0f;
+            for (int w = 0; w < NW; ++w) t += red[w];
+            // rms_norm.slang:60-66 computes (x * scale) * w; here the scale is applied to the finished dot product
+            scale = 1.0f / sqrtf(t / (float)p.ncols + p.eps);
+        }
+        float o = 0.0f;
+        for (int w = 0; w < NW; ++w) o += partial[w * 64 + tid];
+        o *= scale;
+        if constexpr (DUAL) {
+            float up = 0.0f;
+            for (int w = 0; w < NW; ++w) up += partial[(NW + w) * 64 + tid];
+            up *= scale;
+            o = up * (o / (1.0f + expf(-o)));                 // silu.slang:8-26
+        }
+        if (seg.flags & GEMV_BIAS) o += bias;
+        if (seg.flags & GEMV_GELU) o = gelu_f(o);
+        if (seg.flags & GEMV_ACCUM) o = old + o;
+        seg.out[row] = o;
+    }
+}
+
+// TT = block format of every segment, or 0 when the segments differ (the format then is a per-workgroup switch and
+// the kernel needs the registers of its largest case).
+template <int TT, bool DUAL, bool PREP>
+__global__ void __launch_bounds__(1024) gemv_rowtile_kernel(const GemvRowtileParams p) {
+    extern __shared__ float smem[];
+    const int NW = blockDim.x >> 6;
+    float *partial = smem;
+    float *red = smem + (size_t)(DUAL ? 2 : 1) * NW * 64;
+    touch_kernel_arguments<sizeof(GemvRowtileParams)>();
+    // The segment is picked with selects over statically indexed fields: a dynamically indexed p.seg[s] would be
+    // fetched in a second, dependent round trip.
+    const uint32_t n0 = p.seg[0].ntiles, n1 = p.seg[1].ntiles;       // unused segments have ntiles = 0
+    uint32_t tile = blockIdx.x;
+    const int s = tile < n0 ? 0 : (tile - n0 < n1 ? 1 : 2);
+    tile -= s == 0 ? 0u : (s == 1 ? n0 : n0 + n1);
+    GemvRowtileSeg seg;
+    seg.W = s == 0 ? p.seg[0].W : (s == 1 ? p.seg[1].W : p.seg[2].W);
+    seg.W2 = s == 0 ? p.seg[0].W2 : (s == 1 ? p.seg[1].W2 : p.seg[2].W2);
+    seg.type = s == 0 ? p.seg[0].type : (s == 1 ? p.seg[1].type : p.seg[2].type);
+    seg.nrows = s == 0 ? p.seg[0].nrows : (s == 1 ? p.seg[1].nrows : p.seg[2].nrows);
+    seg.out = s == 0 ? p.seg[0].out : (s == 1 ? p.seg[1].out : p.seg[2].out);
+    seg.bias = s == 0 ? p.seg[0].bias : (s == 1 ? p.seg[1].bias : p.seg[2].bias);
+    seg.flags = s == 0 ? p.seg[0].flags : (s == 1 ? p.seg[1].flags : p.seg[2].flags);
+    if constexpr (TT != 0) {
+        tile_body<TT, DUAL, PREP>(p, seg, tile, partial, red);
+    } else {
+        switch (seg.type) {                                    // uniform over the workgroup
+        case T_Q4_K: tile_body<T_Q4_K, DUAL, PREP>(p, seg, tile, partial, red); break;
+        case T_Q6_K: tile_body<T_Q6_K, DUAL, PREP>(p, seg, tile, partial, red); break;
+        default: break;                                        // the launcher sends Q8_0 only to its own kernel
+        }
+    }
+}
+
+template <int TT, bool DUAL>
+hipError_t go(const GemvRowtileParams &p, uint32_t tiles, int NT, size_t smem, hipStream_t s) {
+    if (p.prepared) gemv_rowtile_kernel<TT, DUAL, true><<<tiles, NT, smem, s>>>(p);
+    else gemv_rowtile_kernel<TT, DUAL, false><<<tiles, NT, smem, s>>>(p);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+size_t gemv_rowtile_scratch_floats(const GemvRowtileParams &p) {
+    uint32_t tiles = 0;
+    for (int i = 0; i < p.nseg; ++i) tiles += (p.seg[i].nrows + 63) / 64;
+    return (size_t)tiles * (p.ncols + p.ncols / 16);
+}
+
+hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p) {
+    if (p.ncb == 0 || p.ncols != p.ncb * 256) return hipErrorInvalidValue;
+    int NW = (int)(p.ncb < 16 ? p.ncb : 16);
+    if (p.ncols > 16u * 64u * NW) NW = (int)((p.ncols + 1023) / 1024);       // 4 float4 of x per thread at most
+    if (NW > 16) return hipErrorInvalidValue;
+    bool dual = false;
+    uint32_t tiles = 0;
+    for (int i = 0; i < p.nseg; ++i) {
+        const int t = p.seg[i].type;
+        if (t != T_Q4_K && t != T_Q6_K && t != T_Q8_0) return hipErrorInvalidValue;
+        p.seg[i].ntiles = (p.seg[i].nrows + 63) / 64;
+        tiles += p.seg[i].ntiles;
+        if (p.seg[i].flags & GEMV_SILU_GATE) dual = true;
+        if ((p.seg[i].flags & GEMV_SILU_GATE) && t == T_Q8_0) return hipErrorInvalidValue;
+    }
+    for (int i = 0; i < p.nseg; ++i)
+        if (dual != ((p.seg[i].flags & GEMV_SILU_GATE) != 0)) return hipErrorInvalidValue;
+    p.scratch_stride = p.ncols + p.ncols / 16;
+    const size_t smem = ((size_t)(dual ? 2 : 1) * NW * 64 + NW) * sizeof(float);
+    int tt = p.seg[0].type;
+    for (int i = 1; i < p.nseg; ++i)
+        if (p.seg[i].type != tt) tt = 0;
+    if (tt == 0) {
+        for (int i = 0; i < p.nseg; ++i)
+            if (p.seg[i].type == T_Q8_0) return hipErrorInvalidValue;      // mixed launches: Q4_K with Q6_K only
+    }
+    const int NT = NW * 64;
+    hipStream_t st = ctx->stream;
+    switch (tt) {
+    case T_Q4_K: return dual ? go<T_Q4_K, true>(p, tiles, NT, smem, st) : go<T_Q4_K, false>(p, tiles, NT, smem, st);
+    case T_Q6_K: return dual ? go<T_Q6_K, true>(p, tiles, NT, smem, st) : go<T_Q6_K, false>(p, tiles, NT, smem, st);
+    case T_Q8_0: return go<T_Q8_0, false>(p, tiles, NT, smem, st);
+    default: return dual ? go<0, true>(p, tiles, NT, smem, st) : go<0, false>(p, tiles, NT, smem, st);
+    }
+}
+
+}  // namespace slai

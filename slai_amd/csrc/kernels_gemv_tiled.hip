@@ -10,6 +10,7 @@
 //   * wave w of a workgroup owns column group w; the per-wave partial sums meet in LDS once.
 // HBM-bound by design (packed weights are read exactly once); no MFMA.
 #include "common.h"
+#include "device_util.h"
 #include "quant_tiled.h"
 
 namespace slai {
@@ -55,7 +56,10 @@ struct DevX {
     // Written as assembly: the compiler forms DPP operands only on two-address encodings, which an FMA
     // does not have before register allocation, and it would otherwise hoist all 256 conversions of a
     // super-block ahead of the FMAs and run out of registers.
-    template <int I, int W> __device__ __forceinline__ float fma4(uint32_t w, float acc) const {
+    template <int I1, int I2> struct St {};                   // activations are register resident: a stage is a tag
+    template <int I1, int I2> __device__ __forceinline__ St<I1, I2> stage() const { return {}; }
+    template <int SLOT, int W, int I1, int I2> __device__ __forceinline__ float fma4(St<I1, I2>, uint32_t w, float acc) const {
+        constexpr int I = SLOT ? I2 : I1;
         float t0, t1, t2, t3;
         asm("v_cvt_f32_ubyte0 %1, %5\n\t"
             "v_cvt_f32_ubyte1 %2, %5\n\t"
@@ -94,10 +98,20 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     float *partial = smem;                                   // [DUAL?2:1][NW][64]
     float *red = smem + (size_t)(DUAL ? 2 : 1) * NW * 64;    // [NW]
 
-    int s = 0;
+    touch_kernel_arguments<sizeof(GemvTiledParams)>();
+    // the segment is picked with selects over statically indexed fields (no dependent fetches of the arguments)
+    const uint32_t n0 = p.seg[0].nblocks, n1 = p.seg[1].nblocks;     // unused segments have nblocks = 0
     uint32_t blk = blockIdx.x;
-    while (s < p.nseg - 1 && blk >= p.seg[s].nblocks) { blk -= p.seg[s].nblocks; ++s; }
-    const GemvTiledSeg &seg = p.seg[s];
+    const int s = blk < n0 ? 0 : (blk - n0 < n1 ? 1 : 2);
+    blk -= s == 0 ? 0u : (s == 1 ? n0 : n0 + n1);
+    GemvTiledSeg seg;
+    seg.W = s == 0 ? p.seg[0].W : (s == 1 ? p.seg[1].W : p.seg[2].W);
+    seg.W2 = s == 0 ? p.seg[0].W2 : (s == 1 ? p.seg[1].W2 : p.seg[2].W2);
+    seg.nrows = s == 0 ? p.seg[0].nrows : (s == 1 ? p.seg[1].nrows : p.seg[2].nrows);
+    seg.nblocks = s == 0 ? n0 : (s == 1 ? n1 : p.seg[2].nblocks);
+    seg.out = s == 0 ? p.seg[0].out : (s == 1 ? p.seg[1].out : p.seg[2].out);
+    seg.bias = s == 0 ? p.seg[0].bias : (s == 1 ? p.seg[1].bias : p.seg[2].bias);
+    seg.flags = s == 0 ? p.seg[0].flags : (s == 1 ? p.seg[1].flags : p.seg[2].flags);
     const uint32_t ntiles = (seg.nrows + ROWS - 1) >> p.rows_log2;
     const uint32_t step = seg.nblocks;
 
@@ -123,12 +137,13 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     typename F::Data eA, eB;                                 // second matrix of a gated pair
     uint16_t tA = 0, tB = 0, uA = 0, uB = 0;
     uint32_t tile = blk;
-    float old0 = 0.0f, bias0 = 0.0f;
+    float old0 = 0.0f, bias0 = 0.0f, ew0 = 0.0f;
     {
         const uint32_t row = tile * ROWS + tid;
         if (tid < ROWS && tile < ntiles && row < seg.nrows) {
             if (seg.flags & GEMV_ACCUM) old0 = seg.out[row];
             if (seg.flags & GEMV_BIAS) bias0 = seg.bias[row];
+            if (seg.flags & GEMV_EMIT) ew0 = p.emit_w[row];
         }
     }
     {
@@ -189,16 +204,17 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     // Loads are retired in issue order, so everything the epilogue reads from global memory (the value
     // accumulated into, the bias) is requested BEFORE the next tile's weights; waiting for it then does
     // not wait for the weight stream.
-    auto epi_request = [&](uint32_t t, float &old, float &bias) {
-        old = 0.0f; bias = 0.0f;
+    auto epi_request = [&](uint32_t t, float &old, float &bias, float &ew) {
+        old = 0.0f; bias = 0.0f; ew = 0.0f;
         const uint32_t row = t * ROWS + tid;
         if (tid < ROWS && row < seg.nrows) {
             if (seg.flags & GEMV_ACCUM) old = seg.out[row];
             if (seg.flags & GEMV_BIAS) bias = seg.bias[row];
+            if (seg.flags & GEMV_EMIT) ew = p.emit_w[row];
         }
     };
     auto consume = [&](const typename F::Data &d, uint16_t dt, const typename F::Data &e, uint16_t et, uint32_t t, bool more,
-                       float old, float bias) {
+                       float old, float bias, float ew) {
         float v = F::dot(d, dt, X);
         for (int m = ROWS; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);     // across the KQ super-blocks of the wave
         if (lane < ROWS) partial[wave * 64 + lane] = v;
@@ -222,7 +238,14 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
                 if (seg.flags & GEMV_GELU) o = gelu_f(o);
                 if (seg.flags & GEMV_ACCUM) o = old + o;
                 seg.out[row] = o;
+                ew *= o;
+                if (seg.flags & GEMV_EMIT) p.emit_out[row] = ew;
             }
+        }
+        if ((seg.flags & GEMV_EMIT) && wave == 0) {            // wave-uniform: the sums of 16 consecutive weighted results
+            const float s16 = row16_sum(ew);                   // (ew is 0 in lanes without a row)
+            const uint32_t row = t * ROWS + lane;
+            if (lane < ROWS && (lane & 15) == 0 && row < seg.nrows) p.emit_out[seg.nrows + (row >> 4)] = s16;
         }
         if (more) lds_barrier();                               // partial[] is reused by the next tile
     };
@@ -232,16 +255,16 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
         if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, e, et);
     };
     if (tile < ntiles) {
-        float old = old0, bias = bias0;
+        float old = old0, bias = bias0, ew = ew0;
         for (;;) {
             uint32_t next = tile + step;
-            float oldn = 0.0f, biasn = 0.0f;
-            if (next < ntiles) { epi_request(next, oldn, biasn); request(dB, tB, eB, uB, next); }
-            consume(dA, tA, eA, uA, tile, next < ntiles, old, bias);
+            float oldn = 0.0f, biasn = 0.0f, ewn = 0.0f;
+            if (next < ntiles) { epi_request(next, oldn, biasn, ewn); request(dB, tB, eB, uB, next); }
+            consume(dA, tA, eA, uA, tile, next < ntiles, old, bias, ew);
             if (next >= ntiles) break;
             tile = next; next = tile + step;
-            if (next < ntiles) { epi_request(next, old, bias); request(dA, tA, eA, uA, next); }
-            consume(dB, tB, eB, uB, tile, next < ntiles, oldn, biasn);
+            if (next < ntiles) { epi_request(next, old, bias, ew); request(dA, tA, eA, uA, next); }
+            consume(dB, tB, eB, uB, tile, next < ntiles, oldn, biasn, ewn);
             if (next >= ntiles) break;
             tile = next;
         }
@@ -258,6 +281,9 @@ hipError_t go(hipStream_t s, const GemvTiledParams &p, dim3 grid, int NT, size_t
 
 template <int T> hipError_t launch_t(slai_ctx *ctx, GemvTiledParams &p) {
     if (p.ngroups == 0 || p.ngroups > 16) return hipErrorInvalidValue;
+    for (int i = 0; i < p.nseg; ++i)
+        if ((p.seg[i].flags & GEMV_EMIT) && (i != 0 || !p.emit_w || !p.emit_out || p.seg[i].nrows % 16 || (p.seg[i].flags & GEMV_SILU_GATE)))
+            return hipErrorInvalidValue;
     const int NT = (int)p.ngroups * 64;
     const uint32_t rows = 1u << p.rows_log2;
     bool dual = false;

@@ -77,6 +77,17 @@ __global__ void binop_kernel(VecView a, VecView b) {
     }
 }
 
+// The norm-weighted copy of x that the 64-row-tile GEMV reads through the scalar cache: out[i] = x[i] * w[i] for
+// i < n, followed by the n/16 sums of 16 consecutive products.  n is a multiple of 16.
+__global__ void prepare_kernel(float *out, const float *x, const float *w, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;      // grid covers n exactly (n % 64 == 0 not required)
+    float v = 0.0f;
+    if (i < n) { v = x[i] * w[i]; out[i] = v; }
+    float s = v;
+    s += __shfl_xor(s, 1, 64); s += __shfl_xor(s, 2, 64); s += __shfl_xor(s, 4, 64); s += __shfl_xor(s, 8, 64);
+    if (i < n && (i & 15) == 0) out[n + (i >> 4)] = s;
+}
+
 // silu.slang:11-27: a = b * a / (1 + exp(-a))
 __global__ void silu_kernel(VecView a, VecView b) {
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < a.n; i += gridDim.x * blockDim.x) {
@@ -237,6 +248,10 @@ hipError_t launch_binop(hipStream_t s, int op, VecView a, VecView b) {
     if (op == 0) binop_kernel<0><<<grid, 256, 0, s>>>(a, b);
     else if (op == 1) binop_kernel<1><<<grid, 256, 0, s>>>(a, b);
     else binop_kernel<2><<<grid, 256, 0, s>>>(a, b);
+    return hipGetLastError();
+}
+hipError_t launch_prepare(hipStream_t s, float *out, const float *x, const float *w, uint32_t n) {
+    prepare_kernel<<<(n + 255) / 256, 256, 0, s>>>(out, x, w, n);
     return hipGetLastError();
 }
 hipError_t launch_silu(hipStream_t s, VecView a, VecView b) {

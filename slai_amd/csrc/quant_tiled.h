@@ -43,11 +43,13 @@ SLAI_HD bool tiled_supported(int t) { return t == T_Q4_K || t == T_Q6_K || t == 
 SLAI_HD uint32_t tiled_pieces(int t) { return t == T_Q4_K ? 9u : (t == T_Q6_K ? 13u : 17u); }
 SLAI_HD uint32_t tiled_tail(int t) { return t == T_Q6_K ? 128u : 0u; }
 
-SLAI_HD TiledGeom tiled_geom(int t, uint32_t nrows, uint32_t ncols) {
+// force_rows_log2: 0 = choose by column count, else 4, 5 or 6.
+SLAI_HD TiledGeom tiled_geom(int t, uint32_t nrows, uint32_t ncols, uint32_t force_rows_log2 = 0) {
     TiledGeom g;
     g.type = t; g.nrows = nrows; g.ncols = ncols; g.ncb = ncols / 256;
     uint32_t kq;
-    if (g.ncb % 4 == 0 || g.ncb >= 20) kq = 4;
+    if (force_rows_log2 >= 4 && force_rows_log2 <= 6) kq = 64u >> force_rows_log2;
+    else if (g.ncb % 4 == 0 || g.ncb >= 20) kq = 4;
     else if (g.ncb % 2 == 0 || g.ncb >= 10) kq = 2;
     else kq = 1;
     g.rows_log2 = kq == 4 ? 4 : (kq == 2 ? 5 : 6);
@@ -133,30 +135,23 @@ SLAI_HD float tiled_dequant_elem(const TiledGeom &g, const uint8_t *base, uint32
 }
 
 // ---------------------------------------------------------------------------
-// Per-lane block dot products.  `X` provides the activations of the lane's cblock:
-//   X.fma4<I,W>(w, acc) -> acc + sum_{b<4} byte_b(w) * x[16*I + 4*W + b]
-//        (device: four byte->float conversions and four v_fmac_f32 whose x operand is a
-//         row_newbcast DPP read of register I)
-//   X.sum16(I)   -> sum_k x[16*I + k]  (row sums, loop invariant, precomputed).  Q4_K and Q8_0 only
-//                   ever use sum16(2n) + sum16(2n+1); an accessor may keep that pair sum in the even
-//                   slot and 0 in the odd one.
+// Per-lane block dot products.  Every format walks its 256-column super-block in eight STAGES; a stage
+// multiplies two 16-byte pieces of quantised values with two 16-element chunks (I1, I2) of the activations.
+// `X` provides the activations of the lane's super-block:
+//   X.stage<I1,I2>()          -> whatever X needs to serve chunks I1 and I2 (a tag for register-resident
+//                                activations; the loaded values for activations fetched on demand).  The
+//                                dot products request stage k+1 before they compute stage k.
+//   X.fma4<SLOT,W>(st, w, acc) -> acc + sum_{b<4} byte_b(w) * x[16*I_SLOT + 4*W + b]
+//   X.sum16(i)                -> sum_k x[16*i + k]; all uses come before the first stage.
+// dotn<N> computes the dot products of N matrices' rows with the same activations in lockstep (N = 2: the
+// gate/up pair), so that on-demand activations are fetched once.
 // ---------------------------------------------------------------------------
-template <int I, class X> SLAI_HD float piece_dot(const X &x, const U4 &q, float acc) {
-    // q holds sixteen unsigned byte values; byte k pairs with x[16*I + k]:  acc += q_k * x[16*I + k]
-    acc = x.template fma4<I, 0>(q.x, acc);
-    acc = x.template fma4<I, 1>(q.y, acc);
-    acc = x.template fma4<I, 2>(q.z, acc);
-    acc = x.template fma4<I, 3>(q.w, acc);
-    return acc;
-}
-
-// Two independent accumulation chains interleaved word by word (keeps the FMA pipeline fed when a
-// SIMD holds a single wave).
-template <int I1, int I2, class X> SLAI_HD void piece_dot2(const X &x, const U4 &q1, const U4 &q2, float &a1, float &a2) {
-    a1 = x.template fma4<I1, 0>(q1.x, a1); a2 = x.template fma4<I2, 0>(q2.x, a2);
-    a1 = x.template fma4<I1, 1>(q1.y, a1); a2 = x.template fma4<I2, 1>(q2.y, a2);
-    a1 = x.template fma4<I1, 2>(q1.z, a1); a2 = x.template fma4<I2, 2>(q2.z, a2);
-    a1 = x.template fma4<I1, 3>(q1.w, a1); a2 = x.template fma4<I2, 3>(q2.w, a2);
+template <class X, class S> SLAI_HD void stage_dot(const X &x, const S &st, const U4 &q1, const U4 &q2, float &a1, float &a2) {
+    // q1 pairs with chunk I1, q2 with chunk I2; two independent accumulation chains interleaved word by word
+    a1 = x.template fma4<0, 0>(st, q1.x, a1); a2 = x.template fma4<1, 0>(st, q2.x, a2);
+    a1 = x.template fma4<0, 1>(st, q1.y, a1); a2 = x.template fma4<1, 1>(st, q2.y, a2);
+    a1 = x.template fma4<0, 2>(st, q1.z, a1); a2 = x.template fma4<1, 2>(st, q2.z, a2);
+    a1 = x.template fma4<0, 3>(st, q1.w, a1); a2 = x.template fma4<1, 3>(st, q2.w, a2);
 }
 
 template <int T> struct Tiled;
@@ -165,31 +160,60 @@ template <> struct Tiled<T_Q4_K> {
     static constexpr int PT = 9;
     static constexpr bool TAIL = false;
     struct Data { U4 p[9]; };
-    template <int J, class X> SLAI_HD static void pair(const Data &d, const X &x, uint32_t scw, uint32_t mw, float &accd, float &accm) {
-        // sub-blocks 2J (low nibbles) and 2J+1 (high nibbles) of qs pieces 2J, 2J+1
-        const U4 &a = d.p[1 + 2 * J], &b = d.p[2 + 2 * J];
-        float slo = 0.0f, shi = 0.0f;
-        piece_dot2<4 * J, 4 * J + 2>(x, and4(a, 0x0F0F0F0Fu), and4(shr4(a, 4), 0x0F0F0F0Fu), slo, shi);
-        piece_dot2<4 * J + 1, 4 * J + 3>(x, and4(b, 0x0F0F0F0Fu), and4(shr4(b, 4), 0x0F0F0F0Fu), slo, shi);
-        constexpr int sh = (J & 1) * 16;
-        accd = fmaf((float)((scw >> sh) & 0xffu), slo, accd);
-        accd = fmaf((float)((scw >> (sh + 8)) & 0xffu), shi, accd);
-        accm = fmaf((float)((mw >> sh) & 0xffu), x.sum16(4 * J) + x.sum16(4 * J + 1), accm);
-        accm = fmaf((float)((mw >> (sh + 8)) & 0xffu), x.sum16(4 * J + 2) + x.sum16(4 * J + 3), accm);
+    // stage K: qs piece 1+K; low nibbles <-> chunk 4J+H (sub-block 2J), high nibbles <-> chunk 4J+2+H (sub-block 2J+1)
+    static constexpr int c1(int K) { return 4 * (K / 2) + (K % 2); }
+    static constexpr int c2(int K) { return 4 * (K / 2) + 2 + (K % 2); }
+    template <int N> struct Acc { float accd[N], slo[N], shi[N]; uint32_t sc_lo[N], sc_hi[N]; };
+    template <int K, int N, class X, class S> SLAI_HD static void compute(const Data *const *d, const X &x, const S &st, Acc<N> &a) {
+        constexpr int J = K / 2, H = K % 2;
+        for (int n = 0; n < N; ++n) {
+            const U4 &q = d[n]->p[1 + K];
+            stage_dot(x, st, and4(q, 0x0F0F0F0Fu), and4(shr4(q, 4), 0x0F0F0F0Fu), a.slo[n], a.shi[n]);
+            if (H == 1) {
+                const uint32_t scw = J < 2 ? a.sc_lo[n] : a.sc_hi[n];
+                constexpr int sh = (J & 1) * 16;
+                a.accd[n] = fmaf((float)((scw >> sh) & 0xffu), a.slo[n], a.accd[n]);
+                a.accd[n] = fmaf((float)((scw >> (sh + 8)) & 0xffu), a.shi[n], a.accd[n]);
+                a.slo[n] = 0.0f; a.shi[n] = 0.0f;
+            }
+        }
     }
-    template <class X> SLAI_HD static float dot(const Data &d, uint16_t /*tail*/, const X &x) {
-        const U4 &h = d.p[0];
-        const float dd = decode_f16((uint16_t)(h.x & 0xffffu)), dmin = decode_f16((uint16_t)(h.x >> 16));
-        // all eight 6-bit scales / mins at once (quantization.rs:381-389 applied bytewise)
-        const uint32_t sc_lo = h.y & 0x3f3f3f3fu, m_lo = h.z & 0x3f3f3f3fu;
-        const uint32_t sc_hi = (h.w & 0x0f0f0f0fu) | (((h.y >> 6) & 0x03030303u) << 4);
-        const uint32_t m_hi = ((h.w >> 4) & 0x0f0f0f0fu) | (((h.z >> 6) & 0x03030303u) << 4);
-        float accd = 0.0f, accm = 0.0f;
-        pair<0>(d, x, sc_lo, m_lo, accd, accm);
-        pair<1>(d, x, sc_lo, m_lo, accd, accm);
-        pair<2>(d, x, sc_hi, m_hi, accd, accm);
-        pair<3>(d, x, sc_hi, m_hi, accd, accm);
-        return dd * accd - dmin * accm;
+    template <int K, int N, class X, class S> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, Acc<N> &a) {
+        if constexpr (K < 7) {
+            const auto nxt = x.template stage<c1(K + 1), c2(K + 1)>();
+            compute<K, N>(d, x, st, a);
+            stages<K + 1, N>(d, x, nxt, a);
+        } else {
+            compute<K, N>(d, x, st, a);
+        }
+    }
+    template <int N, class X> SLAI_HD static void dotn(const Data *const *d, const uint16_t * /*tail*/, const X &x, float *out) {
+        Acc<N> a;
+        float dd[N], dmin[N], accm[N];
+        for (int n = 0; n < N; ++n) {
+            const U4 &h = d[n]->p[0];
+            dd[n] = decode_f16((uint16_t)(h.x & 0xffffu)); dmin[n] = decode_f16((uint16_t)(h.x >> 16));
+            // all eight 6-bit scales / mins at once (quantization.rs:381-389 applied bytewise)
+            a.sc_lo[n] = h.y & 0x3f3f3f3fu;
+            a.sc_hi[n] = (h.w & 0x0f0f0f0fu) | (((h.y >> 6) & 0x03030303u) << 4);
+            const uint32_t m_lo = h.z & 0x3f3f3f3fu;
+            const uint32_t m_hi = ((h.w >> 4) & 0x0f0f0f0fu) | (((h.z >> 6) & 0x03030303u) << 4);
+            float am = 0.0f;
+            for (int sb = 0; sb < 8; ++sb) {       // offset term: min of sub-block sb times the sum of its 32 activations
+                const uint32_t mw = sb < 4 ? m_lo : m_hi;
+                am = fmaf((float)((mw >> (8 * (sb & 3))) & 0xffu), x.sum16(2 * sb) + x.sum16(2 * sb + 1), am);
+            }
+            accm[n] = am; a.accd[n] = 0.0f; a.slo[n] = 0.0f; a.shi[n] = 0.0f;
+        }
+        const auto st0 = x.template stage<c1(0), c2(0)>();
+        stages<0, N>(d, x, st0, a);
+        for (int n = 0; n < N; ++n) out[n] = dd[n] * a.accd[n] - dmin[n] * accm[n];
+    }
+    template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
+        const Data *dp[1] = {&d};
+        float out[1];
+        dotn<1>(dp, &tail, x, out);
+        return out[0];
     }
 };
 
@@ -197,34 +221,62 @@ template <> struct Tiled<T_Q6_K> {
     static constexpr int PT = 13;
     static constexpr bool TAIL = true;
     struct Data { U4 p[13]; };
-    template <int I, int M, class X> SLAI_HD static float half_m(const Data &d, const X &x, float acc) {
-        // l = 16M..16M+15 of the 128-half I: four quadrants, scales[8I + 2r + M]
-        const U4 &ql0 = d.p[4 * I + M], &ql32 = d.p[4 * I + 2 + M], &qh = d.p[8 + 2 * I + M];
+    // stage K: 128-half I = K/4, l-range M = (K/2)%2 (l = 16M..16M+15), quadrant pair P = K%2:
+    //   P = 0: quadrants 0,1 <-> chunks 8I+M, 8I+2+M;  P = 1: quadrants 2,3 <-> chunks 8I+4+M, 8I+6+M
+    static constexpr int c1(int K) { return 8 * (K / 4) + 4 * (K % 2) + ((K / 2) % 2); }
+    static constexpr int c2(int K) { return c1(K) + 2; }
+    // scale of quadrant r (0..3) of (I, M): scales[8I + 2r + M]
+    SLAI_HD static float scale_of(const Data &d, int I, int M, int r) {
         const U4 &scp = d.p[12];
-        const uint32_t scw = I == 0 ? scp.x : scp.z;    // scale bytes 8I .. 8I+3
-        const uint32_t scw2 = I == 0 ? scp.y : scp.w;   // scale bytes 8I+4 .. 8I+7
-        const U4 q1 = or4(and4(ql0, 0x0F0F0F0Fu), shl4(and4(qh, 0x03030303u), 4));
-        const U4 q2 = or4(and4(ql32, 0x0F0F0F0Fu), shl4(and4(shr4(qh, 2), 0x03030303u), 4));
-        const U4 q3 = or4(and4(shr4(ql0, 4), 0x0F0F0F0Fu), shl4(and4(shr4(qh, 4), 0x03030303u), 4));
-        const U4 q4 = or4(and4(shr4(ql32, 4), 0x0F0F0F0Fu), shl4(and4(shr4(qh, 6), 0x03030303u), 4));
-        const float s0 = (float)(int8_t)((scw >> (8 * M)) & 0xff), s1 = (float)(int8_t)((scw >> (8 * (M + 2))) & 0xff);
-        const float s2 = (float)(int8_t)((scw2 >> (8 * M)) & 0xff), s3 = (float)(int8_t)((scw2 >> (8 * (M + 2))) & 0xff);
-        float t1 = 0.0f, t2 = 0.0f, t3 = 0.0f, t4 = 0.0f;
-        piece_dot2<8 * I + M, 8 * I + 2 + M>(x, q1, q2, t1, t2);
-        piece_dot2<8 * I + 4 + M, 8 * I + 6 + M>(x, q3, q4, t3, t4);
-        acc = fmaf(s0, t1 - 32.0f * x.sum16(8 * I + M), acc);
-        acc = fmaf(s1, t2 - 32.0f * x.sum16(8 * I + 2 + M), acc);
-        acc = fmaf(s2, t3 - 32.0f * x.sum16(8 * I + 4 + M), acc);
-        acc = fmaf(s3, t4 - 32.0f * x.sum16(8 * I + 6 + M), acc);
-        return acc;
+        const uint32_t w = r < 2 ? (I == 0 ? scp.x : scp.z) : (I == 0 ? scp.y : scp.w);
+        return (float)(int8_t)((w >> (8 * (M + 2 * (r & 1)))) & 0xff);
+    }
+    template <int K, int N, class X, class S> SLAI_HD static void compute(const Data *const *d, const X &x, const S &st, float *acc) {
+        constexpr int I = K / 4, M = (K / 2) % 2, P = K % 2;
+        for (int n = 0; n < N; ++n) {
+            const U4 &ql0 = d[n]->p[4 * I + M], &ql32 = d[n]->p[4 * I + 2 + M], &qh = d[n]->p[8 + 2 * I + M];
+            U4 qa, qb;
+            if (P == 0) {
+                qa = or4(and4(ql0, 0x0F0F0F0Fu), shl4(and4(qh, 0x03030303u), 4));
+                qb = or4(and4(ql32, 0x0F0F0F0Fu), shl4(and4(shr4(qh, 2), 0x03030303u), 4));
+            } else {
+                qa = or4(and4(shr4(ql0, 4), 0x0F0F0F0Fu), shl4(and4(shr4(qh, 4), 0x03030303u), 4));
+                qb = or4(and4(shr4(ql32, 4), 0x0F0F0F0Fu), shl4(and4(shr4(qh, 6), 0x03030303u), 4));
+            }
+            float ta = 0.0f, tb = 0.0f;
+            stage_dot(x, st, qa, qb, ta, tb);
+            acc[n] = fmaf(scale_of(*d[n], I, M, 2 * P), ta, acc[n]);
+            acc[n] = fmaf(scale_of(*d[n], I, M, 2 * P + 1), tb, acc[n]);
+        }
+    }
+    template <int K, int N, class X, class S> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc) {
+        if constexpr (K < 7) {
+            const auto nxt = x.template stage<c1(K + 1), c2(K + 1)>();
+            compute<K, N>(d, x, st, acc);
+            stages<K + 1, N>(d, x, nxt, acc);
+        } else {
+            compute<K, N>(d, x, st, acc);
+        }
+    }
+    template <int N, class X> SLAI_HD static void dotn(const Data *const *d, const uint16_t *tail, const X &x, float *out) {
+        float acc[N];
+        for (int n = 0; n < N; ++n) {
+            // the -32 of every 6-bit value, through the activation sums: -32 * sum_j scale_j * sum16(chunk_j)
+            float c = 0.0f;
+            for (int I = 0; I < 2; ++I)
+                for (int M = 0; M < 2; ++M)
+                    for (int r = 0; r < 4; ++r) c = fmaf(scale_of(*d[n], I, M, r), x.sum16(8 * I + 2 * r + M), c);
+            acc[n] = -32.0f * c;
+        }
+        const auto st0 = x.template stage<c1(0), c2(0)>();
+        stages<0, N>(d, x, st0, acc);
+        for (int n = 0; n < N; ++n) out[n] = decode_f16(tail[n]) * acc[n];
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
-        float acc = 0.0f;
-        acc = half_m<0, 0>(d, x, acc);
-        acc = half_m<0, 1>(d, x, acc);
-        acc = half_m<1, 0>(d, x, acc);
-        acc = half_m<1, 1>(d, x, acc);
-        return decode_f16(tail) * acc;
+        const Data *dp[1] = {&d};
+        float out[1];
+        dotn<1>(dp, &tail, x, out);
+        return out[0];
     }
 };
 
@@ -232,22 +284,47 @@ template <> struct Tiled<T_Q8_0> {
     static constexpr int PT = 17;
     static constexpr bool TAIL = false;
     struct Data { U4 p[17]; };
-    template <int B, class X> SLAI_HD static float blk(const Data &d, const X &x, uint32_t dword, float acc) {
-        // block B of the cblock: qs pieces 2B, 2B+1; int8 -> unsigned via ^0x80, the 128 comes back through the sums
-        float s = 0.0f, s2 = 0.0f;
-        piece_dot2<2 * B, 2 * B + 1>(x, xor4(d.p[2 * B], 0x80808080u), xor4(d.p[2 * B + 1], 0x80808080u), s, s2);
-        s = (s + s2) - 128.0f * (x.sum16(2 * B) + x.sum16(2 * B + 1));
-        const float dd = decode_f16((uint16_t)((B & 1) ? (dword >> 16) : (dword & 0xffffu)));
-        return fmaf(dd, s, acc);
-    }
-    template <class X> SLAI_HD static float dot(const Data &d, uint16_t /*tail*/, const X &x) {
+    // stage K = block K of the super-block: qs pieces 2K, 2K+1 <-> chunks 2K, 2K+1
+    static constexpr int c1(int K) { return 2 * K; }
+    static constexpr int c2(int K) { return 2 * K + 1; }
+    SLAI_HD static float scale_of(const Data &d, int B) {
         const U4 &s = d.p[16];
-        float acc = 0.0f;
-        acc = blk<0>(d, x, s.x, acc); acc = blk<1>(d, x, s.x, acc);
-        acc = blk<2>(d, x, s.y, acc); acc = blk<3>(d, x, s.y, acc);
-        acc = blk<4>(d, x, s.z, acc); acc = blk<5>(d, x, s.z, acc);
-        acc = blk<6>(d, x, s.w, acc); acc = blk<7>(d, x, s.w, acc);
-        return acc;
+        const uint32_t w = B < 2 ? s.x : (B < 4 ? s.y : (B < 6 ? s.z : s.w));
+        return decode_f16((uint16_t)((B & 1) ? (w >> 16) : (w & 0xffffu)));
+    }
+    template <int K, int N, class X, class S> SLAI_HD static void compute(const Data *const *d, const X &x, const S &st, float *acc) {
+        for (int n = 0; n < N; ++n) {
+            // int8 -> unsigned via ^0x80; the 128 comes back through the activation sums
+            float s = 0.0f, s2 = 0.0f;
+            stage_dot(x, st, xor4(d[n]->p[2 * K], 0x80808080u), xor4(d[n]->p[2 * K + 1], 0x80808080u), s, s2);
+            acc[n] = fmaf(scale_of(*d[n], K), s + s2, acc[n]);
+        }
+    }
+    template <int K, int N, class X, class S> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc) {
+        if constexpr (K < 7) {
+            const auto nxt = x.template stage<c1(K + 1), c2(K + 1)>();
+            compute<K, N>(d, x, st, acc);
+            stages<K + 1, N>(d, x, nxt, acc);
+        } else {
+            compute<K, N>(d, x, st, acc);
+        }
+    }
+    template <int N, class X> SLAI_HD static void dotn(const Data *const *d, const uint16_t * /*tail*/, const X &x, float *out) {
+        float acc[N];
+        for (int n = 0; n < N; ++n) {
+            float c = 0.0f;
+            for (int B = 0; B < 8; ++B) c = fmaf(scale_of(*d[n], B), x.sum16(2 * B) + x.sum16(2 * B + 1), c);
+            acc[n] = -128.0f * c;
+        }
+        const auto st0 = x.template stage<c1(0), c2(0)>();
+        stages<0, N>(d, x, st0, acc);
+        for (int n = 0; n < N; ++n) out[n] = acc[n];
+    }
+    template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
+        const Data *dp[1] = {&d};
+        float out[1];
+        dotn<1>(dp, &tail, x, out);
+        return out[0];
     }
 };
 

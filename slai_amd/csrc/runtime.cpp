@@ -81,6 +81,7 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->use_graph = env_int("SLAI_NO_GRAPH", 0) == 0;
     ctx->gemv_max_wgs = env_int("SLAI_GEMV_MAX_WGS", 512);
     ctx->tiled_layout = env_int("SLAI_TILED", 1) != 0;
+    ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
     *out = ctx;
     return SLAI_OK;
 }
@@ -90,6 +91,7 @@ SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     hipSetDevice(ctx->device);
     hipStreamSynchronize(ctx->stream);
     if (ctx->attn_scratch) hipFree(ctx->attn_scratch);
+    if (ctx->gemv_scratch) hipFree(ctx->gemv_scratch);
     if (ctx->timer0) hipEventDestroy(ctx->timer0);
     if (ctx->timer1) hipEventDestroy(ctx->timer1);
     hipStreamDestroy(ctx->stream);
@@ -178,8 +180,14 @@ SLAI_EXPORT int slai_copy_buffer(slai_ctx *ctx, slai_buffer *dst, size_t dst_off
 // ---- quantized matrices ---------------------------------------------------------
 SLAI_EXPORT int slai_qmat_create(slai_ctx *ctx, uint32_t ggml_type, uint32_t nrows, uint32_t ncols, const void *packed,
                                  slai_qmat **out) {
+    return slai_qmat_create_layout(ctx, ggml_type, nrows, ncols, packed, SLAI_LAYOUT_AUTO, out);
+}
+
+SLAI_EXPORT int slai_qmat_create_layout(slai_ctx *ctx, uint32_t ggml_type, uint32_t nrows, uint32_t ncols, const void *packed,
+                                        int layout, slai_qmat **out) {
     if (!ctx || !out || !packed) return SLAI_E_ARG;
     *out = nullptr;
+    if (layout < SLAI_LAYOUT_AUTO || layout > SLAI_LAYOUT_TILE64) return set_error(ctx, SLAI_E_ARG, "slai_qmat_create: unknown layout");
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_qmat_create during graph capture");
     const int t = (int)ggml_type;
     const int be = block_elems(t);
@@ -189,9 +197,14 @@ SLAI_EXPORT int slai_qmat_create(slai_ctx *ctx, uint32_t ggml_type, uint32_t nro
     m->type = t; m->nrows = nrows; m->ncols = ncols; m->nb = ncols / be;
     m->row_stride = device_row_stride(t, ncols);
     m->bytes = m->row_stride * nrows;
-    if (ctx->tiled_layout && tiled_supported(t) && ncols % 256 == 0) {
-        const TiledGeom g = tiled_geom(t, nrows, ncols);
-        if (g.ngroups <= 16) {
+    if (ctx->tiled_layout && layout != SLAI_LAYOUT_ROWS && tiled_supported(t) && ncols % 256 == 0) {
+        // 64-row tiles (wave-uniform GEMV) pay off when there are enough tiles to occupy the device, or when the
+        // caller launches several such matrices together and says so
+        const uint32_t ncb = ncols / 256;
+        bool tile64 = layout == SLAI_LAYOUT_TILE64 || (layout == SLAI_LAYOUT_AUTO && nrows >= 8192 && nrows % 64 == 0 && ncb <= 16);
+        if (!ctx->rowtile_gemv || ncb > 64) tile64 = false;
+        const TiledGeom g = tiled_geom(t, nrows, ncols, tile64 ? 6u : 0u);
+        if (g.ngroups <= 16 || tile64) {
             m->tiled = true; m->rows_log2 = g.rows_log2; m->ncb = g.ncb; m->ngroups = g.ngroups; m->ntiles = g.ntiles;
             m->unit_bytes = g.unit_bytes; m->bytes = tiled_bytes(g);
         }
@@ -251,14 +264,65 @@ SLAI_EXPORT int slai_qmat_dequantize(slai_ctx *ctx, const slai_qmat *m, uint32_t
 
 // ---- GEMV dispatch over the two weight layouts ------------------------------------------------
 namespace slai {
+bool gemv_can_emit(const slai_qmat *m) { return m && m->tiled && m->rows_log2 != 6 && m->ngroups <= 16 && m->nrows % 16 == 0; }
+bool gemv_is_rowtile(const slai_ctx *ctx, const slai_qmat *m) {
+    return ctx->rowtile_gemv && m && m->tiled && m->rows_log2 == 6 && m->ncb <= 64;
+}
+
+int gemv_scratch_reserve(slai_ctx *ctx, size_t floats) {
+    if (floats <= ctx->gemv_scratch_floats) return SLAI_OK;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "GEMV scratch must be reserved before graph capture");
+    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->gemv_scratch) hipFree(ctx->gemv_scratch);
+    ctx->gemv_scratch = nullptr; ctx->gemv_scratch_floats = 0;
+    SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->gemv_scratch, floats * sizeof(float)));
+    ctx->gemv_scratch_floats = floats;
+    return SLAI_OK;
+}
+
 int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who) {
     const slai_qmat *m0 = c.m[0];
     if (!m0 || c.nseg < 1 || c.nseg > 3) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": bad GEMV call");
+    // 64-row tiles: wave-uniform activations, formats may differ between the segments
+    bool rowtile = ctx->rowtile_gemv && (c.prologue == PRO_NONE || (c.prologue == PRO_RMSNORM && !c.norm_b));
+    for (int i = 0; i < c.nseg && rowtile; ++i) {
+        const slai_qmat *m = c.m[i], *m2 = c.m2[i];
+        rowtile = m && m->tiled && m->rows_log2 == 6 && m->ncols == m0->ncols && m->ncb <= 64 &&
+                  (!m2 || (m2->tiled && m2->rows_log2 == 6 && m2->type == m->type && m2->ncols == m->ncols && m2->nrows == m->nrows)) &&
+                  (((c.flags[i] & GEMV_SILU_GATE) != 0) == (m2 != nullptr)) && !(m2 && m->type == T_Q8_0) &&
+                  (((c.flags[i] ^ c.flags[0]) & GEMV_SILU_GATE) == 0);
+    }
+    for (int i = 1; i < c.nseg && rowtile; ++i)
+        if (c.m[i]->type != m0->type && (c.m[i]->type == T_Q8_0 || m0->type == T_Q8_0)) rowtile = false;
+    if (c.flags[0] & GEMV_EMIT) {
+        if (rowtile || !gemv_can_emit(m0) || !c.emit_w || !c.emit_out) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": this GEMV cannot emit a prepared copy");
+    }
+    if (c.prepared && !rowtile) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": prepared activations need 64-row tiles");
+    if (rowtile) {
+        GemvRowtileParams p;
+        p.nseg = c.nseg; p.ncols = m0->ncols; p.ncb = m0->ncb; p.x = c.x; p.prologue = c.prologue; p.norm_w = c.norm_w; p.eps = c.eps;
+        p.prepared = c.prepared;
+        for (int i = 0; i < c.nseg; ++i) {
+            p.seg[i].W = c.m[i]->dptr; p.seg[i].W2 = c.m2[i] ? c.m2[i]->dptr : nullptr; p.seg[i].type = c.m[i]->type;
+            p.seg[i].nrows = c.m[i]->nrows; p.seg[i].out = c.out[i]; p.seg[i].bias = c.bias[i]; p.seg[i].flags = c.flags[i];
+        }
+        if (!p.prepared) {
+            int rc = gemv_scratch_reserve(ctx, gemv_rowtile_scratch_floats(p));
+            if (rc) return rc;
+            p.scratch = ctx->gemv_scratch;
+        }
+        hipError_t e = launch_gemv_rowtile(ctx, p);
+        if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported shape for the row-tile GEMV");
+        if (e != hipSuccess) return hip_fail(ctx, e, who);
+        return SLAI_OK;
+    }
     for (int i = 0; i < c.nseg; ++i) {
         const slai_qmat *m = c.m[i], *m2 = c.m2[i];
-        if (!m || m->type != m0->type || m->ncols != m0->ncols || m->tiled != m0->tiled)
+        if (!m || m->type != m0->type || m->ncols != m0->ncols || m->tiled != m0->tiled ||
+            (m->tiled && (m->rows_log2 != m0->rows_log2 || m->ngroups > 16)))
             return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": matrices of one launch must share format, width and layout");
-        if (m2 && (m2->type != m->type || m2->ncols != m->ncols || m2->nrows != m->nrows || m2->tiled != m->tiled))
+        if (m2 && (m2->type != m->type || m2->ncols != m->ncols || m2->nrows != m->nrows || m2->tiled != m->tiled ||
+                   (m->tiled && m2->rows_log2 != m->rows_log2)))
             return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": gate and up must share format, shape and layout");
         if ((c.flags[i] & GEMV_SILU_GATE) && !m2) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": gated GEMV without a second matrix");
     }
@@ -267,7 +331,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who) {
         GemvTiledParams p;
         p.nseg = c.nseg; p.ncols = m0->ncols; p.ncb = m0->ncb; p.ngroups = m0->ngroups; p.rows_log2 = m0->rows_log2;
         p.unit_bytes = m0->unit_bytes; p.x = c.x; p.prologue = c.prologue; p.norm_w = c.norm_w; p.norm_b = c.norm_b;
-        p.eps = c.eps;
+        p.eps = c.eps; p.emit_w = c.emit_w; p.emit_out = c.emit_out;
         for (int i = 0; i < c.nseg; ++i) {
             p.seg[i].W = c.m[i]->dptr; p.seg[i].W2 = c.m2[i] ? c.m2[i]->dptr : nullptr; p.seg[i].nrows = c.m[i]->nrows;
             p.seg[i].out = c.out[i]; p.seg[i].bias = c.bias[i]; p.seg[i].flags = c.flags[i];
@@ -323,8 +387,11 @@ SLAI_EXPORT int slai_matmul_quant_assign(slai_ctx *ctx, slai_view out, const sla
     return gemv_call(ctx, c, "slai_matmul_quant_assign");
 }
 
+// `prepared` (optional): the slai_rms_norm_prepare form of (x, norm weight); `emit_w` / `emit_out` (optional): leave
+// that form of (result, emit_w) in emit_out.
 static int fused_gemv(slai_ctx *ctx, const char *fn, slai_view out, const slai_qmat *m, const slai_qmat *m2, slai_view v,
-                      const slai_view *norm_weight, float eps, uint32_t flags) {
+                      const slai_view *norm_weight, float eps, uint32_t flags, const slai_view *prepared = nullptr,
+                      const slai_view *emit_w = nullptr, const slai_view *emit_out = nullptr) {
     if (!ctx || !m) return SLAI_E_ARG;
     VecView vo, vv, vw{nullptr, 0, 1};
     if (!as_vec(out, &vo) || !as_vec(v, &vv)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": bad view");
@@ -337,7 +404,46 @@ static int fused_gemv(slai_ctx *ctx, const char *fn, slai_view out, const slai_q
     GemvCall c;
     c.m[0] = m; c.m2[0] = m2; c.out[0] = vo.p; c.flags[0] = flags; c.x = vv.p;
     if (norm_weight) { c.prologue = PRO_RMSNORM; c.norm_w = vw.p; c.eps = eps; }
+    if (prepared) {
+        VecView vp;
+        if (!as_vec(*prepared, &vp) || vp.stride != 1 || vp.n < m->ncols + m->ncols / 16 || (prepared->offset % 16) != 0)
+            return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": prepared activations must be ncols + ncols/16 contiguous floats, 64-byte aligned");
+        if (!gemv_is_rowtile(ctx, m)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": prepared activations need a matrix in the TILE64 layout");
+        c.prologue = PRO_RMSNORM; c.eps = eps; c.prepared = vp.p;
+    }
+    if (emit_w) {
+        VecView ve, vq;
+        if (!emit_out || !as_vec(*emit_w, &ve) || !as_vec(*emit_out, &vq) || ve.stride != 1 || vq.stride != 1 || ve.n != m->nrows ||
+            vq.n < m->nrows + m->nrows / 16 || (emit_out->offset % 16) != 0)
+            return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": bad next-norm weight or prepared output");
+        if (!gemv_can_emit(m)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": this matrix layout cannot emit prepared activations");
+        c.flags[0] |= GEMV_EMIT; c.emit_w = ve.p; c.emit_out = vq.p;
+    }
     return gemv_call(ctx, c, fn);
+}
+
+SLAI_EXPORT int slai_rms_norm_prepare(slai_ctx *ctx, slai_view out_prepared, slai_view x, slai_view norm_weight) {
+    if (!ctx) return SLAI_E_ARG;
+    VecView vo, vx, vw;
+    if (!as_vec(out_prepared, &vo) || !as_vec(x, &vx) || !as_vec(norm_weight, &vw)) return set_error(ctx, SLAI_E_SHAPE, "slai_rms_norm_prepare: bad view");
+    if (vx.n % 16 || vw.n != vx.n || vo.n < vx.n + vx.n / 16 || vo.stride != 1 || vx.stride != 1 || vw.stride != 1 || (out_prepared.offset % 16) != 0)
+        return set_error(ctx, SLAI_E_SHAPE, "slai_rms_norm_prepare: need n % 16 == 0 and n + n/16 contiguous output floats, 64-byte aligned");
+    SLAI_HIP_TRY(ctx, launch_prepare(ctx->stream, vo.p, vx.p, vw.p, vx.n));
+    return SLAI_OK;
+}
+SLAI_EXPORT int slai_rms_norm_matmul_quant_assign_prepared(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view prepared,
+                                                           float eps) {
+    return fused_gemv(ctx, "slai_rms_norm_matmul_quant_assign_prepared", out, m, nullptr, x, nullptr, eps, 0, &prepared);
+}
+SLAI_EXPORT int slai_ffn_gate_up_silu_prepared(slai_ctx *ctx, slai_view out_hb, const slai_qmat *gate, const slai_qmat *up, slai_view x,
+                                               slai_view prepared, float eps) {
+    if (!up) return SLAI_E_ARG;
+    return fused_gemv(ctx, "slai_ffn_gate_up_silu_prepared", out_hb, gate, up, x, nullptr, eps, GEMV_SILU_GATE, &prepared);
+}
+SLAI_EXPORT int slai_matmul_quant_add_assign_emit(slai_ctx *ctx, slai_view in_out_x, const slai_qmat *m, slai_view v, slai_view next_norm_weight,
+                                                  slai_view out_prepared) {
+    return fused_gemv(ctx, "slai_matmul_quant_add_assign_emit", in_out_x, m, nullptr, v, nullptr, 0.0f, GEMV_ACCUM, nullptr, &next_norm_weight,
+                      &out_prepared);
 }
 
 SLAI_EXPORT int slai_rms_norm_matmul_quant_assign(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view norm_weight,

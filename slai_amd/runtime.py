@@ -131,11 +131,11 @@ def _v(t):
 class GpuQuantMatrix:
     """crates/slai/src/quantized_matrix.rs ``GpuQuantMatrix``: packed GGUF rows resident on the device."""
 
-    def __init__(self, backend, ggml_type, nrows, ncols, packed):
+    def __init__(self, backend, ggml_type, nrows, ncols, packed, layout=_ffi.LAYOUT_AUTO):
         self.b = backend
         packed = np.ascontiguousarray(packed).view(np.uint8).reshape(-1)
         h = C.c_void_p()
-        backend.check(backend.L.slai_qmat_create(backend.h, ggml_type, nrows, ncols, packed.ctypes.data, C.byref(h)))
+        backend.check(backend.L.slai_qmat_create_layout(backend.h, ggml_type, nrows, ncols, packed.ctypes.data, layout, C.byref(h)))
         self.h, self.ggml_type, self.nrows, self.ncols = h, ggml_type, nrows, ncols
 
     def shape(self):
@@ -193,6 +193,18 @@ class LlmContext:
 
     def matmul_quant_add_assign(self, in_out_x, m, v):
         self.backend.check(self.L.slai_matmul_quant_add_assign(self.h, _v(in_out_x), m.h, _v(v)))
+
+    def rms_norm_prepare(self, out_prepared, x, norm_weight):
+        self.backend.check(self.L.slai_rms_norm_prepare(self.h, _v(out_prepared), _v(x), _v(norm_weight)))
+
+    def rms_norm_matmul_quant_assign_prepared(self, out, m, x, prepared, eps):
+        self.backend.check(self.L.slai_rms_norm_matmul_quant_assign_prepared(self.h, _v(out), m.h, _v(x), _v(prepared), eps))
+
+    def ffn_gate_up_silu_prepared(self, out_hb, gate, up, x, prepared, eps):
+        self.backend.check(self.L.slai_ffn_gate_up_silu_prepared(self.h, _v(out_hb), gate.h, up.h, _v(x), _v(prepared), eps))
+
+    def matmul_quant_add_assign_emit(self, in_out_x, m, v, next_norm_weight, out_prepared):
+        self.backend.check(self.L.slai_matmul_quant_add_assign_emit(self.h, _v(in_out_x), m.h, _v(v), _v(next_norm_weight), _v(out_prepared)))
 
     def matmul_assign(self, out, a, b, a_mode, b_mode):
         self.backend.check(self.L.slai_matmul_assign(self.h, _v(out), _v(a), _v(b), a_mode, b_mode))

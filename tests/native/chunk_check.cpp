@@ -93,7 +93,10 @@ float cc_decode_f16(uint16_t h) { return decode_f16(h); }
 // ---- tiled layout ---------------------------------------------------------------------------
 struct HostX {
     const float *xb;   // the 256 activations of one cblock
-    template <int I, int W> float fma4(uint32_t w, float acc) const {
+    template <int I1, int I2> struct St {};
+    template <int I1, int I2> St<I1, I2> stage() const { return {}; }
+    template <int SLOT, int W, int I1, int I2> float fma4(St<I1, I2>, uint32_t w, float acc) const {
+        const int I = SLOT ? I2 : I1;
         for (int b = 0; b < 4; ++b) acc = fmaf((float)((w >> (8 * b)) & 0xffu), xb[16 * I + 4 * W + b], acc);
         return acc;
     }

@@ -157,3 +157,124 @@ def test_fused_op_forms(backend, oracle_lib, t):
     assert rel_err(gx.read(), x + d) < 1e-4
     for o in (gate, up, down, gx, gw, ghb, gh):
         o.destroy()
+
+
+# ---- device layouts: every layout must serve every op with the same results -------------------------------
+LAYOUTS = {"rows": 1, "tile16": 2, "tile64": 3}
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS), ids=list(LAYOUTS))
+@pytest.mark.parametrize("t", [8, 12, 14], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("shape", [(64, 256), (200, 1024), (70, 2816), (1027, 4096)])
+def test_layouts_dequantize_and_gemv(backend, oracle_lib, layout, t, shape):
+    """Bit-exact dequantisation and GEMV parity in each device layout (row tails, odd super-block counts)."""
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
+    nrows, ncols = shape
+    print("case", layout, NAMES[t], shape, flush=True)
+    raw = synth.normal_quantized(500 + t, t, nrows, ncols, 0.02)
+    w = oracle_deq(oracle_lib, t, raw, nrows * ncols).reshape(nrows, ncols)
+    m = GpuQuantMatrix(backend, t, nrows, ncols, raw, layout=LAYOUTS[layout])
+    assert np.array_equal(m.dequantize().view(np.uint32), w.view(np.uint32))
+    x = synth.normal(78, ncols, 1.0)
+    ref = np.empty(nrows, np.float32)
+    oracle_lib.slo_gemv(ref.ctypes.data, w.ctypes.data, x.ctypes.data, nrows, ncols)
+    ctxt = LlmContext(backend)
+    v, out = GpuTensor.vector(backend, x), GpuTensor(backend, nrows)
+    ctxt.matmul_quant_assign(out, m, v)
+    got = out.read()
+    scale = np.abs(w).astype(np.float64) @ np.abs(x).astype(np.float64)
+    assert np.all(np.abs(got - ref) <= 3e-5 * scale + 1e-12), float((np.abs(got - ref) / scale).max())
+    for o in (m, v, out):
+        o.destroy()
+
+
+@pytest.mark.parametrize("t", [8, 12, 14], ids=lambda t: NAMES[t])
+def test_tile64_fused_forms_and_changing_input(backend, oracle_lib, t):
+    """64-row tiles: RMSNorm prologue, gate/up + SiLU and residual accumulate; the input vector changes between
+    launches (the kernel reads its activations through the scalar cache, which must never serve stale data)."""
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
+    dim, hid = 1024, 2880
+    ctxt = LlmContext(backend)
+    raws = [synth.normal_quantized(30 + i, t, hid, dim, 0.05) for i in range(2)]
+    ws = [oracle_deq(oracle_lib, t, r, hid * dim).reshape(hid, dim) for r in raws]
+    gate, up = [GpuQuantMatrix(backend, t, hid, dim, r, layout=3) for r in raws]
+    gw_np = (1.0 + synth.normal(2, dim, 0.1)).astype(np.float32)
+    gx, gw, ghb = GpuTensor(backend, dim), GpuTensor.vector(backend, gw_np), GpuTensor(backend, hid)
+    for rep in range(4):
+        x = synth.normal(100 + rep, dim, 1.0 + rep)
+        gx.write(x)
+        xn = np.empty(dim, np.float32)
+        oracle_lib.slo_rms_norm(xn.ctypes.data, x.ctypes.data, gw_np.ctypes.data, dim, 1e-5)
+        g = np.empty(hid, np.float32); u = np.empty(hid, np.float32)
+        oracle_lib.slo_gemv(g.ctypes.data, ws[0].ctypes.data, xn.ctypes.data, hid, dim)
+        oracle_lib.slo_gemv(u.ctypes.data, ws[1].ctypes.data, xn.ctypes.data, hid, dim)
+        ctxt.rms_norm_matmul_quant_assign(ghb, gate, gx, gw, 1e-5)
+        assert rel_err(ghb.read(), g) < 1e-4, rep
+        h = g.copy(); oracle_lib.slo_silu(h.ctypes.data, u.ctypes.data, hid)
+        ctxt.ffn_gate_up_silu(ghb, gate, up, gx, gw, 1e-5)
+        assert rel_err(ghb.read(), h) < 1e-4, rep
+        ctxt.matmul_quant_assign(ghb, up, gx)
+        plain = np.empty(hid, np.float32)
+        oracle_lib.slo_gemv(plain.ctypes.data, ws[1].ctypes.data, x.ctypes.data, hid, dim)
+        assert rel_err(ghb.read(), plain) < 1e-4, rep
+    # residual accumulate over a wide input (43 super-blocks: waves walk several of them)
+    hid2 = 11008
+    rawd = synth.normal_quantized(41, t, 192, hid2, 0.05)
+    wd = oracle_deq(oracle_lib, t, rawd, 192 * hid2).reshape(192, hid2)
+    hv, x0 = synth.normal(42, hid2, 1.0), synth.normal(43, 192, 1.0)
+    d = np.empty(192, np.float32)
+    oracle_lib.slo_gemv(d.ctypes.data, wd.ctypes.data, hv.ctypes.data, 192, hid2)
+    down = GpuQuantMatrix(backend, t, 192, hid2, rawd, layout=3)
+    gh, gacc = GpuTensor.vector(backend, hv), GpuTensor.vector(backend, x0)
+    ctxt.matmul_quant_add_assign(gacc, down, gh)
+    assert rel_err(gacc.read(), x0 + d) < 1e-4
+    for o in (gate, up, down, gx, gw, ghb, gh, gacc):
+        o.destroy()
+
+
+@pytest.mark.parametrize("t", [8, 12, 14], ids=lambda t: NAMES[t])
+def test_prepared_activations_chain(backend, oracle_lib, t):
+    """x += Wd.h leaving the prepared form of the new x, then RMSNorm + gate/up + SiLU (and a plain RMSNorm GEMV) reading
+    it: equal to the unfused oracle sequence; also slai_rms_norm_prepare itself."""
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
+    dim, hid = 1024, 2816
+    ctxt = LlmContext(backend)
+    rawd = synth.normal_quantized(61, t, dim, hid, 0.05)
+    wd = oracle_deq(oracle_lib, t, rawd, dim * hid).reshape(dim, hid)
+    raws = [synth.normal_quantized(62 + i, t, hid, dim, 0.05) for i in range(2)]
+    ws = [oracle_deq(oracle_lib, t, r, hid * dim).reshape(hid, dim) for r in raws]
+    down = GpuQuantMatrix(backend, t, dim, hid, rawd, layout=2)
+    gate, up = [GpuQuantMatrix(backend, t, hid, dim, r, layout=3) for r in raws]
+    nw = (1.0 + synth.normal(3, dim, 0.1)).astype(np.float32)
+    gnw, gprep, ghb = GpuTensor.vector(backend, nw), GpuTensor(backend, dim + dim // 16), GpuTensor(backend, hid)
+    gx, gh = GpuTensor(backend, dim), GpuTensor(backend, hid)
+    for rep in range(3):
+        x0, hv = synth.normal(200 + rep, dim, 1.0), synth.normal(300 + rep, hid, 1.0 + rep)
+        gx.write(x0); gh.write(hv)
+        d = np.empty(dim, np.float32)
+        oracle_lib.slo_gemv(d.ctypes.data, wd.ctypes.data, hv.ctypes.data, dim, hid)
+        x1 = x0 + d
+        ctxt.matmul_quant_add_assign_emit(gx, down, gh, gnw, gprep)
+        got_x = gx.read()
+        assert rel_err(got_x, x1) < 1e-4
+        prep = gprep.read()
+        assert rel_err(prep[:dim], got_x * nw) < 1e-6
+        assert rel_err(prep[dim:], (got_x * nw).reshape(-1, 16).sum(axis=1)) < 1e-5
+        xn = np.empty(dim, np.float32)
+        oracle_lib.slo_rms_norm(xn.ctypes.data, got_x.ctypes.data, nw.ctypes.data, dim, 1e-5)
+        g = np.empty(hid, np.float32); u = np.empty(hid, np.float32)
+        oracle_lib.slo_gemv(g.ctypes.data, ws[0].ctypes.data, xn.ctypes.data, hid, dim)
+        oracle_lib.slo_gemv(u.ctypes.data, ws[1].ctypes.data, xn.ctypes.data, hid, dim)
+        h = g.copy(); oracle_lib.slo_silu(h.ctypes.data, u.ctypes.data, hid)
+        if t != 8:                                     # a gated Q8_0 pair takes the general path, which has no prepared form
+            ctxt.ffn_gate_up_silu_prepared(ghb, gate, up, gx, gprep, 1e-5)
+            assert rel_err(ghb.read(), h) < 1e-4, rep
+        ctxt.rms_norm_matmul_quant_assign_prepared(ghb, up, gx, gprep, 1e-5)
+        assert rel_err(ghb.read(), u) < 1e-4, rep
+        # the stand-alone builder gives the same form
+        gprep2 = GpuTensor(backend, dim + dim // 16)
+        ctxt.rms_norm_prepare(gprep2, gx, gnw)
+        assert rel_err(gprep2.read(), prep) < 1e-6
+        gprep2.destroy()
+    for o in (down, gate, up, gnw, gprep, ghb, gx, gh):
+        o.destroy()
