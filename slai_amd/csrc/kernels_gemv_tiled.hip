@@ -273,8 +273,10 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
 
 template <int T, bool DUAL>
 hipError_t go(hipStream_t s, const GemvTiledParams &p, dim3 grid, int NT, size_t smem) {
+    // the bound decides the register budget: 256/512 threads leave 256, 768 leave 168, 1024 leave 128 per lane
     if (NT <= 256) gemv_tiled_kernel<T, DUAL, 256><<<grid, NT, smem, s>>>(p);
     else if (NT <= 512) gemv_tiled_kernel<T, DUAL, 512><<<grid, NT, smem, s>>>(p);
+    else if (NT <= 768) gemv_tiled_kernel<T, DUAL, 768><<<grid, NT, smem, s>>>(p);
     else gemv_tiled_kernel<T, DUAL, 1024><<<grid, NT, smem, s>>>(p);
     return hipGetLastError();
 }
