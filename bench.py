@@ -50,8 +50,9 @@ def token_bytes(cfg, weight_bytes, pos_lo, pos_hi, kv_bytes=2):
 
 
 def measure_dominant_kernel(backend, reps=20):
-    """Mean launch duration of the fused gate/up GEMV (Q4_K, 11008x4096 twice) over distinct copies."""
-    from slai_amd import synth
+    """Mean launch duration of the fused gate/up GEMV (Q4_K, 11008x4096 twice) over distinct copies, launched the way
+    the decode loop launches it: 64-row-tile layout, activations in the prepared form left by the preceding GEMV."""
+    from slai_amd import _ffi, synth
     from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
     dim, hid, t = CFG["dim"], CFG["hidden_dim"], 12
     ncopies = 8                                     # 8 x 50.7 MB = 406 MB > 256 MB Infinity Cache
@@ -59,21 +60,23 @@ def measure_dominant_kernel(backend, reps=20):
     rb = base.size // hid
     mats = []
     for i in range(2 * ncopies):
-        mats.append(GpuQuantMatrix(backend, t, hid, dim, np.roll(base.reshape(hid, rb), i + 1, axis=0)))
+        mats.append(GpuQuantMatrix(backend, t, hid, dim, np.roll(base.reshape(hid, rb), i + 1, axis=0), layout=_ffi.LAYOUT_TILE64))
     x = GpuTensor.vector(backend, synth.normal(7, dim, 1.0))
     w = GpuTensor.vector(backend, np.ones(dim, np.float32))
     hb = GpuTensor(backend, hid)
+    prep = GpuTensor(backend, dim + dim // 16)
     ctxt = LlmContext(backend)
+    ctxt.rms_norm_prepare(prep, x, w)
     for i in range(ncopies):
-        ctxt.ffn_gate_up_silu(hb, mats[2 * i], mats[2 * i + 1], x, w, 1e-5)
+        ctxt.ffn_gate_up_silu_prepared(hb, mats[2 * i], mats[2 * i + 1], x, prep, 1e-5)
     backend.synchronize()
     backend.timer_begin()
     for _ in range(reps):
         for i in range(ncopies):
-            ctxt.ffn_gate_up_silu(hb, mats[2 * i], mats[2 * i + 1], x, w, 1e-5)
+            ctxt.ffn_gate_up_silu_prepared(hb, mats[2 * i], mats[2 * i + 1], x, prep, 1e-5)
     ms = backend.timer_end() / (reps * ncopies)
-    algo = 2 * mats[0].device_bytes() + dim * 4 * 2 + hid * 4     # 2 packed matrices + x + norm weight + out
-    for o in mats + [x, w, hb]:
+    algo = 2 * mats[0].device_bytes() + dim * 4 * 2 + hid * 4     # 2 packed matrices + x + its weighted copy + out
+    for o in mats + [x, w, hb, prep]:
         o.destroy()
     return ms, algo
 
@@ -190,7 +193,7 @@ def main():
     if not args.no_roofline:
         kms, kalgo = measure_dominant_kernel(backend)
         ach = kalgo / (kms * 1e-3) / 1e9
-        roof = dict(bound="hbm", kernel="gemv_kernel<Q4_K, dual> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096)",
+        roof = dict(bound="hbm", kernel="gemv_rowtile_kernel<Q4_K, dual> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096)",
                     achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
                     traffic=DOMINANT_KERNEL_TRAFFIC_BYTES, launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
         log("dominant kernel: %.2f us/launch, %.1f GB/s" % (kms * 1000, ach))

@@ -185,6 +185,199 @@ __global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_
     }
 }
 
+// ---- the same computation for head sizes that are multiples of 32, organised around 16-byte loads with many of
+// them in flight: scores with 4 lanes per position (each lane a contiguous quarter of the head), values with one
+// lane per 8 elements and several positions per pass.  NT = 1024 serves one workgroup per head over the whole
+// context (no combine pass; short contexts), NT = 256 the split form.
+template <bool F16> struct Vec8;
+template <> struct Vec8<true> {   // 8 f16 = 16 bytes
+    __device__ static void load(const uint16_t *p, float (&o)[8]) {
+        const uint4 w = *reinterpret_cast<const uint4 *>(p);
+        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { o[2 * i] = decode_f16((uint16_t)(u[i] & 0xffffu)); o[2 * i + 1] = decode_f16((uint16_t)(u[i] >> 16)); }
+    }
+};
+template <> struct Vec8<false> {  // 8 f32 = 32 bytes
+    __device__ static void load(const float *p, float (&o)[8]) {
+        const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + 4);
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    }
+};
+
+template <bool F16, int NT, int HS>
+__global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t max_split_len) {
+    touch_kernel_arguments<sizeof(AttnLaunch) + 8>();
+    using C = KV<F16>;
+    using CT = typename C::T;
+    constexpr int NW = NT / 64;
+    constexpr int EPL = HS / 4;                   // elements per lane in the score phase
+    constexpr int LPP = HS / 8;                   // lanes per position in the value phase
+    constexpr int VG = NT / LPP;                  // positions per pass in the value phase
+    extern __shared__ float sscore[];             // [max_split_len]
+    __shared__ float sq[HS], sk[HS], sv[HS];
+    __shared__ float sred[NW];
+    __shared__ float sacc[NW][LPP * 8];           // per-wave partial outputs (= HS floats per wave)
+
+    const uint32_t h = blockIdx.x, split = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t kvh = h / a.kv_mul;
+    const uint32_t pos = *a.pos_ptr;
+    const uint32_t T = pos + 1;
+    const uint32_t chunk = (T + a.n_splits - 1) / a.n_splits;
+    const uint32_t t0 = split * chunk;
+    const uint32_t t1 = min(T, t0 + chunk);
+    CT *kc = reinterpret_cast<CT *>(a.kcache), *vc = reinterpret_cast<CT *>(a.vcache);
+    const size_t hoff = (size_t)kvh * HS;
+    const bool fresh = a.knew != nullptr;
+    const bool own_new = fresh && t0 <= pos && pos < t1;
+
+    // ---- q (and the fresh k/v) into LDS, with bias and RoPE when fused: identical to attn_kernel ------------------
+    if (tid < HS / 2) {
+        const uint32_t i = tid;
+        uint32_t e0, e1;
+        if (a.rope_variant == SLAI_ROPE_NEOX) { e0 = i; e1 = i + HS / 2; } else { e0 = 2 * i; e1 = 2 * i + 1; }
+        float q0 = a.q[(size_t)h * HS + e0], q1 = a.q[(size_t)h * HS + e1];
+        if (fresh) {
+            if (a.qbias) { q0 += a.qbias[(size_t)h * HS + e0]; q1 += a.qbias[(size_t)h * HS + e1]; }
+            const bool rot = a.rope_variant >= 0;
+            float c = 1.0f, s = 0.0f;
+            if (rot) {
+                const float head_dim = (float)((2 * i) % HS);          // rope.slang:36-39
+                const float theta = powf(a.rope_base, -head_dim / (float)HS);
+                const float m_theta = (float)pos * theta;
+                c = cosf(m_theta); s = sinf(m_theta);
+                const float r0 = c * q0 - s * q1, r1 = s * q0 + c * q1;
+                q0 = r0; q1 = r1;
+            }
+            if (own_new) {
+                float k0 = a.knew[hoff + e0], k1 = a.knew[hoff + e1];
+                float v0 = a.vnew[hoff + e0], v1 = a.vnew[hoff + e1];
+                if (a.kbias) { k0 += a.kbias[hoff + e0]; k1 += a.kbias[hoff + e1]; }
+                if (a.vbias) { v0 += a.vbias[hoff + e0]; v1 += a.vbias[hoff + e1]; }
+                if (rot) {
+                    const float kr0 = c * k0 - s * k1, kr1 = s * k0 + c * k1;
+                    k0 = kr0; k1 = kr1;
+                }
+                sk[e0] = C::round(k0); sk[e1] = C::round(k1);
+                sv[e0] = C::round(v0); sv[e1] = C::round(v1);
+                if (h % a.kv_mul == 0) {
+                    CT *kd = kc + (size_t)pos * a.kv_dim + hoff, *vd = vc + (size_t)pos * a.kv_dim + hoff;
+                    C::store(kd + e0, k0); C::store(kd + e1, k1);
+                    C::store(vd + e0, v0); C::store(vd + e1, v1);
+                }
+            }
+        }
+        sq[e0] = q0; sq[e1] = q1;
+    }
+    __syncthreads();
+
+    // ---- scores: 4 lanes per position, each a contiguous quarter of the head ---------------------------------------
+    const uint32_t sub = tid & 3;
+    float qr[EPL];
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) qr[j] = sq[sub * EPL + j];
+    const float root = sqrtf((float)HS);
+    float lmax = -FLT_MAX;
+    for (uint32_t tb = t0; tb < t1; tb += NT / 4) {           // uniform trip count: the shuffles below need whole waves
+        const uint32_t t = tb + tid / 4;
+        const bool live = t < t1;
+        const uint32_t tc = live ? t : t1 - 1;
+        const bool use_new = own_new && tc == pos;           // its cache row is being written by this very launch
+        const CT *kp = kc + (size_t)(use_new ? t0 : tc) * a.kv_dim + hoff + sub * EPL;
+        float kv[EPL];
+#pragma unroll
+        for (int j = 0; j < EPL / 8; ++j) {
+            float tmp[8];
+            Vec8<F16>::load(kp + 8 * j, tmp);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) kv[8 * j + q] = tmp[q];
+        }
+        if (use_new) {
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) kv[j] = sk[sub * EPL + j];
+        }
+        float part = 0.0f;
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) part = fmaf(qr[j], kv[j], part);
+        part += __shfl_xor(part, 1, 64);
+        part += __shfl_xor(part, 2, 64);
+        const float sc = part / root;                        // cpu.rs:521 `score /= sqrt(head_size)`
+        if (live) {
+            if (sub == 0) sscore[t - t0] = sc;
+            lmax = fmaxf(lmax, sc);
+        }
+    }
+    lmax = wave_max(lmax);
+    if (lane == 0) sred[wave] = lmax;
+    __syncthreads();
+    float m = sred[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) m = fmaxf(m, sred[w]);
+    __syncthreads();
+
+    // ---- exp and sum ---------------------------------------------------------------------------------------------
+    float lsum = 0.0f;
+    for (uint32_t t = t0 + tid; t < t1; t += NT) {
+        const float e = expf(sscore[t - t0] - m);
+        sscore[t - t0] = e;
+        lsum += e;
+    }
+    lsum = wave_sum(lsum);
+    if (lane == 0) sred[wave] = lsum;
+    __syncthreads();
+    float l = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) l += sred[w];
+
+    // ---- weighted sum of values: lane = 8 elements of a position, VG positions per pass, 4 passes in flight --------
+    const uint32_t vg = tid / LPP, ve = (tid % LPP) * 8;
+    float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (uint32_t tb = t0; tb < t1; tb += 4 * VG) {
+        float vv[4][8], pp[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t t = tb + u * VG + vg;
+            const bool live = t < t1;
+            const uint32_t tc = live ? t : t0;
+            const bool use_new = own_new && tc == pos;
+            Vec8<F16>::load(vc + (size_t)(use_new ? t0 : tc) * a.kv_dim + hoff + ve, vv[u]);
+            pp[u] = live ? sscore[tc - t0] : 0.0f;
+            if (use_new) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) vv[u][q] = sv[ve + q];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) o[q] = fmaf(pp[u], vv[u][q], o[q]);
+        }
+    }
+    // lanes of a wave that hold the same elements: 64 / LPP position groups per wave
+#pragma unroll
+    for (int msk = LPP; msk < 64; msk <<= 1) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) o[q] += __shfl_xor(o[q], msk, 64);
+    }
+    if (lane < LPP) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) sacc[wave][lane * 8 + q] = o[q];
+    }
+    __syncthreads();
+    if (tid < HS) {
+        float r = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) r += sacc[w][tid];
+        if (a.n_splits == 1) {
+            a.out[(size_t)h * HS + tid] = r / l;
+        } else {
+            float *po = a.scratch + ((size_t)h * a.n_splits + split) * (HS + 2);
+            po[tid] = r;
+            if (tid == 0) { po[HS] = (t1 > t0) ? m : -FLT_MAX; po[HS + 1] = (t1 > t0) ? l : 0.0f; }
+        }
+    }
+}
+
 // grid = n_heads, block = 128: merge the per-split (max, sum, unnormalised output) triples.
 // n_splits <= 64: one lane per split computes its weight exp(m_s - M) / L, then every thread
 // accumulates its output elements with independent loads.
@@ -222,7 +415,14 @@ hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
     const size_t smem = (size_t)max_split_len * sizeof(float);
     if (smem > 48 * 1024) return hipErrorInvalidValue;
     dim3 grid(a.n_heads, a.n_splits);
-    if (a.kv_f16) attn_kernel<true><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
+    const bool fast = (a.head_size == 64 || a.head_size == 128) && a.kv_dim % 8 == 0;
+    if (fast && a.n_splits == 1) {
+        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 1024, 128><<<grid, 1024, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 1024, 128><<<grid, 1024, smem, s>>>(a, max_split_len); }
+        else { if (a.kv_f16) attn_fast_kernel<true, 1024, 64><<<grid, 1024, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 1024, 64><<<grid, 1024, smem, s>>>(a, max_split_len); }
+    } else if (fast) {
+        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 256, 128><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 128><<<grid, 256, smem, s>>>(a, max_split_len); }
+        else { if (a.kv_f16) attn_fast_kernel<true, 256, 64><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 64><<<grid, 256, smem, s>>>(a, max_split_len); }
+    } else if (a.kv_f16) attn_kernel<true><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
     else attn_kernel<false><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

@@ -532,6 +532,8 @@ SLAI_EXPORT int slai_softmax_cols(slai_ctx *ctx, slai_view m) {
 namespace slai {
 uint32_t pick_attn_splits(const slai_ctx *ctx, uint32_t n_heads, uint32_t seq_len) {
     if (ctx->attn_splits > 0) return (uint32_t)ctx->attn_splits;
+    // short contexts: one workgroup per head walks the whole context, no combine pass
+    if (seq_len <= 1024) return 1;
     // enough workgroups to cover the chip, at least ~32 positions per split at full context
     uint32_t s = (512 + n_heads - 1) / n_heads;
     uint32_t cap = seq_len / 32 ? seq_len / 32 : 1;

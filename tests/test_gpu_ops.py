@@ -124,7 +124,12 @@ def test_argmax_first_maximum(backend):
 @pytest.mark.parametrize("cfg", [dict(n_heads=6, kv_mul=1, hs=48, seq=256, pos=37),
                                  dict(n_heads=12, kv_mul=3, hs=64, seq=96, pos=95),
                                  dict(n_heads=32, kv_mul=1, hs=128, seq=512, pos=300),
-                                 dict(n_heads=8, kv_mul=2, hs=128, seq=64, pos=0)])
+                                 dict(n_heads=8, kv_mul=2, hs=128, seq=64, pos=0),
+                                 # long contexts take the split (flash-decoding) form with a combine pass
+                                 dict(n_heads=32, kv_mul=1, hs=128, seq=4096, pos=4000),
+                                 dict(n_heads=8, kv_mul=4, hs=64, seq=2048, pos=1029),
+                                 dict(n_heads=6, kv_mul=1, hs=48, seq=1536, pos=700),
+                                 dict(n_heads=4, kv_mul=1, hs=128, seq=2048, pos=5)])
 @pytest.mark.parametrize("f16", [False, True])
 def test_attention_fused_and_reference_sequence(backend, oracle_lib, cfg, f16):
     """`BatchedMultiqueryAttention::launch`: the fused op and the reference's own four-launch
