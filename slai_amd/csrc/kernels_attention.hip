@@ -35,12 +35,17 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// binary16 <-> binary32 with the hardware converters (round to nearest even, subnormals kept): one instruction per
+// value instead of the bit-level routine the weight decoders share with the host.  Finite values convert identically.
+__device__ __forceinline__ float h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t f2h(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+
 template <bool F16> struct KV;
 template <> struct KV<true> {
     using T = uint16_t;
-    __device__ static float2 load2(const T *p) { uint32_t w = *reinterpret_cast<const uint32_t *>(p); return make_float2(decode_f16((uint16_t)(w & 0xffffu)), decode_f16((uint16_t)(w >> 16))); }
-    __device__ static float round(float v) { return decode_f16(encode_f16(v)); }
-    __device__ static void store(T *p, float v) { *p = encode_f16(v); }
+    __device__ static float2 load2(const T *p) { uint32_t w = *reinterpret_cast<const uint32_t *>(p); return make_float2(h2f((uint16_t)(w & 0xffffu)), h2f((uint16_t)(w >> 16))); }
+    __device__ static float round(float v) { return h2f(f2h(v)); }
+    __device__ static void store(T *p, float v) { *p = f2h(v); }
 };
 template <> struct KV<false> {
     using T = float;
@@ -191,14 +196,26 @@ __global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_
 // context (no combine pass; short contexts), NT = 256 the split form.
 template <bool F16> struct Vec8;
 template <> struct Vec8<true> {   // 8 f16 = 16 bytes
+    struct Raw { uint4 w; };
+    __device__ static Raw load_raw(const uint16_t *p) { return Raw{*reinterpret_cast<const uint4 *>(p)}; }
+    __device__ static void decode(const Raw &r, float (&o)[8]) {
+        const uint32_t u[4] = {r.w.x, r.w.y, r.w.z, r.w.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { o[2 * i] = h2f((uint16_t)(u[i] & 0xffffu)); o[2 * i + 1] = h2f((uint16_t)(u[i] >> 16)); }
+    }
     __device__ static void load(const uint16_t *p, float (&o)[8]) {
         const uint4 w = *reinterpret_cast<const uint4 *>(p);
         const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { o[2 * i] = decode_f16((uint16_t)(u[i] & 0xffffu)); o[2 * i + 1] = decode_f16((uint16_t)(u[i] >> 16)); }
+        for (int i = 0; i < 4; ++i) { o[2 * i] = h2f((uint16_t)(u[i] & 0xffffu)); o[2 * i + 1] = h2f((uint16_t)(u[i] >> 16)); }
     }
 };
 template <> struct Vec8<false> {  // 8 f32 = 32 bytes
+    struct Raw { float4 a, b; };
+    __device__ static Raw load_raw(const float *p) { return Raw{*reinterpret_cast<const float4 *>(p), *reinterpret_cast<const float4 *>(p + 4)}; }
+    __device__ static void decode(const Raw &r, float (&o)[8]) {
+        o[0] = r.a.x; o[1] = r.a.y; o[2] = r.a.z; o[3] = r.a.w; o[4] = r.b.x; o[5] = r.b.y; o[6] = r.b.z; o[7] = r.b.w;
+    }
     __device__ static void load(const float *p, float (&o)[8]) {
         const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + 4);
         o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
@@ -230,6 +247,25 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     const size_t hoff = (size_t)kvh * HS;
     const bool fresh = a.knew != nullptr;
     const bool own_new = fresh && t0 <= pos && pos < t1;
+
+    // ---- the first pass of keys and values is requested before anything else is computed: they depend on nothing
+    // but the position, and their latency then overlaps the q load, the RoPE and the softmax ----------------------
+    const uint32_t sub = tid & 3;
+    const uint32_t vg = tid / LPP, ve = (tid % LPP) * 8;
+    typename Vec8<F16>::Raw kv0[EPL / 8], vv0[4];             // kept undecoded: fewer registers while they wait
+    {
+        const uint32_t t = t0 + tid / 4;
+        const uint32_t tc = (t < t1 && !(own_new && t == pos)) ? t : t0;     // the fresh row comes from LDS later
+        const CT *kp = kc + (size_t)tc * a.kv_dim + hoff + sub * EPL;
+#pragma unroll
+        for (int j = 0; j < EPL / 8; ++j) kv0[j] = Vec8<F16>::load_raw(kp + 8 * j);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t tv = t0 + u * VG + vg;
+            const uint32_t tvc = (tv < t1 && !(own_new && tv == pos)) ? tv : t0;
+            vv0[u] = Vec8<F16>::load_raw(vc + (size_t)tvc * a.kv_dim + hoff + ve);
+        }
+    }
 
     // ---- q (and the fresh k/v) into LDS, with bias and RoPE when fused: identical to attn_kernel ------------------
     if (tid < HS / 2) {
@@ -272,7 +308,6 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     __syncthreads();
 
     // ---- scores: 4 lanes per position, each a contiguous quarter of the head ---------------------------------------
-    const uint32_t sub = tid & 3;
     float qr[EPL];
 #pragma unroll
     for (int j = 0; j < EPL; ++j) qr[j] = sq[sub * EPL + j];
@@ -285,12 +320,22 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
         const bool use_new = own_new && tc == pos;           // its cache row is being written by this very launch
         const CT *kp = kc + (size_t)(use_new ? t0 : tc) * a.kv_dim + hoff + sub * EPL;
         float kv[EPL];
+        if (tb == t0) {
 #pragma unroll
-        for (int j = 0; j < EPL / 8; ++j) {
-            float tmp[8];
-            Vec8<F16>::load(kp + 8 * j, tmp);
+            for (int j = 0; j < EPL / 8; ++j) {
+                float tmp[8];
+                Vec8<F16>::decode(kv0[j], tmp);
 #pragma unroll
-            for (int q = 0; q < 8; ++q) kv[8 * j + q] = tmp[q];
+                for (int q = 0; q < 8; ++q) kv[8 * j + q] = tmp[q];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPL / 8; ++j) {
+                float tmp[8];
+                Vec8<F16>::load(kp + 8 * j, tmp);
+#pragma unroll
+                for (int q = 0; q < 8; ++q) kv[8 * j + q] = tmp[q];
+            }
         }
         if (use_new) {
 #pragma unroll
@@ -330,7 +375,6 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     for (int w = 0; w < NW; ++w) l += sred[w];
 
     // ---- weighted sum of values: lane = 8 elements of a position, VG positions per pass, 4 passes in flight --------
-    const uint32_t vg = tid / LPP, ve = (tid % LPP) * 8;
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     for (uint32_t tb = t0; tb < t1; tb += 4 * VG) {
         float vv[4][8], pp[4];
@@ -340,7 +384,11 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
             const bool live = t < t1;
             const uint32_t tc = live ? t : t0;
             const bool use_new = own_new && tc == pos;
-            Vec8<F16>::load(vc + (size_t)(use_new ? t0 : tc) * a.kv_dim + hoff + ve, vv[u]);
+            if (tb == t0) {
+                Vec8<F16>::decode(vv0[u], vv[u]);
+            } else {
+                Vec8<F16>::load(vc + (size_t)(use_new ? t0 : tc) * a.kv_dim + hoff + ve, vv[u]);
+            }
             pp[u] = live ? sscore[tc - t0] : 0.0f;
             if (use_new) {
 #pragma unroll
