@@ -67,6 +67,15 @@ SLAI_HD float decode_f16(uint16_t h) {
     return bits_to_float(sign | ((e + 112) << 23) | (m << 13));
 #endif
 }
+// binary16 -> binary32 inside the GEMV dot products (not the bit-exact dequantiser): the hardware converter on
+// the device (one instruction; identical to decode_f16 for every non-NaN input), decode_f16 on the host.
+SLAI_HD float gemv_f16(uint16_t h) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (float)__builtin_bit_cast(_Float16, h);
+#else
+    return decode_f16(h);
+#endif
+}
 
 // IEEE binary32 -> binary16, round to nearest even (KV-cache store).
 SLAI_HD uint16_t encode_f16(float f) {
@@ -238,7 +247,7 @@ template <> struct Chunk<T_Q4_K> {
     }
     SLAI_HD static float dot(const Data &d, uint32_t c, const float *x, const float *xs) {
         const int j = (c & 7) >> 1;
-        float dd = decode_f16((uint16_t)(d.hdr.x & 0xffffu)), dmin = decode_f16((uint16_t)(d.hdr.x >> 16));
+        float dd = gemv_f16((uint16_t)(d.hdr.x & 0xffffu)), dmin = gemv_f16((uint16_t)(d.hdr.x >> 16));
         uint32_t sc0, m0, sc1, m1;
         scale_min_k4(d.hdr, 2 * j, sc0, m0);
         scale_min_k4(d.hdr, 2 * j + 1, sc1, m1);
@@ -259,7 +268,7 @@ template <> struct Chunk<T_Q5_K> {
     }
     SLAI_HD static float dot(const Data &d, uint32_t c, const float *x, const float *xs) {
         const int j = (c & 7) >> 1;
-        float dd = decode_f16((uint16_t)(d.hdr.x & 0xffffu)), dmin = decode_f16((uint16_t)(d.hdr.x >> 16));
+        float dd = gemv_f16((uint16_t)(d.hdr.x & 0xffffu)), dmin = gemv_f16((uint16_t)(d.hdr.x >> 16));
         uint32_t sc0, m0, sc1, m1;
         scale_min_k4(d.hdr, 2 * j, sc0, m0);
         scale_min_k4(d.hdr, 2 * j + 1, sc1, m1);
@@ -299,7 +308,7 @@ template <> struct Chunk<T_Q6_K> {
         U4 q4 = or4(and4(shr4(d.ql32, 4), 0x0F0F0F0Fu), shl4(and4(shr4(d.qh, 6), 0x03030303u), 4));
         float a = s0 * (dot16b(q1, x) - 32.0f * xs[0]) + s1 * (dot16b(q2, x + 16) - 32.0f * xs[1]);
         float b = s2 * (dot16b(q3, x + 32) - 32.0f * xs[2]) + s3 * (dot16b(q4, x + 48) - 32.0f * xs[3]);
-        return decode_f16(d.d) * (a + b);
+        return gemv_f16(d.d) * (a + b);
     }
 };
 
@@ -314,7 +323,7 @@ template <> struct Chunk<T_Q8_0> {
     SLAI_HD static float dot(const Data &d, uint32_t c, const float *x, const float *xs) {
         // int8 -> (q + 128) as unsigned bytes; the 128 comes back out through the run sum
         float s = dot16b(xor4(d.qs, 0x80808080u), x);
-        return decode_f16(d.d) * (s - 128.0f * xs[0]);
+        return gemv_f16(d.d) * (s - 128.0f * xs[0]);
     }
 };
 
@@ -329,7 +338,7 @@ template <> struct Chunk<T_Q4_0> {
     SLAI_HD static float dot(const Data &d, uint32_t c, const float *x, const float *xs) {
         float slo = dot16b(and4(d.qs, 0x0F0F0F0Fu), x);
         float shi = dot16b(and4(shr4(d.qs, 4), 0x0F0F0F0Fu), x + 16);
-        return decode_f16(d.d) * ((slo + shi) - 8.0f * (xs[0] + xs[1]));
+        return gemv_f16(d.d) * ((slo + shi) - 8.0f * (xs[0] + xs[1]));
     }
 };
 
@@ -343,8 +352,8 @@ template <> struct Chunk<T_F16> {
         const uint32_t w[4] = {d.v.x, d.v.y, d.v.z, d.v.w};
         float a = 0.0f;
         for (int i = 0; i < 4; ++i) {
-            a = fmaf(decode_f16((uint16_t)(w[i] & 0xffffu)), x[2 * i], a);
-            a = fmaf(decode_f16((uint16_t)(w[i] >> 16)), x[2 * i + 1], a);
+            a = fmaf(gemv_f16((uint16_t)(w[i] & 0xffffu)), x[2 * i], a);
+            a = fmaf(gemv_f16((uint16_t)(w[i] >> 16)), x[2 * i + 1], a);
         }
         return a;
     }

@@ -146,6 +146,16 @@ SLAI_HD float tiled_dequant_elem(const TiledGeom &g, const uint8_t *base, uint32
 // dotn<N> computes the dot products of N matrices' rows with the same activations in lockstep (N = 2: the
 // gate/up pair), so that on-demand activations are fetched once.
 // ---------------------------------------------------------------------------
+// binary16 -> binary32 for block scales inside the dot products: the hardware converter on the device (one
+// instruction; identical to decode_f16 for every non-NaN input), decode_f16 on the host.
+SLAI_HD float scale_f16(uint16_t h) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (float)__builtin_bit_cast(_Float16, h);
+#else
+    return decode_f16(h);
+#endif
+}
+
 template <class X, class S> SLAI_HD void stage_dot(const X &x, const S &st, const U4 &q1, const U4 &q2, float &a1, float &a2) {
     // q1 pairs with chunk I1, q2 with chunk I2; two independent accumulation chains interleaved word by word
     a1 = x.template fma4<0, 0>(st, q1.x, a1); a2 = x.template fma4<1, 0>(st, q2.x, a2);
@@ -192,7 +202,7 @@ template <> struct Tiled<T_Q4_K> {
         float dd[N], dmin[N], accm[N];
         for (int n = 0; n < N; ++n) {
             const U4 &h = d[n]->p[0];
-            dd[n] = decode_f16((uint16_t)(h.x & 0xffffu)); dmin[n] = decode_f16((uint16_t)(h.x >> 16));
+            dd[n] = scale_f16((uint16_t)(h.x & 0xffffu)); dmin[n] = scale_f16((uint16_t)(h.x >> 16));
             // all eight 6-bit scales / mins at once (quantization.rs:381-389 applied bytewise)
             a.sc_lo[n] = h.y & 0x3f3f3f3fu;
             a.sc_hi[n] = (h.w & 0x0f0f0f0fu) | (((h.y >> 6) & 0x03030303u) << 4);
@@ -270,7 +280,7 @@ template <> struct Tiled<T_Q6_K> {
         }
         const auto st0 = x.template stage<c1(0), c2(0)>();
         stages<0, N>(d, x, st0, acc);
-        for (int n = 0; n < N; ++n) out[n] = decode_f16(tail[n]) * acc[n];
+        for (int n = 0; n < N; ++n) out[n] = scale_f16(tail[n]) * acc[n];
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
         const Data *dp[1] = {&d};
@@ -290,7 +300,7 @@ template <> struct Tiled<T_Q8_0> {
     SLAI_HD static float scale_of(const Data &d, int B) {
         const U4 &s = d.p[16];
         const uint32_t w = B < 2 ? s.x : (B < 4 ? s.y : (B < 6 ? s.z : s.w));
-        return decode_f16((uint16_t)((B & 1) ? (w >> 16) : (w & 0xffffu)));
+        return scale_f16((uint16_t)((B & 1) ? (w >> 16) : (w & 0xffffu)));
     }
     template <int K, int N, class X, class S> SLAI_HD static void compute(const Data *const *d, const X &x, const S &st, float *acc) {
         for (int n = 0; n < N; ++n) {
