@@ -232,11 +232,14 @@ struct AttnLaunch {
     const float *knew, *vnew;  // null: caches already hold position pos and q is already rotated
     const float *qbias, *kbias, *vbias;  // optional (Qwen2), added before RoPE
     int rope_variant; float rope_base;
+    const float *rope_theta;   // optional: head_size/2 frequencies base^(-(2i mod hs)/hs), i = pair index (device)
     float *out;              // [n_heads*head_size]
     float *scratch;          // n_heads*n_splits*(head_size+2) floats when n_splits > 1
     uint32_t n_splits;
 };
 hipError_t launch_attention(hipStream_t s, const AttnLaunch &a);
+// out[i] = powf(base, -((2*i) % head_size) / head_size), i < head_size/2
+hipError_t launch_rope_theta(hipStream_t s, float *out, uint32_t head_size, float base);
 size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n_splits);
 
 }  // namespace slai

@@ -99,6 +99,7 @@ struct Llama2Weights {               // transformer.rs:194-199
 struct Llama2State {                 // transformer.rs:16-44
     GpuTensor x, xb, xb2, hb, hb2, q, att, logits;
     GpuTensor kcol, vcol;            // fresh K/V of the current position (fused path, and staging for f16 caches)
+    GpuTensor rope_theta;            // fused path: head_size/2 RoPE frequencies
     GpuTensor xw;                    // fused path: norm-weighted copy of x (+ dim/16 sums of 16) left by the producer of x
     std::vector<GpuTensor> key_cache, value_cache;
     slai_buffer *rope_config = nullptr, *rms_norm_config = nullptr, *attn_params = nullptr;
@@ -200,6 +201,8 @@ int slai_llama2::load(const slai_gguf *gg) {
     TRY(GpuTensor::vector(ctx, dim, STORAGE | COPY_SRC, &s.q));
     TRY(GpuTensor::vector(ctx, kvd, STORAGE, &s.kcol));
     TRY(GpuTensor::vector(ctx, dim + dim / 16 + 16, STORAGE, &s.xw));
+    TRY(GpuTensor::vector(ctx, head_size() / 2, STORAGE, &s.rope_theta));
+    SLAI_HIP_TRY(ctx, launch_rope_theta(ctx->stream, (float *)s.rope_theta.buf->dptr, head_size(), config.rope_base_freq));
     TRY(GpuTensor::vector(ctx, kvd, STORAGE, &s.vcol));
     const int cdt = kv_dtype == SLAI_KV_F16 ? SLAI_DT_F16 : SLAI_DT_F32;
     s.key_cache.resize(config.n_layers); s.value_cache.resize(config.n_layers);
@@ -306,6 +309,7 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
             a.kbias = wl.attn_k_bias.buf ? (const float *)wl.attn_k_bias.buf->dptr : nullptr;
             a.vbias = wl.attn_v_bias.buf ? (const float *)wl.attn_v_bias.buf->dptr : nullptr;
             a.rope_variant = rope_variant(); a.rope_base = config.rope_base_freq;
+            a.rope_theta = (const float *)s.rope_theta.buf->dptr;
             a.out = xb; a.scratch = ctx->attn_scratch; a.n_splits = attn_splits;
             hipError_t e = launch_attention(ctx->stream, a);
             if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "attention: unsupported head size or context length");
@@ -401,7 +405,7 @@ SLAI_EXPORT void slai_llama2_destroy(slai_llama2 *m) {
     slai_qmat_destroy(ctx, m->weights.token_embd);
     m->weights.output_norm.destroy(ctx);
     Llama2State &s = m->state;
-    for (GpuTensor *t : {&s.x, &s.xb, &s.xb2, &s.hb, &s.hb2, &s.q, &s.att, &s.logits, &s.kcol, &s.vcol, &s.xw}) t->destroy(ctx);
+    for (GpuTensor *t : {&s.x, &s.xb, &s.xb2, &s.hb, &s.hb2, &s.q, &s.att, &s.logits, &s.kcol, &s.vcol, &s.xw, &s.rope_theta}) t->destroy(ctx);
     for (auto &t : s.key_cache) t.destroy(ctx);
     for (auto &t : s.value_cache) t.destroy(ctx);
     for (slai_buffer *b : {s.rope_config, s.rms_norm_config, s.attn_params}) if (b) slai_buffer_destroy(ctx, b);

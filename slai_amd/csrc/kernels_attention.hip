@@ -233,7 +233,7 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     constexpr int VG = NT / LPP;                  // positions per pass in the value phase
     extern __shared__ float sscore[];             // [max_split_len]
     __shared__ float sq[HS], sk[HS], sv[HS];
-    __shared__ float sred[NW];
+    __shared__ float sred[NW], sred2[NW];
     __shared__ float sacc[NW][LPP * 8];           // per-wave partial outputs (= HS floats per wave)
 
     const uint32_t h = blockIdx.x, split = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -248,6 +248,26 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     const bool fresh = a.knew != nullptr;
     const bool own_new = fresh && t0 <= pos && pos < t1;
 
+    // ---- requests first: the query pair of this thread (with the fresh key / value and the RoPE frequency), then the
+    // first pass of keys and values.  Nothing below depends on anything but the position. ----------------------------
+    uint32_t e0 = 0, e1 = 1;
+    float q0 = 0.0f, q1 = 0.0f, k0 = 0.0f, k1 = 0.0f, v0 = 0.0f, v1 = 0.0f, theta = 0.0f;
+    const bool rot = fresh && a.rope_variant >= 0;             // GPT-2 has learned positions: no rotation
+    if (tid < HS / 2) {
+        const uint32_t i = tid;
+        if (a.rope_variant == SLAI_ROPE_NEOX) { e0 = i; e1 = i + HS / 2; } else { e0 = 2 * i; e1 = 2 * i + 1; }
+        q0 = a.q[(size_t)h * HS + e0]; q1 = a.q[(size_t)h * HS + e1];
+        if (fresh) {
+            if (a.qbias) { q0 += a.qbias[(size_t)h * HS + e0]; q1 += a.qbias[(size_t)h * HS + e1]; }
+            if (rot && a.rope_theta) theta = a.rope_theta[i];
+            if (own_new) {
+                k0 = a.knew[hoff + e0]; k1 = a.knew[hoff + e1];
+                v0 = a.vnew[hoff + e0]; v1 = a.vnew[hoff + e1];
+                if (a.kbias) { k0 += a.kbias[hoff + e0]; k1 += a.kbias[hoff + e1]; }
+                if (a.vbias) { v0 += a.vbias[hoff + e0]; v1 += a.vbias[hoff + e1]; }
+            }
+        }
+    }
     // ---- the first pass of keys and values is requested before anything else is computed: they depend on nothing
     // but the position, and their latency then overlaps the q load, the RoPE and the softmax ----------------------
     const uint32_t sub = tid & 3;
@@ -267,35 +287,25 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
         }
     }
 
-    // ---- q (and the fresh k/v) into LDS, with bias and RoPE when fused: identical to attn_kernel ------------------
+    // ---- q (and the fresh k/v) into LDS, rotated (rope.slang:27-84) ------------------------------------------------
     if (tid < HS / 2) {
-        const uint32_t i = tid;
-        uint32_t e0, e1;
-        if (a.rope_variant == SLAI_ROPE_NEOX) { e0 = i; e1 = i + HS / 2; } else { e0 = 2 * i; e1 = 2 * i + 1; }
-        float q0 = a.q[(size_t)h * HS + e0], q1 = a.q[(size_t)h * HS + e1];
         if (fresh) {
-            if (a.qbias) { q0 += a.qbias[(size_t)h * HS + e0]; q1 += a.qbias[(size_t)h * HS + e1]; }
-            const bool rot = a.rope_variant >= 0;
-            float c = 1.0f, s = 0.0f;
             if (rot) {
-                const float head_dim = (float)((2 * i) % HS);          // rope.slang:36-39
-                const float theta = powf(a.rope_base, -head_dim / (float)HS);
+                // rope.slang:36-39: the angle depends on (2*i) mod head_size for both variants; the frequencies
+                // base^(-(2i mod hs)/hs) come from a table built once with the same powf
+                if (!a.rope_theta) theta = powf(a.rope_base, -(float)((2 * tid) % HS) / (float)HS);
                 const float m_theta = (float)pos * theta;
-                c = cosf(m_theta); s = sinf(m_theta);
-                const float r0 = c * q0 - s * q1, r1 = s * q0 + c * q1;
+                float c, sn;
+                sincosf(m_theta, &sn, &c);
+                const float r0 = c * q0 - sn * q1, r1 = sn * q0 + c * q1;
                 q0 = r0; q1 = r1;
+                const float kr0 = c * k0 - sn * k1, kr1 = sn * k0 + c * k1;
+                k0 = kr0; k1 = kr1;
             }
             if (own_new) {
-                float k0 = a.knew[hoff + e0], k1 = a.knew[hoff + e1];
-                float v0 = a.vnew[hoff + e0], v1 = a.vnew[hoff + e1];
-                if (a.kbias) { k0 += a.kbias[hoff + e0]; k1 += a.kbias[hoff + e1]; }
-                if (a.vbias) { v0 += a.vbias[hoff + e0]; v1 += a.vbias[hoff + e1]; }
-                if (rot) {
-                    const float kr0 = c * k0 - s * k1, kr1 = s * k0 + c * k1;
-                    k0 = kr0; k1 = kr1;
-                }
                 sk[e0] = C::round(k0); sk[e1] = C::round(k1);
                 sv[e0] = C::round(v0); sv[e1] = C::round(v1);
+                // several query heads share a kv head: the first of the group writes the cache
                 if (h % a.kv_mul == 0) {
                     CT *kd = kc + (size_t)pos * a.kv_dim + hoff, *vd = vc + (size_t)pos * a.kv_dim + hoff;
                     C::store(kd + e0, k0); C::store(kd + e1, k1);
@@ -358,9 +368,8 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     float m = sred[0];
 #pragma unroll
     for (int w = 1; w < NW; ++w) m = fmaxf(m, sred[w]);
-    __syncthreads();
 
-    // ---- exp and sum ---------------------------------------------------------------------------------------------
+    // ---- exp and sum (their reduction uses an array of its own: no barrier needed before reusing one) --------------
     float lsum = 0.0f;
     for (uint32_t t = t0 + tid; t < t1; t += NT) {
         const float e = expf(sscore[t - t0] - m);
@@ -368,11 +377,11 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
         lsum += e;
     }
     lsum = wave_sum(lsum);
-    if (lane == 0) sred[wave] = lsum;
+    if (lane == 0) sred2[wave] = lsum;
     __syncthreads();
     float l = 0.0f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) l += sred[w];
+    for (int w = 0; w < NW; ++w) l += sred2[w];
 
     // ---- weighted sum of values: lane = 8 elements of a position, VG positions per pass, 4 passes in flight --------
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -426,6 +435,11 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     }
 }
 
+__global__ void rope_theta_kernel(float *out, uint32_t hs, float base) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < hs / 2) out[i] = powf(base, -(float)((2 * i) % hs) / (float)hs);      // rope.slang:36-38
+}
+
 // grid = n_heads, block = 128: merge the per-split (max, sum, unnormalised output) triples.
 // n_splits <= 64: one lane per split computes its weight exp(m_s - M) / L, then every thread
 // accumulates its output elements with independent loads.
@@ -452,6 +466,11 @@ __global__ void __launch_bounds__(128) attn_combine_kernel(const float *scratch,
 }
 
 }  // namespace
+
+hipError_t launch_rope_theta(hipStream_t s, float *out, uint32_t head_size, float base) {
+    rope_theta_kernel<<<(head_size / 2 + 63) / 64, 64, 0, s>>>(out, head_size, base);
+    return hipGetLastError();
+}
 
 size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n_splits) {
     return n_splits > 1 ? (size_t)n_heads * n_splits * (head_size + 2) : 0;
