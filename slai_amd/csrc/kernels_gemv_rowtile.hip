@@ -79,6 +79,24 @@ template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, 
     else tail = 0;
 }
 
+// Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product.
+template <int T, int N> struct UnitLoader {
+    static constexpr int DEPTH = 2;               // stages requested ahead of the one being multiplied
+    using F = Tiled<T>;
+    const uint8_t *unit[N];                       // + lane * 16 already applied
+    const uint8_t *tailp[N];
+    typename F::Data *d[N];
+    uint16_t *t[N];
+    template <int P> __device__ __forceinline__ void piece() const {
+#pragma unroll
+        for (int n = 0; n < N; ++n) d[n]->p[P] = ld128(unit[n] + (size_t)P * 1024);
+    }
+    __device__ __forceinline__ void tail() const {
+#pragma unroll
+        for (int n = 0; n < N; ++n) *t[n] = ld16(tailp[n]);
+    }
+};
+
 // The body for one block format.  `partial` = [DUAL?2:1][NW][64] floats, `red` = [NW] floats.
 template <int T, bool DUAL, bool PREP>
 __device__ __forceinline__ void tile_body(const GemvRowtileParams &p, const GemvRowtileSeg &seg, uint32_t tile, float *partial, float *red) {
@@ -107,12 +125,15 @@ __device__ __forceinline__ void tile_body(const GemvRowtileParams &p, const Gemv
     typename F::Data d, e;
     uint16_t dt = 0, et = 0;
     uint32_t cb = wave;
-    auto request_w = [&]() {
-        if (cb < p.ncb) {
-            const size_t off = ((size_t)tile * p.ncb + cb) * unit_bytes;
-            load_unit<T>(seg.W + off, lane, d, dt);
-            if constexpr (BOTH) load_unit<T>(seg.W2 + off, lane, e, et);
-        }
+    constexpr int NM = DUAL ? 2 : 1;
+    UnitLoader<T, NM> ld;
+    auto point = [&]() {                                      // aim the loader at super-block cb of this tile
+        const size_t off = ((size_t)tile * p.ncb + cb) * unit_bytes;
+        ld.unit[0] = seg.W + off + lane * 16; ld.tailp[0] = seg.W + off + (size_t)F::PT * 1024 + lane * 2; ld.d[0] = &d; ld.t[0] = &dt;
+        if constexpr (DUAL) { ld.unit[1] = seg.W2 + off + lane * 16; ld.tailp[1] = seg.W2 + off + (size_t)F::PT * 1024 + lane * 2; ld.d[1] = &e; ld.t[1] = &et; }
+    };
+    auto request_w = [&]() {                                  // the pieces the first stages need; the rest follow inside the dot product
+        if (cb < p.ncb) { point(); F::lead(ld); }
     };
     if constexpr (PREP) { request_w(); if (norm) request_x(); }
     else { request_x(); request_w(); }
@@ -173,22 +194,16 @@ __device__ __forceinline__ void tile_body(const GemvRowtileParams &p, const Gemv
     for (int it = 0; it < 4; ++it) {
         if (cb < p.ncb) {
             ScalarX X{xs + (size_t)cb * 256, xs + p.ncols + (size_t)cb * 16};
-            if constexpr (DUAL) {
-                if constexpr (!BOTH) load_unit<T>(seg.W2 + ((size_t)tile * p.ncb + cb) * unit_bytes, lane, e, et);
-                const typename F::Data *dp[2] = {&d, &e};
-                const uint16_t tails[2] = {dt, et};
-                float o2[2];
-                F::template dotn<2>(dp, tails, X, o2);        // both matrices in lockstep: one pass over the activations
-                v += o2[0]; v2 += o2[1];
-            } else {
-                v += F::dot(d, dt, X);
-            }
+            const typename F::Data *dp[NM];
+            uint16_t tails[NM];
+            float o2[NM];
+            dp[0] = &d; tails[0] = dt;
+            if constexpr (DUAL) { dp[1] = &e; tails[1] = et; }
+            F::template dotn<NM>(dp, tails, X, o2, ld);       // gated pair: both matrices in lockstep, one pass over the activations
+            v += o2[0];
+            if constexpr (DUAL) v2 += o2[1];
             cb += NW;
-            if (it < 3 && cb < p.ncb) {
-                const size_t off = ((size_t)tile * p.ncb + cb) * unit_bytes;
-                load_unit<T>(seg.W + off, lane, d, dt);
-                if constexpr (BOTH) load_unit<T>(seg.W2 + off, lane, e, et);
-            }
+            if (it < 3 && cb < p.ncb) { point(); F::lead(ld); }
         }
     }
     if constexpr (PREP) {

@@ -156,6 +156,22 @@ SLAI_HD float scale_f16(uint16_t h) {
 #endif
 }
 
+// The quantised pieces may be fetched while the dot product runs: `L` (a "loader") issues the load of piece P of
+// every matrix with L.piece<P>() (and L.tail() for the 2-byte tail); the dot products call lead() for what the
+// first stages need and ahead<K>() at stage K for what stage K + L::DEPTH needs, so a wave never has more than a
+// few requests waiting to be issued and starts multiplying as soon as its first pieces arrive.  NoLoader is for
+// data that is already in registers.
+struct NoLoader {
+    static constexpr int DEPTH = 8;
+    template <int P> SLAI_HD void piece() const {}
+    SLAI_HD void tail() const {}
+};
+#if defined(__HIP_DEVICE_COMPILE__)
+#define SLAI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#else
+#define SLAI_SCHED_FENCE() ((void)0)
+#endif
+
 template <class X, class S> SLAI_HD void stage_dot(const X &x, const S &st, const U4 &q1, const U4 &q2, float &a1, float &a2) {
     // q1 pairs with chunk I1, q2 with chunk I2; two independent accumulation chains interleaved word by word
     a1 = x.template fma4<0, 0>(st, q1.x, a1); a2 = x.template fma4<1, 0>(st, q2.x, a2);
@@ -188,16 +204,26 @@ template <> struct Tiled<T_Q4_K> {
             }
         }
     }
-    template <int K, int N, class X, class S> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, Acc<N> &a) {
+    // stage K reads piece 1 + K; the header is piece 0
+    template <int P, class L> SLAI_HD static void lead_from(const L &ld) {
+        if constexpr (P <= L::DEPTH && P < PT) { ld.template piece<P>(); lead_from<P + 1>(ld); }
+    }
+    template <class L> SLAI_HD static void lead(const L &ld) { lead_from<0>(ld); }
+    template <int K, class L> SLAI_HD static void ahead(const L &ld) {
+        if constexpr (1 + K + L::DEPTH < PT) ld.template piece<1 + K + L::DEPTH>();
+    }
+    template <int K, int N, class X, class S, class L> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, Acc<N> &a, const L &ld) {
+        ahead<K>(ld);
+        SLAI_SCHED_FENCE();
         if constexpr (K < 7) {
             const auto nxt = x.template stage<c1(K + 1), c2(K + 1)>();
             compute<K, N>(d, x, st, a);
-            stages<K + 1, N>(d, x, nxt, a);
+            stages<K + 1, N>(d, x, nxt, a, ld);
         } else {
             compute<K, N>(d, x, st, a);
         }
     }
-    template <int N, class X> SLAI_HD static void dotn(const Data *const *d, const uint16_t * /*tail*/, const X &x, float *out) {
+    template <int N, class X, class L = NoLoader> SLAI_HD static void dotn(const Data *const *d, const uint16_t * /*tail*/, const X &x, float *out, const L &ld = L()) {
         Acc<N> a;
         float dd[N], dmin[N], accm[N];
         for (int n = 0; n < N; ++n) {
@@ -216,7 +242,7 @@ template <> struct Tiled<T_Q4_K> {
             accm[n] = am; a.accd[n] = 0.0f; a.slo[n] = 0.0f; a.shi[n] = 0.0f;
         }
         const auto st0 = x.template stage<c1(0), c2(0)>();
-        stages<0, N>(d, x, st0, a);
+        stages<0, N>(d, x, st0, a, ld);
         for (int n = 0; n < N; ++n) out[n] = dd[n] * a.accd[n] - dmin[n] * accm[n];
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
@@ -259,16 +285,32 @@ template <> struct Tiled<T_Q6_K> {
             acc[n] = fmaf(scale_of(*d[n], I, M, 2 * P + 1), tb, acc[n]);
         }
     }
-    template <int K, int N, class X, class S> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc) {
+    // stages 2G and 2G+1 (G = 0..3: I = G/2, M = G%2) read the piece group {4I+M, 4I+2+M, 8+2I+M}; the scales (piece
+    // 12) and the tail are needed first
+    template <int G, class L> SLAI_HD static void group(const L &ld) {
+        constexpr int I = G / 2, M = G % 2;
+        ld.template piece<4 * I + M>(); ld.template piece<4 * I + 2 + M>(); ld.template piece<8 + 2 * I + M>();
+    }
+    template <int G, class L> SLAI_HD static void lead_from(const L &ld) {
+        if constexpr (2 * G <= L::DEPTH && G < 4) { group<G>(ld); lead_from<G + 1>(ld); }
+    }
+    template <class L> SLAI_HD static void lead(const L &ld) { ld.template piece<12>(); ld.tail(); lead_from<0>(ld); }
+    template <int K, class L> SLAI_HD static void ahead(const L &ld) {
+        // group G is first used at stage 2G: led when 2G <= DEPTH, otherwise requested at stage 2G - DEPTH
+        if constexpr (K > 0 && (K + L::DEPTH) % 2 == 0 && (K + L::DEPTH) / 2 < 4) group<(K + L::DEPTH) / 2>(ld);
+    }
+    template <int K, int N, class X, class S, class L> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc, const L &ld) {
+        ahead<K>(ld);
+        SLAI_SCHED_FENCE();
         if constexpr (K < 7) {
             const auto nxt = x.template stage<c1(K + 1), c2(K + 1)>();
             compute<K, N>(d, x, st, acc);
-            stages<K + 1, N>(d, x, nxt, acc);
+            stages<K + 1, N>(d, x, nxt, acc, ld);
         } else {
             compute<K, N>(d, x, st, acc);
         }
     }
-    template <int N, class X> SLAI_HD static void dotn(const Data *const *d, const uint16_t *tail, const X &x, float *out) {
+    template <int N, class X, class L = NoLoader> SLAI_HD static void dotn(const Data *const *d, const uint16_t *tail, const X &x, float *out, const L &ld = L()) {
         float acc[N];
         for (int n = 0; n < N; ++n) {
             // the -32 of every 6-bit value, through the activation sums: -32 * sum_j scale_j * sum16(chunk_j)
@@ -279,7 +321,7 @@ template <> struct Tiled<T_Q6_K> {
             acc[n] = -32.0f * c;
         }
         const auto st0 = x.template stage<c1(0), c2(0)>();
-        stages<0, N>(d, x, st0, acc);
+        stages<0, N>(d, x, st0, acc, ld);
         for (int n = 0; n < N; ++n) out[n] = scale_f16(tail[n]) * acc[n];
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
@@ -310,16 +352,26 @@ template <> struct Tiled<T_Q8_0> {
             acc[n] = fmaf(scale_of(*d[n], K), s + s2, acc[n]);
         }
     }
-    template <int K, int N, class X, class S> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc) {
+    // stage K reads pieces 2K and 2K+1; the scales are piece 16
+    template <int K, class L> SLAI_HD static void lead_from(const L &ld) {
+        if constexpr (K <= L::DEPTH && K < 8) { ld.template piece<2 * K>(); ld.template piece<2 * K + 1>(); lead_from<K + 1>(ld); }
+    }
+    template <class L> SLAI_HD static void lead(const L &ld) { ld.template piece<16>(); lead_from<0>(ld); }
+    template <int K, class L> SLAI_HD static void ahead(const L &ld) {
+        if constexpr (K + 1 + L::DEPTH < 8) { ld.template piece<2 * (K + 1 + L::DEPTH)>(); ld.template piece<2 * (K + 1 + L::DEPTH) + 1>(); }
+    }
+    template <int K, int N, class X, class S, class L> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc, const L &ld) {
+        ahead<K>(ld);
+        SLAI_SCHED_FENCE();
         if constexpr (K < 7) {
             const auto nxt = x.template stage<c1(K + 1), c2(K + 1)>();
             compute<K, N>(d, x, st, acc);
-            stages<K + 1, N>(d, x, nxt, acc);
+            stages<K + 1, N>(d, x, nxt, acc, ld);
         } else {
             compute<K, N>(d, x, st, acc);
         }
     }
-    template <int N, class X> SLAI_HD static void dotn(const Data *const *d, const uint16_t * /*tail*/, const X &x, float *out) {
+    template <int N, class X, class L = NoLoader> SLAI_HD static void dotn(const Data *const *d, const uint16_t * /*tail*/, const X &x, float *out, const L &ld = L()) {
         float acc[N];
         for (int n = 0; n < N; ++n) {
             float c = 0.0f;
@@ -327,7 +379,7 @@ template <> struct Tiled<T_Q8_0> {
             acc[n] = -128.0f * c;
         }
         const auto st0 = x.template stage<c1(0), c2(0)>();
-        stages<0, N>(d, x, st0, acc);
+        stages<0, N>(d, x, st0, acc, ld);
         for (int n = 0; n < N; ++n) out[n] = acc[n];
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
