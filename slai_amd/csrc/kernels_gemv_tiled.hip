@@ -84,6 +84,24 @@ template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, 
     else tail = 0;
 }
 
+// Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product.
+template <int T, int N> struct UnitLoader {
+    static constexpr int DEPTH = 1;               // stages requested ahead of the one being multiplied
+    using F = Tiled<T>;
+    const uint8_t *unit[N];                       // + lane * 16 already applied
+    const uint8_t *tailp[N];
+    typename F::Data *d[N];
+    uint16_t *t[N];
+    template <int P> __device__ __forceinline__ void piece() const {
+#pragma unroll
+        for (int n = 0; n < N; ++n) d[n]->p[P] = ld128(unit[n] + (size_t)P * 1024);
+    }
+    __device__ __forceinline__ void tail() const {
+#pragma unroll
+        for (int n = 0; n < N; ++n) *t[n] = ld16(tailp[n]);
+    }
+};
+
 // One workgroup = `ngroups` waves; wave w owns column group w of every tile the workgroup visits.  The
 // workgroup walks its tiles with a stride of the segment's workgroup count; the next tile's weights
 // are requested before the current tile is consumed.
@@ -132,25 +150,32 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
             for (int i = 0; i < 16; ++i) nb[i] = p.norm_b[xoff + 16 * i];
         }
     }
-    // two register buffers used alternately: while one tile is consumed the other one's loads are in flight
-    typename F::Data dA, dB;
-    typename F::Data eA, eB;                                 // second matrix of a gated pair
-    uint16_t tA = 0, tB = 0, uA = 0, uB = 0;
-    uint32_t tile = blk;
-    float old0 = 0.0f, bias0 = 0.0f, ew0 = 0.0f;
-    {
-        const uint32_t row = tile * ROWS + tid;
-        if (tid < ROWS && tile < ntiles && row < seg.nrows) {
-            if (seg.flags & GEMV_ACCUM) old0 = seg.out[row];
-            if (seg.flags & GEMV_BIAS) bias0 = seg.bias[row];
-            if (seg.flags & GEMV_EMIT) ew0 = p.emit_w[row];
+    // One register set per matrix: the pieces of a unit are requested a stage ahead of their use inside the dot
+    // product (UnitLoader), and the first pieces of the next tile before the current tile's reduction.
+    constexpr int NM = DUAL ? 2 : 1;
+    typename F::Data d, e;                                   // e: second matrix of a gated pair
+    uint16_t dt = 0, et = 0;
+    UnitLoader<T, NM> ld;
+    auto point = [&](uint32_t t) {
+        const size_t off = ((size_t)t * p.ngroups + g) * p.unit_bytes;
+        ld.unit[0] = seg.W + off + lane * 16; ld.tailp[0] = seg.W + off + (size_t)F::PT * 1024 + lane * 2; ld.d[0] = &d; ld.t[0] = &dt;
+        if constexpr (DUAL) { ld.unit[1] = seg.W2 + off + lane * 16; ld.tailp[1] = seg.W2 + off + (size_t)F::PT * 1024 + lane * 2; ld.d[1] = &e; ld.t[1] = &et; }
+    };
+    // Loads are retired in issue order, so everything the epilogue reads from global memory (the value accumulated
+    // into, the bias, the next norm's weight) is requested BEFORE the tile's weights; waiting for it then does not
+    // wait for the weight stream.
+    auto epi_request = [&](uint32_t t, float &old, float &bias, float &ew) {
+        old = 0.0f; bias = 0.0f; ew = 0.0f;
+        const uint32_t row = t * ROWS + tid;
+        if (tid < ROWS && row < seg.nrows) {
+            if (seg.flags & GEMV_ACCUM) old = seg.out[row];
+            if (seg.flags & GEMV_BIAS) bias = seg.bias[row];
+            if (seg.flags & GEMV_EMIT) ew = p.emit_w[row];
         }
-    }
-    {
-        const size_t off = ((size_t)min(tile, ntiles - 1) * p.ngroups + g) * p.unit_bytes;
-        load_unit<T>(seg.W + off, lane, dA, tA);
-        if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, eA, uA);
-    }
+    };
+    uint32_t tile = blk;
+    float old = 0.0f, bias = 0.0f, ew = 0.0f;
+    if (tile < ntiles) { epi_request(tile, old, bias, ew); point(tile); F::lead(ld); }
 #pragma unroll
     for (int i = 0; i < 16; ++i) X.x[i] = valid ? X.x[i] : 0.0f;
 
@@ -201,31 +226,28 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     }
 
     // ---- tiles ------------------------------------------------------------------------------------------
-    // Loads are retired in issue order, so everything the epilogue reads from global memory (the value
-    // accumulated into, the bias) is requested BEFORE the next tile's weights; waiting for it then does
-    // not wait for the weight stream.
-    auto epi_request = [&](uint32_t t, float &old, float &bias, float &ew) {
-        old = 0.0f; bias = 0.0f; ew = 0.0f;
-        const uint32_t row = t * ROWS + tid;
-        if (tid < ROWS && row < seg.nrows) {
-            if (seg.flags & GEMV_ACCUM) old = seg.out[row];
-            if (seg.flags & GEMV_BIAS) bias = seg.bias[row];
-            if (seg.flags & GEMV_EMIT) ew = p.emit_w[row];
-        }
-    };
-    auto consume = [&](const typename F::Data &d, uint16_t dt, const typename F::Data &e, uint16_t et, uint32_t t, bool more,
-                       float old, float bias, float ew) {
-        float v = F::dot(d, dt, X);
+    while (tile < ntiles) {
+        const typename F::Data *dp[NM];
+        uint16_t tails[NM];
+        float o2[NM];
+        dp[0] = &d; tails[0] = dt;
+        if constexpr (DUAL) { dp[1] = &e; tails[1] = et; }
+        F::template dotn<NM>(dp, tails, X, o2, ld);
+        const uint32_t next = tile + step;
+        const float old_c = old, bias_c = bias, ew_c = ew;
+        if (next < ntiles) { epi_request(next, old, bias, ew); point(next); F::lead(ld); }
+        float v = o2[0];
         for (int m = ROWS; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);     // across the KQ super-blocks of the wave
         if (lane < ROWS) partial[wave * 64 + lane] = v;
         if constexpr (DUAL) {
-            float v2 = F::dot(e, et, X);
+            float v2 = o2[1];
             for (int m = ROWS; m < 64; m <<= 1) v2 += __shfl_xor(v2, m, 64);
             if (lane < ROWS) partial[(NW + wave) * 64 + lane] = v2;
         }
         lds_barrier();
+        float ewv = 0.0f;
         if (tid < ROWS) {                                      // epilogue: one thread per output row
-            const uint32_t row = t * ROWS + tid;
+            const uint32_t row = tile * ROWS + tid;
             if (row < seg.nrows) {
                 float o = 0.0f;
                 for (int w = 0; w < NW; ++w) o += partial[w * 64 + tid];
@@ -234,40 +256,21 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
                     for (int w = 0; w < NW; ++w) up += partial[(NW + w) * 64 + tid];
                     o = up * (o / (1.0f + expf(-o)));          // silu.slang:8-26
                 }
-                if (seg.flags & GEMV_BIAS) o += bias;
+                if (seg.flags & GEMV_BIAS) o += bias_c;
                 if (seg.flags & GEMV_GELU) o = gelu_f(o);
-                if (seg.flags & GEMV_ACCUM) o = old + o;
+                if (seg.flags & GEMV_ACCUM) o = old_c + o;
                 seg.out[row] = o;
-                ew *= o;
-                if (seg.flags & GEMV_EMIT) p.emit_out[row] = ew;
+                ewv = ew_c * o;
+                if (seg.flags & GEMV_EMIT) p.emit_out[row] = ewv;
             }
         }
         if ((seg.flags & GEMV_EMIT) && wave == 0) {            // wave-uniform: the sums of 16 consecutive weighted results
-            const float s16 = row16_sum(ew);                   // (ew is 0 in lanes without a row)
-            const uint32_t row = t * ROWS + lane;
+            const float s16 = row16_sum(ewv);                  // (0 in lanes without a row)
+            const uint32_t row = tile * ROWS + lane;
             if (lane < ROWS && (lane & 15) == 0 && row < seg.nrows) p.emit_out[seg.nrows + (row >> 4)] = s16;
         }
-        if (more) lds_barrier();                               // partial[] is reused by the next tile
-    };
-    auto request = [&](typename F::Data &d, uint16_t &dt, typename F::Data &e, uint16_t &et, uint32_t t) {
-        const size_t off = ((size_t)t * p.ngroups + g) * p.unit_bytes;
-        load_unit<T>(seg.W + off, lane, d, dt);
-        if constexpr (DUAL) load_unit<T>(seg.W2 + off, lane, e, et);
-    };
-    if (tile < ntiles) {
-        float old = old0, bias = bias0, ew = ew0;
-        for (;;) {
-            uint32_t next = tile + step;
-            float oldn = 0.0f, biasn = 0.0f, ewn = 0.0f;
-            if (next < ntiles) { epi_request(next, oldn, biasn, ewn); request(dB, tB, eB, uB, next); }
-            consume(dA, tA, eA, uA, tile, next < ntiles, old, bias, ew);
-            if (next >= ntiles) break;
-            tile = next; next = tile + step;
-            if (next < ntiles) { epi_request(next, old, bias, ew); request(dA, tA, eA, uA, next); }
-            consume(dB, tB, eB, uB, tile, next < ntiles, oldn, biasn, ewn);
-            if (next >= ntiles) break;
-            tile = next;
-        }
+        if (next < ntiles) lds_barrier();                      // partial[] is reused by the next tile
+        tile = next;
     }
 }
 
