@@ -82,6 +82,7 @@ template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, 
 // Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product.
 template <int T, int N> struct UnitLoader {
     static constexpr int DEPTH = 1;               // stages requested ahead of the one being multiplied
+    static constexpr int LEAD = 2;                // stages requested before the dot product starts (>= DEPTH)
     using F = Tiled<T>;
     const uint8_t *unit[N];                       // + lane * 16 already applied
     const uint8_t *tailp[N];
@@ -186,6 +187,18 @@ __device__ __forceinline__ void tile_body(const GemvRowtileParams &p, const Gemv
         xs = (cfloat *)slot_bits;
     }
 
+    if constexpr (PREP) {
+        if (norm) {                                           // the sum of squares (for the epilogue), while the first weights travel
+#pragma unroll
+            for (int j = 0; j < XMAX; ++j) {
+                const float4 q = xv[j];
+                const float live = (uint32_t)(j * NT + tid) * 4 < p.ncols ? 1.0f : 0.0f;
+                ss = fmaf(live * q.x, q.x, ss); ss = fmaf(live * q.y, q.y, ss); ss = fmaf(live * q.z, q.z, ss); ss = fmaf(live * q.w, q.w, ss);
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+        }
+    }
     // ---- super-blocks of this wave -------------------------------------------------------------------
     float v = 0.0f, v2 = 0.0f;
     // At most four super-blocks per wave (ncols <= 16384 with 16 waves).  Straight-line code: inside a real loop the
@@ -204,18 +217,6 @@ __device__ __forceinline__ void tile_body(const GemvRowtileParams &p, const Gemv
             if constexpr (DUAL) v2 += o2[1];
             cb += NW;
             if (it < 3 && cb < p.ncb) { point(); F::lead(ld); }
-        }
-    }
-    if constexpr (PREP) {
-        if (norm) {                                           // the sum of squares is only needed by the epilogue
-#pragma unroll
-            for (int j = 0; j < XMAX; ++j) {
-                const float4 q = xv[j];
-                const float live = (uint32_t)(j * NT + tid) * 4 < p.ncols ? 1.0f : 0.0f;
-                ss = fmaf(live * q.x, q.x, ss); ss = fmaf(live * q.y, q.y, ss); ss = fmaf(live * q.z, q.z, ss); ss = fmaf(live * q.w, q.w, ss);
-            }
-            ss = wave_sum(ss);
-            if (lane == 0) red[wave] = ss;
         }
     }
     partial[wave * 64 + lane] = v;

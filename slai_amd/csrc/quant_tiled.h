@@ -158,11 +158,11 @@ SLAI_HD float scale_f16(uint16_t h) {
 
 // The quantised pieces may be fetched while the dot product runs: `L` (a "loader") issues the load of piece P of
 // every matrix with L.piece<P>() (and L.tail() for the 2-byte tail); the dot products call lead() for what the
-// first stages need and ahead<K>() at stage K for what stage K + L::DEPTH needs, so a wave never has more than a
-// few requests waiting to be issued and starts multiplying as soon as its first pieces arrive.  NoLoader is for
+// first L::LEAD (>= L::DEPTH) stages need and ahead<K>() at stage K for what stage K + L::DEPTH needs, so a wave
+// never has more than a few requests waiting to be issued and starts multiplying as soon as its first pieces arrive.  NoLoader is for
 // data that is already in registers.
 struct NoLoader {
-    static constexpr int DEPTH = 8;
+    static constexpr int DEPTH = 8, LEAD = 8;
     template <int P> SLAI_HD void piece() const {}
     SLAI_HD void tail() const {}
 };
@@ -206,11 +206,11 @@ template <> struct Tiled<T_Q4_K> {
     }
     // stage K reads piece 1 + K; the header is piece 0
     template <int P, class L> SLAI_HD static void lead_from(const L &ld) {
-        if constexpr (P <= L::DEPTH && P < PT) { ld.template piece<P>(); lead_from<P + 1>(ld); }
+        if constexpr (P <= L::LEAD && P < PT) { ld.template piece<P>(); lead_from<P + 1>(ld); }
     }
-    template <class L> SLAI_HD static void lead(const L &ld) { lead_from<0>(ld); }
+    template <class L> SLAI_HD static void lead(const L &ld) { lead_from<0>(ld); }      // header + stages 0 .. LEAD-1
     template <int K, class L> SLAI_HD static void ahead(const L &ld) {
-        if constexpr (1 + K + L::DEPTH < PT) ld.template piece<1 + K + L::DEPTH>();
+        if constexpr (1 + K + L::DEPTH < PT && 1 + K + L::DEPTH > L::LEAD) ld.template piece<1 + K + L::DEPTH>();
     }
     template <int K, int N, class X, class S, class L> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, Acc<N> &a, const L &ld) {
         ahead<K>(ld);
@@ -292,12 +292,12 @@ template <> struct Tiled<T_Q6_K> {
         ld.template piece<4 * I + M>(); ld.template piece<4 * I + 2 + M>(); ld.template piece<8 + 2 * I + M>();
     }
     template <int G, class L> SLAI_HD static void lead_from(const L &ld) {
-        if constexpr (2 * G <= L::DEPTH && G < 4) { group<G>(ld); lead_from<G + 1>(ld); }
+        if constexpr (2 * G < L::LEAD && G < 4) { group<G>(ld); lead_from<G + 1>(ld); }
     }
     template <class L> SLAI_HD static void lead(const L &ld) { ld.template piece<12>(); ld.tail(); lead_from<0>(ld); }
     template <int K, class L> SLAI_HD static void ahead(const L &ld) {
-        // group G is first used at stage 2G: led when 2G <= DEPTH, otherwise requested at stage 2G - DEPTH
-        if constexpr (K > 0 && (K + L::DEPTH) % 2 == 0 && (K + L::DEPTH) / 2 < 4) group<(K + L::DEPTH) / 2>(ld);
+        // group G is first used at stage 2G: led when 2G < LEAD, otherwise requested at stage max(2G - DEPTH, 0)
+        if constexpr ((K + L::DEPTH) % 2 == 0 && (K + L::DEPTH) / 2 < 4 && K + L::DEPTH >= L::LEAD) group<(K + L::DEPTH) / 2>(ld);
     }
     template <int K, int N, class X, class S, class L> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc, const L &ld) {
         ahead<K>(ld);
@@ -354,11 +354,11 @@ template <> struct Tiled<T_Q8_0> {
     }
     // stage K reads pieces 2K and 2K+1; the scales are piece 16
     template <int K, class L> SLAI_HD static void lead_from(const L &ld) {
-        if constexpr (K <= L::DEPTH && K < 8) { ld.template piece<2 * K>(); ld.template piece<2 * K + 1>(); lead_from<K + 1>(ld); }
+        if constexpr (K < L::LEAD && K < 8) { ld.template piece<2 * K>(); ld.template piece<2 * K + 1>(); lead_from<K + 1>(ld); }
     }
     template <class L> SLAI_HD static void lead(const L &ld) { ld.template piece<16>(); lead_from<0>(ld); }
     template <int K, class L> SLAI_HD static void ahead(const L &ld) {
-        if constexpr (K + 1 + L::DEPTH < 8) { ld.template piece<2 * (K + 1 + L::DEPTH)>(); ld.template piece<2 * (K + 1 + L::DEPTH) + 1>(); }
+        if constexpr (K + L::DEPTH < 8 && K + L::DEPTH >= L::LEAD) { ld.template piece<2 * (K + L::DEPTH)>(); ld.template piece<2 * (K + L::DEPTH) + 1>(); }
     }
     template <int K, int N, class X, class S, class L> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc, const L &ld) {
         ahead<K>(ld);
