@@ -190,10 +190,25 @@ __global__ void argmax_kernel(const float *v, uint32_t n, int *out_index, Decode
     __shared__ uint32_t bi[16];
     float best = -FLT_MAX;
     uint32_t besti = 0xffffffffu;
-    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
-        const float x = v[i];
-        if (besti == 0xffffffffu || x > best) { best = x; besti = i; }   // ascending i per thread: first max kept
+    // ascending indices per thread, strict comparison: the first maximum is kept (nalgebra `imax`).  16-byte loads,
+    // eight of them in flight per thread.
+    auto take = [&](float x, uint32_t i) { if (besti == 0xffffffffu || x > best) { best = x; besti = i; } };
+    const uint32_t n4 = ((uintptr_t)v % 16 == 0) ? n / 4 : 0;
+    const float4 *v4 = reinterpret_cast<const float4 *>(v);
+    for (uint32_t i = threadIdx.x; i < n4; i += 8 * blockDim.x) {
+        float4 r[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const uint32_t j = i + u * blockDim.x;
+            r[u] = v4[j < n4 ? j : i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const uint32_t j = i + u * blockDim.x;
+            if (j < n4) { take(r[u].x, 4 * j); take(r[u].y, 4 * j + 1); take(r[u].z, 4 * j + 2); take(r[u].w, 4 * j + 3); }
+        }
     }
+    for (uint32_t i = 4 * n4 + threadIdx.x; i < n; i += blockDim.x) take(v[i], i);
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) {
         const float ob = __shfl_xor(best, m, 64);
