@@ -47,7 +47,7 @@ int meta_u32(slai_ctx *ctx, const Gguf &g, const std::string &key, uint32_t *out
 
 // Two matrices over the same input can share a GEMV launch: any formats in 64-row tiles, otherwise one format and layout.
 bool same_launch(const slai_qmat *a, const slai_qmat *b) {
-    if (a->tiled && b->tiled && a->rows_log2 == 6 && b->rows_log2 == 6 && (a->type == b->type || (a->type != T_Q8_0 && b->type != T_Q8_0)))
+    if (a->tiled && b->tiled && a->rows_log2 == 6 && b->rows_log2 == 6 && (a->type == b->type || (a->type != T_Q8_0 && b->type != T_Q8_0 && a->type != T_Q4_0 && b->type != T_Q4_0)))
         return true;
     return a->type == b->type && a->tiled == b->tiled && (!a->tiled || a->rows_log2 == b->rows_log2);
 }

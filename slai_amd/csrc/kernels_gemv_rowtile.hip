@@ -274,7 +274,8 @@ __global__ void __launch_bounds__(1024) gemv_rowtile_kernel(const GemvRowtilePar
         switch (seg.type) {                                    // uniform over the workgroup
         case T_Q4_K: tile_body<T_Q4_K, DUAL, PREP>(p, seg, tile, partial, red); break;
         case T_Q6_K: tile_body<T_Q6_K, DUAL, PREP>(p, seg, tile, partial, red); break;
-        default: break;                                        // the launcher sends Q8_0 only to its own kernel
+        case T_Q5_K: if constexpr (!DUAL) tile_body<T_Q5_K, false, PREP>(p, seg, tile, partial, red); break;
+        default: break;                                        // the launcher sends the other formats to their own kernels
         }
     }
 }
@@ -303,7 +304,7 @@ hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p) {
     uint32_t tiles = 0;
     for (int i = 0; i < p.nseg; ++i) {
         const int t = p.seg[i].type;
-        if (t != T_Q4_K && t != T_Q6_K && t != T_Q8_0) return hipErrorInvalidValue;
+        if (!tiled_supported(t)) return hipErrorInvalidValue;
         p.seg[i].ntiles = (p.seg[i].nrows + 63) / 64;
         tiles += p.seg[i].ntiles;
         if (p.seg[i].flags & GEMV_SILU_GATE) dual = true;
@@ -318,7 +319,8 @@ hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p) {
         if (p.seg[i].type != tt) tt = 0;
     if (tt == 0) {
         for (int i = 0; i < p.nseg; ++i)
-            if (p.seg[i].type == T_Q8_0) return hipErrorInvalidValue;      // mixed launches: Q4_K with Q6_K only
+            if (p.seg[i].type == T_Q8_0 || p.seg[i].type == T_Q4_0 || (dual && p.seg[i].type == T_Q5_K))
+                return hipErrorInvalidValue;                       // mixed launches: the K-quants only
     }
     const int NT = NW * 64;
     hipStream_t st = ctx->stream;
@@ -326,6 +328,8 @@ hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p) {
     case T_Q4_K: return dual ? go<T_Q4_K, true>(p, tiles, NT, smem, st) : go<T_Q4_K, false>(p, tiles, NT, smem, st);
     case T_Q6_K: return dual ? go<T_Q6_K, true>(p, tiles, NT, smem, st) : go<T_Q6_K, false>(p, tiles, NT, smem, st);
     case T_Q8_0: return go<T_Q8_0, false>(p, tiles, NT, smem, st);
+    case T_Q4_0: return dual ? go<T_Q4_0, true>(p, tiles, NT, smem, st) : go<T_Q4_0, false>(p, tiles, NT, smem, st);
+    case T_Q5_K: return dual ? go<T_Q5_K, true>(p, tiles, NT, smem, st) : go<T_Q5_K, false>(p, tiles, NT, smem, st);
     default: return dual ? go<0, true>(p, tiles, NT, smem, st) : go<0, false>(p, tiles, NT, smem, st);
     }
 }

@@ -324,6 +324,8 @@ hipError_t launch_gemv_tiled(slai_ctx *ctx, int type, GemvTiledParams p) {
     case T_Q4_K: return launch_t<T_Q4_K>(ctx, p);
     case T_Q6_K: return launch_t<T_Q6_K>(ctx, p);
     case T_Q8_0: return launch_t<T_Q8_0>(ctx, p);
+    case T_Q4_0: return launch_t<T_Q4_0>(ctx, p);
+    case T_Q5_K: return launch_t<T_Q5_K>(ctx, p);
     default: return hipErrorInvalidValue;
     }
 }

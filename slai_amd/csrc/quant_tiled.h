@@ -16,6 +16,8 @@
 //   Q4_K: cblock = one 144-byte block, pieces = [d,dmin,scales | qs x8]                  PT = 9
 //   Q6_K: cblock = one block, pieces = [ql x8 | qh x4 | scales], tail = d               PT = 13
 //   Q8_0: cblock = eight 34-byte blocks, pieces = [qs x16 | the eight f16 scales]        PT = 17
+//   Q4_0: cblock = eight 18-byte blocks, pieces = [qs x8 (one block each) | the eight f16 scales]  PT = 9
+//   Q5_K: cblock = one 176-byte block, pieces = [d,dmin,scales | qh x2 | qs x8]          PT = 11
 //
 // Activations: a 16-lane DPP row holds the 256 activations of its cblock in 16 registers
 // (register i, lane j <-> x[cb*256 + 16*i + j]); element (i, k) reaches every lane of the row
@@ -39,8 +41,15 @@ struct TiledGeom {
     uint32_t unit_bytes = 0;
 };
 
-SLAI_HD bool tiled_supported(int t) { return t == T_Q4_K || t == T_Q6_K || t == T_Q8_0; }
-SLAI_HD uint32_t tiled_pieces(int t) { return t == T_Q4_K ? 9u : (t == T_Q6_K ? 13u : 17u); }
+SLAI_HD bool tiled_supported(int t) { return t == T_Q4_K || t == T_Q6_K || t == T_Q8_0 || t == T_Q4_0 || t == T_Q5_K; }
+SLAI_HD uint32_t tiled_pieces(int t) {
+    switch (t) {
+    case T_Q4_K: case T_Q4_0: return 9u;
+    case T_Q5_K: return 11u;
+    case T_Q6_K: return 13u;
+    default: return 17u;
+    }
+}
 SLAI_HD uint32_t tiled_tail(int t) { return t == T_Q6_K ? 128u : 0u; }
 
 // force_rows_log2: 0 = choose by column count, else 4, 5 or 6.
@@ -81,6 +90,16 @@ SLAI_HD void tiled_repack_block(const TiledGeom &g, const uint8_t *src, uint8_t 
     case T_Q6_K:   // ql[128] qh[64] scales[16] are pieces 0..12; d is the tail
         for (uint32_t b = 0; b < 210; ++b) dst[tiled_byte_offset(g, row, blk, b)] = src[b];
         break;
+    case T_Q5_K:
+        for (uint32_t b = 0; b < 176; ++b) dst[tiled_byte_offset(g, row, blk, b)] = src[b];
+        break;
+    case T_Q4_0: { // cblock = blocks 8c..8c+7: logical bytes [qs: 16*bi + i][d: 128 + 2*bi]
+        const uint32_t cb = blk / 8, bi = blk % 8;
+        for (uint32_t i = 0; i < 16; ++i) dst[tiled_byte_offset(g, row, cb, 16 * bi + i)] = src[2 + i];
+        dst[tiled_byte_offset(g, row, cb, 128 + 2 * bi)] = src[0];
+        dst[tiled_byte_offset(g, row, cb, 128 + 2 * bi + 1)] = src[1];
+        break;
+    }
     case T_Q8_0: { // cblock = blocks 8c..8c+7: logical bytes [qs: 32*bi + i][d: 256 + 2*bi]
         const uint32_t cb = blk / 8, bi = blk % 8;
         for (uint32_t i = 0; i < 32; ++i) dst[tiled_byte_offset(g, row, cb, 32 * bi + i)] = src[2 + i];
@@ -100,7 +119,7 @@ SLAI_HD float tiled_dequant_elem(const TiledGeom &g, const uint8_t *base, uint32
     const uint32_t cb = col / 256, e = col % 256;
 #define TB(b) base[tiled_byte_offset(g, row, cb, (b))]
     switch (g.type) {
-    case T_Q4_K: {
+    case T_Q4_K: case T_Q5_K: {
         U4 hdr;
         uint8_t hb[16];
         for (int i = 0; i < 16; ++i) hb[i] = TB(i);
@@ -110,9 +129,17 @@ SLAI_HD float tiled_dequant_elem(const TiledGeom &g, const uint8_t *base, uint32
         uint32_t sc, m;
         scale_min_k4(hdr, (int)(jp * 2 + hi), sc, m);
         float d1 = d * (float)sc, m1 = dmin * (float)m;
-        uint8_t byte = TB(16 + jp * 32 + l);
+        uint8_t byte = TB((g.type == T_Q4_K ? 16 : 48) + jp * 32 + l);
         uint32_t q = hi ? (byte >> 4) : (byte & 0xF);
+        if (g.type == T_Q5_K) q += ((TB(16 + l) >> (2 * jp + hi)) & 1u) ? 16u : 0u;
         return d1 * (float)q - m1;
+    }
+    case T_Q4_0: {
+        const uint32_t bi = e / 32, j = e % 32;
+        uint16_t dh = (uint16_t)(TB(128 + 2 * bi) | (TB(128 + 2 * bi + 1) << 8));
+        uint8_t byte = TB(16 * bi + (j & 15));
+        int q = (int)(j < 16 ? (byte & 0xF) : (byte >> 4)) - 8;
+        return (float)q * decode_f16(dh);
     }
     case T_Q6_K: {
         const uint32_t i = e / 128, r = (e % 128) / 32, l = e % 32, is = l / 16;
@@ -381,6 +408,140 @@ template <> struct Tiled<T_Q8_0> {
         const auto st0 = x.template stage<c1(0), c2(0)>();
         stages<0, N>(d, x, st0, acc, ld);
         for (int n = 0; n < N; ++n) out[n] = acc[n];
+    }
+    template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
+        const Data *dp[1] = {&d};
+        float out[1];
+        dotn<1>(dp, &tail, x, out);
+        return out[0];
+    }
+};
+
+template <> struct Tiled<T_Q4_0> {
+    static constexpr int PT = 9;
+    static constexpr bool TAIL = false;
+    struct Data { U4 p[9]; };
+    // stage K = block K of the super-block: its 16 bytes are piece K; low nibbles <-> chunk 2K, high nibbles <-> chunk
+    // 2K+1 (BlockQ4_0, quantization.rs:47-69); the -8 of every value comes back through the activation sums
+    static constexpr int c1(int K) { return 2 * K; }
+    static constexpr int c2(int K) { return 2 * K + 1; }
+    SLAI_HD static float scale_of(const Data &d, int B) {
+        const U4 &s = d.p[8];
+        const uint32_t w = B < 2 ? s.x : (B < 4 ? s.y : (B < 6 ? s.z : s.w));
+        return scale_f16((uint16_t)((B & 1) ? (w >> 16) : (w & 0xffffu)));
+    }
+    template <int K, class L> SLAI_HD static void lead_from(const L &ld) {
+        if constexpr (K < L::LEAD && K < 8) { ld.template piece<K>(); lead_from<K + 1>(ld); }
+    }
+    template <class L> SLAI_HD static void lead(const L &ld) { ld.template piece<8>(); lead_from<0>(ld); }
+    template <int K, class L> SLAI_HD static void ahead(const L &ld) {
+        if constexpr (K + L::DEPTH < 8 && K + L::DEPTH >= L::LEAD) ld.template piece<K + L::DEPTH>();
+    }
+    template <int K, int N, class X, class S> SLAI_HD static void compute(const Data *const *d, const X &x, const S &st, float *acc) {
+        for (int n = 0; n < N; ++n) {
+            const U4 &q = d[n]->p[K];
+            float s = 0.0f, s2 = 0.0f;
+            stage_dot(x, st, and4(q, 0x0F0F0F0Fu), and4(shr4(q, 4), 0x0F0F0F0Fu), s, s2);
+            acc[n] = fmaf(scale_of(*d[n], K), s + s2, acc[n]);
+        }
+    }
+    template <int K, int N, class X, class S, class L> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, float *acc, const L &ld) {
+        ahead<K>(ld);
+        SLAI_SCHED_FENCE();
+        if constexpr (K < 7) {
+            const auto nxt = x.template stage<c1(K + 1), c2(K + 1)>();
+            compute<K, N>(d, x, st, acc);
+            stages<K + 1, N>(d, x, nxt, acc, ld);
+        } else {
+            compute<K, N>(d, x, st, acc);
+        }
+    }
+    template <int N, class X, class L = NoLoader> SLAI_HD static void dotn(const Data *const *d, const uint16_t * /*tail*/, const X &x, float *out, const L &ld = L()) {
+        float acc[N];
+        for (int n = 0; n < N; ++n) {
+            float c = 0.0f;
+            for (int B = 0; B < 8; ++B) c = fmaf(scale_of(*d[n], B), x.sum16(2 * B) + x.sum16(2 * B + 1), c);
+            acc[n] = -8.0f * c;
+        }
+        const auto st0 = x.template stage<c1(0), c2(0)>();
+        stages<0, N>(d, x, st0, acc, ld);
+        for (int n = 0; n < N; ++n) out[n] = acc[n];
+    }
+    template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
+        const Data *dp[1] = {&d};
+        float out[1];
+        dotn<1>(dp, &tail, x, out);
+        return out[0];
+    }
+};
+
+template <> struct Tiled<T_Q5_K> {
+    static constexpr int PT = 11;
+    static constexpr bool TAIL = false;
+    struct Data { U4 p[11]; };
+    // As Q4_K with a fifth bit (BlockQ5K, quantization.rs:249-317): stage K (J = K/2, H = K%2) reads qs piece 3 + K and
+    // the high-bit piece 1 + H (bytes l = 16H..16H+15 of qh); bit 2J of qh[l] belongs to the low nibble (chunk 4J+H),
+    // bit 2J+1 to the high nibble (chunk 4J+2+H)
+    static constexpr int c1(int K) { return 4 * (K / 2) + (K % 2); }
+    static constexpr int c2(int K) { return 4 * (K / 2) + 2 + (K % 2); }
+    template <int N> struct Acc { float accd[N], slo[N], shi[N]; uint32_t sc_lo[N], sc_hi[N]; };
+    template <int K, class L> SLAI_HD static void lead_from(const L &ld) {
+        if constexpr (K < L::LEAD && K < 8) { ld.template piece<3 + K>(); lead_from<K + 1>(ld); }
+    }
+    template <class L> SLAI_HD static void lead(const L &ld) {
+        ld.template piece<0>(); ld.template piece<1>(); ld.template piece<2>();
+        lead_from<0>(ld);
+    }
+    template <int K, class L> SLAI_HD static void ahead(const L &ld) {
+        if constexpr (K + L::DEPTH < 8 && K + L::DEPTH >= L::LEAD) ld.template piece<3 + K + L::DEPTH>();
+    }
+    template <int K, int N, class X, class S> SLAI_HD static void compute(const Data *const *d, const X &x, const S &st, Acc<N> &a) {
+        constexpr int J = K / 2, H = K % 2;
+        for (int n = 0; n < N; ++n) {
+            const U4 &q = d[n]->p[3 + K], &qh = d[n]->p[1 + H];
+            const U4 lo = or4(and4(q, 0x0F0F0F0Fu), shl4(and4(shr4(qh, 2 * J), 0x01010101u), 4));
+            const U4 hi = or4(and4(shr4(q, 4), 0x0F0F0F0Fu), shl4(and4(shr4(qh, 2 * J + 1), 0x01010101u), 4));
+            stage_dot(x, st, lo, hi, a.slo[n], a.shi[n]);
+            if (H == 1) {
+                const uint32_t scw = J < 2 ? a.sc_lo[n] : a.sc_hi[n];
+                constexpr int sh = (J & 1) * 16;
+                a.accd[n] = fmaf((float)((scw >> sh) & 0xffu), a.slo[n], a.accd[n]);
+                a.accd[n] = fmaf((float)((scw >> (sh + 8)) & 0xffu), a.shi[n], a.accd[n]);
+                a.slo[n] = 0.0f; a.shi[n] = 0.0f;
+            }
+        }
+    }
+    template <int K, int N, class X, class S, class L> SLAI_HD static void stages(const Data *const *d, const X &x, const S &st, Acc<N> &a, const L &ld) {
+        ahead<K>(ld);
+        SLAI_SCHED_FENCE();
+        if constexpr (K < 7) {
+            const auto nxt = x.template stage<c1(K + 1), c2(K + 1)>();
+            compute<K, N>(d, x, st, a);
+            stages<K + 1, N>(d, x, nxt, a, ld);
+        } else {
+            compute<K, N>(d, x, st, a);
+        }
+    }
+    template <int N, class X, class L = NoLoader> SLAI_HD static void dotn(const Data *const *d, const uint16_t * /*tail*/, const X &x, float *out, const L &ld = L()) {
+        Acc<N> a;
+        float dd[N], dmin[N], accm[N];
+        for (int n = 0; n < N; ++n) {
+            const U4 &h = d[n]->p[0];
+            dd[n] = scale_f16((uint16_t)(h.x & 0xffffu)); dmin[n] = scale_f16((uint16_t)(h.x >> 16));
+            a.sc_lo[n] = h.y & 0x3f3f3f3fu;
+            a.sc_hi[n] = (h.w & 0x0f0f0f0fu) | (((h.y >> 6) & 0x03030303u) << 4);
+            const uint32_t m_lo = h.z & 0x3f3f3f3fu;
+            const uint32_t m_hi = ((h.w >> 4) & 0x0f0f0f0fu) | (((h.z >> 6) & 0x03030303u) << 4);
+            float am = 0.0f;
+            for (int sb = 0; sb < 8; ++sb) {
+                const uint32_t mw = sb < 4 ? m_lo : m_hi;
+                am = fmaf((float)((mw >> (8 * (sb & 3))) & 0xffu), x.sum16(2 * sb) + x.sum16(2 * sb + 1), am);
+            }
+            accm[n] = am; a.accd[n] = 0.0f; a.slo[n] = 0.0f; a.shi[n] = 0.0f;
+        }
+        const auto st0 = x.template stage<c1(0), c2(0)>();
+        stages<0, N>(d, x, st0, a, ld);
+        for (int n = 0; n < N; ++n) out[n] = dd[n] * a.accd[n] - dmin[n] * accm[n];
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
         const Data *dp[1] = {&d};

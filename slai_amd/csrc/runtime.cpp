@@ -293,7 +293,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who) {
                   (((c.flags[i] ^ c.flags[0]) & GEMV_SILU_GATE) == 0);
     }
     for (int i = 1; i < c.nseg && rowtile; ++i)
-        if (c.m[i]->type != m0->type && (c.m[i]->type == T_Q8_0 || m0->type == T_Q8_0)) rowtile = false;
+        if (c.m[i]->type != m0->type && (c.m[i]->type == T_Q8_0 || m0->type == T_Q8_0 || c.m[i]->type == T_Q4_0 || m0->type == T_Q4_0)) rowtile = false;
     if (c.flags[0] & GEMV_EMIT) {
         if (rowtile || !gemv_can_emit(m0) || !c.emit_w || !c.emit_out) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": this GEMV cannot emit a prepared copy");
     }

@@ -144,6 +144,8 @@ int cc_tiled_gemv(int t, const uint8_t *dev, uint32_t nrows, uint32_t ncols, con
     case T_Q4_K: tiled_gemv_t<T_Q4_K>(g, dev, x, out); break;
     case T_Q6_K: tiled_gemv_t<T_Q6_K>(g, dev, x, out); break;
     case T_Q8_0: tiled_gemv_t<T_Q8_0>(g, dev, x, out); break;
+    case T_Q4_0: tiled_gemv_t<T_Q4_0>(g, dev, x, out); break;
+    case T_Q5_K: tiled_gemv_t<T_Q5_K>(g, dev, x, out); break;
     default: return -1;
     }
     return 0;

@@ -98,7 +98,7 @@ def test_f16_codec_host_side(cc):
     assert np.array_equal(enc, vals.astype(np.float16).view(np.uint16))
 
 
-TILED = [8, 12, 14]
+TILED = [2, 8, 12, 13, 14]
 
 
 @pytest.mark.parametrize("t", TILED)

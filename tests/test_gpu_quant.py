@@ -123,7 +123,7 @@ def test_shape_errors_are_reported_not_fatal(backend):
         o.destroy()
 
 
-@pytest.mark.parametrize("t", [8, 12, 14], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("t", [2, 8, 12, 13, 14], ids=lambda t: NAMES[t])
 def test_fused_op_forms(backend, oracle_lib, t):
     """rms-norm prologue, gate/up + SiLU, and residual-accumulate GEMV against the unfused oracle ops."""
     from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
@@ -145,7 +145,7 @@ def test_fused_op_forms(backend, oracle_lib, t):
     ctxt.ffn_gate_up_silu(ghb, gate, up, gx, gw, 1e-5)
     assert rel_err(ghb.read(), h) < 1e-4
     # residual accumulate: x += Wd . h   (Wd: [dim x hid2])
-    hid2 = 2816 if t == 8 else 3072
+    hid2 = 2816 if t in (2, 8) else 3072
     rawd = synth.normal_quantized(21, t, dim, hid2, 0.05)
     wd = oracle_deq(oracle_lib, t, rawd, dim * hid2).reshape(dim, hid2)
     hv = synth.normal(22, hid2, 1.0)
@@ -164,7 +164,7 @@ LAYOUTS = {"rows": 1, "tile16": 2, "tile64": 3}
 
 
 @pytest.mark.parametrize("layout", list(LAYOUTS), ids=list(LAYOUTS))
-@pytest.mark.parametrize("t", [8, 12, 14], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("t", [2, 8, 12, 13, 14], ids=lambda t: NAMES[t])
 @pytest.mark.parametrize("shape", [(64, 256), (200, 1024), (70, 2816), (1027, 4096)])
 def test_layouts_dequantize_and_gemv(backend, oracle_lib, layout, t, shape):
     """Bit-exact dequantisation and GEMV parity in each device layout (row tails, odd super-block counts)."""
@@ -188,7 +188,7 @@ def test_layouts_dequantize_and_gemv(backend, oracle_lib, layout, t, shape):
         o.destroy()
 
 
-@pytest.mark.parametrize("t", [8, 12, 14], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("t", [2, 8, 12, 13, 14], ids=lambda t: NAMES[t])
 def test_tile64_fused_forms_and_changing_input(backend, oracle_lib, t):
     """64-row tiles: RMSNorm prologue, gate/up + SiLU and residual accumulate; the input vector changes between
     launches (the kernel reads its activations through the scalar cache, which must never serve stale data)."""
@@ -232,7 +232,7 @@ def test_tile64_fused_forms_and_changing_input(backend, oracle_lib, t):
         o.destroy()
 
 
-@pytest.mark.parametrize("t", [8, 12, 14], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("t", [2, 8, 12, 13, 14], ids=lambda t: NAMES[t])
 def test_prepared_activations_chain(backend, oracle_lib, t):
     """x += Wd.h leaving the prepared form of the new x, then RMSNorm + gate/up + SiLU (and a plain RMSNorm GEMV) reading
     it: equal to the unfused oracle sequence; also slai_rms_norm_prepare itself."""
