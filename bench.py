@@ -16,6 +16,7 @@ Also measured here:
     tokens), extrapolated to 32 layers.  A reported baseline, not the target.
 """
 import argparse
+import math
 import ctypes as C
 import json
 import os
@@ -100,6 +101,87 @@ def counter_probe(backend):
                       "gemv_launch_us": round(ms * 1000, 2)}))
 
 
+def graph_time_us(backend, enqueue, n_launches, reps=20):
+    """Mean time per launch of `enqueue` (which issues n_launches kernels) captured in a HIP graph and replayed."""
+    enqueue()                                   # eager once: sizes scratch buffers outside the capture
+    backend.synchronize()
+    backend.graph_begin_capture()
+    enqueue()
+    g = backend.graph_end_capture()
+    backend.graph_launch(g)
+    backend.synchronize()
+    backend.timer_begin()
+    for _ in range(reps):
+        backend.graph_launch(g)
+    ms = backend.timer_end()
+    backend.graph_destroy(g)
+    return ms * 1000.0 / (reps * n_launches)
+
+
+def sweep(backend):
+    """Config 2 (stand-alone GEMV, every block format, two shapes) and the attention kernel at long context (config 5
+    shape): per-launch time and GB/s over rotating weight copies (> 512 MB, so reads come from HBM), launched from a
+    HIP graph so that the host is not in the loop.  Algorithmic bytes = packed W + 4*ncols + 4*nrows."""
+    from slai_amd import _ffi, synth
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
+    ctxt = LlmContext(backend)
+    names = {2: "Q4_0", 12: "Q4_K", 13: "Q5_K", 14: "Q6_K", 8: "Q8_0"}
+    rows = []
+    for (nrows, ncols) in ((4096, 4096), (11008, 4096)):
+        for t in (2, 12, 13, 14, 8):
+            base = synth.normal_quantized(4242 + t, t, nrows, ncols, 0.02)
+            rb = base.size // nrows
+            ncopies = int(math.ceil(560e6 / base.size))
+            x = GpuTensor.vector(backend, synth.normal(7, ncols, 1.0))
+            ones = GpuTensor.vector(backend, np.ones(ncols, np.float32))
+            prep = GpuTensor(backend, ncols + ncols // 16)
+            ctxt.rms_norm_prepare(prep, x, ones)
+            out = GpuTensor(backend, nrows)
+            res = {"format": names[t], "nrows": nrows, "ncols": ncols, "copies": ncopies}
+            algo = base.size + 4 * ncols + 4 * nrows
+            for layout, label in ((_ffi.LAYOUT_TILE16, "tile16"), (_ffi.LAYOUT_TILE64, "tile64")):
+                mats = [GpuQuantMatrix(backend, t, nrows, ncols, np.roll(base.reshape(nrows, rb), i + 1, axis=0), layout=layout)
+                        for i in range(ncopies)]
+                if layout == _ffi.LAYOUT_TILE64:
+                    us = graph_time_us(backend, lambda: [ctxt.matmul_quant_assign_prepared(out, m, prep) for m in mats], ncopies)
+                else:
+                    us = graph_time_us(backend, lambda: [ctxt.matmul_quant_assign(out, m, x) for m in mats], ncopies)
+                res[label + "_us"] = round(us, 2)
+                res[label + "_gbs"] = round(algo / us / 1e3, 1)
+                for m in mats:
+                    m.destroy()
+            res["algorithmic_bytes"] = algo
+            rows.append(res)
+            log("gemv %-5s %5dx%-5d  16-row tiles %6.2f us %7.1f GB/s | 64-row tiles %6.2f us %7.1f GB/s"
+                % (names[t], nrows, ncols, res["tile16_us"], res["tile16_gbs"], res["tile64_us"], res["tile64_gbs"]))
+            for o in (x, ones, prep, out):
+                o.destroy()
+    # attention, config 5 shape: 32 heads x 128, fp16 cache, positions ~4000 of 4096
+    AttnParams = _ffi.AttnParams
+    nh, hs, seq = 32, 128, 4096
+    kv_dim = nh * hs
+    rng = np.random.Generator(np.random.PCG64(5))
+    ncopies = 10                                 # 10 x 2 x 32 MiB of cache > 512 MB
+    caches = [(GpuTensor(backend, kv_dim, seq, _ffi.DT_F16, data=rng.standard_normal((seq, kv_dim), dtype=np.float32).astype(np.float16)),
+               GpuTensor(backend, kv_dim, seq, _ffi.DT_F16, data=rng.standard_normal((seq, kv_dim), dtype=np.float32).astype(np.float16)))
+              for _ in range(ncopies)]
+    gq = GpuTensor.vector(backend, rng.standard_normal(nh * hs, dtype=np.float32))
+    gatt, gxb = GpuTensor(backend, seq, nh), GpuTensor(backend, nh * hs)
+    att = []
+    for pos in (1023, 4047):
+        params = AttnParams(seq, kv_dim, 1, nh, hs, pos, (0, 0))
+        gparams = GpuTensor.scalar(backend, params)
+        us = graph_time_us(backend, lambda: [ctxt.attention(params, gparams, gq, k, v, gatt, gxb) for (k, v) in caches], ncopies)
+        algo = 2 * (pos + 1) * kv_dim * 2
+        att.append({"pos": pos, "us": round(us, 2), "gbs": round(algo / us / 1e3, 1), "algorithmic_bytes": algo})
+        log("attention 32x128 f16, pos %4d: %6.2f us (attention + combine) %7.1f GB/s" % (pos, us, algo / us / 1e3))
+        gparams.destroy()
+    for o in [gq, gatt, gxb] + [t for kv in caches for t in kv]:
+        o.destroy()
+    print(json.dumps({"sweep": "stand-alone GEMV per block format (BASELINE config 2) and long-context attention (config 5 shape)",
+                      "peak_gbs": HBM_PEAK_GBS, "gemv": rows, "attention": att}), flush=True)
+
+
 def cpu_baseline(seed, n_tokens=32):
     """Oracle decode of the same layer shapes at depth 2 and 6, extrapolated linearly to 32 layers."""
     import oracle
@@ -144,15 +226,19 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--probe", action="store_true", help="counter probe: copy kernel + dominant GEMV only")
+    ap.add_argument("--sweep", action="store_true", help="per-format GEMV sweep and long-context attention instead of the decode run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the decode path on ONE GPU (batch-1 decode does not shard usefully); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    if args.probe:
+    if args.probe or args.sweep:
         from slai_amd.runtime import Backend
         backend = Backend(0)
-        counter_probe(backend)
+        if args.probe:
+            counter_probe(backend)
+        else:
+            sweep(backend)
         backend.close()
         return
     K, W = args.steps, max(args.warmup, 1)

@@ -189,6 +189,8 @@ int slai_matmul_quant_add_assign(slai_ctx *ctx, slai_view in_out_x, const slai_q
  * from x; slai_matmul_quant_add_assign_emit is slai_matmul_quant_add_assign that also leaves the form of its result
  * (with the weight of the norm that comes next) for the GEMV after it, so that no separate pass is needed. */
 int slai_rms_norm_prepare(slai_ctx *ctx, slai_view out_prepared, slai_view x, slai_view norm_weight);
+/* out = m . v for v in prepared form built with a weight of all ones (no norm): slai_matmul_quant_assign for TILE64 */
+int slai_matmul_quant_assign_prepared(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view prepared);
 int slai_rms_norm_matmul_quant_assign_prepared(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view prepared,
                                                float eps);
 int slai_ffn_gate_up_silu_prepared(slai_ctx *ctx, slai_view out_hb, const slai_qmat *gate, const slai_qmat *up, slai_view x,

@@ -323,29 +323,26 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     for (int j = 0; j < EPL; ++j) qr[j] = sq[sub * EPL + j];
     const float root = sqrtf((float)HS);
     float lmax = -FLT_MAX;
+    // software pipeline: the keys of the next pass are requested before the current pass is multiplied
     for (uint32_t tb = t0; tb < t1; tb += NT / 4) {           // uniform trip count: the shuffles below need whole waves
         const uint32_t t = tb + tid / 4;
         const bool live = t < t1;
-        const uint32_t tc = live ? t : t1 - 1;
-        const bool use_new = own_new && tc == pos;           // its cache row is being written by this very launch
-        const CT *kp = kc + (size_t)(use_new ? t0 : tc) * a.kv_dim + hoff + sub * EPL;
+        const bool use_new = own_new && live && t == pos;    // its cache row is being written by this very launch
+        typename Vec8<F16>::Raw nxt[EPL / 8] = {};
+        if (tb + NT / 4 < t1) {                               // (uniform) there is a next pass
+            const uint32_t tn = t + NT / 4;
+            const uint32_t tnc = (tn < t1 && !(own_new && tn == pos)) ? tn : t0;
+            const CT *kp = kc + (size_t)tnc * a.kv_dim + hoff + sub * EPL;
+#pragma unroll
+            for (int j = 0; j < EPL / 8; ++j) nxt[j] = Vec8<F16>::load_raw(kp + 8 * j);
+        }
         float kv[EPL];
-        if (tb == t0) {
 #pragma unroll
-            for (int j = 0; j < EPL / 8; ++j) {
-                float tmp[8];
-                Vec8<F16>::decode(kv0[j], tmp);
+        for (int j = 0; j < EPL / 8; ++j) {
+            float tmp[8];
+            Vec8<F16>::decode(kv0[j], tmp);
 #pragma unroll
-                for (int q = 0; q < 8; ++q) kv[8 * j + q] = tmp[q];
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < EPL / 8; ++j) {
-                float tmp[8];
-                Vec8<F16>::load(kp + 8 * j, tmp);
-#pragma unroll
-                for (int q = 0; q < 8; ++q) kv[8 * j + q] = tmp[q];
-            }
+            for (int q = 0; q < 8; ++q) kv[8 * j + q] = tmp[q];
         }
         if (use_new) {
 #pragma unroll
@@ -361,6 +358,8 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
             if (sub == 0) sscore[t - t0] = sc;
             lmax = fmaxf(lmax, sc);
         }
+#pragma unroll
+        for (int j = 0; j < EPL / 8; ++j) kv0[j] = nxt[j];
     }
     lmax = wave_max(lmax);
     if (lane == 0) sred[wave] = lmax;
@@ -386,29 +385,30 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     // ---- weighted sum of values: lane = 8 elements of a position, VG positions per pass, 4 passes in flight --------
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     for (uint32_t tb = t0; tb < t1; tb += 4 * VG) {
-        float vv[4][8], pp[4];
+        typename Vec8<F16>::Raw nxt[4] = {};                  // zero bits decode to 0.0: a skipped pass contributes nothing
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {                         // the next four passes, requested before the current ones are used
+            if (tb + 4 * VG + u * VG >= t1) continue;        // (uniform) no such pass
+            const uint32_t tn = tb + 4 * VG + u * VG + vg;
+            const uint32_t tnc = (tn < t1 && !(own_new && tn == pos)) ? tn : t0;
+            nxt[u] = Vec8<F16>::load_raw(vc + (size_t)tnc * a.kv_dim + hoff + ve);
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const uint32_t t = tb + u * VG + vg;
             const bool live = t < t1;
-            const uint32_t tc = live ? t : t0;
-            const bool use_new = own_new && tc == pos;
-            if (tb == t0) {
-                Vec8<F16>::decode(vv0[u], vv[u]);
-            } else {
-                Vec8<F16>::load(vc + (size_t)(use_new ? t0 : tc) * a.kv_dim + hoff + ve, vv[u]);
-            }
-            pp[u] = live ? sscore[tc - t0] : 0.0f;
-            if (use_new) {
+            const float pw = live ? sscore[t - t0] : 0.0f;
+            float vv[8];
+            Vec8<F16>::decode(vv0[u], vv);
+            if (own_new && live && t == pos) {
 #pragma unroll
-                for (int q = 0; q < 8; ++q) vv[u][q] = sv[ve + q];
+                for (int q = 0; q < 8; ++q) vv[q] = sv[ve + q];
             }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) o[q] = fmaf(pw, vv[q], o[q]);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) o[q] = fmaf(pp[u], vv[u][q], o[q]);
-        }
+        for (int u = 0; u < 4; ++u) vv0[u] = nxt[u];
     }
     // lanes of a wave that hold the same elements: 64 / LPP position groups per wave
 #pragma unroll

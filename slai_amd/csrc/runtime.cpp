@@ -391,7 +391,7 @@ SLAI_EXPORT int slai_matmul_quant_assign(slai_ctx *ctx, slai_view out, const sla
 // that form of (result, emit_w) in emit_out.
 static int fused_gemv(slai_ctx *ctx, const char *fn, slai_view out, const slai_qmat *m, const slai_qmat *m2, slai_view v,
                       const slai_view *norm_weight, float eps, uint32_t flags, const slai_view *prepared = nullptr,
-                      const slai_view *emit_w = nullptr, const slai_view *emit_out = nullptr) {
+                      const slai_view *emit_w = nullptr, const slai_view *emit_out = nullptr, bool plain_prepared = false) {
     if (!ctx || !m) return SLAI_E_ARG;
     VecView vo, vv, vw{nullptr, 0, 1};
     if (!as_vec(out, &vo) || !as_vec(v, &vv)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": bad view");
@@ -409,7 +409,7 @@ static int fused_gemv(slai_ctx *ctx, const char *fn, slai_view out, const slai_q
         if (!as_vec(*prepared, &vp) || vp.stride != 1 || vp.n < m->ncols + m->ncols / 16 || (prepared->offset % 16) != 0)
             return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": prepared activations must be ncols + ncols/16 contiguous floats, 64-byte aligned");
         if (!gemv_is_rowtile(ctx, m)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": prepared activations need a matrix in the TILE64 layout");
-        c.prologue = PRO_RMSNORM; c.eps = eps; c.prepared = vp.p;
+        c.prologue = plain_prepared ? PRO_NONE : PRO_RMSNORM; c.eps = eps; c.prepared = vp.p;
     }
     if (emit_w) {
         VecView ve, vq;
@@ -430,6 +430,12 @@ SLAI_EXPORT int slai_rms_norm_prepare(slai_ctx *ctx, slai_view out_prepared, sla
         return set_error(ctx, SLAI_E_SHAPE, "slai_rms_norm_prepare: need n % 16 == 0 and n + n/16 contiguous output floats, 64-byte aligned");
     SLAI_HIP_TRY(ctx, launch_prepare(ctx->stream, vo.p, vx.p, vw.p, vx.n));
     return SLAI_OK;
+}
+SLAI_EXPORT int slai_matmul_quant_assign_prepared(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view prepared) {
+    if (!m) return SLAI_E_ARG;
+    slai_view v = prepared;                       // the first ncols floats of the prepared form are the vector itself
+    v.size[0] = m->ncols; v.size[1] = v.size[2] = v.size[3] = 1; v.stride[0] = 1;
+    return fused_gemv(ctx, "slai_matmul_quant_assign_prepared", out, m, nullptr, v, nullptr, 0.0f, 0, &prepared, nullptr, nullptr, true);
 }
 SLAI_EXPORT int slai_rms_norm_matmul_quant_assign_prepared(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view prepared,
                                                            float eps) {

@@ -42,6 +42,20 @@ class Backend:
     def synchronize(self):
         self.check(self.L.slai_synchronize(self.h))
 
+    def graph_begin_capture(self):
+        self.check(self.L.slai_graph_begin_capture(self.h))
+
+    def graph_end_capture(self):
+        g = C.c_void_p()
+        self.check(self.L.slai_graph_end_capture(self.h, C.byref(g)))
+        return g
+
+    def graph_launch(self, g):
+        self.check(self.L.slai_graph_launch(self.h, g))
+
+    def graph_destroy(self, g):
+        self.L.slai_graph_destroy(self.h, g)
+
     def timer_begin(self):
         self.check(self.L.slai_timer_begin(self.h))
 
@@ -193,6 +207,9 @@ class LlmContext:
 
     def matmul_quant_add_assign(self, in_out_x, m, v):
         self.backend.check(self.L.slai_matmul_quant_add_assign(self.h, _v(in_out_x), m.h, _v(v)))
+
+    def matmul_quant_assign_prepared(self, out, m, prepared):
+        self.backend.check(self.L.slai_matmul_quant_assign_prepared(self.h, _v(out), m.h, _v(prepared)))
 
     def rms_norm_prepare(self, out_prepared, x, norm_weight):
         self.backend.check(self.L.slai_rms_norm_prepare(self.h, _v(out_prepared), _v(x), _v(norm_weight)))
