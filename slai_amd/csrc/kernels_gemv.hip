@@ -255,7 +255,8 @@ bool gemv_supports(int type, uint32_t ncols) {
     case T_F32: return ncols % 4 == 0 && ncols / 4 <= 4096;
     case T_F16: return ncols % 8 == 0 && ncols / 8 <= 4096;
     case T_Q8_0: return ncols % 32 == 0 && ncols / 16 <= 4096;
-    case T_Q4_0: return ncols % 32 == 0 && ncols / 32 <= 3072;
+    case T_Q4_0: case T_Q4_1: case T_Q5_0: case T_Q5_1: return ncols % 32 == 0 && ncols / 32 <= 3072;
+    case T_Q8_K: return ncols % 256 == 0 && ncols / 16 <= 4096;
     case T_Q4_K: case T_Q5_K: return ncols % 256 == 0 && ncols / 32 <= 3072;
     case T_Q6_K: return ncols % 256 == 0 && ncols / 64 <= 2048;
     default: return false;
@@ -268,6 +269,10 @@ hipError_t launch_gemv(slai_ctx *ctx, int type, GemvParams p) {
     case T_F32: return launch_t<T_F32>(ctx, p);
     case T_F16: return launch_t<T_F16>(ctx, p);
     case T_Q4_0: return launch_t<T_Q4_0>(ctx, p);
+    case T_Q4_1: return launch_t<T_Q4_1>(ctx, p);
+    case T_Q5_0: return launch_t<T_Q5_0>(ctx, p);
+    case T_Q5_1: return launch_t<T_Q5_1>(ctx, p);
+    case T_Q8_K: return launch_t<T_Q8_K>(ctx, p);
     case T_Q8_0: return launch_t<T_Q8_0>(ctx, p);
     case T_Q4_K: return launch_t<T_Q4_K>(ctx, p);
     case T_Q5_K: return launch_t<T_Q5_K>(ctx, p);

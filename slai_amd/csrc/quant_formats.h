@@ -32,19 +32,21 @@
 
 namespace slai {
 
-enum : int { T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14 };
+enum : int { T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q4_1 = 3, T_Q5_0 = 6, T_Q5_1 = 7, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14,
+              T_Q8_K = 15 };
 
 struct U4 { uint32_t x, y, z, w; };
 
 SLAI_HD size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
 
 SLAI_HD int block_elems(int t) {
-    switch (t) { case T_F32: case T_F16: return 1; case T_Q4_0: case T_Q8_0: return 32;
-                 case T_Q4_K: case T_Q5_K: case T_Q6_K: return 256; default: return 0; }
+    switch (t) { case T_F32: case T_F16: return 1; case T_Q4_0: case T_Q4_1: case T_Q5_0: case T_Q5_1: case T_Q8_0: return 32;
+                 case T_Q4_K: case T_Q5_K: case T_Q6_K: case T_Q8_K: return 256; default: return 0; }
 }
 SLAI_HD int block_bytes(int t) {
-    switch (t) { case T_F32: return 4; case T_F16: return 2; case T_Q4_0: return 18; case T_Q8_0: return 34;
-                 case T_Q4_K: return 144; case T_Q5_K: return 176; case T_Q6_K: return 210; default: return 0; }
+    switch (t) { case T_F32: return 4; case T_F16: return 2; case T_Q4_0: return 18; case T_Q4_1: return 20; case T_Q5_0: return 22;
+                 case T_Q5_1: return 24; case T_Q8_0: return 34; case T_Q4_K: return 144; case T_Q5_K: return 176; case T_Q6_K: return 210;
+                 case T_Q8_K: return 292; default: return 0; }
 }
 // bytes of one row in GGUF order / in device order
 SLAI_HD size_t gguf_row_bytes(int t, uint32_t ncols) { return (size_t)(ncols / block_elems(t)) * block_bytes(t); }
@@ -149,6 +151,33 @@ SLAI_HD float dequant_elem(int t, const uint8_t *row, uint32_t nb, uint32_t col)
         int q = (int)(j < 16 ? (byte & 0xF) : (byte >> 4)) - 8;
         return (float)q * d;
     }
+    // Row layout of the remaining 32-element formats: [qs: 16 B per block][qh: 4 B per block (Q5_x)][d or (d, m) per block]
+    case T_Q4_1: {      // BlockQ4_1, quantization.rs:74-99
+        uint32_t b = col / 32, j = col % 32;
+        const uint8_t *dm = row + (size_t)nb * 16 + (size_t)b * 4;
+        float d = decode_f16(ld16(dm)), m = decode_f16(ld16(dm + 2));
+        uint8_t byte = row[(size_t)b * 16 + (j & 15)];
+        uint32_t q = j < 16 ? (byte & 0xFu) : (byte >> 4);
+        return (float)q * d + m;
+    }
+    case T_Q5_0: case T_Q5_1: {     // BlockQ5_0 :103-128, BlockQ5_1 :134-161
+        uint32_t b = col / 32, j = col % 32;
+        uint32_t qh; memcpy(&qh, row + (size_t)nb * 16 + (size_t)b * 4, 4);
+        uint8_t byte = row[(size_t)b * 16 + (j & 15)];
+        uint32_t q = (j < 16 ? (byte & 0xFu) : (uint32_t)(byte >> 4)) | (((qh >> j) & 1u) << 4);
+        if (t == T_Q5_0) {
+            float d = decode_f16(ld16(row + (size_t)nb * 20 + (size_t)b * 2));
+            return (float)((int)q - 16) * d;
+        }
+        const uint8_t *dm = row + (size_t)nb * 20 + (size_t)b * 4;
+        float d = decode_f16(ld16(dm)), m = decode_f16(ld16(dm + 2));
+        return (float)q * d + m;
+    }
+    case T_Q8_K: {      // BlockQ8K, quantization.rs:170-198: [qs: 256 B per block][d: f32 per block]; the block sums are not kept
+        uint32_t b = col / 256;
+        float d; memcpy(&d, row + (size_t)nb * 256 + (size_t)b * 4, 4);
+        return d * (float)(int8_t)row[col];
+    }
     case T_Q4_K: case T_Q5_K: {
         const uint32_t bs = (t == T_Q4_K) ? 144u : 176u;
         const uint8_t *blk = row + (size_t)(col / 256) * bs;
@@ -190,6 +219,24 @@ SLAI_HD void repack_block(int t, const uint8_t *src, uint8_t *dst_row, uint32_t 
     case T_Q4_0:
         for (int i = 0; i < 16; ++i) dst_row[(size_t)b * 16 + i] = src[2 + i];
         dst_row[(size_t)nb * 16 + (size_t)b * 2] = src[0]; dst_row[(size_t)nb * 16 + (size_t)b * 2 + 1] = src[1];
+        break;
+    case T_Q4_1:
+        for (int i = 0; i < 16; ++i) dst_row[(size_t)b * 16 + i] = src[4 + i];
+        for (int i = 0; i < 4; ++i) dst_row[(size_t)nb * 16 + (size_t)b * 4 + i] = src[i];
+        break;
+    case T_Q5_0:
+        for (int i = 0; i < 16; ++i) dst_row[(size_t)b * 16 + i] = src[6 + i];
+        for (int i = 0; i < 4; ++i) dst_row[(size_t)nb * 16 + (size_t)b * 4 + i] = src[2 + i];
+        dst_row[(size_t)nb * 20 + (size_t)b * 2] = src[0]; dst_row[(size_t)nb * 20 + (size_t)b * 2 + 1] = src[1];
+        break;
+    case T_Q5_1:
+        for (int i = 0; i < 16; ++i) dst_row[(size_t)b * 16 + i] = src[8 + i];
+        for (int i = 0; i < 4; ++i) dst_row[(size_t)nb * 16 + (size_t)b * 4 + i] = src[4 + i];
+        for (int i = 0; i < 4; ++i) dst_row[(size_t)nb * 20 + (size_t)b * 4 + i] = src[i];
+        break;
+    case T_Q8_K:
+        for (int i = 0; i < 256; ++i) dst_row[(size_t)b * 256 + i] = src[4 + i];
+        for (int i = 0; i < 4; ++i) dst_row[(size_t)nb * 256 + (size_t)b * 4 + i] = src[i];
         break;
     case T_Q6_K:
         for (int i = 0; i < 128; ++i) dst_row[(size_t)b * 128 + i] = src[i];
@@ -339,6 +386,77 @@ template <> struct Chunk<T_Q4_0> {
         float slo = dot16b(and4(d.qs, 0x0F0F0F0Fu), x);
         float shi = dot16b(and4(shr4(d.qs, 4), 0x0F0F0F0Fu), x + 16);
         return gemv_f16(d.d) * ((slo + shi) - 8.0f * (xs[0] + xs[1]));
+    }
+};
+
+// bit k of the low 4 bits of `nib` into bit 4 of byte k: the fifth bit of four 5-bit values
+SLAI_HD uint32_t spread4(uint32_t nib) { return (((nib & 0xFu) * 0x00204081u) & 0x01010101u) << 4; }
+SLAI_HD U4 high_bits16(uint32_t bits16) {   // bits 0..15 -> 0x10 in bytes 0..15
+    return U4{spread4(bits16), spread4(bits16 >> 4), spread4(bits16 >> 8), spread4(bits16 >> 12)};
+}
+
+template <> struct Chunk<T_Q4_1> {     // one 32-element block: value = q*d + m
+    static constexpr int NRUN = 2, RUNLEN = 16, E = 32;
+    struct Data { U4 qs; uint32_t dm; };
+    SLAI_HD static uint32_t nchunks(uint32_t ncols) { return ncols / 32; }
+    SLAI_HD static uint32_t run_col(uint32_t c, int r) { return c * 32 + r * 16; }
+    SLAI_HD static Data load(const uint8_t *row, uint32_t nb, uint32_t c) {
+        uint32_t dm; memcpy(&dm, row + (size_t)nb * 16 + (size_t)c * 4, 4);
+        return Data{ld128(row + (size_t)c * 16), dm};
+    }
+    SLAI_HD static float dot(const Data &d, uint32_t c, const float *x, const float *xs) {
+        float slo = dot16b(and4(d.qs, 0x0F0F0F0Fu), x);
+        float shi = dot16b(and4(shr4(d.qs, 4), 0x0F0F0F0Fu), x + 16);
+        return gemv_f16((uint16_t)(d.dm & 0xffffu)) * (slo + shi) + gemv_f16((uint16_t)(d.dm >> 16)) * (xs[0] + xs[1]);
+    }
+};
+
+template <> struct Chunk<T_Q5_0> {     // value = (q5 - 16) * d
+    static constexpr int NRUN = 2, RUNLEN = 16, E = 32;
+    struct Data { U4 qs; uint32_t qh; uint16_t d; };
+    SLAI_HD static uint32_t nchunks(uint32_t ncols) { return ncols / 32; }
+    SLAI_HD static uint32_t run_col(uint32_t c, int r) { return c * 32 + r * 16; }
+    SLAI_HD static Data load(const uint8_t *row, uint32_t nb, uint32_t c) {
+        uint32_t qh; memcpy(&qh, row + (size_t)nb * 16 + (size_t)c * 4, 4);
+        return Data{ld128(row + (size_t)c * 16), qh, ld16(row + (size_t)nb * 20 + (size_t)c * 2)};
+    }
+    SLAI_HD static float dot(const Data &d, uint32_t c, const float *x, const float *xs) {
+        float slo = dot16b(or4(and4(d.qs, 0x0F0F0F0Fu), high_bits16(d.qh)), x);
+        float shi = dot16b(or4(and4(shr4(d.qs, 4), 0x0F0F0F0Fu), high_bits16(d.qh >> 16)), x + 16);
+        return gemv_f16(d.d) * ((slo + shi) - 16.0f * (xs[0] + xs[1]));
+    }
+};
+
+template <> struct Chunk<T_Q5_1> {     // value = q5 * d + m
+    static constexpr int NRUN = 2, RUNLEN = 16, E = 32;
+    struct Data { U4 qs; uint32_t qh, dm; };
+    SLAI_HD static uint32_t nchunks(uint32_t ncols) { return ncols / 32; }
+    SLAI_HD static uint32_t run_col(uint32_t c, int r) { return c * 32 + r * 16; }
+    SLAI_HD static Data load(const uint8_t *row, uint32_t nb, uint32_t c) {
+        uint32_t qh, dm;
+        memcpy(&qh, row + (size_t)nb * 16 + (size_t)c * 4, 4);
+        memcpy(&dm, row + (size_t)nb * 20 + (size_t)c * 4, 4);
+        return Data{ld128(row + (size_t)c * 16), qh, dm};
+    }
+    SLAI_HD static float dot(const Data &d, uint32_t c, const float *x, const float *xs) {
+        float slo = dot16b(or4(and4(d.qs, 0x0F0F0F0Fu), high_bits16(d.qh)), x);
+        float shi = dot16b(or4(and4(shr4(d.qs, 4), 0x0F0F0F0Fu), high_bits16(d.qh >> 16)), x + 16);
+        return gemv_f16((uint16_t)(d.dm & 0xffffu)) * (slo + shi) + gemv_f16((uint16_t)(d.dm >> 16)) * (xs[0] + xs[1]);
+    }
+};
+
+template <> struct Chunk<T_Q8_K> {     // 16 of the 256 int8 of a block, f32 scale
+    static constexpr int NRUN = 1, RUNLEN = 16, E = 16;
+    struct Data { U4 qs; float d; };
+    SLAI_HD static uint32_t nchunks(uint32_t ncols) { return ncols / 16; }
+    SLAI_HD static uint32_t run_col(uint32_t c, int r) { return c * 16; }
+    SLAI_HD static Data load(const uint8_t *row, uint32_t nb, uint32_t c) {
+        float d; memcpy(&d, row + (size_t)nb * 256 + (size_t)(c >> 4) * 4, 4);
+        return Data{ld128(row + (size_t)c * 16), d};
+    }
+    SLAI_HD static float dot(const Data &d, uint32_t c, const float *x, const float *xs) {
+        float s = dot16b(xor4(d.qs, 0x80808080u), x);
+        return d.d * (s - 128.0f * xs[0]);
     }
 };
 

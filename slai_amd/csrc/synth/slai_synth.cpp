@@ -1,5 +1,5 @@
 // slai_synth -- synthetic-model support: a deterministic normal generator and
-// fp32 -> GGUF block quantizers (Q8_0, Q4_0, Q4_K, Q5_K, Q6_K, F16).
+// fp32 -> GGUF block quantizers (Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, Q8_K, Q4_K, Q5_K, Q6_K, F16).
 //
 // The reference has no quantizer (crates/slai/src/quantization.rs only dequantizes),
 // so these follow ggml's public `quantize_row_*_ref` algorithms.  They are INPUT
@@ -76,6 +76,74 @@ void quantize_row_q4_0(const float *x, uint8_t *y, size_t k) {
             uint8_t xi1 = (uint8_t)std::min(15, (int)(int8_t)(x1 + 8.5f));
             y[2 + j] = (uint8_t)(xi0 | (xi1 << 4));
         }
+    }
+}
+
+// ---- Q4_1 / Q5_0 / Q5_1 / Q8_K (ggml's quantize_row_*_ref) --------------------
+void quantize_row_q4_1(const float *x, uint8_t *y, size_t k) {
+    for (size_t i = 0; i < k / 32; ++i, y += 20) {
+        float mn = x[i * 32], mx = x[i * 32];
+        for (int j = 1; j < 32; ++j) { mn = std::min(mn, x[i * 32 + j]); mx = std::max(mx, x[i * 32 + j]); }
+        float d = (mx - mn) / 15.0f, id = d ? 1.0f / d : 0.0f;
+        uint16_t dh = f32_to_f16(d), mh = f32_to_f16(mn);
+        std::memcpy(y, &dh, 2); std::memcpy(y + 2, &mh, 2);
+        for (int j = 0; j < 16; ++j) {
+            float x0 = (x[i * 32 + j] - mn) * id, x1 = (x[i * 32 + 16 + j] - mn) * id;
+            uint8_t xi0 = (uint8_t)std::min(15, (int)(int8_t)(x0 + 0.5f)), xi1 = (uint8_t)std::min(15, (int)(int8_t)(x1 + 0.5f));
+            y[4 + j] = (uint8_t)(xi0 | (xi1 << 4));
+        }
+    }
+}
+void quantize_row_q5_0(const float *x, uint8_t *y, size_t k) {
+    for (size_t i = 0; i < k / 32; ++i, y += 22) {
+        float amax = 0.0f, max = 0.0f;
+        for (int j = 0; j < 32; ++j) { float v = x[i * 32 + j]; if (amax < std::fabs(v)) { amax = std::fabs(v); max = v; } }
+        float d = max / -16.0f, id = d ? 1.0f / d : 0.0f;
+        uint16_t dh = f32_to_f16(d); std::memcpy(y, &dh, 2);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; ++j) {
+            float x0 = x[i * 32 + j] * id, x1 = x[i * 32 + 16 + j] * id;
+            uint8_t xi0 = (uint8_t)std::min(31, (int)(int8_t)(x0 + 16.5f)), xi1 = (uint8_t)std::min(31, (int)(int8_t)(x1 + 16.5f));
+            y[6 + j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= (uint32_t)((xi0 & 0x10u) >> 4) << (j + 0);
+            qh |= (uint32_t)((xi1 & 0x10u) >> 4) << (j + 16);
+        }
+        std::memcpy(y + 2, &qh, 4);
+    }
+}
+void quantize_row_q5_1(const float *x, uint8_t *y, size_t k) {
+    for (size_t i = 0; i < k / 32; ++i, y += 24) {
+        float mn = x[i * 32], mx = x[i * 32];
+        for (int j = 1; j < 32; ++j) { mn = std::min(mn, x[i * 32 + j]); mx = std::max(mx, x[i * 32 + j]); }
+        float d = (mx - mn) / 31.0f, id = d ? 1.0f / d : 0.0f;
+        uint16_t dh = f32_to_f16(d), mh = f32_to_f16(mn);
+        std::memcpy(y, &dh, 2); std::memcpy(y + 2, &mh, 2);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; ++j) {
+            float x0 = (x[i * 32 + j] - mn) * id, x1 = (x[i * 32 + 16 + j] - mn) * id;
+            uint8_t xi0 = (uint8_t)(x0 + 0.5f), xi1 = (uint8_t)(x1 + 0.5f);
+            y[8 + j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= (uint32_t)((xi0 & 0x10u) >> 4) << (j + 0);
+            qh |= (uint32_t)((xi1 & 0x10u) >> 4) << (j + 16);
+        }
+        std::memcpy(y + 4, &qh, 4);
+    }
+}
+void quantize_row_q8_k(const float *x, uint8_t *y, size_t k) {
+    for (size_t i = 0; i < k / 256; ++i, y += 292) {
+        float max = 0.0f, amax = 0.0f;
+        for (int j = 0; j < 256; ++j) { float ax = std::fabs(x[i * 256 + j]); if (ax > amax) { amax = ax; max = x[i * 256 + j]; } }
+        int8_t *qs = (int8_t *)(y + 4);
+        int16_t bsums[16];
+        if (!amax) { std::memset(y, 0, 292); continue; }
+        const float iscale = -127.0f / max;
+        for (int j = 0; j < 256; ++j) {
+            int v = (int)std::nearbyintf(iscale * x[i * 256 + j]);
+            qs[j] = (int8_t)std::min(127, v);
+        }
+        for (int j = 0; j < 16; ++j) { int sum = 0; for (int l = 0; l < 16; ++l) sum += qs[j * 16 + l]; bsums[j] = (int16_t)sum; }
+        const float d = 1.0f / iscale;
+        std::memcpy(y, &d, 4); std::memcpy(y + 260, bsums, 32);
     }
 }
 
@@ -281,6 +349,10 @@ size_t row_bytes(int type, size_t ncols) {
     case 0: return ncols * 4;
     case 1: return ncols * 2;
     case 2: return ncols / 32 * 18;
+    case 3: return ncols / 32 * 20;
+    case 6: return ncols / 32 * 22;
+    case 7: return ncols / 32 * 24;
+    case 15: return ncols / 256 * 292;
     case 8: return ncols / 32 * 34;
     case 12: return ncols / 256 * 144;
     case 13: return ncols / 256 * 176;
@@ -295,6 +367,10 @@ void quantize_row(int type, const float *x, uint8_t *y, size_t k) {
     case 0: std::memcpy(y, x, k * 4); break;
     case 1: for (size_t i = 0; i < k; ++i) { uint16_t h = f32_to_f16(x[i]); std::memcpy(y + 2 * i, &h, 2); } break;
     case 2: quantize_row_q4_0(x, y, k); break;
+    case 3: quantize_row_q4_1(x, y, k); break;
+    case 6: quantize_row_q5_0(x, y, k); break;
+    case 7: quantize_row_q5_1(x, y, k); break;
+    case 15: quantize_row_q8_k(x, y, k); break;
     case 8: quantize_row_q8_0(x, y, k); break;
     case 12: quantize_row_q4_k(x, y, k); break;
     case 13: quantize_row_q5_k(x, y, k); break;

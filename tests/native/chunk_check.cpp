@@ -66,6 +66,10 @@ int cc_gemv(int t, const uint8_t *dev, uint32_t nrows, uint32_t ncols, const flo
     case T_F32: gemv_t<T_F32>(dev, nrows, ncols, x, out); break;
     case T_F16: gemv_t<T_F16>(dev, nrows, ncols, x, out); break;
     case T_Q4_0: gemv_t<T_Q4_0>(dev, nrows, ncols, x, out); break;
+    case T_Q4_1: gemv_t<T_Q4_1>(dev, nrows, ncols, x, out); break;
+    case T_Q5_0: gemv_t<T_Q5_0>(dev, nrows, ncols, x, out); break;
+    case T_Q5_1: gemv_t<T_Q5_1>(dev, nrows, ncols, x, out); break;
+    case T_Q8_K: gemv_t<T_Q8_K>(dev, nrows, ncols, x, out); break;
     case T_Q8_0: gemv_t<T_Q8_0>(dev, nrows, ncols, x, out); break;
     case T_Q4_K: gemv_t<T_Q4_K>(dev, nrows, ncols, x, out); break;
     case T_Q5_K: gemv_t<T_Q5_K>(dev, nrows, ncols, x, out); break;
@@ -79,6 +83,10 @@ uint32_t cc_cover(int t, uint32_t ncols) {
     case T_F32: return cover_t<T_F32>(ncols);
     case T_F16: return cover_t<T_F16>(ncols);
     case T_Q4_0: return cover_t<T_Q4_0>(ncols);
+    case T_Q4_1: return cover_t<T_Q4_1>(ncols);
+    case T_Q5_0: return cover_t<T_Q5_0>(ncols);
+    case T_Q5_1: return cover_t<T_Q5_1>(ncols);
+    case T_Q8_K: return cover_t<T_Q8_K>(ncols);
     case T_Q8_0: return cover_t<T_Q8_0>(ncols);
     case T_Q4_K: return cover_t<T_Q4_K>(ncols);
     case T_Q5_K: return cover_t<T_Q5_K>(ncols);

@@ -13,7 +13,7 @@ from slai_amd import synth
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-TYPES = [0, 1, 2, 8, 12, 13, 14]
+TYPES = [0, 1, 2, 3, 6, 7, 8, 12, 13, 14, 15]
 
 
 @pytest.fixture(scope="module")

@@ -86,7 +86,7 @@ def test_llama_kquants_gqa(backend, kv_f16):
     check_llama(backend, data, prompt, 40, kv_f16=kv_f16, check_logit_steps=12)
 
 
-@pytest.mark.parametrize("wtype", [2, 13, 1, 0], ids=["q4_0", "q5_k", "f16", "f32"])
+@pytest.mark.parametrize("wtype", [2, 3, 6, 7, 13, 1, 0], ids=["q4_0", "q4_1", "q5_0", "q5_1", "q5_k", "f16", "f32"])
 def test_llama_other_formats(backend, wtype):
     data = gw.llama_gguf(dim=256, hidden_dim=768, n_layers=2, n_heads=4, n_kv_heads=4, vocab=512, seq_len=32,
                          wtype=wtype, seed=21 + wtype, std=0.08, norm_random=True, with_output=(wtype != 1))

@@ -7,8 +7,8 @@ from helpers import random_blocks, structured_blocks
 from slai_amd import synth
 
 pytestmark = pytest.mark.gpu
-TYPES = [0, 1, 2, 8, 12, 13, 14]
-NAMES = {0: "f32", 1: "f16", 2: "q4_0", 8: "q8_0", 12: "q4_k", 13: "q5_k", 14: "q6_k"}
+TYPES = [0, 1, 2, 3, 6, 7, 8, 12, 13, 14, 15]
+NAMES = {0: "f32", 1: "f16", 2: "q4_0", 3: "q4_1", 6: "q5_0", 7: "q5_1", 8: "q8_0", 12: "q4_k", 13: "q5_k", 14: "q6_k", 15: "q8_k"}
 
 
 def oracle_deq(L, t, raw, n):
