@@ -71,14 +71,6 @@ struct ScalarX {
     __device__ __forceinline__ float sum16(int i) const { return s[i]; }
 };
 
-template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, int lane, typename Tiled<T>::Data &d, uint16_t &tail) {
-    using F = Tiled<T>;
-#pragma unroll
-    for (int p = 0; p < F::PT; ++p) d.p[p] = ld128(unit + (size_t)p * 1024 + lane * 16);
-    if constexpr (F::TAIL) tail = ld16(unit + (size_t)F::PT * 1024 + lane * 2);
-    else tail = 0;
-}
-
 // Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product.
 template <int T, int N> struct UnitLoader {
     static constexpr int DEPTH = 1;               // stages requested ahead of the one being multiplied
@@ -105,8 +97,6 @@ __device__ __forceinline__ void tile_body(const GemvRowtileParams &p, const Gemv
     const int tid = threadIdx.x, lane = tid & 63, NT = blockDim.x, NW = NT >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
-    // both matrices of a gated pair are requested together when their registers fit beside each other
-    constexpr bool BOTH = DUAL && F::PT <= 9;
 
     // ---- requests.  Loads retire in issue order.  With prepared activations nothing before the epilogue needs x, so
     // the weights go first; otherwise x is needed at once (the workgroup stages its copy) and goes first. ----------

@@ -76,14 +76,6 @@ struct DevX {
     __device__ __forceinline__ float sum16(int i) const { return s[i]; }
 };
 
-template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, int lane, typename Tiled<T>::Data &d, uint16_t &tail) {
-    using F = Tiled<T>;
-#pragma unroll
-    for (int p = 0; p < F::PT; ++p) d.p[p] = ld128(unit + (size_t)p * 1024 + lane * 16);
-    if constexpr (F::TAIL) tail = ld16(unit + (size_t)F::PT * 1024 + lane * 2);
-    else tail = 0;
-}
-
 // Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product.
 template <int T, int N> struct UnitLoader {
     static constexpr int DEPTH = 1;               // stages requested ahead of the one being multiplied
