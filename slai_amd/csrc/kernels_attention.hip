@@ -192,8 +192,8 @@ __global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_
 
 // ---- the same computation for head sizes that are multiples of 32, organised around 16-byte loads with many of
 // them in flight: scores with 4 lanes per position (each lane a contiguous quarter of the head), values with one
-// lane per 8 elements and several positions per pass.  NT = 1024 serves one workgroup per head over the whole
-// context (no combine pass; short contexts), NT = 256 the split form.
+// lane per 8 elements and several positions per pass.  NT = 512 serves one workgroup per head over the whole
+// context (no combine pass; short contexts: measured faster than 256 or 1024 threads), NT = 256 the split form.
 template <bool F16> struct Vec8;
 template <> struct Vec8<true> {   // 8 f16 = 16 bytes
     struct Raw { uint4 w; };
@@ -484,8 +484,8 @@ hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
     dim3 grid(a.n_heads, a.n_splits);
     const bool fast = (a.head_size == 64 || a.head_size == 128) && a.kv_dim % 8 == 0;
     if (fast && a.n_splits == 1) {
-        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 1024, 128><<<grid, 1024, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 1024, 128><<<grid, 1024, smem, s>>>(a, max_split_len); }
-        else { if (a.kv_f16) attn_fast_kernel<true, 1024, 64><<<grid, 1024, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 1024, 64><<<grid, 1024, smem, s>>>(a, max_split_len); }
+        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 512, 128><<<grid, 512, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 512, 128><<<grid, 512, smem, s>>>(a, max_split_len); }
+        else { if (a.kv_f16) attn_fast_kernel<true, 512, 64><<<grid, 512, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 512, 64><<<grid, 512, smem, s>>>(a, max_split_len); }
     } else if (fast) {
         if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 256, 128><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 128><<<grid, 256, smem, s>>>(a, max_split_len); }
         else { if (a.kv_f16) attn_fast_kernel<true, 256, 64><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 64><<<grid, 256, smem, s>>>(a, max_split_len); }
