@@ -176,6 +176,8 @@ struct GemvCall {
 bool gemv_can_emit(const slai_qmat *m);
 // True when gemv_call takes the 64-row-tile path for this matrix (and so can use `prepared`).
 bool gemv_is_rowtile(const slai_ctx *ctx, const slai_qmat *m);
+// The same for a SiLU-gated pair launched together (a gated Q8_0 pair needs too many registers there).
+bool gemv_gated_is_rowtile(const slai_ctx *ctx, const slai_qmat *gate, const slai_qmat *up);
 // Returns SLAI_OK or an error code with the message set on ctx.
 int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who);
 // Makes sure the row-tile GEMV's scratch holds `floats` floats (call outside graph capture).

@@ -320,7 +320,10 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
             GemvCall c;
             c.m[0] = wl.attn_output; c.out[0] = x; c.flags[0] = GEMV_ACCUM; c.x = xb;
             prepared = nullptr;
-            if (gemv_can_emit(wl.attn_output) && gemv_is_rowtile(ctx, wl.ffn_gate) && gemv_is_rowtile(ctx, wl.ffn_up)) {
+            const bool gated_launch = wl.ffn_gate->type == wl.ffn_up->type && wl.ffn_gate->tiled == wl.ffn_up->tiled && wl.ffn_gate->rows_log2 == wl.ffn_up->rows_log2;
+            const bool ffn_takes_prepared = gated_launch ? gemv_gated_is_rowtile(ctx, wl.ffn_gate, wl.ffn_up)
+                                                         : (gemv_is_rowtile(ctx, wl.ffn_gate) && gemv_is_rowtile(ctx, wl.ffn_up));
+            if (gemv_can_emit(wl.attn_output) && ffn_takes_prepared) {
                 c.flags[0] |= GEMV_EMIT; c.emit_w = (const float *)wl.ffn_norm.buf->dptr; c.emit_out = xw;
                 prepared = xw;
             }
@@ -577,13 +580,18 @@ int slai_gpt2::load(const slai_gguf *gg) {
             if (c.m->nrows != c.r || c.m->ncols != c.c) return set_error(ctx, SLAI_E_SHAPE, "layer " + std::to_string(l) + ": weight shape does not match the parameters");
         TRY(GpuTensor::matrix(ctx, E, params.n_seq, STORAGE, &w.key_cache, cdt));
         TRY(GpuTensor::matrix(ctx, E, params.n_seq, STORAGE, &w.value_cache, cdt));
-        for (slai_qmat *m : {w.c_attn_attn_w, w.c_attn_proj_w, w.c_mlp_fc_w, w.c_mlp_proj_w}) weight_bytes += m->bytes;
+        for (slai_qmat *m : {w.c_attn_attn_w, w.c_attn_proj_w, w.c_mlp_fc_w, w.c_mlp_proj_w}) {
+            weight_bytes += m->bytes;
+            // activation slots of the 64-row-tile GEMV (one launch per matrix here); must exist before a graph is captured
+            if (gemv_is_rowtile(ctx, m)) TRY(gemv_scratch_reserve(ctx, (size_t)((m->nrows + 63) / 64) * (m->ncols + m->ncols / 16)));
+        }
         weight_bytes += (size_t)(4 * E + 3 * E + E + params.ff_len + E) * 4;
     }
     TRY(f32_vector_from_gguf(ctx, g, "output_norm.weight", true, &ln_f_g));
     TRY(f32_vector_from_gguf(ctx, g, "output_norm.bias", true, &ln_f_b));
     TRY(qmat_from_gguf(ctx, gg, "token_embd.weight", &wte));
     TRY(qmat_from_gguf(ctx, gg, "position_embd.weight", &wpe));
+    if (gemv_is_rowtile(ctx, wte)) TRY(gemv_scratch_reserve(ctx, (size_t)((wte->nrows + 63) / 64) * (wte->ncols + wte->ncols / 16)));
     if (wte->nrows != params.n_vocab || wte->ncols != E || wpe->ncols != E || wpe->nrows < params.n_seq)
         return set_error(ctx, SLAI_E_SHAPE, "embedding shapes do not match the parameters");
     weight_bytes += wte->bytes + 2 * (size_t)E * 4;

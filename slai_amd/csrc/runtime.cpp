@@ -269,6 +269,10 @@ bool gemv_is_rowtile(const slai_ctx *ctx, const slai_qmat *m) {
     return ctx->rowtile_gemv && m && m->tiled && m->rows_log2 == 6 && m->ncb <= 64;
 }
 
+bool gemv_gated_is_rowtile(const slai_ctx *ctx, const slai_qmat *gate, const slai_qmat *up) {
+    return gemv_is_rowtile(ctx, gate) && gemv_is_rowtile(ctx, up) && gate->type == up->type && gate->type != T_Q8_0;
+}
+
 int gemv_scratch_reserve(slai_ctx *ctx, size_t floats) {
     if (floats <= ctx->gemv_scratch_floats) return SLAI_OK;
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "GEMV scratch must be reserved before graph capture");

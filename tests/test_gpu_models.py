@@ -148,3 +148,33 @@ def test_model_load_errors(backend):
     with pytest.raises(SlaiError):
         m.generate([1, 2, 40], 2)                      # token id out of range
     m.destroy(); g.close()
+
+
+def test_generate_works_as_the_first_call_on_a_fresh_context():
+    """The captured decode graph must not need any allocation: everything the kernels use is sized at load time, so
+    `generate` may be the very first thing a context does (no eager forward before it)."""
+    from slai_amd import _ffi, gguf_writer as gw
+    from slai_amd.runtime import Backend, Gguf, Gpt2, Llama2
+    b = Backend(0)
+    try:
+        g = Gguf(gw.gpt2_gguf(n_embd=768, n_layer=2, n_head=12, ff_len=3072, vocab=1000, n_seq=64, wtype=8, seed=5))
+        m = Gpt2(b, g, _ffi.KV_F32)
+        toks, _ = m.generate(np.array([1, 2, 3], np.int32), 8)
+        assert toks.shape == (8,)
+        m.destroy(); g.close()
+        g = Gguf(gw.llama_gguf(dim=512, hidden_dim=1536, n_layers=2, n_heads=8, n_kv_heads=8, vocab=1024, seq_len=64, wtype=12, seed=6))
+        m = Llama2(b, g, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+        toks, _ = m.generate(np.array([1, 2, 3], np.int32), 8)
+        assert toks.shape == (8,)
+        m.destroy(); g.close()
+    finally:
+        b.close()
+
+
+@pytest.mark.parametrize("wtype", [8, 2, 13, 14], ids=["q8_0", "q4_0", "q5_k", "q6_k"])
+def test_llama_tiled_layouts_every_format(backend, wtype):
+    """Widths that take the tiled layouts (multiples of 256) in every format that has them, MHA, fp16 cache: logits and
+    greedy ids against the oracle (a gated Q8_0 pair takes the 16-row-tile kernel, the others the 64-row-tile one)."""
+    data = gw.llama_gguf(dim=512, hidden_dim=1536, n_layers=3, n_heads=8, n_kv_heads=8, vocab=2048, seq_len=128, wtype=wtype, seed=77,
+                         std=0.05, norm_random=True)
+    check_llama(backend, data, [5, 1000, 2047, 9, 77, 3], 40, kv_f16=True, check_logit_steps=12)
