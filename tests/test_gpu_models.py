@@ -178,3 +178,12 @@ def test_llama_tiled_layouts_every_format(backend, wtype):
     data = gw.llama_gguf(dim=512, hidden_dim=1536, n_layers=3, n_heads=8, n_kv_heads=8, vocab=2048, seq_len=128, wtype=wtype, seed=77,
                          std=0.05, norm_random=True)
     check_llama(backend, data, [5, 1000, 2047, 9, 77, 3], 40, kv_f16=True, check_logit_steps=12)
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+def test_llama_context_beyond_1024_uses_split_attention(backend, kv_f16):
+    """A model whose context (1280) is past the single-workgroup attention limit: the decode graph then runs the split
+    (flash-decoding) kernel with its combine pass from position 0 on; ids must match the oracle through position 1100."""
+    data = gw.llama_gguf(dim=256, hidden_dim=512, n_layers=2, n_heads=2, n_kv_heads=2, vocab=512, seq_len=1280, wtype=12, seed=21,
+                         std=0.08, norm_random=True)
+    check_llama(backend, data, [5, 100, 511, 9, 77, 3, 8, 1], 1100, kv_f16=kv_f16, check_logit_steps=6)
