@@ -279,8 +279,9 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
         const Llama2LayerWeights &wl = weights.layers[l];
         // ---- RMSNorm + Q/K/V projections: matrices of one format and layout share a launch
         {
-            const slai_qmat *mats[3] = {wl.attn_q, wl.attn_k, wl.attn_v};
-            float *outs[3] = {q, kcol, vcol};
+            // V first: in the usual mixes it has the widest format, so its workgroups should be dispatched earliest
+            const slai_qmat *mats[3] = {wl.attn_v, wl.attn_k, wl.attn_q};
+            float *outs[3] = {vcol, kcol, q};
             bool done[3] = {false, false, false};
             for (int i = 0; i < 3; ++i) {
                 if (done[i]) continue;
