@@ -190,10 +190,12 @@ __global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_
     }
 }
 
-// ---- the same computation for head sizes that are multiples of 32, organised around 16-byte loads with many of
-// them in flight: scores with 4 lanes per position (each lane a contiguous quarter of the head), values with one
-// lane per 8 elements and several positions per pass.  NT = 512 serves one workgroup per head over the whole
-// context (no combine pass; short contexts: measured faster than 256 or 1024 threads), NT = 256 the split form.
+// ---- the same computation for head sizes 64 and 128, organised around 16-byte loads with many of them in flight:
+// scores with 4 lanes per position (each lane a contiguous quarter of the head), values with one lane per 8
+// elements.  Every wave runs a softmax of its own over the positions it owns (running max and rescaling), so the
+// only workgroup barriers are the one after q is rotated and the one before the waves are merged.  NT = 512 serves
+// one workgroup per head over the whole context (no combine pass; short contexts: measured faster than 256 or 1024
+// threads), NT = 256 the split form.
 template <bool F16> struct Vec8;
 template <> struct Vec8<true> {   // 8 f16 = 16 bytes
     struct Raw { uint4 w; };
@@ -222,7 +224,7 @@ template <> struct Vec8<false> {  // 8 f32 = 32 bytes
     }
 };
 
-template <bool F16, int NT, int HS>
+template <bool F16, int NT, int HS, bool SINGLE>
 __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t max_split_len) {
     touch_kernel_arguments<sizeof(AttnLaunch) + 8>();
     using C = KV<F16>;
@@ -230,23 +232,22 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     constexpr int NW = NT / 64;
     constexpr int EPL = HS / 4;                   // elements per lane in the score phase
     constexpr int LPP = HS / 8;                   // lanes per position in the value phase
-    constexpr int VG = NT / LPP;                  // positions per pass in the value phase
-    extern __shared__ float sscore[];             // [max_split_len]
     __shared__ float sq[HS], sk[HS], sv[HS];
     __shared__ float sred[NW], sred2[NW];
     __shared__ float sacc[NW][LPP * 8];           // per-wave partial outputs (= HS floats per wave)
 
-    const uint32_t h = blockIdx.x, split = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t h = blockIdx.x, split = SINGLE ? 0 : blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t kvh = h / a.kv_mul;
+    // SINGLE: one workgroup per head covers the whole context
     const uint32_t pos = *a.pos_ptr;
     const uint32_t T = pos + 1;
-    const uint32_t chunk = (T + a.n_splits - 1) / a.n_splits;
-    const uint32_t t0 = split * chunk;
-    const uint32_t t1 = min(T, t0 + chunk);
+    const uint32_t chunk = SINGLE ? T : (T + a.n_splits - 1) / a.n_splits;
+    const uint32_t t0 = SINGLE ? 0 : split * chunk;
+    const uint32_t t1 = SINGLE ? T : min(T, t0 + chunk);
     CT *kc = reinterpret_cast<CT *>(a.kcache), *vc = reinterpret_cast<CT *>(a.vcache);
     const size_t hoff = (size_t)kvh * HS;
     const bool fresh = a.knew != nullptr;
-    const bool own_new = fresh && t0 <= pos && pos < t1;
+    const bool own_new = SINGLE ? fresh : (fresh && t0 <= pos && pos < t1);
 
     // ---- requests first: the query pair of this thread (with the fresh key / value and the RoPE frequency), then the
     // first pass of keys and values.  Nothing below depends on anything but the position. ----------------------------
@@ -269,19 +270,25 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
         }
     }
     // ---- the first pass of keys and values is requested before anything else is computed: they depend on nothing
-    // but the position, and their latency then overlaps the q load, the RoPE and the softmax ----------------------
+    // but the position, and their latency then overlaps the q load and the RoPE.  A pass is NT/4 positions; wave w
+    // owns positions 16w..16w+15 of it for both the scores (4 lanes per position) and the values (LPP lanes per
+    // position, PW positions per sub-pass), so nothing but the final merge crosses waves. -----------------------
+    constexpr int PW = 64 / LPP;                  // positions per value sub-pass of a wave
+    constexpr int NU = 16 / PW;                   // value sub-passes per pass
     const uint32_t sub = tid & 3;
-    const uint32_t vg = tid / LPP, ve = (tid % LPP) * 8;
-    typename Vec8<F16>::Raw kv0[EPL / 8], vv0[4];             // kept undecoded: fewer registers while they wait
+    const uint32_t wpos = wave * 16;
+    const uint32_t vgl = lane / LPP, ve = (lane % LPP) * 8;
+    typename Vec8<F16>::Raw kv0[EPL / 8], vv0[NU];            // kept undecoded: fewer registers while they wait
     {
         const uint32_t t = t0 + tid / 4;
-        const uint32_t tc = (t < t1 && !(own_new && t == pos)) ? t : t0;     // the fresh row comes from LDS later
+        // the fresh row comes from LDS later; lanes without a position read a valid address and are masked
+        const uint32_t tc = (t < t1 && !(own_new && t == pos)) ? t : t0;
         const CT *kp = kc + (size_t)tc * a.kv_dim + hoff + sub * EPL;
 #pragma unroll
         for (int j = 0; j < EPL / 8; ++j) kv0[j] = Vec8<F16>::load_raw(kp + 8 * j);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const uint32_t tv = t0 + u * VG + vg;
+        for (int u = 0; u < NU; ++u) {
+            const uint32_t tv = t0 + wpos + u * PW + vgl;
             const uint32_t tvc = (tv < t1 && !(own_new && tv == pos)) ? tv : t0;
             vv0[u] = Vec8<F16>::load_raw(vc + (size_t)tvc * a.kv_dim + hoff + ve);
         }
@@ -317,24 +324,32 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     }
     __syncthreads();
 
-    // ---- scores: 4 lanes per position, each a contiguous quarter of the head ---------------------------------------
+    // ---- per wave, pass by pass: scores of 16 positions, running softmax (max m, sum, rescaled outputs), then the
+    // weighted values of the same 16 positions.  The next pass's keys and values are requested before the current
+    // pass is used. -----------------------------------------------------------------------------------------------
     float qr[EPL];
 #pragma unroll
     for (int j = 0; j < EPL; ++j) qr[j] = sq[sub * EPL + j];
     const float root = sqrtf((float)HS);
-    float lmax = -FLT_MAX;
-    // software pipeline: the keys of the next pass are requested before the current pass is multiplied
+    float m = -FLT_MAX, lsum = 0.0f;
+    float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     for (uint32_t tb = t0; tb < t1; tb += NT / 4) {           // uniform trip count: the shuffles below need whole waves
         const uint32_t t = tb + tid / 4;
         const bool live = t < t1;
         const bool use_new = own_new && live && t == pos;    // its cache row is being written by this very launch
-        typename Vec8<F16>::Raw nxt[EPL / 8] = {};
+        typename Vec8<F16>::Raw nxt[EPL / 8] = {}, nxtv[NU] = {};
         if (tb + NT / 4 < t1) {                               // (uniform) there is a next pass
             const uint32_t tn = t + NT / 4;
             const uint32_t tnc = (tn < t1 && !(own_new && tn == pos)) ? tn : t0;
             const CT *kp = kc + (size_t)tnc * a.kv_dim + hoff + sub * EPL;
 #pragma unroll
             for (int j = 0; j < EPL / 8; ++j) nxt[j] = Vec8<F16>::load_raw(kp + 8 * j);
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                const uint32_t tv = tb + NT / 4 + wpos + u * PW + vgl;
+                const uint32_t tvc = (tv < t1 && !(own_new && tv == pos)) ? tv : t0;
+                nxtv[u] = Vec8<F16>::load_raw(vc + (size_t)tvc * a.kv_dim + hoff + ve);
+            }
         }
         float kv[EPL];
 #pragma unroll
@@ -353,54 +368,21 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
         for (int j = 0; j < EPL; ++j) part = fmaf(qr[j], kv[j], part);
         part += __shfl_xor(part, 1, 64);
         part += __shfl_xor(part, 2, 64);
-        const float sc = part / root;                        // cpu.rs:521 `score /= sqrt(head_size)`
-        if (live) {
-            if (sub == 0) sscore[t - t0] = sc;
-            lmax = fmaxf(lmax, sc);
-        }
+        const float sc = live ? part / root : -FLT_MAX;      // cpu.rs:521 `score /= sqrt(head_size)`
+        const float mn = fmaxf(m, wave_max(sc));
+        const float resc = expf(m - mn);                     // 0 on the first live pass, 1 while nothing was live
+        const float pr = live ? expf(sc - mn) : 0.0f;
+        lsum = fmaf(lsum, resc, sub == 0 ? pr : 0.0f);
 #pragma unroll
-        for (int j = 0; j < EPL / 8; ++j) kv0[j] = nxt[j];
-    }
-    lmax = wave_max(lmax);
-    if (lane == 0) sred[wave] = lmax;
-    __syncthreads();
-    float m = sred[0];
+        for (int q = 0; q < 8; ++q) o[q] *= resc;
+        m = mn;
 #pragma unroll
-    for (int w = 1; w < NW; ++w) m = fmaxf(m, sred[w]);
-
-    // ---- exp and sum (their reduction uses an array of its own: no barrier needed before reusing one) --------------
-    float lsum = 0.0f;
-    for (uint32_t t = t0 + tid; t < t1; t += NT) {
-        const float e = expf(sscore[t - t0] - m);
-        sscore[t - t0] = e;
-        lsum += e;
-    }
-    lsum = wave_sum(lsum);
-    if (lane == 0) sred2[wave] = lsum;
-    __syncthreads();
-    float l = 0.0f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) l += sred2[w];
-
-    // ---- weighted sum of values: lane = 8 elements of a position, VG positions per pass, 4 passes in flight --------
-    float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (uint32_t tb = t0; tb < t1; tb += 4 * VG) {
-        typename Vec8<F16>::Raw nxt[4] = {};                  // zero bits decode to 0.0: a skipped pass contributes nothing
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {                         // the next four passes, requested before the current ones are used
-            if (tb + 4 * VG + u * VG >= t1) continue;        // (uniform) no such pass
-            const uint32_t tn = tb + 4 * VG + u * VG + vg;
-            const uint32_t tnc = (tn < t1 && !(own_new && tn == pos)) ? tn : t0;
-            nxt[u] = Vec8<F16>::load_raw(vc + (size_t)tnc * a.kv_dim + hoff + ve);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const uint32_t t = tb + u * VG + vg;
-            const bool live = t < t1;
-            const float pw = live ? sscore[t - t0] : 0.0f;
+        for (int u = 0; u < NU; ++u) {
+            const uint32_t tv = tb + wpos + u * PW + vgl;
+            const float pw = __shfl(pr, 4 * (u * PW + vgl), 64);      // 0 for positions past the end
             float vv[8];
             Vec8<F16>::decode(vv0[u], vv);
-            if (own_new && live && t == pos) {
+            if (own_new && tv == pos) {
 #pragma unroll
                 for (int q = 0; q < 8; ++q) vv[q] = sv[ve + q];
             }
@@ -408,9 +390,12 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
             for (int q = 0; q < 8; ++q) o[q] = fmaf(pw, vv[q], o[q]);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) vv0[u] = nxt[u];
+        for (int j = 0; j < EPL / 8; ++j) kv0[j] = nxt[j];
+#pragma unroll
+        for (int u = 0; u < NU; ++u) vv0[u] = nxtv[u];
     }
-    // lanes of a wave that hold the same elements: 64 / LPP position groups per wave
+    lsum = wave_sum(lsum);
+    // lanes of a wave that hold the same elements: PW position groups per wave
 #pragma unroll
     for (int msk = LPP; msk < 64; msk <<= 1) {
 #pragma unroll
@@ -420,17 +405,26 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
 #pragma unroll
         for (int q = 0; q < 8; ++q) sacc[wave][lane * 8 + q] = o[q];
     }
+    if (lane == 0) { sred[wave] = m; sred2[wave] = lsum; }
     __syncthreads();
+    // ---- merge the waves: each holds (max, sum, outputs) over its own positions ------------------------------------
     if (tid < HS) {
-        float r = 0.0f;
+        float M = sred[0];
 #pragma unroll
-        for (int w = 0; w < NW; ++w) r += sacc[w][tid];
+        for (int w = 1; w < NW; ++w) M = fmaxf(M, sred[w]);
+        float r = 0.0f, l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float f = expf(sred[w] - M);               // a wave that saw no position has sum 0 and outputs 0
+            r = fmaf(sacc[w][tid], f, r);
+            l = fmaf(sred2[w], f, l);
+        }
         if (a.n_splits == 1) {
             a.out[(size_t)h * HS + tid] = r / l;
         } else {
             float *po = a.scratch + ((size_t)h * a.n_splits + split) * (HS + 2);
             po[tid] = r;
-            if (tid == 0) { po[HS] = (t1 > t0) ? m : -FLT_MAX; po[HS + 1] = (t1 > t0) ? l : 0.0f; }
+            if (tid == 0) { po[HS] = (t1 > t0) ? M : -FLT_MAX; po[HS + 1] = (t1 > t0) ? l : 0.0f; }
         }
     }
 }
@@ -479,16 +473,16 @@ size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n
 hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
     if (a.head_size > MAX_HS || a.head_size % 2 || a.head_size / 2 > ATT_THREADS || a.n_splits == 0 || a.n_splits > 64) return hipErrorInvalidValue;
     const uint32_t max_split_len = (a.seq_len + a.n_splits - 1) / a.n_splits;
-    const size_t smem = (size_t)max_split_len * sizeof(float);
-    if (smem > 48 * 1024) return hipErrorInvalidValue;
     dim3 grid(a.n_heads, a.n_splits);
     const bool fast = (a.head_size == 64 || a.head_size == 128) && a.kv_dim % 8 == 0;
+    const size_t smem = fast ? 0 : (size_t)max_split_len * sizeof(float);   // the general kernel keeps its scores in LDS
+    if (smem > 48 * 1024) return hipErrorInvalidValue;
     if (fast && a.n_splits == 1) {
-        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 512, 128><<<grid, 512, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 512, 128><<<grid, 512, smem, s>>>(a, max_split_len); }
-        else { if (a.kv_f16) attn_fast_kernel<true, 512, 64><<<grid, 512, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 512, 64><<<grid, 512, smem, s>>>(a, max_split_len); }
+        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 512, 128, true><<<grid, 512, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 512, 128, true><<<grid, 512, smem, s>>>(a, max_split_len); }
+        else { if (a.kv_f16) attn_fast_kernel<true, 512, 64, true><<<grid, 512, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 512, 64, true><<<grid, 512, smem, s>>>(a, max_split_len); }
     } else if (fast) {
-        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 256, 128><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 128><<<grid, 256, smem, s>>>(a, max_split_len); }
-        else { if (a.kv_f16) attn_fast_kernel<true, 256, 64><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 64><<<grid, 256, smem, s>>>(a, max_split_len); }
+        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 256, 128, false><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 128, false><<<grid, 256, smem, s>>>(a, max_split_len); }
+        else { if (a.kv_f16) attn_fast_kernel<true, 256, 64, false><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 64, false><<<grid, 256, smem, s>>>(a, max_split_len); }
     } else if (a.kv_f16) attn_kernel<true><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
     else attn_kernel<false><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
     hipError_t e = hipGetLastError();
