@@ -29,11 +29,13 @@ extern "C" {
 #define SLAI_E_PARSE (-5)     /* malformed GGUF */
 #define SLAI_E_MISSING (-6)   /* missing tensor / metadata key */
 #define SLAI_E_STATE (-7)     /* call not valid in the current state */
+#define SLAI_E_IO (-8)        /* a file could not be opened or mapped */
 
 typedef struct slai_ctx slai_ctx;
 typedef struct slai_buffer slai_buffer;
 typedef struct slai_qmat slai_qmat;
 typedef struct slai_graph slai_graph;
+typedef struct slai_tokenizer slai_tokenizer;
 typedef struct slai_gguf slai_gguf;
 typedef struct slai_llama2 slai_llama2;
 typedef struct slai_gpt2 slai_gpt2;
@@ -170,6 +172,14 @@ int slai_attention(slai_ctx *ctx, const slai_attn_params *params, const slai_buf
 /* `Sampler::sample_argmax` (crates/slai/src/models/sampler.rs:55-57; first strict maximum),
  * on the device; out_index is a 1-element I32 buffer. */
 int slai_argmax(slai_ctx *ctx, slai_view logits, slai_buffer *out_index);
+/* `Sampler::sample` (models/sampler.rs:33-53): temperature 0 is the arg-max; otherwise softmax of
+ * logits / temperature, then `sample_mult` (:63-78) when topp is outside (0, 1), else `sample_topp`
+ * (:85-131).  `coin` in [0, 1) is the draw the reference takes from `rand::random()`.  The logits are
+ * not modified.  Sums run in a different order than the reference's sequential ones: the result can
+ * differ from it when `coin` lies within rounding distance of a boundary of the cumulative distribution. */
+int slai_sample(slai_ctx *ctx, slai_view logits, float temperature, float topp, float coin, slai_buffer *out_index);
+/* the draw the device-side loops use at position `pos`: top 24 bits of splitmix64(seed + pos) / 2^24 */
+float slai_sampler_coin(uint64_t seed, uint32_t pos);
 
 /* ---- fused forms of the call sequences `Llama2::launch` issues (no single reference counterpart;
  * each replaces the listed context.rs calls with one kernel, same results up to summation order) */
@@ -214,6 +224,9 @@ void slai_graph_destroy(slai_ctx *ctx, slai_graph *g);
 /* ---- GGUF (crates/slai/src/gguf.rs) -----------------------------------------
  * `Gguf::from_bytes` (gguf.rs:504-524).  The bytes must outlive the handle. */
 int slai_gguf_parse(const void *bytes, size_t len, slai_gguf **out, char *err, size_t err_len);
+/* The same over a read-only mapping of a file, which the handle owns (the headless chat maps the model file and
+ * parses the mapping: crates/slai-chat/src/cli.rs:43-57); tensors are uploaded straight from the mapping. */
+int slai_gguf_open_file(const char *path, slai_gguf **out, char *err, size_t err_len);
 void slai_gguf_free(slai_gguf *g);
 uint32_t slai_gguf_version(const slai_gguf *g);
 uint64_t slai_gguf_tensor_count(const slai_gguf *g);
@@ -228,6 +241,11 @@ int slai_gguf_meta_u32(const slai_gguf *g, const char *key, uint32_t *out);
 int slai_gguf_meta_f32(const slai_gguf *g, const char *key, float *out);
 int slai_gguf_meta_str(const slai_gguf *g, const char *key, const char **out);
 int slai_gguf_meta_array_len(const slai_gguf *g, const char *key, uint64_t *out);
+/* `as_string_array` (gguf.rs:316-322): pointers into the file bytes (not NUL-terminated) and lengths of the first
+ * `capacity` elements; `count` receives the number of elements.  `as_f32_array` (gguf.rs:324-330) likewise. */
+int slai_gguf_meta_array_str(const slai_gguf *g, const char *key, const char **ptrs, uint64_t *lens, uint64_t capacity,
+                             uint64_t *count);
+int slai_gguf_meta_array_f32(const slai_gguf *g, const char *key, float *out, uint64_t capacity, uint64_t *count);
 /* `GgufTensor::to_gpu_matrix` (gguf.rs:357-366) */
 int slai_gguf_tensor_to_qmat(slai_ctx *ctx, const slai_gguf *g, const char *name, slai_qmat **out);
 int slai_gguf_tensor_to_qmat_layout(slai_ctx *ctx, const slai_gguf *g, const char *name, int layout, slai_qmat **out);
@@ -264,6 +282,12 @@ int slai_llama2_forward_logits(slai_llama2 *m, uint32_t pos, uint32_t token, int
 int slai_llama2_generate(slai_llama2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
                          uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms);
 /* Device access for set-up and inspection: layer l's caches ([kv_dim x seq_len]) and the state vectors. */
+/* The same loop with `Sampler::new(vocab, temperature, topp).sample()` run on the device (the chat
+ * samples every generated token with 0.7 / 0.95: crates/slai-chat/src/sampler.rs:100-108), so no
+ * logits cross the bus.  Draws are slai_sampler_coin(seed, pos). */
+int slai_llama2_generate_sampled(slai_llama2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
+                                 uint32_t n_steps, float temperature, float topp, uint64_t seed, int32_t *out_tokens,
+                                 float *elapsed_ms);
 int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache);
 int slai_llama2_logits_buffer(slai_llama2 *m, slai_buffer **logits);
 
@@ -276,6 +300,39 @@ size_t slai_gpt2_weight_bytes(const slai_gpt2 *m);
 int slai_gpt2_forward_logits(slai_gpt2 *m, uint32_t pos, uint32_t token, float *logits_out);
 int slai_gpt2_generate(slai_gpt2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
                        uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms);
+int slai_gpt2_generate_sampled(slai_gpt2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
+                               uint32_t n_steps, float temperature, float topp, uint64_t seed, int32_t *out_tokens,
+                               float *elapsed_ms);
+
+/* ---- Tokenizers (host only) ---------------------------------------------------
+ * `AnyTokenizer` (crates/slai-chat/src/llm.rs:100-164) over `LlamaTokenizer`
+ * (crates/slai/src/models/llama2/tokenizer.rs:23-179) and `Gpt2Tokenizer`
+ * (crates/slai/src/models/gpt2/tokenizer.rs:55-216), read from the GGUF metadata keys
+ * tokenizer.ggml.{model,tokens,scores,merges,bos_token_id,eos_token_id,unknown_token_id}.
+ * Where the reference panics (text that needs a byte-fallback id outside the vocabulary, a
+ * `<...>` span that is not a token, a merge line with fewer than two fields) these return an
+ * error; slai_tokenizer_last_error() gives the message. */
+#define SLAI_TOKENIZER_AUTO (-1)  /* by `tokenizer.ggml.model`, llm.rs:106-118 */
+#define SLAI_TOKENIZER_LLAMA 0
+#define SLAI_TOKENIZER_GPT2 1
+int slai_tokenizer_from_gguf(const slai_gguf *g, int kind, slai_tokenizer **out, char *err, size_t err_len);
+void slai_tokenizer_free(slai_tokenizer *t);
+int slai_tokenizer_kind(const slai_tokenizer *t);
+uint32_t slai_tokenizer_bos(const slai_tokenizer *t);
+uint32_t slai_tokenizer_eos(const slai_tokenizer *t);
+uint32_t slai_tokenizer_unk(const slai_tokenizer *t); /* UINT32_MAX for GPT-2 */
+uint32_t slai_tokenizer_vocab_size(const slai_tokenizer *t);
+const char *slai_tokenizer_last_error(const slai_tokenizer *t);
+/* bytes (not NUL-terminated) and length of a vocabulary entry: `bos_str` / `eos_str` */
+int slai_tokenizer_token_str(const slai_tokenizer *t, uint32_t id, const char **ptr, size_t *len);
+/* `encode(text, bos, eos)`; the GPT-2 tokenizer ignores the two flags (llm.rs:156-162).  `count`
+ * receives the number of ids even when `capacity` is too small (SLAI_E_SHAPE). */
+int slai_tokenizer_encode(slai_tokenizer *t, const char *text, size_t text_len, int bos, int eos, int32_t *out,
+                          size_t capacity, size_t *count);
+/* `decode(prev_token, token)` (llm.rs:149-154) over a run: Llama decodes token i with token i-1
+ * (`prev_token` for the first) as predecessor; GPT-2 decodes the run as a whole. */
+int slai_tokenizer_decode(slai_tokenizer *t, const int32_t *tokens, size_t n, int32_t prev_token, char *out,
+                          size_t capacity, size_t *len);
 
 #ifdef __cplusplus
 }

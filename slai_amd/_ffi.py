@@ -8,7 +8,8 @@ import os
 
 from . import build as _build
 
-OK, E_HIP, E_SHAPE, E_TYPE, E_ARG, E_PARSE, E_MISSING, E_STATE = 0, -1, -2, -3, -4, -5, -6, -7
+OK, E_HIP, E_SHAPE, E_TYPE, E_ARG, E_PARSE, E_MISSING, E_STATE, E_IO = 0, -1, -2, -3, -4, -5, -6, -7, -8
+TOKENIZER_AUTO, TOKENIZER_LLAMA, TOKENIZER_GPT2 = -1, 0, 1
 DT_F32, DT_F16, DT_U8, DT_I32 = 0, 1, 2, 3
 USAGE_MAP_READ, USAGE_COPY_SRC, USAGE_COPY_DST, USAGE_UNIFORM, USAGE_STORAGE = 0x1, 0x4, 0x8, 0x40, 0x80
 ROPE_ORIGINAL, ROPE_NEOX = 0, 1
@@ -91,6 +92,8 @@ SIGNATURES = {
     "slai_softmax_cols": (i32, [vp, View]),
     "slai_attention": (i32, [vp, P(AttnParams), vp, View, View, View, View, View]),
     "slai_argmax": (i32, [vp, View, vp]),
+    "slai_sample": (i32, [vp, View, C.c_float, C.c_float, C.c_float, vp]),
+    "slai_sampler_coin": (C.c_float, [u64, u32]),
     "slai_timer_begin": (i32, [vp]),
     "slai_timer_end": (i32, [vp, P(C.c_float)]),
     "slai_graph_begin_capture": (i32, [vp]),
@@ -109,6 +112,20 @@ SIGNATURES = {
     "slai_gguf_meta_f32": (i32, [vp, C.c_char_p, P(C.c_float)]),
     "slai_gguf_meta_str": (i32, [vp, C.c_char_p, P(C.c_char_p)]),
     "slai_gguf_meta_array_len": (i32, [vp, C.c_char_p, P(u64)]),
+    "slai_gguf_open_file": (i32, [C.c_char_p, P(vp), C.c_char_p, sz]),
+    "slai_gguf_meta_array_str": (i32, [vp, C.c_char_p, P(vp), P(u64), u64, P(u64)]),
+    "slai_gguf_meta_array_f32": (i32, [vp, C.c_char_p, P(C.c_float), u64, P(u64)]),
+    "slai_tokenizer_from_gguf": (i32, [vp, i32, P(vp), C.c_char_p, sz]),
+    "slai_tokenizer_free": (None, [vp]),
+    "slai_tokenizer_kind": (i32, [vp]),
+    "slai_tokenizer_bos": (u32, [vp]),
+    "slai_tokenizer_eos": (u32, [vp]),
+    "slai_tokenizer_unk": (u32, [vp]),
+    "slai_tokenizer_vocab_size": (u32, [vp]),
+    "slai_tokenizer_last_error": (C.c_char_p, [vp]),
+    "slai_tokenizer_token_str": (i32, [vp, u32, P(vp), P(sz)]),
+    "slai_tokenizer_encode": (i32, [vp, C.c_char_p, sz, i32, i32, P(C.c_int32), sz, P(sz)]),
+    "slai_tokenizer_decode": (i32, [vp, P(C.c_int32), sz, C.c_int32, C.c_char_p, sz, P(sz)]),
     "slai_gguf_tensor_to_qmat": (i32, [vp, vp, C.c_char_p, P(vp)]),
     "slai_gguf_tensor_to_qmat_layout": (i32, [vp, vp, C.c_char_p, i32, P(vp)]),
     "slai_llama2_from_gguf": (i32, [vp, vp, i32, i32, P(vp)]),
@@ -117,6 +134,7 @@ SIGNATURES = {
     "slai_llama2_weight_bytes": (sz, [vp]),
     "slai_llama2_forward_logits": (i32, [vp, u32, u32, i32, vp]),
     "slai_llama2_generate": (i32, [vp, vp, u32, u32, u32, vp, P(C.c_float)]),
+    "slai_llama2_generate_sampled": (i32, [vp, vp, u32, u32, u32, C.c_float, C.c_float, u64, vp, P(C.c_float)]),
     "slai_llama2_kv_buffers": (i32, [vp, u32, P(vp), P(vp)]),
     "slai_llama2_logits_buffer": (i32, [vp, P(vp)]),
     "slai_gpt2_from_gguf": (i32, [vp, vp, i32, P(vp)]),
@@ -125,6 +143,7 @@ SIGNATURES = {
     "slai_gpt2_weight_bytes": (sz, [vp]),
     "slai_gpt2_forward_logits": (i32, [vp, u32, u32, vp]),
     "slai_gpt2_generate": (i32, [vp, vp, u32, u32, u32, vp, P(C.c_float)]),
+    "slai_gpt2_generate_sampled": (i32, [vp, vp, u32, u32, u32, C.c_float, C.c_float, u64, vp, P(C.c_float)]),
 }
 
 _lib = None

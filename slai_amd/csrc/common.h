@@ -219,9 +219,17 @@ struct DecodeState {      // lives in device memory; the whole greedy loop runs 
     int token;            // token fed at `pos`
     int n_prompt;         // prompt length (forced tokens while pos < n_prompt-1)
     int step;             // index into out_tokens
+    // sampling (ignored by the greedy kernel): models/sampler.rs `Sampler { temperature, topp }`; the draw for
+    // position pos is the top 24 bits of splitmix64(seed + pos), scaled to [0, 1)
+    float temperature, topp;
+    uint32_t seed_lo, seed_hi;
 };
 hipError_t launch_argmax(hipStream_t s, const float *v, uint32_t n, int *out_index, DecodeState *decode,
                          const int *prompt, int *out_tokens);
+// models/sampler.rs:33-53 `Sampler::sample` with the draw `coin` in [0, 1) given (or, with `decode`, derived from the
+// state's seed and position; temperature and topp then come from the state as well)
+hipError_t launch_sample(hipStream_t s, const float *v, uint32_t n, float temperature, float topp, float coin, int *out_index,
+                         DecodeState *decode, const int *prompt, int *out_tokens);
 
 // ---- attention ---------------------------------------------------------------------
 struct AttnLaunch {

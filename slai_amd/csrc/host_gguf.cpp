@@ -3,8 +3,13 @@
 #include "common.h"
 #include "quant_formats.h"
 
+#include <cerrno>
 #include <cstdio>
 #include <cstring>
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
 namespace slai {
 namespace {
@@ -159,7 +164,32 @@ SLAI_EXPORT int slai_gguf_parse(const void *bytes, size_t len, slai_gguf **out, 
     *out = g;
     return SLAI_OK;
 }
-SLAI_EXPORT void slai_gguf_free(slai_gguf *g) { delete g; }
+// slai-chat/src/cli.rs:43-57: the model file is mapped, not read; tensor data is then uploaded straight from the
+// mapping.  The mapping lives as long as the handle.
+SLAI_EXPORT int slai_gguf_open_file(const char *path, slai_gguf **out, char *err, size_t err_len) {
+    if (!path || !out) return SLAI_E_ARG;
+    *out = nullptr;
+    auto fail = [&](const std::string &m, int rc) { if (err && err_len) snprintf(err, err_len, "%s", m.c_str()); return rc; };
+    const int fd = open(path, O_RDONLY | O_CLOEXEC);
+    if (fd < 0) return fail(std::string("unable to open '") + path + "': " + strerror(errno), SLAI_E_IO);
+    struct stat st;
+    if (fstat(fd, &st) != 0 || st.st_size <= 0) { close(fd); return fail(std::string("'") + path + "' is empty or cannot be examined", SLAI_E_PARSE); }
+    void *map = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    close(fd);
+    if (map == MAP_FAILED) return fail(std::string("unable to map '") + path + "': " + strerror(errno), SLAI_E_IO);
+    slai_gguf *g = new slai_gguf();
+    g->map = map; g->map_len = (size_t)st.st_size;
+    std::string e;
+    const int rc = g->g.parse((const uint8_t *)map, g->map_len, e);
+    if (rc) { slai_gguf_free(g); return fail(e, rc); }
+    *out = g;
+    return SLAI_OK;
+}
+SLAI_EXPORT void slai_gguf_free(slai_gguf *g) {
+    if (!g) return;
+    if (g->map) munmap(g->map, g->map_len);
+    delete g;
+}
 SLAI_EXPORT uint32_t slai_gguf_version(const slai_gguf *g) { return g ? g->g.version : 0; }
 SLAI_EXPORT uint64_t slai_gguf_tensor_count(const slai_gguf *g) { return g ? g->g.tensors.size() : 0; }
 SLAI_EXPORT uint64_t slai_gguf_metadata_count(const slai_gguf *g) { return g ? g->g.metadata.size() : 0; }
@@ -216,6 +246,37 @@ SLAI_EXPORT int slai_gguf_meta_array_len(const slai_gguf *g, const char *key, ui
     if (!v) return SLAI_E_MISSING;
     if (v->type != 9) return SLAI_E_TYPE;
     *out = v->arr_len;
+    return SLAI_OK;
+}
+
+// gguf.rs:316-322 `as_string_array`: pointers into the file bytes (not NUL-terminated) and lengths of the first
+// `capacity` elements; returns the element count through `count`
+SLAI_EXPORT int slai_gguf_meta_array_str(const slai_gguf *g, const char *key, const char **ptrs, uint64_t *lens, uint64_t capacity,
+                                         uint64_t *count) {
+    if (!g || !key) return SLAI_E_ARG;
+    const GgufMetaValue *v = g->g.meta(key);
+    if (!v) return SLAI_E_MISSING;
+    if (v->type != 9 || v->arr_type != 8) return SLAI_E_TYPE;
+    if (count) *count = v->arr_len;
+    size_t off = (size_t)v->arr_offset;
+    for (uint64_t i = 0; i < v->arr_len && i < capacity; ++i) {     // extents were validated by the parse
+        uint64_t n;
+        memcpy(&n, g->g.bytes + off, 8); off += 8;
+        if (ptrs) ptrs[i] = (const char *)g->g.bytes + off;
+        if (lens) lens[i] = n;
+        off += (size_t)n;
+    }
+    return SLAI_OK;
+}
+// gguf.rs:324-330 `as_f32_array`
+SLAI_EXPORT int slai_gguf_meta_array_f32(const slai_gguf *g, const char *key, float *out, uint64_t capacity, uint64_t *count) {
+    if (!g || !key) return SLAI_E_ARG;
+    const GgufMetaValue *v = g->g.meta(key);
+    if (!v) return SLAI_E_MISSING;
+    if (v->type != 9 || v->arr_type != 6) return SLAI_E_TYPE;
+    if (count) *count = v->arr_len;
+    const uint64_t n = v->arr_len < capacity ? v->arr_len : capacity;
+    if (out && n) memcpy(out, g->g.bytes + v->arr_offset, (size_t)n * sizeof(float));
     return SLAI_OK;
 }
 

@@ -50,4 +50,9 @@ struct Gguf {
 
 }  // namespace slai
 
-struct slai_gguf { slai::Gguf g; };
+// `map` is set when the handle owns a read-only mapping of the file (slai_gguf_open_file)
+struct slai_gguf {
+    slai::Gguf g;
+    void *map = nullptr;
+    size_t map_len = 0;
+};

@@ -57,7 +57,8 @@ struct DeviceLoop {           // device-resident state of the greedy loop
     slai_buffer *prompt = nullptr;      // int32[capacity]
     slai_buffer *out_tokens = nullptr;  // int32[capacity]
     uint32_t capacity = 0;
-    slai_graph *graph = nullptr;
+    slai_graph *graph = nullptr;        // one token with the greedy pick
+    slai_graph *graph_sampled = nullptr;  // one token with the temperature / top-p pick
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 };
 int loop_init(slai_ctx *ctx, DeviceLoop &L, uint32_t capacity) {
@@ -71,6 +72,7 @@ int loop_init(slai_ctx *ctx, DeviceLoop &L, uint32_t capacity) {
 }
 void loop_destroy(slai_ctx *ctx, DeviceLoop &L) {
     if (L.graph) slai_graph_destroy(ctx, L.graph);
+    if (L.graph_sampled) slai_graph_destroy(ctx, L.graph_sampled);
     if (L.state) slai_buffer_destroy(ctx, L.state);
     if (L.prompt) slai_buffer_destroy(ctx, L.prompt);
     if (L.out_tokens) slai_buffer_destroy(ctx, L.out_tokens);
@@ -122,7 +124,7 @@ struct slai_llama2 {
 
     int load(const slai_gguf *g);
     int launch(LlmContext &ctxt, const slai_attn_params &attn_params, uint32_t pos);   // transformer.rs:316-381
-    int enqueue_fused(bool with_sampler);
+    int enqueue_fused(int sampler);   // 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state
 };
 
 // models/llama2/cpu.rs:79-109
@@ -264,7 +266,7 @@ int slai_llama2::launch(LlmContext &ctxt, const slai_attn_params &attn_params, u
 // in device memory, so the sequence can be captured once and replayed for every token:
 //   embedding-row gather | per layer: [RMSNorm+QKV GEMV] [RoPE+cache write+attention] [Wo GEMV+residual]
 //   [RMSNorm+gate/up GEMV+SiLU] [down GEMV+residual] | [RMSNorm+logits GEMV] [argmax + loop state]
-int slai_llama2::enqueue_fused(bool with_sampler) {
+int slai_llama2::enqueue_fused(int sampler) {
     Llama2State &s = state;
     DecodeState *ds = (DecodeState *)loop.state->dptr;
     float *x = (float *)s.x.buf->dptr, *xb = (float *)s.xb.buf->dptr, *hb = (float *)s.hb.buf->dptr, *hb2 = (float *)s.hb2.buf->dptr;
@@ -377,8 +379,11 @@ int slai_llama2::enqueue_fused(bool with_sampler) {
         c.prepared = prepared;
         TRY(gemv_call(ctx, c, "llama2 output"));
     }
-    if (with_sampler)
+    if (sampler == 1)
         SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, nullptr, ds,
+                                        (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
+    else if (sampler == 2)
+        SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, 0.0f, 0.0f, 0.0f, nullptr, ds,
                                         (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
     return SLAI_OK;
 }
@@ -459,37 +464,43 @@ SLAI_EXPORT int slai_llama2_forward_logits(slai_llama2 *m, uint32_t pos, uint32_
     return SLAI_OK;
 }
 
+// `sampling`: null for the greedy loop, else temperature / top-p / seed of the device sampler
+struct SamplingParams { float temperature, topp; uint64_t seed; };
 template <class Model>
 static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_len, uint32_t vocab, const int32_t *prompt, uint32_t n_prompt,
-                         uint32_t start_pos, uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms) {
+                         uint32_t start_pos, uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms, const SamplingParams *sampling = nullptr) {
+    if (sampling && !(sampling->temperature >= 0.0f)) return set_error(ctx, SLAI_E_ARG, "generate: the temperature must not be negative");
+    const int mode = sampling ? 2 : 1;
     if (!prompt || !out_tokens || n_prompt == 0 || start_pos >= n_prompt) return set_error(ctx, SLAI_E_ARG, "generate: bad prompt / start position");
     if (n_steps == 0) return SLAI_OK;
     if (start_pos + n_steps > seq_len) return set_error(ctx, SLAI_E_SHAPE, "generate: would run past the context length");
     if (n_prompt > L.capacity || n_steps > L.capacity) return set_error(ctx, SLAI_E_SHAPE, "generate: prompt longer than the context length");
     for (uint32_t i = 0; i < n_prompt; ++i)
         if (prompt[i] < 0 || (uint32_t)prompt[i] >= vocab) return set_error(ctx, SLAI_E_ARG, "generate: prompt token out of range");
-    DecodeState ds{(int)start_pos, prompt[start_pos], (int)n_prompt, 0};     // chat_llama2.rs:105
+    DecodeState ds{(int)start_pos, prompt[start_pos], (int)n_prompt, 0, 0.0f, 0.0f, 0, 0};     // chat_llama2.rs:105
+    if (sampling) { ds.temperature = sampling->temperature; ds.topp = sampling->topp; ds.seed_lo = (uint32_t)sampling->seed; ds.seed_hi = (uint32_t)(sampling->seed >> 32); }
     TRY(slai_write_buffer(ctx, L.state, 0, &ds, sizeof ds));
     TRY(slai_write_buffer(ctx, L.prompt, 0, prompt, (size_t)n_prompt * 4));
     if (!ctx->use_graph) {
         SLAI_HIP_TRY(ctx, hipEventRecord(L.ev0, ctx->stream));
-        for (uint32_t i = 0; i < n_steps; ++i) TRY(m->enqueue_fused(true));
+        for (uint32_t i = 0; i < n_steps; ++i) TRY(m->enqueue_fused(mode));
         SLAI_HIP_TRY(ctx, hipEventRecord(L.ev1, ctx->stream));
         TRY(slai_synchronize(ctx));
         if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, L.ev0, L.ev1));
         return slai_read_buffer(ctx, L.out_tokens, 0, out_tokens, (size_t)n_steps * 4);
     }
-    if (!L.graph) {
+    slai_graph *&graph = sampling ? L.graph_sampled : L.graph;
+    if (!graph) {
         TRY(slai_graph_begin_capture(ctx));
-        int rc = m->enqueue_fused(true);
+        int rc = m->enqueue_fused(mode);
         slai_graph *g = nullptr;
         int rc2 = slai_graph_end_capture(ctx, &g);
         if (rc) { if (g) slai_graph_destroy(ctx, g); return rc; }
         if (rc2) return rc2;
-        L.graph = g;
+        graph = g;
     }
     SLAI_HIP_TRY(ctx, hipEventRecord(L.ev0, ctx->stream));
-    for (uint32_t i = 0; i < n_steps; ++i) TRY(slai_graph_launch(ctx, L.graph));       // chat_llama2.rs:109 loop
+    for (uint32_t i = 0; i < n_steps; ++i) TRY(slai_graph_launch(ctx, graph));         // chat_llama2.rs:109 loop
     SLAI_HIP_TRY(ctx, hipEventRecord(L.ev1, ctx->stream));
     TRY(slai_synchronize(ctx));
     if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, L.ev0, L.ev1));
@@ -500,6 +511,16 @@ SLAI_EXPORT int slai_llama2_generate(slai_llama2 *m, const int32_t *prompt, uint
                                      int32_t *out_tokens, float *elapsed_ms) {
     if (!m) return SLAI_E_ARG;
     return generate_impl(m, m->ctx, m->loop, m->config.seq_len, m->config.vocab_size, prompt, n_prompt, start_pos, n_steps, out_tokens, elapsed_ms);
+}
+
+// The same loop with `Sampler::new(vocab, temperature, topp).sample(logits)` (models/sampler.rs:33-53; the chat uses
+// 0.7 / 0.95, slai-chat/src/sampler.rs:107) on the device instead of a logits readback per token.  The draw for
+// position pos is slai_sampler_coin(seed, pos).
+SLAI_EXPORT int slai_llama2_generate_sampled(slai_llama2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos, uint32_t n_steps,
+                                             float temperature, float topp, uint64_t seed, int32_t *out_tokens, float *elapsed_ms) {
+    if (!m) return SLAI_E_ARG;
+    const SamplingParams sp{temperature, topp, seed};
+    return generate_impl(m, m->ctx, m->loop, m->config.seq_len, m->config.vocab_size, prompt, n_prompt, start_pos, n_steps, out_tokens, elapsed_ms, &sp);
 }
 
 SLAI_EXPORT int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache) {
@@ -539,7 +560,7 @@ struct slai_gpt2 {
     uint32_t attn_splits = 1;
 
     int load(const slai_gguf *g);
-    int enqueue_fused(bool with_sampler);
+    int enqueue_fused(int sampler);   // 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state
 };
 
 int slai_gpt2::load(const slai_gguf *gg) {
@@ -608,7 +629,7 @@ int slai_gpt2::load(const slai_gguf *gg) {
 }
 
 // gpt2/cpu.rs:224-383 as fused kernels (LayerNorm eps 1e-5: ops/layernorm.rs:105)
-int slai_gpt2::enqueue_fused(bool with_sampler) {
+int slai_gpt2::enqueue_fused(int sampler) {
     DecodeState *ds = (DecodeState *)loop.state->dptr;
     const uint32_t E = params.n_embd;
     float *x = (float *)layer_input.buf->dptr, *att_out = (float *)curr_768.buf->dptr, *qkv = (float *)curr_2304.buf->dptr,
@@ -659,8 +680,11 @@ int slai_gpt2::enqueue_fused(bool with_sampler) {
         c.prologue = PRO_LAYERNORM; c.norm_w = (const float *)ln_f_g.buf->dptr; c.norm_b = (const float *)ln_f_b.buf->dptr; c.eps = eps;
         TRY(gemv_call(ctx, c, "gpt2 lm_head"));
     }
-    if (with_sampler)
+    if (sampler == 1)
         SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, logits, params.n_vocab, nullptr, ds, (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
+    else if (sampler == 2)
+        SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, logits, params.n_vocab, 0.0f, 0.0f, 0.0f, nullptr, ds, (const int *)loop.prompt->dptr,
+                                        (int *)loop.out_tokens->dptr));
     return SLAI_OK;
 }
 
@@ -714,4 +738,10 @@ SLAI_EXPORT int slai_gpt2_generate(slai_gpt2 *m, const int32_t *prompt, uint32_t
                                    int32_t *out_tokens, float *elapsed_ms) {
     if (!m) return SLAI_E_ARG;
     return generate_impl(m, m->ctx, m->loop, m->params.n_seq, m->params.n_vocab, prompt, n_prompt, start_pos, n_steps, out_tokens, elapsed_ms);
+}
+SLAI_EXPORT int slai_gpt2_generate_sampled(slai_gpt2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos, uint32_t n_steps,
+                                           float temperature, float topp, uint64_t seed, int32_t *out_tokens, float *elapsed_ms) {
+    if (!m) return SLAI_E_ARG;
+    const SamplingParams sp{temperature, topp, seed};
+    return generate_impl(m, m->ctx, m->loop, m->params.n_seq, m->params.n_vocab, prompt, n_prompt, start_pos, n_steps, out_tokens, elapsed_ms, &sp);
 }

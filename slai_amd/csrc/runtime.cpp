@@ -608,6 +608,26 @@ SLAI_EXPORT int slai_argmax(slai_ctx *ctx, slai_view logits, slai_buffer *out_in
     return SLAI_OK;
 }
 
+// models/sampler.rs:33-53 `Sampler::sample`, with the draw passed in.  The logits are left as they are (the reference
+// overwrites them with the probabilities).
+SLAI_EXPORT int slai_sample(slai_ctx *ctx, slai_view logits, float temperature, float topp, float coin, slai_buffer *out_index) {
+    if (!ctx || !out_index) return SLAI_E_ARG;
+    NEED_VEC(logits, "logits", vl);
+    if (vl.stride != 1 || out_index->dtype != SLAI_DT_I32 || out_index->bytes < 4) return set_error(ctx, SLAI_E_SHAPE, "slai_sample: contiguous logits and an I32 output are required");
+    if (!(temperature >= 0.0f) || !(coin >= 0.0f && coin < 1.0f)) return set_error(ctx, SLAI_E_ARG, "slai_sample: temperature must be >= 0 and the draw in [0, 1)");
+    SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, vl.p, vl.n, temperature, topp, coin, (int *)out_index->dptr, nullptr, nullptr, nullptr));
+    return SLAI_OK;
+}
+// The draw the device loop uses at position `pos`: the top 24 bits of splitmix64(seed + pos), scaled to [0, 1)
+SLAI_EXPORT float slai_sampler_coin(uint64_t seed, uint32_t pos) {
+    uint64_t x = seed + (uint64_t)pos;
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    x ^= x >> 31;
+    return (float)(x >> 40) * (1.0f / 16777216.0f);
+}
+
 // ---- timing ---------------------------------------------------------------------------
 SLAI_EXPORT int slai_timer_begin(slai_ctx *ctx) {
     if (!ctx) return SLAI_E_ARG;

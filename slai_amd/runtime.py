@@ -258,6 +258,15 @@ class LlmContext:
     def argmax(self, logits, out_index):
         self.backend.check(self.L.slai_argmax(self.h, _v(logits), out_index.h))
 
+    def sample(self, logits, temperature, topp, coin, out_index):
+        """models/sampler.rs:33-53 ``Sampler::sample`` with the draw `coin` in [0, 1) passed in."""
+        self.backend.check(self.L.slai_sample(self.h, _v(logits), temperature, topp, coin, out_index.h))
+
+
+def sampler_coin(seed, pos):
+    """The draw the device-side sampling loops use at position `pos`."""
+    return float(_ffi.lib().slai_sampler_coin(seed, pos))
+
 
 class Gguf:
     """crates/slai/src/gguf.rs ``Gguf::from_bytes``; keeps the bytes alive for the handle."""
@@ -272,9 +281,41 @@ class Gguf:
             raise SlaiError(rc, err.value.decode(errors="replace"))
         self.h = h
 
+    @classmethod
+    def open(cls, path):
+        """Maps the file read-only (crates/slai-chat/src/cli.rs:43-57); the handle owns the mapping."""
+        self = cls.__new__(cls)
+        self.L = _ffi.lib()
+        self.data = None
+        h = C.c_void_p()
+        err = C.create_string_buffer(512)
+        rc = self.L.slai_gguf_open_file(str(path).encode(), C.byref(h), err, 512)
+        if rc:
+            raise SlaiError(rc, err.value.decode(errors="replace"))
+        self.h = h
+        return self
+
     @property
     def version(self):
         return self.L.slai_gguf_version(self.h)
+
+    def meta_array_str(self, key):
+        """gguf.rs:316-322 ``as_string_array`` (as bytes objects)."""
+        n = self.meta_array_len(key)
+        ptrs, lens, cnt = (C.c_void_p * max(n, 1))(), (C.c_uint64 * max(n, 1))(), C.c_uint64()
+        rc = self.L.slai_gguf_meta_array_str(self.h, key.encode(), ptrs, lens, n, C.byref(cnt))
+        if rc:
+            raise SlaiError(rc, "metadata string array '%s'" % key)
+        return [C.string_at(ptrs[i], lens[i]) if lens[i] else b"" for i in range(n)]
+
+    def meta_array_f32(self, key):
+        """gguf.rs:324-330 ``as_f32_array``."""
+        n = self.meta_array_len(key)
+        out, cnt = np.zeros(max(n, 1), dtype=np.float32), C.c_uint64()
+        rc = self.L.slai_gguf_meta_array_f32(self.h, key.encode(), out.ctypes.data_as(C.POINTER(C.c_float)), n, C.byref(cnt))
+        if rc:
+            raise SlaiError(rc, "metadata f32 array '%s'" % key)
+        return out[:n]
 
     def tensors(self):
         out = {}
@@ -326,6 +367,70 @@ class Gguf:
             self.h = None
 
 
+class Tokenizer:
+    """``AnyTokenizer`` (crates/slai-chat/src/llm.rs:100-164): the Llama or GPT-2 tokenizer of a GGUF file."""
+
+    def __init__(self, gguf, kind=_ffi.TOKENIZER_AUTO):
+        self.L = _ffi.lib()
+        h = C.c_void_p()
+        err = C.create_string_buffer(512)
+        rc = self.L.slai_tokenizer_from_gguf(gguf.h, kind, C.byref(h), err, 512)
+        if rc:
+            raise SlaiError(rc, err.value.decode(errors="replace"))
+        self.h = h
+        self.kind = self.L.slai_tokenizer_kind(h)
+        self.bos, self.eos, self.unk = (self.L.slai_tokenizer_bos(h), self.L.slai_tokenizer_eos(h), self.L.slai_tokenizer_unk(h))
+        self.vocab_size = self.L.slai_tokenizer_vocab_size(h)
+
+    def _fail(self, rc):
+        raise SlaiError(rc, (self.L.slai_tokenizer_last_error(self.h) or b"").decode(errors="replace"))
+
+    def token_bytes(self, token):
+        ptr, n = C.c_void_p(), C.c_size_t()
+        rc = self.L.slai_tokenizer_token_str(self.h, token, C.byref(ptr), C.byref(n))
+        if rc:
+            raise SlaiError(rc, "token id outside the vocabulary")
+        return C.string_at(ptr, n.value) if n.value else b""
+
+    def bos_str(self):
+        return self.token_bytes(self.bos).decode()
+
+    def eos_str(self):
+        return self.token_bytes(self.eos).decode()
+
+    def encode(self, text, bos=False, eos=False):
+        raw = text.encode("utf-8") if isinstance(text, str) else bytes(text)
+        cap = 4 * len(raw) + 8
+        out, cnt = (C.c_int32 * cap)(), C.c_size_t()
+        rc = self.L.slai_tokenizer_encode(self.h, raw, len(raw), int(bos), int(eos), out, cap, C.byref(cnt))
+        if rc:
+            self._fail(rc)
+        return list(out[:cnt.value])
+
+    def decode_bytes(self, tokens, prev_token=0):
+        tokens = list(tokens)
+        arr = (C.c_int32 * max(len(tokens), 1))(*tokens)
+        n = C.c_size_t()
+        cap = 64
+        while True:
+            buf = C.create_string_buffer(cap)
+            rc = self.L.slai_tokenizer_decode(self.h, arr, len(tokens), prev_token, buf, cap, C.byref(n))
+            if rc == _ffi.E_SHAPE and n.value > cap:
+                cap = n.value
+                continue
+            if rc:
+                self._fail(rc)
+            return buf.raw[:n.value]
+
+    def decode(self, tokens, prev_token=0):
+        return self.decode_bytes(tokens, prev_token).decode("utf-8", errors="replace")
+
+    def close(self):
+        if self.h:
+            self.L.slai_tokenizer_free(self.h)
+            self.h = None
+
+
 class Llama2:
     """``ChatLlama2`` without the tokenizer: config + weights + state + the per-token driver."""
 
@@ -351,6 +456,14 @@ class Llama2:
         out = np.zeros(n_steps, dtype=np.int32)
         ms = C.c_float()
         self.b.check(self.b.L.slai_llama2_generate(self.h, prompt.ctypes.data, prompt.size, start_pos, n_steps, out.ctypes.data, C.byref(ms)))
+        return out, ms.value
+
+    def generate_sampled(self, prompt, n_steps, temperature, topp, seed, start_pos=0):
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        out = np.zeros(n_steps, dtype=np.int32)
+        ms = C.c_float()
+        self.b.check(self.b.L.slai_llama2_generate_sampled(self.h, prompt.ctypes.data, prompt.size, start_pos, n_steps, temperature, topp,
+                                                           seed, out.ctypes.data, C.byref(ms)))
         return out, ms.value
 
     def kv_buffers(self, layer):
@@ -394,6 +507,14 @@ class Gpt2:
         out = np.zeros(n_steps, dtype=np.int32)
         ms = C.c_float()
         self.b.check(self.b.L.slai_gpt2_generate(self.h, prompt.ctypes.data, prompt.size, start_pos, n_steps, out.ctypes.data, C.byref(ms)))
+        return out, ms.value
+
+    def generate_sampled(self, prompt, n_steps, temperature, topp, seed, start_pos=0):
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        out = np.zeros(n_steps, dtype=np.int32)
+        ms = C.c_float()
+        self.b.check(self.b.L.slai_gpt2_generate_sampled(self.h, prompt.ctypes.data, prompt.size, start_pos, n_steps, temperature, topp,
+                                                         seed, out.ctypes.data, C.byref(ms)))
         return out, ms.value
 
     def destroy(self):
