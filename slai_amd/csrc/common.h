@@ -45,6 +45,8 @@ struct slai_ctx {
     // per-workgroup activation slots of the row-tile GEMV (grown on demand, never inside a capture)
     float *gemv_scratch = nullptr;
     size_t gemv_scratch_floats = 0;
+    float *sampler_scratch = nullptr;   // probabilities of the device sampler (one float per vocabulary entry)
+    size_t sampler_scratch_floats = 0;
     // tuning knobs (environment overridable, see runtime.cpp)
     int gemv_rows_per_wg = 8;
     int gemv_max_threads = 1024;
@@ -182,6 +184,7 @@ bool gemv_gated_is_rowtile(const slai_ctx *ctx, const slai_qmat *gate, const sla
 int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who);
 // Makes sure the row-tile GEMV's scratch holds `floats` floats (call outside graph capture).
 int gemv_scratch_reserve(slai_ctx *ctx, size_t floats);
+int sampler_scratch_reserve(slai_ctx *ctx, size_t floats);   // grows the sampler's scratch; not during graph capture
 
 // ---- dequantisation / repack ---------------------------------------------------
 // Device-side description of a quantized matrix in either layout.
@@ -228,7 +231,8 @@ hipError_t launch_argmax(hipStream_t s, const float *v, uint32_t n, int *out_ind
                          const int *prompt, int *out_tokens);
 // models/sampler.rs:33-53 `Sampler::sample` with the draw `coin` in [0, 1) given (or, with `decode`, derived from the
 // state's seed and position; temperature and topp then come from the state as well)
-hipError_t launch_sample(hipStream_t s, const float *v, uint32_t n, float temperature, float topp, float coin, int *out_index,
+// `scratch`: n floats of device memory for the probabilities
+hipError_t launch_sample(hipStream_t s, const float *v, uint32_t n, float temperature, float topp, float coin, float *scratch, int *out_index,
                          DecodeState *decode, const int *prompt, int *out_tokens);
 
 // ---- attention ---------------------------------------------------------------------

@@ -383,7 +383,7 @@ int slai_llama2::enqueue_fused(int sampler) {
         SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, nullptr, ds,
                                         (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
     else if (sampler == 2)
-        SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, 0.0f, 0.0f, 0.0f, nullptr, ds,
+        SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, 0.0f, 0.0f, 0.0f, ctx->sampler_scratch, nullptr, ds,
                                         (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
     return SLAI_OK;
 }
@@ -471,6 +471,7 @@ static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_le
                          uint32_t start_pos, uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms, const SamplingParams *sampling = nullptr) {
     if (sampling && !(sampling->temperature >= 0.0f)) return set_error(ctx, SLAI_E_ARG, "generate: the temperature must not be negative");
     const int mode = sampling ? 2 : 1;
+    if (sampling) TRY(sampler_scratch_reserve(ctx, vocab));
     if (!prompt || !out_tokens || n_prompt == 0 || start_pos >= n_prompt) return set_error(ctx, SLAI_E_ARG, "generate: bad prompt / start position");
     if (n_steps == 0) return SLAI_OK;
     if (start_pos + n_steps > seq_len) return set_error(ctx, SLAI_E_SHAPE, "generate: would run past the context length");
@@ -683,7 +684,7 @@ int slai_gpt2::enqueue_fused(int sampler) {
     if (sampler == 1)
         SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, logits, params.n_vocab, nullptr, ds, (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
     else if (sampler == 2)
-        SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, logits, params.n_vocab, 0.0f, 0.0f, 0.0f, nullptr, ds, (const int *)loop.prompt->dptr,
+        SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, logits, params.n_vocab, 0.0f, 0.0f, 0.0f, ctx->sampler_scratch, nullptr, ds, (const int *)loop.prompt->dptr,
                                         (int *)loop.out_tokens->dptr));
     return SLAI_OK;
 }

@@ -2,9 +2,10 @@
 // (`coin`) supplied by the caller or derived from (seed, position), plus the forced-token rule and loop
 // bookkeeping the greedy kernel applies (crates/slai-chat/src/sampler.rs:100-105, chat_llama2.rs:105-158).
 //
-// One workgroup of 1024 threads.  Wave w owns the contiguous slice [w*seg, (w+1)*seg) of the vocabulary and walks
-// it 64 consecutive entries at a time, so loads are coalesced and index order (which the cumulative distribution
-// and the order among equal probabilities depend on) is wave order, then iteration order, then lane order.
+// One workgroup of 1024 threads.  Wave w owns the contiguous slice [w*slice, (w+1)*slice) of the vocabulary and
+// walks it 64 consecutive entries at a time, so loads are coalesced and index order (which the cumulative
+// distribution and the order among equal probabilities depend on) is wave order, then iteration order, then lane
+// order.  The probabilities are written once to a scratch vector (n floats, L2-resident) and re-read by the passes.
 //
 // The reference sorts the candidates by descending probability and walks the sorted list twice (once up to the
 // nucleus mass `topp`, once up to coin * mass).  Here both walks are one primitive, `crossing(target)`: the first
@@ -23,7 +24,7 @@ namespace slai {
 namespace {
 
 constexpr int NT = 1024, NW = NT / 64;
-constexpr int CACHE = 32;                       // probabilities of a thread's first CACHE entries stay in registers
+constexpr int UNROLL = 16;                      // scratch entries a thread requests before it uses the first
 
 struct Shared {
     float f[NW][16];
@@ -33,6 +34,11 @@ struct Shared {
     float red[NW];
     uint32_t redu[NW];
     uint32_t result;
+    // a bin of at most 64 entries, gathered and ordered by one wave
+    uint32_t gcount;
+    float gp[64], sp[64];
+    uint32_t gi[64], si[64];
+    uint32_t res_key, res_idx, res_pos; float res_cum;
 };
 
 __device__ __forceinline__ float wsum(float v) {
@@ -40,58 +46,75 @@ __device__ __forceinline__ float wsum(float v) {
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
     return v;
 }
-__device__ __forceinline__ float wmax(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
-    return v;
-}
 // 16 values per lane -> their 16 totals over the wave with 17 exchanges instead of 96: every step halves the values
 // a lane is responsible for.  Afterwards a[0] of lane L holds the total of value 8*b5 + 4*b4 + 2*b3 + b2 (bits of L).
-template <class X> __device__ __forceinline__ void wave_reduce16(X (&a)[16], uint32_t lane) {
+template <int HALF, int M, class X> __device__ __forceinline__ void halve(X (&a)[16], uint32_t lane) {
+    const bool up = lane & M;
 #pragma unroll
-    for (int half = 8, m = 32; half >= 1; half >>= 1, m >>= 1) {
-        const bool up = lane & m;
-#pragma unroll
-        for (int k = 0; k < half; ++k) {
-            const X keep = up ? a[k + half] : a[k];
-            const X send = up ? a[k] : a[k + half];
-            a[k] = keep + __shfl_xor(send, m, 64);
-        }
+    for (int k = 0; k < HALF; ++k) {
+        const X keep = up ? a[k + HALF] : a[k];
+        const X send = up ? a[k] : a[k + HALF];
+        a[k] = keep + __shfl_xor(send, M, 64);
     }
+}
+template <class X> __device__ __forceinline__ void wave_reduce16(X (&a)[16], uint32_t lane) {
+    halve<8, 32>(a, lane); halve<4, 16>(a, lane); halve<2, 8>(a, lane); halve<1, 4>(a, lane);
     a[0] += __shfl_xor(a[0], 2, 64);
     a[0] += __shfl_xor(a[0], 1, 64);
 }
 
-struct Dist {                                   // what defines the distribution: p_i = exp(v_i / T - xm) / S
-    const float *v; uint32_t n; float T, xm, S;
-    uint32_t seg, base;                         // slice length (a multiple of 64) and this thread's first index
-    uint32_t iters;                             // 64-entry steps per slice
-    float pc[CACHE];
+// The distribution: probabilities (softmax of v / T, sampler.rs:39-42 with softmax.rs:46-59) of the entries this
+// thread owns, index(k) = wave * slice + 64 * k + lane.  R > 0: the slice is 64 * R entries and they stay in registers
+// (vocabularies up to 16 * 64 * R); R == 0: they are written once to a scratch vector and re-read by every pass (a
+// single compute unit re-reads slowly: this is the fallback for larger vocabularies).  A thread only ever reads
+// back the scratch entries it wrote itself.
+template <int R> struct Dist {
+    float r[R > 0 ? R : 1];
+    const float *p; uint32_t n;
+    uint32_t kmax;                              // bits of the largest probability, 1 / (sum of the exponentials)
+    uint32_t base;                              // this thread's first index: wave * slice + lane
+    uint32_t iters;                             // 64-entry steps per slice (R, or a multiple of UNROLL)
     __device__ __forceinline__ uint32_t index(uint32_t k) const { return base + 64 * k; }
-    __device__ __forceinline__ float raw(uint32_t k) const {          // sampler.rs:39-42 + softmax.rs:46-59
-        const uint32_t i = index(k);
-        return i < n ? expf(v[i] / T - xm) : 0.0f;
-    }
-    __device__ __forceinline__ float prob_uncached(uint32_t k) const { return raw(k) / S; }
 };
 
-// body(p, i) for every step of the thread's slice: p from the registers for the first CACHE steps, recomputed beyond
-template <class F> __device__ __forceinline__ void for_each_prob(const Dist &D, F &&body) {
+// body(p, i) for every entry of the thread's slice, in increasing i
+template <int R, class F> __device__ __forceinline__ void for_each_prob(const Dist<R> &D, F &&body) {
+    if constexpr (R > 0) {
 #pragma unroll
-    for (uint32_t k = 0; k < CACHE; ++k)
-        if (k < D.iters) body(D.pc[k], D.index(k));
-    for (uint32_t k = CACHE; k < D.iters; ++k) body(D.prob_uncached(k), D.index(k));
+        for (int k = 0; k < R; ++k) body(D.r[k], D.index(k));
+    } else {
+        for (uint32_t k0 = 0; k0 < D.iters; k0 += UNROLL) {
+            float v[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) { const uint32_t i = D.index(k0 + u); v[u] = i < D.n ? D.p[i] : 0.0f; }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) body(v[u], D.index(k0 + u));
+        }
+    }
 }
 
-struct Cross { uint32_t key, j, position; float cum; };
+// `index` is the entry itself when the search ended in a bin small enough to order directly; 0xffffffff otherwise:
+// then the entry is the j-th (index order) of those whose probability has the bits `key`
+struct Cross { uint32_t key, j, position, index; float cum; };
 
 // First position of the descending, index-stable order of the candidates (p >= cutoff) at which the running mass
 // exceeds `target`; when it never does, the last position.  `cum` is the running mass there (sampler.rs:108-118).
-__device__ __forceinline__ Cross crossing(const Dist &D, float cutoff, float target, Shared &sh) {
+template <int R> __device__ __forceinline__ Cross crossing(const Dist<R> &D, float cutoff, float target, Shared &sh) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t prefix = 0, cnt_above = 0, ties = 0;
     float mass_above = 0.0f;
-    for (int shift = 28; shift >= 0; shift -= 4) {
+    // every candidate's bits lie between those of the cutoff and of the largest probability: the four-bit groups the
+    // two share need no pass
+    int start = 28;
+    {
+        const uint32_t lo = __float_as_uint(cutoff), hi = D.kmax;
+        if (hi >= lo) {
+            const uint32_t x = lo ^ hi;
+            start = x ? ((31 - __clz((int)x)) / 4) * 4 : 0;
+            prefix = start < 28 ? hi & (0xffffffffu << (start + 4)) : 0u;
+        }
+    }
+    for (int shift = start; shift >= 0; shift -= 4) {
         float m[16];
         uint32_t c[16];
 #pragma unroll
@@ -134,9 +157,48 @@ __device__ __forceinline__ Cross crossing(const Dist &D, float cutoff, float tar
         mass_above = acc; cnt_above = cacc; prefix |= (uint32_t)sel << shift; ties = sh.totu[sel];
         // no barrier here: the totals are rewritten only after the next pass's first barrier, which every thread
         // reaches after this walk
+        if (ties >= 1 && ties <= 64 && shift > 0) {
+            // ---- few entries left: gather them, let one wave put them in the sampler's order (probability descending,
+            // then index) and add them up in that order
+            const uint32_t mask = 0xffffffffu << shift;
+            if (threadIdx.x == 0) sh.gcount = 0;
+            __syncthreads();
+            for_each_prob(D, [&](float p, uint32_t i) {
+                if (i < D.n && p >= cutoff && (__float_as_uint(p) & mask) == prefix) {
+                    const uint32_t slot = atomicAdd(&sh.gcount, 1u);
+                    if (slot < 64) { sh.gp[slot] = p; sh.gi[slot] = i; }
+                }
+            });
+            __syncthreads();
+            if (wave == 0) {
+                const uint32_t cnt = ties;
+                const bool live = lane < cnt;
+                const float mp = live ? sh.gp[lane] : 0.0f;
+                const uint32_t mi = live ? sh.gi[lane] : 0xffffffffu;
+                uint32_t rank = 0;
+                for (uint32_t q = 0; q < cnt; ++q) {
+                    const float op = sh.gp[q]; const uint32_t oi = sh.gi[q];
+                    rank += (op > mp || (op == mp && oi < mi)) ? 1u : 0u;
+                }
+                if (live) { sh.sp[rank] = mp; sh.si[rank] = mi; }
+                // (one wave: its LDS writes are complete before its next LDS reads are issued)
+                float run = live ? sh.sp[lane] : 0.0f;
+#pragma unroll
+                for (int d = 1; d < 64; d <<= 1) { const float o = __shfl_up(run, d, 64); if (lane >= (uint32_t)d) run += o; }
+                run += mass_above;
+                const unsigned long long over = __ballot(live && run > target);
+                const uint32_t at = over ? (uint32_t)__ffsll((long long)over) - 1 : cnt - 1;   // never crossed: the last one
+                if (lane == at) { sh.res_key = __float_as_uint(sh.sp[at]); sh.res_idx = sh.si[at]; sh.res_pos = cnt_above + at; sh.res_cum = run; }
+            }
+            __syncthreads();
+            Cross r;
+            r.key = sh.res_key; r.index = sh.res_idx; r.position = sh.res_pos; r.cum = sh.res_cum; r.j = 0;
+            __syncthreads();
+            return r;
+        }
     }
     Cross r;
-    r.key = prefix;
+    r.key = prefix; r.index = 0xffffffffu;
     const float pv = __uint_as_float(prefix);
     float cc = mass_above; uint32_t j = ties;
     for (uint32_t t = 1; t <= ties; ++t) { cc += pv; if (cc > target) { j = t; break; } }
@@ -145,7 +207,7 @@ __device__ __forceinline__ Cross crossing(const Dist &D, float cutoff, float tar
 }
 
 // index of the j-th (1-based, index order) candidate whose probability has the bits `key`
-__device__ __forceinline__ uint32_t locate(const Dist &D, float cutoff, uint32_t key, uint32_t j, Shared &sh) {
+template <int R> __device__ __forceinline__ uint32_t locate(const Dist<R> &D, float cutoff, uint32_t key, uint32_t j, Shared &sh) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t mine = 0;
     for_each_prob(D, [&](float p, uint32_t i) { mine += (i < D.n && p >= cutoff && __float_as_uint(p) == key) ? 1u : 0u; });
@@ -189,9 +251,68 @@ __device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
     return x ^ (x >> 31);
 }
 
-__global__ void __launch_bounds__(NT) sample_kernel(const float *v, uint32_t n, float temperature, float topp, float coin_arg,
-                                                    int *out_index, DecodeState *st, const int *prompt, int *out_tokens) {
+// sampler.rs:63-78 `sample_mult` on registers: the first index whose cumulative probability exceeds the coin.  Row sums
+// (one per 64-entry step) of all waves are scanned by the first 16 * R threads; the wave that owns the crossing row
+// then scans that row alone.
+template <int R> __device__ __forceinline__ uint32_t sample_mult_rows(const Dist<R> &D, float coin, uint32_t fallback, Shared &sh, float *rows /* [NW * R] */,
+                                                                     float *incl /* [NW * R] */) {
+    static_assert(R == 32, "two 16-value reductions cover the rows");
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float a[16], b[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) { a[k] = D.r[k]; b[k] = D.r[16 + k]; }
+    wave_reduce16(a, lane);
+    wave_reduce16(b, lane);
+    if ((lane & 3) == 0) {
+        const uint32_t idx = ((lane >> 5) & 1) * 8 + ((lane >> 4) & 1) * 4 + ((lane >> 3) & 1) * 2 + ((lane >> 2) & 1);
+        rows[wave * R + idx] = a[0]; rows[wave * R + 16 + idx] = b[0];
+    }
+    if (threadIdx.x == 0) sh.result = 0xffffffffu;
+    __syncthreads();
+    // inclusive scan of the NW * R row sums in index order (row t belongs to wave t / R, step t % R)
+    const uint32_t t = threadIdx.x;
+    float inc = t < NW * R ? rows[t] : 0.0f;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) { const float o = __shfl_up(inc, d, 64); if (lane >= (uint32_t)d) inc += o; }
+    if (lane == 63) sh.red[wave] = inc;
+    __syncthreads();
+    float before = 0.0f;
+    for (uint32_t w = 0; w < wave; ++w) before += sh.red[w];
+    inc += before;
+    if (t < NW * R) incl[t] = inc;
+    const unsigned long long hits = __ballot(t < NW * R && coin < inc);
+    if (lane == 0 && hits) atomicMin(&sh.result, (t & ~63u) + (uint32_t)__ffsll((long long)hits) - 1);
+    __syncthreads();
+    const uint32_t row = sh.result;                           // first row whose running total exceeds the coin
+    __syncthreads();
+    if (row == 0xffffffffu) return fallback;                  // rounding left the total below the coin (:77)
+    if (wave == row / R) {
+        const uint32_t k = row % R;
+        float x = 0.0f;
+#pragma unroll
+        for (int q = 0; q < R; ++q) x = k == (uint32_t)q ? D.r[q] : x;
+        const float start = row ? incl[row - 1] : 0.0f;
+        float run = x;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) { const float o = __shfl_up(run, d, 64); if (lane >= (uint32_t)d) run += o; }
+        const uint32_t i = D.index(k);
+        const unsigned long long mask = __ballot(i < D.n && coin < start + run);
+        const unsigned long long valid = __ballot(i < D.n);
+        // the row total said the crossing is here; if the finer sums disagree, it is the row's last entry
+        const uint32_t at = mask ? (uint32_t)__ffsll((long long)mask) - 1 : 63u - (uint32_t)__clzll((long long)valid);
+        if (lane == at) sh.result = i;
+    }
+    __syncthreads();
+    const uint32_t r = sh.result;
+    __syncthreads();
+    return r;
+}
+
+template <int R>
+__global__ void __launch_bounds__(NT) sample_kernel(const float *__restrict__ v, uint32_t n, float temperature, float topp, float coin_arg,
+                                                    float *pbuf, int *out_index, DecodeState *st, const int *prompt, int *out_tokens) {
     __shared__ Shared sh;
+    __shared__ float rows[R > 0 ? NW * R : 1], rows_incl[R > 0 ? NW * R : 1];
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float coin = coin_arg;
     if (st) {                                                   // the decode loop: parameters and counter live in device memory
@@ -199,16 +320,32 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *v, uint32_t n, 
         const uint64_t seed = ((uint64_t)st->seed_hi << 32) | st->seed_lo;
         coin = (float)(splitmix64(seed + (uint64_t)(uint32_t)st->pos) >> 40) * (1.0f / 16777216.0f);
     }
-    Dist D;
-    D.v = v; D.n = n; D.T = temperature;
-    D.seg = ((n + NW - 1) / NW + 63) / 64 * 64;
-    D.base = wave * D.seg + lane;
-    D.iters = D.seg / 64;
+    const uint32_t slice = R > 0 ? 64u * R : ((n + NW - 1) / NW + 64 * UNROLL - 1) / (64 * UNROLL) * (64 * UNROLL);
+    Dist<R> D;
+    D.p = pbuf; D.n = n;
+    D.base = wave * slice + lane;
+    D.iters = slice / 64;
     // ---- max (of v / T: division by a positive T is monotonic, so it is max(v) / T) and first index of the maximum
     float best = -FLT_MAX; uint32_t besti = 0xffffffffu;
-    for (uint32_t k = 0; k < D.iters; ++k) {
-        const uint32_t i = D.index(k);
-        if (i < n) { const float x = v[i]; if (besti == 0xffffffffu || x > best) { best = x; besti = i; } }
+    if constexpr (R > 0) {
+#pragma unroll
+        for (int k = 0; k < R; ++k) { const uint32_t i = D.index(k); D.r[k] = v[i < n ? i : 0]; }
+#pragma unroll
+        for (int k = 0; k < R; ++k) {
+            const uint32_t i = D.index(k);
+            if (i < n && (besti == 0xffffffffu || D.r[k] > best)) { best = D.r[k]; besti = i; }
+        }
+    } else {
+        for (uint32_t k0 = 0; k0 < D.iters; k0 += UNROLL) {
+            float x[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) { const uint32_t i = D.index(k0 + u); x[u] = v[i < n ? i : 0]; }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint32_t i = D.index(k0 + u);
+                if (i < n && (besti == 0xffffffffu || x[u] > best)) { best = x[u]; besti = i; }
+            }
+        }
     }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) {
@@ -226,23 +363,51 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *v, uint32_t n, 
     if (temperature == 0.0f) {
         chosen = besti;                                         // sampler.rs:34-36: greedy
     } else {
-        D.xm = best / temperature;
-        // ---- normaliser
+        // ---- exp(v / T - max), their sum, then the probabilities (in the registers, or in the scratch)
+        const float xm = best / temperature;
         float part = 0.0f;
-        for (uint32_t k = 0; k < D.iters; ++k) part += D.raw(k);
+        if constexpr (R > 0) {
+#pragma unroll
+            for (int k = 0; k < R; ++k) { D.r[k] = D.index(k) < n ? expf(D.r[k] / temperature - xm) : 0.0f; part += D.r[k]; }
+        } else {
+            for (uint32_t k0 = 0; k0 < D.iters; k0 += UNROLL) {
+                float x[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) { const uint32_t i = D.index(k0 + u); x[u] = v[i < n ? i : 0]; }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const uint32_t i = D.index(k0 + u);
+                    if (i < n) { const float e = expf(x[u] / temperature - xm); pbuf[i] = e; part += e; }
+                }
+            }
+        }
         part = wsum(part);
         if (lane == 0) sh.red[wave] = part;
         __syncthreads();
         float S = 0.0f;
         for (int w = 0; w < NW; ++w) S += sh.red[w];
         __syncthreads();
-        D.S = S;
+        D.kmax = __float_as_uint(1.0f / S);                 // the maximum's exponential is exp(0) = 1
+        if constexpr (R > 0) {
 #pragma unroll
-        for (uint32_t k = 0; k < CACHE; ++k) D.pc[k] = k < D.iters ? D.prob_uncached(k) : 0.0f;
+            for (int k = 0; k < R; ++k) D.r[k] = D.r[k] / S;
+        } else {
+            for (uint32_t k0 = 0; k0 < D.iters; k0 += UNROLL) {
+                float e[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) { const uint32_t i = D.index(k0 + u); e[u] = i < n ? pbuf[i] : 0.0f; }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) { const uint32_t i = D.index(k0 + u); if (i < n) pbuf[i] = e[u] / S; }
+            }
+        }
         if (topp <= 0.0f || topp >= 1.0f) {
+            if constexpr (R > 0) {
+                chosen = sample_mult_rows(D, coin, n - 1, sh, rows, rows_incl);
+            } else {
             // ---- sampler.rs:63-78 `sample_mult`: the first index whose cumulative probability exceeds the coin
             float tot = 0.0f;
-            for_each_prob(D, [&](float p, uint32_t) { tot += wsum(p); });
+            for_each_prob(D, [&](float p, uint32_t) { tot += p; });
+            tot = wsum(tot);
             if (lane == 0) sh.red[wave] = tot;
             if (threadIdx.x == 0) sh.result = n - 1;           // rounding may leave the total below the coin
             __syncthreads();
@@ -263,6 +428,7 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *v, uint32_t n, 
             if (lane == 0 && found != 0xffffffffu) atomicMin(&sh.result, found);
             __syncthreads();
             chosen = sh.result;
+            }
         } else {
             // ---- sampler.rs:85-131 `sample_topp`
             const float cutoff = (1.0f - topp) / ((float)n - 1.0f);
@@ -270,7 +436,7 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *v, uint32_t n, 
             const float r = coin * nucleus.cum;
             Cross pick = crossing(D, cutoff, r, sh);
             if (pick.position > nucleus.position) pick = nucleus;     // rounding: stay inside the nucleus (:130)
-            chosen = locate(D, cutoff, pick.key, pick.j, sh);
+            chosen = pick.index != 0xffffffffu ? pick.index : locate(D, cutoff, pick.key, pick.j, sh);
             if (chosen == 0xffffffffu) chosen = besti;          // not reachable with finite logits; keeps the id valid
         }
     }
@@ -290,9 +456,10 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *v, uint32_t n, 
 
 }  // namespace
 
-hipError_t launch_sample(hipStream_t s, const float *v, uint32_t n, float temperature, float topp, float coin, int *out_index,
+hipError_t launch_sample(hipStream_t s, const float *v, uint32_t n, float temperature, float topp, float coin, float *scratch, int *out_index,
                          DecodeState *decode, const int *prompt, int *out_tokens) {
-    sample_kernel<<<1, NT, 0, s>>>(v, n, temperature, topp, coin, out_index, decode, prompt, out_tokens);
+    if (n <= NW * 64 * 32) sample_kernel<32><<<1, NT, 0, s>>>(v, n, temperature, topp, coin, scratch, out_index, decode, prompt, out_tokens);
+    else sample_kernel<0><<<1, NT, 0, s>>>(v, n, temperature, topp, coin, scratch, out_index, decode, prompt, out_tokens);
     return hipGetLastError();
 }
 

@@ -92,6 +92,7 @@ SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     hipStreamSynchronize(ctx->stream);
     if (ctx->attn_scratch) hipFree(ctx->attn_scratch);
     if (ctx->gemv_scratch) hipFree(ctx->gemv_scratch);
+    if (ctx->sampler_scratch) hipFree(ctx->sampler_scratch);
     if (ctx->timer0) hipEventDestroy(ctx->timer0);
     if (ctx->timer1) hipEventDestroy(ctx->timer1);
     hipStreamDestroy(ctx->stream);
@@ -281,6 +282,17 @@ int gemv_scratch_reserve(slai_ctx *ctx, size_t floats) {
     ctx->gemv_scratch = nullptr; ctx->gemv_scratch_floats = 0;
     SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->gemv_scratch, floats * sizeof(float)));
     ctx->gemv_scratch_floats = floats;
+    return SLAI_OK;
+}
+
+int sampler_scratch_reserve(slai_ctx *ctx, size_t floats) {
+    if (floats <= ctx->sampler_scratch_floats) return SLAI_OK;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "sampler scratch must be reserved before graph capture");
+    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->sampler_scratch) hipFree(ctx->sampler_scratch);
+    ctx->sampler_scratch = nullptr; ctx->sampler_scratch_floats = 0;
+    SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->sampler_scratch, floats * sizeof(float)));
+    ctx->sampler_scratch_floats = floats;
     return SLAI_OK;
 }
 
@@ -615,7 +627,9 @@ SLAI_EXPORT int slai_sample(slai_ctx *ctx, slai_view logits, float temperature, 
     NEED_VEC(logits, "logits", vl);
     if (vl.stride != 1 || out_index->dtype != SLAI_DT_I32 || out_index->bytes < 4) return set_error(ctx, SLAI_E_SHAPE, "slai_sample: contiguous logits and an I32 output are required");
     if (!(temperature >= 0.0f) || !(coin >= 0.0f && coin < 1.0f)) return set_error(ctx, SLAI_E_ARG, "slai_sample: temperature must be >= 0 and the draw in [0, 1)");
-    SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, vl.p, vl.n, temperature, topp, coin, (int *)out_index->dptr, nullptr, nullptr, nullptr));
+    if (int rc = sampler_scratch_reserve(ctx, vl.n)) return rc;
+    SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, vl.p, vl.n, temperature, topp, coin, ctx->sampler_scratch, (int *)out_index->dptr, nullptr, nullptr,
+                                    nullptr));
     return SLAI_OK;
 }
 // The draw the device loop uses at position `pos`: the top 24 bits of splitmix64(seed + pos), scaled to [0, 1)
