@@ -71,13 +71,29 @@ class GgufWriter:
         return out
 
 
+def add_tokenizer_meta(w, tok):
+    """tokenizer.* keys read by crates/slai/src/models/{llama2,gpt2}/tokenizer.rs and slai-chat/src/{llm,chat_template}.rs."""
+    w.add_meta("tokenizer.ggml.model", T_STR, tok["model"])
+    w.add_meta("tokenizer.ggml.tokens", T_ARR, list(tok["tokens"]), elem_type=T_STR)
+    if "scores" in tok:
+        w.add_meta("tokenizer.ggml.scores", T_ARR, [float(x) for x in tok["scores"]], elem_type=T_F32)
+    if "merges" in tok:
+        w.add_meta("tokenizer.ggml.merges", T_ARR, list(tok["merges"]), elem_type=T_STR)
+    w.add_meta("tokenizer.ggml.bos_token_id", T_U32, tok["bos"])
+    w.add_meta("tokenizer.ggml.eos_token_id", T_U32, tok["eos"])
+    if "unk" in tok:
+        w.add_meta("tokenizer.ggml.unknown_token_id", T_U32, tok["unk"])
+    if tok.get("chat_template"):
+        w.add_meta("tokenizer.chat_template", T_STR, tok["chat_template"])
+
+
 def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32).view(np.uint8).reshape(-1)
 
 
 def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, wtype, seed=1234,
                std=0.02, rope_base=10000.0, rms_eps=1e-5, out_type=None, v_type=None, embd_type=None,
-               with_output=True, arch="llama", bias=False, norm_random=False, distinct_layers=None):
+               with_output=True, arch="llama", bias=False, norm_random=False, distinct_layers=None, tokenizer=None):
     """Synthetic Llama-2-shape model file (uint8 numpy array).
 
     Weights are seeded std*N(0,1) quantized to `wtype` (`v_type` for attn_v, `out_type` for
@@ -85,6 +101,8 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
     `distinct_layers`: when set, only that many layers are generated from scratch and the
     others reuse their packed bytes with the rows rotated (still distinct memory and the same
     value distribution; used to bound set-up time of the largest benchmark model).
+    `tokenizer`: optional dict(model=, tokens=, scores=|merges=, bos=, eos=, unk=, chat_template=) written as the
+    tokenizer.* metadata a chat front end reads; `vocab` must then equal len(tokens).
     """
     out_type = wtype if out_type is None else out_type
     v_type = wtype if v_type is None else v_type
@@ -101,7 +119,11 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
     w.add_meta(arch + ".context_length", T_U32, seq_len)
     w.add_meta(arch + ".rope.freq_base", T_F32, rope_base)
     w.add_meta(arch + ".attention.layer_norm_rms_epsilon", T_F32, rms_eps)
-    w.add_meta("tokenizer.ggml.tokens", T_ARR, [""] * vocab, elem_type=T_STR)
+    if tokenizer is None:
+        w.add_meta("tokenizer.ggml.tokens", T_ARR, [""] * vocab, elem_type=T_STR)
+    else:
+        assert len(tokenizer["tokens"]) == vocab
+        add_tokenizer_meta(w, tokenizer)
     rng = np.random.Generator(np.random.PCG64(seed))
     ctr = [seed * 1000003]
 
