@@ -273,6 +273,11 @@ def main():
     tb = token_bytes(cfg, model.weight_bytes(), W, W + K - 1)
     log("decode: %.3f ms/token (events), wall %.3f ms/token, %.1f tok/s, %.2f GB/token -> %.1f GB/s"
         % (ms_per_step, wall * 1000 / K, tok_s, tb / 1e9, tb / ms_per_step / 1e6))
+    # the same K positions with the chat's sampler (temperature 0.7, top-p 0.95) picked on the device: reported beside
+    # the headline, never as it.  Random weights give nearly flat logits, the slow case of the nucleus search.
+    _, ms_s = model.generate_sampled(seq, K, 0.7, 0.95, args.seed, start_pos=W)
+    sampled = dict(tok_s=round(1000.0 * K / ms_s, 2), ms_per_step=round(ms_s / K, 4), temperature=0.7, top_p=0.95)
+    log("sampled decode (device sampler, T=0.7, top-p 0.95): %.3f ms/token, %.1f tok/s" % (ms_s / K, 1000.0 * K / ms_s))
     model.destroy(); g.close(); del data
 
     roof = None
@@ -304,6 +309,7 @@ def main():
         "token_bytes": int(tb), "hbm_gbs": round(tb / ms_per_step / 1e6, 1),
         "hbm_roofline_frac": round(tb / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
         "roofline_tok_s": round(HBM_PEAK_GBS * 1e9 / tb, 1),
+        "sampled_decode": sampled,
         "roofline": roof, "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)
