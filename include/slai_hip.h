@@ -241,6 +241,9 @@ int slai_gguf_meta_u32(const slai_gguf *g, const char *key, uint32_t *out);
 int slai_gguf_meta_f32(const slai_gguf *g, const char *key, float *out);
 int slai_gguf_meta_str(const slai_gguf *g, const char *key, const char **out);
 int slai_gguf_meta_array_len(const slai_gguf *g, const char *key, uint64_t *out);
+/* `metadata_debug_strings` (gguf.rs:686-695): entry i of slai_gguf_metadata_count(), keys in sorted order, as
+ * "key = Type(value)" or "key = array[len]" */
+int slai_gguf_meta_describe(const slai_gguf *g, uint64_t i, char *out, size_t out_len);
 /* `as_string_array` (gguf.rs:316-322): pointers into the file bytes (not NUL-terminated) and lengths of the first
  * `capacity` elements; `count` receives the number of elements.  `as_f32_array` (gguf.rs:324-330) likewise. */
 int slai_gguf_meta_array_str(const slai_gguf *g, const char *key, const char **ptrs, uint64_t *lens, uint64_t capacity,

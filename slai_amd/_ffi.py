@@ -112,6 +112,7 @@ SIGNATURES = {
     "slai_gguf_meta_f32": (i32, [vp, C.c_char_p, P(C.c_float)]),
     "slai_gguf_meta_str": (i32, [vp, C.c_char_p, P(C.c_char_p)]),
     "slai_gguf_meta_array_len": (i32, [vp, C.c_char_p, P(u64)]),
+    "slai_gguf_meta_describe": (i32, [vp, u64, C.c_char_p, sz]),
     "slai_gguf_open_file": (i32, [C.c_char_p, P(vp), C.c_char_p, sz]),
     "slai_gguf_meta_array_str": (i32, [vp, C.c_char_p, P(vp), P(u64), u64, P(u64)]),
     "slai_gguf_meta_array_f32": (i32, [vp, C.c_char_p, P(C.c_float), u64, P(u64)]),

@@ -141,9 +141,12 @@ class ChatLlm:
 
 
 def inspect(gguf):
-    """`gguf.print_tensors()` (crates/slai/src/gguf.rs:697-711)."""
-    for name, info in gguf.tensors().items():
-        print("%-40s type %2d dims %s" % (name, info["type"], info["dims"]))
+    """`gguf.print_metadata()` and `gguf.print_tensors()` (crates/slai/src/gguf.rs:681-711)."""
+    for line in gguf.metadata_debug_strings():
+        print(line)
+    tensors = gguf.tensors()
+    for name in sorted(tensors):
+        print("%s -> %s" % (name, tensors[name]["dims"]))
 
 
 def main(argv=None):

@@ -6,6 +6,7 @@
 #include <cerrno>
 #include <cstdio>
 #include <cstring>
+#include <iterator>
 #include <fcntl.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
@@ -246,6 +247,27 @@ SLAI_EXPORT int slai_gguf_meta_array_len(const slai_gguf *g, const char *key, ui
     if (!v) return SLAI_E_MISSING;
     if (v->type != 9) return SLAI_E_TYPE;
     *out = v->arr_len;
+    return SLAI_OK;
+}
+
+// gguf.rs:686-695 `metadata_debug_strings`: entry i (keys in sorted order; the reference's map has no order) as
+// "key = value" for scalars and strings, "key = array[len]" for arrays
+SLAI_EXPORT int slai_gguf_meta_describe(const slai_gguf *g, uint64_t i, char *out, size_t out_len) {
+    if (!g || !out || !out_len || i >= g->g.metadata.size()) return SLAI_E_ARG;
+    auto it = g->g.metadata.begin();
+    std::advance(it, (size_t)i);
+    const GgufMetaValue &v = it->second;
+    static const char *const names[] = {"U8", "I8", "U16", "I16", "U32", "I32", "F32", "Bool", "String", "Array", "U64", "I64", "F64"};
+    std::string val;
+    switch (v.type) {
+    case 0: case 2: case 4: case 10: val = std::string(names[v.type]) + "(" + std::to_string(v.u) + ")"; break;
+    case 1: case 3: case 5: case 11: val = std::string(names[v.type]) + "(" + std::to_string(v.i) + ")"; break;
+    case 6: case 12: { char b[64]; snprintf(b, sizeof b, "%s(%g)", names[v.type], v.f); val = b; break; }
+    case 7: val = v.u ? "Bool(true)" : "Bool(false)"; break;
+    case 8: val = "String(\"" + v.s + "\")"; break;
+    default: val = "array[" + std::to_string(v.arr_len) + "]"; break;
+    }
+    snprintf(out, out_len, "%s = %s", it->first.c_str(), val.c_str());
     return SLAI_OK;
 }
 

@@ -76,8 +76,8 @@ void loop_destroy(slai_ctx *ctx, DeviceLoop &L) {
     if (L.state) slai_buffer_destroy(ctx, L.state);
     if (L.prompt) slai_buffer_destroy(ctx, L.prompt);
     if (L.out_tokens) slai_buffer_destroy(ctx, L.out_tokens);
-    if (L.ev0) hipEventDestroy(L.ev0);
-    if (L.ev1) hipEventDestroy(L.ev1);
+    if (L.ev0) (void)hipEventDestroy(L.ev0);
+    if (L.ev1) (void)hipEventDestroy(L.ev1);
 }
 }  // namespace
 

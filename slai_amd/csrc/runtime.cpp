@@ -88,14 +88,14 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
 
 SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     if (!ctx) return;
-    hipSetDevice(ctx->device);
-    hipStreamSynchronize(ctx->stream);
-    if (ctx->attn_scratch) hipFree(ctx->attn_scratch);
-    if (ctx->gemv_scratch) hipFree(ctx->gemv_scratch);
-    if (ctx->sampler_scratch) hipFree(ctx->sampler_scratch);
-    if (ctx->timer0) hipEventDestroy(ctx->timer0);
-    if (ctx->timer1) hipEventDestroy(ctx->timer1);
-    hipStreamDestroy(ctx->stream);
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
+    if (ctx->gemv_scratch) (void)hipFree(ctx->gemv_scratch);
+    if (ctx->sampler_scratch) (void)hipFree(ctx->sampler_scratch);
+    if (ctx->timer0) (void)hipEventDestroy(ctx->timer0);
+    if (ctx->timer1) (void)hipEventDestroy(ctx->timer1);
+    (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
 
@@ -123,7 +123,7 @@ SLAI_EXPORT int slai_buffer_create(slai_ctx *ctx, size_t bytes, int dtype, uint3
     if (e == hipSuccess) e = hipMemsetAsync(b->dptr, 0, alloc, ctx->stream);
     if (e == hipSuccess && (usage & SLAI_USAGE_MAP_READ)) e = hipHostMalloc(&b->host_staging, alloc, hipHostMallocDefault);
     if (e != hipSuccess) {
-        if (b->dptr) hipFree(b->dptr);
+        if (b->dptr) (void)hipFree(b->dptr);
         delete b;
         return hip_fail(ctx, e, "slai_buffer_create");
     }
@@ -133,9 +133,9 @@ SLAI_EXPORT int slai_buffer_create(slai_ctx *ctx, size_t bytes, int dtype, uint3
 
 SLAI_EXPORT void slai_buffer_destroy(slai_ctx *ctx, slai_buffer *b) {
     if (!b) return;
-    if (ctx) hipStreamSynchronize(ctx->stream);
-    if (b->dptr) hipFree(b->dptr);
-    if (b->host_staging) hipHostFree(b->host_staging);
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    if (b->dptr) (void)hipFree(b->dptr);
+    if (b->host_staging) (void)hipHostFree(b->host_staging);
     delete b;
 }
 SLAI_EXPORT size_t slai_buffer_size(const slai_buffer *b) { return b ? b->bytes : 0; }
@@ -225,9 +225,9 @@ SLAI_EXPORT int slai_qmat_create_layout(slai_ctx *ctx, uint32_t ggml_type, uint3
         }
     }
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
-    if (staging) hipFree(staging);
+    if (staging) (void)hipFree(staging);
     if (e != hipSuccess) {
-        if (m->dptr) hipFree(m->dptr);
+        if (m->dptr) (void)hipFree(m->dptr);
         delete m;
         return hip_fail(ctx, e, "slai_qmat_create");
     }
@@ -237,8 +237,8 @@ SLAI_EXPORT int slai_qmat_create_layout(slai_ctx *ctx, uint32_t ggml_type, uint3
 
 SLAI_EXPORT void slai_qmat_destroy(slai_ctx *ctx, slai_qmat *m) {
     if (!m) return;
-    if (ctx) hipStreamSynchronize(ctx->stream);
-    if (m->dptr) hipFree(m->dptr);
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    if (m->dptr) (void)hipFree(m->dptr);
     delete m;
 }
 SLAI_EXPORT int slai_qmat_shape(const slai_qmat *m, uint32_t *nrows, uint32_t *ncols, uint32_t *ggml_type) {
@@ -278,7 +278,7 @@ int gemv_scratch_reserve(slai_ctx *ctx, size_t floats) {
     if (floats <= ctx->gemv_scratch_floats) return SLAI_OK;
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "GEMV scratch must be reserved before graph capture");
     SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->gemv_scratch) hipFree(ctx->gemv_scratch);
+    if (ctx->gemv_scratch) (void)hipFree(ctx->gemv_scratch);
     ctx->gemv_scratch = nullptr; ctx->gemv_scratch_floats = 0;
     SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->gemv_scratch, floats * sizeof(float)));
     ctx->gemv_scratch_floats = floats;
@@ -289,7 +289,7 @@ int sampler_scratch_reserve(slai_ctx *ctx, size_t floats) {
     if (floats <= ctx->sampler_scratch_floats) return SLAI_OK;
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "sampler scratch must be reserved before graph capture");
     SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->sampler_scratch) hipFree(ctx->sampler_scratch);
+    if (ctx->sampler_scratch) (void)hipFree(ctx->sampler_scratch);
     ctx->sampler_scratch = nullptr; ctx->sampler_scratch_floats = 0;
     SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->sampler_scratch, floats * sizeof(float)));
     ctx->sampler_scratch_floats = floats;
@@ -567,7 +567,7 @@ int ensure_attn_scratch(slai_ctx *ctx, size_t floats) {
     if (floats <= ctx->attn_scratch_floats) return SLAI_OK;
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "attention scratch must be sized before graph capture");
     SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->attn_scratch) hipFree(ctx->attn_scratch);
+    if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
     ctx->attn_scratch = nullptr; ctx->attn_scratch_floats = 0;
     SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->attn_scratch, floats * sizeof(float)));
     ctx->attn_scratch_floats = floats;
@@ -677,7 +677,7 @@ SLAI_EXPORT int slai_graph_end_capture(slai_ctx *ctx, slai_graph **out) {
     hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
     if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
     if (e != hipSuccess) {
-        if (g->graph) hipGraphDestroy(g->graph);
+        if (g->graph) (void)hipGraphDestroy(g->graph);
         delete g;
         return hip_fail(ctx, e, "slai_graph_end_capture");
     }
@@ -691,8 +691,8 @@ SLAI_EXPORT int slai_graph_launch(slai_ctx *ctx, slai_graph *g) {
 }
 SLAI_EXPORT void slai_graph_destroy(slai_ctx *ctx, slai_graph *g) {
     if (!g) return;
-    if (ctx) hipStreamSynchronize(ctx->stream);
-    if (g->exec) hipGraphExecDestroy(g->exec);
-    if (g->graph) hipGraphDestroy(g->graph);
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
     delete g;
 }

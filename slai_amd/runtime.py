@@ -299,6 +299,15 @@ class Gguf:
     def version(self):
         return self.L.slai_gguf_version(self.h)
 
+    def metadata_debug_strings(self):
+        """gguf.rs:686-695."""
+        out = []
+        for i in range(self.L.slai_gguf_metadata_count(self.h)):
+            buf = C.create_string_buffer(512)
+            if self.L.slai_gguf_meta_describe(self.h, i, buf, 512) == 0:
+                out.append(buf.value.decode(errors="replace"))
+        return out
+
     def meta_array_str(self, key):
         """gguf.rs:316-322 ``as_string_array`` (as bytes objects)."""
         n = self.meta_array_len(key)

@@ -148,6 +148,10 @@ def test_dummy_gguf_string_array():
     keys = [k for k in ("some.parameter.arr.str", "arr.str") if _has(g, k)]
     assert keys, "the fixture's string array was not found"
     assert g.meta_array_str(keys[0]) == [b"hello", b"world", b"!"]
+    lines = g.metadata_debug_strings()
+    assert len(lines) == 15 and lines == sorted(lines)
+    assert any(l.endswith("= array[3]") for l in lines) and any('String("hello world")' in l for l in lines)
+    assert any(l.endswith("U8(18)") for l in lines)                 # some.parameter.uint8 = 0x12
     g.close()
 
 
