@@ -78,8 +78,8 @@ struct DevX {
 
 // Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product.
 template <int T, int N> struct UnitLoader {
-    static constexpr int DEPTH = 1;               // stages requested ahead of the one being multiplied
-    static constexpr int LEAD = 1;                // stages requested before the dot product starts (>= DEPTH)
+    static constexpr int DEPTH = 2;               // stages requested ahead of the one being multiplied
+    static constexpr int LEAD = 2;                // stages requested before the dot product starts (>= DEPTH)
     using F = Tiled<T>;
     const uint8_t *unit[N];                       // + lane * 16 already applied
     const uint8_t *tailp[N];
