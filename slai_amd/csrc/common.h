@@ -47,6 +47,9 @@ struct slai_ctx {
     size_t gemv_scratch_floats = 0;
     float *sampler_scratch = nullptr;   // probabilities of the device sampler (one float per vocabulary entry)
     size_t sampler_scratch_floats = 0;
+    uint32_t *handoff_counters = nullptr;   // q/k/v + attention in one launch: one 128-byte line per head, then a timeout flag
+    uint32_t handoff_heads = 0;
+    bool fuse_qkv_attention = true;     // SLAI_FUSE_QKV_ATTN=0: always separate launches
     // tuning knobs (environment overridable, see runtime.cpp)
     int gemv_rows_per_wg = 8;
     int gemv_max_threads = 1024;
@@ -181,7 +184,13 @@ bool gemv_is_rowtile(const slai_ctx *ctx, const slai_qmat *m);
 // The same for a SiLU-gated pair launched together (a gated Q8_0 pair needs too many registers there).
 bool gemv_gated_is_rowtile(const slai_ctx *ctx, const slai_qmat *gate, const slai_qmat *up);
 // Returns SLAI_OK or an error code with the message set on ctx.
-int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who);
+// `fused_attn`: also run this attention in the same launch (see launch_qkv_attention; the caller has checked
+// qkv_attention_fusable).
+struct AttnLaunch;
+int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunch *fused_attn = nullptr);
+bool qkv_attention_fusable(const slai_ctx *ctx, const slai_qmat *v, const slai_qmat *k, const slai_qmat *q, const AttnLaunch &a);
+int handoff_reserve(slai_ctx *ctx, uint32_t n_heads);   // not during graph capture
+int handoff_check(slai_ctx *ctx);                        // after a synchronize: error if a hand-off ever timed out
 // Makes sure the row-tile GEMV's scratch holds `floats` floats (call outside graph capture).
 int gemv_scratch_reserve(slai_ctx *ctx, size_t floats);
 int sampler_scratch_reserve(slai_ctx *ctx, size_t floats);   // grows the sampler's scratch; not during graph capture
@@ -252,6 +261,8 @@ struct AttnLaunch {
     uint32_t n_splits;
 };
 hipError_t launch_attention(hipStream_t s, const AttnLaunch &a);
+// q/k/v GEMV (three segments in the order v, k, q) and the attention over their results in one launch
+hipError_t launch_qkv_attention(slai_ctx *ctx, GemvRowtileParams p, const AttnLaunch &a);
 // out[i] = powf(base, -((2*i) % head_size) / head_size), i < head_size/2
 hipError_t launch_rope_theta(hipStream_t s, float *out, uint32_t head_size, float base);
 size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n_splits);

@@ -192,6 +192,7 @@ int slai_llama2::load(const slai_gguf *gg) {
     {   // activation slots of the 64-row-tile GEMV: the largest launch is q/k/v together, gate/up, or the output matrix
         const uint32_t t64 = std::max(std::max((dim + 63) / 64 + 2 * ((kvd + 63) / 64), (config.hidden_dim + 63) / 64), (config.vocab_size + 63) / 64);
         TRY(gemv_scratch_reserve(ctx, (size_t)t64 * (dim + dim / 16 + 16)));
+        TRY(handoff_reserve(ctx, config.n_q_heads));
     }
     // ---- Llama2State::new (transformer.rs:47-140); buffers are zero-initialised
     Llama2State &s = state;
@@ -279,6 +280,21 @@ int slai_llama2::enqueue_fused(int sampler) {
     const float *prepared = nullptr;                           // valid copy for the next consumer of x, or none
     for (uint32_t l = 0; l < config.n_layers; ++l) {
         const Llama2LayerWeights &wl = weights.layers[l];
+        // ---- bias + RoPE + cache write + attention (described first: it may join the q/k/v launch)
+        AttnLaunch a{};
+        a.q = q; a.kcache = s.key_cache[l].buf->dptr; a.vcache = s.value_cache[l].buf->dptr;
+        a.kv_f16 = kv_dtype == SLAI_KV_F16;
+        a.n_heads = config.n_q_heads; a.kv_mul = config.n_q_heads / config.n_kv_heads; a.head_size = head_size();
+        a.kv_dim = kvd; a.seq_len = config.seq_len;
+        a.pos_ptr = (const uint32_t *)&ds->pos;
+        a.knew = kcol; a.vnew = vcol;
+        a.qbias = wl.attn_q_bias.buf ? (const float *)wl.attn_q_bias.buf->dptr : nullptr;
+        a.kbias = wl.attn_k_bias.buf ? (const float *)wl.attn_k_bias.buf->dptr : nullptr;
+        a.vbias = wl.attn_v_bias.buf ? (const float *)wl.attn_v_bias.buf->dptr : nullptr;
+        a.rope_variant = rope_variant(); a.rope_base = config.rope_base_freq;
+        a.rope_theta = (const float *)s.rope_theta.buf->dptr;
+        a.out = xb; a.scratch = ctx->attn_scratch; a.n_splits = attn_splits;
+        bool attention_done = false;
         // ---- RMSNorm + Q/K/V projections: matrices of one format and layout share a launch
         {
             // V first: in the usual mixes it has the widest format, so its workgroups should be dispatched earliest
@@ -296,24 +312,16 @@ int slai_llama2::enqueue_fused(int sampler) {
                     c.m[c.nseg] = mats[j]; c.out[c.nseg] = outs[j]; ++c.nseg;
                     done[j] = true;
                 }
-                TRY(gemv_call(ctx, c, "llama2 qkv"));
+                // all three in one launch of 64-row tiles, one workgroup per head for the attention: one launch does both
+                if (c.nseg == 3 && qkv_attention_fusable(ctx, mats[0], mats[1], mats[2], a)) {
+                    TRY(gemv_call(ctx, c, "llama2 qkv + attention", &a));
+                    attention_done = true;
+                } else {
+                    TRY(gemv_call(ctx, c, "llama2 qkv"));
+                }
             }
         }
-        // ---- bias + RoPE + cache write + attention
-        {
-            AttnLaunch a{};
-            a.q = q; a.kcache = s.key_cache[l].buf->dptr; a.vcache = s.value_cache[l].buf->dptr;
-            a.kv_f16 = kv_dtype == SLAI_KV_F16;
-            a.n_heads = config.n_q_heads; a.kv_mul = config.n_q_heads / config.n_kv_heads; a.head_size = head_size();
-            a.kv_dim = kvd; a.seq_len = config.seq_len;
-            a.pos_ptr = (const uint32_t *)&ds->pos;
-            a.knew = kcol; a.vnew = vcol;
-            a.qbias = wl.attn_q_bias.buf ? (const float *)wl.attn_q_bias.buf->dptr : nullptr;
-            a.kbias = wl.attn_k_bias.buf ? (const float *)wl.attn_k_bias.buf->dptr : nullptr;
-            a.vbias = wl.attn_v_bias.buf ? (const float *)wl.attn_v_bias.buf->dptr : nullptr;
-            a.rope_variant = rope_variant(); a.rope_base = config.rope_base_freq;
-            a.rope_theta = (const float *)s.rope_theta.buf->dptr;
-            a.out = xb; a.scratch = ctx->attn_scratch; a.n_splits = attn_splits;
+        if (!attention_done) {
             hipError_t e = launch_attention(ctx->stream, a);
             if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "attention: unsupported head size or context length");
             SLAI_HIP_TRY(ctx, e);
@@ -460,6 +468,7 @@ SLAI_EXPORT int slai_llama2_forward_logits(slai_llama2 *m, uint32_t pos, uint32_
         TRY(m->enqueue_fused(false));
     }
     TRY(slai_synchronize(ctx));                                          // :219
+    TRY(handoff_check(ctx));
     if (logits_out) TRY(slai_read_buffer(ctx, s.logits.buf, 0, logits_out, (size_t)m->config.vocab_size * 4));   // :225-227
     return SLAI_OK;
 }
@@ -487,6 +496,7 @@ static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_le
         for (uint32_t i = 0; i < n_steps; ++i) TRY(m->enqueue_fused(mode));
         SLAI_HIP_TRY(ctx, hipEventRecord(L.ev1, ctx->stream));
         TRY(slai_synchronize(ctx));
+        TRY(handoff_check(ctx));
         if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, L.ev0, L.ev1));
         return slai_read_buffer(ctx, L.out_tokens, 0, out_tokens, (size_t)n_steps * 4);
     }
@@ -504,6 +514,7 @@ static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_le
     for (uint32_t i = 0; i < n_steps; ++i) TRY(slai_graph_launch(ctx, graph));         // chat_llama2.rs:109 loop
     SLAI_HIP_TRY(ctx, hipEventRecord(L.ev1, ctx->stream));
     TRY(slai_synchronize(ctx));
+    TRY(handoff_check(ctx));
     if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, L.ev0, L.ev1));
     return slai_read_buffer(ctx, L.out_tokens, 0, out_tokens, (size_t)n_steps * 4);
 }

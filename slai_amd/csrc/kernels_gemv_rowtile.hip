@@ -17,6 +17,7 @@
 // One workgroup = one tile = 64 complete output rows; wave w owns super-blocks w, w+NW, ...; partial
 // sums meet in LDS once.  Segments of one launch may differ in block format (Q4_K q/k with a Q6_K v).
 #include "common.h"
+#include "attention_fast.h"
 #include "device_util.h"
 #include "quant_tiled.h"
 
@@ -270,6 +271,67 @@ __global__ void __launch_bounds__(1024) gemv_rowtile_kernel(const GemvRowtilePar
     }
 }
 
+// ---- q/k/v projections and attention in ONE launch ----------------------------------------------------------------
+// For layers with as many kv heads as q heads, head size 128 and a context served by one workgroup per head.  The six
+// 64-row tiles that make up a head's q, k and v (two each; segments in the order v, k, q) go to six workgroups of the
+// SAME XCD: workgroup i runs on XCD i % 8, so head h = (i % 8) + 8 * ((i / 8) / 6) takes the workgroups i = (h % 8) +
+// 8 * (6 * (h / 8) + t), t = 0..5.  Each writes its 64 results, waits until the stores have reached the XCD's L2
+// (s_waitcnt vmcnt(0)) and bumps the head's counter with an atomic that executes in that L2.  The workgroup of the last
+// tile (t = 5) then runs the attention of the head: it requests the cache rows first, spins on the counter until all six
+// tiles are in, and reads q, k, v from L2.  Its five producers have smaller indices and are therefore dispatched before
+// it, so it never waits for a workgroup that has no compute unit.  The spin is bounded: if the counter does not fill
+// (it always has) the workgroup sets counters[timeout_slot] and goes on.
+constexpr uint32_t HANDOFF_SPIN_LIMIT = 1u << 24;
+
+template <bool F16, bool PREP>
+__global__ void __launch_bounds__(512) qkv_attention_kernel(const GemvRowtileParams p, const AttnLaunch a, uint32_t *counters, uint32_t timeout_slot) {
+    extern __shared__ float smem[];
+    const int NW = blockDim.x >> 6;
+    float *partial = smem;
+    float *red = smem + (size_t)NW * 64;
+    touch_kernel_arguments<((sizeof(GemvRowtileParams) + 63) / 64 + (sizeof(AttnLaunch) + 63) / 64) * 64>();
+    const uint32_t i = blockIdx.x, j = i >> 3, t = j % 6;
+    const uint32_t h = (i & 7u) + 8u * (j / 6);
+    const int s = (int)(t >> 1);
+    const uint32_t tile = 2 * h + (t & 1u);
+    GemvRowtileSeg seg;
+    seg.W = s == 0 ? p.seg[0].W : (s == 1 ? p.seg[1].W : p.seg[2].W);
+    seg.W2 = nullptr;
+    seg.type = s == 0 ? p.seg[0].type : (s == 1 ? p.seg[1].type : p.seg[2].type);
+    seg.nrows = s == 0 ? p.seg[0].nrows : (s == 1 ? p.seg[1].nrows : p.seg[2].nrows);
+    seg.out = s == 0 ? p.seg[0].out : (s == 1 ? p.seg[1].out : p.seg[2].out);
+    seg.bias = s == 0 ? p.seg[0].bias : (s == 1 ? p.seg[1].bias : p.seg[2].bias);
+    seg.flags = s == 0 ? p.seg[0].flags : (s == 1 ? p.seg[1].flags : p.seg[2].flags);
+    switch (seg.type) {                                        // uniform over the workgroup
+    case T_Q4_K: tile_body<T_Q4_K, false, PREP>(p, seg, tile, partial, red); break;
+    case T_Q6_K: tile_body<T_Q6_K, false, PREP>(p, seg, tile, partial, red); break;
+    case T_Q5_K: tile_body<T_Q5_K, false, PREP>(p, seg, tile, partial, red); break;
+    default: break;
+    }
+    uint32_t *counter = counters + (size_t)h * 32;             // one 128-byte line per head
+    if (threadIdx.x < 64) {                                    // the wave that wrote the tile's results
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (threadIdx.x == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    if (t != 5) return;
+    attn::attn_fast_body<F16, 512, 128, true, true>(a, h, 0u, threadIdx.x, [&]() {
+        if (threadIdx.x == 0) {
+            uint32_t seen = 0, spins = 0;
+            do {
+                // a read-modify-write that returns the value: it executes in the L2 (the compiler would turn an
+                // atomic add of 0 into a load, which may be served by this compute unit's own cache for ever)
+                const uint32_t zero = 0;
+                asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=&v"(seen) : "v"(counter), "v"(zero) : "memory");
+                ++spins;
+            } while (seen < 6u && spins < HANDOFF_SPIN_LIMIT);
+            if (seen < 6u) counters[timeout_slot] = 1u;
+            *counter = 0u;                                     // for the next launch; nobody else touches it any more
+        }
+        __syncthreads();
+        asm volatile("" ::: "memory");
+    });
+}
+
 template <int TT, bool DUAL>
 hipError_t go(const GemvRowtileParams &p, uint32_t tiles, int NT, size_t smem, hipStream_t s) {
     if (p.prepared) gemv_rowtile_kernel<TT, DUAL, true><<<tiles, NT, smem, s>>>(p);
@@ -322,6 +384,36 @@ hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p) {
     case T_Q5_K: return dual ? go<T_Q5_K, true>(p, tiles, NT, smem, st) : go<T_Q5_K, false>(p, tiles, NT, smem, st);
     default: return dual ? go<0, true>(p, tiles, NT, smem, st) : go<0, false>(p, tiles, NT, smem, st);
     }
+}
+
+hipError_t launch_qkv_attention(slai_ctx *ctx, GemvRowtileParams p, const AttnLaunch &a) {
+    if (p.nseg != 3 || p.ncb == 0 || p.ncb > 16 || p.ncols != p.ncb * 256) return hipErrorInvalidValue;
+    if (a.head_size != 128 || a.kv_mul != 1 || a.n_splits != 1 || a.n_heads % 8 || a.kv_dim % 8 || !a.knew || !a.vnew || !ctx->handoff_counters ||
+        a.n_heads > ctx->handoff_heads)
+        return hipErrorInvalidValue;
+    for (int i = 0; i < 3; ++i) {
+        const int t = p.seg[i].type;
+        if ((t != T_Q4_K && t != T_Q6_K && t != T_Q5_K) || p.seg[i].nrows != a.n_heads * 128 || p.seg[i].W2 || (p.seg[i].flags & GEMV_SILU_GATE))
+            return hipErrorInvalidValue;
+        p.seg[i].ntiles = p.seg[i].nrows / 64;
+    }
+    // eight waves: what the attention part uses, and 256 registers per lane for it; a wave then walks two super-blocks
+    const int NW = 8;
+    if (p.ncb < 8) return hipErrorInvalidValue;                 // (narrower models take the separate kernels)
+    p.scratch_stride = p.ncols + p.ncols / 16;
+    const size_t smem = ((size_t)NW * 64 + NW) * sizeof(float);
+    const uint32_t grid = a.n_heads * 6;
+    const int NT = NW * 64;
+    uint32_t *c = ctx->handoff_counters;
+    const uint32_t slot = ctx->handoff_heads * 32;
+    if (a.kv_f16) {
+        if (p.prepared) qkv_attention_kernel<true, true><<<grid, NT, smem, ctx->stream>>>(p, a, c, slot);
+        else qkv_attention_kernel<true, false><<<grid, NT, smem, ctx->stream>>>(p, a, c, slot);
+    } else {
+        if (p.prepared) qkv_attention_kernel<false, true><<<grid, NT, smem, ctx->stream>>>(p, a, c, slot);
+        else qkv_attention_kernel<false, false><<<grid, NT, smem, ctx->stream>>>(p, a, c, slot);
+    }
+    return hipGetLastError();
 }
 
 }  // namespace slai

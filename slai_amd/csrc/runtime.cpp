@@ -82,6 +82,7 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->gemv_max_wgs = env_int("SLAI_GEMV_MAX_WGS", 512);
     ctx->tiled_layout = env_int("SLAI_TILED", 1) != 0;
     ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
+    ctx->fuse_qkv_attention = env_int("SLAI_FUSE_QKV_ATTN", 1) != 0;
     *out = ctx;
     return SLAI_OK;
 }
@@ -93,6 +94,7 @@ SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
     if (ctx->gemv_scratch) (void)hipFree(ctx->gemv_scratch);
     if (ctx->sampler_scratch) (void)hipFree(ctx->sampler_scratch);
+    if (ctx->handoff_counters) (void)hipFree(ctx->handoff_counters);
     if (ctx->timer0) (void)hipEventDestroy(ctx->timer0);
     if (ctx->timer1) (void)hipEventDestroy(ctx->timer1);
     (void)hipStreamDestroy(ctx->stream);
@@ -285,6 +287,36 @@ int gemv_scratch_reserve(slai_ctx *ctx, size_t floats) {
     return SLAI_OK;
 }
 
+bool qkv_attention_fusable(const slai_ctx *ctx, const slai_qmat *v, const slai_qmat *k, const slai_qmat *q, const AttnLaunch &a) {
+    if (!ctx->fuse_qkv_attention || !ctx->handoff_counters || a.n_heads > ctx->handoff_heads) return false;
+    if (a.head_size != 128 || a.kv_mul != 1 || a.n_splits != 1 || a.n_heads % 8 || a.kv_dim % 8 || !a.knew || !a.vnew) return false;
+    for (const slai_qmat *m : {v, k, q}) {
+        if (!gemv_is_rowtile(ctx, m) || m->ncb != 16 || m->nrows != a.n_heads * 128u) return false;
+        if (m->type != T_Q4_K && m->type != T_Q6_K && m->type != T_Q5_K) return false;
+    }
+    return true;
+}
+// Allocated once per context and never moved (captured graphs hold the address): models with more heads than the
+// first reservation allows simply keep separate launches.
+int handoff_reserve(slai_ctx *ctx, uint32_t n_heads) {
+    if (ctx->handoff_counters) return SLAI_OK;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "hand-off counters must be reserved before graph capture");
+    if (n_heads < 256) n_heads = 256;
+    const size_t bytes = ((size_t)n_heads * 32 + 32) * sizeof(uint32_t);
+    SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->handoff_counters, bytes));
+    SLAI_HIP_TRY(ctx, hipMemsetAsync(ctx->handoff_counters, 0, bytes, ctx->stream));
+    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    ctx->handoff_heads = n_heads;
+    return SLAI_OK;
+}
+int handoff_check(slai_ctx *ctx) {
+    if (!ctx->handoff_counters) return SLAI_OK;
+    uint32_t flag = 0;
+    SLAI_HIP_TRY(ctx, hipMemcpy(&flag, ctx->handoff_counters + (size_t)ctx->handoff_heads * 32, sizeof flag, hipMemcpyDeviceToHost));
+    if (flag) return set_error(ctx, SLAI_E_HIP, "q/k/v -> attention hand-off timed out inside a launch; results are invalid");
+    return SLAI_OK;
+}
+
 int sampler_scratch_reserve(slai_ctx *ctx, size_t floats) {
     if (floats <= ctx->sampler_scratch_floats) return SLAI_OK;
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "sampler scratch must be reserved before graph capture");
@@ -296,7 +328,7 @@ int sampler_scratch_reserve(slai_ctx *ctx, size_t floats) {
     return SLAI_OK;
 }
 
-int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who) {
+int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunch *fused_attn) {
     const slai_qmat *m0 = c.m[0];
     if (!m0 || c.nseg < 1 || c.nseg > 3) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": bad GEMV call");
     // 64-row tiles: wave-uniform activations, formats may differ between the segments
@@ -327,11 +359,12 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who) {
             if (rc) return rc;
             p.scratch = ctx->gemv_scratch;
         }
-        hipError_t e = launch_gemv_rowtile(ctx, p);
+        hipError_t e = fused_attn ? launch_qkv_attention(ctx, p, *fused_attn) : launch_gemv_rowtile(ctx, p);
         if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported shape for the row-tile GEMV");
         if (e != hipSuccess) return hip_fail(ctx, e, who);
         return SLAI_OK;
     }
+    if (fused_attn) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": attention can only join a 64-row-tile launch");
     for (int i = 0; i < c.nseg; ++i) {
         const slai_qmat *m = c.m[i], *m2 = c.m2[i];
         if (!m || m->type != m0->type || m->ncols != m0->ncols || m->tiled != m0->tiled ||
