@@ -212,6 +212,8 @@ hipError_t launch_embed(hipStream_t s, const slai_qmat *a, const int *row_a, con
 
 // ---- element-wise / normalisation ops -------------------------------------------------
 struct VecView { float *p; uint32_t n; uint32_t stride; };  // element i at p[i*stride]
+// out[i] = id of the XCD workgroup i of a launch of n_workgroups runs on
+hipError_t launch_xcd_of_workgroup(hipStream_t s, uint32_t *out, uint32_t n_workgroups);
 hipError_t launch_rms_norm(hipStream_t s, VecView out, VecView v, VecView w, const float *eps_ptr, float eps);
 hipError_t launch_layernorm(hipStream_t s, VecView out, VecView v, float eps);
 hipError_t launch_binop(hipStream_t s, int op /*0 add,1 mul,2 copy(a<-b)*/, VecView a, VecView b);

@@ -242,10 +242,21 @@ __global__ void store_kv_kernel(const float *src, void *dst, uint32_t n, int f16
     else reinterpret_cast<float *>(dst)[i] = src[i];
 }
 
+// which XCD each workgroup of a launch runs on (hardware id register)
+__global__ void xcd_of_workgroup_kernel(uint32_t *out) {
+    uint32_t v;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+    if (threadIdx.x == 0) out[blockIdx.x] = v & 0xfu;
+}
+
 inline uint32_t grid_for(uint32_t n, uint32_t block) { uint32_t g = (n + block - 1) / block; return g ? (g > 4096 ? 4096 : g) : 1; }
 
 }  // namespace
 
+hipError_t launch_xcd_of_workgroup(hipStream_t s, uint32_t *out, uint32_t n_workgroups) {
+    xcd_of_workgroup_kernel<<<n_workgroups, 64, 0, s>>>(out);
+    return hipGetLastError();
+}
 hipError_t launch_store_kv(hipStream_t s, const float *src, void *dst, uint32_t n, int f16) {
     store_kv_kernel<<<(n + 255) / 256, 256, 0, s>>>(src, dst, n, f16);
     return hipGetLastError();

@@ -304,6 +304,14 @@ int handoff_reserve(slai_ctx *ctx, uint32_t n_heads) {
     if (n_heads < 256) n_heads = 256;
     const size_t bytes = ((size_t)n_heads * 32 + 32) * sizeof(uint32_t);
     SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->handoff_counters, bytes));
+    // The hand-off relies on workgroup i running on XCD i mod 8 (workgroups with equal i mod 8 then share an L2):
+    // look before relying on it, and keep separate launches on a device that places workgroups differently.
+    uint32_t where[192];
+    SLAI_HIP_TRY(ctx, launch_xcd_of_workgroup(ctx->stream, ctx->handoff_counters, 192));
+    SLAI_HIP_TRY(ctx, hipMemcpyAsync(where, ctx->handoff_counters, sizeof where, hipMemcpyDeviceToHost, ctx->stream));
+    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    for (uint32_t i = 8; i < 192; ++i)
+        if (where[i] != where[i % 8]) ctx->fuse_qkv_attention = false;
     SLAI_HIP_TRY(ctx, hipMemsetAsync(ctx->handoff_counters, 0, bytes, ctx->stream));
     SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     ctx->handoff_heads = n_heads;
