@@ -331,7 +331,7 @@ class Gguf:
         for i in range(self.L.slai_gguf_tensor_count(self.h)):
             name, dims, t, off = C.c_char_p(), (C.c_uint64 * 4)(), C.c_uint32(), C.c_uint64()
             self.L.slai_gguf_tensor_info(self.h, i, C.byref(name), C.byref(dims), C.byref(t), C.byref(off))
-            out[name.value.decode()] = dict(dims=list(dims), type=t.value, offset=off.value)
+            out[name.value.decode(errors="replace")] = dict(dims=list(dims), type=t.value, offset=off.value)
         return out
 
     def meta_u32(self, key):
