@@ -38,7 +38,7 @@ template <> struct KV<false> {
     __device__ static void store(T *p, float v) { *p = v; }
 };
 
-// ---- the same computation for head sizes 64 and 128, organised around 16-byte loads with many of them in flight:
+// ---- the same computation for head sizes 64 and 128, built on 16-byte loads with many of them in flight:
 // scores with 4 lanes per position (each lane a contiguous quarter of the head), values with one lane per 8
 // elements.  Every wave runs a softmax of its own over the positions it owns (running max and rescaling), so the
 // only workgroup barriers are the one after q is rotated and the one before the waves are merged.  NT = 512 serves
