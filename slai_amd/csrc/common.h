@@ -120,6 +120,9 @@ struct GemvTiledParams {
     GemvTiledSeg seg[3];
     int nseg = 1;
     uint32_t ncols = 0, ncb = 0, ngroups = 0, rows_log2 = 4, unit_bytes = 0;
+    // A workgroup has one wave per column group, at most 16: wider matrices take several launches, each over the
+    // groups [group0, group0 + launch_groups) and all but the first accumulating into the output.
+    uint32_t group0 = 0, launch_groups = 0;   // launch_groups = 0: all of them
     const float *x = nullptr;
     int prologue = PRO_NONE;
     const float *norm_w = nullptr, *norm_b = nullptr;

@@ -168,7 +168,8 @@ int slai_llama2::load(const slai_gguf *gg) {
         TRY(f32_vector_from_gguf(ctx, g, p + "attn_k.bias", false, &w.attn_k_bias));
         TRY(f32_vector_from_gguf(ctx, g, p + "attn_v.bias", false, &w.attn_v_bias));
         TRY(qmat_from_gguf(ctx, gg, p + "attn_output.weight", &w.attn_output));
-        TRY(qmat_from_gguf(ctx, gg, p + "ffn_down.weight", &w.ffn_down));
+        // (explicit 16-row tiles: a feed-forward width beyond 16384 then still gets the tiled layout, in column slices)
+        TRY(qmat_from_gguf(ctx, gg, p + "ffn_down.weight", &w.ffn_down, SLAI_LAYOUT_TILE16));
         TRY(qmat_from_gguf(ctx, gg, p + "ffn_gate.weight", &w.ffn_gate, SLAI_LAYOUT_TILE64));
         TRY(qmat_from_gguf(ctx, gg, p + "ffn_up.weight", &w.ffn_up, SLAI_LAYOUT_TILE64));
         TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.weight", true, &w.ffn_norm));

@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     const uint32_t step = seg.nblocks;
 
     // ---- requests first: activations (small, cache resident), then the first tile's weights --------
-    const uint32_t g = wave;                                 // column group owned by this wave
+    const uint32_t g = p.group0 + wave;                      // column group owned by this wave
     const uint32_t cb = g * KQ + kq;
     const bool valid = cb < p.ncb;
     const size_t xoff = (size_t)(valid ? cb : 0) * 256 + lane16;
@@ -278,11 +278,14 @@ hipError_t go(hipStream_t s, const GemvTiledParams &p, dim3 grid, int NT, size_t
 }
 
 template <int T> hipError_t launch_t(slai_ctx *ctx, GemvTiledParams &p) {
-    if (p.ngroups == 0 || p.ngroups > 16) return hipErrorInvalidValue;
+    if (p.launch_groups == 0) p.launch_groups = p.ngroups;
+    if (p.ngroups == 0 || p.launch_groups > 16 || p.group0 + p.launch_groups > p.ngroups) return hipErrorInvalidValue;
+    // a partial launch cannot normalise its input (that needs every column) or apply a non-linear epilogue
+    if (p.launch_groups != p.ngroups && p.prologue != PRO_NONE) return hipErrorInvalidValue;
     for (int i = 0; i < p.nseg; ++i)
         if ((p.seg[i].flags & GEMV_EMIT) && (i != 0 || !p.emit_w || !p.emit_out || p.seg[i].nrows % 16 || (p.seg[i].flags & GEMV_SILU_GATE)))
             return hipErrorInvalidValue;
-    const int NT = (int)p.ngroups * 64;
+    const int NT = (int)p.launch_groups * 64;
     const uint32_t rows = 1u << p.rows_log2;
     bool dual = false;
     uint32_t total_tiles = 0;

@@ -5,6 +5,7 @@
 #include "quant_formats.h"
 #include "quant_tiled.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -207,7 +208,9 @@ SLAI_EXPORT int slai_qmat_create_layout(slai_ctx *ctx, uint32_t ggml_type, uint3
         bool tile64 = layout == SLAI_LAYOUT_TILE64 || (layout == SLAI_LAYOUT_AUTO && nrows >= 8192 && nrows % 64 == 0 && ncb <= 16);
         if (!ctx->rowtile_gemv || ncb > 64) tile64 = false;
         const TiledGeom g = tiled_geom(t, nrows, ncols, tile64 ? 6u : 0u);
-        if (g.ngroups <= 16 || tile64) {
+        // more than 16 column groups (over 16384 columns in 16-row tiles): only on request, the GEMV then takes several
+        // launches and supports neither a normalisation prologue nor a non-linear epilogue
+        if (g.ngroups <= 16 || tile64 || (layout == SLAI_LAYOUT_TILE16 && g.ngroups <= 64)) {
             m->tiled = true; m->rows_log2 = g.rows_log2; m->ncb = g.ncb; m->ngroups = g.ngroups; m->ntiles = g.ntiles;
             m->unit_bytes = g.unit_bytes; m->bytes = tiled_bytes(g);
         }
@@ -267,7 +270,7 @@ SLAI_EXPORT int slai_qmat_dequantize(slai_ctx *ctx, const slai_qmat *m, uint32_t
 
 // ---- GEMV dispatch over the two weight layouts ------------------------------------------------
 namespace slai {
-bool gemv_can_emit(const slai_qmat *m) { return m && m->tiled && m->rows_log2 != 6 && m->ngroups <= 16 && m->nrows % 16 == 0; }
+bool gemv_can_emit(const slai_qmat *m) { return m && m->tiled && m->rows_log2 != 6 && m->ngroups <= 64 && m->nrows % 16 == 0; }
 bool gemv_is_rowtile(const slai_ctx *ctx, const slai_qmat *m) {
     return ctx->rowtile_gemv && m && m->tiled && m->rows_log2 == 6 && m->ncb <= 64;
 }
@@ -376,7 +379,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunc
     for (int i = 0; i < c.nseg; ++i) {
         const slai_qmat *m = c.m[i], *m2 = c.m2[i];
         if (!m || m->type != m0->type || m->ncols != m0->ncols || m->tiled != m0->tiled ||
-            (m->tiled && (m->rows_log2 != m0->rows_log2 || m->ngroups > 16)))
+            (m->tiled && (m->rows_log2 != m0->rows_log2 || m->ngroups > 64)))
             return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": matrices of one launch must share format, width and layout");
         if (m2 && (m2->type != m->type || m2->ncols != m->ncols || m2->nrows != m->nrows || m2->tiled != m->tiled ||
                    (m->tiled && m2->rows_log2 != m->rows_log2)))
@@ -393,7 +396,27 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunc
             p.seg[i].W = c.m[i]->dptr; p.seg[i].W2 = c.m2[i] ? c.m2[i]->dptr : nullptr; p.seg[i].nrows = c.m[i]->nrows;
             p.seg[i].out = c.out[i]; p.seg[i].bias = c.bias[i]; p.seg[i].flags = c.flags[i];
         }
-        e = launch_gemv_tiled(ctx, m0->type, p);
+        if (m0->ngroups <= 16) {
+            e = launch_gemv_tiled(ctx, m0->type, p);
+        } else {
+            // wide matrix: balanced slices of at most 16 column groups, one launch each; the first writes (or adds to
+            // the residual), the others accumulate, the last one emits
+            if (c.prologue != PRO_NONE) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": no normalisation prologue over more than 16384 columns in 16-row tiles");
+            for (int i = 0; i < c.nseg; ++i)
+                if (c.flags[i] & (GEMV_GELU | GEMV_SILU_GATE)) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": no non-linear epilogue over more than 16384 columns in 16-row tiles");
+            const uint32_t nchunks = (m0->ngroups + 15) / 16, per = (m0->ngroups + nchunks - 1) / nchunks;
+            e = hipSuccess;
+            for (uint32_t k = 0; k < nchunks && e == hipSuccess; ++k) {
+                GemvTiledParams q = p;
+                q.group0 = k * per;
+                q.launch_groups = std::min(per, m0->ngroups - q.group0);
+                for (int i = 0; i < c.nseg; ++i) {
+                    if (k > 0) { q.seg[i].flags = (q.seg[i].flags | GEMV_ACCUM) & ~GEMV_BIAS; }
+                    if (k + 1 < nchunks) q.seg[i].flags &= ~GEMV_EMIT;
+                }
+                e = launch_gemv_tiled(ctx, m0->type, q);
+            }
+        }
     } else {
         if (!gemv_supports(m0->type, m0->ncols)) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported column count for this format");
         GemvParams p;

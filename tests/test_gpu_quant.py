@@ -281,3 +281,38 @@ def test_prepared_activations_chain(backend, oracle_lib, t):
         gprep2.destroy()
     for o in (down, gate, up, gnw, gprep, ghb, gx, gh):
         o.destroy()
+
+
+@pytest.mark.parametrize("t", [12, 14, 8], ids=lambda t: NAMES[t])
+def test_wide_matrix_in_16_row_tiles_takes_several_launches(backend, oracle_lib, t):
+    """More than 16384 columns in 16-row tiles (a feed-forward width like 18944): the GEMV runs as several launches over
+    column slices.  Plain product, residual accumulate with the prepared copy emitted by the last slice, and bit-exact
+    dequantisation of the layout."""
+    import os
+    if os.environ.get("SLAI_TILED") == "0":
+        pytest.skip("needs the tiled layouts")
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
+    nrows, ncols = 272, 18944                                  # 74 super-blocks -> 19 column groups -> two launches
+    ctxt = LlmContext(backend)
+    raw = synth.normal_quantized(900 + t, t, nrows, ncols, 0.02)
+    w = oracle_deq(oracle_lib, t, raw, nrows * ncols).reshape(nrows, ncols)
+    m = GpuQuantMatrix(backend, t, nrows, ncols, raw, layout=2)
+    assert np.array_equal(m.dequantize().view(np.uint32), w.view(np.uint32))
+    hv = synth.normal(5, ncols, 1.0)
+    ref = np.empty(nrows, np.float32)
+    oracle_lib.slo_gemv(ref.ctypes.data, w.ctypes.data, hv.ctypes.data, nrows, ncols)
+    gh, out = GpuTensor.vector(backend, hv), GpuTensor(backend, nrows)
+    out.write(np.full(nrows, 7.0, np.float32))                 # must be overwritten, not added to
+    ctxt.matmul_quant_assign(out, m, gh)
+    assert rel_err(out.read(), ref) < 1e-4
+    x0 = synth.normal(6, nrows, 1.0)
+    nw = (1.0 + synth.normal(7, nrows, 0.1)).astype(np.float32)
+    gx, gnw, gprep = GpuTensor.vector(backend, x0), GpuTensor.vector(backend, nw), GpuTensor(backend, nrows + nrows // 16)
+    ctxt.matmul_quant_add_assign_emit(gx, m, gh, gnw, gprep)
+    got = gx.read()
+    assert rel_err(got, x0 + ref) < 1e-4
+    prep = gprep.read()
+    assert rel_err(prep[:nrows], got * nw) < 1e-6
+    assert rel_err(prep[nrows:], (got * nw).reshape(-1, 16).sum(axis=1)) < 1e-5
+    for o in (m, gh, out, gx, gnw, gprep):
+        o.destroy()
