@@ -245,7 +245,8 @@ hipError_t launch_argmax(hipStream_t s, const float *v, uint32_t n, int *out_ind
                          const int *prompt, int *out_tokens);
 // models/sampler.rs:33-53 `Sampler::sample` with the draw `coin` in [0, 1) given (or, with `decode`, derived from the
 // state's seed and position; temperature and topp then come from the state as well)
-// `scratch`: n floats of device memory for the probabilities
+// `scratch`: sample_scratch_floats(n) floats of device memory
+size_t sample_scratch_floats(uint32_t n);
 hipError_t launch_sample(hipStream_t s, const float *v, uint32_t n, float temperature, float topp, float coin, float *scratch, int *out_index,
                          DecodeState *decode, const int *prompt, int *out_tokens);
 

@@ -481,7 +481,7 @@ static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_le
                          uint32_t start_pos, uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms, const SamplingParams *sampling = nullptr) {
     if (sampling && !(sampling->temperature >= 0.0f)) return set_error(ctx, SLAI_E_ARG, "generate: the temperature must not be negative");
     const int mode = sampling ? 2 : 1;
-    if (sampling) TRY(sampler_scratch_reserve(ctx, vocab));
+    if (sampling) TRY(sampler_scratch_reserve(ctx, sample_scratch_floats(vocab)));
     if (!prompt || !out_tokens || n_prompt == 0 || start_pos >= n_prompt) return set_error(ctx, SLAI_E_ARG, "generate: bad prompt / start position");
     if (n_steps == 0) return SLAI_OK;
     if (start_pos + n_steps > seq_len) return set_error(ctx, SLAI_E_SHAPE, "generate: would run past the context length");

@@ -388,6 +388,8 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *__restrict__ v,
         for (int w = 0; w < NW; ++w) S += sh.red[w];
         __syncthreads();
         D.kmax = __float_as_uint(1.0f / S);                 // the maximum's exponential is exp(0) = 1
+        const float cutoff_all = (1.0f - topp) / ((float)n - 1.0f);     // sampler.rs:93 (only meaningful with top-p)
+        uint32_t candidates = 0;
         if constexpr (R > 0) {
 #pragma unroll
             for (int k = 0; k < R; ++k) D.r[k] = D.r[k] / S;
@@ -397,7 +399,12 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *__restrict__ v,
 #pragma unroll
                 for (int u = 0; u < UNROLL; ++u) { const uint32_t i = D.index(k0 + u); e[u] = i < n ? pbuf[i] : 0.0f; }
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) { const uint32_t i = D.index(k0 + u); if (i < n) pbuf[i] = e[u] / S; }
+                for (int u = 0; u < UNROLL; ++u) {
+                    const uint32_t i = D.index(k0 + u);
+                    const float pv = e[u] / S;
+                    if (i < n) pbuf[i] = pv;
+                    candidates += (uint32_t)__popcll(__ballot(i < n && pv >= cutoff_all));   // (wave-uniform) for the top-p search
+                }
             }
         }
         if (topp <= 0.0f || topp >= 1.0f) {
@@ -432,6 +439,43 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *__restrict__ v,
         } else {
             // ---- sampler.rs:85-131 `sample_topp`
             const float cutoff = (1.0f - topp) / ((float)n - 1.0f);
+            if constexpr (R == 0) {
+                // A large vocabulary: the candidates (p >= cutoff, sampler.rs:93-103) are first packed, in index order,
+                // behind the probabilities in the scratch; when at most 32768 are left (any distribution a model
+                // produces in practice) the search runs over them in registers instead of re-reading the whole
+                // vocabulary in every pass.
+                float *cp = pbuf + (size_t)NW * slice;                         // packed probabilities
+                uint32_t *ci = reinterpret_cast<uint32_t *>(cp + (size_t)NW * slice);   // and their vocabulary indices
+                if (lane == 0) sh.redu[wave] = candidates;                     // counted while the probabilities were written
+                __syncthreads();
+                uint32_t at = 0, n0 = 0;
+                for (uint32_t w = 0; w < NW; ++w) { if (w < wave) at += sh.redu[w]; n0 += sh.redu[w]; }
+                __syncthreads();
+                if (n0 <= NW * 64 * 32) {
+                    for_each_prob(D, [&](float p, uint32_t i) {
+                        const bool on = i < n && p >= cutoff;
+                        const unsigned long long mask = __ballot(on);
+                        if (on) {
+                            const uint32_t pos = at + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+                            cp[pos] = p; ci[pos] = i;
+                        }
+                        at += (uint32_t)__popcll(mask);
+                    });
+                    __syncthreads();                                           // other waves read what this one packed
+                    Dist<32> C;
+                    C.p = cp; C.n = n0; C.kmax = D.kmax;
+                    C.base = wave * (64u * 32u) + lane; C.iters = 32;
+#pragma unroll
+                    for (int k = 0; k < 32; ++k) { const uint32_t i = C.index(k); C.r[k] = i < n0 ? cp[i] : 0.0f; }
+                    const Cross nucleus = crossing(C, cutoff, topp, sh);
+                    const float r = coin * nucleus.cum;
+                    Cross pick = crossing(C, cutoff, r, sh);
+                    if (pick.position > nucleus.position) pick = nucleus;
+                    uint32_t slot = pick.index != 0xffffffffu ? pick.index : locate(C, cutoff, pick.key, pick.j, sh);
+                    chosen = slot < n0 ? ci[slot] : besti;
+                    goto picked;
+                }
+            }
             const Cross nucleus = crossing(D, cutoff, topp, sh);
             const float r = coin * nucleus.cum;
             Cross pick = crossing(D, cutoff, r, sh);
@@ -440,6 +484,7 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *__restrict__ v,
             if (chosen == 0xffffffffu) chosen = besti;          // not reachable with finite logits; keeps the id valid
         }
     }
+picked:
     if (threadIdx.x == 0) {
         int next = (int)chosen;
         if (out_index) *out_index = next;
@@ -455,6 +500,14 @@ __global__ void __launch_bounds__(NT) sample_kernel(const float *__restrict__ v,
 }
 
 }  // namespace
+
+// floats of scratch a launch over n logits needs: none below 32769, else the probabilities and the packed candidates
+// (probabilities + indices), each padded to the slices of the 16 waves
+size_t sample_scratch_floats(uint32_t n) {
+    if (n <= NW * 64 * 32) return 1;
+    const size_t slice = ((size_t)(n + NW - 1) / NW + 64 * UNROLL - 1) / (64 * UNROLL) * (64 * UNROLL);
+    return 3 * NW * slice;
+}
 
 hipError_t launch_sample(hipStream_t s, const float *v, uint32_t n, float temperature, float topp, float coin, float *scratch, int *out_index,
                          DecodeState *decode, const int *prompt, int *out_tokens) {

@@ -691,7 +691,7 @@ SLAI_EXPORT int slai_sample(slai_ctx *ctx, slai_view logits, float temperature, 
     NEED_VEC(logits, "logits", vl);
     if (vl.stride != 1 || out_index->dtype != SLAI_DT_I32 || out_index->bytes < 4) return set_error(ctx, SLAI_E_SHAPE, "slai_sample: contiguous logits and an I32 output are required");
     if (!(temperature >= 0.0f) || !(coin >= 0.0f && coin < 1.0f)) return set_error(ctx, SLAI_E_ARG, "slai_sample: temperature must be >= 0 and the draw in [0, 1)");
-    if (int rc = sampler_scratch_reserve(ctx, vl.n)) return rc;
+    if (int rc = sampler_scratch_reserve(ctx, sample_scratch_floats(vl.n))) return rc;
     SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, vl.p, vl.n, temperature, topp, coin, ctx->sampler_scratch, (int *)out_index->dptr, nullptr, nullptr,
                                     nullptr));
     return SLAI_OK;
