@@ -76,12 +76,14 @@ template <> struct Vec8<false> {  // 8 f32 = 32 bytes
 // others must have left the kernel).  `wait_inputs()` is called once, by every thread, before q / knew / vnew are read:
 // a launch in which this workgroup's inputs are produced by other workgroups of the same launch blocks there (FUSED:
 // the requests for the cache, which depend on nothing but the position, then go first).
-template <bool F16, int NT, int HS, bool SINGLE, bool FUSED, class Wait>
+template <bool F16, int NT, int HS, bool SINGLE, bool FUSED, int KL = 4, class Wait>
 __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, uint32_t split, uint32_t tid, Wait &&wait_inputs) {
     using C = KV<F16>;
     using CT = typename C::T;
     constexpr int NW = NT / 64;
-    constexpr int EPL = HS / 4;                   // elements per lane in the score phase
+    // KL lanes share a position in the score phase (4, or 8 where registers are scarce: half as many elements per lane)
+    constexpr int EPL = HS / KL;                  // elements per lane in the score phase
+    constexpr int PPW = 64 / KL;                  // positions a wave owns per pass
     constexpr int LPP = HS / 8;                   // lanes per position in the value phase
     __shared__ float sq[HS], sk[HS], sv[HS];
     __shared__ float sred[NW], sred2[NW];
@@ -124,17 +126,17 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
     };
     if constexpr (!FUSED) { wait_inputs(); load_inputs(); }
     // ---- the first pass of keys and values is requested before anything else is computed: they depend on nothing
-    // but the position, and their latency then overlaps the q load and the RoPE.  A pass is NT/4 positions; wave w
-    // owns positions 16w..16w+15 of it for both the scores (4 lanes per position) and the values (LPP lanes per
+    // but the position, and their latency then overlaps the q load and the RoPE.  A pass is NT/KL positions; wave w
+    // owns PPW consecutive ones for both the scores (KL lanes per position) and the values (LPP lanes per
     // position, PW positions per sub-pass), so nothing but the final merge crosses waves. -----------------------
     constexpr int PW = 64 / LPP;                  // positions per value sub-pass of a wave
-    constexpr int NU = 16 / PW;                   // value sub-passes per pass
-    const uint32_t sub = tid & 3;
-    const uint32_t wpos = wave * 16;
+    constexpr int NU = PPW / PW;                  // value sub-passes per pass
+    const uint32_t sub = tid & (KL - 1);
+    const uint32_t wpos = wave * PPW;
     const uint32_t vgl = lane / LPP, ve = (lane % LPP) * 8;
     typename Vec8<F16>::Raw kv0[EPL / 8], vv0[NU];            // kept undecoded: fewer registers while they wait
     {
-        const uint32_t t = t0 + tid / 4;
+        const uint32_t t = t0 + tid / KL;
         // the fresh row comes from LDS later; lanes without a position read a valid address and are masked
         const uint32_t tc = (t < t1 && !(own_new && t == pos)) ? t : t0;
         const CT *kp = kc + (size_t)tc * a.kv_dim + hoff + sub * EPL;
@@ -189,20 +191,20 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
     const float root = sqrtf((float)HS);
     float m = -FLT_MAX, lsum = 0.0f;
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (uint32_t tb = t0; tb < t1; tb += NT / 4) {           // uniform trip count: the shuffles below need whole waves
-        const uint32_t t = tb + tid / 4;
+    for (uint32_t tb = t0; tb < t1; tb += NT / KL) {           // uniform trip count: the shuffles below need whole waves
+        const uint32_t t = tb + tid / KL;
         const bool live = t < t1;
         const bool use_new = own_new && live && t == pos;    // its cache row is being written by this very launch
         typename Vec8<F16>::Raw nxt[EPL / 8] = {}, nxtv[NU] = {};
-        if (tb + NT / 4 < t1) {                               // (uniform) there is a next pass
-            const uint32_t tn = t + NT / 4;
+        if (tb + NT / KL < t1) {                               // (uniform) there is a next pass
+            const uint32_t tn = t + NT / KL;
             const uint32_t tnc = (tn < t1 && !(own_new && tn == pos)) ? tn : t0;
             const CT *kp = kc + (size_t)tnc * a.kv_dim + hoff + sub * EPL;
 #pragma unroll
             for (int j = 0; j < EPL / 8; ++j) nxt[j] = Vec8<F16>::load_raw(kp + 8 * j);
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
-                const uint32_t tv = tb + NT / 4 + wpos + u * PW + vgl;
+                const uint32_t tv = tb + NT / KL + wpos + u * PW + vgl;
                 const uint32_t tvc = (tv < t1 && !(own_new && tv == pos)) ? tv : t0;
                 nxtv[u] = Vec8<F16>::load_raw(vc + (size_t)tvc * a.kv_dim + hoff + ve);
             }
@@ -224,6 +226,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
         for (int j = 0; j < EPL; ++j) part = fmaf(qr[j], kv[j], part);
         part += __shfl_xor(part, 1, 64);
         part += __shfl_xor(part, 2, 64);
+        if constexpr (KL == 8) part += __shfl_xor(part, 4, 64);
         const float sc = live ? part / root : -FLT_MAX;      // cpu.rs:521 `score /= sqrt(head_size)`
         const float mn = fmaxf(m, wave_max(sc));
         const float resc = expf(m - mn);                     // 0 on the first live pass, 1 while nothing was live
@@ -235,7 +238,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
             const uint32_t tv = tb + wpos + u * PW + vgl;
-            const float pw = __shfl(pr, 4 * (u * PW + vgl), 64);      // 0 for positions past the end
+            const float pw = __shfl(pr, KL * (u * PW + vgl), 64);      // 0 for positions past the end
             float vv[8];
             Vec8<F16>::decode(vv0[u], vv);
             if (own_new && tv == pos) {

@@ -284,7 +284,7 @@ __global__ void __launch_bounds__(1024) gemv_rowtile_kernel(const GemvRowtilePar
 constexpr uint32_t HANDOFF_SPIN_LIMIT = 1u << 24;
 
 template <bool F16, bool PREP>
-__global__ void __launch_bounds__(512) qkv_attention_kernel(const GemvRowtileParams p, const AttnLaunch a, uint32_t *counters, uint32_t timeout_slot) {
+__global__ void __launch_bounds__(1024) qkv_attention_kernel(const GemvRowtileParams p, const AttnLaunch a, uint32_t *counters, uint32_t timeout_slot) {
     extern __shared__ float smem[];
     const int NW = blockDim.x >> 6;
     float *partial = smem;
@@ -314,7 +314,7 @@ __global__ void __launch_bounds__(512) qkv_attention_kernel(const GemvRowtilePar
         if (threadIdx.x == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     if (t != 5) return;
-    attn::attn_fast_body<F16, 512, 128, true, true>(a, h, 0u, threadIdx.x, [&]() {
+    attn::attn_fast_body<F16, 1024, 128, true, true, 8>(a, h, 0u, threadIdx.x, [&]() {
         if (threadIdx.x == 0) {
             uint32_t seen = 0, spins = 0;
             do {
@@ -397,9 +397,10 @@ hipError_t launch_qkv_attention(slai_ctx *ctx, GemvRowtileParams p, const AttnLa
             return hipErrorInvalidValue;
         p.seg[i].ntiles = p.seg[i].nrows / 64;
     }
-    // eight waves: what the attention part uses, and 256 registers per lane for it; a wave then walks two super-blocks
-    const int NW = 8;
-    if (p.ncb < 8) return hipErrorInvalidValue;                 // (narrower models take the separate kernels)
+    // sixteen waves, one per super-block; the attention part uses all of them, eight lanes per position so that it fits
+    // the 128 registers per lane a workgroup of this size leaves
+    const int NW = 16;
+    if (p.ncb != 16) return hipErrorInvalidValue;               // (other widths take the separate kernels)
     p.scratch_stride = p.ncols + p.ncols / 16;
     const size_t smem = ((size_t)NW * 64 + NW) * sizeof(float);
     const uint32_t grid = a.n_heads * 6;
