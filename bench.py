@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the dominant kernel moves: rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch (two counter
 # runs of `bench.py --probe`), each scaled by what the same counter reads for the 64 MiB copy kernel of that probe.
 # The summary of those runs is kept under profiles/.
-DOMINANT_KERNEL_TRAFFIC_BYTES = 51385522
+DOMINANT_KERNEL_TRAFFIC_BYTES = 51385751
 CFG = dict(dim=4096, hidden_dim=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000)
 
 
