@@ -284,13 +284,24 @@ int slai_llama2_forward_logits(slai_llama2 *m, uint32_t pos, uint32_t token, int
  * elapsed_ms (optional) = stream time of the n_steps replays measured with HIP events. */
 int slai_llama2_generate(slai_llama2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
                          uint32_t n_steps, int32_t *out_tokens, float *elapsed_ms);
-/* Device access for set-up and inspection: layer l's caches ([kv_dim x seq_len]) and the state vectors. */
 /* The same loop with `Sampler::new(vocab, temperature, topp).sample()` run on the device (the chat
  * samples every generated token with 0.7 / 0.95: crates/slai-chat/src/sampler.rs:100-108), so no
  * logits cross the bus.  Draws are slai_sampler_coin(seed, pos). */
 int slai_llama2_generate_sampled(slai_llama2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
                                  uint32_t n_steps, float temperature, float topp, uint64_t seed, int32_t *out_tokens,
                                  float *elapsed_ms);
+/* Prompt tokens in chunks.  The reference feeds a prompt one token per forward pass and discards the logits of every
+ * prompt position but the last (chat_llama2.rs:105-158 with the forced-token rule, slai-chat/src/sampler.rs:100-105);
+ * this fills the caches for positions start_pos .. start_pos+n_tokens-1 with `chunk` tokens per pass over the
+ * weights and computes no logits (chunk: 0 = the path's default, 1 = token by token, at most 64).  Generation then
+ * continues with slai_llama2_generate(prompt, n_prompt, n_prompt - 1, ...).  slai_llama2_prefill_supported() says which
+ * path a model takes: 2 = fp32 matrix-core GEMM over the dequantised K-quant tiles, at most 32 tokens per pass;
+ * 1 = the GEMV kernels with one workgroup per token and tile sharing the weights through L2 (other tiled formats);
+ * 0 = layouts without chunked kernels, run token by token with the same result. */
+int slai_llama2_prefill(slai_llama2 *m, const int32_t *tokens, uint32_t n_tokens, uint32_t start_pos, uint32_t chunk,
+                        float *elapsed_ms);
+int slai_llama2_prefill_supported(const slai_llama2 *m);
+/* Device access for set-up and inspection: layer l's caches ([kv_dim x seq_len]) and the state vectors. */
 int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache);
 int slai_llama2_logits_buffer(slai_llama2 *m, slai_buffer **logits);
 

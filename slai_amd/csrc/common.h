@@ -50,6 +50,7 @@ struct slai_ctx {
     uint32_t *handoff_counters = nullptr;   // q/k/v + attention in one launch: one 128-byte line per head, then a timeout flag
     uint32_t handoff_heads = 0;
     bool fuse_qkv_attention = true;     // SLAI_FUSE_QKV_ATTN=0: always separate launches
+    bool prompt_gemm = true;            // SLAI_PROMPT_GEMM=0: prompt chunks never take the matrix-core kernels
     // tuning knobs (environment overridable, see runtime.cpp)
     int gemv_rows_per_wg = 8;
     int gemv_max_threads = 1024;
@@ -107,6 +108,16 @@ hipError_t launch_gemv(slai_ctx *ctx, int type, GemvParams p);
 bool gemv_supports(int type, uint32_t ncols);
 
 // GEMV over the tiled layout (kernels_gemv_tiled.hip); all segments share type and column geometry.
+// Several input vectors through one launch (a chunk of prompt tokens): vector b reads x + b * x_stride (and prepared + b *
+// prepared_stride), writes segment i to out + b * out_stride[i] and its emitted copy to emit_out + b * emit_stride (strides
+// in floats).  The workgroups that read the same weights run next to each other on one XCD, so the weights come from
+// memory once per launch and from that XCD's L2 for the other vectors.  n = 1: a plain launch.
+struct GemvBatch {
+    uint32_t n = 1;
+    uint32_t x_stride = 0, prepared_stride = 0, emit_stride = 0;
+    uint32_t out_stride[3] = {0, 0, 0};
+};
+
 struct GemvTiledSeg {
     const uint8_t *W = nullptr;
     const uint8_t *W2 = nullptr;
@@ -130,7 +141,7 @@ struct GemvTiledParams {
     const float *emit_w = nullptr;    // GEMV_EMIT (segment 0): weights of the next norm
     float *emit_out = nullptr;        // [nrows + nrows/16]
 };
-hipError_t launch_gemv_tiled(slai_ctx *ctx, int type, GemvTiledParams p);
+hipError_t launch_gemv_tiled(slai_ctx *ctx, int type, GemvTiledParams p, const GemvBatch *batch = nullptr);
 
 // GEMV over 64-row tiles with wave-uniform activations (kernels_gemv_rowtile.hip).  Segments share the
 // input, the prologue and the column count; their block formats may differ.
@@ -159,7 +170,35 @@ struct GemvRowtileParams {
     uint32_t scratch_stride = 0;      // filled by the launcher
 };
 size_t gemv_rowtile_scratch_floats(const GemvRowtileParams &p);
-hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p);
+// With a batch of more than one vector the input must come `prepared`.
+hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p, const GemvBatch *batch = nullptr);
+
+// A chunk of up to 32 input vectors ("prompt tokens") through up to three matrices on the matrix cores
+// (kernels_gemm_chunk.hip): out[t][r] = sum_c deq(W[r][c]) * x[t][c] (+ bias[r]) (+ the old out[t][r]), token t at
+// x + t * x_stride and out + t * out_stride.  K-quants in 64-row tiles (any number of segments, formats may differ) or in
+// 16-row tiles of at most 16 column groups (one segment).
+struct GemmChunkSeg {
+    const uint8_t *W = nullptr;
+    int type = 0;
+    uint32_t nrows = 0;
+    uint32_t ntiles = 0;   // filled by the launcher
+    float *out = nullptr;
+    const float *bias = nullptr;
+    uint32_t flags = 0;    // GEMV_BIAS, GEMV_ACCUM
+    uint32_t out_stride = 0;
+};
+struct GemmChunkParams {
+    GemmChunkSeg seg[3];
+    int nseg = 1;
+    uint32_t ncols = 0, ncb = 0, ngroups = 0, rows_log2 = 6;
+    const float *x = nullptr;   // 16-byte aligned
+    uint32_t x_stride = 0;      // floats, a multiple of 4
+    uint32_t ntokens = 0;
+};
+bool gemm_chunk_supports(const slai_qmat *m);
+hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p);
+// out[t][i] = (x[t][i] / sqrt(mean(x[t]^2) + eps)) * w[i] for `rows` vectors of n floats
+hipError_t launch_rms_norm_rows(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t rows, uint32_t out_stride, uint32_t x_stride, float eps);
 
 // One GEMV launch over up to three matrices of one format and layout: out[i] = epilogue(m[i] . prologue(x)).
 struct GemvCall {
@@ -179,6 +218,7 @@ struct GemvCall {
     float *emit_out = nullptr;
     // Consumer side: such a copy of norm_w-weighted x (see GemvRowtileParams::prepared); nullptr = none.
     const float *prepared = nullptr;
+    GemvBatch batch;   // more than one input vector (64-row-tile launches with prepared input and 16-row-tile launches only)
 };
 // True when gemv_call would honour GEMV_EMIT for this matrix as segment 0.
 bool gemv_can_emit(const slai_qmat *m);
@@ -267,6 +307,13 @@ struct AttnLaunch {
     uint32_t n_splits;
 };
 hipError_t launch_attention(hipStream_t s, const AttnLaunch &a);
+// A chunk of `n` consecutive tokens whose keys and values are already in the caches: token b attends from q + b * q_stride
+// over positions [0, pos_ptr[b]] into out + b * out_stride; knew / vnew must be null.  One workgroup per head and token.
+hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride);
+// The step before it: for token b (position pos_ptr[b]) add the biases, rotate q + b * q_stride in place and write the
+// rotated key k + b * kv_stride and the value v + b * kv_stride to row pos_ptr[b] of the caches.  Uses the q / cache /
+// bias / rope fields of `a`.
+hipError_t launch_rope_store_batch(hipStream_t s, const AttnLaunch &a, float *q, const float *k, const float *v, uint32_t n, uint32_t q_stride, uint32_t kv_stride);
 // q/k/v GEMV (three segments in the order v, k, q) and the attention over their results in one launch
 hipError_t launch_qkv_attention(slai_ctx *ctx, GemvRowtileParams p, const AttnLaunch &a);
 // out[i] = powf(base, -((2*i) % head_size) / head_size), i < head_size/2

@@ -107,6 +107,16 @@ struct Llama2State {                 // transformer.rs:16-44
     slai_buffer *rope_config = nullptr, *rms_norm_config = nullptr, *attn_params = nullptr;
 };
 
+// Activations of a chunk of prompt tokens that go through the layers together (one row per token), and the
+// positions 0, 1, 2, ... as device words (token b of a chunk at pos0 reads its position from positions + pos0 + b).
+struct PromptChunkState {
+    uint32_t rows = 0;
+    GpuTensor x, xw, xb, q, k, v, hb;
+    GpuTensor xn, hb2;                 // matrix-core path: normalised activations, the up projection
+    slai_buffer *positions = nullptr;
+    slai_buffer *tokens = nullptr;     // int32[seq_len]
+};
+
 struct slai_llama2 {
     slai_ctx *ctx = nullptr;
     int model_type = SLAI_MODEL_LLAMA;
@@ -125,6 +135,15 @@ struct slai_llama2 {
     int load(const slai_gguf *g);
     int launch(LlmContext &ctxt, const slai_attn_params &attn_params, uint32_t pos);   // transformer.rs:316-381
     int enqueue_fused(int sampler);   // 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state
+
+    // Prompt tokens in chunks: every weight matrix is read once per chunk instead of once per token.
+    PromptChunkState chunk;
+    bool chunk_supported() const;        // per-token workgroups over shared weights (any tiled format)
+    bool chunk_gemm_supported() const;   // matrix cores (K-quants)
+    int chunk_reserve(uint32_t rows);
+    int enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev);   // fills the caches for positions pos0 .. pos0 + n - 1
+    int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev);   // the same on the matrix cores, n <= 32
+    int chunk_attention(uint32_t l, uint32_t pos0, uint32_t n);
 };
 
 // models/llama2/cpu.rs:79-109
@@ -397,6 +416,215 @@ int slai_llama2::enqueue_fused(int sampler) {
     return SLAI_OK;
 }
 
+// The chunked path covers the layouts the loader picks for models whose widths are multiples of 256: q/k/v and the
+// gate/up pair in 64-row tiles (they take the norm-weighted copy of x the previous launch leaves), attention output and
+// down projection in 16- or 32-row tiles (they leave it).
+bool slai_llama2::chunk_supported() const {
+    const uint32_t hs = head_size();
+    if ((hs != 64 && hs != 128) || kv_dim() % 8 || config.dim % 16) return false;
+    for (const Llama2LayerWeights &w : weights.layers) {
+        for (const slai_qmat *m : {w.attn_q, w.attn_k, w.attn_v})
+            if (!gemv_is_rowtile(ctx, m)) return false;
+        if (!gemv_gated_is_rowtile(ctx, w.ffn_gate, w.ffn_up)) return false;
+        if (!gemv_can_emit(w.attn_output) || !gemv_can_emit(w.ffn_down)) return false;
+    }
+    return true;
+}
+
+int slai_llama2::chunk_reserve(uint32_t rows) {
+    PromptChunkState &c = chunk;
+    if (rows <= c.rows) return SLAI_OK;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "prompt chunk buffers must be reserved before graph capture");
+    TRY(slai_synchronize(ctx));
+    for (GpuTensor *t : {&c.x, &c.xw, &c.xb, &c.q, &c.k, &c.v, &c.hb, &c.xn, &c.hb2}) t->destroy(ctx);
+    c.rows = 0;
+    const uint32_t dim = config.dim, kvd = kv_dim();
+    TRY(GpuTensor::matrix(ctx, dim, rows, STORAGE, &c.x));
+    TRY(GpuTensor::matrix(ctx, dim + dim / 16, rows, STORAGE, &c.xw));
+    TRY(GpuTensor::matrix(ctx, dim, rows, STORAGE, &c.xb));
+    TRY(GpuTensor::matrix(ctx, dim, rows, STORAGE, &c.q));
+    TRY(GpuTensor::matrix(ctx, kvd, rows, STORAGE, &c.k));
+    TRY(GpuTensor::matrix(ctx, kvd, rows, STORAGE, &c.v));
+    TRY(GpuTensor::matrix(ctx, config.hidden_dim, rows, STORAGE, &c.hb));
+    TRY(GpuTensor::matrix(ctx, dim, rows, STORAGE, &c.xn));
+    TRY(GpuTensor::matrix(ctx, config.hidden_dim, rows, STORAGE, &c.hb2));
+    if (!c.positions) {
+        TRY(slai_buffer_create(ctx, (size_t)config.seq_len * 4, SLAI_DT_I32, STORAGE | COPY_DST, &c.positions));
+        TRY(slai_buffer_create(ctx, (size_t)config.seq_len * 4, SLAI_DT_I32, STORAGE | COPY_DST, &c.tokens));
+        std::vector<uint32_t> iota(config.seq_len);
+        for (uint32_t i = 0; i < config.seq_len; ++i) iota[i] = i;
+        TRY(slai_write_buffer(ctx, c.positions, 0, iota.data(), iota.size() * 4));
+    }
+    c.rows = rows;
+    return SLAI_OK;
+}
+
+// The layer loop of enqueue_fused for n tokens at once.  Token b of the chunk lives in row b of every activation
+// matrix; the GEMV launches take all rows (GemvBatch), bias + RoPE + cache write run for all rows before the attention
+// of any row (a token attends to the earlier tokens of its chunk), and the logits are not computed.
+int slai_llama2::enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev) {
+    PromptChunkState &pc = chunk;
+    if (n == 0 || n > pc.rows || pos0 + n > config.seq_len) return set_error(ctx, SLAI_E_ARG, "prompt chunk out of range");
+    Llama2State &s = state;
+    const uint32_t dim = config.dim, kvd = kv_dim(), hid = config.hidden_dim, xws = dim + dim / 16;
+    float *x = (float *)pc.x.buf->dptr, *xw = (float *)pc.xw.buf->dptr, *xb = (float *)pc.xb.buf->dptr, *q = (float *)pc.q.buf->dptr;
+    float *k = (float *)pc.k.buf->dptr, *v = (float *)pc.v.buf->dptr, *hb = (float *)pc.hb.buf->dptr;
+    for (uint32_t b = 0; b < n; ++b) {
+        SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, tokens_dev + b, nullptr, nullptr, dim, x + (size_t)b * dim));
+        SLAI_HIP_TRY(ctx, launch_prepare(ctx->stream, xw + (size_t)b * xws, x + (size_t)b * dim, (const float *)weights.layers[0].attn_norm.buf->dptr, dim));
+    }
+    for (uint32_t l = 0; l < config.n_layers; ++l) {
+        const Llama2LayerWeights &wl = weights.layers[l];
+        {   // ---- RMSNorm + q/k/v
+            const slai_qmat *mats[3] = {wl.attn_v, wl.attn_k, wl.attn_q};
+            float *outs[3] = {v, k, q};
+            const uint32_t strides[3] = {kvd, kvd, dim};
+            bool done[3] = {false, false, false};
+            for (int i = 0; i < 3; ++i) {
+                if (done[i]) continue;
+                GemvCall c;
+                c.nseg = 0; c.x = x; c.prepared = xw;
+                c.prologue = PRO_RMSNORM; c.norm_w = (const float *)wl.attn_norm.buf->dptr; c.eps = config.rms_norm_eps;
+                c.batch.n = n; c.batch.x_stride = dim; c.batch.prepared_stride = xws;
+                for (int j = i; j < 3; ++j) {
+                    if (done[j] || !same_launch(mats[i], mats[j])) continue;
+                    c.m[c.nseg] = mats[j]; c.out[c.nseg] = outs[j]; c.batch.out_stride[c.nseg] = strides[j]; ++c.nseg;
+                    done[j] = true;
+                }
+                TRY(gemv_call(ctx, c, "llama2 qkv (prompt chunk)"));
+            }
+        }
+        TRY(chunk_attention(l, pos0, n));
+        {   // ---- attention output, residual, copy for the feed-forward norm
+            GemvCall c;
+            c.m[0] = wl.attn_output; c.out[0] = x; c.flags[0] = GEMV_ACCUM | GEMV_EMIT; c.x = xb;
+            c.emit_w = (const float *)wl.ffn_norm.buf->dptr; c.emit_out = xw;
+            c.batch.n = n; c.batch.x_stride = dim; c.batch.out_stride[0] = dim; c.batch.emit_stride = xws;
+            TRY(gemv_call(ctx, c, "llama2 attn_output (prompt chunk)"));
+        }
+        {   // ---- RMSNorm + gate/up + SiLU
+            GemvCall c;
+            c.m[0] = wl.ffn_gate; c.m2[0] = wl.ffn_up; c.out[0] = hb; c.flags[0] = GEMV_SILU_GATE; c.x = x; c.prepared = xw;
+            c.prologue = PRO_RMSNORM; c.norm_w = (const float *)wl.ffn_norm.buf->dptr; c.eps = config.rms_norm_eps;
+            c.batch.n = n; c.batch.x_stride = dim; c.batch.prepared_stride = xws; c.batch.out_stride[0] = hid;
+            TRY(gemv_call(ctx, c, "llama2 ffn gate/up (prompt chunk)"));
+        }
+        {   // ---- down projection, residual, copy for the next layer's norm (nothing reads it after the last layer)
+            GemvCall c;
+            c.m[0] = wl.ffn_down; c.out[0] = x; c.flags[0] = GEMV_ACCUM; c.x = hb;
+            if (l + 1 < config.n_layers) {
+                c.flags[0] |= GEMV_EMIT; c.emit_w = (const float *)weights.layers[l + 1].attn_norm.buf->dptr; c.emit_out = xw;
+            }
+            c.batch.n = n; c.batch.x_stride = hid; c.batch.out_stride[0] = dim; c.batch.emit_stride = xws;
+            TRY(gemv_call(ctx, c, "llama2 ffn_down (prompt chunk)"));
+        }
+    }
+    return SLAI_OK;
+}
+
+// Bias + RoPE + cache write for the n tokens of a chunk (their q / k / v are in the chunk's matrices), then their
+// attention into the chunk's xb.
+int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n) {
+    PromptChunkState &pc = chunk;
+    Llama2State &s = state;
+    const Llama2LayerWeights &wl = weights.layers[l];
+    const uint32_t dim = config.dim, kvd = kv_dim();
+    float *q = (float *)pc.q.buf->dptr;
+    AttnLaunch a{};
+    a.q = q; a.kcache = s.key_cache[l].buf->dptr; a.vcache = s.value_cache[l].buf->dptr;
+    a.kv_f16 = kv_dtype == SLAI_KV_F16;
+    a.n_heads = config.n_q_heads; a.kv_mul = config.n_q_heads / config.n_kv_heads; a.head_size = head_size();
+    a.kv_dim = kvd; a.seq_len = config.seq_len;
+    a.pos_ptr = (const uint32_t *)pc.positions->dptr + pos0;
+    a.qbias = wl.attn_q_bias.buf ? (const float *)wl.attn_q_bias.buf->dptr : nullptr;
+    a.kbias = wl.attn_k_bias.buf ? (const float *)wl.attn_k_bias.buf->dptr : nullptr;
+    a.vbias = wl.attn_v_bias.buf ? (const float *)wl.attn_v_bias.buf->dptr : nullptr;
+    a.rope_variant = rope_variant(); a.rope_base = config.rope_base_freq;
+    a.rope_theta = (const float *)s.rope_theta.buf->dptr;
+    a.out = (float *)pc.xb.buf->dptr; a.scratch = nullptr; a.n_splits = 1;
+    SLAI_HIP_TRY(ctx, launch_rope_store_batch(ctx->stream, a, q, (const float *)pc.k.buf->dptr, (const float *)pc.v.buf->dptr, n, dim, kvd));
+    SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, dim, dim));
+    return SLAI_OK;
+}
+
+bool slai_llama2::chunk_gemm_supported() const {
+    const uint32_t hs = head_size();
+    if ((hs != 64 && hs != 128) || kv_dim() % 8 || config.dim % 4 || config.hidden_dim % 4) return false;
+    for (const Llama2LayerWeights &w : weights.layers)
+        for (const slai_qmat *m : {w.attn_q, w.attn_k, w.attn_v, w.attn_output, w.ffn_gate, w.ffn_up, w.ffn_down})
+            if (!gemm_chunk_supports(m)) return false;
+    return true;
+}
+
+namespace {
+// matrices (with the same input) through the matrix-core kernel: 64-row-tile matrices share a launch
+int gemm_chunk_call(slai_ctx *ctx, int nmat, const slai_qmat *const *mats, float *const *outs, const uint32_t *out_strides, uint32_t flags,
+                    const float *x, uint32_t x_stride, uint32_t ntokens, const char *who) {
+    bool done[3] = {false, false, false};
+    for (int i = 0; i < nmat; ++i) {
+        if (done[i]) continue;
+        GemmChunkParams p;
+        p.nseg = 0; p.ncols = mats[i]->ncols; p.ncb = mats[i]->ncb; p.ngroups = mats[i]->ngroups; p.rows_log2 = mats[i]->rows_log2;
+        p.x = x; p.x_stride = x_stride; p.ntokens = ntokens;
+        for (int j = i; j < nmat; ++j) {
+            if (done[j] || (j != i && (mats[j]->rows_log2 != 6 || mats[i]->rows_log2 != 6 || mats[j]->ncols != mats[i]->ncols))) continue;
+            GemmChunkSeg &sg = p.seg[p.nseg++];
+            sg.W = mats[j]->dptr; sg.type = mats[j]->type; sg.nrows = mats[j]->nrows; sg.out = outs[j]; sg.out_stride = out_strides[j]; sg.flags = flags;
+            done[j] = true;
+        }
+        hipError_t e = launch_gemm_chunk(ctx, p);
+        if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported shape for the prompt-chunk GEMM");
+        if (e != hipSuccess) return hip_fail(ctx, e, who);
+    }
+    return SLAI_OK;
+}
+}  // namespace
+
+// The layer loop for a chunk of up to 32 tokens with every projection on the matrix cores (kernels_gemm_chunk.hip):
+// RMSNorm of all rows, q/k/v, bias + RoPE + cache write, attention, output projection into the residual, RMSNorm,
+// gate and up, SiLU, down projection into the residual (transformer.rs:316-381 per token).
+int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev) {
+    PromptChunkState &pc = chunk;
+    if (n == 0 || n > 32 || n > pc.rows || pos0 + n > config.seq_len) return set_error(ctx, SLAI_E_ARG, "prompt chunk out of range");
+    const uint32_t dim = config.dim, kvd = kv_dim(), hid = config.hidden_dim;
+    float *x = (float *)pc.x.buf->dptr, *xn = (float *)pc.xn.buf->dptr, *xb = (float *)pc.xb.buf->dptr, *q = (float *)pc.q.buf->dptr;
+    float *k = (float *)pc.k.buf->dptr, *v = (float *)pc.v.buf->dptr, *hb = (float *)pc.hb.buf->dptr, *hb2 = (float *)pc.hb2.buf->dptr;
+    for (uint32_t b = 0; b < n; ++b)
+        SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, tokens_dev + b, nullptr, nullptr, dim, x + (size_t)b * dim));
+    for (uint32_t l = 0; l < config.n_layers; ++l) {
+        const Llama2LayerWeights &wl = weights.layers[l];
+        SLAI_HIP_TRY(ctx, launch_rms_norm_rows(ctx->stream, xn, x, (const float *)wl.attn_norm.buf->dptr, dim, n, dim, dim, config.rms_norm_eps));
+        {
+            const slai_qmat *mats[3] = {wl.attn_v, wl.attn_k, wl.attn_q};
+            float *outs[3] = {v, k, q};
+            const uint32_t strides[3] = {kvd, kvd, dim};
+            TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, dim, n, "llama2 qkv (prompt chunk)"));
+        }
+        TRY(chunk_attention(l, pos0, n));
+        {
+            const slai_qmat *mats[1] = {wl.attn_output};
+            float *outs[1] = {x};
+            const uint32_t strides[1] = {dim};
+            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, xb, dim, n, "llama2 attn_output (prompt chunk)"));
+        }
+        SLAI_HIP_TRY(ctx, launch_rms_norm_rows(ctx->stream, xn, x, (const float *)wl.ffn_norm.buf->dptr, dim, n, dim, dim, config.rms_norm_eps));
+        {
+            const slai_qmat *mats[2] = {wl.ffn_gate, wl.ffn_up};
+            float *outs[2] = {hb, hb2};
+            const uint32_t strides[2] = {hid, hid};
+            TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, 0, xn, dim, n, "llama2 ffn gate/up (prompt chunk)"));
+        }
+        SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, n * hid, 1}, VecView{hb2, n * hid, 1}));
+        {
+            const slai_qmat *mats[1] = {wl.ffn_down};
+            float *outs[1] = {x};
+            const uint32_t strides[1] = {dim};
+            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, hb, hid, n, "llama2 ffn_down (prompt chunk)"));
+        }
+    }
+    return SLAI_OK;
+}
+
 SLAI_EXPORT int slai_llama2_from_gguf(slai_ctx *ctx, const slai_gguf *g, int model_type, int kv_dtype, slai_llama2 **out) {
     if (!ctx || !g || !out) return SLAI_E_ARG;
     *out = nullptr;
@@ -427,6 +655,9 @@ SLAI_EXPORT void slai_llama2_destroy(slai_llama2 *m) {
     for (auto &t : s.key_cache) t.destroy(ctx);
     for (auto &t : s.value_cache) t.destroy(ctx);
     for (slai_buffer *b : {s.rope_config, s.rms_norm_config, s.attn_params}) if (b) slai_buffer_destroy(ctx, b);
+    PromptChunkState &pc = m->chunk;
+    for (GpuTensor *t : {&pc.x, &pc.xw, &pc.xb, &pc.q, &pc.k, &pc.v, &pc.hb, &pc.xn, &pc.hb2}) t->destroy(ctx);
+    for (slai_buffer *b : {pc.positions, pc.tokens}) if (b) slai_buffer_destroy(ctx, b);
     delete m;
 }
 
@@ -534,6 +765,55 @@ SLAI_EXPORT int slai_llama2_generate_sampled(slai_llama2 *m, const int32_t *prom
     if (!m) return SLAI_E_ARG;
     const SamplingParams sp{temperature, topp, seed};
     return generate_impl(m, m->ctx, m->loop, m->config.seq_len, m->config.vocab_size, prompt, n_prompt, start_pos, n_steps, out_tokens, elapsed_ms, &sp);
+}
+
+// 0: the ordinary loop, 1: per-token workgroups over shared weights, 2: matrix cores
+SLAI_EXPORT int slai_llama2_prefill_supported(const slai_llama2 *m) {
+    if (!m) return 0;
+    if (m->ctx->prompt_gemm && m->chunk_gemm_supported()) return 2;
+    return m->chunk_supported() ? 1 : 0;
+}
+
+// The prompt loop of chat_llama2.rs:105-158 feeds the prompt one token per forward pass and throws the logits of all but
+// the last away.  This runs positions start_pos .. start_pos + n_tokens - 1 through the layers `chunk` tokens at a time
+// and computes no logits; afterwards the caches are what the token-by-token loop would have left, and generation
+// continues with slai_llama2_generate(prompt, n_prompt, start_pos = n_prompt - 1, ...).
+SLAI_EXPORT int slai_llama2_prefill(slai_llama2 *m, const int32_t *tokens, uint32_t n_tokens, uint32_t start_pos, uint32_t chunk, float *elapsed_ms) {
+    if (!m) return SLAI_E_ARG;
+    slai_ctx *ctx = m->ctx;
+    if (elapsed_ms) *elapsed_ms = 0.0f;
+    if (n_tokens == 0) return SLAI_OK;
+    if (!tokens) return set_error(ctx, SLAI_E_ARG, "slai_llama2_prefill: no tokens");
+    if ((uint64_t)start_pos + n_tokens > m->config.seq_len) return set_error(ctx, SLAI_E_SHAPE, "slai_llama2_prefill: would run past the context length");
+    for (uint32_t i = 0; i < n_tokens; ++i)
+        if (tokens[i] < 0 || (uint32_t)tokens[i] >= m->config.vocab_size) return set_error(ctx, SLAI_E_ARG, "slai_llama2_prefill: token out of range");
+    if (chunk > 64) return set_error(ctx, SLAI_E_ARG, "slai_llama2_prefill: at most 64 tokens per chunk");
+    // K-quants in the tiled layouts: matrix cores, 32 tokens per pass; other tiled formats: one workgroup per token and
+    // tile over shared weights; anything else: the ordinary loop
+    const bool gemm = ctx->prompt_gemm && m->chunk_gemm_supported();
+    const bool shared = !gemm && m->chunk_supported();
+    if (chunk == 0) chunk = gemm ? 32 : 16;
+    if (chunk == 1 || (!gemm && !shared)) {
+        // one token per pass, picks discarded
+        std::vector<int32_t> prompt((size_t)start_pos + n_tokens, 0), picks(n_tokens);
+        std::copy(tokens, tokens + n_tokens, prompt.begin() + start_pos);
+        return generate_impl(m, ctx, m->loop, m->config.seq_len, m->config.vocab_size, prompt.data(), (uint32_t)prompt.size(), start_pos, n_tokens,
+                             picks.data(), elapsed_ms);
+    }
+    if (gemm && chunk > 32) chunk = 32;
+    TRY(m->chunk_reserve(chunk));
+    TRY(slai_write_buffer(ctx, m->chunk.tokens, 0, tokens, (size_t)n_tokens * 4));
+    const int *tokens_dev = (const int *)m->chunk.tokens->dptr;
+    SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev0, ctx->stream));
+    for (uint32_t i = 0; i < n_tokens; i += chunk) {
+        const uint32_t n = std::min(chunk, n_tokens - i);
+        if (gemm) TRY(m->enqueue_chunk_gemm(start_pos + i, n, tokens_dev + i));
+        else TRY(m->enqueue_chunk(start_pos + i, n, tokens_dev + i));
+    }
+    SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev1, ctx->stream));
+    TRY(slai_synchronize(ctx));
+    if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, m->loop.ev0, m->loop.ev1));
+    return SLAI_OK;
 }
 
 SLAI_EXPORT int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache) {

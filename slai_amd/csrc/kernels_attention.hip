@@ -170,6 +170,59 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
     attn_fast_body<F16, NT, HS, SINGLE, false>(a, blockIdx.x, SINGLE ? 0u : blockIdx.y, threadIdx.x, []() {});
 }
 
+// A chunk of tokens whose keys and values are already in the caches: grid = (n_heads, tokens), whole context in one
+// workgroup; token b reads q + b * q_stride and its position pos_ptr[b].
+template <bool F16, int HS>
+__global__ void __launch_bounds__(512) attn_fast_batch_kernel(AttnLaunch a0, uint32_t q_stride, uint32_t out_stride) {
+    touch_kernel_arguments<sizeof(AttnLaunch) + 8>();
+    AttnLaunch a = a0;
+    const uint32_t b = blockIdx.y;
+    a.q = a0.q + (size_t)b * q_stride;
+    a.out = a0.out + (size_t)b * out_stride;
+    a.pos_ptr = a0.pos_ptr + b;
+    a.knew = nullptr; a.vnew = nullptr;
+    attn_fast_body<F16, 512, HS, true, false>(a, blockIdx.x, 0u, threadIdx.x, []() {});
+}
+
+// The bias / RoPE / cache-write part of attn_fast_body for a chunk of tokens, as a launch of its own: a token's
+// attention reads the rows of the earlier tokens of its chunk, so all rows are written before any attention starts.
+// grid = (n_heads, tokens), block = head_size / 2 (one rotation pair per thread; rope.slang:27-84).
+template <bool F16>
+__global__ void rope_store_batch_kernel(AttnLaunch a, float *q, const float *k, const float *v, uint32_t q_stride, uint32_t kv_stride) {
+    using C = KV<F16>;
+    using CT = typename C::T;
+    const uint32_t h = blockIdx.x, b = blockIdx.y, i = threadIdx.x, HS = a.head_size;
+    const uint32_t kvh = h / a.kv_mul;
+    const uint32_t pos = a.pos_ptr[b];
+    const size_t hoff = (size_t)kvh * HS;
+    uint32_t e0, e1;
+    if (a.rope_variant == SLAI_ROPE_NEOX) { e0 = i; e1 = i + HS / 2; } else { e0 = 2 * i; e1 = 2 * i + 1; }
+    float *qb = q + (size_t)b * q_stride + (size_t)h * HS;
+    const float *kb = k + (size_t)b * kv_stride + hoff, *vb = v + (size_t)b * kv_stride + hoff;
+    float q0 = qb[e0], q1 = qb[e1];
+    if (a.qbias) { q0 += a.qbias[(size_t)h * HS + e0]; q1 += a.qbias[(size_t)h * HS + e1]; }
+    float k0 = kb[e0], k1 = kb[e1], v0 = vb[e0], v1 = vb[e1];
+    if (a.kbias) { k0 += a.kbias[hoff + e0]; k1 += a.kbias[hoff + e1]; }
+    if (a.vbias) { v0 += a.vbias[hoff + e0]; v1 += a.vbias[hoff + e1]; }
+    if (a.rope_variant >= 0) {
+        const float theta = a.rope_theta ? a.rope_theta[i] : powf(a.rope_base, -(float)((2 * i) % HS) / (float)HS);
+        const float m_theta = (float)pos * theta;
+        float c, sn;
+        sincosf(m_theta, &sn, &c);
+        const float r0 = c * q0 - sn * q1, r1 = sn * q0 + c * q1;
+        q0 = r0; q1 = r1;
+        const float kr0 = c * k0 - sn * k1, kr1 = sn * k0 + c * k1;
+        k0 = kr0; k1 = kr1;
+    }
+    qb[e0] = q0; qb[e1] = q1;
+    if (h % a.kv_mul == 0) {                                   // several query heads share a kv head: the first of the group writes
+        CT *kc = reinterpret_cast<CT *>(a.kcache), *vc = reinterpret_cast<CT *>(a.vcache);
+        CT *kd = kc + (size_t)pos * a.kv_dim + hoff, *vd = vc + (size_t)pos * a.kv_dim + hoff;
+        C::store(kd + e0, k0); C::store(kd + e1, k1);
+        C::store(vd + e0, v0); C::store(vd + e1, v1);
+    }
+}
+
 __global__ void rope_theta_kernel(float *out, uint32_t hs, float base) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < hs / 2) out[i] = powf(base, -(float)((2 * i) % hs) / (float)hs);      // rope.slang:36-38
@@ -233,6 +286,27 @@ hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
         e = hipGetLastError();
     }
     return e;
+}
+
+hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
+    if ((a.head_size != 64 && a.head_size != 128) || a.kv_dim % 8 || a.knew || a.vnew || n == 0 || n > 65535) return hipErrorInvalidValue;
+    dim3 grid(a.n_heads, n);
+    if (a.head_size == 128) {
+        if (a.kv_f16) attn_fast_batch_kernel<true, 128><<<grid, 512, 0, s>>>(a, q_stride, out_stride);
+        else attn_fast_batch_kernel<false, 128><<<grid, 512, 0, s>>>(a, q_stride, out_stride);
+    } else {
+        if (a.kv_f16) attn_fast_batch_kernel<true, 64><<<grid, 512, 0, s>>>(a, q_stride, out_stride);
+        else attn_fast_batch_kernel<false, 64><<<grid, 512, 0, s>>>(a, q_stride, out_stride);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_rope_store_batch(hipStream_t s, const AttnLaunch &a, float *q, const float *k, const float *v, uint32_t n, uint32_t q_stride, uint32_t kv_stride) {
+    if (a.head_size % 2 || a.head_size / 2 > 1024 || n == 0 || n > 65535 || a.kv_mul == 0) return hipErrorInvalidValue;
+    dim3 grid(a.n_heads, n);
+    if (a.kv_f16) rope_store_batch_kernel<true><<<grid, a.head_size / 2, 0, s>>>(a, q, k, v, q_stride, kv_stride);
+    else rope_store_batch_kernel<false><<<grid, a.head_size / 2, 0, s>>>(a, q, k, v, q_stride, kv_stride);
+    return hipGetLastError();
 }
 
 }  // namespace slai

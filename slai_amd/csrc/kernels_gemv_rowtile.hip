@@ -271,6 +271,47 @@ __global__ void __launch_bounds__(1024) gemv_rowtile_kernel(const GemvRowtilePar
     }
 }
 
+// The same tiles for several input vectors (a chunk of prompt tokens; prepared input only).  Workgroup i runs on XCD
+// i % 8, and workgroups are dispatched in index order: the bt.n workgroups of one tile get consecutive indices on ONE
+// XCD, i = ((tile / 8) * bt.n + b) * 8 + tile % 8, so they run at the same time on neighbouring compute units, the
+// first request for a piece of the tile brings it from memory and the others find it in that XCD's L2.
+template <int TT, bool DUAL>
+__global__ void __launch_bounds__(1024) gemv_rowtile_batch_kernel(const GemvRowtileParams p0, const GemvBatch bt, uint32_t total_tiles) {
+    extern __shared__ float smem[];
+    const int NW = blockDim.x >> 6;
+    float *partial = smem;
+    float *red = smem + (size_t)(DUAL ? 2 : 1) * NW * 64;
+    touch_kernel_arguments<((sizeof(GemvRowtileParams) + 63) / 64 + 1) * 64>();
+    const uint32_t i = blockIdx.x, j = i >> 3, b = j % bt.n;
+    uint32_t tile = (j / bt.n) * 8 + (i & 7u);
+    if (tile >= total_tiles) return;                             // (uniform) the tile count rounded up to the eight XCDs
+    const uint32_t n0 = p0.seg[0].ntiles, n1 = p0.seg[1].ntiles;
+    const int s = tile < n0 ? 0 : (tile - n0 < n1 ? 1 : 2);
+    tile -= s == 0 ? 0u : (s == 1 ? n0 : n0 + n1);
+    GemvRowtileSeg seg;
+    seg.W = s == 0 ? p0.seg[0].W : (s == 1 ? p0.seg[1].W : p0.seg[2].W);
+    seg.W2 = s == 0 ? p0.seg[0].W2 : (s == 1 ? p0.seg[1].W2 : p0.seg[2].W2);
+    seg.type = s == 0 ? p0.seg[0].type : (s == 1 ? p0.seg[1].type : p0.seg[2].type);
+    seg.nrows = s == 0 ? p0.seg[0].nrows : (s == 1 ? p0.seg[1].nrows : p0.seg[2].nrows);
+    seg.out = s == 0 ? p0.seg[0].out : (s == 1 ? p0.seg[1].out : p0.seg[2].out);
+    seg.bias = s == 0 ? p0.seg[0].bias : (s == 1 ? p0.seg[1].bias : p0.seg[2].bias);
+    seg.flags = s == 0 ? p0.seg[0].flags : (s == 1 ? p0.seg[1].flags : p0.seg[2].flags);
+    seg.out += (size_t)b * (s == 0 ? bt.out_stride[0] : (s == 1 ? bt.out_stride[1] : bt.out_stride[2]));
+    GemvRowtileParams p = p0;
+    p.x = p0.x + (size_t)b * bt.x_stride;
+    p.prepared = p0.prepared + (size_t)b * bt.prepared_stride;
+    if constexpr (TT != 0) {
+        tile_body<TT, DUAL, true>(p, seg, tile, partial, red);
+    } else {
+        switch (seg.type) {                                    // uniform over the workgroup
+        case T_Q4_K: tile_body<T_Q4_K, DUAL, true>(p, seg, tile, partial, red); break;
+        case T_Q6_K: tile_body<T_Q6_K, DUAL, true>(p, seg, tile, partial, red); break;
+        case T_Q5_K: if constexpr (!DUAL) tile_body<T_Q5_K, false, true>(p, seg, tile, partial, red); break;
+        default: break;
+        }
+    }
+}
+
 // ---- q/k/v projections and attention in ONE launch ----------------------------------------------------------------
 // For layers with as many kv heads as q heads, head size 128 and a context served by one workgroup per head.  The six
 // 64-row tiles that make up a head's q, k and v (two each; segments in the order v, k, q) go to six workgroups of the
@@ -333,7 +374,12 @@ __global__ void __launch_bounds__(1024) qkv_attention_kernel(const GemvRowtilePa
 }
 
 template <int TT, bool DUAL>
-hipError_t go(const GemvRowtileParams &p, uint32_t tiles, int NT, size_t smem, hipStream_t s) {
+hipError_t go(const GemvRowtileParams &p, uint32_t tiles, int NT, size_t smem, hipStream_t s, const GemvBatch *bt) {
+    if (bt && bt->n > 1) {
+        if (!p.prepared) return hipErrorInvalidValue;
+        gemv_rowtile_batch_kernel<TT, DUAL><<<(tiles + 7) / 8 * 8 * bt->n, NT, smem, s>>>(p, *bt, tiles);
+        return hipGetLastError();
+    }
     if (p.prepared) gemv_rowtile_kernel<TT, DUAL, true><<<tiles, NT, smem, s>>>(p);
     else gemv_rowtile_kernel<TT, DUAL, false><<<tiles, NT, smem, s>>>(p);
     return hipGetLastError();
@@ -347,7 +393,7 @@ size_t gemv_rowtile_scratch_floats(const GemvRowtileParams &p) {
     return (size_t)tiles * (p.ncols + p.ncols / 16);
 }
 
-hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p) {
+hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p, const GemvBatch *bt) {
     if (p.ncb == 0 || p.ncols != p.ncb * 256) return hipErrorInvalidValue;
     int NW = (int)(p.ncb < 16 ? p.ncb : 16);
     if (p.ncols > 16u * 64u * NW) NW = (int)((p.ncols + 1023) / 1024);       // 4 float4 of x per thread at most
@@ -377,12 +423,12 @@ hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p) {
     const int NT = NW * 64;
     hipStream_t st = ctx->stream;
     switch (tt) {
-    case T_Q4_K: return dual ? go<T_Q4_K, true>(p, tiles, NT, smem, st) : go<T_Q4_K, false>(p, tiles, NT, smem, st);
-    case T_Q6_K: return dual ? go<T_Q6_K, true>(p, tiles, NT, smem, st) : go<T_Q6_K, false>(p, tiles, NT, smem, st);
-    case T_Q8_0: return go<T_Q8_0, false>(p, tiles, NT, smem, st);
-    case T_Q4_0: return dual ? go<T_Q4_0, true>(p, tiles, NT, smem, st) : go<T_Q4_0, false>(p, tiles, NT, smem, st);
-    case T_Q5_K: return dual ? go<T_Q5_K, true>(p, tiles, NT, smem, st) : go<T_Q5_K, false>(p, tiles, NT, smem, st);
-    default: return dual ? go<0, true>(p, tiles, NT, smem, st) : go<0, false>(p, tiles, NT, smem, st);
+    case T_Q4_K: return dual ? go<T_Q4_K, true>(p, tiles, NT, smem, st, bt) : go<T_Q4_K, false>(p, tiles, NT, smem, st, bt);
+    case T_Q6_K: return dual ? go<T_Q6_K, true>(p, tiles, NT, smem, st, bt) : go<T_Q6_K, false>(p, tiles, NT, smem, st, bt);
+    case T_Q8_0: return go<T_Q8_0, false>(p, tiles, NT, smem, st, bt);
+    case T_Q4_0: return dual ? go<T_Q4_0, true>(p, tiles, NT, smem, st, bt) : go<T_Q4_0, false>(p, tiles, NT, smem, st, bt);
+    case T_Q5_K: return dual ? go<T_Q5_K, true>(p, tiles, NT, smem, st, bt) : go<T_Q5_K, false>(p, tiles, NT, smem, st, bt);
+    default: return dual ? go<0, true>(p, tiles, NT, smem, st, bt) : go<0, false>(p, tiles, NT, smem, st, bt);
     }
 }
 

@@ -98,10 +98,11 @@ template <int T, int N> struct UnitLoader {
 // One workgroup = `ngroups` waves; wave w owns column group w of every tile the workgroup visits.  The
 // workgroup walks its tiles with a stride of the segment's workgroup count; the next tile's weights
 // are requested before the current tile is consumed.
-template <int T, bool DUAL, int MAXT>
-__global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams p) {
+// `vec`: which input vector of a batched launch (0 otherwise) and its strides (see GemvBatch).
+struct TiledVec { size_t x_off, emit_off, out0, out1, out2; };
+template <int T, bool DUAL>
+__device__ __forceinline__ void tiled_body(const GemvTiledParams &p, uint32_t blk, float *smem, const TiledVec vec) {
     using F = Tiled<T>;
-    extern __shared__ float smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, NW = blockDim.x >> 6;
     const int ROWS = 1 << p.rows_log2, KQ = 64 >> p.rows_log2;
     const int lane16 = lane & 15;
@@ -109,10 +110,8 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     float *partial = smem;                                   // [DUAL?2:1][NW][64]
     float *red = smem + (size_t)(DUAL ? 2 : 1) * NW * 64;    // [NW]
 
-    touch_kernel_arguments<sizeof(GemvTiledParams)>();
     // the segment is picked with selects over statically indexed fields (no dependent fetches of the arguments)
     const uint32_t n0 = p.seg[0].nblocks, n1 = p.seg[1].nblocks;     // unused segments have nblocks = 0
-    uint32_t blk = blockIdx.x;
     const int s = blk < n0 ? 0 : (blk - n0 < n1 ? 1 : 2);
     blk -= s == 0 ? 0u : (s == 1 ? n0 : n0 + n1);
     GemvTiledSeg seg;
@@ -120,7 +119,7 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     seg.W2 = s == 0 ? p.seg[0].W2 : (s == 1 ? p.seg[1].W2 : p.seg[2].W2);
     seg.nrows = s == 0 ? p.seg[0].nrows : (s == 1 ? p.seg[1].nrows : p.seg[2].nrows);
     seg.nblocks = s == 0 ? n0 : (s == 1 ? n1 : p.seg[2].nblocks);
-    seg.out = s == 0 ? p.seg[0].out : (s == 1 ? p.seg[1].out : p.seg[2].out);
+    seg.out = (s == 0 ? p.seg[0].out : (s == 1 ? p.seg[1].out : p.seg[2].out)) + (s == 0 ? vec.out0 : (s == 1 ? vec.out1 : vec.out2));
     seg.bias = s == 0 ? p.seg[0].bias : (s == 1 ? p.seg[1].bias : p.seg[2].bias);
     seg.flags = s == 0 ? p.seg[0].flags : (s == 1 ? p.seg[1].flags : p.seg[2].flags);
     const uint32_t ntiles = (seg.nrows + ROWS - 1) >> p.rows_log2;
@@ -133,7 +132,7 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
     const size_t xoff = (size_t)(valid ? cb : 0) * 256 + lane16;
     DevX X;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) X.x[i] = p.x[xoff + 16 * i];
+    for (int i = 0; i < 16; ++i) X.x[i] = p.x[vec.x_off + xoff + 16 * i];
     float nw[16], nb[16];
     if (p.prologue != PRO_NONE) {
 #pragma unroll
@@ -254,21 +253,53 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams 
                 if (seg.flags & GEMV_ACCUM) o = old_c + o;
                 seg.out[row] = o;
                 ewv = ew_c * o;
-                if (seg.flags & GEMV_EMIT) p.emit_out[row] = ewv;
+                if (seg.flags & GEMV_EMIT) p.emit_out[vec.emit_off + row] = ewv;
             }
         }
         if ((seg.flags & GEMV_EMIT) && wave == 0) {            // wave-uniform: the sums of 16 consecutive weighted results
             const float s16 = row16_sum(ewv);                  // (0 in lanes without a row)
             const uint32_t row = tile * ROWS + lane;
-            if (lane < ROWS && (lane & 15) == 0 && row < seg.nrows) p.emit_out[seg.nrows + (row >> 4)] = s16;
+            if (lane < ROWS && (lane & 15) == 0 && row < seg.nrows) p.emit_out[vec.emit_off + seg.nrows + (row >> 4)] = s16;
         }
         if (next < ntiles) lds_barrier();                      // partial[] is reused by the next tile
         tile = next;
     }
 }
 
+template <int T, bool DUAL, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams p) {
+    extern __shared__ float smem[];
+    touch_kernel_arguments<sizeof(GemvTiledParams)>();
+    tiled_body<T, DUAL>(p, blockIdx.x, smem, TiledVec{0, 0, 0, 0, 0});
+}
+
+// The same for several input vectors (a chunk of prompt tokens).  Workgroup i runs on XCD i % 8 and workgroups are
+// dispatched in index order: the bt.n workgroups that walk the same tiles get consecutive indices on ONE XCD,
+// i = ((blk / 8) * bt.n + b) * 8 + blk % 8, so the first request for a piece of a tile brings it from memory and the
+// others find it in that XCD's L2.
+template <int T, bool DUAL, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_tiled_batch_kernel(const GemvTiledParams p, const GemvBatch bt, uint32_t total_blocks) {
+    extern __shared__ float smem[];
+    touch_kernel_arguments<((sizeof(GemvTiledParams) + 63) / 64 + 1) * 64>();
+    const uint32_t i = blockIdx.x, j = i >> 3, b = j % bt.n;
+    const uint32_t blk = (j / bt.n) * 8 + (i & 7u);
+    if (blk >= total_blocks) return;                            // (uniform) the block count rounded up to the eight XCDs
+    const TiledVec vec{(size_t)b * bt.x_stride, (size_t)b * bt.emit_stride,
+                       (size_t)b * bt.out_stride[0], (size_t)b * bt.out_stride[1], (size_t)b * bt.out_stride[2]};
+    tiled_body<T, DUAL>(p, blk, smem, vec);
+}
+
 template <int T, bool DUAL>
-hipError_t go(hipStream_t s, const GemvTiledParams &p, dim3 grid, int NT, size_t smem) {
+hipError_t go(hipStream_t s, const GemvTiledParams &p, dim3 grid, int NT, size_t smem, const GemvBatch *bt) {
+    if (bt && bt->n > 1) {
+        const uint32_t total = grid.x;
+        const dim3 g((total + 7) / 8 * 8 * bt->n);
+        if (NT <= 256) gemv_tiled_batch_kernel<T, DUAL, 256><<<g, NT, smem, s>>>(p, *bt, total);
+        else if (NT <= 512) gemv_tiled_batch_kernel<T, DUAL, 512><<<g, NT, smem, s>>>(p, *bt, total);
+        else if (NT <= 768) gemv_tiled_batch_kernel<T, DUAL, 768><<<g, NT, smem, s>>>(p, *bt, total);
+        else gemv_tiled_batch_kernel<T, DUAL, 1024><<<g, NT, smem, s>>>(p, *bt, total);
+        return hipGetLastError();
+    }
     // the bound decides the register budget: 256/512 threads leave 256, 768 leave 168, 1024 leave 128 per lane
     if (NT <= 256) gemv_tiled_kernel<T, DUAL, 256><<<grid, NT, smem, s>>>(p);
     else if (NT <= 512) gemv_tiled_kernel<T, DUAL, 512><<<grid, NT, smem, s>>>(p);
@@ -277,7 +308,7 @@ hipError_t go(hipStream_t s, const GemvTiledParams &p, dim3 grid, int NT, size_t
     return hipGetLastError();
 }
 
-template <int T> hipError_t launch_t(slai_ctx *ctx, GemvTiledParams &p) {
+template <int T> hipError_t launch_t(slai_ctx *ctx, GemvTiledParams &p, const GemvBatch *bt) {
     if (p.launch_groups == 0) p.launch_groups = p.ngroups;
     if (p.ngroups == 0 || p.launch_groups > 16 || p.group0 + p.launch_groups > p.ngroups) return hipErrorInvalidValue;
     // a partial launch cannot normalise its input (that needs every column) or apply a non-linear epilogue
@@ -308,19 +339,19 @@ template <int T> hipError_t launch_t(slai_ctx *ctx, GemvTiledParams &p) {
     const int NW = NT / 64;
     const size_t smem = ((size_t)(dual ? 2 : 1) * NW * 64 + NW) * sizeof(float);
     dim3 grid(total);
-    if (dual) return go<T, true>(ctx->stream, p, grid, NT, smem);
-    return go<T, false>(ctx->stream, p, grid, NT, smem);
+    if (dual) return go<T, true>(ctx->stream, p, grid, NT, smem, bt);
+    return go<T, false>(ctx->stream, p, grid, NT, smem, bt);
 }
 
 }  // namespace
 
-hipError_t launch_gemv_tiled(slai_ctx *ctx, int type, GemvTiledParams p) {
+hipError_t launch_gemv_tiled(slai_ctx *ctx, int type, GemvTiledParams p, const GemvBatch *bt) {
     switch (type) {
-    case T_Q4_K: return launch_t<T_Q4_K>(ctx, p);
-    case T_Q6_K: return launch_t<T_Q6_K>(ctx, p);
-    case T_Q8_0: return launch_t<T_Q8_0>(ctx, p);
-    case T_Q4_0: return launch_t<T_Q4_0>(ctx, p);
-    case T_Q5_K: return launch_t<T_Q5_K>(ctx, p);
+    case T_Q4_K: return launch_t<T_Q4_K>(ctx, p, bt);
+    case T_Q6_K: return launch_t<T_Q6_K>(ctx, p, bt);
+    case T_Q8_0: return launch_t<T_Q8_0>(ctx, p, bt);
+    case T_Q4_0: return launch_t<T_Q4_0>(ctx, p, bt);
+    case T_Q5_K: return launch_t<T_Q5_K>(ctx, p, bt);
     default: return hipErrorInvalidValue;
     }
 }

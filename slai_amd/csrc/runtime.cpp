@@ -80,6 +80,7 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->gemv_max_threads = env_int("SLAI_GEMV_MAX_THREADS", 512);
     ctx->attn_splits = env_int("SLAI_ATTN_SPLITS", 0);
     ctx->use_graph = env_int("SLAI_NO_GRAPH", 0) == 0;
+    ctx->prompt_gemm = env_int("SLAI_PROMPT_GEMM", 1) != 0;
     ctx->gemv_max_wgs = env_int("SLAI_GEMV_MAX_WGS", 512);
     ctx->tiled_layout = env_int("SLAI_TILED", 1) != 0;
     ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
@@ -357,6 +358,9 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunc
         if (rowtile || !gemv_can_emit(m0) || !c.emit_w || !c.emit_out) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": this GEMV cannot emit a prepared copy");
     }
     if (c.prepared && !rowtile) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": prepared activations need 64-row tiles");
+    const GemvBatch *batch = c.batch.n > 1 ? &c.batch : nullptr;
+    if (batch && (fused_attn || (rowtile && !c.prepared) || (!rowtile && !m0->tiled)))
+        return set_error(ctx, SLAI_E_ARG, std::string(who) + ": several input vectors need prepared input (64-row tiles) or 16-row tiles");
     if (rowtile) {
         GemvRowtileParams p;
         p.nseg = c.nseg; p.ncols = m0->ncols; p.ncb = m0->ncb; p.x = c.x; p.prologue = c.prologue; p.norm_w = c.norm_w; p.eps = c.eps;
@@ -370,7 +374,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunc
             if (rc) return rc;
             p.scratch = ctx->gemv_scratch;
         }
-        hipError_t e = fused_attn ? launch_qkv_attention(ctx, p, *fused_attn) : launch_gemv_rowtile(ctx, p);
+        hipError_t e = fused_attn ? launch_qkv_attention(ctx, p, *fused_attn) : launch_gemv_rowtile(ctx, p, batch);
         if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported shape for the row-tile GEMV");
         if (e != hipSuccess) return hip_fail(ctx, e, who);
         return SLAI_OK;
@@ -397,7 +401,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunc
             p.seg[i].out = c.out[i]; p.seg[i].bias = c.bias[i]; p.seg[i].flags = c.flags[i];
         }
         if (m0->ngroups <= 16) {
-            e = launch_gemv_tiled(ctx, m0->type, p);
+            e = launch_gemv_tiled(ctx, m0->type, p, batch);
         } else {
             // wide matrix: balanced slices of at most 16 column groups, one launch each; the first writes (or adds to
             // the residual), the others accumulate, the last one emits
@@ -414,7 +418,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunc
                     if (k > 0) { q.seg[i].flags = (q.seg[i].flags | GEMV_ACCUM) & ~GEMV_BIAS; }
                     if (k + 1 < nchunks) q.seg[i].flags &= ~GEMV_EMIT;
                 }
-                e = launch_gemv_tiled(ctx, m0->type, q);
+                e = launch_gemv_tiled(ctx, m0->type, q, batch);
             }
         }
     } else {

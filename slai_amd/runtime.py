@@ -475,6 +475,18 @@ class Llama2:
                                                            seed, out.ctypes.data, C.byref(ms)))
         return out, ms.value
 
+    def prefill_path(self):
+        """2: matrix-core GEMM, 1: per-token workgroups over shared weights, 0: the token-by-token loop."""
+        return int(self.b.L.slai_llama2_prefill_supported(self.h))
+
+    def prefill(self, tokens, start_pos=0, chunk=0):
+        """Fill the caches for positions start_pos .. start_pos+len(tokens)-1, `chunk` tokens per pass over the
+        weights (0 = the library's default); returns the stream time in ms."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        ms = C.c_float()
+        self.b.check(self.b.L.slai_llama2_prefill(self.h, tokens.ctypes.data, tokens.size, start_pos, chunk, C.byref(ms)))
+        return ms.value
+
     def kv_buffers(self, layer):
         k, v = C.c_void_p(), C.c_void_p()
         self.b.check(self.b.L.slai_llama2_kv_buffers(self.h, layer, C.byref(k), C.byref(v)))

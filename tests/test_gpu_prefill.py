@@ -1,0 +1,168 @@
+"""Prompt tokens in chunks (slai_llama2_prefill) against the oracle and against the token-by-token device loop.
+
+Three paths, picked by the model's layouts (Llama2.prefill_path): 2 = fp32 matrix-core GEMM (K-quants in 64- and 16-row
+tiles), 1 = the GEMV kernels with one workgroup per token and tile (other tiled layouts), 0 = the ordinary loop.
+
+The reference has no batched prompt pass: it feeds the prompt one token per forward pass (chat_llama2.rs:105-158).
+The chunked pass must leave the caches that loop leaves, so: greedy ids after the prompt identical to the oracle's,
+logits at the last prompt position within 1e-2 of the oracle's (the bar of every model test) and within 1e-4 of the
+device's own token-by-token result (same kernels per token, only the attention's summation order can differ), cache
+rows equal to the token-by-token ones within f16 rounding."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gpu_common import backend, rel_err  # noqa: F401
+from test_gpu_models import oracle_llama
+from slai_amd import _ffi
+from slai_amd import gguf_writer as gw
+from slai_amd.runtime import Gguf, Llama2, SlaiError
+
+pytestmark = pytest.mark.gpu
+LOGIT_TOL = 1e-2      # against the oracle
+SELF_TOL = 1e-4       # against the device's token-by-token pass
+CACHE_TOL = 2e-3      # cache rows, relative to the largest entry (f16 rounding of values that differ in the last bits)
+
+
+def read_cache(backend, m, layer, nbytes):
+    k, v = m.kv_buffers(layer)
+    out = []
+    for h in (k, v):
+        a = np.empty(nbytes, np.uint8)
+        backend.check(backend.L.slai_read_buffer(backend.h, h, 0, a.ctypes.data, a.nbytes))
+        out.append(a)
+    return out
+
+
+def check_prefill(backend, data, prompt, n_gen, chunks, kv_f16, model_type=_ffi.MODEL_LLAMA, neox=0, name=b"llama", expect_path=2,
+                  split_at=None):
+    g, om = oracle_llama(data, 1, neox, int(kv_f16), name)
+    L = g.L
+    prompt = np.asarray(prompt, np.int32)
+    n = prompt.size
+    n_steps = n - 1 + n_gen
+    gg = Gguf(data)
+    kv = _ffi.KV_F16 if kv_f16 else _ffi.KV_F32
+    m = Llama2(backend, gg, model_type, kv)
+    vocab = m.config.vocab_size
+    kv_dim = m.config.dim * m.config.n_kv_heads // m.config.n_q_heads
+    ref_tokens = np.zeros(n_steps, np.int32)
+    ref_logits = np.zeros((n_steps, vocab), np.float32)
+    assert L.slo_llama2_generate(om, prompt.ctypes.data, n, 0, n_steps, -1, ref_tokens.ctypes.data, ref_logits.ctypes.data) == n_steps
+    assert m.prefill_path() == expect_path
+    # the token-by-token device pass: caches and the logits at the last prompt position
+    m.generate(prompt, n - 1)
+    esz = 2 if kv_f16 else 4
+    row_bytes = kv_dim * esz
+    base = [read_cache(backend, m, l, (n - 1) * row_bytes) for l in range(m.config.n_layers)]
+    base_logits = m.forward_logits(n - 1, int(prompt[-1]), fused=True)
+    m.destroy()
+    dt = np.float16 if kv_f16 else np.float32
+    for chunk in chunks:
+        m = Llama2(backend, gg, model_type, kv)
+        if split_at is None:
+            m.prefill(prompt[:-1], 0, chunk)
+        else:                                               # two calls: the second continues at a later position
+            m.prefill(prompt[:split_at], 0, chunk)
+            m.prefill(prompt[split_at:-1], split_at, chunk)
+        for l in range(m.config.n_layers):
+            got = read_cache(backend, m, l, (n - 1) * row_bytes)
+            for a, b in zip(got, base[l]):
+                fa, fb = a.view(dt).astype(np.float32), b.view(dt).astype(np.float32)
+                assert np.abs(fa - fb).max() <= CACHE_TOL * np.abs(fb).max(), (chunk, l)
+        logits = m.forward_logits(n - 1, int(prompt[-1]), fused=True)
+        assert rel_err(logits, ref_logits[n - 1]) < LOGIT_TOL, chunk
+        assert rel_err(logits, base_logits) < SELF_TOL, (chunk, rel_err(logits, base_logits))
+        got, _ = m.generate(prompt, n_gen, start_pos=n - 1)
+        assert np.array_equal(got, ref_tokens[n - 1:]), (chunk, got.tolist(), ref_tokens[n - 1:].tolist())
+        m.destroy()
+    gg.close(); L.slo_llama2_free(om); g.close()
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+def test_prefill_matrix_cores_kquants_gqa_ragged_chunks(backend, kv_f16):
+    """Q4_K with Q6_K v / output, grouped-query attention (4 query heads per kv head), head size 128; a prompt of 45
+    tokens in chunks of 1 (the plain loop), 5, 32 (ragged last chunk) and 64 (clamped to 32)."""
+    data = gw.llama_gguf(dim=1024, hidden_dim=2048, n_layers=3, n_heads=8, n_kv_heads=2, vocab=1000, seq_len=64,
+                         wtype=12, v_type=14, out_type=14, embd_type=12, seed=11, std=0.04, norm_random=True)
+    prompt = np.random.Generator(np.random.PCG64(8)).integers(0, 1000, 45)
+    check_prefill(backend, data, prompt, 16, [1, 5, 32, 64], kv_f16, expect_path=2)
+
+
+@pytest.mark.parametrize("wtype", [13, 14], ids=["q5_k", "q6_k"])
+def test_prefill_matrix_cores_other_kquants(backend, wtype):
+    """Every matrix in Q5_K / Q6_K, head size 64, multi-head attention."""
+    data = gw.llama_gguf(dim=1024, hidden_dim=1024, n_layers=2, n_heads=16, n_kv_heads=16, vocab=800, seq_len=64, wtype=wtype, seed=5 + wtype,
+                         std=0.04, norm_random=True)
+    prompt = np.random.Generator(np.random.PCG64(wtype)).integers(0, 800, 37)
+    check_prefill(backend, data, prompt, 12, [32], True, expect_path=2)
+
+
+def test_prefill_7b_width_head_128(backend):
+    """The shapes of BASELINE configuration 4 at depth 2 (dim 4096, hidden 11008, 32 heads of 128, fp16 cache): here
+    the token-by-token pass runs q/k/v and attention as one launch, the chunked pass as three."""
+    data = gw.llama_gguf(dim=4096, hidden_dim=11008, n_layers=2, n_heads=32, n_kv_heads=32, vocab=32000, seq_len=128,
+                         wtype=12, v_type=14, out_type=14, embd_type=12, seed=41)
+    prompt = np.random.Generator(np.random.PCG64(41)).integers(0, 32000, 41)
+    check_prefill(backend, data, prompt, 12, [8, 32], True, expect_path=2)
+
+
+def test_prefill_matrix_cores_qwen2_bias_neox(backend):
+    """Qwen2: q/k/v biases and Neox pairs in the chunk's bias + RoPE + cache-write launch."""
+    data = gw.llama_gguf(dim=1024, hidden_dim=1024, n_layers=2, n_heads=8, n_kv_heads=2, vocab=400, seq_len=48, wtype=12,
+                         seed=31, std=0.05, arch="qwen2", bias=True, norm_random=True, rope_base=1000000.0, rms_eps=1e-6)
+    prompt = np.random.Generator(np.random.PCG64(3)).integers(0, 400, 35)
+    check_prefill(backend, data, prompt, 12, [32], True, model_type=_ffi.MODEL_QWEN2, neox=1, name=b"qwen2", expect_path=2)
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+def test_prefill_shared_weights_kquants_gqa_ragged_chunks(backend, kv_f16):
+    """A width (512) whose attention output matrix gets 32-row tiles: the chunks then go through the GEMV kernels, one
+    workgroup per token and tile.  Chunks of 3, 8 (ragged last chunk) and 32 (one chunk)."""
+    data = gw.llama_gguf(dim=512, hidden_dim=2816, n_layers=3, n_heads=8, n_kv_heads=2, vocab=1000, seq_len=64,
+                         wtype=12, v_type=14, out_type=14, embd_type=12, seed=11, std=0.06, norm_random=True)
+    prompt = np.random.Generator(np.random.PCG64(8)).integers(0, 1000, 22)
+    check_prefill(backend, data, prompt, 16, [3, 8, 32], kv_f16, expect_path=1)
+
+
+def test_prefill_shared_weights_q4_0_qwen2(backend):
+    """Q4_0 has no matrix-core kernel; q/k/v biases and Neox pairs."""
+    data = gw.llama_gguf(dim=1024, hidden_dim=1024, n_layers=2, n_heads=8, n_kv_heads=2, vocab=400, seq_len=48, wtype=2,
+                         seed=31, std=0.05, arch="qwen2", bias=True, norm_random=True, rope_base=1000000.0, rms_eps=1e-6)
+    prompt = np.random.Generator(np.random.PCG64(3)).integers(0, 400, 19)
+    check_prefill(backend, data, prompt, 12, [4, 8], True, model_type=_ffi.MODEL_QWEN2, neox=1, name=b"qwen2", expect_path=1)
+
+
+def test_prefill_continues_at_a_later_position(backend):
+    data = gw.llama_gguf(dim=1024, hidden_dim=2048, n_layers=2, n_heads=8, n_kv_heads=8, vocab=2048, seq_len=128, wtype=13, seed=77,
+                         std=0.04, norm_random=True)
+    prompt = np.random.Generator(np.random.PCG64(5)).integers(0, 2048, 80)
+    check_prefill(backend, data, prompt, 10, [32], True, split_at=13, expect_path=2)
+
+
+def test_prefill_falls_back_to_the_token_loop_for_other_layouts(backend):
+    """Widths that are no multiple of 256 keep the row layout, which has no chunked kernels: the call then runs the
+    ordinary loop and still leaves the same caches."""
+    data = gw.tiny_llama_gguf(seed=99, std=0.1, norm_random=True, vocab=4096)
+    prompt = np.random.Generator(np.random.PCG64(5)).integers(0, 4096, 12)
+    check_prefill(backend, data, prompt, 10, [8], False, expect_path=0)
+
+
+def test_prefill_argument_errors(backend):
+    data = gw.llama_gguf(dim=256, hidden_dim=512, n_layers=1, n_heads=4, n_kv_heads=4, vocab=300, seq_len=16, wtype=12, seed=2)
+    gg = Gguf(data)
+    m = Llama2(backend, gg, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+    assert m.prefill(np.zeros(0, np.int32)) == 0.0                       # nothing to do
+    with pytest.raises(SlaiError):
+        m.prefill(np.arange(17, dtype=np.int32))                         # past the context
+    with pytest.raises(SlaiError):
+        m.prefill(np.arange(10, dtype=np.int32), start_pos=8)
+    with pytest.raises(SlaiError):
+        m.prefill(np.array([1, 300], np.int32))                          # token out of range
+    with pytest.raises(SlaiError):
+        m.prefill(np.array([1, -1], np.int32))
+    with pytest.raises(SlaiError):
+        m.prefill(np.array([1, 2, 3], np.int32), chunk=65)
+    m.prefill(np.arange(16, dtype=np.int32))                             # exactly the context
+    m.destroy(); gg.close()
