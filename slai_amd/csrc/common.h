@@ -80,6 +80,7 @@ enum : uint32_t {
     GEMV_SILU_GATE = 4u, // dual: val = up * gate/(1+exp(-gate))   (W = gate, W2 = up)
     GEMV_GELU = 8u,      // val = gelu(val)
     GEMV_EMIT = 16u,     // also write the weighted copy of the result for the next row-tile GEMV (tiled kernel only)
+    GEMM_OUT_QUADS = 32u, // prompt-chunk GEMM only: write the result quad-major (the layout its input has)
 };
 enum : int { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_LAYERNORM = 2 };
 
@@ -174,9 +175,11 @@ size_t gemv_rowtile_scratch_floats(const GemvRowtileParams &p);
 hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p, const GemvBatch *batch = nullptr);
 
 // A chunk of up to 32 input vectors ("prompt tokens") through up to three matrices on the matrix cores
-// (kernels_gemm_chunk.hip): out[t][r] = sum_c deq(W[r][c]) * x[t][c] (+ bias[r]) (+ the old out[t][r]), token t at
-// x + t * x_stride and out + t * out_stride.  K-quants in 64-row tiles (any number of segments, formats may differ) or in
-// 16-row tiles of at most 16 column groups (one segment).
+// (kernels_gemm_chunk.hip): out[t][r] = sum_c deq(W[r][c]) * x[t][c] (+ bias[r]) (+ the old out[t][r]).  The input is
+// "quad-major": the float4 of columns c .. c + 3 of token t at x + ((c / 4) * 32 + t) * 4 (32 token slots whatever
+// ntokens is); the output is row-major (token t at out + t * out_stride) or, with GEMM_OUT_QUADS, quad-major as well.
+// K-quants in 64-row tiles (any number of segments, formats may differ) or in 16-row tiles of at most 16 column groups
+// (one segment).
 struct GemmChunkSeg {
     const uint8_t *W = nullptr;
     int type = 0;
@@ -184,21 +187,22 @@ struct GemmChunkSeg {
     uint32_t ntiles = 0;   // filled by the launcher
     float *out = nullptr;
     const float *bias = nullptr;
-    uint32_t flags = 0;    // GEMV_BIAS, GEMV_ACCUM
+    uint32_t flags = 0;    // GEMV_BIAS, GEMV_ACCUM, GEMM_OUT_QUADS
     uint32_t out_stride = 0;
 };
 struct GemmChunkParams {
     GemmChunkSeg seg[3];
     int nseg = 1;
     uint32_t ncols = 0, ncb = 0, ngroups = 0, rows_log2 = 6;
-    const float *x = nullptr;   // 16-byte aligned
-    uint32_t x_stride = 0;      // floats, a multiple of 4
+    const float *x = nullptr;   // quad-major, 16-byte aligned
     uint32_t ntokens = 0;
 };
 bool gemm_chunk_supports(const slai_qmat *m);
 hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p);
-// out[t][i] = (x[t][i] / sqrt(mean(x[t]^2) + eps)) * w[i] for `rows` vectors of n floats
-hipError_t launch_rms_norm_rows(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t rows, uint32_t out_stride, uint32_t x_stride, float eps);
+// quad-major out = RMSNorm of the `ntokens` row-major vectors of n floats at x + t * x_stride
+hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps);
+// quad-major copy of row-major vectors
+hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride);
 
 // One GEMV launch over up to three matrices of one format and layout: out[i] = epilogue(m[i] . prologue(x)).
 struct GemvCall {

@@ -433,6 +433,7 @@ bool slai_llama2::chunk_supported() const {
 
 int slai_llama2::chunk_reserve(uint32_t rows) {
     PromptChunkState &c = chunk;
+    if (rows < 32) rows = 32;                                   // the quad-major buffers always have 32 token slots
     if (rows <= c.rows) return SLAI_OK;
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "prompt chunk buffers must be reserved before graph capture");
     TRY(slai_synchronize(ctx));
@@ -559,13 +560,13 @@ bool slai_llama2::chunk_gemm_supported() const {
 namespace {
 // matrices (with the same input) through the matrix-core kernel: 64-row-tile matrices share a launch
 int gemm_chunk_call(slai_ctx *ctx, int nmat, const slai_qmat *const *mats, float *const *outs, const uint32_t *out_strides, uint32_t flags,
-                    const float *x, uint32_t x_stride, uint32_t ntokens, const char *who) {
+                    const float *xq, uint32_t ntokens, const char *who) {
     bool done[3] = {false, false, false};
     for (int i = 0; i < nmat; ++i) {
         if (done[i]) continue;
         GemmChunkParams p;
         p.nseg = 0; p.ncols = mats[i]->ncols; p.ncb = mats[i]->ncb; p.ngroups = mats[i]->ngroups; p.rows_log2 = mats[i]->rows_log2;
-        p.x = x; p.x_stride = x_stride; p.ntokens = ntokens;
+        p.x = xq; p.ntokens = ntokens;
         for (int j = i; j < nmat; ++j) {
             if (done[j] || (j != i && (mats[j]->rows_log2 != 6 || mats[i]->rows_log2 != 6 || mats[j]->ncols != mats[i]->ncols))) continue;
             GemmChunkSeg &sg = p.seg[p.nseg++];
@@ -591,35 +592,38 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
     float *k = (float *)pc.k.buf->dptr, *v = (float *)pc.v.buf->dptr, *hb = (float *)pc.hb.buf->dptr, *hb2 = (float *)pc.hb2.buf->dptr;
     for (uint32_t b = 0; b < n; ++b)
         SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, tokens_dev + b, nullptr, nullptr, dim, x + (size_t)b * dim));
+    // xn, xb -> xq (via xn) and hb, hb2 are quad-major with 32 token slots: the layout the GEMM kernels read
     for (uint32_t l = 0; l < config.n_layers; ++l) {
         const Llama2LayerWeights &wl = weights.layers[l];
-        SLAI_HIP_TRY(ctx, launch_rms_norm_rows(ctx->stream, xn, x, (const float *)wl.attn_norm.buf->dptr, dim, n, dim, dim, config.rms_norm_eps));
+        SLAI_HIP_TRY(ctx, launch_rms_norm_quads(ctx->stream, xn, x, (const float *)wl.attn_norm.buf->dptr, dim, n, dim, config.rms_norm_eps));
         {
             const slai_qmat *mats[3] = {wl.attn_v, wl.attn_k, wl.attn_q};
             float *outs[3] = {v, k, q};
             const uint32_t strides[3] = {kvd, kvd, dim};
-            TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, dim, n, "llama2 qkv (prompt chunk)"));
+            TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)"));
         }
         TRY(chunk_attention(l, pos0, n));
+        SLAI_HIP_TRY(ctx, launch_rows_to_quads(ctx->stream, xn, xb, dim, n, dim));
         {
             const slai_qmat *mats[1] = {wl.attn_output};
             float *outs[1] = {x};
             const uint32_t strides[1] = {dim};
-            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, xb, dim, n, "llama2 attn_output (prompt chunk)"));
+            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, xn, n, "llama2 attn_output (prompt chunk)"));
         }
-        SLAI_HIP_TRY(ctx, launch_rms_norm_rows(ctx->stream, xn, x, (const float *)wl.ffn_norm.buf->dptr, dim, n, dim, dim, config.rms_norm_eps));
+        SLAI_HIP_TRY(ctx, launch_rms_norm_quads(ctx->stream, xn, x, (const float *)wl.ffn_norm.buf->dptr, dim, n, dim, config.rms_norm_eps));
         {
             const slai_qmat *mats[2] = {wl.ffn_gate, wl.ffn_up};
             float *outs[2] = {hb, hb2};
             const uint32_t strides[2] = {hid, hid};
-            TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, 0, xn, dim, n, "llama2 ffn gate/up (prompt chunk)"));
+            TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, GEMM_OUT_QUADS, xn, n, "llama2 ffn gate/up (prompt chunk)"));
         }
-        SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, n * hid, 1}, VecView{hb2, n * hid, 1}));
+        // element-wise, so the layout does not matter (slots of tokens past the chunk hold stale values nobody reads)
+        SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, 32 * hid, 1}, VecView{hb2, 32 * hid, 1}));
         {
             const slai_qmat *mats[1] = {wl.ffn_down};
             float *outs[1] = {x};
             const uint32_t strides[1] = {dim};
-            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, hb, hid, n, "llama2 ffn_down (prompt chunk)"));
+            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, hb, n, "llama2 ffn_down (prompt chunk)"));
         }
     }
     return SLAI_OK;

@@ -14,8 +14,13 @@
 //                                         instruction advances FOUR columns (one per super-block) for 16 rows x 16
 //                                         tokens; two instructions cover 32 tokens; the four blocks are added at the end.
 // One lane register of weights thus feeds 64 x 32 multiply-adds; the activations (32 tokens x ncols floats, a few
-// hundred KB) are read straight from L2, 16 bytes (four consecutive columns of the lane's token) per load.  A wave
-// owns whole super-blocks; the waves of a workgroup meet in LDS once per tile.
+// hundred KB) are read straight from L2, 16 bytes (four consecutive columns of the lane's token) per load.  They are
+// stored "quad-major" for that: xq[(c / 4) * 32 + t] is the float4 of columns c .. c + 3 of token t, so the 32 tokens
+// of one load instruction are 512 contiguous bytes (row-major activations would touch 32 cache lines per load and
+// saturate L1 and L2 with quarter-used lines).  A wave owns whole super-blocks; the waves of a workgroup meet in LDS
+// once per tile.
+#include <algorithm>
+
 #include "common.h"
 #include "device_util.h"
 #include "quant_tiled.h"
@@ -125,12 +130,13 @@ template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, 
 // ---- 64-row tiles ------------------------------------------------------------------------------------------------------
 struct X64 { float4 a[4], b[4]; };                             // the lane's token: chunks c1 and c2 of a stage, four columns per entry
 
-template <int T, int K> __device__ __forceinline__ void request_x64(const float *xcb, X64 &x) {
+// xcb: the lane's token in the first quad of the super-block; consecutive quads are 32 float4 apart
+template <int T, int K> __device__ __forceinline__ void request_x64(const float4 *xcb, X64 &x) {
     using F = Tiled<T>;
 #pragma unroll
     for (int W = 0; W < 4; ++W) {
-        x.a[W] = *(const float4 *)(xcb + 16 * F::c1(K) + 4 * W);
-        x.b[W] = *(const float4 *)(xcb + 16 * F::c2(K) + 4 * W);
+        x.a[W] = xcb[(4 * F::c1(K) + W) * 32];
+        x.b[W] = xcb[(4 * F::c2(K) + W) * 32];
     }
 }
 
@@ -148,49 +154,39 @@ template <int T, int K, int W> __device__ __forceinline__ void mac64(const Deq<T
     acc = __builtin_amdgcn_mfma_f32_32x32x1f32(hi[3], xb.w, acc, 0, 0, 0);
 }
 
-// stage K of the current super-block: request the activations of the next stage (`xnext`: those of stage 0 of the wave's
-// next super-block after the last stage), multiply, move on
-template <int T, int K> __device__ __forceinline__ void stages64(const Deq<T> &q, const typename Tiled<T>::Data &d, const float *xcb, const float *xcb_next,
-                                                                  X64 &x, f32x32 &acc) {
-    X64 nx;
+// stage K of the current super-block: request the activations of the next stage, multiply, move on
+template <int T, int K> __device__ __forceinline__ void stages64(const Deq<T> &q, const typename Tiled<T>::Data &d, const float4 *xcb, X64 &x, f32x32 &acc) {
+    X64 nx = x;
     if constexpr (K < 7) request_x64<T, K + 1>(xcb, nx);
-    else request_x64<T, 0>(xcb_next, nx);
     mac64<T, K, 0>(q, d, x, acc); mac64<T, K, 1>(q, d, x, acc); mac64<T, K, 2>(q, d, x, acc); mac64<T, K, 3>(q, d, x, acc);
     x = nx;
-    if constexpr (K < 7) stages64<T, K + 1>(q, d, xcb, xcb_next, x, acc);
+    if constexpr (K < 7) stages64<T, K + 1>(q, d, xcb, x, acc);
 }
 
-constexpr int G64_WAVES = 4;
 constexpr int G64_LDS_ROW = 68;                                // floats per token in the LDS partials (64 rows + padding)
 
+// The activation loads run only a stage ahead of their use (more would not fit the registers), which is less than an
+// L2 round trip: the matrix pipe is kept busy by several waves per SIMD instead, each with a super-block of its own.
 template <int T>
 __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const GemmChunkSeg &seg, uint32_t tile, float *part) {
     using F = Tiled<T>;
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63, NW = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
     const uint32_t token = min((uint32_t)(lane & 31), p.ntokens - 1);            // lanes past the chunk repeat its last token
-    const float *xrow = p.x + (size_t)token * p.x_stride;
+    const float4 *xrow = (const float4 *)p.x + token;                             // + 64 * 32 per super-block
     f32x32 acc;
 #pragma unroll
     for (int i = 0; i < 32; ++i) acc[i] = 0.0f;
-    typename F::Data d, dn;
-    uint16_t dt = 0, dnt = 0;
-    uint32_t cb = wave;
-    X64 x;
-    if (cb < p.ncb) {
+    for (uint32_t cb = wave; cb < p.ncb; cb += NW) {
+        typename F::Data d;
+        uint16_t dt = 0;
+        X64 x;
         load_unit<T>(seg.W + ((size_t)tile * p.ncb + cb) * unit_bytes, lane, d, dt);
-        request_x64<T, 0>(xrow + (size_t)cb * 256, x);
-    }
-    while (cb < p.ncb) {
-        const uint32_t nb = cb + G64_WAVES;
-        const bool more = nb < p.ncb;
-        if (more) load_unit<T>(seg.W + ((size_t)tile * p.ncb + nb) * unit_bytes, lane, dn, dnt);
+        request_x64<T, 0>(xrow + (size_t)cb * 2048, x);
         Deq<T> q;
         q.head(d, dt);
-        stages64<T, 0>(q, d, xrow + (size_t)cb * 256, xrow + (size_t)(more ? nb : cb) * 256, x, acc);
-        if (more) { d = dn; dt = dnt; }
-        cb = nb;
+        stages64<T, 0>(q, d, xrow + (size_t)cb * 2048, x, acc);
     }
     // ---- the waves meet: part[wave][token][row]; register v of block b holds row 32b + 8(v/4) + 4(lane/32) + v%4 of token lane%32
     float *mine = part + (size_t)wave * 32 * G64_LDS_ROW + (size_t)(lane & 31) * G64_LDS_ROW + 4 * (lane >> 5);
@@ -200,15 +196,13 @@ __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const Gemm
         for (int g = 0; g < 4; ++g)
             *(float4 *)(mine + 32 * b + 8 * g) = make_float4(acc[16 * b + 4 * g], acc[16 * b + 4 * g + 1], acc[16 * b + 4 * g + 2], acc[16 * b + 4 * g + 3]);
     lds_barrier();
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const uint32_t idx = (uint32_t)tid + 256u * e, r = idx & 63u, t = idx >> 6;
+    for (uint32_t idx = tid; idx < 2048; idx += blockDim.x) {
+        const uint32_t r = idx & 63u, t = idx >> 6;
         const uint32_t row = tile * 64 + r;
         if (t < p.ntokens && row < seg.nrows) {
             float o = 0.0f;
-#pragma unroll
-            for (int w = 0; w < G64_WAVES; ++w) o += part[(size_t)w * 32 * G64_LDS_ROW + (size_t)t * G64_LDS_ROW + r];
-            float *dst = seg.out + (size_t)t * seg.out_stride + row;
+            for (int w = 0; w < NW; ++w) o += part[(size_t)w * 32 * G64_LDS_ROW + (size_t)t * G64_LDS_ROW + r];
+            float *dst = (seg.flags & GEMM_OUT_QUADS) ? seg.out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3) : seg.out + (size_t)t * seg.out_stride + row;
             if (seg.flags & GEMV_BIAS) o += seg.bias[row];
             if (seg.flags & GEMV_ACCUM) o = *dst + o;
             *dst = o;
@@ -216,10 +210,10 @@ __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const Gemm
     }
 }
 
-// grid = tiles of all segments, block = 256 (four waves, each a quarter of the super-blocks)
-template <int TT>
-__global__ void __launch_bounds__(256) gemm64_kernel(const GemmChunkParams p) {
-    __shared__ float part[G64_WAVES * 32 * G64_LDS_ROW];
+// grid = tiles of all segments, block = 64 * (waves: each takes every NW-th super-block)
+template <int TT, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemm64_kernel(const GemmChunkParams p) {
+    extern __shared__ float part[];                            // [waves][32 tokens][G64_LDS_ROW]
     touch_kernel_arguments<sizeof(GemmChunkParams)>();
     const uint32_t n0 = p.seg[0].ntiles, n1 = p.seg[1].ntiles;
     uint32_t tile = blockIdx.x;
@@ -246,78 +240,89 @@ __global__ void __launch_bounds__(256) gemm64_kernel(const GemmChunkParams p) {
 }
 
 // ---- 16-row tiles ------------------------------------------------------------------------------------------------------
-struct X16 { float4 a0, b0, a1, b1; };                         // tokens lane%16 (0) and 16 + lane%16 (1): four columns of chunk c1 (a) and c2 (b)
+// NACC = 2: the workgroup serves all 32 tokens (two accumulators: tokens lane % 16 and 16 + lane % 16); NACC = 1: 16 of
+// them, the half given by blockIdx.y (narrow matrices: twice the workgroups, so that every SIMD has several waves).
+template <int NACC> struct X16 { float4 a[NACC], b[NACC]; };    // four columns of chunk c1 (a) and c2 (b) per token
 
-template <int T, int K, int W> __device__ __forceinline__ void request_x16(const float *x0, const float *x1, X16 &x) {
+template <int T, int K, int W, int NACC> __device__ __forceinline__ void request_x16(const float4 *const (&xt)[NACC], X16<NACC> &x) {
     using F = Tiled<T>;
-    x.a0 = *(const float4 *)(x0 + 16 * F::c1(K) + 4 * W); x.b0 = *(const float4 *)(x0 + 16 * F::c2(K) + 4 * W);
-    x.a1 = *(const float4 *)(x1 + 16 * F::c1(K) + 4 * W); x.b1 = *(const float4 *)(x1 + 16 * F::c2(K) + 4 * W);
+#pragma unroll
+    for (int n = 0; n < NACC; ++n) { x.a[n] = xt[n][(4 * F::c1(K) + W) * 32]; x.b[n] = xt[n][(4 * F::c2(K) + W) * 32]; }
 }
 
-template <int T, int K, int W> __device__ __forceinline__ void steps16(const Deq<T> &q, const typename Tiled<T>::Data &d, const float *x0, const float *x1,
-                                                                       X16 &x, f32x16 &acc0, f32x16 &acc1) {
+template <int T, int K, int W, int NACC> __device__ __forceinline__ void steps16(const Deq<T> &q, const typename Tiled<T>::Data &d, const float4 *const (&xt)[NACC],
+                                                                                 X16<NACC> &x, f32x16 (&acc)[NACC]) {
     constexpr int NK = W == 3 ? K + 1 : K, NW = W == 3 ? 0 : W + 1;
-    X16 nx = x;
-    if constexpr (NK < 8) request_x16<T, NK, NW>(x0, x1, nx);
+    X16<NACC> nx = x;
+    if constexpr (NK < 8) request_x16<T, NK, NW, NACC>(xt, nx);
     float lo[4], hi[4];
     q.template quad<K, W>(d, lo, hi);
-    const float xa0[4] = {x.a0.x, x.a0.y, x.a0.z, x.a0.w}, xb0[4] = {x.b0.x, x.b0.y, x.b0.z, x.b0.w};
-    const float xa1[4] = {x.a1.x, x.a1.y, x.a1.z, x.a1.w}, xb1[4] = {x.b1.x, x.b1.y, x.b1.z, x.b1.w};
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-        acc0 = __builtin_amdgcn_mfma_f32_16x16x1f32(lo[b], xa0[b], acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_16x16x1f32(lo[b], xa1[b], acc1, 0, 0, 0);
-        acc0 = __builtin_amdgcn_mfma_f32_16x16x1f32(hi[b], xb0[b], acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_16x16x1f32(hi[b], xb1[b], acc1, 0, 0, 0);
+#pragma unroll
+        for (int n = 0; n < NACC; ++n) {
+            const float xa = b == 0 ? x.a[n].x : (b == 1 ? x.a[n].y : (b == 2 ? x.a[n].z : x.a[n].w));
+            acc[n] = __builtin_amdgcn_mfma_f32_16x16x1f32(lo[b], xa, acc[n], 0, 0, 0);
+        }
+#pragma unroll
+        for (int n = 0; n < NACC; ++n) {
+            const float xb = b == 0 ? x.b[n].x : (b == 1 ? x.b[n].y : (b == 2 ? x.b[n].z : x.b[n].w));
+            acc[n] = __builtin_amdgcn_mfma_f32_16x16x1f32(hi[b], xb, acc[n], 0, 0, 0);
+        }
     }
     x = nx;
-    if constexpr (NK < 8) steps16<T, NK, NW>(q, d, x0, x1, x, acc0, acc1);
+    if constexpr (NK < 8) steps16<T, NK, NW, NACC>(q, d, xt, x, acc);
 }
 
 constexpr int G16_LDS_ROW = 20;                                // floats per token in the LDS partials (16 rows + padding)
 
-// grid = tiles, block = 64 * ngroups (one wave per column group of four super-blocks)
-template <int T, int MAXT>
+// grid = (tiles, 2 / NACC), block = 64 * ngroups (one wave per column group of four super-blocks)
+template <int T, int MAXT, int NACC>
 __global__ void __launch_bounds__(MAXT) gemm16_kernel(const GemmChunkParams p) {
     using F = Tiled<T>;
-    extern __shared__ float part[];                            // [waves][32 tokens][G16_LDS_ROW]
+    extern __shared__ float part[];                            // [waves][16 * NACC tokens][G16_LDS_ROW]
     touch_kernel_arguments<sizeof(GemmChunkParams)>();
     const int tid = threadIdx.x, lane = tid & 63, NW = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = blockIdx.x, tbase = NACC == 2 ? 0u : 16u * blockIdx.y;
+    if (tbase >= p.ntokens) return;                            // (uniform) a short chunk has no second half
     const uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
     const uint32_t cb = min((uint32_t)wave * 4 + (uint32_t)(lane >> 4), p.ncb - 1);   // (super-blocks past the end are zero weights)
-    const uint32_t t0 = min((uint32_t)(lane & 15), p.ntokens - 1), t1 = min(16u + (uint32_t)(lane & 15), p.ntokens - 1);
-    const float *x0 = p.x + (size_t)t0 * p.x_stride + (size_t)cb * 256, *x1 = p.x + (size_t)t1 * p.x_stride + (size_t)cb * 256;
+    const float4 *xt[NACC];
+#pragma unroll
+    for (int n = 0; n < NACC; ++n) xt[n] = (const float4 *)p.x + (size_t)cb * 2048 + min(tbase + 16u * n + (uint32_t)(lane & 15), p.ntokens - 1);
     typename F::Data d;
     uint16_t dt = 0;
     load_unit<T>(p.seg[0].W + ((size_t)tile * p.ngroups + wave) * unit_bytes, lane, d, dt);
-    X16 x;
-    request_x16<T, 0, 0>(x0, x1, x);
-    f32x16 acc0, acc1;
+    X16<NACC> x;
+    request_x16<T, 0, 0, NACC>(xt, x);
+    f32x16 acc[NACC];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; }
+    for (int n = 0; n < NACC; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[n][i] = 0.0f;
     Deq<T> q;
     q.head(d, dt);
-    steps16<T, 0, 0>(q, d, x0, x1, x, acc0, acc1);
+    steps16<T, 0, 0, NACC>(q, d, xt, x, acc);
     // the four blocks hold the same rows and tokens over different super-blocks: add them.  Register v of a block holds
     // row 4 * (lane / 16) + v of token lane % 16.
-    float4 s0, s1;
-    s0.x = (acc0[0] + acc0[4]) + (acc0[8] + acc0[12]); s0.y = (acc0[1] + acc0[5]) + (acc0[9] + acc0[13]);
-    s0.z = (acc0[2] + acc0[6]) + (acc0[10] + acc0[14]); s0.w = (acc0[3] + acc0[7]) + (acc0[11] + acc0[15]);
-    s1.x = (acc1[0] + acc1[4]) + (acc1[8] + acc1[12]); s1.y = (acc1[1] + acc1[5]) + (acc1[9] + acc1[13]);
-    s1.z = (acc1[2] + acc1[6]) + (acc1[10] + acc1[14]); s1.w = (acc1[3] + acc1[7]) + (acc1[11] + acc1[15]);
-    float *mine = part + (size_t)wave * 32 * G16_LDS_ROW + 4 * (lane >> 4);
-    *(float4 *)(mine + (size_t)(lane & 15) * G16_LDS_ROW) = s0;
-    *(float4 *)(mine + (size_t)(16 + (lane & 15)) * G16_LDS_ROW) = s1;
+    float *mine = part + (size_t)wave * 16 * NACC * G16_LDS_ROW + 4 * (lane >> 4);
+#pragma unroll
+    for (int n = 0; n < NACC; ++n) {
+        float4 sm;
+        sm.x = (acc[n][0] + acc[n][4]) + (acc[n][8] + acc[n][12]); sm.y = (acc[n][1] + acc[n][5]) + (acc[n][9] + acc[n][13]);
+        sm.z = (acc[n][2] + acc[n][6]) + (acc[n][10] + acc[n][14]); sm.w = (acc[n][3] + acc[n][7]) + (acc[n][11] + acc[n][15]);
+        *(float4 *)(mine + (size_t)(16 * n + (lane & 15)) * G16_LDS_ROW) = sm;
+    }
     lds_barrier();
-    for (uint32_t idx = tid; idx < 512; idx += blockDim.x) {
-        const uint32_t r = idx & 15u, t = idx >> 4;
+    for (uint32_t idx = tid; idx < 256u * NACC; idx += blockDim.x) {
+        const uint32_t r = idx & 15u, tl = idx >> 4, t = tbase + tl;
         const uint32_t row = tile * 16 + r;
         if (t < p.ntokens && row < p.seg[0].nrows) {
             float o = 0.0f;
-            for (int w = 0; w < NW; ++w) o += part[(size_t)w * 32 * G16_LDS_ROW + (size_t)t * G16_LDS_ROW + r];
-            float *dst = p.seg[0].out + (size_t)t * p.seg[0].out_stride + row;
+            for (int w = 0; w < NW; ++w) o += part[(size_t)w * 16 * NACC * G16_LDS_ROW + (size_t)tl * G16_LDS_ROW + r];
+            float *dst = (p.seg[0].flags & GEMM_OUT_QUADS) ? p.seg[0].out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3)
+                                                           : p.seg[0].out + (size_t)t * p.seg[0].out_stride + row;
             if (p.seg[0].flags & GEMV_BIAS) o += p.seg[0].bias[row];
             if (p.seg[0].flags & GEMV_ACCUM) o = *dst + o;
             *dst = o;
@@ -325,19 +330,38 @@ __global__ void __launch_bounds__(MAXT) gemm16_kernel(const GemmChunkParams p) {
     }
 }
 
-// out[t][i] = (x[t][i] * 1/sqrt(mean(x[t]^2) + eps)) * w[i] (rms_norm.slang:48-67), one workgroup per token
-__global__ void __launch_bounds__(256) rms_norm_rows_kernel(float *out, const float *x, const float *w, uint32_t n, uint32_t out_stride, uint32_t x_stride, float eps) {
+// RMSNorm of token t = blockIdx.x (rms_norm.slang:48-67: (x * 1/sqrt(mean(x^2) + eps)) * w), written quad-major for the
+// GEMM kernels above.  n % 4 == 0, n <= 16384 (16 float4 per thread).
+__global__ void __launch_bounds__(256) rms_norm_quads_kernel(float4 *out, const float *x, const float *w, uint32_t n, uint32_t x_stride, float eps) {
     __shared__ float red[4];
-    const float *xr = x + (size_t)blockIdx.x * x_stride;
-    float *o = out + (size_t)blockIdx.x * out_stride;
+    const uint32_t t = blockIdx.x, nq = n / 4;
+    const float4 *xr = (const float4 *)(x + (size_t)t * x_stride), *wr = (const float4 *)w;
+    float4 v[16], g[16];
     float ss = 0.0f;
-    for (uint32_t i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const uint32_t i = threadIdx.x + 256u * j;
+        if (i < nq) {
+            v[j] = xr[i]; g[j] = wr[i];
+            ss = fmaf(v[j].x, v[j].x, ss); ss = fmaf(v[j].y, v[j].y, ss); ss = fmaf(v[j].z, v[j].z, ss); ss = fmaf(v[j].w, v[j].w, ss);
+        }
+    }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float scale = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)n + eps);
-    for (uint32_t i = threadIdx.x; i < n; i += 256) o[i] = (xr[i] * scale) * w[i];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const uint32_t i = threadIdx.x + 256u * j;
+        if (i < nq) out[(size_t)i * 32 + t] = make_float4((v[j].x * scale) * g[j].x, (v[j].y * scale) * g[j].y, (v[j].z * scale) * g[j].z, (v[j].w * scale) * g[j].w);
+    }
+}
+
+// row-major [tokens][n] -> quad-major; thread = (quad, token), token fastest so that the stores are contiguous
+__global__ void rows_to_quads_kernel(float4 *out, const float *x, uint32_t n, uint32_t x_stride, uint32_t ntokens) {
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x, t = idx & 31u, qd = idx >> 5;
+    if (qd < n / 4 && t < ntokens) out[(size_t)qd * 32 + t] = *(const float4 *)(x + (size_t)t * x_stride + 4 * qd);
 }
 
 }  // namespace
@@ -348,14 +372,20 @@ bool gemm_chunk_supports(const slai_qmat *m) {
     return m->rows_log2 == 4 && m->ngroups <= 16;
 }
 
-hipError_t launch_rms_norm_rows(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t rows, uint32_t out_stride, uint32_t x_stride, float eps) {
-    if (rows == 0 || n == 0) return hipErrorInvalidValue;
-    rms_norm_rows_kernel<<<rows, 256, 0, s>>>(out, x, w, n, out_stride, x_stride, eps);
+hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps) {
+    if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || n > 16384 || x_stride % 4) return hipErrorInvalidValue;
+    rms_norm_quads_kernel<<<ntokens, 256, 0, s>>>((float4 *)out, x, w, n, x_stride, eps);
+    return hipGetLastError();
+}
+
+hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride) {
+    if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || x_stride % 4) return hipErrorInvalidValue;
+    rows_to_quads_kernel<<<(n / 4 * 32 + 255) / 256, 256, 0, s>>>((float4 *)out, x, n, x_stride, ntokens);
     return hipGetLastError();
 }
 
 hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
-    if (p.nseg < 1 || p.nseg > 3 || p.ntokens == 0 || p.ntokens > 32 || p.ncb == 0 || p.ncols != p.ncb * 256 || p.x_stride % 4 || ((uintptr_t)p.x & 15))
+    if (p.nseg < 1 || p.nseg > 3 || p.ntokens == 0 || p.ntokens > 32 || p.ncb == 0 || p.ncols != p.ncb * 256 || ((uintptr_t)p.x & 15))
         return hipErrorInvalidValue;
     for (int i = 0; i < p.nseg; ++i)
         if (p.seg[i].type != T_Q4_K && p.seg[i].type != T_Q6_K && p.seg[i].type != T_Q5_K) return hipErrorInvalidValue;
@@ -369,26 +399,31 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
             if (p.seg[i].type != tt) tt = 0;
         }
         for (int i = p.nseg; i < 3; ++i) p.seg[i].ntiles = 0;
+        // up to sixteen waves, one super-block each at the usual widths (every format fits the 128 registers per lane that leaves)
+        const uint32_t nw = std::min(p.ncb, 16u);
+        const size_t smem = (size_t)nw * 32 * G64_LDS_ROW * sizeof(float);
+        const int NT = (int)nw * 64;
         switch (tt) {
-        case T_Q4_K: gemm64_kernel<T_Q4_K><<<tiles, 256, 0, st>>>(p); break;
-        case T_Q6_K: gemm64_kernel<T_Q6_K><<<tiles, 256, 0, st>>>(p); break;
-        case T_Q5_K: gemm64_kernel<T_Q5_K><<<tiles, 256, 0, st>>>(p); break;
-        default: gemm64_kernel<0><<<tiles, 256, 0, st>>>(p); break;
+        case T_Q4_K: gemm64_kernel<T_Q4_K, 1024><<<tiles, NT, smem, st>>>(p); break;
+        case T_Q5_K: gemm64_kernel<T_Q5_K, 1024><<<tiles, NT, smem, st>>>(p); break;
+        case T_Q6_K: gemm64_kernel<T_Q6_K, 1024><<<tiles, NT, smem, st>>>(p); break;
+        default: gemm64_kernel<0, 1024><<<tiles, NT, smem, st>>>(p); break;
         }
         return hipGetLastError();
     }
     if (p.rows_log2 != 4 || p.nseg != 1 || p.ngroups == 0 || p.ngroups > 16) return hipErrorInvalidValue;
     const uint32_t tiles = (p.seg[0].nrows + 15) / 16;
     const int NT = (int)p.ngroups * 64;
-    const size_t smem = (size_t)p.ngroups * 32 * G16_LDS_ROW * sizeof(float);
-    // the thread bound decides the register budget (256 threads leave 256 registers per lane, 1024 leave 128)
-#define SLAI_G16(TY)                                                                         \
-    do {                                                                                     \
-        if (NT <= 256) gemm16_kernel<TY, 256><<<tiles, NT, smem, st>>>(p);                   \
-        else if (NT <= 512) gemm16_kernel<TY, 512><<<tiles, NT, smem, st>>>(p);              \
-        else if (NT <= 768) gemm16_kernel<TY, 768><<<tiles, NT, smem, st>>>(p);              \
-        else gemm16_kernel<TY, 1024><<<tiles, NT, smem, st>>>(p);                            \
+    // the thread bound decides the register budget (256 threads leave 256 registers per lane, 1024 leave 128); narrow
+    // matrices (few waves per workgroup) split the tokens over two workgroups
+#define SLAI_G16(TY)                                                                                       \
+    do {                                                                                                   \
+        if (NT <= 256) gemm16_kernel<TY, 256, 1><<<dim3(tiles, 2), NT, smem1, st>>>(p);                    \
+        else if (NT <= 512) gemm16_kernel<TY, 512, 1><<<dim3(tiles, 2), NT, smem1, st>>>(p);               \
+        else if (NT <= 768) gemm16_kernel<TY, 768, 2><<<tiles, NT, smem2, st>>>(p);                        \
+        else gemm16_kernel<TY, 1024, 2><<<tiles, NT, smem2, st>>>(p);                                      \
     } while (0)
+    const size_t smem1 = (size_t)p.ngroups * 16 * G16_LDS_ROW * sizeof(float), smem2 = 2 * smem1;
     switch (p.seg[0].type) {
     case T_Q4_K: SLAI_G16(T_Q4_K); break;
     case T_Q6_K: SLAI_G16(T_Q6_K); break;

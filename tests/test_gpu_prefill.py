@@ -21,7 +21,7 @@ from slai_amd.runtime import Gguf, Llama2, SlaiError
 
 pytestmark = pytest.mark.gpu
 LOGIT_TOL = 1e-2      # against the oracle
-SELF_TOL = 1e-4       # against the device's token-by-token pass
+SELF_TOL = 1e-3       # against the device's token-by-token pass (fp32 sums in another order; an f16 cache entry may round the other way)
 CACHE_TOL = 2e-3      # cache rows, relative to the largest entry (f16 rounding of values that differ in the last bits)
 
 
