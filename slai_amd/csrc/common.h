@@ -189,6 +189,7 @@ struct GemmChunkSeg {
     const float *bias = nullptr;
     uint32_t flags = 0;    // GEMV_BIAS, GEMV_ACCUM, GEMM_OUT_QUADS
     uint32_t out_stride = 0;
+    uint32_t part_stride = 0;   // ksplit > 1: floats between the partial results
 };
 struct GemmChunkParams {
     GemmChunkSeg seg[3];
@@ -196,6 +197,10 @@ struct GemmChunkParams {
     uint32_t ncols = 0, ncb = 0, ngroups = 0, rows_log2 = 6;
     const float *x = nullptr;   // quad-major, 16-byte aligned
     uint32_t ntokens = 0;
+    // 64-row tiles only.  ksplit > 1: the columns are cut into ksplit ranges of whole super-blocks, each computed by a
+    // workgroup of its own (tile counts rarely divide the compute units evenly; smaller units do); range s writes its
+    // partial result to out + s * part_stride and the reader adds them up.  No bias, no accumulation then.
+    uint32_t ksplit = 1;
 };
 bool gemm_chunk_supports(const slai_qmat *m);
 hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p);
@@ -317,7 +322,12 @@ hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n
 // The step before it: for token b (position pos_ptr[b]) add the biases, rotate q + b * q_stride in place and write the
 // rotated key k + b * kv_stride and the value v + b * kv_stride to row pos_ptr[b] of the caches.  Uses the q / cache /
 // bias / rope fields of `a`.
-hipError_t launch_rope_store_batch(hipStream_t s, const AttnLaunch &a, float *q, const float *k, const float *v, uint32_t n, uint32_t q_stride, uint32_t kv_stride);
+// q, k, v may come as `nparts` partial results to be added first (q + i * q_part, k / v + i * kv_part, i < nparts); the
+// rotated q is written to part 0.
+hipError_t launch_rope_store_batch(hipStream_t s, const AttnLaunch &a, float *q, const float *k, const float *v, uint32_t n, uint32_t q_stride, uint32_t kv_stride,
+                                   uint32_t nparts = 1, uint32_t q_part = 0, uint32_t kv_part = 0);
+// a[i] = silu(sum_s a[i + s * part]) * sum_s b[i + s * part], i < n (silu.slang:11-27 over partial results)
+hipError_t launch_silu_parts(hipStream_t s, float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part);
 // q/k/v GEMV (three segments in the order v, k, q) and the attention over their results in one launch
 hipError_t launch_qkv_attention(slai_ctx *ctx, GemvRowtileParams p, const AttnLaunch &a);
 // out[i] = powf(base, -((2*i) % head_size) / head_size), i < head_size/2

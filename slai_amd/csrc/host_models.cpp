@@ -143,7 +143,7 @@ struct slai_llama2 {
     int chunk_reserve(uint32_t rows);
     int enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev);   // fills the caches for positions pos0 .. pos0 + n - 1
     int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev);   // the same on the matrix cores, n <= 32
-    int chunk_attention(uint32_t l, uint32_t pos0, uint32_t n);
+    int chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts = 1);   // q / k / v given as nparts partial sums, 32 rows apart
 };
 
 // models/llama2/cpu.rs:79-109
@@ -443,12 +443,13 @@ int slai_llama2::chunk_reserve(uint32_t rows) {
     TRY(GpuTensor::matrix(ctx, dim, rows, STORAGE, &c.x));
     TRY(GpuTensor::matrix(ctx, dim + dim / 16, rows, STORAGE, &c.xw));
     TRY(GpuTensor::matrix(ctx, dim, rows, STORAGE, &c.xb));
-    TRY(GpuTensor::matrix(ctx, dim, rows, STORAGE, &c.q));
-    TRY(GpuTensor::matrix(ctx, kvd, rows, STORAGE, &c.k));
-    TRY(GpuTensor::matrix(ctx, kvd, rows, STORAGE, &c.v));
-    TRY(GpuTensor::matrix(ctx, config.hidden_dim, rows, STORAGE, &c.hb));
+    // (room for the partial results of a projection split four ways over its columns, see GemmChunkParams::ksplit)
+    TRY(GpuTensor::matrix(ctx, dim, 4 * rows, STORAGE, &c.q));
+    TRY(GpuTensor::matrix(ctx, kvd, 4 * rows, STORAGE, &c.k));
+    TRY(GpuTensor::matrix(ctx, kvd, 4 * rows, STORAGE, &c.v));
+    TRY(GpuTensor::matrix(ctx, config.hidden_dim, 4 * rows, STORAGE, &c.hb));
     TRY(GpuTensor::matrix(ctx, dim, rows, STORAGE, &c.xn));
-    TRY(GpuTensor::matrix(ctx, config.hidden_dim, rows, STORAGE, &c.hb2));
+    TRY(GpuTensor::matrix(ctx, config.hidden_dim, 4 * rows, STORAGE, &c.hb2));
     if (!c.positions) {
         TRY(slai_buffer_create(ctx, (size_t)config.seq_len * 4, SLAI_DT_I32, STORAGE | COPY_DST, &c.positions));
         TRY(slai_buffer_create(ctx, (size_t)config.seq_len * 4, SLAI_DT_I32, STORAGE | COPY_DST, &c.tokens));
@@ -525,7 +526,7 @@ int slai_llama2::enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev)
 
 // Bias + RoPE + cache write for the n tokens of a chunk (their q / k / v are in the chunk's matrices), then their
 // attention into the chunk's xb.
-int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n) {
+int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts) {
     PromptChunkState &pc = chunk;
     Llama2State &s = state;
     const Llama2LayerWeights &wl = weights.layers[l];
@@ -543,7 +544,7 @@ int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n) {
     a.rope_variant = rope_variant(); a.rope_base = config.rope_base_freq;
     a.rope_theta = (const float *)s.rope_theta.buf->dptr;
     a.out = (float *)pc.xb.buf->dptr; a.scratch = nullptr; a.n_splits = 1;
-    SLAI_HIP_TRY(ctx, launch_rope_store_batch(ctx->stream, a, q, (const float *)pc.k.buf->dptr, (const float *)pc.v.buf->dptr, n, dim, kvd));
+    SLAI_HIP_TRY(ctx, launch_rope_store_batch(ctx->stream, a, q, (const float *)pc.k.buf->dptr, (const float *)pc.v.buf->dptr, n, dim, kvd, nparts, 32 * dim, 32 * kvd));
     SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, dim, dim));
     return SLAI_OK;
 }
@@ -560,17 +561,18 @@ bool slai_llama2::chunk_gemm_supported() const {
 namespace {
 // matrices (with the same input) through the matrix-core kernel: 64-row-tile matrices share a launch
 int gemm_chunk_call(slai_ctx *ctx, int nmat, const slai_qmat *const *mats, float *const *outs, const uint32_t *out_strides, uint32_t flags,
-                    const float *xq, uint32_t ntokens, const char *who) {
+                    const float *xq, uint32_t ntokens, const char *who, uint32_t ksplit = 1) {
     bool done[3] = {false, false, false};
     for (int i = 0; i < nmat; ++i) {
         if (done[i]) continue;
         GemmChunkParams p;
         p.nseg = 0; p.ncols = mats[i]->ncols; p.ncb = mats[i]->ncb; p.ngroups = mats[i]->ngroups; p.rows_log2 = mats[i]->rows_log2;
-        p.x = xq; p.ntokens = ntokens;
+        p.x = xq; p.ntokens = ntokens; p.ksplit = ksplit;
         for (int j = i; j < nmat; ++j) {
             if (done[j] || (j != i && (mats[j]->rows_log2 != 6 || mats[i]->rows_log2 != 6 || mats[j]->ncols != mats[i]->ncols))) continue;
             GemmChunkSeg &sg = p.seg[p.nseg++];
             sg.W = mats[j]->dptr; sg.type = mats[j]->type; sg.nrows = mats[j]->nrows; sg.out = outs[j]; sg.out_stride = out_strides[j]; sg.flags = flags;
+            sg.part_stride = 32 * out_strides[j];
             done[j] = true;
         }
         hipError_t e = launch_gemm_chunk(ctx, p);
@@ -592,7 +594,9 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
     float *k = (float *)pc.k.buf->dptr, *v = (float *)pc.v.buf->dptr, *hb = (float *)pc.hb.buf->dptr, *hb2 = (float *)pc.hb2.buf->dptr;
     for (uint32_t b = 0; b < n; ++b)
         SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, tokens_dev + b, nullptr, nullptr, dim, x + (size_t)b * dim));
-    // xn, xb -> xq (via xn) and hb, hb2 are quad-major with 32 token slots: the layout the GEMM kernels read
+    // xn, xb -> xq (via xn) and hb, hb2 are quad-major with 32 token slots: the layout the GEMM kernels read.
+    // q/k/v and gate/up (64-row tiles) are split four ways over their columns when every matrix involved has such tiles:
+    // 192 or 344 tiles do not divide 256 compute units evenly, four times as many quarter-sized units nearly do.
     for (uint32_t l = 0; l < config.n_layers; ++l) {
         const Llama2LayerWeights &wl = weights.layers[l];
         SLAI_HIP_TRY(ctx, launch_rms_norm_quads(ctx->stream, xn, x, (const float *)wl.attn_norm.buf->dptr, dim, n, dim, config.rms_norm_eps));
@@ -600,9 +604,12 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
             const slai_qmat *mats[3] = {wl.attn_v, wl.attn_k, wl.attn_q};
             float *outs[3] = {v, k, q};
             const uint32_t strides[3] = {kvd, kvd, dim};
-            TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)"));
+            bool all64 = true;
+            for (const slai_qmat *m : mats) all64 = all64 && m->rows_log2 == 6;
+            const uint32_t ks = all64 && mats[0]->ncb % 4 == 0 && mats[0]->ncb >= 8 ? 4u : 1u;
+            TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)", ks));
+            TRY(chunk_attention(l, pos0, n, ks));
         }
-        TRY(chunk_attention(l, pos0, n));
         SLAI_HIP_TRY(ctx, launch_rows_to_quads(ctx->stream, xn, xb, dim, n, dim));
         {
             const slai_qmat *mats[1] = {wl.attn_output};
@@ -615,10 +622,12 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
             const slai_qmat *mats[2] = {wl.ffn_gate, wl.ffn_up};
             float *outs[2] = {hb, hb2};
             const uint32_t strides[2] = {hid, hid};
-            TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, GEMM_OUT_QUADS, xn, n, "llama2 ffn gate/up (prompt chunk)"));
+            const bool all64 = mats[0]->rows_log2 == 6 && mats[1]->rows_log2 == 6;
+            const uint32_t ks = all64 && mats[0]->ncb % 4 == 0 && mats[0]->ncb >= 8 ? 4u : 1u;
+            TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, GEMM_OUT_QUADS, xn, n, "llama2 ffn gate/up (prompt chunk)", ks));
+            // element-wise, so the layout does not matter (slots of tokens past the chunk hold stale values nobody reads)
+            SLAI_HIP_TRY(ctx, launch_silu_parts(ctx->stream, hb, hb2, 32 * hid, ks, 32 * hid));
         }
-        // element-wise, so the layout does not matter (slots of tokens past the chunk hold stale values nobody reads)
-        SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, 32 * hid, 1}, VecView{hb2, 32 * hid, 1}));
         {
             const slai_qmat *mats[1] = {wl.ffn_down};
             float *outs[1] = {x};

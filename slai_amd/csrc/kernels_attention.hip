@@ -188,7 +188,8 @@ __global__ void __launch_bounds__(512) attn_fast_batch_kernel(AttnLaunch a0, uin
 // attention reads the rows of the earlier tokens of its chunk, so all rows are written before any attention starts.
 // grid = (n_heads, tokens), block = head_size / 2 (one rotation pair per thread; rope.slang:27-84).
 template <bool F16>
-__global__ void rope_store_batch_kernel(AttnLaunch a, float *q, const float *k, const float *v, uint32_t q_stride, uint32_t kv_stride) {
+__global__ void rope_store_batch_kernel(AttnLaunch a, float *q, const float *k, const float *v, uint32_t q_stride, uint32_t kv_stride,
+                                        uint32_t nparts, uint32_t q_part, uint32_t kv_part) {
     using C = KV<F16>;
     using CT = typename C::T;
     const uint32_t h = blockIdx.x, b = blockIdx.y, i = threadIdx.x, HS = a.head_size;
@@ -200,8 +201,13 @@ __global__ void rope_store_batch_kernel(AttnLaunch a, float *q, const float *k, 
     float *qb = q + (size_t)b * q_stride + (size_t)h * HS;
     const float *kb = k + (size_t)b * kv_stride + hoff, *vb = v + (size_t)b * kv_stride + hoff;
     float q0 = qb[e0], q1 = qb[e1];
-    if (a.qbias) { q0 += a.qbias[(size_t)h * HS + e0]; q1 += a.qbias[(size_t)h * HS + e1]; }
     float k0 = kb[e0], k1 = kb[e1], v0 = vb[e0], v1 = vb[e1];
+    for (uint32_t s = 1; s < nparts; ++s) {                      // partial results of a projection split over its columns
+        q0 += qb[(size_t)s * q_part + e0]; q1 += qb[(size_t)s * q_part + e1];
+        k0 += kb[(size_t)s * kv_part + e0]; k1 += kb[(size_t)s * kv_part + e1];
+        v0 += vb[(size_t)s * kv_part + e0]; v1 += vb[(size_t)s * kv_part + e1];
+    }
+    if (a.qbias) { q0 += a.qbias[(size_t)h * HS + e0]; q1 += a.qbias[(size_t)h * HS + e1]; }
     if (a.kbias) { k0 += a.kbias[hoff + e0]; k1 += a.kbias[hoff + e1]; }
     if (a.vbias) { v0 += a.vbias[hoff + e0]; v1 += a.vbias[hoff + e1]; }
     if (a.rope_variant >= 0) {
@@ -301,11 +307,12 @@ hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n
     return hipGetLastError();
 }
 
-hipError_t launch_rope_store_batch(hipStream_t s, const AttnLaunch &a, float *q, const float *k, const float *v, uint32_t n, uint32_t q_stride, uint32_t kv_stride) {
-    if (a.head_size % 2 || a.head_size / 2 > 1024 || n == 0 || n > 65535 || a.kv_mul == 0) return hipErrorInvalidValue;
+hipError_t launch_rope_store_batch(hipStream_t s, const AttnLaunch &a, float *q, const float *k, const float *v, uint32_t n, uint32_t q_stride, uint32_t kv_stride,
+                                   uint32_t nparts, uint32_t q_part, uint32_t kv_part) {
+    if (a.head_size % 2 || a.head_size / 2 > 1024 || n == 0 || n > 65535 || a.kv_mul == 0 || nparts == 0) return hipErrorInvalidValue;
     dim3 grid(a.n_heads, n);
-    if (a.kv_f16) rope_store_batch_kernel<true><<<grid, a.head_size / 2, 0, s>>>(a, q, k, v, q_stride, kv_stride);
-    else rope_store_batch_kernel<false><<<grid, a.head_size / 2, 0, s>>>(a, q, k, v, q_stride, kv_stride);
+    if (a.kv_f16) rope_store_batch_kernel<true><<<grid, a.head_size / 2, 0, s>>>(a, q, k, v, q_stride, kv_stride, nparts, q_part, kv_part);
+    else rope_store_batch_kernel<false><<<grid, a.head_size / 2, 0, s>>>(a, q, k, v, q_stride, kv_stride, nparts, q_part, kv_part);
     return hipGetLastError();
 }
 

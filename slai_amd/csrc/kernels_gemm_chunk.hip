@@ -178,7 +178,9 @@ __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const Gemm
     f32x32 acc;
 #pragma unroll
     for (int i = 0; i < 32; ++i) acc[i] = 0.0f;
-    for (uint32_t cb = wave; cb < p.ncb; cb += NW) {
+    // the workgroup's range of super-blocks: all of them, or the blockIdx.y-th of ksplit ranges
+    const uint32_t per = (p.ncb + p.ksplit - 1) / p.ksplit, cb0 = blockIdx.y * per, cb1 = min(p.ncb, cb0 + per);
+    for (uint32_t cb = cb0 + wave; cb < cb1; cb += NW) {
         typename F::Data d;
         uint16_t dt = 0;
         X64 x;
@@ -202,7 +204,8 @@ __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const Gemm
         if (t < p.ntokens && row < seg.nrows) {
             float o = 0.0f;
             for (int w = 0; w < NW; ++w) o += part[(size_t)w * 32 * G64_LDS_ROW + (size_t)t * G64_LDS_ROW + r];
-            float *dst = (seg.flags & GEMM_OUT_QUADS) ? seg.out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3) : seg.out + (size_t)t * seg.out_stride + row;
+            float *out = seg.out + (size_t)blockIdx.y * seg.part_stride;
+            float *dst = (seg.flags & GEMM_OUT_QUADS) ? out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3) : out + (size_t)t * seg.out_stride + row;
             if (seg.flags & GEMV_BIAS) o += seg.bias[row];
             if (seg.flags & GEMV_ACCUM) o = *dst + o;
             *dst = o;
@@ -210,7 +213,7 @@ __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const Gemm
     }
 }
 
-// grid = tiles of all segments, block = 64 * (waves: each takes every NW-th super-block)
+// grid = (tiles of all segments, ksplit), block = 64 * (waves: each takes every NW-th super-block)
 template <int TT, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemm64_kernel(const GemmChunkParams p) {
     extern __shared__ float part[];                            // [waves][32 tokens][G64_LDS_ROW]
@@ -225,6 +228,7 @@ __global__ void __launch_bounds__(MAXT) gemm64_kernel(const GemmChunkParams p) {
     seg.nrows = s == 0 ? p.seg[0].nrows : (s == 1 ? p.seg[1].nrows : p.seg[2].nrows);
     seg.out = s == 0 ? p.seg[0].out : (s == 1 ? p.seg[1].out : p.seg[2].out);
     seg.out_stride = s == 0 ? p.seg[0].out_stride : (s == 1 ? p.seg[1].out_stride : p.seg[2].out_stride);
+    seg.part_stride = s == 0 ? p.seg[0].part_stride : (s == 1 ? p.seg[1].part_stride : p.seg[2].part_stride);
     seg.bias = s == 0 ? p.seg[0].bias : (s == 1 ? p.seg[1].bias : p.seg[2].bias);
     seg.flags = s == 0 ? p.seg[0].flags : (s == 1 ? p.seg[1].flags : p.seg[2].flags);
     if constexpr (TT != 0) {
@@ -399,19 +403,26 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
             if (p.seg[i].type != tt) tt = 0;
         }
         for (int i = p.nseg; i < 3; ++i) p.seg[i].ntiles = 0;
-        // up to sixteen waves, one super-block each at the usual widths (every format fits the 128 registers per lane that leaves)
-        const uint32_t nw = std::min(p.ncb, 16u);
+        // one wave per super-block of the workgroup's range, at most sixteen (every format fits the 128 registers per
+        // lane that leaves)
+        if (p.ksplit == 0 || p.ksplit > p.ncb) return hipErrorInvalidValue;
+        if (p.ksplit > 1)
+            for (int i = 0; i < p.nseg; ++i)
+                if (p.seg[i].flags & (GEMV_BIAS | GEMV_ACCUM)) return hipErrorInvalidValue;
+        const uint32_t per = (p.ncb + p.ksplit - 1) / p.ksplit;
+        const uint32_t nw = std::min(per, 16u);
         const size_t smem = (size_t)nw * 32 * G64_LDS_ROW * sizeof(float);
         const int NT = (int)nw * 64;
+        const dim3 grid(tiles, p.ksplit);
         switch (tt) {
-        case T_Q4_K: gemm64_kernel<T_Q4_K, 1024><<<tiles, NT, smem, st>>>(p); break;
-        case T_Q5_K: gemm64_kernel<T_Q5_K, 1024><<<tiles, NT, smem, st>>>(p); break;
-        case T_Q6_K: gemm64_kernel<T_Q6_K, 1024><<<tiles, NT, smem, st>>>(p); break;
-        default: gemm64_kernel<0, 1024><<<tiles, NT, smem, st>>>(p); break;
+        case T_Q4_K: gemm64_kernel<T_Q4_K, 1024><<<grid, NT, smem, st>>>(p); break;
+        case T_Q5_K: gemm64_kernel<T_Q5_K, 1024><<<grid, NT, smem, st>>>(p); break;
+        case T_Q6_K: gemm64_kernel<T_Q6_K, 1024><<<grid, NT, smem, st>>>(p); break;
+        default: gemm64_kernel<0, 1024><<<grid, NT, smem, st>>>(p); break;
         }
         return hipGetLastError();
     }
-    if (p.rows_log2 != 4 || p.nseg != 1 || p.ngroups == 0 || p.ngroups > 16) return hipErrorInvalidValue;
+    if (p.rows_log2 != 4 || p.nseg != 1 || p.ngroups == 0 || p.ngroups > 16 || p.ksplit != 1) return hipErrorInvalidValue;
     const uint32_t tiles = (p.seg[0].nrows + 15) / 16;
     const int NT = (int)p.ngroups * 64;
     // the thread bound decides the register budget (256 threads leave 256 registers per lane, 1024 leave 128); narrow

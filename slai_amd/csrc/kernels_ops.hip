@@ -97,6 +97,15 @@ __global__ void silu_kernel(VecView a, VecView b) {
     }
 }
 
+// the same over gate and up given as `nparts` partial sums each
+__global__ void silu_parts_kernel(float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part) {
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        float l = 0.0f, r = 0.0f;
+        for (uint32_t s = 0; s < nparts; ++s) { l += a[i + (size_t)s * part]; r += b[i + (size_t)s * part]; }
+        a[i] = r * (l / (1.0f + expf(-1.0f * l)));
+    }
+}
+
 // ops/unary.rs:81-85 (UnaryOp::Gelu)
 __global__ void gelu_kernel(VecView a) {
     const float GELU_COEF_A = 0.044715f, SQRT_2_OVER_PI = 0.7978846f;
@@ -282,6 +291,10 @@ hipError_t launch_prepare(hipStream_t s, float *out, const float *x, const float
 }
 hipError_t launch_silu(hipStream_t s, VecView a, VecView b) {
     silu_kernel<<<grid_for(a.n, 256), 256, 0, s>>>(a, b);
+    return hipGetLastError();
+}
+hipError_t launch_silu_parts(hipStream_t s, float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part) {
+    silu_parts_kernel<<<grid_for(n, 256), 256, 0, s>>>(a, b, n, nparts, part);
     return hipGetLastError();
 }
 hipError_t launch_gelu(hipStream_t s, VecView a) {
