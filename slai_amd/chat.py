@@ -108,6 +108,12 @@ class ChatLlm:
         out_text, pos, n_new, t0, t_start = [], start_pos, 0, None, start_pos + 1
         next_pos = start_pos                                        # position of the last reported token (cli.rs:139)
         done = False
+        # the prompt up to its last token in chunks (no logits are needed there: the tokens are forced,
+        # slai-chat/src/sampler.rs:100-105); the loop below then starts at the last prompt token
+        if hasattr(self.model, "prefill") and len(toks) - 1 - pos >= 8:
+            self.model.prefill(np.asarray(toks[pos:len(toks) - 1], np.int32), pos)
+            pos = len(toks) - 1
+            t_start = pos + 1
         while not done and pos < self.seq_len:
             steps = min(self.chunk if pos + 1 >= len(toks) else (len(toks) - 1 - pos) + self.chunk, self.seq_len - pos)
             ids, _ = self.model.generate_sampled(np.asarray(fed, np.int32), steps, self.temperature, self.topp, self.seed, start_pos=pos)
