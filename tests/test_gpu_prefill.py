@@ -141,6 +141,15 @@ def test_prefill_continues_at_a_later_position(backend):
     check_prefill(backend, data, prompt, 10, [32], True, split_at=13, expect_path=2)
 
 
+def test_prefill_long_prompt(backend):
+    """1100 prompt tokens in a context of 1280: every chunk's attention runs over the whole cache in one workgroup per
+    head and token, while the token-by-token pass it is compared with uses the split kernel at this context length."""
+    data = gw.llama_gguf(dim=1024, hidden_dim=1024, n_layers=1, n_heads=8, n_kv_heads=4, vocab=512, seq_len=1280, wtype=12, seed=21,
+                         std=0.05, norm_random=True)
+    prompt = np.random.Generator(np.random.PCG64(9)).integers(0, 512, 1100)
+    check_prefill(backend, data, prompt, 8, [0], True, expect_path=2)
+
+
 def test_prefill_falls_back_to_the_token_loop_for_other_layouts(backend):
     """Widths that are no multiple of 256 keep the row layout, which has no chunked kernels: the call then runs the
     ordinary loop and still leaves the same caches."""
