@@ -75,9 +75,11 @@ template <> struct Vec8<false> {  // 8 f32 = 32 bytes
 // `h`, `split`: head and split of the calling workgroup; `tid`: 0 .. NT-1 (the first NT threads of the workgroup; any
 // others must have left the kernel).  `wait_inputs()` is called once, by every thread, before q / knew / vnew are read:
 // a launch in which this workgroup's inputs are produced by other workgroups of the same launch blocks there (FUSED:
-// the requests for the cache, which depend on nothing but the position, then go first).
+// the requests for the cache, which depend on nothing but the position, then go first).  `quad_token` (single-split
+// form only): write the result as that token's column of a quad-major matrix instead of a plain vector.
 template <bool F16, int NT, int HS, bool SINGLE, bool FUSED, int KL = 4, class Wait>
-__device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, uint32_t split, uint32_t tid, Wait &&wait_inputs) {
+__device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, uint32_t split, uint32_t tid, Wait &&wait_inputs,
+                                               uint32_t quad_token = 0xffffffffu) {
     using C = KV<F16>;
     using CT = typename C::T;
     constexpr int NW = NT / 64;
@@ -279,7 +281,10 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
             l = fmaf(sred2[w], f, l);
         }
         if (a.n_splits == 1) {
-            a.out[(size_t)h * HS + tid] = r / l;
+            const uint32_t e = h * HS + tid;
+            // (a chunk of prompt tokens: token `quad_token` of a [columns / 4][32 tokens][4] matrix)
+            if (quad_token != 0xffffffffu) a.out[((size_t)(e >> 2) * 32 + quad_token) * 4 + (e & 3u)] = r / l;
+            else a.out[e] = r / l;
         } else {
             float *po = a.scratch + ((size_t)h * a.n_splits + split) * (HS + 2);
             po[tid] = r;

@@ -317,8 +317,11 @@ struct AttnLaunch {
 };
 hipError_t launch_attention(hipStream_t s, const AttnLaunch &a);
 // A chunk of `n` consecutive tokens whose keys and values are already in the caches: token b attends from q + b * q_stride
-// over positions [0, pos_ptr[b]] into out + b * out_stride; knew / vnew must be null.  One workgroup per head and token.
-hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride);
+// over positions [0, pos_ptr[b]] into out + b * out_stride (out_quads: into column b of the quad-major matrix `out`,
+// n <= 32); knew / vnew must be null.  One workgroup per head and token.
+hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride, bool out_quads = false);
+// out[b] = embedding row tokens[b] (dequantised), b < n
+hipError_t launch_embed_rows(hipStream_t s, const slai_qmat *m, const int *tokens, uint32_t n, uint32_t ncols, float *out, uint32_t out_stride);
 // The step before it: for token b (position pos_ptr[b]) add the biases, rotate q + b * q_stride in place and write the
 // rotated key k + b * kv_stride and the value v + b * kv_stride to row pos_ptr[b] of the caches.  Uses the q / cache /
 // bias / rope fields of `a`.

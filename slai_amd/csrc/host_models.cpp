@@ -143,7 +143,8 @@ struct slai_llama2 {
     int chunk_reserve(uint32_t rows);
     int enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev);   // fills the caches for positions pos0 .. pos0 + n - 1
     int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev);   // the same on the matrix cores, n <= 32
-    int chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts = 1);   // q / k / v given as nparts partial sums, 32 rows apart
+    // q / k / v given as nparts partial sums, 32 rows apart; out_quads: the result goes to xn, quad-major, instead of xb
+    int chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts = 1, bool out_quads = false);
 };
 
 // models/llama2/cpu.rs:79-109
@@ -526,7 +527,7 @@ int slai_llama2::enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev)
 
 // Bias + RoPE + cache write for the n tokens of a chunk (their q / k / v are in the chunk's matrices), then their
 // attention into the chunk's xb.
-int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts) {
+int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts, bool out_quads) {
     PromptChunkState &pc = chunk;
     Llama2State &s = state;
     const Llama2LayerWeights &wl = weights.layers[l];
@@ -543,9 +544,9 @@ int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t
     a.vbias = wl.attn_v_bias.buf ? (const float *)wl.attn_v_bias.buf->dptr : nullptr;
     a.rope_variant = rope_variant(); a.rope_base = config.rope_base_freq;
     a.rope_theta = (const float *)s.rope_theta.buf->dptr;
-    a.out = (float *)pc.xb.buf->dptr; a.scratch = nullptr; a.n_splits = 1;
+    a.out = out_quads ? (float *)pc.xn.buf->dptr : (float *)pc.xb.buf->dptr; a.scratch = nullptr; a.n_splits = 1;
     SLAI_HIP_TRY(ctx, launch_rope_store_batch(ctx->stream, a, q, (const float *)pc.k.buf->dptr, (const float *)pc.v.buf->dptr, n, dim, kvd, nparts, 32 * dim, 32 * kvd));
-    SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, dim, dim));
+    SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, dim, dim, out_quads));
     return SLAI_OK;
 }
 
@@ -590,11 +591,11 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
     PromptChunkState &pc = chunk;
     if (n == 0 || n > 32 || n > pc.rows || pos0 + n > config.seq_len) return set_error(ctx, SLAI_E_ARG, "prompt chunk out of range");
     const uint32_t dim = config.dim, kvd = kv_dim(), hid = config.hidden_dim;
-    float *x = (float *)pc.x.buf->dptr, *xn = (float *)pc.xn.buf->dptr, *xb = (float *)pc.xb.buf->dptr, *q = (float *)pc.q.buf->dptr;
+    float *x = (float *)pc.x.buf->dptr, *xn = (float *)pc.xn.buf->dptr, *q = (float *)pc.q.buf->dptr;
     float *k = (float *)pc.k.buf->dptr, *v = (float *)pc.v.buf->dptr, *hb = (float *)pc.hb.buf->dptr, *hb2 = (float *)pc.hb2.buf->dptr;
-    for (uint32_t b = 0; b < n; ++b)
-        SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, tokens_dev + b, nullptr, nullptr, dim, x + (size_t)b * dim));
-    // xn, xb -> xq (via xn) and hb, hb2 are quad-major with 32 token slots: the layout the GEMM kernels read.
+    SLAI_HIP_TRY(ctx, launch_embed_rows(ctx->stream, weights.token_embd, tokens_dev, n, dim, x, dim));
+    // xn (the normalised rows, then the attention output) and hb, hb2 are quad-major with 32 token slots: the layout the
+    // GEMM kernels read.
     // q/k/v and gate/up (64-row tiles) are split four ways over their columns when every matrix involved has such tiles:
     // 192 or 344 tiles do not divide 256 compute units evenly, four times as many quarter-sized units nearly do.
     for (uint32_t l = 0; l < config.n_layers; ++l) {
@@ -608,9 +609,8 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
             for (const slai_qmat *m : mats) all64 = all64 && m->rows_log2 == 6;
             const uint32_t ks = all64 && mats[0]->ncb % 4 == 0 && mats[0]->ncb >= 8 ? 4u : 1u;
             TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)", ks));
-            TRY(chunk_attention(l, pos0, n, ks));
+            TRY(chunk_attention(l, pos0, n, ks, true));       // straight into xn, quad-major
         }
-        SLAI_HIP_TRY(ctx, launch_rows_to_quads(ctx->stream, xn, xb, dim, n, dim));
         {
             const slai_qmat *mats[1] = {wl.attn_output};
             float *outs[1] = {x};

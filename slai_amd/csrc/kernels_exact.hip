@@ -67,6 +67,12 @@ __global__ void embed_kernel(QMatDev a, const int *row_a, QMatDev b, const int *
     out[c] = v;
 }
 
+// one embedding row per token of a chunk: grid = (columns / 256, tokens)
+__global__ void embed_rows_kernel(QMatDev a, const int *rows, uint32_t ncols, float *out, uint32_t out_stride) {
+    const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    if (c < ncols) out[(size_t)b * out_stride + c] = qmat_elem(a, (uint32_t)rows[b], c);
+}
+
 }  // namespace
 
 hipError_t launch_repack(hipStream_t s, const slai_qmat *m, const uint8_t *src) {
@@ -91,6 +97,12 @@ hipError_t launch_dequant_rows(hipStream_t s, const slai_qmat *m, uint32_t row0,
 
 hipError_t launch_embed(hipStream_t s, const slai_qmat *a, const int *row_a, const slai_qmat *b, const int *row_b, uint32_t ncols, float *out) {
     embed_kernel<<<(ncols + 255) / 256, 256, 0, s>>>(qmat_dev(a), row_a, qmat_dev(b), row_b, b ? 1 : 0, ncols, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_embed_rows(hipStream_t s, const slai_qmat *m, const int *tokens, uint32_t n, uint32_t ncols, float *out, uint32_t out_stride) {
+    if (n == 0 || n > 65535) return hipErrorInvalidValue;
+    embed_rows_kernel<<<dim3((ncols + 255) / 256, n), 256, 0, s>>>(qmat_dev(m), tokens, ncols, out, out_stride);
     return hipGetLastError();
 }
 
