@@ -5,9 +5,9 @@ tiles), 1 = the GEMV kernels with one workgroup per token and tile (other tiled 
 
 The reference has no batched prompt pass: it feeds the prompt one token per forward pass (chat_llama2.rs:105-158).
 The chunked pass must leave the caches that loop leaves, so: greedy ids after the prompt identical to the oracle's,
-logits at the last prompt position within 1e-2 of the oracle's (the bar of every model test) and within 1e-4 of the
-device's own token-by-token result (same kernels per token, only the attention's summation order can differ), cache
-rows equal to the token-by-token ones within f16 rounding."""
+logits at the last prompt position within 1e-2 of the oracle's (the bar of every model test) and within 1e-3 of the
+device's own token-by-token result (fp32 sums in another order), cache rows equal to the token-by-token ones within
+f16 rounding."""
 import ctypes as C
 
 import numpy as np
