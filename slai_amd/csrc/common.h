@@ -178,8 +178,8 @@ hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p, const GemvBat
 // (kernels_gemm_chunk.hip): out[t][r] = sum_c deq(W[r][c]) * x[t][c] (+ bias[r]) (+ the old out[t][r]).  The input is
 // "quad-major": the float4 of columns c .. c + 3 of token t at x + ((c / 4) * 32 + t) * 4 (32 token slots whatever
 // ntokens is); the output is row-major (token t at out + t * out_stride) or, with GEMM_OUT_QUADS, quad-major as well.
-// K-quants in 64-row tiles (any number of segments, formats may differ) or in 16-row tiles of at most 16 column groups
-// (one segment).
+// K-quants in 64-row tiles (any number of segments, formats may differ) or in 16- / 32-row tiles (one segment; more than
+// 16 column groups take several launches).
 struct GemmChunkSeg {
     const uint8_t *W = nullptr;
     int type = 0;
@@ -195,6 +195,7 @@ struct GemmChunkParams {
     GemmChunkSeg seg[3];
     int nseg = 1;
     uint32_t ncols = 0, ncb = 0, ngroups = 0, rows_log2 = 6;
+    uint32_t group0 = 0;        // 16- / 32-row tiles: first column group of this launch (set by the launcher)
     const float *x = nullptr;   // quad-major, 16-byte aligned
     uint32_t ntokens = 0;
     // 64-row tiles only.  ksplit > 1: the columns are cut into ksplit ranges of whole super-blocks, each computed by a

@@ -10,6 +10,9 @@
 // the A-operand layout of the one-column-deep MFMA shapes:
 //   64-row tiles (lane = row):            v_mfma_f32_32x32x1 (2 blocks): block = rows 0-31 / 32-63, both with the same
 //                                         column k; B = x[token = lane % 32][k]; 64 rows x 32 tokens per instruction.
+//   32-row tiles (lane = 32 * kq + row):  v_mfma_f32_32x32x1 (2 blocks): block kq = super-block 2g + kq, so one
+//                                         instruction advances two columns for 32 rows x 32 tokens; the blocks are added
+//                                         at the end.
 //   16-row tiles (lane = 16 * kq + row):  v_mfma_f32_16x16x1 (4 blocks): block kq = super-block 4g + kq, so one
 //                                         instruction advances FOUR columns (one per super-block) for 16 rows x 16
 //                                         tokens; two instructions cover 32 tokens; the four blocks are added at the end.
@@ -291,13 +294,14 @@ __global__ void __launch_bounds__(MAXT) gemm16_kernel(const GemmChunkParams p) {
     const uint32_t tile = blockIdx.x, tbase = NACC == 2 ? 0u : 16u * blockIdx.y;
     if (tbase >= p.ntokens) return;                            // (uniform) a short chunk has no second half
     const uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
-    const uint32_t cb = min((uint32_t)wave * 4 + (uint32_t)(lane >> 4), p.ncb - 1);   // (super-blocks past the end are zero weights)
+    const uint32_t g = p.group0 + wave;                        // this launch covers the column groups group0 .. group0 + NW - 1
+    const uint32_t cb = min(g * 4 + (uint32_t)(lane >> 4), p.ncb - 1);   // (super-blocks past the end are zero weights)
     const float4 *xt[NACC];
 #pragma unroll
     for (int n = 0; n < NACC; ++n) xt[n] = (const float4 *)p.x + (size_t)cb * 2048 + min(tbase + 16u * n + (uint32_t)(lane & 15), p.ntokens - 1);
     typename F::Data d;
     uint16_t dt = 0;
-    load_unit<T>(p.seg[0].W + ((size_t)tile * p.ngroups + wave) * unit_bytes, lane, d, dt);
+    load_unit<T>(p.seg[0].W + ((size_t)tile * p.ngroups + g) * unit_bytes, lane, d, dt);
     X16<NACC> x;
     request_x16<T, 0, 0, NACC>(xt, x);
     f32x16 acc[NACC];
@@ -325,6 +329,56 @@ __global__ void __launch_bounds__(MAXT) gemm16_kernel(const GemmChunkParams p) {
         if (t < p.ntokens && row < p.seg[0].nrows) {
             float o = 0.0f;
             for (int w = 0; w < NW; ++w) o += part[(size_t)w * 16 * NACC * G16_LDS_ROW + (size_t)tl * G16_LDS_ROW + r];
+            float *dst = (p.seg[0].flags & GEMM_OUT_QUADS) ? p.seg[0].out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3)
+                                                           : p.seg[0].out + (size_t)t * p.seg[0].out_stride + row;
+            if (p.seg[0].flags & GEMV_BIAS) o += p.seg[0].bias[row];
+            if (p.seg[0].flags & GEMV_ACCUM) o = *dst + o;
+            *dst = o;
+        }
+    }
+}
+
+// ---- 32-row tiles ------------------------------------------------------------------------------------------------------
+constexpr int G32_LDS_ROW = 36;                                // floats per token in the LDS partials (32 rows + padding)
+
+// grid = tiles, block = 64 * (column groups of this launch): one wave per group of two super-blocks, lane = 32 * kq + row
+template <int T, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemm32_kernel(const GemmChunkParams p) {
+    using F = Tiled<T>;
+    extern __shared__ float part[];                            // [waves][32 tokens][G32_LDS_ROW]
+    touch_kernel_arguments<sizeof(GemmChunkParams)>();
+    const int tid = threadIdx.x, lane = tid & 63, NW = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t tile = blockIdx.x;
+    const uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
+    const uint32_t g = p.group0 + wave;
+    const uint32_t cb = min(g * 2 + (uint32_t)(lane >> 5), p.ncb - 1);              // (a super-block past the end is zero weights)
+    const float4 *xcb = (const float4 *)p.x + (size_t)cb * 2048 + min((uint32_t)(lane & 31), p.ntokens - 1);
+    typename F::Data d;
+    uint16_t dt = 0;
+    load_unit<T>(p.seg[0].W + ((size_t)tile * p.ngroups + g) * unit_bytes, lane, d, dt);
+    X64 x;
+    request_x64<T, 0>(xcb, x);
+    f32x32 acc;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) acc[i] = 0.0f;
+    Deq<T> q;
+    q.head(d, dt);
+    stages64<T, 0>(q, d, xcb, x, acc);
+    // the two blocks hold the same rows and tokens over different super-blocks: add them.  Register v of a block holds row
+    // 8 * (v / 4) + 4 * (lane / 32) + v % 4 of token lane % 32.
+    float *mine = part + (size_t)wave * 32 * G32_LDS_ROW + (size_t)(lane & 31) * G32_LDS_ROW + 4 * (lane >> 5);
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4)
+        *(float4 *)(mine + 8 * g4) = make_float4(acc[4 * g4] + acc[16 + 4 * g4], acc[4 * g4 + 1] + acc[16 + 4 * g4 + 1],
+                                                 acc[4 * g4 + 2] + acc[16 + 4 * g4 + 2], acc[4 * g4 + 3] + acc[16 + 4 * g4 + 3]);
+    lds_barrier();
+    for (uint32_t idx = tid; idx < 1024; idx += blockDim.x) {
+        const uint32_t r = idx & 31u, t = idx >> 5;
+        const uint32_t row = tile * 32 + r;
+        if (t < p.ntokens && row < p.seg[0].nrows) {
+            float o = 0.0f;
+            for (int w = 0; w < NW; ++w) o += part[(size_t)w * 32 * G32_LDS_ROW + (size_t)t * G32_LDS_ROW + r];
             float *dst = (p.seg[0].flags & GEMM_OUT_QUADS) ? p.seg[0].out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3)
                                                            : p.seg[0].out + (size_t)t * p.seg[0].out_stride + row;
             if (p.seg[0].flags & GEMV_BIAS) o += p.seg[0].bias[row];
@@ -372,8 +426,7 @@ __global__ void rows_to_quads_kernel(float4 *out, const float *x, uint32_t n, ui
 
 bool gemm_chunk_supports(const slai_qmat *m) {
     if (!m || !m->tiled || (m->type != T_Q4_K && m->type != T_Q6_K && m->type != T_Q5_K)) return false;
-    if (m->rows_log2 == 6) return true;
-    return m->rows_log2 == 4 && m->ngroups <= 16;
+    return m->rows_log2 >= 4 && m->rows_log2 <= 6 && m->ngroups <= 64;
 }
 
 hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps) {
@@ -422,26 +475,54 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
         }
         return hipGetLastError();
     }
-    if (p.rows_log2 != 4 || p.nseg != 1 || p.ngroups == 0 || p.ngroups > 16 || p.ksplit != 1) return hipErrorInvalidValue;
-    const uint32_t tiles = (p.seg[0].nrows + 15) / 16;
-    const int NT = (int)p.ngroups * 64;
-    // the thread bound decides the register budget (256 threads leave 256 registers per lane, 1024 leave 128); narrow
-    // matrices (few waves per workgroup) split the tokens over two workgroups
+    if ((p.rows_log2 != 4 && p.rows_log2 != 5) || p.nseg != 1 || p.ngroups == 0 || p.ngroups > 64 || p.ksplit != 1) return hipErrorInvalidValue;
+    // One wave per column group, at most 16 per workgroup: wider matrices take several launches over balanced slices
+    // of the groups, the first one writing (or adding to the residual) and the others accumulating.
+    const uint32_t nslices = (p.ngroups + 15) / 16, per_slice = (p.ngroups + nslices - 1) / nslices;
+    const uint32_t rows = 1u << p.rows_log2;
+    const uint32_t tiles = (p.seg[0].nrows + rows - 1) / rows;
+    for (uint32_t sl = 0; sl < nslices; ++sl) {
+        GemmChunkParams q = p;
+        q.group0 = sl * per_slice;
+        const uint32_t ng = std::min(per_slice, p.ngroups - q.group0);
+        if (sl > 0) q.seg[0].flags = (q.seg[0].flags | GEMV_ACCUM) & ~GEMV_BIAS;
+        const int NT = (int)ng * 64;
+        if (p.rows_log2 == 5) {
+            const size_t smem = (size_t)ng * 32 * G32_LDS_ROW * sizeof(float);
+#define SLAI_G32(TY)                                                                       \
+    do {                                                                                   \
+        if (NT <= 256) gemm32_kernel<TY, 256><<<tiles, NT, smem, st>>>(q);                 \
+        else if (NT <= 512) gemm32_kernel<TY, 512><<<tiles, NT, smem, st>>>(q);            \
+        else gemm32_kernel<TY, 1024><<<tiles, NT, smem, st>>>(q);                          \
+    } while (0)
+            switch (p.seg[0].type) {
+            case T_Q4_K: SLAI_G32(T_Q4_K); break;
+            case T_Q6_K: SLAI_G32(T_Q6_K); break;
+            default: SLAI_G32(T_Q5_K); break;
+            }
+#undef SLAI_G32
+        } else {
+            // the thread bound decides the register budget (256 threads leave 256 registers per lane, 1024 leave 128);
+            // narrow matrices (few waves per workgroup) split the tokens over two workgroups
+            const size_t smem1 = (size_t)ng * 16 * G16_LDS_ROW * sizeof(float), smem2 = 2 * smem1;
 #define SLAI_G16(TY)                                                                                       \
     do {                                                                                                   \
-        if (NT <= 256) gemm16_kernel<TY, 256, 1><<<dim3(tiles, 2), NT, smem1, st>>>(p);                    \
-        else if (NT <= 512) gemm16_kernel<TY, 512, 1><<<dim3(tiles, 2), NT, smem1, st>>>(p);               \
-        else if (NT <= 768) gemm16_kernel<TY, 768, 2><<<tiles, NT, smem2, st>>>(p);                        \
-        else gemm16_kernel<TY, 1024, 2><<<tiles, NT, smem2, st>>>(p);                                      \
+        if (NT <= 256) gemm16_kernel<TY, 256, 1><<<dim3(tiles, 2), NT, smem1, st>>>(q);                    \
+        else if (NT <= 512) gemm16_kernel<TY, 512, 1><<<dim3(tiles, 2), NT, smem1, st>>>(q);               \
+        else if (NT <= 768) gemm16_kernel<TY, 768, 2><<<tiles, NT, smem2, st>>>(q);                        \
+        else gemm16_kernel<TY, 1024, 2><<<tiles, NT, smem2, st>>>(q);                                      \
     } while (0)
-    const size_t smem1 = (size_t)p.ngroups * 16 * G16_LDS_ROW * sizeof(float), smem2 = 2 * smem1;
-    switch (p.seg[0].type) {
-    case T_Q4_K: SLAI_G16(T_Q4_K); break;
-    case T_Q6_K: SLAI_G16(T_Q6_K); break;
-    default: SLAI_G16(T_Q5_K); break;
-    }
+            switch (p.seg[0].type) {
+            case T_Q4_K: SLAI_G16(T_Q4_K); break;
+            case T_Q6_K: SLAI_G16(T_Q6_K); break;
+            default: SLAI_G16(T_Q5_K); break;
+            }
 #undef SLAI_G16
-    return hipGetLastError();
+        }
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 }  // namespace slai

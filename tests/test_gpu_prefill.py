@@ -117,11 +117,31 @@ def test_prefill_matrix_cores_qwen2_bias_neox(backend):
 
 
 @pytest.mark.parametrize("kv_f16", [False, True])
-def test_prefill_shared_weights_kquants_gqa_ragged_chunks(backend, kv_f16):
-    """A width (512) whose attention output matrix gets 32-row tiles: the chunks then go through the GEMV kernels, one
-    workgroup per token and tile.  Chunks of 3, 8 (ragged last chunk) and 32 (one chunk)."""
+def test_prefill_matrix_cores_32_row_tiles(backend, kv_f16):
+    """A width (512) whose attention output and down matrices get 32-row tiles (two super-blocks per wave), head size 64,
+    grouped-query attention.  Chunks of 3, 8 (ragged last chunk) and 32 (one chunk)."""
     data = gw.llama_gguf(dim=512, hidden_dim=2816, n_layers=3, n_heads=8, n_kv_heads=2, vocab=1000, seq_len=64,
                          wtype=12, v_type=14, out_type=14, embd_type=12, seed=11, std=0.06, norm_random=True)
+    prompt = np.random.Generator(np.random.PCG64(8)).integers(0, 1000, 22)
+    check_prefill(backend, data, prompt, 16, [3, 8, 32], kv_f16, expect_path=2)
+
+
+@pytest.mark.parametrize("wtype,path", [(12, 2), (2, 1)], ids=["q4_k-matrix-cores", "q4_0-shared-weights"])
+def test_prefill_feed_forward_wider_than_16384(backend, wtype, path):
+    """A down projection of 16640 columns (17 column groups of 16-row tiles): more groups than a workgroup has waves,
+    so it takes two launches over slices of the groups, the second accumulating."""
+    data = gw.llama_gguf(dim=512, hidden_dim=16640, n_layers=2, n_heads=8, n_kv_heads=8, vocab=600, seq_len=48, wtype=wtype, seed=19,
+                         std=0.03, norm_random=True)
+    prompt = np.random.Generator(np.random.PCG64(19)).integers(0, 600, 25)
+    check_prefill(backend, data, prompt, 10, [16], True, expect_path=path)
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+def test_prefill_shared_weights_q4_0_gqa_ragged_chunks(backend, kv_f16):
+    """Q4_0 has no matrix-core kernel: the chunks go through the GEMV kernels, one workgroup per token and tile.
+    Chunks of 3, 8 (ragged last chunk) and 32 (one chunk)."""
+    data = gw.llama_gguf(dim=512, hidden_dim=2816, n_layers=3, n_heads=8, n_kv_heads=2, vocab=1000, seq_len=64,
+                         wtype=2, seed=11, std=0.06, norm_random=True)
     prompt = np.random.Generator(np.random.PCG64(8)).integers(0, 1000, 22)
     check_prefill(backend, data, prompt, 16, [3, 8, 32], kv_f16, expect_path=1)
 
