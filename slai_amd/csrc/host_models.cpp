@@ -607,7 +607,7 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
             const uint32_t strides[3] = {kvd, kvd, dim};
             bool all64 = true;
             for (const slai_qmat *m : mats) all64 = all64 && m->rows_log2 == 6;
-            const uint32_t ks = all64 && mats[0]->ncb % 4 == 0 && mats[0]->ncb >= 8 ? 4u : 1u;
+            const uint32_t ks = all64 && mats[0]->ncb >= 8 ? 4u : 1u;
             TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)", ks));
             TRY(chunk_attention(l, pos0, n, ks, true));       // straight into xn, quad-major
         }
@@ -623,7 +623,7 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
             float *outs[2] = {hb, hb2};
             const uint32_t strides[2] = {hid, hid};
             const bool all64 = mats[0]->rows_log2 == 6 && mats[1]->rows_log2 == 6;
-            const uint32_t ks = all64 && mats[0]->ncb % 4 == 0 && mats[0]->ncb >= 8 ? 4u : 1u;
+            const uint32_t ks = all64 && mats[0]->ncb >= 8 ? 4u : 1u;
             TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, GEMM_OUT_QUADS, xn, n, "llama2 ffn gate/up (prompt chunk)", ks));
             // element-wise, so the layout does not matter (slots of tokens past the chunk hold stale values nobody reads)
             SLAI_HIP_TRY(ctx, launch_silu_parts(ctx->stream, hb, hb2, 32 * hid, ks, 32 * hid));
