@@ -201,17 +201,35 @@ __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const Gemm
         for (int g = 0; g < 4; ++g)
             *(float4 *)(mine + 32 * b + 8 * g) = make_float4(acc[16 * b + 4 * g], acc[16 * b + 4 * g + 1], acc[16 * b + 4 * g + 2], acc[16 * b + 4 * g + 3]);
     lds_barrier();
-    for (uint32_t idx = tid; idx < 2048; idx += blockDim.x) {
-        const uint32_t r = idx & 63u, t = idx >> 6;
-        const uint32_t row = tile * 64 + r;
-        if (t < p.ntokens && row < seg.nrows) {
-            float o = 0.0f;
-            for (int w = 0; w < NW; ++w) o += part[(size_t)w * 32 * G64_LDS_ROW + (size_t)t * G64_LDS_ROW + r];
-            float *out = seg.out + (size_t)blockIdx.y * seg.part_stride;
-            float *dst = (seg.flags & GEMM_OUT_QUADS) ? out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3) : out + (size_t)t * seg.out_stride + row;
-            if (seg.flags & GEMV_BIAS) o += seg.bias[row];
-            if (seg.flags & GEMV_ACCUM) o = *dst + o;
-            *dst = o;
+    // four consecutive rows of a token per thread: float4 reads of the partials, one float4 store.  Consecutive threads
+    // write consecutive addresses: the row quads of a token, or (quad-major output) the 32 tokens of a row quad.
+    const bool quads = (seg.flags & GEMM_OUT_QUADS) != 0;
+    float *out = seg.out + (size_t)blockIdx.y * seg.part_stride;
+    const bool vec_ok = quads || (seg.out_stride % 4 == 0 && ((uintptr_t)out & 15) == 0);
+    for (uint32_t idx = tid; idx < 512; idx += blockDim.x) {
+        const uint32_t t = quads ? idx & 31u : idx >> 4, rq = quads ? idx >> 5 : idx & 15u;
+        const uint32_t row = tile * 64 + 4 * rq;
+        if (t >= p.ntokens || row >= seg.nrows) continue;
+        const float *src = part + (size_t)t * G64_LDS_ROW + 4 * rq;
+        float4 o = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll 4
+        for (int w = 0; w < NW; ++w) {
+            const float4 v = *(const float4 *)(src + (size_t)w * 32 * G64_LDS_ROW);
+            o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
+        }
+        float *dst = quads ? out + ((size_t)(row >> 2) * 32 + t) * 4 : out + (size_t)t * seg.out_stride + row;
+        if (vec_ok && row + 3 < seg.nrows) {
+            if (seg.flags & GEMV_BIAS) { const float4 b = *(const float4 *)(seg.bias + row); o.x += b.x; o.y += b.y; o.z += b.z; o.w += b.w; }
+            if (seg.flags & GEMV_ACCUM) { const float4 a = *(const float4 *)dst; o.x += a.x; o.y += a.y; o.z += a.z; o.w += a.w; }
+            *(float4 *)dst = o;
+        } else {
+            const float ov[4] = {o.x, o.y, o.z, o.w};
+            for (uint32_t e = 0; e < 4 && row + e < seg.nrows; ++e) {
+                float v = ov[e];
+                if (seg.flags & GEMV_BIAS) v += seg.bias[row + e];
+                if (seg.flags & GEMV_ACCUM) v = dst[e] + v;
+                dst[e] = v;
+            }
         }
     }
 }
