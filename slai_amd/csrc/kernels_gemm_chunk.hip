@@ -130,6 +130,32 @@ template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, 
     tail = F::TAIL ? ld16(unit + (size_t)F::PT * 1024 + lane * 2) : (uint16_t)0;
 }
 
+// The end of every kernel here: thread -> four consecutive rows (row .. row + 3) of token t whose partial sums lie
+// `wave_stride` floats apart in LDS; adds them, then bias / old value, and stores (one float4 where alignment allows).
+__device__ __forceinline__ void reduce_store4(const GemmChunkSeg &seg, float *out, const float *src, int nw, uint32_t wave_stride, uint32_t row, uint32_t t, bool quads,
+                                              bool vec_ok) {
+    float4 o = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll 4
+    for (int w = 0; w < nw; ++w) {
+        const float4 v = *(const float4 *)(src + (size_t)w * wave_stride);
+        o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
+    }
+    float *dst = quads ? out + ((size_t)(row >> 2) * 32 + t) * 4 : out + (size_t)t * seg.out_stride + row;
+    if (vec_ok && row + 3 < seg.nrows) {
+        if (seg.flags & GEMV_BIAS) { const float4 b = *(const float4 *)(seg.bias + row); o.x += b.x; o.y += b.y; o.z += b.z; o.w += b.w; }
+        if (seg.flags & GEMV_ACCUM) { const float4 a = *(const float4 *)dst; o.x += a.x; o.y += a.y; o.z += a.z; o.w += a.w; }
+        *(float4 *)dst = o;
+    } else {
+        const float ov[4] = {o.x, o.y, o.z, o.w};
+        for (uint32_t e = 0; e < 4 && row + e < seg.nrows; ++e) {
+            float v = ov[e];
+            if (seg.flags & GEMV_BIAS) v += seg.bias[row + e];
+            if (seg.flags & GEMV_ACCUM) v = dst[e] + v;
+            dst[e] = v;
+        }
+    }
+}
+
 // ---- 64-row tiles ------------------------------------------------------------------------------------------------------
 struct X64 { float4 a[4], b[4]; };                             // the lane's token: chunks c1 and c2 of a stage, four columns per entry
 
@@ -210,27 +236,7 @@ __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const Gemm
         const uint32_t t = quads ? idx & 31u : idx >> 4, rq = quads ? idx >> 5 : idx & 15u;
         const uint32_t row = tile * 64 + 4 * rq;
         if (t >= p.ntokens || row >= seg.nrows) continue;
-        const float *src = part + (size_t)t * G64_LDS_ROW + 4 * rq;
-        float4 o = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-#pragma unroll 4
-        for (int w = 0; w < NW; ++w) {
-            const float4 v = *(const float4 *)(src + (size_t)w * 32 * G64_LDS_ROW);
-            o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
-        }
-        float *dst = quads ? out + ((size_t)(row >> 2) * 32 + t) * 4 : out + (size_t)t * seg.out_stride + row;
-        if (vec_ok && row + 3 < seg.nrows) {
-            if (seg.flags & GEMV_BIAS) { const float4 b = *(const float4 *)(seg.bias + row); o.x += b.x; o.y += b.y; o.z += b.z; o.w += b.w; }
-            if (seg.flags & GEMV_ACCUM) { const float4 a = *(const float4 *)dst; o.x += a.x; o.y += a.y; o.z += a.z; o.w += a.w; }
-            *(float4 *)dst = o;
-        } else {
-            const float ov[4] = {o.x, o.y, o.z, o.w};
-            for (uint32_t e = 0; e < 4 && row + e < seg.nrows; ++e) {
-                float v = ov[e];
-                if (seg.flags & GEMV_BIAS) v += seg.bias[row + e];
-                if (seg.flags & GEMV_ACCUM) v = dst[e] + v;
-                dst[e] = v;
-            }
-        }
+        reduce_store4(seg, out, part + (size_t)t * G64_LDS_ROW + 4 * rq, NW, 32 * G64_LDS_ROW, row, t, quads, vec_ok);
     }
 }
 
@@ -341,18 +347,14 @@ __global__ void __launch_bounds__(MAXT) gemm16_kernel(const GemmChunkParams p) {
         *(float4 *)(mine + (size_t)(16 * n + (lane & 15)) * G16_LDS_ROW) = sm;
     }
     lds_barrier();
-    for (uint32_t idx = tid; idx < 256u * NACC; idx += blockDim.x) {
-        const uint32_t r = idx & 15u, tl = idx >> 4, t = tbase + tl;
-        const uint32_t row = tile * 16 + r;
-        if (t < p.ntokens && row < p.seg[0].nrows) {
-            float o = 0.0f;
-            for (int w = 0; w < NW; ++w) o += part[(size_t)w * 16 * NACC * G16_LDS_ROW + (size_t)tl * G16_LDS_ROW + r];
-            float *dst = (p.seg[0].flags & GEMM_OUT_QUADS) ? p.seg[0].out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3)
-                                                           : p.seg[0].out + (size_t)t * p.seg[0].out_stride + row;
-            if (p.seg[0].flags & GEMV_BIAS) o += p.seg[0].bias[row];
-            if (p.seg[0].flags & GEMV_ACCUM) o = *dst + o;
-            *dst = o;
-        }
+    const GemmChunkSeg &seg = p.seg[0];
+    const bool quads = (seg.flags & GEMM_OUT_QUADS) != 0;
+    const bool vec_ok = quads || (seg.out_stride % 4 == 0 && ((uintptr_t)seg.out & 15) == 0);
+    for (uint32_t idx = tid; idx < 64u * NACC; idx += blockDim.x) {     // four rows of a token per thread
+        const uint32_t rq = idx & 3u, tl = idx >> 2, t = tbase + tl;
+        const uint32_t row = tile * 16 + 4 * rq;
+        if (t < p.ntokens && row < seg.nrows)
+            reduce_store4(seg, seg.out, part + (size_t)tl * G16_LDS_ROW + 4 * rq, NW, 16 * NACC * G16_LDS_ROW, row, t, quads, vec_ok);
     }
 }
 
@@ -391,18 +393,14 @@ __global__ void __launch_bounds__(MAXT) gemm32_kernel(const GemmChunkParams p) {
         *(float4 *)(mine + 8 * g4) = make_float4(acc[4 * g4] + acc[16 + 4 * g4], acc[4 * g4 + 1] + acc[16 + 4 * g4 + 1],
                                                  acc[4 * g4 + 2] + acc[16 + 4 * g4 + 2], acc[4 * g4 + 3] + acc[16 + 4 * g4 + 3]);
     lds_barrier();
-    for (uint32_t idx = tid; idx < 1024; idx += blockDim.x) {
-        const uint32_t r = idx & 31u, t = idx >> 5;
-        const uint32_t row = tile * 32 + r;
-        if (t < p.ntokens && row < p.seg[0].nrows) {
-            float o = 0.0f;
-            for (int w = 0; w < NW; ++w) o += part[(size_t)w * 32 * G32_LDS_ROW + (size_t)t * G32_LDS_ROW + r];
-            float *dst = (p.seg[0].flags & GEMM_OUT_QUADS) ? p.seg[0].out + ((size_t)(row >> 2) * 32 + t) * 4 + (row & 3)
-                                                           : p.seg[0].out + (size_t)t * p.seg[0].out_stride + row;
-            if (p.seg[0].flags & GEMV_BIAS) o += p.seg[0].bias[row];
-            if (p.seg[0].flags & GEMV_ACCUM) o = *dst + o;
-            *dst = o;
-        }
+    const GemmChunkSeg &seg = p.seg[0];
+    const bool quads = (seg.flags & GEMM_OUT_QUADS) != 0;
+    const bool vec_ok = quads || (seg.out_stride % 4 == 0 && ((uintptr_t)seg.out & 15) == 0);
+    for (uint32_t idx = tid; idx < 256; idx += blockDim.x) {            // four rows of a token per thread
+        const uint32_t rq = idx & 7u, t = idx >> 3;
+        const uint32_t row = tile * 32 + 4 * rq;
+        if (t < p.ntokens && row < seg.nrows)
+            reduce_store4(seg, seg.out, part + (size_t)t * G32_LDS_ROW + 4 * rq, NW, 32 * G32_LDS_ROW, row, t, quads, vec_ok);
     }
 }
 
