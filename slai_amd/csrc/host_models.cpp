@@ -560,6 +560,19 @@ bool slai_llama2::chunk_gemm_supported() const {
 }
 
 namespace {
+// Into how many column ranges a launch over 64-row-tile matrices is cut (GemmChunkParams::ksplit): tile counts such as
+// 192 or 344 do not divide 256 compute units evenly, two or four times as many smaller units nearly do; four ranges
+// while that stays within about four workgroups per compute unit, else two (measured on the 7B shapes).
+uint32_t chunk_ksplit(int nmat, const slai_qmat *const *mats) {
+    uint32_t tiles = 0;
+    for (int i = 0; i < nmat; ++i) {
+        if (mats[i]->rows_log2 != 6) return 1;
+        tiles += (mats[i]->nrows + 63) / 64;
+    }
+    if (mats[0]->ncb < 8) return 1;
+    return tiles * 4 <= 1024 ? 4 : 2;
+}
+
 // matrices (with the same input) through the matrix-core kernel: 64-row-tile matrices share a launch
 int gemm_chunk_call(slai_ctx *ctx, int nmat, const slai_qmat *const *mats, float *const *outs, const uint32_t *out_strides, uint32_t flags,
                     const float *xq, uint32_t ntokens, const char *who, uint32_t ksplit = 1) {
@@ -596,8 +609,7 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
     SLAI_HIP_TRY(ctx, launch_embed_rows(ctx->stream, weights.token_embd, tokens_dev, n, dim, x, dim));
     // xn (the normalised rows, then the attention output) and hb, hb2 are quad-major with 32 token slots: the layout the
     // GEMM kernels read.
-    // q/k/v and gate/up (64-row tiles) are split four ways over their columns when every matrix involved has such tiles:
-    // 192 or 344 tiles do not divide 256 compute units evenly, four times as many quarter-sized units nearly do.
+    // q/k/v and gate/up are cut into column ranges when every matrix involved has 64-row tiles (chunk_ksplit).
     for (uint32_t l = 0; l < config.n_layers; ++l) {
         const Llama2LayerWeights &wl = weights.layers[l];
         SLAI_HIP_TRY(ctx, launch_rms_norm_quads(ctx->stream, xn, x, (const float *)wl.attn_norm.buf->dptr, dim, n, dim, config.rms_norm_eps));
@@ -605,9 +617,7 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
             const slai_qmat *mats[3] = {wl.attn_v, wl.attn_k, wl.attn_q};
             float *outs[3] = {v, k, q};
             const uint32_t strides[3] = {kvd, kvd, dim};
-            bool all64 = true;
-            for (const slai_qmat *m : mats) all64 = all64 && m->rows_log2 == 6;
-            const uint32_t ks = all64 && mats[0]->ncb >= 8 ? 4u : 1u;
+            const uint32_t ks = chunk_ksplit(3, mats);
             TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)", ks));
             TRY(chunk_attention(l, pos0, n, ks, true));       // straight into xn, quad-major
         }
@@ -622,8 +632,7 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
             const slai_qmat *mats[2] = {wl.ffn_gate, wl.ffn_up};
             float *outs[2] = {hb, hb2};
             const uint32_t strides[2] = {hid, hid};
-            const bool all64 = mats[0]->rows_log2 == 6 && mats[1]->rows_log2 == 6;
-            const uint32_t ks = all64 && mats[0]->ncb >= 8 ? 4u : 1u;
+            const uint32_t ks = chunk_ksplit(2, mats);
             TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, GEMM_OUT_QUADS, xn, n, "llama2 ffn gate/up (prompt chunk)", ks));
             // element-wise, so the layout does not matter (slots of tokens past the chunk hold stale values nobody reads)
             SLAI_HIP_TRY(ctx, launch_silu_parts(ctx->stream, hb, hb2, 32 * hid, ks, 32 * hid));
