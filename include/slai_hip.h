@@ -295,9 +295,10 @@ int slai_llama2_generate_sampled(slai_llama2 *m, const int32_t *prompt, uint32_t
  * this fills the caches for positions start_pos .. start_pos+n_tokens-1 with `chunk` tokens per pass over the
  * weights and computes no logits (chunk: 0 = the path's default, 1 = token by token, at most 64).  Generation then
  * continues with slai_llama2_generate(prompt, n_prompt, n_prompt - 1, ...).  slai_llama2_prefill_supported() says which
- * path a model takes: 2 = fp32 matrix-core GEMM over the dequantised K-quant tiles, at most 32 tokens per pass;
- * 1 = the GEMV kernels with one workgroup per token and tile sharing the weights through L2 (other tiled formats);
- * 0 = layouts without chunked kernels, run token by token with the same result. */
+ * path a model takes: 2 = fp32 matrix-core GEMM over the dequantised tiles (every format with a tiled layout), at most
+ * 32 tokens per pass; 1 = the GEMV kernels with one workgroup per token and tile sharing the weights through L2 (the
+ * same layouts when the context was created with SLAI_PROMPT_GEMM=0); 0 = layouts without chunked kernels, run token by
+ * token with the same result. */
 int slai_llama2_prefill(slai_llama2 *m, const int32_t *tokens, uint32_t n_tokens, uint32_t start_pos, uint32_t chunk,
                         float *elapsed_ms);
 int slai_llama2_prefill_supported(const slai_llama2 *m);

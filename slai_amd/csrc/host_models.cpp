@@ -583,7 +583,10 @@ int gemm_chunk_call(slai_ctx *ctx, int nmat, const slai_qmat *const *mats, float
         p.nseg = 0; p.ncols = mats[i]->ncols; p.ncb = mats[i]->ncb; p.ngroups = mats[i]->ngroups; p.rows_log2 = mats[i]->rows_log2;
         p.x = xq; p.ntokens = ntokens; p.ksplit = ksplit;
         for (int j = i; j < nmat; ++j) {
-            if (done[j] || (j != i && (mats[j]->rows_log2 != 6 || mats[i]->rows_log2 != 6 || mats[j]->ncols != mats[i]->ncols))) continue;
+            // (one launch: 64-row tiles of the same width, and of the same format unless both are K-quants)
+            const auto kquant = [](int t) { return t == T_Q4_K || t == T_Q5_K || t == T_Q6_K; };
+            if (done[j] || (j != i && (mats[j]->rows_log2 != 6 || mats[i]->rows_log2 != 6 || mats[j]->ncols != mats[i]->ncols ||
+                                       (mats[j]->type != mats[i]->type && !(kquant(mats[j]->type) && kquant(mats[i]->type)))))) continue;
             GemmChunkSeg &sg = p.seg[p.nseg++];
             sg.W = mats[j]->dptr; sg.type = mats[j]->type; sg.nrows = mats[j]->nrows; sg.out = outs[j]; sg.out_stride = out_strides[j]; sg.flags = flags;
             sg.part_stride = 32 * out_strides[j];

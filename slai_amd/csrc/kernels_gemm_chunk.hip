@@ -4,7 +4,7 @@
 // once per prompt token (crates/slai-chat/src/chat_llama2.rs:105-158).  Here out[t][r] = sum_c deq(W[r][c]) * x[t][c]
 // for all tokens t of the chunk in one pass over W, in fp32 throughout: the weights are dequantised exactly as the
 // per-block `dequantize` of crates/slai/src/quantization.rs does (d * sc * q - dmin * m for Q4_K / Q5_K, d * sc * (q - 32)
-// for Q6_K) and fed to fp32 MFMA instructions, so the result differs from the GEMV's only in the order of the sum.
+// for Q6_K, d * q for Q8_0, d * (q - 8) for Q4_0) and fed to fp32 MFMA instructions, so the result differs from the GEMV's only in the order of the sum.
 //
 // The tiled weight layouts (quant_tiled.h) give every lane ONE ROW of a tile and whole 256-column super-blocks, which is
 // the A-operand layout of the one-column-deep MFMA shapes:
@@ -120,6 +120,36 @@ template <> struct Deq<T_Q6_K> {
         constexpr int C1 = F::c1(K), C2 = F::c2(K);
 #pragma unroll
         for (int b = 0; b < 4; ++b) { lo[b] = ds[C1] * (ub(qa, b) - 32.0f); hi[b] = ds[C2] * (ub(qb, b) - 32.0f); }
+    }
+};
+
+template <> struct Deq<T_Q8_0> {          // BlockQ8_0, quantization.rs:29-42: value = int8 * scale; stage K = block K
+    using F = Tiled<T_Q8_0>;
+    float sc[8], off[8];                                       // scale and -128 * scale of the eight 32-element blocks
+    __device__ __forceinline__ void head(const typename F::Data &d, uint16_t) {
+#pragma unroll
+        for (int B = 0; B < 8; ++B) { sc[B] = F::scale_of(d, B); off[B] = -128.0f * sc[B]; }
+    }
+    template <int K, int W> __device__ __forceinline__ void quad(const typename F::Data &d, float (&lo)[4], float (&hi)[4]) const {
+        // int8 -> unsigned through ^0x80 (one byte conversion instruction), the 128 taken off again with the scale
+        const uint32_t qa = word(d.p[2 * K], W) ^ 0x80808080u, qb = word(d.p[2 * K + 1], W) ^ 0x80808080u;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) { lo[b] = fmaf(sc[K], ub(qa, b), off[K]); hi[b] = fmaf(sc[K], ub(qb, b), off[K]); }
+    }
+};
+
+template <> struct Deq<T_Q4_0> {          // BlockQ4_0, quantization.rs:47-69: value = (nibble - 8) * scale; stage K = block K
+    using F = Tiled<T_Q4_0>;
+    float sc[8], off[8];
+    __device__ __forceinline__ void head(const typename F::Data &d, uint16_t) {
+#pragma unroll
+        for (int B = 0; B < 8; ++B) { sc[B] = F::scale_of(d, B); off[B] = -8.0f * sc[B]; }
+    }
+    template <int K, int W> __device__ __forceinline__ void quad(const typename F::Data &d, float (&lo)[4], float (&hi)[4]) const {
+        const uint32_t q = word(d.p[K], W);
+        const uint32_t ql = q & 0x0F0F0F0Fu, qh = (q >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) { lo[b] = fmaf(sc[K], ub(ql, b), off[K]); hi[b] = fmaf(sc[K], ub(qh, b), off[K]); }
     }
 };
 
@@ -441,7 +471,7 @@ __global__ void rows_to_quads_kernel(float4 *out, const float *x, uint32_t n, ui
 }  // namespace
 
 bool gemm_chunk_supports(const slai_qmat *m) {
-    if (!m || !m->tiled || (m->type != T_Q4_K && m->type != T_Q6_K && m->type != T_Q5_K)) return false;
+    if (!m || !m->tiled || !tiled_supported(m->type)) return false;
     return m->rows_log2 >= 4 && m->rows_log2 <= 6 && m->ngroups <= 64;
 }
 
@@ -460,8 +490,12 @@ hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint3
 hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
     if (p.nseg < 1 || p.nseg > 3 || p.ntokens == 0 || p.ntokens > 32 || p.ncb == 0 || p.ncols != p.ncb * 256 || ((uintptr_t)p.x & 15))
         return hipErrorInvalidValue;
-    for (int i = 0; i < p.nseg; ++i)
-        if (p.seg[i].type != T_Q4_K && p.seg[i].type != T_Q6_K && p.seg[i].type != T_Q5_K) return hipErrorInvalidValue;
+    for (int i = 0; i < p.nseg; ++i) {
+        const int t = p.seg[i].type;
+        if (!tiled_supported(t)) return hipErrorInvalidValue;
+        // segments of different formats in one launch: the K-quants only
+        if (t != p.seg[0].type && (t == T_Q8_0 || t == T_Q4_0 || p.seg[0].type == T_Q8_0 || p.seg[0].type == T_Q4_0)) return hipErrorInvalidValue;
+    }
     hipStream_t st = ctx->stream;
     if (p.rows_log2 == 6) {
         uint32_t tiles = 0;
@@ -479,7 +513,8 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
             for (int i = 0; i < p.nseg; ++i)
                 if (p.seg[i].flags & (GEMV_BIAS | GEMV_ACCUM)) return hipErrorInvalidValue;
         const uint32_t per = (p.ncb + p.ksplit - 1) / p.ksplit;
-        const uint32_t nw = std::min(per, 16u);
+        // (a Q8_0 super-block is 68 registers of weights per lane: eight waves, whose bound leaves 256 registers)
+        const uint32_t nw = std::min(per, tt == T_Q8_0 ? 8u : 16u);
         const size_t smem = (size_t)nw * 32 * G64_LDS_ROW * sizeof(float);
         const int NT = (int)nw * 64;
         const dim3 grid(tiles, p.ksplit);
@@ -487,6 +522,8 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
         case T_Q4_K: gemm64_kernel<T_Q4_K, 1024><<<grid, NT, smem, st>>>(p); break;
         case T_Q5_K: gemm64_kernel<T_Q5_K, 1024><<<grid, NT, smem, st>>>(p); break;
         case T_Q6_K: gemm64_kernel<T_Q6_K, 1024><<<grid, NT, smem, st>>>(p); break;
+        case T_Q4_0: gemm64_kernel<T_Q4_0, 1024><<<grid, NT, smem, st>>>(p); break;
+        case T_Q8_0: gemm64_kernel<T_Q8_0, 512><<<grid, NT, smem, st>>>(p); break;
         default: gemm64_kernel<0, 1024><<<grid, NT, smem, st>>>(p); break;
         }
         return hipGetLastError();
@@ -514,6 +551,8 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
             switch (p.seg[0].type) {
             case T_Q4_K: SLAI_G32(T_Q4_K); break;
             case T_Q6_K: SLAI_G32(T_Q6_K); break;
+            case T_Q8_0: SLAI_G32(T_Q8_0); break;
+            case T_Q4_0: SLAI_G32(T_Q4_0); break;
             default: SLAI_G32(T_Q5_K); break;
             }
 #undef SLAI_G32
@@ -531,6 +570,8 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
             switch (p.seg[0].type) {
             case T_Q4_K: SLAI_G16(T_Q4_K); break;
             case T_Q6_K: SLAI_G16(T_Q6_K); break;
+            case T_Q8_0: SLAI_G16(T_Q8_0); break;
+            case T_Q4_0: SLAI_G16(T_Q4_0); break;
             default: SLAI_G16(T_Q5_K); break;
             }
 #undef SLAI_G16

@@ -1,7 +1,8 @@
 """Prompt tokens in chunks (slai_llama2_prefill) against the oracle and against the token-by-token device loop.
 
-Three paths, picked by the model's layouts (Llama2.prefill_path): 2 = fp32 matrix-core GEMM (K-quants in 64- and 16-row
-tiles), 1 = the GEMV kernels with one workgroup per token and tile (other tiled layouts), 0 = the ordinary loop.
+Three paths, picked by the model's layouts (Llama2.prefill_path): 2 = fp32 matrix-core GEMM (every format with a tiled
+layout), 1 = the GEMV kernels with one workgroup per token and tile (the same layouts with SLAI_PROMPT_GEMM=0; a gated
+Q8_0 pair has no such kernel), 0 = the ordinary loop.
 
 The reference has no batched prompt pass: it feeds the prompt one token per forward pass (chat_llama2.rs:105-158).
 The chunked pass must leave the caches that loop leaves, so: greedy ids after the prompt identical to the oracle's,
@@ -20,6 +21,26 @@ from slai_amd import gguf_writer as gw
 from slai_amd.runtime import Gguf, Llama2, SlaiError
 
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def backend_no_gemm():
+    """A context created with SLAI_PROMPT_GEMM=0: chunks never take the matrix-core kernels."""
+    import os
+    from slai_amd.runtime import Backend
+    old = os.environ.get("SLAI_PROMPT_GEMM")
+    os.environ["SLAI_PROMPT_GEMM"] = "0"
+    try:
+        b = Backend(0)
+    finally:
+        if old is None:
+            del os.environ["SLAI_PROMPT_GEMM"]
+        else:
+            os.environ["SLAI_PROMPT_GEMM"] = old
+    yield b
+    b.close()
+
+
 LOGIT_TOL = 1e-2      # against the oracle
 SELF_TOL = 1e-3       # against the device's token-by-token pass (fp32 sums in another order; an f16 cache entry may round the other way)
 CACHE_TOL = 2e-3      # cache rows, relative to the largest entry (f16 rounding of values that differ in the last bits)
@@ -126,32 +147,44 @@ def test_prefill_matrix_cores_32_row_tiles(backend, kv_f16):
     check_prefill(backend, data, prompt, 16, [3, 8, 32], kv_f16, expect_path=2)
 
 
-@pytest.mark.parametrize("wtype,path", [(12, 2), (2, 1)], ids=["q4_k-matrix-cores", "q4_0-shared-weights"])
-def test_prefill_feed_forward_wider_than_16384(backend, wtype, path):
+@pytest.mark.parametrize("wtype", [12, 2], ids=["q4_k", "q4_0"])
+def test_prefill_feed_forward_wider_than_16384(backend, backend_no_gemm, wtype):
     """A down projection of 16640 columns (17 column groups of 16-row tiles): more groups than a workgroup has waves,
-    so it takes two launches over slices of the groups, the second accumulating."""
+    so it takes two launches over slices of the groups, the second accumulating; on the matrix cores and through the
+    GEMV kernels."""
     data = gw.llama_gguf(dim=512, hidden_dim=16640, n_layers=2, n_heads=8, n_kv_heads=8, vocab=600, seq_len=48, wtype=wtype, seed=19,
                          std=0.03, norm_random=True)
     prompt = np.random.Generator(np.random.PCG64(19)).integers(0, 600, 25)
-    check_prefill(backend, data, prompt, 10, [16], True, expect_path=path)
+    check_prefill(backend, data, prompt, 10, [16], True, expect_path=2)
+    check_prefill(backend_no_gemm, data, prompt, 10, [16], True, expect_path=1)
+
+
+@pytest.mark.parametrize("wtype", [8, 2], ids=["q8_0", "q4_0"])
+def test_prefill_matrix_cores_q8_0_q4_0(backend, wtype):
+    """The two 32-element block formats on the matrix cores: 64-row tiles (q/k/v, gate/up), 32-row tiles (attention
+    output at this width) and 16-row tiles (down), ragged chunks, f16 cache."""
+    data = gw.llama_gguf(dim=512, hidden_dim=1024, n_layers=3, n_heads=8, n_kv_heads=2, vocab=1000, seq_len=64,
+                         wtype=wtype, seed=11, std=0.06, norm_random=True)
+    prompt = np.random.Generator(np.random.PCG64(8)).integers(0, 1000, 40)
+    check_prefill(backend, data, prompt, 16, [7, 32], True, expect_path=2)
 
 
 @pytest.mark.parametrize("kv_f16", [False, True])
-def test_prefill_shared_weights_q4_0_gqa_ragged_chunks(backend, kv_f16):
-    """Q4_0 has no matrix-core kernel: the chunks go through the GEMV kernels, one workgroup per token and tile.
+def test_prefill_shared_weights_q4_0_gqa_ragged_chunks(backend_no_gemm, kv_f16):
+    """Without the matrix-core kernels the chunks go through the GEMV kernels, one workgroup per token and tile.
     Chunks of 3, 8 (ragged last chunk) and 32 (one chunk)."""
     data = gw.llama_gguf(dim=512, hidden_dim=2816, n_layers=3, n_heads=8, n_kv_heads=2, vocab=1000, seq_len=64,
                          wtype=2, seed=11, std=0.06, norm_random=True)
     prompt = np.random.Generator(np.random.PCG64(8)).integers(0, 1000, 22)
-    check_prefill(backend, data, prompt, 16, [3, 8, 32], kv_f16, expect_path=1)
+    check_prefill(backend_no_gemm, data, prompt, 16, [3, 8, 32], kv_f16, expect_path=1)
 
 
-def test_prefill_shared_weights_q4_0_qwen2(backend):
-    """Q4_0 has no matrix-core kernel; q/k/v biases and Neox pairs."""
-    data = gw.llama_gguf(dim=1024, hidden_dim=1024, n_layers=2, n_heads=8, n_kv_heads=2, vocab=400, seq_len=48, wtype=2,
+def test_prefill_shared_weights_kquants_qwen2(backend_no_gemm):
+    """The GEMV path with q/k/v biases and Neox pairs, Q4_K with a Q6_K v projection."""
+    data = gw.llama_gguf(dim=1024, hidden_dim=1024, n_layers=2, n_heads=8, n_kv_heads=2, vocab=400, seq_len=48, wtype=12, v_type=14,
                          seed=31, std=0.05, arch="qwen2", bias=True, norm_random=True, rope_base=1000000.0, rms_eps=1e-6)
     prompt = np.random.Generator(np.random.PCG64(3)).integers(0, 400, 19)
-    check_prefill(backend, data, prompt, 12, [4, 8], True, model_type=_ffi.MODEL_QWEN2, neox=1, name=b"qwen2", expect_path=1)
+    check_prefill(backend_no_gemm, data, prompt, 12, [4, 8], True, model_type=_ffi.MODEL_QWEN2, neox=1, name=b"qwen2", expect_path=1)
 
 
 def test_prefill_continues_at_a_later_position(backend):
