@@ -200,6 +200,11 @@ int slai_matmul_quant_add_assign(slai_ctx *ctx, slai_view in_out_x, const slai_q
  * (with the weight of the norm that comes next) for the GEMV after it, so that no separate pass is needed. */
 int slai_rms_norm_prepare(slai_ctx *ctx, slai_view out_prepared, slai_view x, slai_view norm_weight);
 /* out = m . v for v in prepared form built with a weight of all ones (no norm): slai_matmul_quant_assign for TILE64 */
+/* Up to 32 vectors through one quantised matrix in one pass over it, on the fp32 matrix cores: out[:, t] = m * x[:, t]
+ * (accumulate != 0: +=) for contiguous column-major `out` (nrows x n) and `x` (ncols x n), n <= 32.  The operator under
+ * slai_llama2_prefill; matrices in a tiled layout only (SLAI_E_SHAPE otherwise).  No counterpart in the reference, whose
+ * `matmul_quant` (context.rs:355-399) takes one vector. */
+int slai_matmul_quant_columns(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, int accumulate);
 int slai_matmul_quant_assign_prepared(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view prepared);
 int slai_rms_norm_matmul_quant_assign_prepared(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, slai_view prepared,
                                                float eps);

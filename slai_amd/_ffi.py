@@ -78,6 +78,7 @@ SIGNATURES = {
     "slai_ffn_gate_up_silu": (i32, [vp, View, vp, vp, View, View, C.c_float]),
     "slai_matmul_quant_add_assign": (i32, [vp, View, vp, View]),
     "slai_rms_norm_prepare": (i32, [vp, View, View, View]),
+    "slai_matmul_quant_columns": (i32, [vp, View, vp, View, C.c_int]),
     "slai_matmul_quant_assign_prepared": (i32, [vp, View, vp, View]),
     "slai_rms_norm_matmul_quant_assign_prepared": (i32, [vp, View, vp, View, View, C.c_float]),
     "slai_ffn_gate_up_silu_prepared": (i32, [vp, View, vp, vp, View, View, C.c_float]),

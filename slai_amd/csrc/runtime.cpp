@@ -471,6 +471,39 @@ SLAI_EXPORT int slai_matmul_quant_assign(slai_ctx *ctx, slai_view out, const sla
     return gemv_call(ctx, c, "slai_matmul_quant_assign");
 }
 
+// Several vectors through one quantised matrix on the matrix cores (kernels_gemm_chunk.hip): out[:, t] (+)= m * x[:, t]
+// for the ntokens <= 32 columns of two contiguous column-major matrices.  The operator under the chunked prompt pass of
+// the models, exposed for tests and callers with their own layer loop; the reference only has the one-vector product
+// (context.rs:355-399).
+SLAI_EXPORT int slai_matmul_quant_columns(slai_ctx *ctx, slai_view out, const slai_qmat *m, slai_view x, int accumulate) {
+    if (!ctx || !m) return SLAI_E_ARG;
+    const char *fn = "slai_matmul_quant_columns";
+    if (!out.buf || !x.buf || out.buf->dtype != SLAI_DT_F32 || x.buf->dtype != SLAI_DT_F32) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": f32 views needed");
+    const uint32_t nt = x.size[1];
+    if (nt == 0 || nt > 32 || out.size[1] != nt || x.size[0] != m->ncols || out.size[0] != m->nrows || x.size[2] != 1 || x.size[3] != 1 ||
+        out.size[2] != 1 || out.size[3] != 1)
+        return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": out must be nrows x n, x ncols x n, n <= 32");
+    if (x.stride[0] != 1 || out.stride[0] != 1 || (nt > 1 && (x.stride[1] != m->ncols || out.stride[1] != m->nrows)) || x.offset % 4)
+        return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": contiguous column-major matrices needed, input offset a multiple of 4");
+    if ((x.offset + (size_t)nt * m->ncols) * 4 > x.buf->bytes || (out.offset + (size_t)nt * m->nrows) * 4 > out.buf->bytes)
+        return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": view beyond its buffer");
+    if (!gemm_chunk_supports(m)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": the matrix has no tiled layout");
+    // the kernels read the activations quad-major with 32 token slots; the GEMV scratch holds that copy
+    if (int rc = gemv_scratch_reserve(ctx, (size_t)32 * m->ncols)) return rc;
+    const float *xp = reinterpret_cast<const float *>(x.buf->dptr) + x.offset;
+    float *op = reinterpret_cast<float *>(out.buf->dptr) + out.offset;
+    SLAI_HIP_TRY(ctx, launch_rows_to_quads(ctx->stream, ctx->gemv_scratch, xp, m->ncols, nt, m->ncols));
+    GemmChunkParams p;
+    p.nseg = 1; p.ncols = m->ncols; p.ncb = m->ncb; p.ngroups = m->ngroups; p.rows_log2 = m->rows_log2;
+    p.x = ctx->gemv_scratch; p.ntokens = nt;
+    p.seg[0].W = m->dptr; p.seg[0].type = m->type; p.seg[0].nrows = m->nrows; p.seg[0].out = op; p.seg[0].out_stride = m->nrows;
+    p.seg[0].flags = accumulate ? GEMV_ACCUM : 0;
+    hipError_t e = launch_gemm_chunk(ctx, p);
+    if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": unsupported shape");
+    if (e != hipSuccess) return hip_fail(ctx, e, fn);
+    return SLAI_OK;
+}
+
 // `prepared` (optional): the slai_rms_norm_prepare form of (x, norm weight); `emit_w` / `emit_out` (optional): leave
 // that form of (result, emit_w) in emit_out.
 static int fused_gemv(slai_ctx *ctx, const char *fn, slai_view out, const slai_qmat *m, const slai_qmat *m2, slai_view v,

@@ -208,6 +208,10 @@ class LlmContext:
     def matmul_quant_add_assign(self, in_out_x, m, v):
         self.backend.check(self.L.slai_matmul_quant_add_assign(self.h, _v(in_out_x), m.h, _v(v)))
 
+    def matmul_quant_columns(self, out, m, x, accumulate=False):
+        """out[:, t] (+)= m * x[:, t] for up to 32 columns, on the matrix cores (tiled layouts only)."""
+        self.backend.check(self.L.slai_matmul_quant_columns(self.h, _v(out), m.h, _v(x), 1 if accumulate else 0))
+
     def matmul_quant_assign_prepared(self, out, m, prepared):
         self.backend.check(self.L.slai_matmul_quant_assign_prepared(self.h, _v(out), m.h, _v(prepared)))
 

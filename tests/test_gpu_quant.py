@@ -316,3 +316,46 @@ def test_wide_matrix_in_16_row_tiles_takes_several_launches(backend, oracle_lib,
     assert rel_err(prep[nrows:], (got * nw).reshape(-1, 16).sum(axis=1)) < 1e-5
     for o in (m, gh, out, gx, gnw, gprep):
         o.destroy()
+
+
+@pytest.mark.parametrize("t", [12, 13, 14, 8, 2], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("shape,layout", [((202, 1024), 3), ((64, 4096), 3), ((102, 1024), 2), ((50, 1536), 2), ((42, 16640), 2)],
+                         ids=["64-row-tiles-row-tail", "64-row-tiles-16-super-blocks", "16-row-tiles-row-tail", "32-row-tiles", "16-row-tiles-17-groups"])
+def test_matmul_quant_columns_on_the_matrix_cores(backend, oracle_lib, t, shape, layout):
+    """slai_matmul_quant_columns (the fp32 MFMA kernels under the chunked prompt pass) against the dequantised matrix
+    times the vectors in float64: every format with a tiled layout, the three tile heights, row counts that end inside a
+    tile and inside a group of four rows, 1 / 7 / 32 vectors, assign and accumulate."""
+    import os
+    if os.environ.get("SLAI_TILED") == "0":
+        pytest.skip("needs the tiled layouts")
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext
+    nrows, ncols = shape
+    ctxt = LlmContext(backend)
+    raw = synth.normal_quantized(1300 + t, t, nrows, ncols, 0.02)
+    w = oracle_deq(oracle_lib, t, raw, nrows * ncols).reshape(nrows, ncols).astype(np.float64)
+    m = GpuQuantMatrix(backend, t, nrows, ncols, raw, layout=layout)
+    for n in (1, 7, 32):
+        x = synth.normal(40 + n, ncols * n, 1.0).reshape(ncols, n)
+        ref = w @ x.astype(np.float64)
+        gx = GpuTensor.matrix(backend, x)
+        out = GpuTensor(backend, nrows, n)
+        out.write(np.full(nrows * n, 3.0, np.float32))          # must be overwritten, not added to
+        ctxt.matmul_quant_columns(out, m, gx)
+        got = out.read_matrix()
+        assert rel_err(got, ref) < 1e-5, (n, rel_err(got, ref))
+        old = synth.normal(90 + n, nrows * n, 1.0).reshape(nrows, n)
+        acc = GpuTensor.matrix(backend, old)
+        ctxt.matmul_quant_columns(acc, m, gx, accumulate=True)
+        assert rel_err(acc.read_matrix(), old + ref) < 1e-5
+        for o in (gx, out, acc):
+            o.destroy()
+    # error paths: too many vectors, wrong shapes
+    gx = GpuTensor(backend, ncols, 33); out = GpuTensor(backend, nrows, 33)
+    with pytest.raises(Exception):
+        ctxt.matmul_quant_columns(out, m, gx)
+    bad = GpuTensor(backend, ncols + 4, 2); out2 = GpuTensor(backend, nrows, 2)
+    with pytest.raises(Exception):
+        ctxt.matmul_quant_columns(out2, m, bad)
+    for o in (gx, out, bad, out2):
+        o.destroy()
+    m.destroy()
