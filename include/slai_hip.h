@@ -323,6 +323,12 @@ int slai_gpt2_generate(slai_gpt2 *m, const int32_t *prompt, uint32_t n_prompt, u
 int slai_gpt2_generate_sampled(slai_gpt2 *m, const int32_t *prompt, uint32_t n_prompt, uint32_t start_pos,
                                uint32_t n_steps, float temperature, float topp, uint64_t seed, int32_t *out_tokens,
                                float *elapsed_ms);
+/* slai_llama2_prefill for GPT-2 (gpt2/cpu.rs:225-383 for a chunk of tokens; no counterpart in the reference): 32 tokens
+ * per pass over the weights on the fp32 matrix cores where every layer matrix has a tiled layout
+ * (slai_gpt2_prefill_supported() == 2), token by token with the same result otherwise (0). */
+int slai_gpt2_prefill(slai_gpt2 *m, const int32_t *tokens, uint32_t n_tokens, uint32_t start_pos, uint32_t chunk,
+                      float *elapsed_ms);
+int slai_gpt2_prefill_supported(const slai_gpt2 *m);
 
 /* ---- Tokenizers (host only) ---------------------------------------------------
  * `AnyTokenizer` (crates/slai-chat/src/llm.rs:100-164) over `LlamaTokenizer`

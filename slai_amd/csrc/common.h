@@ -207,6 +207,8 @@ bool gemm_chunk_supports(const slai_qmat *m);
 hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p);
 // quad-major out = RMSNorm of the `ntokens` row-major vectors of n floats at x + t * x_stride
 hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps);
+// the same with LayerNorm (mean-centred, * g + b)
+hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps);
 // quad-major copy of row-major vectors
 hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride);
 
@@ -322,7 +324,9 @@ hipError_t launch_attention(hipStream_t s, const AttnLaunch &a);
 // n <= 32); knew / vnew must be null.  One workgroup per head and token.
 hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride, bool out_quads = false);
 // out[b] = embedding row tokens[b] (dequantised), b < n
-hipError_t launch_embed_rows(hipStream_t s, const slai_qmat *m, const int *tokens, uint32_t n, uint32_t ncols, float *out, uint32_t out_stride);
+// (+ row positions[b] of `pos_m` when that is given: learned position embeddings)
+hipError_t launch_embed_rows(hipStream_t s, const slai_qmat *m, const int *tokens, uint32_t n, uint32_t ncols, float *out, uint32_t out_stride,
+                             const slai_qmat *pos_m = nullptr, const int *positions = nullptr);
 // The step before it: for token b (position pos_ptr[b]) add the biases, rotate q + b * q_stride in place and write the
 // rotated key k + b * kv_stride and the value v + b * kv_stride to row pos_ptr[b] of the caches.  Uses the q / cache /
 // bias / rope fields of `a`.

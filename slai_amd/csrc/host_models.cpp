@@ -879,6 +879,13 @@ struct slai_gpt2 {
 
     int load(const slai_gguf *g);
     int enqueue_fused(int sampler);   // 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state
+
+    // Prompt tokens in chunks of up to 32 on the matrix cores (see slai_llama2::enqueue_chunk_gemm); row-major x and qkv,
+    // quad-major xn (normalised rows, then the attention output) and h.
+    struct { GpuTensor x, xn, qkv, h; slai_buffer *positions = nullptr, *tokens = nullptr; bool ready = false; } chunk;
+    bool chunk_gemm_supported() const;
+    int chunk_reserve();
+    int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev);
 };
 
 int slai_gpt2::load(const slai_gguf *gg) {
@@ -1006,6 +1013,75 @@ int slai_gpt2::enqueue_fused(int sampler) {
     return SLAI_OK;
 }
 
+bool slai_gpt2::chunk_gemm_supported() const {
+    const uint32_t hs = params.n_embd / params.n_head;
+    if ((hs != 64 && hs != 128) || params.n_embd % 8 || params.n_embd > 16384) return false;
+    for (const Gpt2Layer &w : layers)
+        for (const slai_qmat *m : {w.c_attn_attn_w, w.c_attn_proj_w, w.c_mlp_fc_w, w.c_mlp_proj_w})
+            if (!gemm_chunk_supports(m)) return false;
+    return true;
+}
+
+int slai_gpt2::chunk_reserve() {
+    if (chunk.ready) return SLAI_OK;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "prompt chunk buffers must be reserved before graph capture");
+    const uint32_t E = params.n_embd;
+    TRY(GpuTensor::matrix(ctx, E, 32, STORAGE, &chunk.x));
+    TRY(GpuTensor::matrix(ctx, E, 32, STORAGE, &chunk.xn));
+    TRY(GpuTensor::matrix(ctx, 3 * E, 32, STORAGE, &chunk.qkv));
+    TRY(GpuTensor::matrix(ctx, params.ff_len, 32, STORAGE, &chunk.h));
+    TRY(slai_buffer_create(ctx, (size_t)params.n_seq * 4, SLAI_DT_I32, STORAGE | COPY_DST, &chunk.positions));
+    TRY(slai_buffer_create(ctx, (size_t)params.n_seq * 4, SLAI_DT_I32, STORAGE | COPY_DST, &chunk.tokens));
+    std::vector<uint32_t> iota(params.n_seq);
+    for (uint32_t i = 0; i < params.n_seq; ++i) iota[i] = i;
+    TRY(slai_write_buffer(ctx, chunk.positions, 0, iota.data(), iota.size() * 4));
+    chunk.ready = true;
+    return SLAI_OK;
+}
+
+// gpt2/cpu.rs:225-383 for n <= 32 tokens at once, every projection on the matrix cores: embeddings, then per layer
+// LayerNorm, qkv + bias, cache write, attention, projection + bias into the residual, LayerNorm, fc + bias, GELU,
+// projection + bias into the residual.  No logits.
+int slai_gpt2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev) {
+    if (n == 0 || n > 32 || pos0 + n > params.n_seq) return set_error(ctx, SLAI_E_ARG, "prompt chunk out of range");
+    const uint32_t E = params.n_embd, F = params.ff_len;
+    float *x = (float *)chunk.x.buf->dptr, *xn = (float *)chunk.xn.buf->dptr, *qkv = (float *)chunk.qkv.buf->dptr, *h = (float *)chunk.h.buf->dptr;
+    const int *positions = (const int *)chunk.positions->dptr + pos0;
+    const float eps = 1.0e-5f;
+    SLAI_HIP_TRY(ctx, launch_embed_rows(ctx->stream, wte, tokens_dev, n, E, x, E, wpe, positions));
+    const auto gemm = [&](const slai_qmat *m, const float *bias, float *out, uint32_t out_stride, uint32_t flags, const float *xq, const char *who) -> int {
+        GemmChunkParams p;
+        p.nseg = 1; p.ncols = m->ncols; p.ncb = m->ncb; p.ngroups = m->ngroups; p.rows_log2 = m->rows_log2;
+        p.x = xq; p.ntokens = n;
+        p.seg[0].W = m->dptr; p.seg[0].type = m->type; p.seg[0].nrows = m->nrows; p.seg[0].out = out; p.seg[0].out_stride = out_stride;
+        p.seg[0].bias = bias; p.seg[0].flags = flags;
+        hipError_t e = launch_gemm_chunk(ctx, p);
+        if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, std::string(who) + ": unsupported shape for the prompt-chunk GEMM");
+        if (e != hipSuccess) return hip_fail(ctx, e, who);
+        return SLAI_OK;
+    };
+    for (uint32_t l = 0; l < params.n_layer; ++l) {
+        Gpt2Layer &w = layers[l];
+        SLAI_HIP_TRY(ctx, launch_layernorm_quads(ctx->stream, xn, x, (const float *)w.ln_1_g.buf->dptr, (const float *)w.ln_1_b.buf->dptr, E, n, E, eps));
+        TRY(gemm(w.c_attn_attn_w, (const float *)w.c_attn_attn_b.buf->dptr, qkv, 3 * E, GEMV_BIAS, xn, "gpt2 qkv (prompt chunk)"));
+        AttnLaunch a{};
+        a.q = qkv; a.kcache = w.key_cache.buf->dptr; a.vcache = w.value_cache.buf->dptr; a.kv_f16 = kv_dtype == SLAI_KV_F16;
+        a.n_heads = params.n_head; a.kv_mul = 1; a.head_size = E / params.n_head; a.kv_dim = E; a.seq_len = params.n_seq;
+        a.pos_ptr = (const uint32_t *)positions;
+        a.rope_variant = -1; a.rope_base = 0.0f;
+        a.out = xn; a.scratch = nullptr; a.n_splits = 1;
+        // keys and values of all tokens into the caches first (no rotation: learned positions), then the attention of each
+        SLAI_HIP_TRY(ctx, launch_rope_store_batch(ctx->stream, a, qkv, qkv + E, qkv + 2 * E, n, 3 * E, 3 * E));
+        SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, 3 * E, E, true));
+        TRY(gemm(w.c_attn_proj_w, (const float *)w.c_attn_proj_b.buf->dptr, x, E, GEMV_BIAS | GEMV_ACCUM, xn, "gpt2 attn proj (prompt chunk)"));
+        SLAI_HIP_TRY(ctx, launch_layernorm_quads(ctx->stream, xn, x, (const float *)w.ln_2_g.buf->dptr, (const float *)w.ln_2_b.buf->dptr, E, n, E, eps));
+        TRY(gemm(w.c_mlp_fc_w, (const float *)w.c_mlp_fc_b.buf->dptr, h, F, GEMV_BIAS | GEMM_OUT_QUADS, xn, "gpt2 mlp fc (prompt chunk)"));
+        SLAI_HIP_TRY(ctx, launch_gelu(ctx->stream, VecView{h, 32 * F, 1}));     // element-wise: the layout does not matter
+        TRY(gemm(w.c_mlp_proj_w, (const float *)w.c_mlp_proj_b.buf->dptr, x, E, GEMV_BIAS | GEMV_ACCUM, h, "gpt2 mlp proj (prompt chunk)"));
+    }
+    return SLAI_OK;
+}
+
 SLAI_EXPORT int slai_gpt2_from_gguf(slai_ctx *ctx, const slai_gguf *g, int kv_dtype, slai_gpt2 **out) {
     if (!ctx || !g || !out) return SLAI_E_ARG;
     *out = nullptr;
@@ -1030,6 +1106,8 @@ SLAI_EXPORT void slai_gpt2_destroy(slai_gpt2 *m) {
     }
     slai_qmat_destroy(ctx, m->wte); slai_qmat_destroy(ctx, m->wpe);
     for (GpuTensor *t : {&m->ln_f_g, &m->ln_f_b, &m->layer_input, &m->curr_768, &m->curr_2304, &m->curr_3072, &m->curr_vocab}) t->destroy(ctx);
+    for (GpuTensor *t : {&m->chunk.x, &m->chunk.xn, &m->chunk.qkv, &m->chunk.h}) t->destroy(ctx);
+    for (slai_buffer *b : {m->chunk.positions, m->chunk.tokens}) if (b) slai_buffer_destroy(ctx, b);
     delete m;
 }
 
@@ -1062,4 +1140,39 @@ SLAI_EXPORT int slai_gpt2_generate_sampled(slai_gpt2 *m, const int32_t *prompt, 
     if (!m) return SLAI_E_ARG;
     const SamplingParams sp{temperature, topp, seed};
     return generate_impl(m, m->ctx, m->loop, m->params.n_seq, m->params.n_vocab, prompt, n_prompt, start_pos, n_steps, out_tokens, elapsed_ms, &sp);
+}
+
+// 0: the ordinary loop, 2: matrix cores (see slai_llama2_prefill_supported)
+SLAI_EXPORT int slai_gpt2_prefill_supported(const slai_gpt2 *m) { return m && m->ctx->prompt_gemm && m->chunk_gemm_supported() ? 2 : 0; }
+
+// slai_llama2_prefill for GPT-2: fills the caches for positions start_pos .. start_pos + n_tokens - 1, 32 tokens per pass
+// over the weights where every layer matrix has a tiled layout, token by token otherwise; no logits.
+SLAI_EXPORT int slai_gpt2_prefill(slai_gpt2 *m, const int32_t *tokens, uint32_t n_tokens, uint32_t start_pos, uint32_t chunk, float *elapsed_ms) {
+    if (!m) return SLAI_E_ARG;
+    slai_ctx *ctx = m->ctx;
+    if (elapsed_ms) *elapsed_ms = 0.0f;
+    if (n_tokens == 0) return SLAI_OK;
+    if (!tokens) return set_error(ctx, SLAI_E_ARG, "slai_gpt2_prefill: no tokens");
+    if ((uint64_t)start_pos + n_tokens > m->params.n_seq) return set_error(ctx, SLAI_E_SHAPE, "slai_gpt2_prefill: would run past the context length");
+    for (uint32_t i = 0; i < n_tokens; ++i)
+        if (tokens[i] < 0 || (uint32_t)tokens[i] >= m->params.n_vocab) return set_error(ctx, SLAI_E_ARG, "slai_gpt2_prefill: token out of range");
+    if (chunk > 64) return set_error(ctx, SLAI_E_ARG, "slai_gpt2_prefill: at most 64 tokens per chunk");
+    const bool gemm = ctx->prompt_gemm && m->chunk_gemm_supported();
+    if (chunk == 0) chunk = 32;
+    if (chunk == 1 || !gemm) {
+        std::vector<int32_t> prompt((size_t)start_pos + n_tokens, 0), picks(n_tokens);
+        std::copy(tokens, tokens + n_tokens, prompt.begin() + start_pos);
+        return generate_impl(m, ctx, m->loop, m->params.n_seq, m->params.n_vocab, prompt.data(), (uint32_t)prompt.size(), start_pos, n_tokens, picks.data(),
+                             elapsed_ms);
+    }
+    if (chunk > 32) chunk = 32;
+    TRY(m->chunk_reserve());
+    TRY(slai_write_buffer(ctx, m->chunk.tokens, 0, tokens, (size_t)n_tokens * 4));
+    const int *tokens_dev = (const int *)m->chunk.tokens->dptr;
+    SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev0, ctx->stream));
+    for (uint32_t i = 0; i < n_tokens; i += chunk) TRY(m->enqueue_chunk_gemm(start_pos + i, std::min(chunk, n_tokens - i), tokens_dev + i));
+    SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev1, ctx->stream));
+    TRY(slai_synchronize(ctx));
+    if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, m->loop.ev0, m->loop.ev1));
+    return SLAI_OK;
 }

@@ -68,9 +68,12 @@ __global__ void embed_kernel(QMatDev a, const int *row_a, QMatDev b, const int *
 }
 
 // one embedding row per token of a chunk: grid = (columns / 256, tokens)
-__global__ void embed_rows_kernel(QMatDev a, const int *rows, uint32_t ncols, float *out, uint32_t out_stride) {
+__global__ void embed_rows_kernel(QMatDev a, const int *rows, QMatDev pm, const int *positions, int has_pos, uint32_t ncols, float *out, uint32_t out_stride) {
     const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
-    if (c < ncols) out[(size_t)b * out_stride + c] = qmat_elem(a, (uint32_t)rows[b], c);
+    if (c >= ncols) return;
+    float v = qmat_elem(a, (uint32_t)rows[b], c);
+    if (has_pos) v = v + qmat_elem(pm, (uint32_t)positions[b], c);     // gpt2/cpu.rs:227-228
+    out[(size_t)b * out_stride + c] = v;
 }
 
 }  // namespace
@@ -100,9 +103,10 @@ hipError_t launch_embed(hipStream_t s, const slai_qmat *a, const int *row_a, con
     return hipGetLastError();
 }
 
-hipError_t launch_embed_rows(hipStream_t s, const slai_qmat *m, const int *tokens, uint32_t n, uint32_t ncols, float *out, uint32_t out_stride) {
-    if (n == 0 || n > 65535) return hipErrorInvalidValue;
-    embed_rows_kernel<<<dim3((ncols + 255) / 256, n), 256, 0, s>>>(qmat_dev(m), tokens, ncols, out, out_stride);
+hipError_t launch_embed_rows(hipStream_t s, const slai_qmat *m, const int *tokens, uint32_t n, uint32_t ncols, float *out, uint32_t out_stride,
+                             const slai_qmat *pos_m, const int *positions) {
+    if (n == 0 || n > 65535 || (pos_m && !positions)) return hipErrorInvalidValue;
+    embed_rows_kernel<<<dim3((ncols + 255) / 256, n), 256, 0, s>>>(qmat_dev(m), tokens, qmat_dev(pos_m), positions, pos_m ? 1 : 0, ncols, out, out_stride);
     return hipGetLastError();
 }
 

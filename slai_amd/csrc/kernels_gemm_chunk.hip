@@ -462,6 +462,50 @@ __global__ void __launch_bounds__(256) rms_norm_quads_kernel(float4 *out, const 
     }
 }
 
+// LayerNorm of token t = blockIdx.x (ops/layernorm.rs:104-111: mean, centred values, variance = their squared norm / n,
+// 1 / sqrt(variance + eps)), then * g + b, written quad-major.  n % 4 == 0, n <= 16384.
+__global__ void __launch_bounds__(256) layernorm_quads_kernel(float4 *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t x_stride, float eps) {
+    __shared__ float red[4], red2[4];
+    const uint32_t t = blockIdx.x, nq = n / 4;
+    const float4 *xr = (const float4 *)(x + (size_t)t * x_stride), *gr = (const float4 *)g, *br = (const float4 *)b;
+    float4 v[16];
+    float sm = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const uint32_t i = threadIdx.x + 256u * j;
+        v[j] = i < nq ? xr[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        sm += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) sm += __shfl_xor(sm, m, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sm;
+    __syncthreads();
+    const float mean = ((red[0] + red[1]) + (red[2] + red[3])) / (float)n;
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const uint32_t i = threadIdx.x + 256u * j;
+        if (i < nq) {
+            v[j].x -= mean; v[j].y -= mean; v[j].z -= mean; v[j].w -= mean;
+            ss = fmaf(v[j].x, v[j].x, ss); ss = fmaf(v[j].y, v[j].y, ss); ss = fmaf(v[j].z, v[j].z, ss); ss = fmaf(v[j].w, v[j].w, ss);
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
+    if ((threadIdx.x & 63) == 0) red2[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float scale = 1.0f / sqrtf(((red2[0] + red2[1]) + (red2[2] + red2[3])) / (float)n + eps);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const uint32_t i = threadIdx.x + 256u * j;
+        if (i < nq) {
+            const float4 gg = gr[i], bb = br[i];
+            out[(size_t)i * 32 + t] = make_float4((v[j].x * scale) * gg.x + bb.x, (v[j].y * scale) * gg.y + bb.y, (v[j].z * scale) * gg.z + bb.z,
+                                                  (v[j].w * scale) * gg.w + bb.w);
+        }
+    }
+}
+
 // row-major [tokens][n] -> quad-major; thread = (quad, token), token fastest so that the stores are contiguous
 __global__ void rows_to_quads_kernel(float4 *out, const float *x, uint32_t n, uint32_t x_stride, uint32_t ntokens) {
     const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x, t = idx & 31u, qd = idx >> 5;
@@ -478,6 +522,12 @@ bool gemm_chunk_supports(const slai_qmat *m) {
 hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps) {
     if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || n > 16384 || x_stride % 4) return hipErrorInvalidValue;
     rms_norm_quads_kernel<<<ntokens, 256, 0, s>>>((float4 *)out, x, w, n, x_stride, eps);
+    return hipGetLastError();
+}
+
+hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps) {
+    if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || n > 16384 || x_stride % 4) return hipErrorInvalidValue;
+    layernorm_quads_kernel<<<ntokens, 256, 0, s>>>((float4 *)out, x, g, b, n, x_stride, eps);
     return hipGetLastError();
 }
 

@@ -542,6 +542,17 @@ class Gpt2:
                                                          seed, out.ctypes.data, C.byref(ms)))
         return out, ms.value
 
+    def prefill_path(self):
+        """2: matrix-core GEMM, 0: the token-by-token loop."""
+        return int(self.b.L.slai_gpt2_prefill_supported(self.h))
+
+    def prefill(self, tokens, start_pos=0, chunk=0):
+        """Fill the caches for positions start_pos .. start_pos+len(tokens)-1; returns the stream time in ms."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        ms = C.c_float()
+        self.b.check(self.b.L.slai_gpt2_prefill(self.h, tokens.ctypes.data, tokens.size, start_pos, chunk, C.byref(ms)))
+        return ms.value
+
     def destroy(self):
         if self.h:
             self.b.L.slai_gpt2_destroy(self.h)

@@ -228,3 +228,51 @@ def test_prefill_argument_errors(backend):
         m.prefill(np.array([1, 2, 3], np.int32), chunk=65)
     m.prefill(np.arange(16, dtype=np.int32))                             # exactly the context
     m.destroy(); gg.close()
+
+
+@pytest.mark.parametrize("kv_f16", [False, True])
+def test_gpt2_prefill_matrix_cores(backend, kv_f16):
+    """GPT-2-small widths (dim 768, 12 heads of 64, ff 3072, Q8_0) at depth 2: LayerNorm, biases, learned positions and
+    GELU in the chunked pass.  Greedy ids after a 45-token prompt identical to the oracle's, logits at the last prompt
+    position within 1e-2 of the oracle's and within 1e-3 of the device's token-by-token pass; chunks of 7 and 32, and a
+    continuation at a later position."""
+    from helpers import OracleGguf
+    from slai_amd.runtime import Gpt2
+    data = gw.gpt2_gguf(n_layer=2, seed=51, std=0.05)
+    g = OracleGguf(data); L = g.L
+    om = L.slo_gpt2_from_gguf(g.h, int(kv_f16))
+    assert om
+    prompt = np.random.Generator(np.random.PCG64(52)).integers(0, 50257, 45).astype(np.int32)
+    n, n_gen = prompt.size, 10
+    n_steps = n - 1 + n_gen
+    ref_tokens = np.zeros(n_steps, np.int32); ref_logits = np.zeros((n_steps, 50257), np.float32)
+    assert L.slo_gpt2_generate(om, prompt.ctypes.data, n, 0, n_steps, -1, ref_tokens.ctypes.data, ref_logits.ctypes.data) == n_steps
+    gg = Gguf(data)
+    kv = _ffi.KV_F16 if kv_f16 else _ffi.KV_F32
+    m = Gpt2(backend, gg, kv)
+    assert m.prefill_path() == 2
+    m.generate(prompt, n - 1)
+    base_logits = m.forward_logits(n - 1, int(prompt[-1]))
+    m.destroy()
+    for chunk, split_at in ((7, None), (32, None), (32, 13)):
+        m = Gpt2(backend, gg, kv)
+        if split_at is None:
+            m.prefill(prompt[:-1], 0, chunk)
+        else:
+            m.prefill(prompt[:split_at], 0, chunk)
+            m.prefill(prompt[split_at:-1], split_at, chunk)
+        logits = m.forward_logits(n - 1, int(prompt[-1]))
+        assert rel_err(logits, ref_logits[n - 1]) < LOGIT_TOL, chunk
+        assert rel_err(logits, base_logits) < SELF_TOL, (chunk, rel_err(logits, base_logits))
+        got, _ = m.generate(prompt, n_gen, start_pos=n - 1)
+        assert np.array_equal(got, ref_tokens[n - 1:]), (chunk, got.tolist(), ref_tokens[n - 1:].tolist())
+        m.destroy()
+    # the plain loop behind the same call, and argument errors
+    m = Gpt2(backend, gg, kv)
+    m.prefill(prompt[:-1], 0, 1)
+    assert rel_err(m.forward_logits(n - 1, int(prompt[-1])), base_logits) < 1e-6
+    with pytest.raises(SlaiError):
+        m.prefill(np.array([1, 50257], np.int32))
+    with pytest.raises(SlaiError):
+        m.prefill(np.arange(10, dtype=np.int32), start_pos=1020)
+    m.destroy(); gg.close(); L.slo_gpt2_free(om); g.close()
