@@ -77,9 +77,9 @@ struct DevX {
 };
 
 // Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product.
-template <int T, int N> struct UnitLoader {
-    static constexpr int DEPTH = 2;               // stages requested ahead of the one being multiplied
-    static constexpr int LEAD = 2;                // stages requested before the dot product starts (>= DEPTH)
+template <int T, int N, int LD> struct UnitLoader {
+    static constexpr int DEPTH = LD;              // stages requested ahead of the one being multiplied
+    static constexpr int LEAD = LD;               // stages requested before the dot product starts (>= DEPTH)
     using F = Tiled<T>;
     const uint8_t *unit[N];                       // + lane * 16 already applied
     const uint8_t *tailp[N];
@@ -100,7 +100,7 @@ template <int T, int N> struct UnitLoader {
 // are requested before the current tile is consumed.
 // `vec`: which input vector of a batched launch (0 otherwise) and its strides (see GemvBatch).
 struct TiledVec { size_t x_off, emit_off, out0, out1, out2; };
-template <int T, bool DUAL>
+template <int T, bool DUAL, int LD>
 __device__ __forceinline__ void tiled_body(const GemvTiledParams &p, uint32_t blk, float *smem, const TiledVec vec) {
     using F = Tiled<T>;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, NW = blockDim.x >> 6;
@@ -147,7 +147,7 @@ __device__ __forceinline__ void tiled_body(const GemvTiledParams &p, uint32_t bl
     constexpr int NM = DUAL ? 2 : 1;
     typename F::Data d, e;                                   // e: second matrix of a gated pair
     uint16_t dt = 0, et = 0;
-    UnitLoader<T, NM> ld;
+    UnitLoader<T, NM, LD> ld;
     auto point = [&](uint32_t t) {
         const size_t off = ((size_t)t * p.ngroups + g) * p.unit_bytes;
         ld.unit[0] = seg.W + off + lane * 16; ld.tailp[0] = seg.W + off + (size_t)F::PT * 1024 + lane * 2; ld.d[0] = &d; ld.t[0] = &dt;
@@ -266,11 +266,16 @@ __device__ __forceinline__ void tiled_body(const GemvTiledParams &p, uint32_t bl
     }
 }
 
+// Stages of weights a wave requests ahead.  Workgroups of up to four waves (narrow matrices: one wave per four
+// super-blocks) have little in flight per compute unit and gain from four (+0.3 % on the 7B decode); wider ones lose
+// with more than two, and so do the narrow ones with six or eight.
+constexpr int lead_stages(int maxt) { return maxt <= 256 ? 4 : 2; }
+
 template <int T, bool DUAL, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemv_tiled_kernel(const GemvTiledParams p) {
     extern __shared__ float smem[];
     touch_kernel_arguments<sizeof(GemvTiledParams)>();
-    tiled_body<T, DUAL>(p, blockIdx.x, smem, TiledVec{0, 0, 0, 0, 0});
+    tiled_body<T, DUAL, lead_stages(MAXT)>(p, blockIdx.x, smem, TiledVec{0, 0, 0, 0, 0});
 }
 
 // The same for several input vectors (a chunk of prompt tokens).  Workgroup i runs on XCD i % 8 and workgroups are
@@ -286,7 +291,7 @@ __global__ void __launch_bounds__(MAXT) gemv_tiled_batch_kernel(const GemvTiledP
     if (blk >= total_blocks) return;                            // (uniform) the block count rounded up to the eight XCDs
     const TiledVec vec{(size_t)b * bt.x_stride, (size_t)b * bt.emit_stride,
                        (size_t)b * bt.out_stride[0], (size_t)b * bt.out_stride[1], (size_t)b * bt.out_stride[2]};
-    tiled_body<T, DUAL>(p, blk, smem, vec);
+    tiled_body<T, DUAL, lead_stages(MAXT)>(p, blk, smem, vec);
 }
 
 template <int T, bool DUAL>
