@@ -300,13 +300,17 @@ int slai_llama2_generate_sampled(slai_llama2 *m, const int32_t *prompt, uint32_t
  * this fills the caches for positions start_pos .. start_pos+n_tokens-1 with `chunk` tokens per pass over the
  * weights and computes no logits (chunk: 0 = the path's default, 1 = token by token, at most 64).  Generation then
  * continues with slai_llama2_generate(prompt, n_prompt, n_prompt - 1, ...).  slai_llama2_prefill_supported() says which
- * path a model takes: 2 = fp32 matrix-core GEMM over the dequantised tiles (every format with a tiled layout), at most
- * 32 tokens per pass; 1 = the GEMV kernels with one workgroup per token and tile sharing the weights through L2 (the
+ * path a model takes: 2 = matrix-core GEMM over the dequantised tiles (every format with a tiled layout), at most
+ * 32 tokens per pass: on the half-precision units with every weight and activation split into an f16 head and an f16
+ * remainder (about 22 bits of each, fp32 accumulation), repeated with fp32 MFMA when an activation turns out to be beyond
+ * the f16 range (slai_llama2_prefill_fp32_repeats counts those calls), in fp32 MFMA from the start when the context was
+ * created with SLAI_PROMPT_SPLIT_F16=0; 1 = the GEMV kernels with one workgroup per token and tile sharing the weights through L2 (the
  * same layouts when the context was created with SLAI_PROMPT_GEMM=0); 0 = layouts without chunked kernels, run token by
  * token with the same result. */
 int slai_llama2_prefill(slai_llama2 *m, const int32_t *tokens, uint32_t n_tokens, uint32_t start_pos, uint32_t chunk,
                         float *elapsed_ms);
 int slai_llama2_prefill_supported(const slai_llama2 *m);
+uint32_t slai_llama2_prefill_fp32_repeats(const slai_llama2 *m);
 /* Device access for set-up and inspection: layer l's caches ([kv_dim x seq_len]) and the state vectors. */
 int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache);
 int slai_llama2_logits_buffer(slai_llama2 *m, slai_buffer **logits);

@@ -50,6 +50,8 @@ struct slai_ctx {
     uint32_t *handoff_counters = nullptr;   // q/k/v + attention in one launch: one 128-byte line per head, then a timeout flag
     uint32_t handoff_heads = 0;
     bool fuse_qkv_attention = true;     // SLAI_FUSE_QKV_ATTN=0: always separate launches
+    int prompt_split_f16 = 1;           // SLAI_PROMPT_SPLIT_F16: 0 = prompt-chunk GEMMs in fp32 MFMA, 1 = the models' on the f16 matrix cores (f16 head + remainder), 2 = slai_matmul_quant_columns too
+    int *split_flag = nullptr;          // device word the kernels that write split activations set when a value is beyond f16
     bool prompt_gemm = true;            // SLAI_PROMPT_GEMM=0: prompt chunks never take the matrix-core kernels
     // tuning knobs (environment overridable, see runtime.cpp)
     int gemv_rows_per_wg = 8;
@@ -202,15 +204,20 @@ struct GemmChunkParams {
     // workgroup of its own (tile counts rarely divide the compute units evenly; smaller units do); range s writes its
     // partial result to out + s * part_stride and the reader adds them up.  No bias, no accumulation then.
     uint32_t ksplit = 1;
+    // weights and activations as f16 head + remainder pairs on the half-precision matrix cores (about 22 bits of each;
+    // |x| < 65504, |w| < 255) instead of fp32 MFMA; x must then hold the split form (split_flag of the kernels that write it).
+    bool split_f16 = false;
 };
 bool gemm_chunk_supports(const slai_qmat *m);
 hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p);
 // quad-major out = RMSNorm of the `ntokens` row-major vectors of n floats at x + t * x_stride
-hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps);
+hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps, int *split_flag = nullptr);
 // the same with LayerNorm (mean-centred, * g + b)
 hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps);
 // quad-major copy of row-major vectors
-hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride);
+hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride, int *split_flag = nullptr);
+// quad-major f32 -> f16 heads and remainders in place (see GemmChunkParams::split_f16); *split_flag = 1 when a value is beyond f16
+hipError_t launch_quads_split(hipStream_t s, float *x, uint32_t n, uint32_t ntokens, int *split_flag);
 
 // One GEMV launch over up to three matrices of one format and layout: out[i] = epilogue(m[i] . prologue(x)).
 struct GemvCall {
@@ -335,7 +342,7 @@ hipError_t launch_embed_rows(hipStream_t s, const slai_qmat *m, const int *token
 hipError_t launch_rope_store_batch(hipStream_t s, const AttnLaunch &a, float *q, const float *k, const float *v, uint32_t n, uint32_t q_stride, uint32_t kv_stride,
                                    uint32_t nparts = 1, uint32_t q_part = 0, uint32_t kv_part = 0);
 // a[i] = silu(sum_s a[i + s * part]) * sum_s b[i + s * part], i < n (silu.slang:11-27 over partial results)
-hipError_t launch_silu_parts(hipStream_t s, float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part);
+hipError_t launch_silu_parts(hipStream_t s, float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part, int *split_flag = nullptr, uint32_t ntokens = 32);
 // q/k/v GEMV (three segments in the order v, k, q) and the attention over their results in one launch
 hipError_t launch_qkv_attention(slai_ctx *ctx, GemvRowtileParams p, const AttnLaunch &a);
 // out[i] = powf(base, -((2*i) % head_size) / head_size), i < head_size/2

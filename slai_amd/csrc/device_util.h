@@ -18,4 +18,24 @@ template <int BYTES> __device__ __forceinline__ void touch_kernel_arguments() {
     asm volatile("" : : "s"(w));
 }
 
+// A value as an f16 head plus an f16 remainder (both rounded toward zero; the remainder of the head is exact in f32), about
+// 22 bits together: the form in which the prompt-chunk GEMM reads activations for the half-precision matrix cores.
+// split_quad packs four values as {heads 0-1, heads 2-3, remainders 0-1, remainders 2-3} into the 16 bytes of the float4.
+__device__ __forceinline__ void split_pair_f16(float a, float b, uint32_t &h, uint32_t &l) {
+    const auto hh = __builtin_amdgcn_cvt_pkrtz(a, b);
+    const auto ll = __builtin_amdgcn_cvt_pkrtz(fmaf((float)hh[0], -1.0f, a), fmaf((float)hh[1], -1.0f, b));
+    h = __builtin_bit_cast(uint32_t, hh);
+    l = __builtin_bit_cast(uint32_t, ll);
+}
+__device__ __forceinline__ float4 split_quad(float4 v) {
+    uint32_t h0, h1, l0, l1;
+    split_pair_f16(v.x, v.y, h0, l0);
+    split_pair_f16(v.z, v.w, h1, l1);
+    return make_float4(__uint_as_float(h0), __uint_as_float(h1), __uint_as_float(l0), __uint_as_float(l1));
+}
+// true when a value does not fit the f16 head (NaN included)
+__device__ __forceinline__ bool split_overflows(float4 v) {
+    return !(fabsf(v.x) < 65504.0f && fabsf(v.y) < 65504.0f && fabsf(v.z) < 65504.0f && fabsf(v.w) < 65504.0f);
+}
+
 }  // namespace slai

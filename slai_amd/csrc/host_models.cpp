@@ -142,7 +142,8 @@ struct slai_llama2 {
     bool chunk_gemm_supported() const;   // matrix cores (K-quants)
     int chunk_reserve(uint32_t rows);
     int enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev);   // fills the caches for positions pos0 .. pos0 + n - 1
-    int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev);   // the same on the matrix cores, n <= 32
+    uint32_t prefill_fp32_repeats = 0;   // prefill calls repeated in fp32 because an activation was beyond the f16 range
+    int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev, bool split_f16);   // the same on the matrix cores, n <= 32
     // q / k / v given as nparts partial sums, 32 rows apart; out_quads: the result goes to xn, quad-major, instead of xb
     int chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts = 1, bool out_quads = false);
 };
@@ -575,13 +576,13 @@ uint32_t chunk_ksplit(int nmat, const slai_qmat *const *mats) {
 
 // matrices (with the same input) through the matrix-core kernel: 64-row-tile matrices share a launch
 int gemm_chunk_call(slai_ctx *ctx, int nmat, const slai_qmat *const *mats, float *const *outs, const uint32_t *out_strides, uint32_t flags,
-                    const float *xq, uint32_t ntokens, const char *who, uint32_t ksplit = 1) {
+                    const float *xq, uint32_t ntokens, const char *who, uint32_t ksplit = 1, bool split_f16 = false) {
     bool done[3] = {false, false, false};
     for (int i = 0; i < nmat; ++i) {
         if (done[i]) continue;
         GemmChunkParams p;
         p.nseg = 0; p.ncols = mats[i]->ncols; p.ncb = mats[i]->ncb; p.ngroups = mats[i]->ngroups; p.rows_log2 = mats[i]->rows_log2;
-        p.x = xq; p.ntokens = ntokens; p.ksplit = ksplit;
+        p.x = xq; p.ntokens = ntokens; p.ksplit = ksplit; p.split_f16 = split_f16;
         for (int j = i; j < nmat; ++j) {
             // (one launch: 64-row tiles of the same width, and of the same format unless both are K-quants)
             const auto kquant = [](int t) { return t == T_Q4_K || t == T_Q5_K || t == T_Q6_K; };
@@ -603,8 +604,11 @@ int gemm_chunk_call(slai_ctx *ctx, int nmat, const slai_qmat *const *mats, float
 // The layer loop for a chunk of up to 32 tokens with every projection on the matrix cores (kernels_gemm_chunk.hip):
 // RMSNorm of all rows, q/k/v, bias + RoPE + cache write, attention, output projection into the residual, RMSNorm,
 // gate and up, SiLU, down projection into the residual (transformer.rs:316-381 per token).
-int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev) {
+// split_f16: the GEMMs on the half-precision matrix cores, their inputs written as f16 heads and remainders by the kernels
+// before them (which set *ctx->split_flag when a value does not fit: the caller then repeats the pass without).
+int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev, bool split_f16) {
     PromptChunkState &pc = chunk;
+    int *const sf = split_f16 ? ctx->split_flag : nullptr;
     if (n == 0 || n > 32 || n > pc.rows || pos0 + n > config.seq_len) return set_error(ctx, SLAI_E_ARG, "prompt chunk out of range");
     const uint32_t dim = config.dim, kvd = kv_dim(), hid = config.hidden_dim;
     float *x = (float *)pc.x.buf->dptr, *xn = (float *)pc.xn.buf->dptr, *q = (float *)pc.q.buf->dptr;
@@ -615,36 +619,37 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
     // q/k/v and gate/up are cut into column ranges when every matrix involved has 64-row tiles (chunk_ksplit).
     for (uint32_t l = 0; l < config.n_layers; ++l) {
         const Llama2LayerWeights &wl = weights.layers[l];
-        SLAI_HIP_TRY(ctx, launch_rms_norm_quads(ctx->stream, xn, x, (const float *)wl.attn_norm.buf->dptr, dim, n, dim, config.rms_norm_eps));
+        SLAI_HIP_TRY(ctx, launch_rms_norm_quads(ctx->stream, xn, x, (const float *)wl.attn_norm.buf->dptr, dim, n, dim, config.rms_norm_eps, sf));
         {
             const slai_qmat *mats[3] = {wl.attn_v, wl.attn_k, wl.attn_q};
             float *outs[3] = {v, k, q};
             const uint32_t strides[3] = {kvd, kvd, dim};
             const uint32_t ks = chunk_ksplit(3, mats);
-            TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)", ks));
+            TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)", ks, split_f16));
             TRY(chunk_attention(l, pos0, n, ks, true));       // straight into xn, quad-major
+            if (sf) SLAI_HIP_TRY(ctx, launch_quads_split(ctx->stream, xn, dim, n, sf));
         }
         {
             const slai_qmat *mats[1] = {wl.attn_output};
             float *outs[1] = {x};
             const uint32_t strides[1] = {dim};
-            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, xn, n, "llama2 attn_output (prompt chunk)"));
+            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, xn, n, "llama2 attn_output (prompt chunk)", 1, split_f16));
         }
-        SLAI_HIP_TRY(ctx, launch_rms_norm_quads(ctx->stream, xn, x, (const float *)wl.ffn_norm.buf->dptr, dim, n, dim, config.rms_norm_eps));
+        SLAI_HIP_TRY(ctx, launch_rms_norm_quads(ctx->stream, xn, x, (const float *)wl.ffn_norm.buf->dptr, dim, n, dim, config.rms_norm_eps, sf));
         {
             const slai_qmat *mats[2] = {wl.ffn_gate, wl.ffn_up};
             float *outs[2] = {hb, hb2};
             const uint32_t strides[2] = {hid, hid};
             const uint32_t ks = chunk_ksplit(2, mats);
-            TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, GEMM_OUT_QUADS, xn, n, "llama2 ffn gate/up (prompt chunk)", ks));
-            // element-wise, so the layout does not matter (slots of tokens past the chunk hold stale values nobody reads)
-            SLAI_HIP_TRY(ctx, launch_silu_parts(ctx->stream, hb, hb2, 32 * hid, ks, 32 * hid));
+            TRY(gemm_chunk_call(ctx, 2, mats, outs, strides, GEMM_OUT_QUADS, xn, n, "llama2 ffn gate/up (prompt chunk)", ks, split_f16));
+            // element-wise over the token slots in use (those past the chunk hold stale values)
+            SLAI_HIP_TRY(ctx, launch_silu_parts(ctx->stream, hb, hb2, 32 * hid, ks, 32 * hid, sf, n));
         }
         {
             const slai_qmat *mats[1] = {wl.ffn_down};
             float *outs[1] = {x};
             const uint32_t strides[1] = {dim};
-            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, hb, n, "llama2 ffn_down (prompt chunk)"));
+            TRY(gemm_chunk_call(ctx, 1, mats, outs, strides, GEMV_ACCUM, hb, n, "llama2 ffn_down (prompt chunk)", 1, split_f16));
         }
     }
     return SLAI_OK;
@@ -830,16 +835,30 @@ SLAI_EXPORT int slai_llama2_prefill(slai_llama2 *m, const int32_t *tokens, uint3
     TRY(slai_write_buffer(ctx, m->chunk.tokens, 0, tokens, (size_t)n_tokens * 4));
     const int *tokens_dev = (const int *)m->chunk.tokens->dptr;
     SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev0, ctx->stream));
-    for (uint32_t i = 0; i < n_tokens; i += chunk) {
-        const uint32_t n = std::min(chunk, n_tokens - i);
-        if (gemm) TRY(m->enqueue_chunk_gemm(start_pos + i, n, tokens_dev + i));
-        else TRY(m->enqueue_chunk(start_pos + i, n, tokens_dev + i));
+    // The matrix-core pass runs on the half-precision units with split activations; if one of them turns out to be
+    // beyond the f16 range the whole pass is repeated in fp32 (it only writes the caches, so that is safe).
+    bool split = gemm && ctx->prompt_split_f16 != 0 && ctx->split_flag;
+    for (;;) {
+        if (split) SLAI_HIP_TRY(ctx, hipMemsetAsync(ctx->split_flag, 0, sizeof(int), ctx->stream));
+        for (uint32_t i = 0; i < n_tokens; i += chunk) {
+            const uint32_t n = std::min(chunk, n_tokens - i);
+            if (gemm) TRY(m->enqueue_chunk_gemm(start_pos + i, n, tokens_dev + i, split));
+            else TRY(m->enqueue_chunk(start_pos + i, n, tokens_dev + i));
+        }
+        SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev1, ctx->stream));
+        TRY(slai_synchronize(ctx));
+        if (!split) break;
+        int beyond = 0;
+        SLAI_HIP_TRY(ctx, hipMemcpy(&beyond, ctx->split_flag, sizeof(int), hipMemcpyDeviceToHost));
+        if (!beyond) break;
+        ++m->prefill_fp32_repeats;
+        split = false;
     }
-    SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev1, ctx->stream));
-    TRY(slai_synchronize(ctx));
     if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, m->loop.ev0, m->loop.ev1));
     return SLAI_OK;
 }
+
+SLAI_EXPORT uint32_t slai_llama2_prefill_fp32_repeats(const slai_llama2 *m) { return m ? m->prefill_fp32_repeats : 0; }
 
 SLAI_EXPORT int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache) {
     if (!m || layer >= m->config.n_layers) return SLAI_E_ARG;

@@ -61,6 +61,10 @@ template <> struct Deq<T_Q4_K> {
             m1[sb] = dmin * ub(sb < 4 ? m_lo : m_hi, sb & 3);
         }
     }
+    __device__ __forceinline__ void scale(float s) {
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) { d1[sb] *= s; m1[sb] *= s; }
+    }
     template <int K, int W> __device__ __forceinline__ void quad(const typename F::Data &d, float (&lo)[4], float (&hi)[4]) const {
         constexpr int J = K / 2;                                 // low nibbles: sub-block 2J, high nibbles: sub-block 2J + 1
         const uint32_t q = word(d.p[1 + K], W);
@@ -84,6 +88,10 @@ template <> struct Deq<T_Q5_K> {
             m1[sb] = dmin * ub(sb < 4 ? m_lo : m_hi, sb & 3);
         }
     }
+    __device__ __forceinline__ void scale(float s) {
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) { d1[sb] *= s; m1[sb] *= s; }
+    }
     template <int K, int W> __device__ __forceinline__ void quad(const typename F::Data &d, float (&lo)[4], float (&hi)[4]) const {
         constexpr int J = K / 2, H = K % 2;
         const uint32_t q = word(d.p[3 + K], W), qb = word(d.p[1 + H], W);
@@ -105,6 +113,10 @@ template <> struct Deq<T_Q6_K> {
             for (int M = 0; M < 2; ++M)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) ds[8 * I + 2 * r + M] = dd * F::scale_of(d, I, M, r);
+    }
+    __device__ __forceinline__ void scale(float s) {
+#pragma unroll
+        for (int c = 0; c < 16; ++c) ds[c] *= s;
     }
     template <int K, int W> __device__ __forceinline__ void quad(const typename F::Data &d, float (&lo)[4], float (&hi)[4]) const {
         constexpr int I = K / 4, M = (K / 2) % 2, P = K % 2;
@@ -130,6 +142,10 @@ template <> struct Deq<T_Q8_0> {          // BlockQ8_0, quantization.rs:29-42: v
 #pragma unroll
         for (int B = 0; B < 8; ++B) { sc[B] = F::scale_of(d, B); off[B] = -128.0f * sc[B]; }
     }
+    __device__ __forceinline__ void scale(float s) {
+#pragma unroll
+        for (int B = 0; B < 8; ++B) { sc[B] *= s; off[B] *= s; }
+    }
     template <int K, int W> __device__ __forceinline__ void quad(const typename F::Data &d, float (&lo)[4], float (&hi)[4]) const {
         // int8 -> unsigned through ^0x80 (one byte conversion instruction), the 128 taken off again with the scale
         const uint32_t qa = word(d.p[2 * K], W) ^ 0x80808080u, qb = word(d.p[2 * K + 1], W) ^ 0x80808080u;
@@ -144,6 +160,10 @@ template <> struct Deq<T_Q4_0> {          // BlockQ4_0, quantization.rs:47-69: v
     __device__ __forceinline__ void head(const typename F::Data &d, uint16_t) {
 #pragma unroll
         for (int B = 0; B < 8; ++B) { sc[B] = F::scale_of(d, B); off[B] = -8.0f * sc[B]; }
+    }
+    __device__ __forceinline__ void scale(float s) {
+#pragma unroll
+        for (int B = 0; B < 8; ++B) { sc[B] *= s; off[B] *= s; }
     }
     template <int K, int W> __device__ __forceinline__ void quad(const typename F::Data &d, float (&lo)[4], float (&hi)[4]) const {
         const uint32_t q = word(d.p[K], W);
@@ -270,8 +290,120 @@ __device__ __forceinline__ void gemm64_body(const GemmChunkParams &p, const Gemm
     }
 }
 
+// ---- 64-row tiles on the half-precision matrix cores ---------------------------------------------------------------------
+// The f16 matrix rate is sixteen times the fp32 one.  Every dequantised weight w (scaled by 2^8, so that the remainder
+// stays a normal f16 number) and every activation x is split into an f16 head and an f16 remainder, w = wh + wl,
+// x = xh + xl, each pair keeping about 22 bits; wh*xh + wh*xl + wl*xh is accumulated in fp32 by three
+// v_mfma_f32_32x32x16_f16 (the dropped wl*xl is below 2^-22 of the product).  Valid while |x| < 65504 and |w| < 255.
+// The activations arrive split (split_quad in the kernels that write them, which also report values beyond the range).
+// An instruction takes 32 rows x 16 columns: lanes 0-31 hold eight columns of chunk c1 for rows (A) / tokens (B) 0-31,
+// lanes 32-63 eight columns of chunk c2.  The lane = row registers of the tile become the A operands of its two row
+// halves through v_permlane32_swap: [c1 of rows 0-63], [c2 of rows 0-63] -> [c1 | c2 of rows 0-31], [c1 | c2 of rows 32-63].
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t H8 __attribute__((ext_vector_type(4)));       // eight f16
+
+__device__ __forceinline__ void split8(const float (&a)[4], const float (&b)[4], H8 &h, H8 &l) {
+    uint32_t h0, h1, h2, h3, l0, l1, l2, l3;
+    split_pair_f16(a[0], a[1], h0, l0); split_pair_f16(a[2], a[3], h1, l1);
+    split_pair_f16(b[0], b[1], h2, l2); split_pair_f16(b[2], b[3], h3, l3);
+    h = H8{h0, h1, h2, h3}; l = H8{l0, l1, l2, l3};
+}
+// the activations arrive split (split_quad): heads and remainders of two quads as B operands
+__device__ __forceinline__ void split_x(const H8 a, const H8 b, H8 &h, H8 &l) {
+    h = __builtin_shufflevector(a, b, 0, 1, 4, 5);
+    l = __builtin_shufflevector(a, b, 2, 3, 6, 7);
+}
+// a = [a of lanes 0-31 | b of lanes 0-31], b = [a of lanes 32-63 | b of lanes 32-63]
+__device__ __forceinline__ void swap_halves(H8 &a, H8 &b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const auto r = __builtin_amdgcn_permlane32_swap(a[i], b[i], false, false);
+        a[i] = r[0]; b[i] = r[1];
+    }
+}
+__device__ __forceinline__ f32x16 mfma_h(const H8 &a, const H8 &b, f32x16 acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
+}
+
+struct X64H { H8 a[4]; };                                  // the lane's token: its half's chunk of a stage, four columns per entry
+
+// xl: the lane's token in the first quad of the super-block, moved on to chunk c2 for lanes 32-63
+template <int T, int K> __device__ __forceinline__ void request_x64h(const H8 *xl, X64H &x) {
+#pragma unroll
+    for (int W = 0; W < 4; ++W) x.a[W] = xl[(4 * Tiled<T>::c1(K) + W) * 32];
+}
+
+template <int T, int K, int WP> __device__ __forceinline__ void mac64h(const Deq<T> &q, const typename Tiled<T>::Data &d, const X64H &x, f32x16 &top, f32x16 &bot) {
+    float lo0[4], hi0[4], lo1[4], hi1[4];
+    q.template quad<K, WP>(d, lo0, hi0);
+    q.template quad<K, WP + 1>(d, lo1, hi1);
+    H8 ah, al, bh, bl;                                         // a: chunk c1, b: chunk c2, columns 4WP .. 4WP + 7, all 64 rows
+    split8(lo0, lo1, ah, al);
+    split8(hi0, hi1, bh, bl);
+    swap_halves(ah, bh);                                       // ah: rows 0-31, bh: rows 32-63
+    swap_halves(al, bl);
+    H8 xh, xl;
+    split_x(x.a[WP], x.a[WP + 1], xh, xl);
+    top = mfma_h(ah, xh, top); bot = mfma_h(bh, xh, bot);
+    top = mfma_h(ah, xl, top); bot = mfma_h(bh, xl, bot);
+    top = mfma_h(al, xh, top); bot = mfma_h(bl, xh, bot);
+}
+
+template <int T, int K> __device__ __forceinline__ void stages64h(const Deq<T> &q, const typename Tiled<T>::Data &d, const H8 *xl, X64H &x, f32x16 &top, f32x16 &bot) {
+    X64H nx = x;
+    if constexpr (K < 7) request_x64h<T, K + 1>(xl, nx);
+    mac64h<T, K, 0>(q, d, x, top, bot);
+    mac64h<T, K, 2>(q, d, x, top, bot);
+    x = nx;
+    if constexpr (K < 7) stages64h<T, K + 1>(q, d, xl, x, top, bot);
+}
+
+template <int T>
+__device__ __forceinline__ void gemm64h_body(const GemmChunkParams &p, const GemmChunkSeg &seg, uint32_t tile, float *part) {
+    using F = Tiled<T>;
+    constexpr int D = F::c2(0) - F::c1(0);                     // chunk c2 of a stage is D chunks after c1
+    static_assert(F::c2(3) - F::c1(3) == D && F::c2(7) - F::c1(7) == D, "c2 - c1 must not depend on the stage");
+    const int tid = threadIdx.x, lane = tid & 63, NW = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
+    const uint32_t token = min((uint32_t)(lane & 31), p.ntokens - 1);            // lanes past the chunk repeat its last token
+    const H8 *xrow = (const H8 *)p.x + token + (lane >> 5) * (4 * D * 32);
+    f32x16 top, bot;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { top[i] = 0.0f; bot[i] = 0.0f; }
+    const uint32_t per = (p.ncb + p.ksplit - 1) / p.ksplit, cb0 = blockIdx.y * per, cb1 = min(p.ncb, cb0 + per);
+    for (uint32_t cb = cb0 + wave; cb < cb1; cb += NW) {
+        typename F::Data d;
+        uint16_t dt = 0;
+        X64H x;
+        load_unit<T>(seg.W + ((size_t)tile * p.ncb + cb) * unit_bytes, lane, d, dt);
+        request_x64h<T, 0>(xrow + (size_t)cb * 2048, x);
+        Deq<T> q;
+        q.head(d, dt);
+        q.scale(256.0f);
+        stages64h<T, 0>(q, d, xrow + (size_t)cb * 2048, x, top, bot);
+    }
+    float *mine = part + (size_t)wave * 32 * G64_LDS_ROW + (size_t)(lane & 31) * G64_LDS_ROW + 4 * (lane >> 5);
+    const float back = 1.0f / 256.0f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        *(float4 *)(mine + 8 * g) = make_float4(top[4 * g] * back, top[4 * g + 1] * back, top[4 * g + 2] * back, top[4 * g + 3] * back);
+        *(float4 *)(mine + 32 + 8 * g) = make_float4(bot[4 * g] * back, bot[4 * g + 1] * back, bot[4 * g + 2] * back, bot[4 * g + 3] * back);
+    }
+    lds_barrier();
+    const bool quads = (seg.flags & GEMM_OUT_QUADS) != 0;
+    float *out = seg.out + (size_t)blockIdx.y * seg.part_stride;
+    const bool vec_ok = quads || (seg.out_stride % 4 == 0 && ((uintptr_t)out & 15) == 0);
+    for (uint32_t idx = tid; idx < 512; idx += blockDim.x) {
+        const uint32_t t = quads ? idx & 31u : idx >> 4, rq = quads ? idx >> 5 : idx & 15u;
+        const uint32_t row = tile * 64 + 4 * rq;
+        if (t >= p.ntokens || row >= seg.nrows) continue;
+        reduce_store4(seg, out, part + (size_t)t * G64_LDS_ROW + 4 * rq, NW, 32 * G64_LDS_ROW, row, t, quads, vec_ok);
+    }
+}
+
 // grid = (tiles of all segments, ksplit), block = 64 * (waves: each takes every NW-th super-block)
-template <int TT, int MAXT>
+template <int TT, int MAXT, bool H = false>
 __global__ void __launch_bounds__(MAXT) gemm64_kernel(const GemmChunkParams p) {
     extern __shared__ float part[];                            // [waves][32 tokens][G64_LDS_ROW]
     touch_kernel_arguments<sizeof(GemmChunkParams)>();
@@ -288,7 +420,18 @@ __global__ void __launch_bounds__(MAXT) gemm64_kernel(const GemmChunkParams p) {
     seg.part_stride = s == 0 ? p.seg[0].part_stride : (s == 1 ? p.seg[1].part_stride : p.seg[2].part_stride);
     seg.bias = s == 0 ? p.seg[0].bias : (s == 1 ? p.seg[1].bias : p.seg[2].bias);
     seg.flags = s == 0 ? p.seg[0].flags : (s == 1 ? p.seg[1].flags : p.seg[2].flags);
-    if constexpr (TT != 0) {
+    if constexpr (H) {
+        if constexpr (TT != 0) {
+            gemm64h_body<TT>(p, seg, tile, part);
+        } else {
+            switch (seg.type) {                                // uniform over the workgroup
+            case T_Q4_K: gemm64h_body<T_Q4_K>(p, seg, tile, part); break;
+            case T_Q6_K: gemm64h_body<T_Q6_K>(p, seg, tile, part); break;
+            case T_Q5_K: gemm64h_body<T_Q5_K>(p, seg, tile, part); break;
+            default: break;
+            }
+        }
+    } else if constexpr (TT != 0) {
         gemm64_body<TT>(p, seg, tile, part);
     } else {
         switch (seg.type) {                                    // uniform over the workgroup
@@ -335,10 +478,41 @@ template <int T, int K, int W, int NACC> __device__ __forceinline__ void steps16
     if constexpr (NK < 8) steps16<T, NK, NW, NACC>(q, d, xt, x, acc);
 }
 
+// The same steps on the half-precision matrix cores (see the 64-row form): lane = 16 * kq + row is the A layout of
+// v_mfma_f32_16x16x32_f16 as it stands, k group kq = the lane's super-block, eight columns (four of chunk c1, four of c2)
+// per instruction, which adds up the four super-blocks itself.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+template <int NACC> struct X16H { H8 a[NACC], b[NACC]; };      // the split forms of four columns of chunk c1 (a) and c2 (b) per token
+template <int T, int K, int W, int NACC> __device__ __forceinline__ void request_x16h(const H8 *const (&xt)[NACC], X16H<NACC> &x) {
+    using F = Tiled<T>;
+#pragma unroll
+    for (int n = 0; n < NACC; ++n) { x.a[n] = xt[n][(4 * F::c1(K) + W) * 32]; x.b[n] = xt[n][(4 * F::c2(K) + W) * 32]; }
+}
+template <int T, int K, int W, int NACC> __device__ __forceinline__ void steps16h(const Deq<T> &q, const typename Tiled<T>::Data &d, const H8 *const (&xt)[NACC],
+                                                                                  X16H<NACC> &x, f32x4 (&acc)[NACC]) {
+    constexpr int NK = W == 3 ? K + 1 : K, NW = W == 3 ? 0 : W + 1;
+    X16H<NACC> nx = x;
+    if constexpr (NK < 8) request_x16h<T, NK, NW, NACC>(xt, nx);
+    float lo[4], hi[4];
+    q.template quad<K, W>(d, lo, hi);
+    H8 ah, al;
+    split8(lo, hi, ah, al);
+#pragma unroll
+    for (int n = 0; n < NACC; ++n) {
+        H8 xh, xl;
+        split_x(x.a[n], x.b[n], xh, xl);
+        acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, ah), __builtin_bit_cast(f16x8, xh), acc[n], 0, 0, 0);
+        acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, ah), __builtin_bit_cast(f16x8, xl), acc[n], 0, 0, 0);
+        acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, al), __builtin_bit_cast(f16x8, xh), acc[n], 0, 0, 0);
+    }
+    x = nx;
+    if constexpr (NK < 8) steps16h<T, NK, NW, NACC>(q, d, xt, x, acc);
+}
+
 constexpr int G16_LDS_ROW = 20;                                // floats per token in the LDS partials (16 rows + padding)
 
 // grid = (tiles, 2 / NACC), block = 64 * ngroups (one wave per column group of four super-blocks)
-template <int T, int MAXT, int NACC>
+template <int T, int MAXT, int NACC, bool H = false>
 __global__ void __launch_bounds__(MAXT) gemm16_kernel(const GemmChunkParams p) {
     using F = Tiled<T>;
     extern __shared__ float part[];                            // [waves][16 * NACC tokens][G16_LDS_ROW]
@@ -356,25 +530,44 @@ __global__ void __launch_bounds__(MAXT) gemm16_kernel(const GemmChunkParams p) {
     typename F::Data d;
     uint16_t dt = 0;
     load_unit<T>(p.seg[0].W + ((size_t)tile * p.ngroups + g) * unit_bytes, lane, d, dt);
-    X16<NACC> x;
-    request_x16<T, 0, 0, NACC>(xt, x);
-    f32x16 acc[NACC];
-#pragma unroll
-    for (int n = 0; n < NACC; ++n)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[n][i] = 0.0f;
-    Deq<T> q;
-    q.head(d, dt);
-    steps16<T, 0, 0, NACC>(q, d, xt, x, acc);
-    // the four blocks hold the same rows and tokens over different super-blocks: add them.  Register v of a block holds
-    // row 4 * (lane / 16) + v of token lane % 16.
+    // Register v of a block (of the one block of the f16 form) holds row 4 * (lane / 16) + v of token lane % 16.
     float *mine = part + (size_t)wave * 16 * NACC * G16_LDS_ROW + 4 * (lane >> 4);
+    if constexpr (H) {
+        const H8 *xh[NACC];
 #pragma unroll
-    for (int n = 0; n < NACC; ++n) {
-        float4 sm;
-        sm.x = (acc[n][0] + acc[n][4]) + (acc[n][8] + acc[n][12]); sm.y = (acc[n][1] + acc[n][5]) + (acc[n][9] + acc[n][13]);
-        sm.z = (acc[n][2] + acc[n][6]) + (acc[n][10] + acc[n][14]); sm.w = (acc[n][3] + acc[n][7]) + (acc[n][11] + acc[n][15]);
-        *(float4 *)(mine + (size_t)(16 * n + (lane & 15)) * G16_LDS_ROW) = sm;
+        for (int n = 0; n < NACC; ++n) xh[n] = (const H8 *)xt[n];
+        X16H<NACC> x;
+        request_x16h<T, 0, 0, NACC>(xh, x);
+        Deq<T> q;
+        q.head(d, dt);
+        f32x4 acc[NACC];
+#pragma unroll
+        for (int n = 0; n < NACC; ++n) acc[n] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        q.scale(256.0f);
+        steps16h<T, 0, 0, NACC>(q, d, xh, x, acc);
+        const float back = 1.0f / 256.0f;
+#pragma unroll
+        for (int n = 0; n < NACC; ++n)
+            *(float4 *)(mine + (size_t)(16 * n + (lane & 15)) * G16_LDS_ROW) = make_float4(acc[n][0] * back, acc[n][1] * back, acc[n][2] * back, acc[n][3] * back);
+    } else {
+        X16<NACC> x;
+        request_x16<T, 0, 0, NACC>(xt, x);
+        Deq<T> q;
+        q.head(d, dt);
+        f32x16 acc[NACC];
+#pragma unroll
+        for (int n = 0; n < NACC; ++n)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[n][i] = 0.0f;
+        steps16<T, 0, 0, NACC>(q, d, xt, x, acc);
+        // the four blocks hold the same rows and tokens over different super-blocks: add them
+#pragma unroll
+        for (int n = 0; n < NACC; ++n) {
+            float4 sm;
+            sm.x = (acc[n][0] + acc[n][4]) + (acc[n][8] + acc[n][12]); sm.y = (acc[n][1] + acc[n][5]) + (acc[n][9] + acc[n][13]);
+            sm.z = (acc[n][2] + acc[n][6]) + (acc[n][10] + acc[n][14]); sm.w = (acc[n][3] + acc[n][7]) + (acc[n][11] + acc[n][15]);
+            *(float4 *)(mine + (size_t)(16 * n + (lane & 15)) * G16_LDS_ROW) = sm;
+        }
     }
     lds_barrier();
     const GemmChunkSeg &seg = p.seg[0];
@@ -392,7 +585,30 @@ __global__ void __launch_bounds__(MAXT) gemm16_kernel(const GemmChunkParams p) {
 constexpr int G32_LDS_ROW = 36;                                // floats per token in the LDS partials (32 rows + padding)
 
 // grid = tiles, block = 64 * (column groups of this launch): one wave per group of two super-blocks, lane = 32 * kq + row
-template <int T, int MAXT>
+// f16 form: lane = 32 * kq + row is the A layout of v_mfma_f32_32x32x16_f16, k group kq = the lane's super-block
+struct X32H { H8 a[4], b[4]; };
+template <int T, int K> __device__ __forceinline__ void request_x32h(const H8 *xcb, X32H &x) {
+    using F = Tiled<T>;
+#pragma unroll
+    for (int W = 0; W < 4; ++W) { x.a[W] = xcb[(4 * F::c1(K) + W) * 32]; x.b[W] = xcb[(4 * F::c2(K) + W) * 32]; }
+}
+template <int T, int K, int W> __device__ __forceinline__ void mac32h(const Deq<T> &q, const typename Tiled<T>::Data &d, const X32H &x, f32x16 &acc) {
+    float lo[4], hi[4];
+    q.template quad<K, W>(d, lo, hi);
+    H8 ah, al, xh, xl;
+    split8(lo, hi, ah, al);
+    split_x(x.a[W], x.b[W], xh, xl);
+    acc = mfma_h(ah, xh, acc); acc = mfma_h(ah, xl, acc); acc = mfma_h(al, xh, acc);
+}
+template <int T, int K> __device__ __forceinline__ void stages32h(const Deq<T> &q, const typename Tiled<T>::Data &d, const H8 *xcb, X32H &x, f32x16 &acc) {
+    X32H nx = x;
+    if constexpr (K < 7) request_x32h<T, K + 1>(xcb, nx);
+    mac32h<T, K, 0>(q, d, x, acc); mac32h<T, K, 1>(q, d, x, acc); mac32h<T, K, 2>(q, d, x, acc); mac32h<T, K, 3>(q, d, x, acc);
+    x = nx;
+    if constexpr (K < 7) stages32h<T, K + 1>(q, d, xcb, x, acc);
+}
+
+template <int T, int MAXT, bool H = false>
 __global__ void __launch_bounds__(MAXT) gemm32_kernel(const GemmChunkParams p) {
     using F = Tiled<T>;
     extern __shared__ float part[];                            // [waves][32 tokens][G32_LDS_ROW]
@@ -407,21 +623,37 @@ __global__ void __launch_bounds__(MAXT) gemm32_kernel(const GemmChunkParams p) {
     typename F::Data d;
     uint16_t dt = 0;
     load_unit<T>(p.seg[0].W + ((size_t)tile * p.ngroups + g) * unit_bytes, lane, d, dt);
-    X64 x;
-    request_x64<T, 0>(xcb, x);
-    f32x32 acc;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) acc[i] = 0.0f;
-    Deq<T> q;
-    q.head(d, dt);
-    stages64<T, 0>(q, d, xcb, x, acc);
-    // the two blocks hold the same rows and tokens over different super-blocks: add them.  Register v of a block holds row
-    // 8 * (v / 4) + 4 * (lane / 32) + v % 4 of token lane % 32.
+    // Register v of a block (of the one block of the f16 form) holds row 8 * (v / 4) + 4 * (lane / 32) + v % 4 of token lane % 32.
     float *mine = part + (size_t)wave * 32 * G32_LDS_ROW + (size_t)(lane & 31) * G32_LDS_ROW + 4 * (lane >> 5);
+    if constexpr (H) {
+        X32H x;
+        request_x32h<T, 0>((const H8 *)xcb, x);
+        Deq<T> q;
+        q.head(d, dt);
+        f32x16 acc;
 #pragma unroll
-    for (int g4 = 0; g4 < 4; ++g4)
-        *(float4 *)(mine + 8 * g4) = make_float4(acc[4 * g4] + acc[16 + 4 * g4], acc[4 * g4 + 1] + acc[16 + 4 * g4 + 1],
-                                                 acc[4 * g4 + 2] + acc[16 + 4 * g4 + 2], acc[4 * g4 + 3] + acc[16 + 4 * g4 + 3]);
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+        q.scale(256.0f);
+        stages32h<T, 0>(q, d, (const H8 *)xcb, x, acc);
+        const float back = 1.0f / 256.0f;
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4)
+            *(float4 *)(mine + 8 * g4) = make_float4(acc[4 * g4] * back, acc[4 * g4 + 1] * back, acc[4 * g4 + 2] * back, acc[4 * g4 + 3] * back);
+    } else {
+        X64 x;
+        request_x64<T, 0>(xcb, x);
+        Deq<T> q;
+        q.head(d, dt);
+        f32x32 acc;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) acc[i] = 0.0f;
+        stages64<T, 0>(q, d, xcb, x, acc);
+        // the two blocks hold the same rows and tokens over different super-blocks: add them
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4)
+            *(float4 *)(mine + 8 * g4) = make_float4(acc[4 * g4] + acc[16 + 4 * g4], acc[4 * g4 + 1] + acc[16 + 4 * g4 + 1],
+                                                     acc[4 * g4 + 2] + acc[16 + 4 * g4 + 2], acc[4 * g4 + 3] + acc[16 + 4 * g4 + 3]);
+    }
     lds_barrier();
     const GemmChunkSeg &seg = p.seg[0];
     const bool quads = (seg.flags & GEMM_OUT_QUADS) != 0;
@@ -436,7 +668,7 @@ __global__ void __launch_bounds__(MAXT) gemm32_kernel(const GemmChunkParams p) {
 
 // RMSNorm of token t = blockIdx.x (rms_norm.slang:48-67: (x * 1/sqrt(mean(x^2) + eps)) * w), written quad-major for the
 // GEMM kernels above.  n % 4 == 0, n <= 16384 (16 float4 per thread).
-__global__ void __launch_bounds__(256) rms_norm_quads_kernel(float4 *out, const float *x, const float *w, uint32_t n, uint32_t x_stride, float eps) {
+__global__ void __launch_bounds__(256) rms_norm_quads_kernel(float4 *out, const float *x, const float *w, uint32_t n, uint32_t x_stride, float eps, int *split_flag) {
     __shared__ float red[4];
     const uint32_t t = blockIdx.x, nq = n / 4;
     const float4 *xr = (const float4 *)(x + (size_t)t * x_stride), *wr = (const float4 *)w;
@@ -458,7 +690,15 @@ __global__ void __launch_bounds__(256) rms_norm_quads_kernel(float4 *out, const 
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
         const uint32_t i = threadIdx.x + 256u * j;
-        if (i < nq) out[(size_t)i * 32 + t] = make_float4((v[j].x * scale) * g[j].x, (v[j].y * scale) * g[j].y, (v[j].z * scale) * g[j].z, (v[j].w * scale) * g[j].w);
+        if (i < nq) {
+            const float4 r = make_float4((v[j].x * scale) * g[j].x, (v[j].y * scale) * g[j].y, (v[j].z * scale) * g[j].z, (v[j].w * scale) * g[j].w);
+            if (split_flag) {                                  // (uniform) f16 heads and remainders; values beyond f16 are reported
+                if (split_overflows(r)) *split_flag = 1;                // 1: a normalised row
+                out[(size_t)i * 32 + t] = split_quad(r);
+            } else {
+                out[(size_t)i * 32 + t] = r;
+            }
+        }
     }
 }
 
@@ -507,9 +747,23 @@ __global__ void __launch_bounds__(256) layernorm_quads_kernel(float4 *out, const
 }
 
 // row-major [tokens][n] -> quad-major; thread = (quad, token), token fastest so that the stores are contiguous
-__global__ void rows_to_quads_kernel(float4 *out, const float *x, uint32_t n, uint32_t x_stride, uint32_t ntokens) {
+__global__ void rows_to_quads_kernel(float4 *out, const float *x, uint32_t n, uint32_t x_stride, uint32_t ntokens, int *split_flag) {
     const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x, t = idx & 31u, qd = idx >> 5;
-    if (qd < n / 4 && t < ntokens) out[(size_t)qd * 32 + t] = *(const float4 *)(x + (size_t)t * x_stride + 4 * qd);
+    if (qd < n / 4 && t < ntokens) {
+        const float4 r = *(const float4 *)(x + (size_t)t * x_stride + 4 * qd);
+        if (split_flag && split_overflows(r)) *split_flag = 1;
+        out[(size_t)qd * 32 + t] = split_flag ? split_quad(r) : r;
+    }
+}
+
+// quad-major f32 -> the split form, in place (both are 16 bytes per quad and token)
+__global__ void quads_split_kernel(float4 *x, uint32_t nquads, uint32_t ntokens, int *split_flag) {
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x, t = idx & 31u, qd = idx >> 5;
+    if (qd < nquads && t < ntokens) {
+        const float4 r = x[idx];
+        if (split_overflows(r)) *split_flag = 2;                        // 2: converted in place
+        x[idx] = split_quad(r);
+    }
 }
 
 }  // namespace
@@ -519,9 +773,9 @@ bool gemm_chunk_supports(const slai_qmat *m) {
     return m->rows_log2 >= 4 && m->rows_log2 <= 6 && m->ngroups <= 64;
 }
 
-hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps) {
+hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps, int *split_flag) {
     if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || n > 16384 || x_stride % 4) return hipErrorInvalidValue;
-    rms_norm_quads_kernel<<<ntokens, 256, 0, s>>>((float4 *)out, x, w, n, x_stride, eps);
+    rms_norm_quads_kernel<<<ntokens, 256, 0, s>>>((float4 *)out, x, w, n, x_stride, eps, split_flag);
     return hipGetLastError();
 }
 
@@ -531,9 +785,15 @@ hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, con
     return hipGetLastError();
 }
 
-hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride) {
+hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride, int *split_flag) {
     if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || x_stride % 4) return hipErrorInvalidValue;
-    rows_to_quads_kernel<<<(n / 4 * 32 + 255) / 256, 256, 0, s>>>((float4 *)out, x, n, x_stride, ntokens);
+    rows_to_quads_kernel<<<(n / 4 * 32 + 255) / 256, 256, 0, s>>>((float4 *)out, x, n, x_stride, ntokens, split_flag);
+    return hipGetLastError();
+}
+
+hipError_t launch_quads_split(hipStream_t s, float *x, uint32_t n, uint32_t ntokens, int *split_flag) {
+    if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || !split_flag) return hipErrorInvalidValue;
+    quads_split_kernel<<<(n / 4 * 32 + 255) / 256, 256, 0, s>>>((float4 *)x, n / 4, ntokens, split_flag);
     return hipGetLastError();
 }
 
@@ -568,6 +828,24 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
         const size_t smem = (size_t)nw * 32 * G64_LDS_ROW * sizeof(float);
         const int NT = (int)nw * 64;
         const dim3 grid(tiles, p.ksplit);
+        if (p.split_f16) {
+            // (up to eight waves: the bound that leaves 256 registers, which the mixed-format kernel needs not to spill)
+#define SLAI_G64H(TY)                                                                      \
+    do {                                                                                   \
+        if (NT <= 512) gemm64_kernel<TY, 512, true><<<grid, NT, smem, st>>>(p);            \
+        else gemm64_kernel<TY, 1024, true><<<grid, NT, smem, st>>>(p);                     \
+    } while (0)
+            switch (tt) {
+            case T_Q4_K: SLAI_G64H(T_Q4_K); break;
+            case T_Q5_K: SLAI_G64H(T_Q5_K); break;
+            case T_Q6_K: SLAI_G64H(T_Q6_K); break;
+            case T_Q4_0: SLAI_G64H(T_Q4_0); break;
+            case T_Q8_0: gemm64_kernel<T_Q8_0, 512, true><<<grid, NT, smem, st>>>(p); break;
+            default: SLAI_G64H(0); break;
+            }
+#undef SLAI_G64H
+            return hipGetLastError();
+        }
         switch (tt) {
         case T_Q4_K: gemm64_kernel<T_Q4_K, 1024><<<grid, NT, smem, st>>>(p); break;
         case T_Q5_K: gemm64_kernel<T_Q5_K, 1024><<<grid, NT, smem, st>>>(p); break;
@@ -592,11 +870,15 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
         const int NT = (int)ng * 64;
         if (p.rows_log2 == 5) {
             const size_t smem = (size_t)ng * 32 * G32_LDS_ROW * sizeof(float);
+#define SLAI_G32H(TY, HH)                                                                  \
+    do {                                                                                   \
+        if (NT <= 256) gemm32_kernel<TY, 256, HH><<<tiles, NT, smem, st>>>(q);             \
+        else if (NT <= 512) gemm32_kernel<TY, 512, HH><<<tiles, NT, smem, st>>>(q);        \
+        else gemm32_kernel<TY, 1024, HH><<<tiles, NT, smem, st>>>(q);                      \
+    } while (0)
 #define SLAI_G32(TY)                                                                       \
     do {                                                                                   \
-        if (NT <= 256) gemm32_kernel<TY, 256><<<tiles, NT, smem, st>>>(q);                 \
-        else if (NT <= 512) gemm32_kernel<TY, 512><<<tiles, NT, smem, st>>>(q);            \
-        else gemm32_kernel<TY, 1024><<<tiles, NT, smem, st>>>(q);                          \
+        if (p.split_f16) SLAI_G32H(TY, true); else SLAI_G32H(TY, false);                   \
     } while (0)
             switch (p.seg[0].type) {
             case T_Q4_K: SLAI_G32(T_Q4_K); break;
@@ -606,16 +888,21 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
             default: SLAI_G32(T_Q5_K); break;
             }
 #undef SLAI_G32
+#undef SLAI_G32H
         } else {
             // the thread bound decides the register budget (256 threads leave 256 registers per lane, 1024 leave 128);
             // narrow matrices (few waves per workgroup) split the tokens over two workgroups
             const size_t smem1 = (size_t)ng * 16 * G16_LDS_ROW * sizeof(float), smem2 = 2 * smem1;
+#define SLAI_G16H(TY, HH)                                                                                  \
+    do {                                                                                                   \
+        if (NT <= 256) gemm16_kernel<TY, 256, 1, HH><<<dim3(tiles, 2), NT, smem1, st>>>(q);                \
+        else if (NT <= 512) gemm16_kernel<TY, 512, 1, HH><<<dim3(tiles, 2), NT, smem1, st>>>(q);           \
+        else if (NT <= 768) gemm16_kernel<TY, 768, 2, HH><<<tiles, NT, smem2, st>>>(q);                    \
+        else gemm16_kernel<TY, 1024, 2, HH><<<tiles, NT, smem2, st>>>(q);                                  \
+    } while (0)
 #define SLAI_G16(TY)                                                                                       \
     do {                                                                                                   \
-        if (NT <= 256) gemm16_kernel<TY, 256, 1><<<dim3(tiles, 2), NT, smem1, st>>>(q);                    \
-        else if (NT <= 512) gemm16_kernel<TY, 512, 1><<<dim3(tiles, 2), NT, smem1, st>>>(q);               \
-        else if (NT <= 768) gemm16_kernel<TY, 768, 2><<<tiles, NT, smem2, st>>>(q);                        \
-        else gemm16_kernel<TY, 1024, 2><<<tiles, NT, smem2, st>>>(q);                                      \
+        if (p.split_f16) SLAI_G16H(TY, true); else SLAI_G16H(TY, false);                                   \
     } while (0)
             switch (p.seg[0].type) {
             case T_Q4_K: SLAI_G16(T_Q4_K); break;
@@ -625,6 +912,7 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p) {
             default: SLAI_G16(T_Q5_K); break;
             }
 #undef SLAI_G16
+#undef SLAI_G16H
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;

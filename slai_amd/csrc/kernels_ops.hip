@@ -1,6 +1,7 @@
 // Element-wise, normalisation, softmax, f32 matmul and argmax kernels of the decode path.
 // Each kernel names the reference shader / CPU routine whose result it reproduces.
 #include "common.h"
+#include "device_util.h"
 #include <float.h>
 #include <hip/hip_fp16.h>
 
@@ -98,11 +99,26 @@ __global__ void silu_kernel(VecView a, VecView b) {
 }
 
 // the same over gate and up given as `nparts` partial sums each
-__global__ void silu_parts_kernel(float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part) {
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
-        float l = 0.0f, r = 0.0f;
-        for (uint32_t s = 0; s < nparts; ++s) { l += a[i + (size_t)s * part]; r += b[i + (size_t)s * part]; }
-        a[i] = r * (l / (1.0f + expf(-1.0f * l)));
+// (n, part: multiples of four, 16-byte aligned; ntokens < 32: a quad-major matrix of which only the first ntokens token
+// slots are in use.  split_flag: write each group of four as f16 heads and remainders, the
+// form the prompt-chunk GEMM reads on the half-precision matrix cores, and report values beyond the f16 range.)
+__global__ void silu_parts_kernel(float4 *a, const float4 *b, uint32_t n4, uint32_t nparts, uint32_t part4, int *split_flag, uint32_t ntokens) {
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += gridDim.x * blockDim.x) {
+        if ((i & 31u) >= ntokens) continue;                    // quad-major: group i belongs to token slot i % 32; unused slots hold stale values
+        float4 l = make_float4(0.0f, 0.0f, 0.0f, 0.0f), r = l;
+        for (uint32_t s = 0; s < nparts; ++s) {
+            const float4 la = a[i + (size_t)s * part4], rb = b[i + (size_t)s * part4];
+            l.x += la.x; l.y += la.y; l.z += la.z; l.w += la.w;
+            r.x += rb.x; r.y += rb.y; r.z += rb.z; r.w += rb.w;
+        }
+        const float4 o = make_float4(r.x * (l.x / (1.0f + expf(-1.0f * l.x))), r.y * (l.y / (1.0f + expf(-1.0f * l.y))),
+                                     r.z * (l.z / (1.0f + expf(-1.0f * l.z))), r.w * (l.w / (1.0f + expf(-1.0f * l.w))));
+        if (split_flag) {
+            if (split_overflows(o)) *split_flag = 3;            // 3: a gated hidden value
+            a[i] = split_quad(o);
+        } else {
+            a[i] = o;
+        }
     }
 }
 
@@ -293,8 +309,9 @@ hipError_t launch_silu(hipStream_t s, VecView a, VecView b) {
     silu_kernel<<<grid_for(a.n, 256), 256, 0, s>>>(a, b);
     return hipGetLastError();
 }
-hipError_t launch_silu_parts(hipStream_t s, float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part) {
-    silu_parts_kernel<<<grid_for(n, 256), 256, 0, s>>>(a, b, n, nparts, part);
+hipError_t launch_silu_parts(hipStream_t s, float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part, int *split_flag, uint32_t ntokens) {
+    if (n % 4 || part % 4 || (((uintptr_t)a | (uintptr_t)b) & 15)) return hipErrorInvalidValue;
+    silu_parts_kernel<<<grid_for(n / 4, 256), 256, 0, s>>>((float4 *)a, (const float4 *)b, n / 4, nparts, part / 4, split_flag, ntokens);
     return hipGetLastError();
 }
 hipError_t launch_gelu(hipStream_t s, VecView a) {

@@ -81,6 +81,10 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->attn_splits = env_int("SLAI_ATTN_SPLITS", 0);
     ctx->use_graph = env_int("SLAI_NO_GRAPH", 0) == 0;
     ctx->prompt_gemm = env_int("SLAI_PROMPT_GEMM", 1) != 0;
+    ctx->prompt_split_f16 = env_int("SLAI_PROMPT_SPLIT_F16", 1);
+    if (hipMalloc((void **)&ctx->split_flag, sizeof(int)) != hipSuccess || hipMemset(ctx->split_flag, 0, sizeof(int)) != hipSuccess) {
+        (void)hipStreamDestroy(ctx->stream); delete ctx; return SLAI_E_HIP;
+    }
     ctx->gemv_max_wgs = env_int("SLAI_GEMV_MAX_WGS", 512);
     ctx->tiled_layout = env_int("SLAI_TILED", 1) != 0;
     ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
@@ -95,6 +99,7 @@ SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
     if (ctx->gemv_scratch) (void)hipFree(ctx->gemv_scratch);
+    if (ctx->split_flag) (void)hipFree(ctx->split_flag);
     if (ctx->sampler_scratch) (void)hipFree(ctx->sampler_scratch);
     if (ctx->handoff_counters) (void)hipFree(ctx->handoff_counters);
     if (ctx->timer0) (void)hipEventDestroy(ctx->timer0);
@@ -492,10 +497,11 @@ SLAI_EXPORT int slai_matmul_quant_columns(slai_ctx *ctx, slai_view out, const sl
     if (int rc = gemv_scratch_reserve(ctx, (size_t)32 * m->ncols)) return rc;
     const float *xp = reinterpret_cast<const float *>(x.buf->dptr) + x.offset;
     float *op = reinterpret_cast<float *>(out.buf->dptr) + out.offset;
-    SLAI_HIP_TRY(ctx, launch_rows_to_quads(ctx->stream, ctx->gemv_scratch, xp, m->ncols, nt, m->ncols));
+    // (SLAI_PROMPT_SPLIT_F16=2, for kernel tests: the f16 form, whose range the caller then has to keep)
+    SLAI_HIP_TRY(ctx, launch_rows_to_quads(ctx->stream, ctx->gemv_scratch, xp, m->ncols, nt, m->ncols, ctx->prompt_split_f16 == 2 ? ctx->split_flag : nullptr));
     GemmChunkParams p;
     p.nseg = 1; p.ncols = m->ncols; p.ncb = m->ncb; p.ngroups = m->ngroups; p.rows_log2 = m->rows_log2;
-    p.x = ctx->gemv_scratch; p.ntokens = nt;
+    p.x = ctx->gemv_scratch; p.ntokens = nt; p.split_f16 = ctx->prompt_split_f16 == 2;
     p.seg[0].W = m->dptr; p.seg[0].type = m->type; p.seg[0].nrows = m->nrows; p.seg[0].out = op; p.seg[0].out_stride = m->nrows;
     p.seg[0].flags = accumulate ? GEMV_ACCUM : 0;
     hipError_t e = launch_gemm_chunk(ctx, p);

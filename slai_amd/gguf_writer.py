@@ -93,7 +93,8 @@ def _f32(a):
 
 def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, wtype, seed=1234,
                std=0.02, rope_base=10000.0, rms_eps=1e-5, out_type=None, v_type=None, embd_type=None,
-               with_output=True, arch="llama", bias=False, norm_random=False, distinct_layers=None, tokenizer=None):
+               with_output=True, arch="llama", bias=False, norm_random=False, distinct_layers=None, tokenizer=None,
+               ffn_norm_scale=1.0):
     """Synthetic Llama-2-shape model file (uint8 numpy array).
 
     Weights are seeded std*N(0,1) quantized to `wtype` (`v_type` for attn_v, `out_type` for
@@ -101,6 +102,7 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
     `distinct_layers`: when set, only that many layers are generated from scratch and the
     others reuse their packed bytes with the rows rotated (still distinct memory and the same
     value distribution; used to bound set-up time of the largest benchmark model).
+    `ffn_norm_scale`: factor on the ffn_norm weights (large values push the normalised rows beyond the f16 range).
     `tokenizer`: optional dict(model=, tokens=, scores=|merges=, bos=, eos=, unk=, chat_template=) written as the
     tokenizer.* metadata a chat front end reads; `vocab` must then equal len(tokens).
     """
@@ -131,10 +133,10 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
         ctr[0] += 1
         return synth.normal_quantized(ctr[0], t, nrows, ncols, std)
 
-    def norm_vec(n):
+    def norm_vec(n, scale=1.0):
         if norm_random:
-            return _f32(rng.normal(1.0, 0.02, n))
-        return _f32(np.ones(n))
+            return _f32(rng.normal(1.0, 0.02, n) * scale)
+        return _f32(np.ones(n) * scale)
 
     def rot(packed, nrows, shift):
         rb = packed.size // nrows
@@ -158,7 +160,7 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
             w.add_tensor(p + nm + ".weight", [nc, nr], t, data)
             if bias and nm in ("attn_q", "attn_k", "attn_v"):
                 w.add_tensor(p + nm + ".bias", [nr], 0, _f32(rng.normal(0.0, std, nr)))
-        w.add_tensor(p + "ffn_norm.weight", [dim], 0, norm_vec(dim))
+        w.add_tensor(p + "ffn_norm.weight", [dim], 0, norm_vec(dim, ffn_norm_scale))
     w.add_tensor("output_norm.weight", [dim], 0, norm_vec(dim))
     if with_output:
         w.add_tensor("output.weight", [dim, vocab], out_type, qmat(vocab, dim, out_type))

@@ -483,6 +483,10 @@ class Llama2:
         """2: matrix-core GEMM, 1: per-token workgroups over shared weights, 0: the token-by-token loop."""
         return int(self.b.L.slai_llama2_prefill_supported(self.h))
 
+    def prefill_fp32_repeats(self):
+        """Prefill calls that were repeated with fp32 MFMA because an activation was beyond the f16 range."""
+        return int(self.b.L.slai_llama2_prefill_fp32_repeats(self.h))
+
     def prefill(self, tokens, start_pos=0, chunk=0):
         """Fill the caches for positions start_pos .. start_pos+len(tokens)-1, `chunk` tokens per pass over the
         weights (0 = the library's default); returns the stream time in ms."""

@@ -57,7 +57,7 @@ def read_cache(backend, m, layer, nbytes):
 
 
 def check_prefill(backend, data, prompt, n_gen, chunks, kv_f16, model_type=_ffi.MODEL_LLAMA, neox=0, name=b"llama", expect_path=2,
-                  split_at=None):
+                  split_at=None, expect_repeats=None):
     g, om = oracle_llama(data, 1, neox, int(kv_f16), name)
     L = g.L
     prompt = np.asarray(prompt, np.int32)
@@ -97,6 +97,8 @@ def check_prefill(backend, data, prompt, n_gen, chunks, kv_f16, model_type=_ffi.
         assert rel_err(logits, base_logits) < SELF_TOL, (chunk, rel_err(logits, base_logits))
         got, _ = m.generate(prompt, n_gen, start_pos=n - 1)
         assert np.array_equal(got, ref_tokens[n - 1:]), (chunk, got.tolist(), ref_tokens[n - 1:].tolist())
+        if expect_repeats is not None:
+            assert m.prefill_fp32_repeats() == expect_repeats, (chunk, m.prefill_fp32_repeats())
         m.destroy()
     gg.close(); L.slo_llama2_free(om); g.close()
 
@@ -276,3 +278,17 @@ def test_gpt2_prefill_matrix_cores(backend, kv_f16):
     with pytest.raises(SlaiError):
         m.prefill(np.arange(10, dtype=np.int32), start_pos=1020)
     m.destroy(); gg.close(); L.slo_gpt2_free(om); g.close()
+
+
+def test_prefill_split_f16_and_its_fp32_repeat(backend):
+    """The matrix-core path runs on the half-precision units with f16 head + remainder pairs; a model whose normalised
+    rows exceed the f16 range (ffn_norm weights of 5e4) must notice, repeat the call with fp32 MFMA and still match the
+    oracle; an ordinary model must not repeat."""
+    import os
+    if os.environ.get("SLAI_PROMPT_SPLIT_F16") == "0" or os.environ.get("SLAI_PROMPT_GEMM") == "0":
+        pytest.skip("needs the split path")
+    for scale, repeats in ((1.0, 0), (5.0e4, 1)):
+        data = gw.llama_gguf(dim=1024, hidden_dim=2816, n_layers=2, n_heads=8, n_kv_heads=8, vocab=500, seq_len=64, wtype=12, v_type=14, seed=77,
+                             std=0.05, ffn_norm_scale=scale)
+        prompt = np.random.Generator(np.random.PCG64(78)).integers(0, 500, 40).astype(np.int32)
+        check_prefill(backend, data, prompt, 6, (32,), True, expect_repeats=repeats)

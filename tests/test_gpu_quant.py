@@ -325,6 +325,38 @@ def test_matmul_quant_columns_on_the_matrix_cores(backend, oracle_lib, t, shape,
     """slai_matmul_quant_columns (the fp32 MFMA kernels under the chunked prompt pass) against the dequantised matrix
     times the vectors in float64: every format with a tiled layout, the three tile heights, row counts that end inside a
     tile and inside a group of four rows, 1 / 7 / 32 vectors, assign and accumulate."""
+    check_matmul_quant_columns(backend, oracle_lib, t, shape, layout)
+
+
+@pytest.fixture(scope="module")
+def backend_split_ops():
+    """A context created with SLAI_PROMPT_SPLIT_F16=2: slai_matmul_quant_columns takes the half-precision matrix-core
+    kernels (weights and vectors as f16 head + remainder pairs) the models' prompt pass uses."""
+    import os
+    from slai_amd.runtime import Backend
+    old = os.environ.get("SLAI_PROMPT_SPLIT_F16")
+    os.environ["SLAI_PROMPT_SPLIT_F16"] = "2"
+    try:
+        b = Backend(0)
+    finally:
+        if old is None:
+            del os.environ["SLAI_PROMPT_SPLIT_F16"]
+        else:
+            os.environ["SLAI_PROMPT_SPLIT_F16"] = old
+    yield b
+    b.close()
+
+
+@pytest.mark.parametrize("t", [12, 13, 14, 8, 2], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("shape,layout", [((202, 1024), 3), ((64, 4096), 3), ((102, 1024), 2), ((50, 1536), 2), ((42, 16640), 2)],
+                         ids=["64-row-tiles-row-tail", "64-row-tiles-16-super-blocks", "16-row-tiles-row-tail", "32-row-tiles", "16-row-tiles-17-groups"])
+def test_matmul_quant_columns_split_f16(backend_split_ops, oracle_lib, t, shape, layout):
+    """The same bar (1e-5 of the float64 product) for the f16 head + remainder kernels: three half-precision MFMAs per
+    step keep about 22 bits of every weight and of every vector element."""
+    check_matmul_quant_columns(backend_split_ops, oracle_lib, t, shape, layout)
+
+
+def check_matmul_quant_columns(backend, oracle_lib, t, shape, layout):
     import os
     if os.environ.get("SLAI_TILED") == "0":
         pytest.skip("needs the tiled layouts")
