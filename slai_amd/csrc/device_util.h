@@ -18,14 +18,16 @@ template <int BYTES> __device__ __forceinline__ void touch_kernel_arguments() {
     asm volatile("" : : "s"(w));
 }
 
-// A value as an f16 head plus an f16 remainder (both rounded toward zero; the remainder of the head is exact in f32), about
+// A value as an f16 head plus an f16 remainder (both rounded toward zero; value - head is exact in f32), about
 // 22 bits together: the form in which the prompt-chunk GEMM reads activations for the half-precision matrix cores.
 // split_quad packs four values as {heads 0-1, heads 2-3, remainders 0-1, remainders 2-3} into the 16 bytes of the float4.
 __device__ __forceinline__ void split_pair_f16(float a, float b, uint32_t &h, uint32_t &l) {
-    const auto hh = __builtin_amdgcn_cvt_pkrtz(a, b);
-    const auto ll = __builtin_amdgcn_cvt_pkrtz(fmaf((float)hh[0], -1.0f, a), fmaf((float)hh[1], -1.0f, b));
-    h = __builtin_bit_cast(uint32_t, hh);
-    l = __builtin_bit_cast(uint32_t, ll);
+    h = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
+    // value - head, the head converted inside the instruction (the compiler would emit a conversion and a subtraction)
+    float ra, rb;
+    asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(ra) : "v"(h), "v"(a));
+    asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(rb) : "v"(h), "v"(b));
+    l = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(ra, rb));
 }
 __device__ __forceinline__ float4 split_quad(float4 v) {
     uint32_t h0, h1, l0, l1;
