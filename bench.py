@@ -279,14 +279,15 @@ def main():
     sampled = dict(tok_s=round(1000.0 * K / ms_s, 2), ms_per_step=round(ms_s / K, 4), temperature=0.7, top_p=0.95)
     log("sampled decode (device sampler, T=0.7, top-p 0.95): %.3f ms/token, %.1f tok/s" % (ms_s / K, 1000.0 * K / ms_s))
     # prompt processing, reported beside the headline: the reference feeds a prompt token by token (chat_llama2.rs:105-158);
-    # the chunked pass runs 32 tokens per pass over the weights on the matrix cores and computes no logits
+    # the chunked pass runs 32 tokens per pass over the weights on the matrix cores (weights and activations as f16 head +
+    # remainder pairs, fp32 accumulation; a call repeats in fp32 MFMA when an activation is beyond f16) and computes no logits
     n_prompt = min(256, seq_len)
     ptoks = np.random.Generator(np.random.PCG64(args.seed + 1)).integers(0, cfg["vocab"], n_prompt).astype(np.int32)
     model.prefill(ptoks, 0, 0)                                   # untimed: buffers, first touch
     ms_p = min(model.prefill(ptoks, 0, 0) for _ in range(3))
     ms_loop = model.prefill(ptoks[:64], 0, 1)
     prompt_chunks = dict(tok_s=round(1000.0 * n_prompt / ms_p, 1), tokens=n_prompt, ms=round(ms_p, 3), path=model.prefill_path(),
-                         token_by_token_tok_s=round(1000.0 * 64 / ms_loop, 1))
+                         token_by_token_tok_s=round(1000.0 * 64 / ms_loop, 1), fp32_repeats=model.prefill_fp32_repeats())
     log("prompt: %d tokens in %.2f ms (%.0f tok/s) in chunks; token by token %.0f tok/s" % (n_prompt, ms_p, 1000.0 * n_prompt / ms_p, 1000.0 * 64 / ms_loop))
     model.destroy(); g.close(); del data
 
