@@ -76,10 +76,11 @@ template <> struct Vec8<false> {  // 8 f32 = 32 bytes
 // others must have left the kernel).  `wait_inputs()` is called once, by every thread, before q / knew / vnew are read:
 // a launch in which this workgroup's inputs are produced by other workgroups of the same launch blocks there (FUSED:
 // the requests for the cache, which depend on nothing but the position, then go first).  `quad_token` (single-split
-// form only): write the result as that token's column of a quad-major matrix instead of a plain vector.
+// form only): write the result as that token's column of a quad-major matrix instead of a plain vector; with
+// `split_flag` as f16 head + remainder pairs (split_quad's layout), *split_flag set when a value is beyond f16.
 template <bool F16, int NT, int HS, bool SINGLE, bool FUSED, int KL = 4, class Wait>
 __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, uint32_t split, uint32_t tid, Wait &&wait_inputs,
-                                               uint32_t quad_token = 0xffffffffu) {
+                                               uint32_t quad_token = 0xffffffffu, int *split_flag = nullptr) {
     using C = KV<F16>;
     using CT = typename C::T;
     constexpr int NW = NT / 64;
@@ -283,8 +284,22 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
         if (a.n_splits == 1) {
             const uint32_t e = h * HS + tid;
             // (a chunk of prompt tokens: token `quad_token` of a [columns / 4][32 tokens][4] matrix)
-            if (quad_token != 0xffffffffu) a.out[((size_t)(e >> 2) * 32 + quad_token) * 4 + (e & 3u)] = r / l;
-            else a.out[e] = r / l;
+            if (quad_token != 0xffffffffu) {
+                float *slot = a.out + ((size_t)(e >> 2) * 32 + quad_token) * 4;
+                if (split_flag) {
+                    const float v = r / l;
+                    uint32_t hd, rm;
+                    split_pair_f16(v, 0.0f, hd, rm);
+                    if (!(fabsf(v) < 65504.0f)) *split_flag = 2;
+                    uint16_t *s16 = reinterpret_cast<uint16_t *>(slot);
+                    s16[e & 3u] = (uint16_t)hd;
+                    s16[4 + (e & 3u)] = (uint16_t)rm;
+                } else {
+                    slot[e & 3u] = r / l;
+                }
+            } else {
+                a.out[e] = r / l;
+            }
         } else {
             float *po = a.scratch + ((size_t)h * a.n_splits + split) * (HS + 2);
             po[tid] = r;

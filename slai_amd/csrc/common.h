@@ -216,8 +216,6 @@ hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, cons
 hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps);
 // quad-major copy of row-major vectors
 hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride, int *split_flag = nullptr);
-// quad-major f32 -> f16 heads and remainders in place (see GemmChunkParams::split_f16); *split_flag = 1 when a value is beyond f16
-hipError_t launch_quads_split(hipStream_t s, float *x, uint32_t n, uint32_t ntokens, int *split_flag);
 
 // One GEMV launch over up to three matrices of one format and layout: out[i] = epilogue(m[i] . prologue(x)).
 struct GemvCall {
@@ -329,7 +327,8 @@ hipError_t launch_attention(hipStream_t s, const AttnLaunch &a);
 // A chunk of `n` consecutive tokens whose keys and values are already in the caches: token b attends from q + b * q_stride
 // over positions [0, pos_ptr[b]] into out + b * out_stride (out_quads: into column b of the quad-major matrix `out`,
 // n <= 32); knew / vnew must be null.  One workgroup per head and token.
-hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride, bool out_quads = false);
+hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride, bool out_quads = false,
+                                  int *split_flag = nullptr);
 // out[b] = embedding row tokens[b] (dequantised), b < n
 // (+ row positions[b] of `pos_m` when that is given: learned position embeddings)
 hipError_t launch_embed_rows(hipStream_t s, const slai_qmat *m, const int *tokens, uint32_t n, uint32_t ncols, float *out, uint32_t out_stride,

@@ -145,7 +145,7 @@ struct slai_llama2 {
     uint32_t prefill_fp32_repeats = 0;   // prefill calls repeated in fp32 because an activation was beyond the f16 range
     int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev, bool split_f16);   // the same on the matrix cores, n <= 32
     // q / k / v given as nparts partial sums, 32 rows apart; out_quads: the result goes to xn, quad-major, instead of xb
-    int chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts = 1, bool out_quads = false);
+    int chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts = 1, bool out_quads = false, int *split_flag = nullptr);
 };
 
 // models/llama2/cpu.rs:79-109
@@ -528,7 +528,7 @@ int slai_llama2::enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev)
 
 // Bias + RoPE + cache write for the n tokens of a chunk (their q / k / v are in the chunk's matrices), then their
 // attention into the chunk's xb.
-int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts, bool out_quads) {
+int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t nparts, bool out_quads, int *split_flag) {
     PromptChunkState &pc = chunk;
     Llama2State &s = state;
     const Llama2LayerWeights &wl = weights.layers[l];
@@ -547,7 +547,7 @@ int slai_llama2::chunk_attention(uint32_t l, uint32_t pos0, uint32_t n, uint32_t
     a.rope_theta = (const float *)s.rope_theta.buf->dptr;
     a.out = out_quads ? (float *)pc.xn.buf->dptr : (float *)pc.xb.buf->dptr; a.scratch = nullptr; a.n_splits = 1;
     SLAI_HIP_TRY(ctx, launch_rope_store_batch(ctx->stream, a, q, (const float *)pc.k.buf->dptr, (const float *)pc.v.buf->dptr, n, dim, kvd, nparts, 32 * dim, 32 * kvd));
-    SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, dim, dim, out_quads));
+    SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, dim, dim, out_quads, split_flag));
     return SLAI_OK;
 }
 
@@ -626,8 +626,7 @@ int slai_llama2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens
             const uint32_t strides[3] = {kvd, kvd, dim};
             const uint32_t ks = chunk_ksplit(3, mats);
             TRY(gemm_chunk_call(ctx, 3, mats, outs, strides, 0, xn, n, "llama2 qkv (prompt chunk)", ks, split_f16));
-            TRY(chunk_attention(l, pos0, n, ks, true));       // straight into xn, quad-major
-            if (sf) SLAI_HIP_TRY(ctx, launch_quads_split(ctx->stream, xn, dim, n, sf));
+            TRY(chunk_attention(l, pos0, n, ks, true, sf));   // straight into xn, quad-major (as f16 pairs for the f16 form)
         }
         {
             const slai_qmat *mats[1] = {wl.attn_output};

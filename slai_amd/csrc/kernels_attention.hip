@@ -172,17 +172,18 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
 
 // A chunk of tokens whose keys and values are already in the caches: grid = (n_heads, tokens), whole context in one
 // workgroup; token b reads q + b * q_stride and its position pos_ptr[b], and writes out + b * out_stride or, with
-// out_quads, column b of the quad-major matrix `out` ([columns / 4][32 tokens][4], the prompt-chunk GEMM's input).
+// out_quads, column b of the quad-major matrix `out` ([columns / 4][32 tokens][4], the prompt-chunk GEMM's input; with
+// split_flag as f16 head + remainder pairs).
 template <bool F16, int HS>
-__global__ void __launch_bounds__(512) attn_fast_batch_kernel(AttnLaunch a0, uint32_t q_stride, uint32_t out_stride, uint32_t out_quads) {
-    touch_kernel_arguments<sizeof(AttnLaunch) + 12>();
+__global__ void __launch_bounds__(512) attn_fast_batch_kernel(AttnLaunch a0, uint32_t q_stride, uint32_t out_stride, uint32_t out_quads, int *split_flag) {
+    touch_kernel_arguments<sizeof(AttnLaunch) + 24>();
     AttnLaunch a = a0;
     const uint32_t b = blockIdx.y;
     a.q = a0.q + (size_t)b * q_stride;
     a.out = out_quads ? a0.out : a0.out + (size_t)b * out_stride;
     a.pos_ptr = a0.pos_ptr + b;
     a.knew = nullptr; a.vnew = nullptr;
-    attn_fast_body<F16, 512, HS, true, false>(a, blockIdx.x, 0u, threadIdx.x, []() {}, out_quads ? b : 0xffffffffu);
+    attn_fast_body<F16, 512, HS, true, false>(a, blockIdx.x, 0u, threadIdx.x, []() {}, out_quads ? b : 0xffffffffu, out_quads ? split_flag : nullptr);
 }
 
 // The bias / RoPE / cache-write part of attn_fast_body for a chunk of tokens, as a launch of its own: a token's
@@ -295,16 +296,16 @@ hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
     return e;
 }
 
-hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride, bool out_quads) {
+hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride, bool out_quads, int *split_flag) {
     if ((a.head_size != 64 && a.head_size != 128) || a.kv_dim % 8 || a.knew || a.vnew || n == 0 || n > 65535 || (out_quads && n > 32)) return hipErrorInvalidValue;
     const uint32_t oq = out_quads ? 1u : 0u;
     dim3 grid(a.n_heads, n);
     if (a.head_size == 128) {
-        if (a.kv_f16) attn_fast_batch_kernel<true, 128><<<grid, 512, 0, s>>>(a, q_stride, out_stride, oq);
-        else attn_fast_batch_kernel<false, 128><<<grid, 512, 0, s>>>(a, q_stride, out_stride, oq);
+        if (a.kv_f16) attn_fast_batch_kernel<true, 128><<<grid, 512, 0, s>>>(a, q_stride, out_stride, oq, split_flag);
+        else attn_fast_batch_kernel<false, 128><<<grid, 512, 0, s>>>(a, q_stride, out_stride, oq, split_flag);
     } else {
-        if (a.kv_f16) attn_fast_batch_kernel<true, 64><<<grid, 512, 0, s>>>(a, q_stride, out_stride, oq);
-        else attn_fast_batch_kernel<false, 64><<<grid, 512, 0, s>>>(a, q_stride, out_stride, oq);
+        if (a.kv_f16) attn_fast_batch_kernel<true, 64><<<grid, 512, 0, s>>>(a, q_stride, out_stride, oq, split_flag);
+        else attn_fast_batch_kernel<false, 64><<<grid, 512, 0, s>>>(a, q_stride, out_stride, oq, split_flag);
     }
     return hipGetLastError();
 }

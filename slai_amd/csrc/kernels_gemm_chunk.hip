@@ -756,16 +756,6 @@ __global__ void rows_to_quads_kernel(float4 *out, const float *x, uint32_t n, ui
     }
 }
 
-// quad-major f32 -> the split form, in place (both are 16 bytes per quad and token)
-__global__ void quads_split_kernel(float4 *x, uint32_t nquads, uint32_t ntokens, int *split_flag) {
-    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x, t = idx & 31u, qd = idx >> 5;
-    if (qd < nquads && t < ntokens) {
-        const float4 r = x[idx];
-        if (split_overflows(r)) *split_flag = 2;                        // 2: converted in place
-        x[idx] = split_quad(r);
-    }
-}
-
 }  // namespace
 
 bool gemm_chunk_supports(const slai_qmat *m) {
@@ -788,12 +778,6 @@ hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, con
 hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride, int *split_flag) {
     if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || x_stride % 4) return hipErrorInvalidValue;
     rows_to_quads_kernel<<<(n / 4 * 32 + 255) / 256, 256, 0, s>>>((float4 *)out, x, n, x_stride, ntokens, split_flag);
-    return hipGetLastError();
-}
-
-hipError_t launch_quads_split(hipStream_t s, float *x, uint32_t n, uint32_t ntokens, int *split_flag) {
-    if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || !split_flag) return hipErrorInvalidValue;
-    quads_split_kernel<<<(n / 4 * 32 + 255) / 256, 256, 0, s>>>((float4 *)x, n / 4, ntokens, split_flag);
     return hipGetLastError();
 }
 
