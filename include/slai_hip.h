@@ -304,8 +304,8 @@ int slai_llama2_generate_sampled(slai_llama2 *m, const int32_t *prompt, uint32_t
  * 32 tokens per pass: on the half-precision units with every weight and activation split into an f16 head and an f16
  * remainder (about 22 bits of each, fp32 accumulation), repeated with fp32 MFMA when an activation turns out to be beyond
  * the f16 range (slai_llama2_prefill_fp32_repeats counts those calls), in fp32 MFMA from the start when the context was
- * created with SLAI_PROMPT_SPLIT_F16=0 (the pair form also needs every dequantised weight below 255 in magnitude, which
- * the weights of a trained model are by orders of magnitude); 1 = the GEMV kernels with one workgroup per token and tile sharing the weights through L2 (the
+ * created with SLAI_PROMPT_SPLIT_F16=0 or when the block scales of a layer matrix allow a weight of 255 or more in
+ * magnitude (the pair form holds 256 * w in f16; trained models are orders of magnitude below); 1 = the GEMV kernels with one workgroup per token and tile sharing the weights through L2 (the
  * same layouts when the context was created with SLAI_PROMPT_GEMM=0); 0 = layouts without chunked kernels, run token by
  * token with the same result. */
 int slai_llama2_prefill(slai_llama2 *m, const int32_t *tokens, uint32_t n_tokens, uint32_t start_pos, uint32_t chunk,

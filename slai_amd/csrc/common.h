@@ -27,6 +27,9 @@ struct slai_qmat {
     uint32_t rows_log2 = 0, ncb = 0, ngroups = 0, ntiles = 0, unit_bytes = 0;
     uint8_t *dptr = nullptr;
     size_t bytes = 0;
+    // tiled layouts: an upper bound of |w| over the matrix, from its block headers (the prompt pass takes the f16 matrix
+    // cores only where 256 * |w| fits f16)
+    float wbound = 0.0f;
 };
 
 struct slai_graph {

@@ -142,6 +142,7 @@ struct slai_llama2 {
     bool chunk_gemm_supported() const;   // matrix cores (K-quants)
     int chunk_reserve(uint32_t rows);
     int enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev);   // fills the caches for positions pos0 .. pos0 + n - 1
+    bool chunk_split_ok() const;         // every layer matrix small enough for the f16 head + remainder form (256 * |w| within f16)
     uint32_t prefill_fp32_repeats = 0;   // prefill calls repeated in fp32 because an activation was beyond the f16 range
     int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev, bool split_f16);   // the same on the matrix cores, n <= 32
     // q / k / v given as nparts partial sums, 32 rows apart; out_quads: the result goes to xn, quad-major, instead of xb
@@ -602,6 +603,13 @@ int gemm_chunk_call(slai_ctx *ctx, int nmat, const slai_qmat *const *mats, float
 }  // namespace
 
 // The layer loop for a chunk of up to 32 tokens with every projection on the matrix cores (kernels_gemm_chunk.hip):
+bool slai_llama2::chunk_split_ok() const {
+    for (const Llama2LayerWeights &wl : weights.layers)
+        for (const slai_qmat *m : {wl.attn_q, wl.attn_k, wl.attn_v, wl.attn_output, wl.ffn_gate, wl.ffn_up, wl.ffn_down})
+            if (!(m->wbound < 255.0f)) return false;
+    return true;
+}
+
 // RMSNorm of all rows, q/k/v, bias + RoPE + cache write, attention, output projection into the residual, RMSNorm,
 // gate and up, SiLU, down projection into the residual (transformer.rs:316-381 per token).
 // split_f16: the GEMMs on the half-precision matrix cores, their inputs written as f16 heads and remainders by the kernels
@@ -836,7 +844,7 @@ SLAI_EXPORT int slai_llama2_prefill(slai_llama2 *m, const int32_t *tokens, uint3
     SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev0, ctx->stream));
     // The matrix-core pass runs on the half-precision units with split activations; if one of them turns out to be
     // beyond the f16 range the whole pass is repeated in fp32 (it only writes the caches, so that is safe).
-    bool split = gemm && ctx->prompt_split_f16 != 0 && ctx->split_flag;
+    bool split = gemm && ctx->prompt_split_f16 != 0 && ctx->split_flag && m->chunk_split_ok();
     for (;;) {
         if (split) SLAI_HIP_TRY(ctx, hipMemsetAsync(ctx->split_flag, 0, sizeof(int), ctx->stream));
         for (uint32_t i = 0; i < n_tokens; i += chunk) {

@@ -188,6 +188,37 @@ SLAI_EXPORT int slai_copy_buffer(slai_ctx *ctx, slai_buffer *dst, size_t dst_off
 }
 
 // ---- quantized matrices ---------------------------------------------------------
+// Upper bound of |w| over a matrix in GGUF block order, from the block scales alone: |d| * 63 * 15 + |dmin| * 63 (Q4_K;
+// 31 for Q5_K), |d| * 128 * 32 (Q6_K), |d| * 128 (Q8_0), |d| * 8 (Q4_0).  binary16 magnitudes order like their bit
+// patterns, so the scan compares integers and converts once.
+static float weight_bound(int t, size_t nblocks, const uint8_t *packed) {
+    size_t stride, d_off;
+    switch (t) {
+    case T_Q4_K: stride = 144; d_off = 0; break;
+    case T_Q5_K: stride = 176; d_off = 0; break;
+    case T_Q6_K: stride = 210; d_off = 208; break;
+    case T_Q8_0: stride = 34; d_off = 0; break;
+    case T_Q4_0: stride = 18; d_off = 0; break;
+    default: return INFINITY;
+    }
+    const bool has_min = t == T_Q4_K || t == T_Q5_K;
+    uint16_t dmax = 0, mmax = 0;
+    for (size_t b = 0; b < nblocks; ++b) {
+        const uint8_t *p = packed + b * stride + d_off;
+        dmax = std::max<uint16_t>(dmax, (uint16_t)((p[0] | (p[1] << 8)) & 0x7fff));
+        if (has_min) mmax = std::max<uint16_t>(mmax, (uint16_t)((p[2] | (p[3] << 8)) & 0x7fff));
+    }
+    if (dmax >= 0x7c00 || mmax >= 0x7c00) return INFINITY;    // an infinite or NaN scale
+    const float d = decode_f16(dmax), dm = decode_f16(mmax);
+    switch (t) {
+    case T_Q4_K: return d * 63.0f * 15.0f + dm * 63.0f;
+    case T_Q5_K: return d * 63.0f * 31.0f + dm * 63.0f;
+    case T_Q6_K: return d * 128.0f * 32.0f;
+    case T_Q8_0: return d * 128.0f;
+    default: return d * 8.0f;
+    }
+}
+
 SLAI_EXPORT int slai_qmat_create(slai_ctx *ctx, uint32_t ggml_type, uint32_t nrows, uint32_t ncols, const void *packed,
                                  slai_qmat **out) {
     return slai_qmat_create_layout(ctx, ggml_type, nrows, ncols, packed, SLAI_LAYOUT_AUTO, out);
@@ -235,6 +266,8 @@ SLAI_EXPORT int slai_qmat_create_layout(slai_ctx *ctx, uint32_t ggml_type, uint3
             if (e == hipSuccess) e = launch_repack(ctx->stream, m, staging);
         }
     }
+    // (while the copies run) the bound the prompt pass needs to choose between the f16 and the fp32 matrix instructions
+    if (e == hipSuccess && m->tiled) m->wbound = weight_bound(t, (size_t)nrows * m->nb, (const uint8_t *)packed);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (staging) (void)hipFree(staging);
     if (e != hipSuccess) {
@@ -498,10 +531,10 @@ SLAI_EXPORT int slai_matmul_quant_columns(slai_ctx *ctx, slai_view out, const sl
     const float *xp = reinterpret_cast<const float *>(x.buf->dptr) + x.offset;
     float *op = reinterpret_cast<float *>(out.buf->dptr) + out.offset;
     // (SLAI_PROMPT_SPLIT_F16=2, for kernel tests: the f16 form, whose range the caller then has to keep)
-    SLAI_HIP_TRY(ctx, launch_rows_to_quads(ctx->stream, ctx->gemv_scratch, xp, m->ncols, nt, m->ncols, ctx->prompt_split_f16 == 2 ? ctx->split_flag : nullptr));
+    SLAI_HIP_TRY(ctx, launch_rows_to_quads(ctx->stream, ctx->gemv_scratch, xp, m->ncols, nt, m->ncols, ctx->prompt_split_f16 == 2 && m->wbound < 255.0f ? ctx->split_flag : nullptr));
     GemmChunkParams p;
     p.nseg = 1; p.ncols = m->ncols; p.ncb = m->ncb; p.ngroups = m->ngroups; p.rows_log2 = m->rows_log2;
-    p.x = ctx->gemv_scratch; p.ntokens = nt; p.split_f16 = ctx->prompt_split_f16 == 2;
+    p.x = ctx->gemv_scratch; p.ntokens = nt; p.split_f16 = ctx->prompt_split_f16 == 2 && m->wbound < 255.0f;
     p.seg[0].W = m->dptr; p.seg[0].type = m->type; p.seg[0].nrows = m->nrows; p.seg[0].out = op; p.seg[0].out_stride = m->nrows;
     p.seg[0].flags = accumulate ? GEMV_ACCUM : 0;
     hipError_t e = launch_gemm_chunk(ctx, p);

@@ -292,3 +292,12 @@ def test_prefill_split_f16_and_its_fp32_repeat(backend):
                              std=0.05, ffn_norm_scale=scale)
         prompt = np.random.Generator(np.random.PCG64(78)).integers(0, 500, 40).astype(np.int32)
         check_prefill(backend, data, prompt, 6, (32,), True, expect_repeats=repeats)
+
+
+def test_prefill_large_weights_take_fp32_from_the_start(backend):
+    """The f16 head + remainder form needs 256 * |w| within f16; the block scales of every matrix bound |w| at load time,
+    and a model beyond the bound (weights of std 40) takes the fp32 kernels at once: same parity, no repeated call."""
+    data = gw.llama_gguf(dim=1024, hidden_dim=2816, n_layers=2, n_heads=8, n_kv_heads=8, vocab=500, seq_len=64, wtype=12, v_type=14, seed=79,
+                         std=40.0)
+    prompt = np.random.Generator(np.random.PCG64(80)).integers(0, 500, 40).astype(np.int32)
+    check_prefill(backend, data, prompt, 6, (32,), True, expect_repeats=0)
