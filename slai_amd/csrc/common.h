@@ -216,7 +216,8 @@ hipError_t launch_gemm_chunk(slai_ctx *ctx, GemmChunkParams p);
 // quad-major out = RMSNorm of the `ntokens` row-major vectors of n floats at x + t * x_stride
 hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, const float *w, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps, int *split_flag = nullptr);
 // the same with LayerNorm (mean-centred, * g + b)
-hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps);
+hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps,
+                                  int *split_flag = nullptr);
 // quad-major copy of row-major vectors
 hipError_t launch_rows_to_quads(hipStream_t s, float *out, const float *x, uint32_t n, uint32_t ntokens, uint32_t x_stride, int *split_flag = nullptr);
 
@@ -284,6 +285,8 @@ hipError_t launch_silu(hipStream_t s, VecView a, VecView b);
 // out[i] = x[i]*w[i] (i < n), out[n + j] = sum of products 16j..16j+15; n % 16 == 0
 hipError_t launch_prepare(hipStream_t s, float *out, const float *x, const float *w, uint32_t n);
 hipError_t launch_gelu(hipStream_t s, VecView a);
+// GELU over the first ntokens token slots of a quad-major matrix of n floats, in place (split_flag: see launch_silu_parts)
+hipError_t launch_gelu_quads(hipStream_t s, float *a, uint32_t n, uint32_t ntokens, int *split_flag = nullptr);
 hipError_t launch_rope(hipStream_t s, int variant, const slai_rope_config *cfg_dev, VecView q, VecView k);
 hipError_t launch_attn_mask(hipStream_t s, const slai_attn_params *params_dev, float *attn, uint32_t nthreads);
 struct View4 { float *p; uint32_t size[4]; uint32_t stride[4]; };

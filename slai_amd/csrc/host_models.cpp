@@ -911,7 +911,8 @@ struct slai_gpt2 {
     struct { GpuTensor x, xn, qkv, h; slai_buffer *positions = nullptr, *tokens = nullptr; bool ready = false; } chunk;
     bool chunk_gemm_supported() const;
     int chunk_reserve();
-    int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev);
+    bool chunk_split_ok() const;
+    int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev, bool split_f16);
 };
 
 int slai_gpt2::load(const slai_gguf *gg) {
@@ -1068,17 +1069,25 @@ int slai_gpt2::chunk_reserve() {
 // gpt2/cpu.rs:225-383 for n <= 32 tokens at once, every projection on the matrix cores: embeddings, then per layer
 // LayerNorm, qkv + bias, cache write, attention, projection + bias into the residual, LayerNorm, fc + bias, GELU,
 // projection + bias into the residual.  No logits.
-int slai_gpt2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev) {
+bool slai_gpt2::chunk_split_ok() const {
+    for (const Gpt2Layer &w : layers)
+        for (const slai_qmat *m : {w.c_attn_attn_w, w.c_attn_proj_w, w.c_mlp_fc_w, w.c_mlp_proj_w})
+            if (!(m->wbound < 255.0f)) return false;
+    return true;
+}
+
+int slai_gpt2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev, bool split_f16) {
     if (n == 0 || n > 32 || pos0 + n > params.n_seq) return set_error(ctx, SLAI_E_ARG, "prompt chunk out of range");
     const uint32_t E = params.n_embd, F = params.ff_len;
     float *x = (float *)chunk.x.buf->dptr, *xn = (float *)chunk.xn.buf->dptr, *qkv = (float *)chunk.qkv.buf->dptr, *h = (float *)chunk.h.buf->dptr;
     const int *positions = (const int *)chunk.positions->dptr + pos0;
     const float eps = 1.0e-5f;
+    int *const sf = split_f16 ? ctx->split_flag : nullptr;     // see slai_llama2::enqueue_chunk_gemm
     SLAI_HIP_TRY(ctx, launch_embed_rows(ctx->stream, wte, tokens_dev, n, E, x, E, wpe, positions));
     const auto gemm = [&](const slai_qmat *m, const float *bias, float *out, uint32_t out_stride, uint32_t flags, const float *xq, const char *who) -> int {
         GemmChunkParams p;
         p.nseg = 1; p.ncols = m->ncols; p.ncb = m->ncb; p.ngroups = m->ngroups; p.rows_log2 = m->rows_log2;
-        p.x = xq; p.ntokens = n;
+        p.x = xq; p.ntokens = n; p.split_f16 = split_f16;
         p.seg[0].W = m->dptr; p.seg[0].type = m->type; p.seg[0].nrows = m->nrows; p.seg[0].out = out; p.seg[0].out_stride = out_stride;
         p.seg[0].bias = bias; p.seg[0].flags = flags;
         hipError_t e = launch_gemm_chunk(ctx, p);
@@ -1088,7 +1097,7 @@ int slai_gpt2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_d
     };
     for (uint32_t l = 0; l < params.n_layer; ++l) {
         Gpt2Layer &w = layers[l];
-        SLAI_HIP_TRY(ctx, launch_layernorm_quads(ctx->stream, xn, x, (const float *)w.ln_1_g.buf->dptr, (const float *)w.ln_1_b.buf->dptr, E, n, E, eps));
+        SLAI_HIP_TRY(ctx, launch_layernorm_quads(ctx->stream, xn, x, (const float *)w.ln_1_g.buf->dptr, (const float *)w.ln_1_b.buf->dptr, E, n, E, eps, sf));
         TRY(gemm(w.c_attn_attn_w, (const float *)w.c_attn_attn_b.buf->dptr, qkv, 3 * E, GEMV_BIAS, xn, "gpt2 qkv (prompt chunk)"));
         AttnLaunch a{};
         a.q = qkv; a.kcache = w.key_cache.buf->dptr; a.vcache = w.value_cache.buf->dptr; a.kv_f16 = kv_dtype == SLAI_KV_F16;
@@ -1098,11 +1107,11 @@ int slai_gpt2::enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_d
         a.out = xn; a.scratch = nullptr; a.n_splits = 1;
         // keys and values of all tokens into the caches first (no rotation: learned positions), then the attention of each
         SLAI_HIP_TRY(ctx, launch_rope_store_batch(ctx->stream, a, qkv, qkv + E, qkv + 2 * E, n, 3 * E, 3 * E));
-        SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, 3 * E, E, true));
+        SLAI_HIP_TRY(ctx, launch_attention_batch(ctx->stream, a, n, 3 * E, E, true, sf));
         TRY(gemm(w.c_attn_proj_w, (const float *)w.c_attn_proj_b.buf->dptr, x, E, GEMV_BIAS | GEMV_ACCUM, xn, "gpt2 attn proj (prompt chunk)"));
-        SLAI_HIP_TRY(ctx, launch_layernorm_quads(ctx->stream, xn, x, (const float *)w.ln_2_g.buf->dptr, (const float *)w.ln_2_b.buf->dptr, E, n, E, eps));
+        SLAI_HIP_TRY(ctx, launch_layernorm_quads(ctx->stream, xn, x, (const float *)w.ln_2_g.buf->dptr, (const float *)w.ln_2_b.buf->dptr, E, n, E, eps, sf));
         TRY(gemm(w.c_mlp_fc_w, (const float *)w.c_mlp_fc_b.buf->dptr, h, F, GEMV_BIAS | GEMM_OUT_QUADS, xn, "gpt2 mlp fc (prompt chunk)"));
-        SLAI_HIP_TRY(ctx, launch_gelu(ctx->stream, VecView{h, 32 * F, 1}));     // element-wise: the layout does not matter
+        SLAI_HIP_TRY(ctx, launch_gelu_quads(ctx->stream, h, 32 * F, n, sf));
         TRY(gemm(w.c_mlp_proj_w, (const float *)w.c_mlp_proj_b.buf->dptr, x, E, GEMV_BIAS | GEMV_ACCUM, h, "gpt2 mlp proj (prompt chunk)"));
     }
     return SLAI_OK;
@@ -1196,9 +1205,19 @@ SLAI_EXPORT int slai_gpt2_prefill(slai_gpt2 *m, const int32_t *tokens, uint32_t 
     TRY(slai_write_buffer(ctx, m->chunk.tokens, 0, tokens, (size_t)n_tokens * 4));
     const int *tokens_dev = (const int *)m->chunk.tokens->dptr;
     SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev0, ctx->stream));
-    for (uint32_t i = 0; i < n_tokens; i += chunk) TRY(m->enqueue_chunk_gemm(start_pos + i, std::min(chunk, n_tokens - i), tokens_dev + i));
-    SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev1, ctx->stream));
-    TRY(slai_synchronize(ctx));
+    // on the half-precision matrix cores first, repeated in fp32 when an activation was beyond f16 (see slai_llama2_prefill)
+    bool split = ctx->prompt_split_f16 != 0 && ctx->split_flag && m->chunk_split_ok();
+    for (;;) {
+        if (split) SLAI_HIP_TRY(ctx, hipMemsetAsync(ctx->split_flag, 0, sizeof(int), ctx->stream));
+        for (uint32_t i = 0; i < n_tokens; i += chunk) TRY(m->enqueue_chunk_gemm(start_pos + i, std::min(chunk, n_tokens - i), tokens_dev + i, split));
+        SLAI_HIP_TRY(ctx, hipEventRecord(m->loop.ev1, ctx->stream));
+        TRY(slai_synchronize(ctx));
+        if (!split) break;
+        int beyond = 0;
+        SLAI_HIP_TRY(ctx, hipMemcpy(&beyond, ctx->split_flag, sizeof(int), hipMemcpyDeviceToHost));
+        if (!beyond) break;
+        split = false;
+    }
     if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, m->loop.ev0, m->loop.ev1));
     return SLAI_OK;
 }

@@ -704,7 +704,8 @@ __global__ void __launch_bounds__(256) rms_norm_quads_kernel(float4 *out, const 
 
 // LayerNorm of token t = blockIdx.x (ops/layernorm.rs:104-111: mean, centred values, variance = their squared norm / n,
 // 1 / sqrt(variance + eps)), then * g + b, written quad-major.  n % 4 == 0, n <= 16384.
-__global__ void __launch_bounds__(256) layernorm_quads_kernel(float4 *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t x_stride, float eps) {
+__global__ void __launch_bounds__(256) layernorm_quads_kernel(float4 *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t x_stride, float eps,
+                                                              int *split_flag) {
     __shared__ float red[4], red2[4];
     const uint32_t t = blockIdx.x, nq = n / 4;
     const float4 *xr = (const float4 *)(x + (size_t)t * x_stride), *gr = (const float4 *)g, *br = (const float4 *)b;
@@ -740,8 +741,14 @@ __global__ void __launch_bounds__(256) layernorm_quads_kernel(float4 *out, const
         const uint32_t i = threadIdx.x + 256u * j;
         if (i < nq) {
             const float4 gg = gr[i], bb = br[i];
-            out[(size_t)i * 32 + t] = make_float4((v[j].x * scale) * gg.x + bb.x, (v[j].y * scale) * gg.y + bb.y, (v[j].z * scale) * gg.z + bb.z,
-                                                  (v[j].w * scale) * gg.w + bb.w);
+            const float4 r = make_float4((v[j].x * scale) * gg.x + bb.x, (v[j].y * scale) * gg.y + bb.y, (v[j].z * scale) * gg.z + bb.z,
+                                         (v[j].w * scale) * gg.w + bb.w);
+            if (split_flag) {                                  // (uniform) f16 heads and remainders; values beyond f16 are reported
+                if (split_overflows(r)) *split_flag = 1;
+                out[(size_t)i * 32 + t] = split_quad(r);
+            } else {
+                out[(size_t)i * 32 + t] = r;
+            }
         }
     }
 }
@@ -769,9 +776,10 @@ hipError_t launch_rms_norm_quads(hipStream_t s, float *out, const float *x, cons
     return hipGetLastError();
 }
 
-hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps) {
+hipError_t launch_layernorm_quads(hipStream_t s, float *out, const float *x, const float *g, const float *b, uint32_t n, uint32_t ntokens, uint32_t x_stride, float eps,
+                                  int *split_flag) {
     if (ntokens == 0 || ntokens > 32 || n == 0 || n % 4 || n > 16384 || x_stride % 4) return hipErrorInvalidValue;
-    layernorm_quads_kernel<<<ntokens, 256, 0, s>>>((float4 *)out, x, g, b, n, x_stride, eps);
+    layernorm_quads_kernel<<<ntokens, 256, 0, s>>>((float4 *)out, x, g, b, n, x_stride, eps, split_flag);
     return hipGetLastError();
 }
 

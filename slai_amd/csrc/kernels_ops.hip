@@ -122,6 +122,26 @@ __global__ void silu_parts_kernel(float4 *a, const float4 *b, uint32_t n4, uint3
     }
 }
 
+// ops/unary.rs:81-85 (UnaryOp::Gelu) over a quad-major matrix (groups of four columns, 32 token slots of which the
+// first ntokens are in use), in place; with split_flag written as f16 heads and remainders like silu_parts_kernel does
+__global__ void gelu_quads_kernel(float4 *a, uint32_t n4, uint32_t ntokens, int *split_flag) {
+    const float GELU_COEF_A = 0.044715f, SQRT_2_OVER_PI = 0.7978846f;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += gridDim.x * blockDim.x) {
+        if ((i & 31u) >= ntokens) continue;
+        const float4 x = a[i];
+        const float4 o = make_float4(0.5f * x.x * (1.0f + tanhf(SQRT_2_OVER_PI * x.x * (1.0f + GELU_COEF_A * x.x * x.x))),
+                                     0.5f * x.y * (1.0f + tanhf(SQRT_2_OVER_PI * x.y * (1.0f + GELU_COEF_A * x.y * x.y))),
+                                     0.5f * x.z * (1.0f + tanhf(SQRT_2_OVER_PI * x.z * (1.0f + GELU_COEF_A * x.z * x.z))),
+                                     0.5f * x.w * (1.0f + tanhf(SQRT_2_OVER_PI * x.w * (1.0f + GELU_COEF_A * x.w * x.w))));
+        if (split_flag) {
+            if (split_overflows(o)) *split_flag = 3;            // 3: a hidden value
+            a[i] = split_quad(o);
+        } else {
+            a[i] = o;
+        }
+    }
+}
+
 // ops/unary.rs:81-85 (UnaryOp::Gelu)
 __global__ void gelu_kernel(VecView a) {
     const float GELU_COEF_A = 0.044715f, SQRT_2_OVER_PI = 0.7978846f;
@@ -312,6 +332,11 @@ hipError_t launch_silu(hipStream_t s, VecView a, VecView b) {
 hipError_t launch_silu_parts(hipStream_t s, float *a, const float *b, uint32_t n, uint32_t nparts, uint32_t part, int *split_flag, uint32_t ntokens) {
     if (n % 4 || part % 4 || (((uintptr_t)a | (uintptr_t)b) & 15)) return hipErrorInvalidValue;
     silu_parts_kernel<<<grid_for(n / 4, 256), 256, 0, s>>>((float4 *)a, (const float4 *)b, n / 4, nparts, part / 4, split_flag, ntokens);
+    return hipGetLastError();
+}
+hipError_t launch_gelu_quads(hipStream_t s, float *a, uint32_t n, uint32_t ntokens, int *split_flag) {
+    if (n % 4 || ((uintptr_t)a & 15) || ntokens == 0 || ntokens > 32) return hipErrorInvalidValue;
+    gelu_quads_kernel<<<grid_for(n / 4, 256), 256, 0, s>>>((float4 *)a, n / 4, ntokens, split_flag);
     return hipGetLastError();
 }
 hipError_t launch_gelu(hipStream_t s, VecView a) {
