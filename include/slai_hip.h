@@ -329,11 +329,13 @@ int slai_gpt2_generate_sampled(slai_gpt2 *m, const int32_t *prompt, uint32_t n_p
                                uint32_t n_steps, float temperature, float topp, uint64_t seed, int32_t *out_tokens,
                                float *elapsed_ms);
 /* slai_llama2_prefill for GPT-2 (gpt2/cpu.rs:225-383 for a chunk of tokens; no counterpart in the reference): 32 tokens
- * per pass over the weights on the fp32 matrix cores where every layer matrix has a tiled layout
- * (slai_gpt2_prefill_supported() == 2), token by token with the same result otherwise (0). */
+ * per pass over the weights on the matrix cores where every layer matrix has a tiled layout
+ * (slai_gpt2_prefill_supported() == 2; f16 head + remainder pairs with the fp32 repeat of slai_llama2_prefill, counted by
+ * slai_gpt2_prefill_fp32_repeats), token by token with the same result otherwise (0). */
 int slai_gpt2_prefill(slai_gpt2 *m, const int32_t *tokens, uint32_t n_tokens, uint32_t start_pos, uint32_t chunk,
                       float *elapsed_ms);
 int slai_gpt2_prefill_supported(const slai_gpt2 *m);
+uint32_t slai_gpt2_prefill_fp32_repeats(const slai_gpt2 *m);
 
 /* ---- Tokenizers (host only) ---------------------------------------------------
  * `AnyTokenizer` (crates/slai-chat/src/llm.rs:100-164) over `LlamaTokenizer`

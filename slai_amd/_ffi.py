@@ -150,6 +150,7 @@ SIGNATURES = {
     "slai_llama2_prefill_fp32_repeats": (C.c_uint32, [vp]),
     "slai_gpt2_prefill": (i32, [vp, vp, u32, u32, u32, P(C.c_float)]),
     "slai_gpt2_prefill_supported": (i32, [vp]),
+    "slai_gpt2_prefill_fp32_repeats": (C.c_uint32, [vp]),
     "slai_gpt2_generate_sampled": (i32, [vp, vp, u32, u32, u32, C.c_float, C.c_float, u64, vp, P(C.c_float)]),
 }
 

@@ -912,6 +912,7 @@ struct slai_gpt2 {
     bool chunk_gemm_supported() const;
     int chunk_reserve();
     bool chunk_split_ok() const;
+    uint32_t prefill_fp32_repeats = 0;
     int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev, bool split_f16);
 };
 
@@ -1216,8 +1217,11 @@ SLAI_EXPORT int slai_gpt2_prefill(slai_gpt2 *m, const int32_t *tokens, uint32_t 
         int beyond = 0;
         SLAI_HIP_TRY(ctx, hipMemcpy(&beyond, ctx->split_flag, sizeof(int), hipMemcpyDeviceToHost));
         if (!beyond) break;
+        ++m->prefill_fp32_repeats;
         split = false;
     }
     if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, m->loop.ev0, m->loop.ev1));
     return SLAI_OK;
 }
+
+SLAI_EXPORT uint32_t slai_gpt2_prefill_fp32_repeats(const slai_gpt2 *m) { return m ? m->prefill_fp32_repeats : 0; }

@@ -168,8 +168,9 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
 
 
 def gpt2_gguf(n_embd=768, n_layer=12, n_head=12, ff_len=3072, vocab=50257, n_seq=1024, wtype=8, seed=1234,
-              std=0.02):
-    """Synthetic GPT-2-shape model file: LayerNorm g~N(1,.02), b~N(0,.02), biases N(0,.02)."""
+              std=0.02, ffn_norm_scale=1.0):
+    """Synthetic GPT-2-shape model file: LayerNorm g~N(1,.02), b~N(0,.02), biases N(0,.02); `ffn_norm_scale`: factor on
+    the ffn_norm gains (large values push the normalised rows beyond the f16 range)."""
     w = GgufWriter()
     w.add_meta("general.architecture", T_STR, "gpt2")
     w.add_meta("general.file_type", T_U32, 7)
@@ -186,8 +187,8 @@ def gpt2_gguf(n_embd=768, n_layer=12, n_head=12, ff_len=3072, vocab=50257, n_seq
         ctr[0] += 1
         return synth.normal_quantized(ctr[0], t, nrows, ncols, std)
 
-    def vec(mean, n):
-        return _f32(rng.normal(mean, 0.02, n))
+    def vec(mean, n, scale=1.0):
+        return _f32(rng.normal(mean, 0.02, n) * scale)
 
     w.add_tensor("token_embd.weight", [n_embd, vocab], wtype, qmat(vocab, n_embd, wtype))
     w.add_tensor("position_embd.weight", [n_embd, n_seq], 0, _f32(rng.normal(0.0, std, (n_seq, n_embd))))
@@ -199,7 +200,7 @@ def gpt2_gguf(n_embd=768, n_layer=12, n_head=12, ff_len=3072, vocab=50257, n_seq
         w.add_tensor(p + "attn_qkv.bias", [3 * n_embd], 0, vec(0.0, 3 * n_embd))
         w.add_tensor(p + "attn_output.weight", [n_embd, n_embd], wtype, qmat(n_embd, n_embd, wtype))
         w.add_tensor(p + "attn_output.bias", [n_embd], 0, vec(0.0, n_embd))
-        w.add_tensor(p + "ffn_norm.weight", [n_embd], 0, vec(1.0, n_embd))
+        w.add_tensor(p + "ffn_norm.weight", [n_embd], 0, vec(1.0, n_embd, ffn_norm_scale))
         w.add_tensor(p + "ffn_norm.bias", [n_embd], 0, vec(0.0, n_embd))
         w.add_tensor(p + "ffn_up.weight", [n_embd, ff_len], wtype, qmat(ff_len, n_embd, wtype))
         w.add_tensor(p + "ffn_up.bias", [ff_len], 0, vec(0.0, ff_len))

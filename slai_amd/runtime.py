@@ -550,6 +550,10 @@ class Gpt2:
         """2: matrix-core GEMM, 0: the token-by-token loop."""
         return int(self.b.L.slai_gpt2_prefill_supported(self.h))
 
+    def prefill_fp32_repeats(self):
+        """Prefill calls that were repeated with fp32 MFMA because an activation was beyond the f16 range."""
+        return int(self.b.L.slai_gpt2_prefill_fp32_repeats(self.h))
+
     def prefill(self, tokens, start_pos=0, chunk=0):
         """Fill the caches for positions start_pos .. start_pos+len(tokens)-1; returns the stream time in ms."""
         tokens = np.ascontiguousarray(tokens, dtype=np.int32)

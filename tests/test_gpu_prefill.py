@@ -301,3 +301,32 @@ def test_prefill_large_weights_take_fp32_from_the_start(backend):
                          std=40.0)
     prompt = np.random.Generator(np.random.PCG64(80)).integers(0, 500, 40).astype(np.int32)
     check_prefill(backend, data, prompt, 6, (32,), True, expect_repeats=0)
+
+
+def test_gpt2_prefill_fp32_repeat(backend):
+    """GPT-2 with ffn_norm gains of 5e4: the normalised rows do not fit the f16 heads, the call is repeated with the
+    fp32 kernels and the continuation still matches the oracle's greedy ids."""
+    import os
+    if os.environ.get("SLAI_PROMPT_SPLIT_F16") == "0" or os.environ.get("SLAI_PROMPT_GEMM") == "0":
+        pytest.skip("needs the split path")
+    from helpers import OracleGguf
+    from slai_amd.runtime import Gpt2
+    for scale, repeats in ((1.0, 0), (5.0e4, 1)):
+        data = gw.gpt2_gguf(n_layer=2, seed=53, std=0.05, ffn_norm_scale=scale)
+        g = OracleGguf(data); L = g.L
+        om = L.slo_gpt2_from_gguf(g.h, 0)
+        assert om
+        prompt = np.random.Generator(np.random.PCG64(54)).integers(0, 50257, 40).astype(np.int32)
+        n, n_gen = prompt.size, 6
+        n_steps = n - 1 + n_gen
+        ref_tokens = np.zeros(n_steps, np.int32); ref_logits = np.zeros((n_steps, 50257), np.float32)
+        assert L.slo_gpt2_generate(om, prompt.ctypes.data, n, 0, n_steps, -1, ref_tokens.ctypes.data, ref_logits.ctypes.data) == n_steps
+        gg = Gguf(data)
+        m = Gpt2(backend, gg, _ffi.KV_F32)
+        m.prefill(prompt[:-1], 0, 32)
+        assert m.prefill_fp32_repeats() == repeats, (scale, m.prefill_fp32_repeats())
+        logits = m.forward_logits(n - 1, int(prompt[-1]))
+        assert rel_err(logits, ref_logits[n - 1]) < LOGIT_TOL, scale
+        got, _ = m.generate(prompt, n_gen, start_pos=n - 1)
+        assert np.array_equal(got, ref_tokens[n - 1:]), (scale, got.tolist(), ref_tokens[n - 1:].tolist())
+        m.destroy(); gg.close(); L.slo_gpt2_free(om); g.close()
