@@ -273,6 +273,11 @@ typedef struct {
 } slai_llama2_config;   /* models/llama2/cpu.rs:46-67 */
 
 int slai_llama2_from_gguf(slai_ctx *ctx, const slai_gguf *g, int model_type, int kv_dtype, slai_llama2 **out);
+/* Host-only check of everything slai_llama2_from_gguf reads: hyper-parameters, then presence, block format and shape of
+ * every tensor against them (the kernels index norm vectors and biases by the model's widths).  Replaces the `unwrap()`s
+ * and shape asserts of `Llama2Weights::from_gguf` (transformer.rs:202-297) with an error code and message; needs no
+ * device.  slai_llama2_from_gguf runs it first and uploads nothing when it fails. */
+int slai_llama2_check_gguf(const slai_gguf *g, int model_type, char *err, size_t err_len);
 void slai_llama2_destroy(slai_llama2 *m);
 int slai_llama2_get_config(const slai_llama2 *m, slai_llama2_config *out);
 /* Bytes of packed weights resident in device memory (roofline denominator). */
@@ -319,6 +324,8 @@ int slai_llama2_logits_buffer(slai_llama2 *m, slai_buffer **logits);
 /* ---- GPT-2 model assembly (crates/slai/src/models/gpt2/cpu.rs:19-48,113-217,224-383) */
 typedef struct { uint32_t n_vocab, n_seq, n_embd, n_head, n_layer, ff_len, attn_b; } slai_gpt2_params;
 int slai_gpt2_from_gguf(slai_ctx *ctx, const slai_gguf *g, int kv_dtype, slai_gpt2 **out);
+/* The same host-only check for a GPT-2 file (`Gpt2Model::from_gguf`, gpt2/cpu.rs:118-190, unwraps instead). */
+int slai_gpt2_check_gguf(const slai_gguf *g, char *err, size_t err_len);
 void slai_gpt2_destroy(slai_gpt2 *m);
 int slai_gpt2_get_params(const slai_gpt2 *m, slai_gpt2_params *out);
 size_t slai_gpt2_weight_bytes(const slai_gpt2 *m);

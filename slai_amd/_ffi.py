@@ -131,6 +131,8 @@ SIGNATURES = {
     "slai_gguf_tensor_to_qmat": (i32, [vp, vp, C.c_char_p, P(vp)]),
     "slai_gguf_tensor_to_qmat_layout": (i32, [vp, vp, C.c_char_p, i32, P(vp)]),
     "slai_llama2_from_gguf": (i32, [vp, vp, i32, i32, P(vp)]),
+    "slai_llama2_check_gguf": (i32, [vp, i32, C.c_char_p, sz]),
+    "slai_gpt2_check_gguf": (i32, [vp, C.c_char_p, sz]),
     "slai_llama2_destroy": (None, [vp]),
     "slai_llama2_get_config": (i32, [vp, P(Llama2Config)]),
     "slai_llama2_weight_bytes": (sz, [vp]),

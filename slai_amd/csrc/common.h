@@ -63,6 +63,9 @@ struct slai_ctx {
     bool tiled_layout = true;   // SLAI_TILED=0 keeps every matrix in the row layout
     bool rowtile_gemv = true;   // SLAI_ROWTILE=0: no 64-row tiles / wave-uniform GEMV
     int attn_splits = 0;  // 0 = automatic
+    // Scratch blocks that a larger one has replaced.  Captured graphs (and launches already queued) hold the old
+    // addresses, so a block is only freed with the context.
+    std::vector<void *> retired_scratch;
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
     bool use_graph = true;  // SLAI_NO_GRAPH=1 replays the token sequence eagerly (profilers that cannot trace graph launches)
 };

@@ -27,11 +27,18 @@ const uint32_t STORAGE = SLAI_USAGE_STORAGE, UNIFORM = SLAI_USAGE_UNIFORM, COPY_
                COPY_SRC = SLAI_USAGE_COPY_SRC, MAP_READ = SLAI_USAGE_MAP_READ;
 
 // `gguf.tensors[name].data().as_f32().unwrap()` + `GpuTensor::vector` (transformer.rs:250-263)
-int f32_vector_from_gguf(slai_ctx *ctx, const Gguf &g, const std::string &name, bool required, GpuTensor *out) {
+// The kernels index these vectors by the model's widths, so a tensor of any other length is refused here, before
+// anything is launched (`expected` elements: the width the readers assume).
+int f32_vector_from_gguf(slai_ctx *ctx, const Gguf &g, const std::string &name, bool required, uint32_t expected, GpuTensor *out) {
     const GgufTensorInfo *t = g.find(name);
     if (!t) return required ? set_error(ctx, SLAI_E_MISSING, "missing tensor '" + name + "'") : SLAI_OK;
     if (t->type != 0) return set_error(ctx, SLAI_E_TYPE, "tensor '" + name + "' must be F32");
-    uint64_t n = t->dims[0] * t->dims[1] * t->dims[2] * t->dims[3];
+    uint64_t n = 1;
+    for (int d = 0; d < 4; ++d) {
+        if (t->dims[d] == 0 || t->dims[d] > UINT32_MAX || (n *= t->dims[d]) > UINT32_MAX) { n = 0; break; }
+    }
+    if (n != expected)
+        return set_error(ctx, SLAI_E_SHAPE, "tensor '" + name + "' has " + std::to_string(n) + " elements, the model needs " + std::to_string(expected));
     return GpuTensor::vector_from(ctx, reinterpret_cast<const float *>(g.bytes + t->offset), (uint32_t)n, STORAGE, out);
 }
 int qmat_from_gguf(slai_ctx *ctx, const slai_gguf *g, const std::string &name, slai_qmat **out, int layout = SLAI_LAYOUT_AUTO) {
@@ -42,6 +49,34 @@ int meta_u32(slai_ctx *ctx, const Gguf &g, const std::string &key, uint32_t *out
     if (!v) return set_error(ctx, SLAI_E_MISSING, "missing metadata key '" + key + "'");
     if (v->type != 4) return set_error(ctx, SLAI_E_TYPE, "unwrap: unexpected GGUF attribute type for '" + key + "'");
     *out = (uint32_t)v->u;
+    return SLAI_OK;
+}
+
+// Host-only shape checks of a model file, run before anything is uploaded or launched: the kernels index weights and
+// vectors by the model's widths, so a tensor of any other shape must never reach them.  `err` receives the message.
+int check_matrix(const Gguf &g, const std::string &name, bool required, uint64_t nrows, uint64_t ncols, std::string &err) {
+    const GgufTensorInfo *t = g.find(name);
+    if (!t) { if (!required) return SLAI_OK; err = "missing tensor '" + name + "'"; return SLAI_E_MISSING; }
+    const int be = block_elems((int)t->type);
+    if (!be) { err = "tensor '" + name + "' has ggml type " + std::to_string(t->type) + " which has no device kernel"; return SLAI_E_TYPE; }
+    if (t->dims[2] != 1 || t->dims[3] != 1 || t->dims[0] != nrows || t->dims[1] != ncols) {
+        err = "tensor '" + name + "' is " + std::to_string(t->dims[0]) + " x " + std::to_string(t->dims[1]) + ", the model needs " + std::to_string(nrows) + " x " + std::to_string(ncols);
+        return SLAI_E_SHAPE;
+    }
+    if (ncols % be) { err = "tensor '" + name + "': row length is not a multiple of the block length"; return SLAI_E_SHAPE; }
+    if (t->offset > g.len || gguf_row_bytes((int)t->type, (uint32_t)ncols) * nrows > g.len - t->offset) { err = "tensor '" + name + "' runs past the end of the file"; return SLAI_E_PARSE; }
+    return SLAI_OK;
+}
+int check_vector(const Gguf &g, const std::string &name, bool required, uint64_t n, std::string &err) {
+    const GgufTensorInfo *t = g.find(name);
+    if (!t) { if (!required) return SLAI_OK; err = "missing tensor '" + name + "'"; return SLAI_E_MISSING; }
+    if (t->type != 0) { err = "tensor '" + name + "' must be F32"; return SLAI_E_TYPE; }
+    uint64_t have = 1;
+    for (int d = 0; d < 4; ++d) {
+        if (t->dims[d] == 0 || t->dims[d] > UINT32_MAX || (have *= t->dims[d]) > UINT32_MAX) { have = 0; break; }
+    }
+    if (have != n) { err = "tensor '" + name + "' has " + std::to_string(have) + " elements, the model needs " + std::to_string(n); return SLAI_E_SHAPE; }
+    if (t->offset > g.len || n * 4 > g.len - t->offset) { err = "tensor '" + name + "' runs past the end of the file"; return SLAI_E_PARSE; }
     return SLAI_OK;
 }
 
@@ -173,9 +208,51 @@ static int llama2_config_from_gguf(slai_ctx *ctx, const Gguf &g, int model_type,
     return SLAI_OK;
 }
 
+// Everything `load` is going to read, checked on the host alone: hyper-parameters, then the presence, block format and
+// shape of every tensor (`Llama2Weights::from_gguf`, transformer.rs:202-297, unwraps and asserts where this returns a code).
+static int llama2_check_gguf(const Gguf &g, int model_type, slai_llama2_config *cfg, std::string &err) {
+    slai_ctx scratch_ctx;                                  // (only carries the message of the config reader)
+    if (int rc = llama2_config_from_gguf(&scratch_ctx, g, model_type, cfg)) { err = scratch_ctx.err; return rc; }
+    const slai_llama2_config &c = *cfg;
+    const uint64_t dim = c.dim, kvd = (uint64_t)c.dim * c.n_kv_heads / c.n_q_heads, hid = c.hidden_dim, hs = c.dim / c.n_q_heads;
+    if (hs % 2 || hs > 256) { err = "head size must be even and <= 256"; return SLAI_E_SHAPE; }
+    if (!hid || !c.n_layers) { err = "inconsistent model hyper-parameters"; return SLAI_E_SHAPE; }
+    for (uint32_t l = 0; l < c.n_layers; ++l) {
+        const std::string p = "blk." + std::to_string(l) + ".";
+        const struct { const char *name; bool required; uint64_t r, k; } mats[] = {
+            {"attn_q.weight", true, dim, dim}, {"attn_k.weight", true, kvd, dim}, {"attn_v.weight", true, kvd, dim}, {"attn_output.weight", true, dim, dim},
+            {"ffn_down.weight", true, dim, hid}, {"ffn_gate.weight", true, hid, dim}, {"ffn_up.weight", true, hid, dim}};
+        for (const auto &m : mats)
+            if (int rc = check_matrix(g, p + m.name, m.required, m.r, m.k, err)) return rc;
+        const struct { const char *name; bool required; uint64_t n; } vecs[] = {
+            {"attn_q.bias", false, dim}, {"attn_k.bias", false, kvd}, {"attn_v.bias", false, kvd}, {"ffn_norm.weight", true, dim}, {"attn_norm.weight", true, dim}};
+        for (const auto &v : vecs)
+            if (int rc = check_vector(g, p + v.name, v.required, v.n, err)) return rc;
+    }
+    if (int rc = check_matrix(g, "token_embd.weight", true, c.vocab_size, dim, err)) return rc;
+    if (int rc = check_matrix(g, "output.weight", false, c.vocab_size, dim, err)) return rc;
+    return check_vector(g, "output_norm.weight", true, dim, err);
+}
+
+static int copy_message(int rc, const std::string &msg, char *err, size_t err_len) {
+    if (err && err_len) { const size_t n = std::min(msg.size(), err_len - 1); memcpy(err, msg.data(), n); err[n] = 0; }
+    return rc;
+}
+
+SLAI_EXPORT int slai_llama2_check_gguf(const slai_gguf *g, int model_type, char *err, size_t err_len) {
+    if (!g || (model_type != SLAI_MODEL_LLAMA && model_type != SLAI_MODEL_QWEN2)) return copy_message(SLAI_E_ARG, "slai_llama2_check_gguf: bad argument", err, err_len);
+    slai_llama2_config cfg{};
+    std::string msg;
+    const int rc = llama2_check_gguf(g->g, model_type, &cfg, msg);
+    return copy_message(rc, msg, err, err_len);
+}
+
 int slai_llama2::load(const slai_gguf *gg) {
     const Gguf &g = gg->g;
-    TRY(llama2_config_from_gguf(ctx, g, model_type, &config));
+    {   // nothing is uploaded or launched for a file whose tensors do not fit the hyper-parameters
+        std::string msg;
+        if (int rc = llama2_check_gguf(g, model_type, &config, msg)) return set_error(ctx, rc, msg);
+    }
     const uint32_t dim = config.dim, kvd = kv_dim();
     if (head_size() % 2 || head_size() > 256) return set_error(ctx, SLAI_E_SHAPE, "head size must be even and <= 256");
     // ---- Llama2Weights::from_gguf (transformer.rs:202-297)
@@ -186,16 +263,16 @@ int slai_llama2::load(const slai_gguf *gg) {
         TRY(qmat_from_gguf(ctx, gg, p + "attn_q.weight", &w.attn_q, SLAI_LAYOUT_TILE64));
         TRY(qmat_from_gguf(ctx, gg, p + "attn_k.weight", &w.attn_k, SLAI_LAYOUT_TILE64));
         TRY(qmat_from_gguf(ctx, gg, p + "attn_v.weight", &w.attn_v, SLAI_LAYOUT_TILE64));
-        TRY(f32_vector_from_gguf(ctx, g, p + "attn_q.bias", false, &w.attn_q_bias));
-        TRY(f32_vector_from_gguf(ctx, g, p + "attn_k.bias", false, &w.attn_k_bias));
-        TRY(f32_vector_from_gguf(ctx, g, p + "attn_v.bias", false, &w.attn_v_bias));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_q.bias", false, dim, &w.attn_q_bias));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_k.bias", false, kvd, &w.attn_k_bias));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_v.bias", false, kvd, &w.attn_v_bias));
         TRY(qmat_from_gguf(ctx, gg, p + "attn_output.weight", &w.attn_output));
         // (explicit 16-row tiles: a feed-forward width beyond 16384 then still gets the tiled layout, in column slices)
         TRY(qmat_from_gguf(ctx, gg, p + "ffn_down.weight", &w.ffn_down, SLAI_LAYOUT_TILE16));
         TRY(qmat_from_gguf(ctx, gg, p + "ffn_gate.weight", &w.ffn_gate, SLAI_LAYOUT_TILE64));
         TRY(qmat_from_gguf(ctx, gg, p + "ffn_up.weight", &w.ffn_up, SLAI_LAYOUT_TILE64));
-        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.weight", true, &w.ffn_norm));
-        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.weight", true, &w.attn_norm));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.weight", true, dim, &w.ffn_norm));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.weight", true, dim, &w.attn_norm));
         struct { slai_qmat *m; uint32_t r, c; } chk[] = {{w.attn_q, dim, dim}, {w.attn_k, kvd, dim}, {w.attn_v, kvd, dim},
             {w.attn_output, dim, dim}, {w.ffn_down, dim, config.hidden_dim}, {w.ffn_gate, config.hidden_dim, dim}, {w.ffn_up, config.hidden_dim, dim}};
         for (auto &c : chk)
@@ -206,7 +283,7 @@ int slai_llama2::load(const slai_gguf *gg) {
     TRY(qmat_from_gguf(ctx, gg, "token_embd.weight", &weights.token_embd, SLAI_LAYOUT_TILE64));
     if (g.find("output.weight")) TRY(qmat_from_gguf(ctx, gg, "output.weight", &weights.output, SLAI_LAYOUT_TILE64));
     else weights.output = weights.token_embd;                                       // transformer.rs:279-285
-    TRY(f32_vector_from_gguf(ctx, g, "output_norm.weight", true, &weights.output_norm));
+    TRY(f32_vector_from_gguf(ctx, g, "output_norm.weight", true, dim, &weights.output_norm));
     if (weights.token_embd->nrows != config.vocab_size || weights.token_embd->ncols != dim || weights.output->nrows != config.vocab_size ||
         weights.output->ncols != dim)
         return set_error(ctx, SLAI_E_SHAPE, "embedding / output shape does not match the config");
@@ -916,9 +993,9 @@ struct slai_gpt2 {
     int enqueue_chunk_gemm(uint32_t pos0, uint32_t n, const int *tokens_dev, bool split_f16);
 };
 
-int slai_gpt2::load(const slai_gguf *gg) {
-    const Gguf &g = gg->g;
-    // Gpt2Params::from_gguf (gpt2/cpu.rs:37-48)
+// Gpt2Params::from_gguf (gpt2/cpu.rs:37-48)
+static int gpt2_params_from_gguf(slai_ctx *ctx, const Gguf &g, slai_gpt2_params *out) {
+    slai_gpt2_params &params = *out;
     const GgufMetaValue *tok = g.meta("tokenizer.ggml.tokens");
     if (!tok) return set_error(ctx, SLAI_E_MISSING, "missing metadata key 'tokenizer.ggml.tokens'");
     if (tok->type != 9) return set_error(ctx, SLAI_E_TYPE, "unwrap: unexpected GGUF attribute type for 'tokenizer.ggml.tokens'");
@@ -932,24 +1009,69 @@ int slai_gpt2::load(const slai_gguf *gg) {
     // (gpt2/cpu.rs:46 + gguf.rs:581); the forward needs 3*n_embd (:252-270).
     params.attn_b = 3 * params.n_embd;
     const uint32_t E = params.n_embd;
-    if (!E || !params.n_head || E % params.n_head || (E / params.n_head) % 2 || E / params.n_head > 256) return set_error(ctx, SLAI_E_SHAPE, "inconsistent GPT-2 hyper-parameters");
+    if (!E || !params.n_head || E % params.n_head || (E / params.n_head) % 2 || E / params.n_head > 256 || !params.ff_len || !params.n_seq || !params.n_vocab)
+        return set_error(ctx, SLAI_E_SHAPE, "inconsistent GPT-2 hyper-parameters");
+    return SLAI_OK;
+}
+
+// The host-only check of a GPT-2 file (see llama2_check_gguf): gpt2/cpu.rs:118-190 unwraps where this returns a code.
+static int gpt2_check_gguf(const Gguf &g, slai_gpt2_params *params, std::string &err) {
+    slai_ctx scratch_ctx;
+    if (int rc = gpt2_params_from_gguf(&scratch_ctx, g, params)) { err = scratch_ctx.err; return rc; }
+    const uint64_t E = params->n_embd, F = params->ff_len;
+    for (uint32_t l = 0; l < params->n_layer; ++l) {
+        const std::string p = "blk." + std::to_string(l) + ".";
+        const struct { const char *name; uint64_t r, k; } mats[] = {
+            {"attn_qkv.weight", 3 * E, E}, {"attn_output.weight", E, E}, {"ffn_up.weight", F, E}, {"ffn_down.weight", E, F}};
+        for (const auto &m : mats)
+            if (int rc = check_matrix(g, p + m.name, true, m.r, m.k, err)) return rc;
+        const struct { const char *name; uint64_t n; } vecs[] = {
+            {"attn_norm.weight", E}, {"attn_norm.bias", E}, {"ffn_norm.weight", E}, {"ffn_norm.bias", E}, {"attn_qkv.bias", 3 * E},
+            {"attn_output.bias", E}, {"ffn_up.bias", F}, {"ffn_down.bias", E}};
+        for (const auto &v : vecs)
+            if (int rc = check_vector(g, p + v.name, true, v.n, err)) return rc;
+    }
+    if (int rc = check_vector(g, "output_norm.weight", true, E, err)) return rc;
+    if (int rc = check_vector(g, "output_norm.bias", true, E, err)) return rc;
+    if (int rc = check_matrix(g, "token_embd.weight", true, params->n_vocab, E, err)) return rc;
+    const GgufTensorInfo *wpe = g.find("position_embd.weight");
+    if (!wpe) { err = "missing tensor 'position_embd.weight'"; return SLAI_E_MISSING; }
+    if (wpe->dims[0] < params->n_seq) { err = "embedding shapes do not match the parameters"; return SLAI_E_SHAPE; }
+    return check_matrix(g, "position_embd.weight", true, wpe->dims[0], E, err);
+}
+
+SLAI_EXPORT int slai_gpt2_check_gguf(const slai_gguf *g, char *err, size_t err_len) {
+    if (!g) return copy_message(SLAI_E_ARG, "slai_gpt2_check_gguf: bad argument", err, err_len);
+    slai_gpt2_params params{};
+    std::string msg;
+    const int rc = gpt2_check_gguf(g->g, &params, msg);
+    return copy_message(rc, msg, err, err_len);
+}
+
+int slai_gpt2::load(const slai_gguf *gg) {
+    const Gguf &g = gg->g;
+    {
+        std::string msg;
+        if (int rc = gpt2_check_gguf(g, &params, msg)) return set_error(ctx, rc, msg);
+    }
+    const uint32_t E = params.n_embd;
     const int cdt = kv_dtype == SLAI_KV_F16 ? SLAI_DT_F16 : SLAI_DT_F32;
     layers.resize(params.n_layer);
     for (uint32_t l = 0; l < params.n_layer; ++l) {       // gpt2/cpu.rs:118-179
         Gpt2Layer &w = layers[l];
         const std::string p = "blk." + std::to_string(l) + ".";
-        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.weight", true, &w.ln_1_g));
-        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.bias", true, &w.ln_1_b));
-        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.weight", true, &w.ln_2_g));
-        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.bias", true, &w.ln_2_b));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.weight", true, E, &w.ln_1_g));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_norm.bias", true, E, &w.ln_1_b));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.weight", true, E, &w.ln_2_g));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_norm.bias", true, E, &w.ln_2_b));
         TRY(qmat_from_gguf(ctx, gg, p + "attn_qkv.weight", &w.c_attn_attn_w));
-        TRY(f32_vector_from_gguf(ctx, g, p + "attn_qkv.bias", true, &w.c_attn_attn_b));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_qkv.bias", true, 3 * E, &w.c_attn_attn_b));
         TRY(qmat_from_gguf(ctx, gg, p + "attn_output.weight", &w.c_attn_proj_w));
-        TRY(f32_vector_from_gguf(ctx, g, p + "attn_output.bias", true, &w.c_attn_proj_b));
+        TRY(f32_vector_from_gguf(ctx, g, p + "attn_output.bias", true, E, &w.c_attn_proj_b));
         TRY(qmat_from_gguf(ctx, gg, p + "ffn_up.weight", &w.c_mlp_fc_w));
-        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_up.bias", true, &w.c_mlp_fc_b));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_up.bias", true, params.ff_len, &w.c_mlp_fc_b));
         TRY(qmat_from_gguf(ctx, gg, p + "ffn_down.weight", &w.c_mlp_proj_w));
-        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_down.bias", true, &w.c_mlp_proj_b));
+        TRY(f32_vector_from_gguf(ctx, g, p + "ffn_down.bias", true, E, &w.c_mlp_proj_b));
         struct { slai_qmat *m; uint32_t r, c; } chk[] = {{w.c_attn_attn_w, 3 * E, E}, {w.c_attn_proj_w, E, E}, {w.c_mlp_fc_w, params.ff_len, E}, {w.c_mlp_proj_w, E, params.ff_len}};
         for (auto &c : chk)
             if (c.m->nrows != c.r || c.m->ncols != c.c) return set_error(ctx, SLAI_E_SHAPE, "layer " + std::to_string(l) + ": weight shape does not match the parameters");
@@ -962,8 +1084,8 @@ int slai_gpt2::load(const slai_gguf *gg) {
         }
         weight_bytes += (size_t)(4 * E + 3 * E + E + params.ff_len + E) * 4;
     }
-    TRY(f32_vector_from_gguf(ctx, g, "output_norm.weight", true, &ln_f_g));
-    TRY(f32_vector_from_gguf(ctx, g, "output_norm.bias", true, &ln_f_b));
+    TRY(f32_vector_from_gguf(ctx, g, "output_norm.weight", true, E, &ln_f_g));
+    TRY(f32_vector_from_gguf(ctx, g, "output_norm.bias", true, E, &ln_f_b));
     TRY(qmat_from_gguf(ctx, gg, "token_embd.weight", &wte));
     TRY(qmat_from_gguf(ctx, gg, "position_embd.weight", &wpe));
     if (gemv_is_rowtile(ctx, wte)) TRY(gemv_scratch_reserve(ctx, (size_t)((wte->nrows + 63) / 64) * (wte->ncols + wte->ncols / 16)));

@@ -102,6 +102,7 @@ SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     if (ctx->split_flag) (void)hipFree(ctx->split_flag);
     if (ctx->sampler_scratch) (void)hipFree(ctx->sampler_scratch);
     if (ctx->handoff_counters) (void)hipFree(ctx->handoff_counters);
+    for (void *p : ctx->retired_scratch) (void)hipFree(p);
     if (ctx->timer0) (void)hipEventDestroy(ctx->timer0);
     if (ctx->timer1) (void)hipEventDestroy(ctx->timer1);
     (void)hipStreamDestroy(ctx->stream);
@@ -318,15 +319,22 @@ bool gemv_gated_is_rowtile(const slai_ctx *ctx, const slai_qmat *gate, const sla
     return gemv_is_rowtile(ctx, gate) && gemv_is_rowtile(ctx, up) && gate->type == up->type && gate->type != T_Q8_0;
 }
 
-int gemv_scratch_reserve(slai_ctx *ctx, size_t floats) {
-    if (floats <= ctx->gemv_scratch_floats) return SLAI_OK;
-    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "GEMV scratch must be reserved before graph capture");
-    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->gemv_scratch) (void)hipFree(ctx->gemv_scratch);
-    ctx->gemv_scratch = nullptr; ctx->gemv_scratch_floats = 0;
-    SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->gemv_scratch, floats * sizeof(float)));
-    ctx->gemv_scratch_floats = floats;
+// Grows one of the context's scratch blocks.  The block it replaces stays allocated until the context goes: graphs
+// captured earlier (a model's decode graph) and launches already queued keep using the old address, which still holds
+// as much as they were built for.  Growth is at least twofold, so the retired blocks together stay below the live one.
+int scratch_grow(slai_ctx *ctx, float **block, size_t *have, size_t floats, const char *what) {
+    if (floats <= *have) return SLAI_OK;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, std::string(what) + " must be reserved before graph capture");
+    floats = std::max(floats, 2 * *have);
+    float *fresh = nullptr;
+    SLAI_HIP_TRY(ctx, hipMalloc((void **)&fresh, floats * sizeof(float)));
+    if (*block) ctx->retired_scratch.push_back(*block);
+    *block = fresh; *have = floats;
     return SLAI_OK;
+}
+
+int gemv_scratch_reserve(slai_ctx *ctx, size_t floats) {
+    return scratch_grow(ctx, &ctx->gemv_scratch, &ctx->gemv_scratch_floats, floats, "GEMV scratch");
 }
 
 bool qkv_attention_fusable(const slai_ctx *ctx, const slai_qmat *v, const slai_qmat *k, const slai_qmat *q, const AttnLaunch &a) {
@@ -363,19 +371,16 @@ int handoff_check(slai_ctx *ctx) {
     if (!ctx->handoff_counters) return SLAI_OK;
     uint32_t flag = 0;
     SLAI_HIP_TRY(ctx, hipMemcpy(&flag, ctx->handoff_counters + (size_t)ctx->handoff_heads * 32, sizeof flag, hipMemcpyDeviceToHost));
-    if (flag) return set_error(ctx, SLAI_E_HIP, "q/k/v -> attention hand-off timed out inside a launch; results are invalid");
+    if (flag) {
+        // reported once: the slot is cleared so that later, healthy calls are not failed for an old time-out
+        (void)hipMemset(ctx->handoff_counters + (size_t)ctx->handoff_heads * 32, 0, sizeof flag);
+        return set_error(ctx, SLAI_E_HIP, "q/k/v -> attention hand-off timed out inside a launch; results are invalid");
+    }
     return SLAI_OK;
 }
 
 int sampler_scratch_reserve(slai_ctx *ctx, size_t floats) {
-    if (floats <= ctx->sampler_scratch_floats) return SLAI_OK;
-    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "sampler scratch must be reserved before graph capture");
-    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->sampler_scratch) (void)hipFree(ctx->sampler_scratch);
-    ctx->sampler_scratch = nullptr; ctx->sampler_scratch_floats = 0;
-    SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->sampler_scratch, floats * sizeof(float)));
-    ctx->sampler_scratch_floats = floats;
-    return SLAI_OK;
+    return scratch_grow(ctx, &ctx->sampler_scratch, &ctx->sampler_scratch_floats, floats, "sampler scratch");
 }
 
 int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunch *fused_attn) {
@@ -704,14 +709,7 @@ uint32_t pick_attn_splits(const slai_ctx *ctx, uint32_t n_heads, uint32_t seq_le
     return s ? s : 1;
 }
 int ensure_attn_scratch(slai_ctx *ctx, size_t floats) {
-    if (floats <= ctx->attn_scratch_floats) return SLAI_OK;
-    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "attention scratch must be sized before graph capture");
-    SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
-    ctx->attn_scratch = nullptr; ctx->attn_scratch_floats = 0;
-    SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->attn_scratch, floats * sizeof(float)));
-    ctx->attn_scratch_floats = floats;
-    return SLAI_OK;
+    return scratch_grow(ctx, &ctx->attn_scratch, &ctx->attn_scratch_floats, floats, "attention scratch");
 }
 }  // namespace slai
 

@@ -29,6 +29,7 @@ class GgufWriter:
         self.alignment = alignment
         self.meta = []      # (key, type, payload-bytes)
         self.tensors = []   # (name, dims(ne order), ggml_type, data: np.uint8 array)
+        self.tensor_hook = None   # optional f(name, ne_dims, ggml_type, data) -> (ne_dims, ggml_type, data) or None to drop
 
     def add_meta(self, key, vtype, value, elem_type=None):
         if vtype == T_STR:
@@ -46,6 +47,11 @@ class GgufWriter:
     def add_tensor(self, name, ne_dims, ggml_type, data):
         """ne_dims: GGUF order (ne0 = ncols first).  data: bytes-like of packed blocks."""
         data = np.frombuffer(data, dtype=np.uint8) if not isinstance(data, np.ndarray) else data.view(np.uint8).reshape(-1)
+        if self.tensor_hook is not None:
+            r = self.tensor_hook(name, list(ne_dims), ggml_type, data)
+            if r is None:
+                return
+            ne_dims, ggml_type, data = r
         self.tensors.append((name, list(ne_dims), ggml_type, data))
 
     def to_bytes(self):
@@ -94,7 +100,7 @@ def _f32(a):
 def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, wtype, seed=1234,
                std=0.02, rope_base=10000.0, rms_eps=1e-5, out_type=None, v_type=None, embd_type=None,
                with_output=True, arch="llama", bias=False, norm_random=False, distinct_layers=None, tokenizer=None,
-               ffn_norm_scale=1.0):
+               ffn_norm_scale=1.0, tensor_hook=None):
     """Synthetic Llama-2-shape model file (uint8 numpy array).
 
     Weights are seeded std*N(0,1) quantized to `wtype` (`v_type` for attn_v, `out_type` for
@@ -105,12 +111,14 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
     `ffn_norm_scale`: factor on the ffn_norm weights (large values push the normalised rows beyond the f16 range).
     `tokenizer`: optional dict(model=, tokens=, scores=|merges=, bos=, eos=, unk=, chat_template=) written as the
     tokenizer.* metadata a chat front end reads; `vocab` must then equal len(tokens).
+    `tensor_hook`: see GgufWriter.tensor_hook (tests use it to write malformed files).
     """
     out_type = wtype if out_type is None else out_type
     v_type = wtype if v_type is None else v_type
     embd_type = wtype if embd_type is None else embd_type
     kv_dim = dim * n_kv_heads // n_heads
     w = GgufWriter()
+    w.tensor_hook = tensor_hook
     w.add_meta("general.architecture", T_STR, arch)
     w.add_meta("general.alignment", T_U32, 32)
     w.add_meta(arch + ".embedding_length", T_U32, dim)
@@ -168,10 +176,11 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
 
 
 def gpt2_gguf(n_embd=768, n_layer=12, n_head=12, ff_len=3072, vocab=50257, n_seq=1024, wtype=8, seed=1234,
-              std=0.02, ffn_norm_scale=1.0):
+              std=0.02, ffn_norm_scale=1.0, tensor_hook=None):
     """Synthetic GPT-2-shape model file: LayerNorm g~N(1,.02), b~N(0,.02), biases N(0,.02); `ffn_norm_scale`: factor on
     the ffn_norm gains (large values push the normalised rows beyond the f16 range)."""
     w = GgufWriter()
+    w.tensor_hook = tensor_hook
     w.add_meta("general.architecture", T_STR, "gpt2")
     w.add_meta("general.file_type", T_U32, 7)
     w.add_meta("gpt2.context_length", T_U32, n_seq)

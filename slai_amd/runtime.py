@@ -374,6 +374,19 @@ class Gguf:
         m.nrows, m.ncols, m.ggml_type = m.shape()
         return m
 
+    def check_llama2(self, model_type=_ffi.MODEL_LLAMA):
+        """Host-only check of every tensor a Llama-2 / Qwen2 load would read; raises SlaiError on the first mismatch."""
+        err = C.create_string_buffer(512)
+        rc = self.L.slai_llama2_check_gguf(self.h, model_type, err, 512)
+        if rc:
+            raise SlaiError(rc, err.value.decode(errors="replace"))
+
+    def check_gpt2(self):
+        err = C.create_string_buffer(512)
+        rc = self.L.slai_gpt2_check_gguf(self.h, err, 512)
+        if rc:
+            raise SlaiError(rc, err.value.decode(errors="replace"))
+
     def close(self):
         if self.h:
             self.L.slai_gguf_free(self.h)

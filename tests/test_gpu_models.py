@@ -187,3 +187,68 @@ def test_llama_context_beyond_1024_uses_split_attention(backend, kv_f16):
     data = gw.llama_gguf(dim=256, hidden_dim=512, n_layers=2, n_heads=2, n_kv_heads=2, vocab=512, seq_len=1280, wtype=12, seed=21,
                          std=0.08, norm_random=True)
     check_llama(backend, data, [5, 100, 511, 9, 77, 3, 8, 1], 1100, kv_f16=kv_f16, check_logit_steps=6)
+
+
+def test_model_load_refuses_vectors_of_the_wrong_length(backend):
+    """A file whose norm vector or bias is shorter than the model's width is refused by the load itself (E_SHAPE), with
+    nothing uploaded or launched: the fused kernels would otherwise read past the allocation."""
+    from slai_amd.runtime import Gguf, Gpt2, Llama2, SlaiError
+
+    def short(target, n):
+        return lambda name, d, t, x: ([n], t, x[:4 * n]) if name == target else (d, t, x)
+    for target, n in (("blk.1.attn_norm.weight", 100), ("blk.0.attn_k.bias", 64), ("output_norm.weight", 8)):
+        g = Gguf(gw.llama_gguf(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab=64, seq_len=16, wtype=8, seed=5,
+                               bias=True, tensor_hook=short(target, n)))
+        with pytest.raises(SlaiError) as e:
+            Llama2(backend, g)
+        assert e.value.code == _ffi.E_SHAPE and target in str(e.value)
+        g.close()
+    g = Gguf(gw.gpt2_gguf(n_embd=64, n_layer=2, n_head=2, ff_len=128, vocab=50, n_seq=16, tensor_hook=short("blk.1.ffn_up.bias", 64)))
+    with pytest.raises(SlaiError) as e:
+        Gpt2(backend, g)
+    assert e.value.code == _ffi.E_SHAPE
+    g.close()
+
+
+def test_small_model_keeps_working_after_the_context_scratch_grew():
+    """The decode graph of a model holds the addresses of the context's scratch blocks.  A second, larger model, a long
+    slai_attention call, a wide slai_matmul_quant_columns and a sampler over a larger vocabulary all make those blocks
+    grow; the first model's graph must go on reading and writing valid memory and produce the oracle's tokens."""
+    from slai_amd.runtime import Backend, Gguf, GpuQuantMatrix, GpuTensor, Llama2, LlmContext
+    from slai_amd import synth
+    b = Backend(0)
+    try:
+        # a context of 1280 positions: the small model's graph uses the split attention kernel and its scratch
+        small = gw.llama_gguf(dim=256, hidden_dim=512, n_layers=2, n_heads=2, n_kv_heads=2, vocab=512, seq_len=1280, wtype=12, seed=21,
+                              std=0.08, norm_random=True)
+        prompt = np.array([5, 100, 511, 9], np.int32)
+        n = 24
+        og, om = oracle_llama(small, 1, 0, 1)
+        ref = np.zeros(n, np.int32)
+        assert og.L.slo_llama2_generate(om, prompt.ctypes.data, prompt.size, 0, n, -1, ref.ctypes.data, None) == n
+        g1 = Gguf(small)
+        m1 = Llama2(b, g1, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+        got, _ = m1.generate(prompt, n)                                   # captures the graph
+        assert np.array_equal(got, ref)
+        # now everything that grows the context's scratch blocks
+        big = gw.llama_gguf(dim=1024, hidden_dim=2816, n_layers=1, n_heads=8, n_kv_heads=8, vocab=40000, seq_len=4096, wtype=12, seed=22)
+        g2 = Gguf(big)
+        m2 = Llama2(b, g2, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+        m2.generate(np.array([1, 2, 3], np.int32), 4)
+        m2.generate_sampled(np.array([1, 2, 3], np.int32), 4, 0.7, 0.95, 1)
+        ctxt = LlmContext(b)
+        w = GpuQuantMatrix(b, 12, 64, 8192, synth.normal_quantized(3, 12, 64, 8192, 0.02), layout=_ffi.LAYOUT_TILE16)
+        x = GpuTensor.matrix(b, np.ones((8192, 32), np.float32))
+        out = GpuTensor(b, 64, 32)
+        ctxt.matmul_quant_columns(out, w, x)
+        b.synchronize()
+        got, _ = m1.generate(prompt, n)                                   # replays the graph captured before
+        assert np.array_equal(got, ref)
+        got, _ = m1.generate_sampled(prompt, n, 0.0, 1.0, 7)              # and a graph captured afterwards
+        assert np.array_equal(got, ref)
+        for t in (w, x, out):
+            t.destroy()
+        m2.destroy(); g2.close(); m1.destroy(); g1.close()
+        og.L.slo_llama2_free(om); og.close()
+    finally:
+        b.close()
