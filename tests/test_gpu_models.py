@@ -252,3 +252,46 @@ def test_small_model_keeps_working_after_the_context_scratch_grew():
         og.L.slo_llama2_free(om); og.close()
     finally:
         b.close()
+
+
+def test_device_against_the_transformers_library_directly(backend):
+    """The device path against an implementation that shares nothing with this repository: tiny seeded
+    LlamaForCausalLM (grouped-query attention, rows permuted to adjacent-pair order), Qwen2ForCausalLM (biases, NeoX
+    pairs) and GPT2LMHeadModel from the `transformers` library in fp32 on the CPU, exported as F32 GGUF tensors.  Logits
+    within 1e-4 of the library's at every step, greedy ids identical."""
+    hf = pytest.importorskip("test_oracle_models_hf")
+    from slai_amd.runtime import Gguf, Gpt2, Llama2
+    prompt = hf.PROMPT
+    n = len(prompt) - 1 + 24
+
+    def run(model, tok0):
+        got_logits, got_ids = [], []
+        tok = tok0
+        for pos in range(n):
+            lg = model.forward_logits(pos, tok)
+            got_logits.append(lg)
+            tok = int(prompt[pos + 1]) if pos < len(prompt) - 1 else int(np.argmax(lg))
+            got_ids.append(tok)
+        return np.stack(got_logits), np.array(got_ids, np.int32)
+
+    cases = []
+    m = hf.llama_model(202, 2, 500000.0, 1e-6)
+    cases.append(("llama gqa", m, hf.llama_family_gguf(m, "llama", permute=True), _ffi.MODEL_LLAMA))
+    cfg = hf.transformers.Qwen2Config(hidden_size=64, intermediate_size=176, num_hidden_layers=3, num_attention_heads=4, num_key_value_heads=2,
+                                      vocab_size=160, max_position_embeddings=64, rms_norm_eps=1e-6,
+                                      rope_parameters={"rope_type": "default", "rope_theta": 1000000.0}, tie_word_embeddings=False,
+                                      use_sliding_window=False, attn_implementation="eager")
+    q = hf.transformers.Qwen2ForCausalLM(cfg).eval()
+    hf.seeded_weights(q, 204)
+    cases.append(("qwen2", q, hf.llama_family_gguf(q, "qwen2", permute=False), _ffi.MODEL_QWEN2))
+    for what, model, data, mtype in cases:
+        lib_logits, lib_ids = hf.library_run(model, prompt, n)
+        gg = Gguf(data)
+        for kv in (_ffi.KV_F32,):
+            dm = Llama2(backend, gg, mtype, kv)
+            got_logits, got_ids = run(dm, int(prompt[0]))
+            hf.compare(lib_logits, lib_ids, got_logits, got_ids, what + " on the device")
+            ids, _ = dm.generate(np.array(prompt, np.int32), n)
+            assert np.array_equal(ids, lib_ids), what
+            dm.destroy()
+        gg.close()

@@ -58,7 +58,8 @@ def test_dequantize_f16_specials(backend, oracle_lib):
     m.destroy()
 
 
-GEMV_SHAPES = [(64, 256), (37, 768), (8, 11008), (1027, 4096), (4096, 4096)]
+# (the last three are the benchmark's GEMV sweep shapes and the down-projection shape of the 7B layer)
+GEMV_SHAPES = [(64, 256), (37, 768), (8, 11008), (1027, 4096), (4096, 4096), (11008, 4096), (4096, 11008)]
 
 
 @pytest.mark.parametrize("t", TYPES, ids=lambda t: NAMES[t])
