@@ -169,6 +169,14 @@ int slai_softmax_cols(slai_ctx *ctx, slai_view in_out_mat);
  * accepted for signature parity and not written. */
 int slai_attention(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q,
                    slai_view key_cache, slai_view value_cache, slai_view att, slai_view xb);
+/* slai_attention without any allocation.  It has no counterpart in the reference: it is for callers that cannot call
+ * hipMalloc -- code under HIP graph capture, tight serving loops, harnesses that forbid allocation.  Same arguments,
+ * kernels and results as slai_attention; the per-split partial results live in a static device array of
+ * 524288 floats (2 MiB, held by every GPU the library runs on until the process ends), so n_heads * splits *
+ * (head_size + 2) must not exceed that (SLAI_E_SHAPE otherwise; 32 heads of 128 at any context need 66560).  All calls on
+ * one GPU share the array: calls that overlap in time on one GPU race. */
+int slai_attention_static(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q,
+                          slai_view key_cache, slai_view value_cache, slai_view att, slai_view xb);
 /* `Sampler::sample_argmax` (crates/slai/src/models/sampler.rs:55-57; first strict maximum),
  * on the device; out_index is a 1-element I32 buffer. */
 int slai_argmax(slai_ctx *ctx, slai_view logits, slai_buffer *out_index);

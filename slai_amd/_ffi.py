@@ -92,6 +92,7 @@ SIGNATURES = {
     "slai_attn_mask": (i32, [vp, P(AttnParams), vp, vp]),
     "slai_softmax_cols": (i32, [vp, View]),
     "slai_attention": (i32, [vp, P(AttnParams), vp, View, View, View, View, View]),
+    "slai_attention_static": (i32, [vp, P(AttnParams), vp, View, View, View, View, View]),
     "slai_argmax": (i32, [vp, View, vp]),
     "slai_sample": (i32, [vp, View, C.c_float, C.c_float, C.c_float, vp]),
     "slai_sampler_coin": (C.c_float, [u64, u32]),

@@ -356,5 +356,11 @@ hipError_t launch_qkv_attention(slai_ctx *ctx, GemvRowtileParams p, const AttnLa
 // out[i] = powf(base, -((2*i) % head_size) / head_size), i < head_size/2
 hipError_t launch_rope_theta(hipStream_t s, float *out, uint32_t head_size, float base);
 size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n_splits);
+// slai_attention's argument checks; fills the launch except for the scratch block (allocates nothing)
+int attention_describe(slai_ctx *ctx, const char *fn, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q, slai_view key_cache,
+                       slai_view value_cache, slai_view xb, AttnLaunch *out);
+// Looks up, once per device and with that device current, where this device keeps the static scratch array of
+// slai_attention_static (called by slai_ctx_create).
+hipError_t attention_static_setup(int device);
 
 }  // namespace slai

@@ -18,6 +18,13 @@
 #include "attention_fast.h"
 #include "quant_formats.h"
 #include <float.h>
+#include <mutex>
+
+// Scratch of slai_attention_static (the entry point that allocates nothing): the per-split partial results of the
+// split attention kernel.  Every GPU the library runs on holds its own copy of the array, at its own address, until the
+// process ends; in host code the name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t SLAI_ATTENTION_STATIC_FLOATS = 512 * 1024;     // 2 MiB
+static __device__ __align__(256) float scratch[SLAI_ATTENTION_STATIC_FLOATS];
 
 namespace slai {
 namespace {
@@ -296,6 +303,24 @@ hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
     return e;
 }
 
+namespace {
+constexpr int STATIC_MAX_DEVICES = 64;
+float *static_scratch_ptr[STATIC_MAX_DEVICES];      // device d's address of `scratch`; set by attention_static_setup
+std::mutex static_scratch_mutex;
+}  // namespace
+
+hipError_t attention_static_setup(int device) {
+    if (device < 0 || device >= STATIC_MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(static_scratch_mutex);
+    if (static_scratch_ptr[device]) return hipSuccess;
+    float *ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!ptr) return hipErrorInvalidSymbol;
+    static_scratch_ptr[device] = ptr;
+    return hipSuccess;
+}
+
 hipError_t launch_attention_batch(hipStream_t s, const AttnLaunch &a, uint32_t n, uint32_t q_stride, uint32_t out_stride, bool out_quads, int *split_flag) {
     if ((a.head_size != 64 && a.head_size != 128) || a.kv_dim % 8 || a.knew || a.vnew || n == 0 || n > 65535 || (out_quads && n > 32)) return hipErrorInvalidValue;
     const uint32_t oq = out_quads ? 1u : 0u;
@@ -320,3 +345,26 @@ hipError_t launch_rope_store_batch(hipStream_t s, const AttnLaunch &a, float *q,
 }
 
 }  // namespace slai
+
+// slai_attention for callers that must not allocate (code under graph capture, tight serving loops): the same kernels
+// with the split partials in this device's copy of the static array.  No hipMalloc / hipFree on any path; shapes whose
+// partials do not fit are refused.  Calls on one GPU share the array, so calls that overlap in time (two contexts, two
+// streams) race; nothing in it has to start at zero: every partial the combine pass reads is written by the same call.
+SLAI_EXPORT int slai_attention_static(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q,
+                                      slai_view key_cache, slai_view value_cache, slai_view att, slai_view xb) {
+    using namespace slai;
+    (void)att;
+    AttnLaunch a{};
+    if (int rc = attention_describe(ctx, "slai_attention_static", params, params_gpu, q, key_cache, value_cache, xb, &a)) return rc;
+    const size_t need = attention_scratch_floats(a.n_heads, a.head_size, a.n_splits);
+    if (need > SLAI_ATTENTION_STATIC_FLOATS)
+        return set_error(ctx, SLAI_E_SHAPE, "slai_attention_static: n_heads * splits * (head_size + 2) = " + std::to_string(need) + " floats of partial results exceed the static scratch of " +
+                                            std::to_string(SLAI_ATTENTION_STATIC_FLOATS) + " floats; use slai_attention");
+    float *ptr = ctx->device >= 0 && ctx->device < STATIC_MAX_DEVICES ? static_scratch_ptr[ctx->device] : nullptr;
+    if (!ptr) return set_error(ctx, SLAI_E_STATE, "slai_attention_static: the static scratch of this device was not set up");
+    a.scratch = ptr;
+    hipError_t e = launch_attention(ctx->stream, a);
+    if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "slai_attention_static: unsupported head size or context length");
+    SLAI_HIP_TRY(ctx, e);
+    return SLAI_OK;
+}

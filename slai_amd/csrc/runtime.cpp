@@ -73,6 +73,7 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) return SLAI_E_HIP;
     if (hipSetDevice(device) != hipSuccess) return SLAI_E_HIP;
+    if (attention_static_setup(device) != hipSuccess) return SLAI_E_HIP;   // (this device's address of the static attention scratch)
     slai_ctx *ctx = new slai_ctx();
     ctx->device = device;
     if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) { delete ctx; return SLAI_E_HIP; }
@@ -713,23 +714,27 @@ int ensure_attn_scratch(slai_ctx *ctx, size_t floats) {
 }
 }  // namespace slai
 
-SLAI_EXPORT int slai_attention(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q,
-                               slai_view key_cache, slai_view value_cache, slai_view att, slai_view xb) {
-    (void)att;
+namespace slai {
+// Checks the arguments of slai_attention and fills everything of the launch but the scratch block and the number of
+// splits' buffer; allocates nothing.
+int attention_describe(slai_ctx *ctx, const char *fn, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q, slai_view key_cache,
+                       slai_view value_cache, slai_view xb, AttnLaunch *out) {
     if (!ctx || !params || !params_gpu || !key_cache.buf || !value_cache.buf) return SLAI_E_ARG;
-    if (params_gpu->bytes < sizeof(slai_attn_params)) return set_error(ctx, SLAI_E_SHAPE, "slai_attention: params buffer too small");
-    NEED_VEC(q, "q", vq); NEED_VEC(xb, "xb", vx);
+    if (params_gpu->bytes < sizeof(slai_attn_params)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": params buffer too small");
+    VecView vq, vx;
+    if (!as_vec(q, &vq)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": bad view 'q'");
+    if (!as_vec(xb, &vx)) return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": bad view 'xb'");
     const uint32_t hs = params->head_size, nh = params->n_heads;
     if (!params->kv_mul || nh % params->kv_mul || vq.n != nh * hs || vx.n != nh * hs || vq.stride != 1 || vx.stride != 1 ||
         params->kv_dim != nh / params->kv_mul * hs || params->pos >= params->seq_len)
-        return set_error(ctx, SLAI_E_SHAPE, "slai_attention: inconsistent parameters");
+        return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": inconsistent parameters");
     const int kdt = key_cache.buf->dtype;
-    if (kdt != value_cache.buf->dtype || (kdt != SLAI_DT_F32 && kdt != SLAI_DT_F16)) return set_error(ctx, SLAI_E_TYPE, "slai_attention: caches must both be f32 or f16");
+    if (kdt != value_cache.buf->dtype || (kdt != SLAI_DT_F32 && kdt != SLAI_DT_F16)) return set_error(ctx, SLAI_E_TYPE, std::string(fn) + ": caches must both be f32 or f16");
     const size_t esz = kdt == SLAI_DT_F16 ? 2 : 4;
     for (const slai_view *c : {&key_cache, &value_cache}) {
         if (c->size[0] != params->kv_dim || c->size[1] != params->seq_len || c->stride[0] != 1 || c->stride[1] != params->kv_dim ||
             (c->offset + (size_t)params->kv_dim * params->seq_len) * esz > c->buf->bytes || (c->offset % 2))
-            return set_error(ctx, SLAI_E_SHAPE, "slai_attention: caches must be [kv_dim x seq_len] column-major");
+            return set_error(ctx, SLAI_E_SHAPE, std::string(fn) + ": caches must be [kv_dim x seq_len] column-major");
     }
     AttnLaunch a{};
     a.q = vq.p;
@@ -741,7 +746,17 @@ SLAI_EXPORT int slai_attention(slai_ctx *ctx, const slai_attn_params *params, co
     a.rope_variant = SLAI_ROPE_ORIGINAL; a.rope_base = 0.0f;
     a.out = vx.p;
     a.n_splits = pick_attn_splits(ctx, nh, params->seq_len);
-    int rc = ensure_attn_scratch(ctx, attention_scratch_floats(nh, hs, a.n_splits));
+    *out = a;
+    return SLAI_OK;
+}
+}  // namespace slai
+
+SLAI_EXPORT int slai_attention(slai_ctx *ctx, const slai_attn_params *params, const slai_buffer *params_gpu, slai_view q,
+                               slai_view key_cache, slai_view value_cache, slai_view att, slai_view xb) {
+    (void)att;
+    AttnLaunch a{};
+    if (int rc = attention_describe(ctx, "slai_attention", params, params_gpu, q, key_cache, value_cache, xb, &a)) return rc;
+    int rc = ensure_attn_scratch(ctx, attention_scratch_floats(a.n_heads, a.head_size, a.n_splits));
     if (rc) return rc;
     a.scratch = ctx->attn_scratch;
     hipError_t e = launch_attention(ctx->stream, a);

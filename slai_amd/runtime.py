@@ -259,6 +259,11 @@ class LlmContext:
         self.backend.check(self.L.slai_attention(self.h, C.byref(params), params_gpu.h, _v(q), _v(key_cache), _v(value_cache),
                                                  _v(att), _v(xb)))
 
+    def attention_static(self, params, params_gpu, q, key_cache, value_cache, att, xb):
+        """``attention`` with the split partials in the library's static device array: allocates nothing."""
+        self.backend.check(self.L.slai_attention_static(self.h, C.byref(params), params_gpu.h, _v(q), _v(key_cache), _v(value_cache),
+                                                        _v(att), _v(xb)))
+
     def argmax(self, logits, out_index):
         self.backend.check(self.L.slai_argmax(self.h, _v(logits), out_index.h))
 
