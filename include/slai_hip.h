@@ -35,6 +35,7 @@ typedef struct slai_ctx slai_ctx;
 typedef struct slai_buffer slai_buffer;
 typedef struct slai_qmat slai_qmat;
 typedef struct slai_graph slai_graph;
+typedef struct slai_tensor_cache slai_tensor_cache;
 typedef struct slai_tokenizer slai_tokenizer;
 typedef struct slai_gguf slai_gguf;
 typedef struct slai_llama2 slai_llama2;
@@ -102,6 +103,21 @@ int slai_buffer_create(slai_ctx *ctx, size_t bytes, int dtype, uint32_t usage, s
 void slai_buffer_destroy(slai_ctx *ctx, slai_buffer *buf);
 size_t slai_buffer_size(const slai_buffer *buf);
 void *slai_buffer_device_ptr(const slai_buffer *buf);
+/* `TensorCache` (crates/slai/src/tensor_cache.rs:126-204), the pool of temporaries behind `LlmContext`
+ * (context.rs:69-76,107-127): idle buffers keyed by element type, shape[4] and usage.
+ *   get_or_insert (:162-188)  an idle buffer with this key (contents as its last holder left them) or a new zero-filled
+ *                             one; a hit allocates nothing and is legal during graph capture, a miss is SLAI_E_STATE there
+ *   reclaim (:118-124,199-203, what dropping a `CachedTensor` does)  back into the pool under its key
+ *   clear (:195-197; the chat calls it once per token, chat_llama2.rs:174)  frees the idle buffers
+ *   idle  number of buffers in the pool.
+ * The models of this library do not use it: `Llama2State` preallocates every activation (transformer.rs:47-140). */
+int slai_tensor_cache_create(slai_ctx *ctx, slai_tensor_cache **out);
+void slai_tensor_cache_destroy(slai_ctx *ctx, slai_tensor_cache *cache);
+int slai_tensor_cache_get_or_insert(slai_ctx *ctx, slai_tensor_cache *cache, int dtype, const uint32_t shape[4], uint32_t usage,
+                                    slai_buffer **out);
+int slai_tensor_cache_reclaim(slai_ctx *ctx, slai_tensor_cache *cache, slai_buffer *buf);
+int slai_tensor_cache_clear(slai_ctx *ctx, slai_tensor_cache *cache);
+size_t slai_tensor_cache_idle(const slai_tensor_cache *cache);
 /* `Backend::write_buffer` (crates/slai-chat/src/chat_llama2.rs:180-185); byte offsets. */
 int slai_write_buffer(slai_ctx *ctx, slai_buffer *buf, size_t offset, const void *src, size_t bytes);
 /* `Backend::read_buffer` (crates/slai-chat/src/chat_llama2.rs:225-227); synchronises. */

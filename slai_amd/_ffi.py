@@ -96,6 +96,12 @@ SIGNATURES = {
     "slai_argmax": (i32, [vp, View, vp]),
     "slai_sample": (i32, [vp, View, C.c_float, C.c_float, C.c_float, vp]),
     "slai_sampler_coin": (C.c_float, [u64, u32]),
+    "slai_tensor_cache_create": (i32, [vp, P(vp)]),
+    "slai_tensor_cache_destroy": (None, [vp, vp]),
+    "slai_tensor_cache_get_or_insert": (i32, [vp, vp, i32, P(u32 * 4), u32, P(vp)]),
+    "slai_tensor_cache_reclaim": (i32, [vp, vp, vp]),
+    "slai_tensor_cache_clear": (i32, [vp, vp]),
+    "slai_tensor_cache_idle": (sz, [vp]),
     "slai_timer_begin": (i32, [vp]),
     "slai_timer_end": (i32, [vp, P(C.c_float)]),
     "slai_graph_begin_capture": (i32, [vp]),

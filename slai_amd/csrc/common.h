@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <map>
 #include <string>
 #include <vector>
 
@@ -15,6 +16,7 @@ struct slai_buffer {
     int dtype = SLAI_DT_F32;
     uint32_t usage = 0;
     void *host_staging = nullptr;  // pinned, when created with SLAI_USAGE_MAP_READ
+    uint32_t shape[4] = {0, 0, 0, 0};  // set for buffers handed out by a slai_tensor_cache (its key)
 };
 
 struct slai_qmat {
@@ -32,6 +34,19 @@ struct slai_qmat {
     float wbound = 0.0f;
 };
 
+// `TensorCache` (crates/slai/src/tensor_cache.rs:126-204): idle temporaries keyed by element type, shape and usage.
+struct slai_tensor_key {
+    int dtype; uint32_t shape[4]; uint32_t usage;
+    bool operator<(const slai_tensor_key &o) const {
+        if (dtype != o.dtype) return dtype < o.dtype;
+        for (int i = 0; i < 4; ++i) if (shape[i] != o.shape[i]) return shape[i] < o.shape[i];
+        return usage < o.usage;
+    }
+};
+struct slai_tensor_cache {
+    std::map<slai_tensor_key, std::vector<slai_buffer *>> tensors;
+};
+
 struct slai_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -42,6 +57,7 @@ struct slai_ctx {
     hipStream_t stream = nullptr;
     std::string err;
     bool capturing = false;
+    bool submission_open = false;   // between slai_begin_submission and slai_submit
     // attention split-K partials (grown on demand, never inside a capture)
     float *attn_scratch = nullptr;
     size_t attn_scratch_floats = 0;

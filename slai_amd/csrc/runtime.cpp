@@ -113,8 +113,20 @@ SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
 SLAI_EXPORT const char *slai_last_error(slai_ctx *ctx) { return ctx ? ctx->err.c_str() : "null context"; }
 SLAI_EXPORT void *slai_ctx_stream(slai_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 
-SLAI_EXPORT int slai_begin_submission(slai_ctx *ctx) { return ctx ? SLAI_OK : SLAI_E_ARG; }
-SLAI_EXPORT int slai_submit(slai_ctx *ctx) { return ctx ? SLAI_OK : SLAI_E_ARG; }
+// context.rs:79-95.  The reference records launches into an encoder and hands it to the queue on submit; here every
+// launch goes to the context's stream at once, so the pair only keeps the reference's state rules: beginning while a
+// submission is open submits it first, submitting with none open does nothing.  Both are legal inside a graph capture.
+SLAI_EXPORT int slai_begin_submission(slai_ctx *ctx) {
+    if (!ctx) return SLAI_E_ARG;
+    if (ctx->submission_open) slai_submit(ctx);
+    ctx->submission_open = true;
+    return SLAI_OK;
+}
+SLAI_EXPORT int slai_submit(slai_ctx *ctx) {
+    if (!ctx) return SLAI_E_ARG;
+    ctx->submission_open = false;
+    return SLAI_OK;
+}
 SLAI_EXPORT int slai_synchronize(slai_ctx *ctx) {
     if (!ctx) return SLAI_E_ARG;
     SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
@@ -187,6 +199,67 @@ SLAI_EXPORT int slai_copy_buffer(slai_ctx *ctx, slai_buffer *dst, size_t dst_off
     SLAI_HIP_TRY(ctx, hipMemcpyAsync((char *)dst->dptr + dst_offset, (const char *)src->dptr + src_offset, bytes,
                                      hipMemcpyDeviceToDevice, ctx->stream));
     return SLAI_OK;
+}
+
+// ---- temporaries (crates/slai/src/tensor_cache.rs) ---------------------------------------------
+SLAI_EXPORT int slai_tensor_cache_create(slai_ctx *ctx, slai_tensor_cache **out) {
+    if (!ctx || !out) return SLAI_E_ARG;
+    *out = new slai_tensor_cache();
+    return SLAI_OK;
+}
+// `TensorCache::clear` (tensor_cache.rs:195-197): idle tensors are freed; those handed out stay with their holders.
+SLAI_EXPORT int slai_tensor_cache_clear(slai_ctx *ctx, slai_tensor_cache *c) {
+    if (!ctx || !c) return SLAI_E_ARG;
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_tensor_cache_clear during graph capture");
+    for (auto &kv : c->tensors)
+        for (slai_buffer *b : kv.second) slai_buffer_destroy(ctx, b);
+    c->tensors.clear();
+    return SLAI_OK;
+}
+SLAI_EXPORT void slai_tensor_cache_destroy(slai_ctx *ctx, slai_tensor_cache *c) {
+    if (!c) return;
+    if (ctx) { ctx->capturing = false; slai_tensor_cache_clear(ctx, c); }
+    delete c;
+}
+// `TensorCache::get_or_insert` (tensor_cache.rs:162-188) with the insert closure of context.rs:107-127: an idle tensor of
+// this element type, shape and usage if the cache has one (its contents are whatever its last holder left), a new
+// zero-filled buffer otherwise.  A hit allocates nothing and is legal during graph capture; a miss is not.
+SLAI_EXPORT int slai_tensor_cache_get_or_insert(slai_ctx *ctx, slai_tensor_cache *c, int dtype, const uint32_t shape[4], uint32_t usage, slai_buffer **out) {
+    if (!ctx || !c || !shape || !out) return SLAI_E_ARG;
+    *out = nullptr;
+    if (dtype < SLAI_DT_F32 || dtype > SLAI_DT_I32) return set_error(ctx, SLAI_E_ARG, "bad dtype");
+    slai_tensor_key key{dtype, {shape[0], shape[1], shape[2], shape[3]}, usage};
+    auto it = c->tensors.find(key);
+    if (it != c->tensors.end() && !it->second.empty()) {
+        *out = it->second.back();
+        it->second.pop_back();
+        return SLAI_OK;
+    }
+    static const size_t esz[] = {4, 2, 1, 4};
+    uint64_t n = 1;
+    for (int i = 0; i < 4; ++i) {
+        n *= shape[i];
+        if (n > (uint64_t)1 << 40) return set_error(ctx, SLAI_E_SHAPE, "slai_tensor_cache_get_or_insert: shape too large");
+    }
+    slai_buffer *b = nullptr;
+    if (int rc = slai_buffer_create(ctx, (size_t)n * esz[dtype], dtype, usage, &b)) return rc;
+    for (int i = 0; i < 4; ++i) b->shape[i] = shape[i];
+    *out = b;
+    return SLAI_OK;
+}
+// What dropping a `CachedTensor` does (tensor_cache.rs:118-124, `reclaim` :199-203): the buffer goes back to the cache
+// under the key it was handed out with.  Buffers that did not come from a cache are refused.
+SLAI_EXPORT int slai_tensor_cache_reclaim(slai_ctx *ctx, slai_tensor_cache *c, slai_buffer *b) {
+    if (!ctx || !c || !b) return SLAI_E_ARG;
+    if (!b->shape[0]) return set_error(ctx, SLAI_E_ARG, "slai_tensor_cache_reclaim: not a cached tensor");
+    slai_tensor_key key{b->dtype, {b->shape[0], b->shape[1], b->shape[2], b->shape[3]}, b->usage};
+    c->tensors[key].push_back(b);
+    return SLAI_OK;
+}
+SLAI_EXPORT size_t slai_tensor_cache_idle(const slai_tensor_cache *c) {
+    size_t n = 0;
+    if (c) for (const auto &kv : c->tensors) n += kv.second.size();
+    return n;
 }
 
 // ---- quantized matrices ---------------------------------------------------------

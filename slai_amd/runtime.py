@@ -176,6 +176,42 @@ class GpuQuantMatrix:
             self.h = None
 
 
+class TensorCache:
+    """crates/slai/src/tensor_cache.rs ``TensorCache``: idle temporaries keyed by element type, shape and usage."""
+
+    def __init__(self, backend):
+        self.b = backend
+        h = C.c_void_p()
+        backend.check(backend.L.slai_tensor_cache_create(backend.h, C.byref(h)))
+        self.h = h
+
+    def get_or_insert(self, nrows, ncols=1, dtype=_ffi.DT_F32, usage=STORAGE):
+        """An idle tensor of this shape (contents as its last holder left them) or a new zero-filled one."""
+        shape = (C.c_uint32 * 4)(int(nrows), int(ncols), 1, 1)
+        h = C.c_void_p()
+        self.b.check(self.b.L.slai_tensor_cache_get_or_insert(self.b.h, self.h, dtype, C.byref(shape), usage, C.byref(h)))
+        t = GpuTensor.__new__(GpuTensor)
+        t.b, t.nrows, t.ncols, t.dtype, t.h = self.b, int(nrows), int(ncols), dtype, h
+        t.nbytes = t.nrows * t.ncols * np.dtype(_NP[dtype]).itemsize
+        return t
+
+    def reclaim(self, tensor):
+        """What dropping a ``CachedTensor`` does: the tensor goes back into the pool; the handle must not be used after."""
+        self.b.check(self.b.L.slai_tensor_cache_reclaim(self.b.h, self.h, tensor.h))
+        tensor.h = None
+
+    def clear(self):
+        self.b.check(self.b.L.slai_tensor_cache_clear(self.b.h, self.h))
+
+    def idle(self):
+        return int(self.b.L.slai_tensor_cache_idle(self.h))
+
+    def destroy(self):
+        if self.h:
+            self.b.L.slai_tensor_cache_destroy(self.b.h, self.h)
+            self.h = None
+
+
 class LlmContext:
     """crates/slai/src/context.rs ``LlmContext``: same method names and argument order (out first)."""
 

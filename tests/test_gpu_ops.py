@@ -177,3 +177,86 @@ def test_attention_fused_and_reference_sequence(backend, oracle_lib, cfg, f16):
             gxb2.destroy()
     for o in (gparams, gq, gk, gv, gatt, gxb):
         o.destroy()
+
+
+def test_submission_bracket_and_graph_replay_of_an_op_sequence(backend, oracle_lib):
+    """`LlmContext::begin_submission` / `submit` (context.rs:79-95) around op-level launches, eagerly and captured into
+    a graph that is replayed several times with eager work and synchronisations in between; every replay must
+    reproduce the eager result, which must be the oracle's.  The sequence is a feed-forward block: RMSNorm, gate and up
+    projections, SiLU, down projection, residual add (transformer.rs:356-365)."""
+    from slai_amd import synth
+    from slai_amd.runtime import GpuQuantMatrix, GpuTensor, LlmContext, TensorCache
+    dim, hid, t = 512, 1536, 12
+    ctxt = LlmContext(backend)
+    cache = TensorCache(backend)
+    x0 = rnd(1, dim)
+    w = (1.0 + 0.1 * rnd(2, dim)).astype(np.float32)
+    raws = [synth.normal_quantized(40 + i, t, r, c, 0.05) for i, (r, c) in enumerate(((hid, dim), (hid, dim), (dim, hid)))]
+    shapes = ((hid, dim), (hid, dim), (dim, hid))
+    deq = []
+    for raw, (r, c) in zip(raws, shapes):
+        a = np.empty(r * c, np.float32)
+        assert oracle_lib.slo_dequantize(t, raw.ctypes.data, r * c, a.ctypes.data) == 0
+        deq.append(a.reshape(r, c))
+    # oracle: ops of cpu.rs:340-376,555-560 in the same order
+    xb = np.empty(dim, np.float32); oracle_lib.slo_rms_norm(xb.ctypes.data, x0.ctypes.data, w.ctypes.data, dim, 1e-5)
+    hb = np.empty(hid, np.float32); hb2 = np.empty(hid, np.float32)
+    oracle_lib.slo_gemv(hb.ctypes.data, deq[0].ctypes.data, xb.ctypes.data, hid, dim)
+    oracle_lib.slo_gemv(hb2.ctypes.data, deq[1].ctypes.data, xb.ctypes.data, hid, dim)
+    oracle_lib.slo_silu(hb.ctypes.data, hb2.ctypes.data, hid)
+    xb2 = np.empty(dim, np.float32)
+    oracle_lib.slo_gemv(xb2.ctypes.data, deq[2].ctypes.data, hb.ctypes.data, dim, hid)
+    ref = x0 + xb2
+
+    gate, up, down = [GpuQuantMatrix(backend, t, r, c, raw) for raw, (r, c) in zip(raws, shapes)]
+    gx0 = GpuTensor.vector(backend, x0)
+    gw = GpuTensor.vector(backend, w)
+    cfg = GpuTensor.scalar(backend, _ffi.RmsNormConfig(1e-5, (0, 0, 0)))
+    gx = GpuTensor(backend, dim)
+    # the temporaries come from the cache, as they do behind the reference's LlmContext
+    gxb, gxb2 = cache.get_or_insert(dim), cache.get_or_insert(dim)
+    ghb, ghb2 = cache.get_or_insert(hid), cache.get_or_insert(hid)
+    assert cache.idle() == 0
+
+    def block():
+        ctxt.begin_submission()
+        ctxt.copy(gx0, gx)
+        ctxt.rms_norm_assign(cfg, gxb, gx, gw)
+        ctxt.matmul_quant_assign(ghb, gate, gxb)
+        ctxt.matmul_quant_assign(ghb2, up, gxb)
+        ctxt.silu(ghb, ghb2)
+        ctxt.matmul_quant_assign(gxb2, down, ghb)
+        ctxt.add_assign(gx, gxb2)
+        ctxt.submit()
+
+    block()
+    backend.synchronize()
+    eager = gx.read()
+    assert rel_err(eager, ref) < 1e-4
+    ctxt.begin_submission(); ctxt.begin_submission(); ctxt.submit(); ctxt.submit()     # re-begin submits; a second submit is a no-op
+    backend.graph_begin_capture()
+    block()
+    g = backend.graph_end_capture()
+    for rep in range(4):
+        gx.write(np.full(dim, float(rep), np.float32))       # eager work between the replays: the graph must overwrite it
+        ghb.write(np.zeros(hid, np.float32))
+        backend.synchronize()
+        backend.graph_launch(g)
+        backend.synchronize()
+        assert np.array_equal(gx.read().view(np.uint32), eager.view(np.uint32)), rep
+    backend.graph_destroy(g)
+    # back into the pool, out again: the same buffers, no new allocation; clear frees the idle ones
+    for tns in (gxb, gxb2, ghb, ghb2):
+        cache.reclaim(tns)
+    assert cache.idle() == 4
+    again = cache.get_or_insert(hid)
+    assert cache.idle() == 3
+    assert again.read().shape == (hid,)                                                  # contents are the last holder's
+    other = cache.get_or_insert(hid, 2)                                                  # another shape: a miss, a new zeroed buffer
+    assert cache.idle() == 3 and not other.read().any()
+    cache.reclaim(again); cache.reclaim(other)
+    cache.clear()
+    assert cache.idle() == 0
+    cache.destroy()
+    for o in (gate, up, down, gx0, gw, cfg, gx):
+        o.destroy()
