@@ -3,17 +3,25 @@
 fp16 KV cache, batch 1 -- BASELINE configuration 4.
 
 One "step" = one token through the whole layer stack (greedy decode loop on the device).  The
-prompt (W = --warmup positions, processed token by token like the reference) is untimed; the next
-K = --steps generated tokens are timed with HIP events on the library's stream, with inputs and
-weights resident in HBM.  Prints ONE JSON line.
+64 prompt positions of the configuration are always processed first, untimed (62 of them in chunks
+through slai_llama2_prefill); then W = --warmup tokens are decoded untimed (the first of them from the
+last prompt token: the reference excludes the first generated token as well), and the next K = --steps
+generated tokens are timed with HIP events on the library's stream, with inputs and weights resident
+in HBM.  The default W = 1, K = 256 times exactly the positions the metric is quoted on (64 .. 319).
+Prints ONE JSON line.
 
 Also measured here:
-  * roofline: the dominant kernel (fused RMSNorm + gate/up Q4_K GEMV + SiLU, 11008x4096 x2) timed
-    alone with HIP events while rotating over enough distinct weight copies to defeat the 256 MB
-    Infinity Cache; achieved = algorithmic bytes / mean launch time, peak = 8 TB/s.
-  * cpu_baseline: the CPU oracle (a C restatement of the reference's CPU path) on the host cores,
-    on a bounded sample of the same workload (the same layer shapes at depth 2 and 4, a few
-    tokens), extrapolated to 32 layers.  A reported baseline, not the target.
+  * roofline: the dominant kernel.  When the model takes the one-launch-per-token form, that launch IS
+    the token (every layer and the output matrix): achieved = the token's algorithmic bytes / the
+    launch's mean duration inside the timed loop.  Otherwise the two largest kernels of a token are
+    timed alone with HIP events while rotating over enough distinct weight copies to defeat the
+    256 MB Infinity Cache.  peak = 8 TB/s.
+  * cpu_baseline: the CPU oracle (a C restatement of the reference's CPU path) on the host cores:
+    configuration 1 in full on one thread (the reference's CPU path is single-threaded) and on all
+    cores, and a bounded sample of the headline shapes (depth 2 and 6, a few tokens) extrapolated to
+    32 layers.  A reported baseline, not the target.
+  * config5: the long-context configuration (Q8_0, cache pre-filled to 4000 positions), attention and
+    GEMV rates apart.
 """
 import argparse
 import math
@@ -182,8 +190,37 @@ def sweep(backend):
                       "peak_gbs": HBM_PEAK_GBS, "gemv": rows, "attention": att}), flush=True)
 
 
+def cpu_config1(seed):
+    """BASELINE configuration 1 in full on the oracle: tiny Llama (dim 288, 6 layers, Q8_0), 16 prompt ids + 128 greedy
+    tokens, on ONE thread (the reference's CPU path is single-threaded nalgebra, models/llama2/cpu.rs:370-376) and on all
+    cores; tok/s over the 143 forward passes of the run (the reference feeds a prompt token by token, chat_llama2.rs:105-158)."""
+    import oracle
+    from slai_amd import gguf_writer as gw
+    L = oracle.load()
+    data = gw.tiny_llama_gguf(seed=seed)
+    err = C.c_int(0)
+    g = L.slo_gguf_parse(data.ctypes.data, data.size, C.byref(err))
+    prompt = np.random.Generator(np.random.PCG64(seed)).integers(0, 32000, 16).astype(np.int32)
+    out = {}
+    ncores = os.cpu_count() or 1
+    n = 16 + 128 - 1                              # forward passes of the configuration: 16 prompt ids, 128 tokens out
+    for label, threads in (("one_thread", 1), ("all_cores", min(16, ncores))):
+        L.slo_set_threads(threads)
+        m = L.slo_llama2_from_gguf(g, b"llama", 0, 0, 0)
+        toks = np.zeros(n, np.int32)
+        t0 = time.perf_counter()
+        L.slo_llama2_generate(m, prompt.ctypes.data, 16, 0, n, -1, toks.ctypes.data, None)
+        dt = time.perf_counter() - t0
+        L.slo_llama2_free(m)
+        out[label] = dict(tok_s=round(n / dt, 2), threads=threads, forward_passes=n)
+    L.slo_gguf_free(g)
+    out["nproc"] = ncores
+    return out
+
+
 def cpu_baseline(seed, n_tokens=32):
-    """Oracle decode of the same layer shapes at depth 2 and 6, extrapolated linearly to 32 layers."""
+    """Oracle decode of the headline layer shapes at depth 2 and 6, extrapolated linearly to 32 layers; beside it
+    configuration 1 in full (cpu_config1)."""
     import oracle
     from slai_amd import gguf_writer as gw
     L = oracle.load()
@@ -209,22 +246,77 @@ def cpu_baseline(seed, n_tokens=32):
     per_layer = (times[6] - times[2]) / 4.0
     head = max(times[2] - 2 * per_layer, 0.0)
     full = head + CFG["n_layers"] * per_layer
-    return dict(value=1.0 / full, unit="tok/s", cores=threads, kind="port",
+    return dict(value=1.0 / full, unit="tok/s", cores=threads, kind="port", nproc=os.cpu_count() or 1,
                 sample="oracle (C restatement of models/llama2/cpu.rs, OpenMP over GEMV rows) on the same layer shapes and "
                        "quantization at depth 2 and 6, %d tokens each; %.2f ms per layer + %.2f ms embedding/head per token, "
-                       "extrapolated to 32 layers" % (n_tokens, per_layer * 1e3, head * 1e3))
+                       "extrapolated to 32 layers" % (n_tokens, per_layer * 1e3, head * 1e3),
+                config1=cpu_config1(seed))
+
+
+def config5_block(backend, seed, n_steps=96):
+    """BASELINE configuration 5: the 7B shape with Q8_0 weights and an fp16 cache pre-filled to 4000 positions with seeded
+    N(0,1) rows, 96 tokens decoded up to the 4096th position.  Attention rate: the attention kernels (split + combine)
+    timed alone at position 4047 over rotating caches; GEMV rate: the weight bytes over what is left of the token."""
+    from slai_amd import _ffi
+    from slai_amd import gguf_writer as gw
+    from slai_amd.runtime import Gguf, GpuTensor, Llama2, LlmContext
+    t0 = time.perf_counter()
+    data = gw.llama_gguf(dim=CFG["dim"], hidden_dim=CFG["hidden_dim"], n_layers=CFG["n_layers"], n_heads=CFG["n_heads"], n_kv_heads=CFG["n_kv_heads"],
+                         vocab=CFG["vocab"], seq_len=4096, wtype=8, seed=seed + 5, distinct_layers=2)
+    g = Gguf(data)
+    m = Llama2(backend, g, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+    rng = np.random.Generator(np.random.PCG64(seed + 6))
+    fills = [(rng.standard_normal((4000, CFG["dim"]), dtype=np.float32).astype(np.float16),
+              rng.standard_normal((4000, CFG["dim"]), dtype=np.float32).astype(np.float16)) for _ in range(4)]
+    for l in range(CFG["n_layers"]):
+        m.write_kv(l, *fills[l % 4])
+    log("config 5 model: %.2f GB, set up in %.1f s" % (data.size / 1e9, time.perf_counter() - t0))
+    seq = np.zeros(4001, np.int32); seq[4000] = 17
+    m.generate(seq, 8, start_pos=4000)                                    # untimed: graph capture, first touch
+    _, ms = m.generate(seq, n_steps, start_pos=4000)
+    ms_tok = ms / n_steps
+    wbytes = m.weight_bytes()
+    kv_dim = CFG["dim"]
+    kv_read = 2 * CFG["n_layers"] * (4000 + (n_steps + 1) / 2.0) * kv_dim * 2
+    form = m.decode_form()
+    m.destroy(); g.close(); del data
+    # the attention kernels alone at position 4047 (the mean of the 96 positions), rotating over > 512 MB of caches
+    ctxt = LlmContext(backend)
+    nh, hs, seq_len, pos = CFG["n_heads"], CFG["dim"] // CFG["n_heads"], 4096, 4047
+    caches = [(GpuTensor(backend, kv_dim, seq_len, _ffi.DT_F16, data=np.resize(fills[i % 4][0], (seq_len, kv_dim))),
+               GpuTensor(backend, kv_dim, seq_len, _ffi.DT_F16, data=np.resize(fills[i % 4][1], (seq_len, kv_dim)))) for i in range(10)]
+    params = _ffi.AttnParams(seq_len, kv_dim, 1, nh, hs, pos, (0, 0))
+    gparams = GpuTensor.scalar(backend, params)
+    gq = GpuTensor.vector(backend, rng.standard_normal(nh * hs, dtype=np.float32))
+    gatt, gxb = GpuTensor(backend, seq_len, nh), GpuTensor(backend, nh * hs)
+    us = graph_time_us(backend, lambda: [ctxt.attention(params, gparams, gq, kc, vc, gatt, gxb) for (kc, vc) in caches], len(caches))
+    attn_bytes = 2 * (pos + 1) * kv_dim * 2
+    for o in [gparams, gq, gatt, gxb] + [t for kv in caches for t in kv]:
+        o.destroy()
+    attn_ms_tok = us * CFG["n_layers"] / 1000.0
+    rest_ms = max(ms_tok - attn_ms_tok, 1e-6)
+    total = wbytes + kv_read
+    return dict(workload="7B shape, Q8_0, fp16 cache pre-filled to 4000 positions, %d tokens at positions 4000..%d" % (n_steps, 3999 + n_steps),
+                tok_s=round(1000.0 / ms_tok, 1), ms_per_step=round(ms_tok, 4), token_bytes=int(total),
+                hbm_gbs=round(total / ms_tok / 1e6, 1), hbm_roofline_frac=round(total / ms_tok / 1e6 / HBM_PEAK_GBS, 4),
+                attention=dict(us_per_layer=round(us, 2), gbs=round(attn_bytes / us / 1e3, 1), frac=round(attn_bytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                               algorithmic_bytes=attn_bytes, how="split + combine kernels alone at position %d over 10 rotating cache pairs" % pos),
+                gemv=dict(gbs=round(wbytes / rest_ms / 1e6, 1), frac=round(wbytes / rest_ms / 1e6 / HBM_PEAK_GBS, 4), weight_bytes=int(wbytes),
+                          how="weight bytes over the token time less 32 x the attention time"),
+                decode_form=form)
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
-    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--layers", type=int, default=CFG["n_layers"], help="depth (32 = the benchmark configuration)")
     ap.add_argument("--distinct-layers", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-side", action="store_true", help="only the headline decode (no sampled decode, prompt chunks, config 5)")
     ap.add_argument("--probe", action="store_true", help="counter probe: copy kernel + dominant GEMV only")
     ap.add_argument("--sweep", action="store_true", help="per-format GEMV sweep and long-context attention instead of the decode run")
     args = ap.parse_args()
@@ -242,8 +334,9 @@ def main():
         backend.close()
         return
     K, W = args.steps, max(args.warmup, 1)
+    P = 64                                       # prompt positions of the configuration, always processed first
     cfg = dict(CFG, n_layers=args.layers)
-    seq_len = max(512, ((W + K + 63) // 64) * 64)
+    seq_len = max(512, ((P + W + K + 63) // 64) * 64)
 
     from slai_amd import _ffi
     from slai_amd import gguf_writer as gw
@@ -258,54 +351,76 @@ def main():
     t0 = time.perf_counter()
     g = Gguf(data)
     model = Llama2(backend, g, _ffi.MODEL_LLAMA, _ffi.KV_F16)
-    log("upload: %.1f s, weights %.3f GB" % (time.perf_counter() - t0, model.weight_bytes() / 1e9))
+    form = model.decode_form()
+    log("upload: %.1f s, weights %.3f GB, decode form %d (%s)" % (time.perf_counter() - t0, model.weight_bytes() / 1e9, form,
+                                                                  "one resident launch per token" if form else "one launch per step"))
 
-    prompt = np.random.Generator(np.random.PCG64(args.seed)).integers(0, cfg["vocab"], W).astype(np.int32)
-    # warmup: the W prompt positions (forced tokens), untimed; the last one yields the first generated token
-    warm, _ = model.generate(prompt, W, start_pos=0)
-    seq = np.concatenate([prompt, warm[W - 1:W]]).astype(np.int32)
-    # timed: K tokens at positions W .. W+K-1
+    prompt = np.random.Generator(np.random.PCG64(args.seed)).integers(0, cfg["vocab"], P).astype(np.int32)
+    # untimed: prompt positions 0 .. P-2 in chunks (caches only), then W tokens decoded from the last prompt token on
+    model.prefill(prompt[:P - 1], 0, 0)
+    warm, _ = model.generate(prompt, W, start_pos=P - 1)
+    seq = np.concatenate([prompt, warm]).astype(np.int32)
+    # timed: K tokens at positions P-1+W .. P-2+W+K
+    pos0 = P - 1 + W
     wall0 = time.perf_counter()
-    toks, ms = model.generate(seq, K, start_pos=W)
+    toks, ms = model.generate(seq, K, start_pos=pos0)
     wall = time.perf_counter() - wall0
     ms_per_step = ms / K
     tok_s = 1000.0 / ms_per_step
-    tb = token_bytes(cfg, model.weight_bytes(), W, W + K - 1)
+    tb = token_bytes(cfg, model.weight_bytes(), pos0, pos0 + K - 1)
     log("decode: %.3f ms/token (events), wall %.3f ms/token, %.1f tok/s, %.2f GB/token -> %.1f GB/s"
         % (ms_per_step, wall * 1000 / K, tok_s, tb / 1e9, tb / ms_per_step / 1e6))
-    # the same K positions with the chat's sampler (temperature 0.7, top-p 0.95) picked on the device: reported beside
-    # the headline, never as it.  Random weights give nearly flat logits, the slow case of the nucleus search.
-    _, ms_s = model.generate_sampled(seq, K, 0.7, 0.95, args.seed, start_pos=W)
-    sampled = dict(tok_s=round(1000.0 * K / ms_s, 2), ms_per_step=round(ms_s / K, 4), temperature=0.7, top_p=0.95)
-    log("sampled decode (device sampler, T=0.7, top-p 0.95): %.3f ms/token, %.1f tok/s" % (ms_s / K, 1000.0 * K / ms_s))
-    # prompt processing, reported beside the headline: the reference feeds a prompt token by token (chat_llama2.rs:105-158);
-    # the chunked pass runs 32 tokens per pass over the weights on the matrix cores (weights and activations as f16 head +
-    # remainder pairs, fp32 accumulation; a call repeats in fp32 MFMA when an activation is beyond f16) and computes no logits
-    n_prompt = min(256, seq_len)
-    ptoks = np.random.Generator(np.random.PCG64(args.seed + 1)).integers(0, cfg["vocab"], n_prompt).astype(np.int32)
-    model.prefill(ptoks, 0, 0)                                   # untimed: buffers, first touch
-    ms_p = min(model.prefill(ptoks, 0, 0) for _ in range(3))
-    ms_loop = model.prefill(ptoks[:64], 0, 1)
-    prompt_chunks = dict(tok_s=round(1000.0 * n_prompt / ms_p, 1), tokens=n_prompt, ms=round(ms_p, 3), path=model.prefill_path(),
-                         token_by_token_tok_s=round(1000.0 * 64 / ms_loop, 1), fp32_repeats=model.prefill_fp32_repeats())
-    log("prompt: %d tokens in %.2f ms (%.0f tok/s) in chunks; token by token %.0f tok/s" % (n_prompt, ms_p, 1000.0 * n_prompt / ms_p, 1000.0 * 64 / ms_loop))
+    sampled = prompt_chunks = None
+    if not args.no_side:
+        # the same K positions with the chat's sampler (temperature 0.7, top-p 0.95) picked on the device: reported beside
+        # the headline, never as it.  Random weights give nearly flat logits, the slow case of the nucleus search.
+        _, ms_s = model.generate_sampled(seq, K, 0.7, 0.95, args.seed, start_pos=pos0)
+        sampled = dict(tok_s=round(1000.0 * K / ms_s, 2), ms_per_step=round(ms_s / K, 4), temperature=0.7, top_p=0.95)
+        log("sampled decode (device sampler, T=0.7, top-p 0.95): %.3f ms/token, %.1f tok/s" % (ms_s / K, 1000.0 * K / ms_s))
+        # prompt processing, reported beside the headline: the reference feeds a prompt token by token (chat_llama2.rs:105-158);
+        # the chunked pass runs 32 tokens per pass over the weights on the matrix cores and computes no logits
+        n_prompt = min(256, seq_len)
+        ptoks = np.random.Generator(np.random.PCG64(args.seed + 1)).integers(0, cfg["vocab"], n_prompt).astype(np.int32)
+        model.prefill(ptoks, 0, 0)                                   # untimed: buffers, first touch
+        ms_p = min(model.prefill(ptoks, 0, 0) for _ in range(3))
+        ms_loop = model.prefill(ptoks[:64], 0, 1)
+        prompt_chunks = dict(tok_s=round(1000.0 * n_prompt / ms_p, 1), tokens=n_prompt, ms=round(ms_p, 3), path=model.prefill_path(),
+                             token_by_token_tok_s=round(1000.0 * 64 / ms_loop, 1), fp32_repeats=model.prefill_fp32_repeats())
+        log("prompt: %d tokens in %.2f ms (%.0f tok/s) in chunks; token by token %.0f tok/s" % (n_prompt, ms_p, 1000.0 * n_prompt / ms_p, 1000.0 * 64 / ms_loop))
     model.destroy(); g.close(); del data
 
     roof = None
     if not args.no_roofline:
-        kms, kalgo = measure_dominant_kernel(backend)
-        ach = kalgo / (kms * 1e-3) / 1e9
-        roof = dict(bound="hbm", kernel="gemv_rowtile_kernel<Q4_K, dual> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096)",
-                    achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
-                    traffic=DOMINANT_KERNEL_TRAFFIC_BYTES, launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
-        log("dominant kernel: %.2f us/launch, %.1f GB/s" % (kms * 1000, ach))
+        if form == 1:
+            # the resident launch is the token: embedding gather, buffer fill and the pick (three small launches) are the
+            # only other kernels and are part of the measured time, so this is a lower bound of the launch's own rate
+            ach = tb / (ms_per_step * 1e-3) / 1e9
+            roof = dict(bound="hbm", kernel="llama_decode_persistent_kernel (all 32 layers: RMSNorm + q/k/v, RoPE + attention, output projection, "
+                                            "RMSNorm + gate/up + SiLU, down projection; final norm + output matrix): one launch per token",
+                        achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4), traffic=None,
+                        launch_us=round(ms_per_step * 1000, 2), algorithmic_bytes=int(tb),
+                        how="token bytes over the mean time per token of the timed loop (HIP events on the library's stream)")
+        else:
+            kms, kalgo = measure_dominant_kernel(backend)
+            ach = kalgo / (kms * 1e-3) / 1e9
+            roof = dict(bound="hbm", kernel="gemv_rowtile_kernel<Q4_K, dual> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096); the launch with q/k/v and the "
+                                            "attention is longer per token but cannot be launched alone through the operator API",
+                        achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
+                        traffic=DOMINANT_KERNEL_TRAFFIC_BYTES, traffic_source="profiles/gate_up_gemv_q4k_hbm_counters.md",
+                        launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
+        log("dominant kernel: %s us/launch, %.1f GB/s" % (roof["launch_us"], roof["achieved"]))
+    c5 = None
+    if not args.no_side:
+        c5 = config5_block(backend, args.seed)
+        log("config 5: %.1f tok/s (%.3f ms/token); attention %.2f us/layer = %.1f GB/s; GEMV %.1f GB/s"
+            % (c5["tok_s"], c5["ms_per_step"], c5["attention"]["us_per_layer"], c5["attention"]["gbs"], c5["gemv"]["gbs"]))
     backend.close()
 
     cpu = None
     if not args.no_cpu_baseline:
         t0 = time.perf_counter()
         cpu = cpu_baseline(args.seed)
-        log("cpu baseline: %.3f tok/s on %d threads (%.1f s)" % (cpu["value"], cpu["cores"], time.perf_counter() - t0))
+        log("cpu baseline: %.3f tok/s on %d threads (%.1f s); config 1 in full: %s" % (cpu["value"], cpu["cores"], time.perf_counter() - t0, cpu["config1"]))
 
     out = {
         "metric": "decode tok/s & % of HBM roofline, Llama-2-7B-shape Q4_K, batch 1",
@@ -315,12 +430,14 @@ def main():
                                 "(%d layers generated, the rest are row-rotated copies in distinct memory), seeded prompt ids"
                                 % min(args.distinct_layers, cfg["n_layers"]),
         "config": {"workload": "BASELINE config 4: Llama-2-7B-shape greedy decode, dim 4096, %d layers, 32 heads, FFN 11008, "
-                               "vocab 32000, Q4_K weights (Q6_K v-proj/output), fp16 KV, %d prompt + %d generated tokens"
-                               % (cfg["n_layers"], W, K), "batch": 1, "kv_dtype": "f16", "context": seq_len},
+                               "vocab 32000, Q4_K weights (Q6_K v-proj/output), fp16 KV; 64 prompt positions processed untimed, "
+                               "%d token(s) decoded untimed, then %d tokens timed at positions %d..%d"
+                               % (cfg["n_layers"], W, K, pos0, pos0 + K - 1), "batch": 1, "kv_dtype": "f16", "context": seq_len,
+                   "decode_form": "one resident launch per token" if form else "one launch per step"},
         "token_bytes": int(tb), "hbm_gbs": round(tb / ms_per_step / 1e6, 1),
         "hbm_roofline_frac": round(tb / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
         "roofline_tok_s": round(HBM_PEAK_GBS * 1e9 / tb, 1),
-        "sampled_decode": sampled, "prompt_chunks": prompt_chunks,
+        "sampled_decode": sampled, "prompt_chunks": prompt_chunks, "config5": c5,
         "roofline": roof, "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

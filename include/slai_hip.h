@@ -341,6 +341,17 @@ int slai_llama2_prefill(slai_llama2 *m, const int32_t *tokens, uint32_t n_tokens
                         float *elapsed_ms);
 int slai_llama2_prefill_supported(const slai_llama2 *m);
 uint32_t slai_llama2_prefill_fp32_repeats(const slai_llama2 *m);
+/* Which form the per-token loop of this model takes: 0 = one launch per step of `Llama2::launch` (transformer.rs:316-381;
+ * four to five per layer), 1 = the whole layer stack and the output matrix in one resident launch per token (widths of
+ * 1024 .. 4096 in steps of 1024, as many cache heads as query heads of size 128, contexts up to 1024, Q4_K / Q5_K / Q6_K
+ * mixes; SLAI_PERSISTENT=0 at slai_ctx_create switches it off).  Results are the same to within summation order. */
+int slai_llama2_decode_form(const slai_llama2 *m);
+/* Measurement aid without a reference counterpart (profilers see the resident launch as one kernel): runs one token at
+ * (pos, token) with in-kernel time stamps and returns them, n_workgroups x stamps_per_workgroup 64-bit ticks of the
+ * constant 100 MHz clock; per workgroup 16 per layer -- 4 per phase (q/k/v + attention, output projection, gate/up, down
+ * projection): entered, input staged, multiplied, reduced -- then 8 for the output matrix.  Zero = phase not taken. */
+int slai_llama2_trace_token(slai_llama2 *m, uint32_t pos, uint32_t token, uint64_t *out, size_t capacity, uint32_t *n_workgroups,
+                            uint32_t *stamps_per_workgroup);
 /* Device access for set-up and inspection: layer l's caches ([kv_dim x seq_len]) and the state vectors. */
 int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache);
 int slai_llama2_logits_buffer(slai_llama2 *m, slai_buffer **logits);

@@ -78,7 +78,9 @@ template <> struct Vec8<false> {  // 8 f32 = 32 bytes
 // the requests for the cache, which depend on nothing but the position, then go first).  `quad_token` (single-split
 // form only): write the result as that token's column of a quad-major matrix instead of a plain vector; with
 // `split_flag` as f16 head + remainder pairs (split_quad's layout), *split_flag set when a value is beyond f16.
-template <bool F16, int NT, int HS, bool SINGLE, bool FUSED, int KL = 4, class Wait>
+// FLOW: q / knew / vnew were written by other workgroups of this very launch and the result is read by others again:
+// they are read and written with the coherent accesses of device_util.h (no cache of this compute unit may serve them).
+template <bool F16, int NT, int HS, bool SINGLE, bool FUSED, int KL = 4, bool FLOW = false, class Wait>
 __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, uint32_t split, uint32_t tid, Wait &&wait_inputs,
                                                uint32_t quad_token = 0xffffffffu, int *split_flag = nullptr) {
     using C = KV<F16>;
@@ -114,13 +116,19 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
         if (tid < HS / 2) {
             const uint32_t i = tid;
             if (a.rope_variant == SLAI_ROPE_NEOX) { e0 = i; e1 = i + HS / 2; } else { e0 = 2 * i; e1 = 2 * i + 1; }
-            q0 = a.q[(size_t)h * HS + e0]; q1 = a.q[(size_t)h * HS + e1];
+            if constexpr (FLOW) { q0 = flow_load(a.q + (size_t)h * HS + e0); q1 = flow_load(a.q + (size_t)h * HS + e1); }
+            else { q0 = a.q[(size_t)h * HS + e0]; q1 = a.q[(size_t)h * HS + e1]; }
             if (fresh) {
                 if (a.qbias) { q0 += a.qbias[(size_t)h * HS + e0]; q1 += a.qbias[(size_t)h * HS + e1]; }
                 if (rot && a.rope_theta) theta = a.rope_theta[i];
                 if (own_new) {
-                    k0 = a.knew[hoff + e0]; k1 = a.knew[hoff + e1];
-                    v0 = a.vnew[hoff + e0]; v1 = a.vnew[hoff + e1];
+                    if constexpr (FLOW) {
+                        k0 = flow_load(a.knew + hoff + e0); k1 = flow_load(a.knew + hoff + e1);
+                        v0 = flow_load(a.vnew + hoff + e0); v1 = flow_load(a.vnew + hoff + e1);
+                    } else {
+                        k0 = a.knew[hoff + e0]; k1 = a.knew[hoff + e1];
+                        v0 = a.vnew[hoff + e0]; v1 = a.vnew[hoff + e1];
+                    }
                     if (a.kbias) { k0 += a.kbias[hoff + e0]; k1 += a.kbias[hoff + e1]; }
                     if (a.vbias) { v0 += a.vbias[hoff + e0]; v1 += a.vbias[hoff + e1]; }
                 }
@@ -297,6 +305,8 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
                 } else {
                     slot[e & 3u] = r / l;
                 }
+            } else if constexpr (FLOW) {
+                flow_store(a.out + e, r / l);
             } else {
                 a.out[e] = r / l;
             }

@@ -83,6 +83,8 @@ struct slai_ctx {
     // addresses, so a block is only freed with the context.
     std::vector<void *> retired_scratch;
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
+    // SLAI_PERSISTENT=0: never the one-launch-per-token form of the Llama-2 layer stack
+    bool persistent = true;
     bool use_graph = true;  // SLAI_NO_GRAPH=1 replays the token sequence eagerly (profilers that cannot trace graph launches)
 };
 
@@ -378,5 +380,41 @@ int attention_describe(slai_ctx *ctx, const char *fn, const slai_attn_params *pa
 // Looks up, once per device and with that device current, where this device keeps the static scratch array of
 // slai_attention_static (called by slai_ctx_create).
 hipError_t attention_static_setup(int device);
+
+
+// ---- the whole layer stack of a Llama-2 token in one resident launch (kernels_decode_persistent.hip) ----------------------
+struct PersistentLayer {                 // one per layer, in device memory
+    const uint8_t *wq, *wk, *wv;         // 64-row tiles; K-quant formats tq / tk / tv
+    const uint8_t *wo;                   // 16-row tiles, Q4_K or Q6_K (to)
+    const uint8_t *wgate, *wup;          // 64-row tiles, both Q4_K (tg)
+    const uint8_t *wdown;                // 16-row tiles, Q4_K or Q6_K (td)
+    const float *attn_norm, *ffn_norm;
+    const float *bq, *bk, *bv;           // optional biases
+    void *kcache, *vcache;               // [seq_len][dim]
+    int tq, tk, tv, to, tg, td;
+};
+struct PersistentParams {
+    const PersistentLayer *layers;
+    uint32_t n_layers, dim, hidden, n_heads, seq_len, vocab;
+    float eps;
+    int rope_variant; float rope_base; const float *rope_theta;
+    int kv_f16;
+    const uint8_t *wout; int tout; const float *out_norm;     // output matrix (64-row tiles) and the final norm
+    const float *x;                      // the embedding row of the token (written by the launch before this one)
+    float *logits;
+    const uint32_t *pos_ptr;
+    // hand-off buffers, filled with FLOW_EMPTY before every launch: xa [(n_layers + 1) x dim] (layer inputs; row 0 unused),
+    // xb, xm [n_layers x dim] (attention output, residual after the attention), hb [n_layers x hidden]
+    float *xa, *xb, *xm, *hb;
+    float *slots; uint32_t slot_stride;  // per-workgroup staging of the normalised input of a 64-row-tile phase
+    float *q, *kcol, *vcol;              // q / k / v of the current layer (handed over inside one XCD)
+    uint32_t *counters;                  // one 128-byte line per head
+    uint32_t *abort_flag;                // set when a reader gave up
+    uint64_t *trace;                     // optional: per workgroup 16 * n_layers + 8 time stamps (100 MHz clock); null = none
+};
+size_t persistent_smem_bytes(const PersistentParams &p);
+hipError_t persistent_capacity(const PersistentParams &p, int device, uint32_t *resident);
+hipError_t launch_flow_fill(hipStream_t s, void *buf, size_t bytes);
+hipError_t launch_decode_persistent(hipStream_t s, const PersistentParams &p, uint32_t grid);
 
 }  // namespace slai

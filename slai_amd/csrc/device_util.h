@@ -18,6 +18,25 @@ template <int BYTES> __device__ __forceinline__ void touch_kernel_arguments() {
     asm volatile("" : : "s"(w));
 }
 
+// ---- data exchanged between workgroups of one running kernel ---------------------------------------------------------
+// The eight dies of the device have an L2 each, and a die's L2 is not kept coherent with what other dies write while a
+// kernel runs.  Accesses at agent scope (the sc1 cache-policy bit) are: a store is written through to memory, a load does
+// not take a line that another die may since have changed.  Producer and consumer workgroups of one launch therefore
+// exchange data with these accesses only, and the data itself says when it has arrived: the buffers are filled with
+// FLOW_EMPTY (a NaN no computation produces) before the launch, and a reader repeats its load until no element is empty.
+constexpr uint32_t FLOW_EMPTY = 0xFFFFFFFFu;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float flow_load(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void flow_store(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// 16 bytes at once (the compiler has no 16-byte atomic): the load is issued and waited for
+__device__ __forceinline__ u32x4 flow_load16(const void *p) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void flow_store16(void *p, u32x4 v) { asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory"); }
+__device__ __forceinline__ bool flow_empty(u32x4 v) { return v.x == FLOW_EMPTY || v.y == FLOW_EMPTY || v.z == FLOW_EMPTY || v.w == FLOW_EMPTY; }
+
 // A value as an f16 head plus an f16 remainder (both rounded toward zero; value - head is exact in f32), about
 // 22 bits together: the form in which the prompt-chunk GEMM reads activations for the half-precision matrix cores.
 // split_quad packs four values as {heads 0-1, heads 2-3, remainders 0-1, remainders 2-3} into the 16 bytes of the float4.

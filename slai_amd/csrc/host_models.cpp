@@ -171,6 +171,18 @@ struct slai_llama2 {
     int launch(LlmContext &ctxt, const slai_attn_params &attn_params, uint32_t pos);   // transformer.rs:316-381
     int enqueue_fused(int sampler);   // 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state
 
+    // The layer stack as ONE resident launch per token (kernels_decode_persistent.hip), for the models it covers.
+    struct {
+        bool ready = false;
+        uint32_t grid = 0;
+        PersistentParams params{};
+        slai_buffer *layers = nullptr, *flow = nullptr, *slots = nullptr;
+        size_t flow_bytes = 0;
+    } persistent;
+    bool persistent_supported() const;
+    int persistent_setup();
+    int enqueue_persistent(int sampler);
+
     // Prompt tokens in chunks: every weight matrix is read once per chunk instead of once per token.
     PromptChunkState chunk;
     bool chunk_supported() const;        // per-token workgroups over shared weights (any tiled format)
@@ -322,7 +334,98 @@ int slai_llama2::load(const slai_gguf *gg) {
     attn_splits = pick_attn_splits(ctx, config.n_q_heads, config.seq_len);
     TRY(ensure_attn_scratch(ctx, attention_scratch_floats(config.n_q_heads, head_size(), attn_splits)));
     TRY(loop_init(ctx, loop, config.seq_len + 1));
+    TRY(persistent_setup());
     return slai_synchronize(ctx);
+}
+
+// The resident launch covers the shapes of the headline configuration and its smaller relatives: as many cache heads as
+// query heads of size 128, a width of 1024 .. 4096 in steps of 1024, a context one workgroup per head can walk, q / k / v,
+// gate / up and the output matrix in 64-row tiles of K-quants (gate and up both Q4_K), the two projections into the
+// residual in 16-row tiles of Q4_K or Q6_K.  Everything else keeps the launch-per-step form.
+bool slai_llama2::persistent_supported() const {
+    const uint32_t dim = config.dim, hid = config.hidden_dim, nh = config.n_q_heads;
+    if (!ctx->persistent || !ctx->fuse_qkv_attention || !ctx->rowtile_gemv || !ctx->handoff_counters || nh > ctx->handoff_heads) return false;
+    if (config.n_kv_heads != nh || head_size() != 128 || nh % 8 || dim % 1024 || dim > 4096 || hid % 256 || hid / 256 > 64 || attn_splits != 1 || config.seq_len > 1024)
+        return false;
+    const auto kquant = [](int t) { return t == T_Q4_K || t == T_Q5_K || t == T_Q6_K; };
+    const auto proj = [&](const slai_qmat *m, uint32_t cols) {
+        return m->tiled && m->rows_log2 == 4 && (m->type == T_Q4_K || m->type == T_Q6_K) && m->ncb == cols / 256 && m->ngroups == (cols / 256 + 3) / 4 && m->ngroups <= 16;
+    };
+    for (const Llama2LayerWeights &w : weights.layers) {
+        for (const slai_qmat *m : {w.attn_q, w.attn_k, w.attn_v})
+            if (!gemv_is_rowtile(ctx, m) || !kquant(m->type) || m->ncb != dim / 256) return false;
+        if (!gemv_is_rowtile(ctx, w.ffn_gate) || !gemv_is_rowtile(ctx, w.ffn_up) || w.ffn_gate->type != T_Q4_K || w.ffn_up->type != T_Q4_K) return false;
+        if (!proj(w.attn_output, dim) || !proj(w.ffn_down, hid)) return false;
+    }
+    return gemv_is_rowtile(ctx, weights.output) && kquant(weights.output->type) && weights.output->ncb == dim / 256;
+}
+
+int slai_llama2::persistent_setup() {
+    if (!persistent_supported()) return SLAI_OK;
+    const uint32_t dim = config.dim, hid = config.hidden_dim, nh = config.n_q_heads, nl = config.n_layers;
+    PersistentParams &p = persistent.params;
+    p.n_layers = nl; p.dim = dim; p.hidden = hid; p.n_heads = nh; p.seq_len = config.seq_len; p.vocab = config.vocab_size;
+    p.eps = config.rms_norm_eps; p.rope_variant = rope_variant(); p.rope_base = config.rope_base_freq;
+    p.rope_theta = (const float *)state.rope_theta.buf->dptr;
+    p.kv_f16 = kv_dtype == SLAI_KV_F16;
+    p.wout = weights.output->dptr; p.tout = weights.output->type; p.out_norm = (const float *)weights.output_norm.buf->dptr;
+    p.x = (const float *)state.x.buf->dptr; p.logits = (float *)state.logits.buf->dptr;
+    p.pos_ptr = (const uint32_t *)&((DecodeState *)loop.state->dptr)->pos;
+    p.q = (float *)state.q.buf->dptr; p.kcol = (float *)state.kcol.buf->dptr; p.vcol = (float *)state.vcol.buf->dptr;
+    p.counters = ctx->handoff_counters; p.abort_flag = ctx->handoff_counters + (size_t)ctx->handoff_heads * 32;
+    // the device must keep the whole grid resident: every compute unit one workgroup, and enough of them for every role
+    uint32_t resident = 0;
+    if (persistent_capacity(p, ctx->device, &resident) != hipSuccess) return SLAI_OK;
+    const uint32_t need = std::max(std::max(7 * nh, dim / 16), hid / 64);
+    hipDeviceProp_t prop;
+    SLAI_HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    const uint32_t grid = std::min(resident, (uint32_t)prop.multiProcessorCount) / 8 * 8;
+    if (grid < need) return SLAI_OK;
+    std::vector<PersistentLayer> host(nl);
+    for (uint32_t l = 0; l < nl; ++l) {
+        const Llama2LayerWeights &w = weights.layers[l];
+        PersistentLayer &d = host[l];
+        d.wq = w.attn_q->dptr; d.wk = w.attn_k->dptr; d.wv = w.attn_v->dptr; d.tq = w.attn_q->type; d.tk = w.attn_k->type; d.tv = w.attn_v->type;
+        d.wo = w.attn_output->dptr; d.to = w.attn_output->type;
+        d.wgate = w.ffn_gate->dptr; d.wup = w.ffn_up->dptr; d.tg = w.ffn_gate->type;
+        d.wdown = w.ffn_down->dptr; d.td = w.ffn_down->type;
+        d.attn_norm = (const float *)w.attn_norm.buf->dptr; d.ffn_norm = (const float *)w.ffn_norm.buf->dptr;
+        d.bq = w.attn_q_bias.buf ? (const float *)w.attn_q_bias.buf->dptr : nullptr;
+        d.bk = w.attn_k_bias.buf ? (const float *)w.attn_k_bias.buf->dptr : nullptr;
+        d.bv = w.attn_v_bias.buf ? (const float *)w.attn_v_bias.buf->dptr : nullptr;
+        d.kcache = state.key_cache[l].buf->dptr; d.vcache = state.value_cache[l].buf->dptr;
+    }
+    TRY(slai_buffer_create(ctx, host.size() * sizeof(PersistentLayer), SLAI_DT_U8, STORAGE | COPY_DST, &persistent.layers));
+    TRY(slai_write_buffer(ctx, persistent.layers, 0, host.data(), host.size() * sizeof(PersistentLayer)));
+    persistent.flow_bytes = ((size_t)(3 * nl + 1) * dim + (size_t)nl * hid) * sizeof(float);
+    TRY(slai_buffer_create(ctx, persistent.flow_bytes, SLAI_DT_F32, STORAGE, &persistent.flow));
+    p.slot_stride = dim + dim / 16 + 16;
+    TRY(slai_buffer_create(ctx, (size_t)grid * p.slot_stride * sizeof(float), SLAI_DT_F32, STORAGE, &persistent.slots));
+    p.layers = (const PersistentLayer *)persistent.layers->dptr;
+    p.xa = (float *)persistent.flow->dptr;
+    p.xb = p.xa + (size_t)(nl + 1) * dim;
+    p.xm = p.xb + (size_t)nl * dim;
+    p.hb = p.xm + (size_t)nl * dim;
+    p.slots = (float *)persistent.slots->dptr;
+    persistent.grid = grid;
+    persistent.ready = true;
+    return SLAI_OK;
+}
+
+// embedding row | hand-off buffers emptied | the layer stack and the output matrix | pick
+int slai_llama2::enqueue_persistent(int sampler) {
+    Llama2State &s = state;
+    DecodeState *ds = (DecodeState *)loop.state->dptr;
+    SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, &ds->token, nullptr, nullptr, config.dim, (float *)s.x.buf->dptr));
+    SLAI_HIP_TRY(ctx, launch_flow_fill(ctx->stream, persistent.flow->dptr, persistent.flow_bytes));
+    SLAI_HIP_TRY(ctx, launch_decode_persistent(ctx->stream, persistent.params, persistent.grid));
+    if (sampler == 1)
+        SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, nullptr, ds,
+                                        (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
+    else if (sampler == 2)
+        SLAI_HIP_TRY(ctx, launch_sample(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, 0.0f, 0.0f, 0.0f, ctx->sampler_scratch, nullptr, ds,
+                                        (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
+    return SLAI_OK;
 }
 
 // `Llama2::launch` (transformer.rs:316-381), one kernel per op in the reference's order.
@@ -368,6 +471,7 @@ int slai_llama2::launch(LlmContext &ctxt, const slai_attn_params &attn_params, u
 //   embedding-row gather | per layer: [RMSNorm+QKV GEMV] [RoPE+cache write+attention] [Wo GEMV+residual]
 //   [RMSNorm+gate/up GEMV+SiLU] [down GEMV+residual] | [RMSNorm+logits GEMV] [argmax + loop state]
 int slai_llama2::enqueue_fused(int sampler) {
+    if (persistent.ready) return enqueue_persistent(sampler);
     Llama2State &s = state;
     DecodeState *ds = (DecodeState *)loop.state->dptr;
     float *x = (float *)s.x.buf->dptr, *xb = (float *)s.xb.buf->dptr, *hb = (float *)s.hb.buf->dptr, *hb2 = (float *)s.hb2.buf->dptr;
@@ -769,10 +873,40 @@ SLAI_EXPORT void slai_llama2_destroy(slai_llama2 *m) {
     for (auto &t : s.key_cache) t.destroy(ctx);
     for (auto &t : s.value_cache) t.destroy(ctx);
     for (slai_buffer *b : {s.rope_config, s.rms_norm_config, s.attn_params}) if (b) slai_buffer_destroy(ctx, b);
+    for (slai_buffer *b : {m->persistent.layers, m->persistent.flow, m->persistent.slots}) if (b) slai_buffer_destroy(ctx, b);
     PromptChunkState &pc = m->chunk;
     for (GpuTensor *t : {&pc.x, &pc.xw, &pc.xb, &pc.q, &pc.k, &pc.v, &pc.hb, &pc.xn, &pc.hb2}) t->destroy(ctx);
     for (slai_buffer *b : {pc.positions, pc.tokens}) if (b) slai_buffer_destroy(ctx, b);
     delete m;
+}
+
+SLAI_EXPORT int slai_llama2_decode_form(const slai_llama2 *m) { return m && m->persistent.ready ? 1 : 0; }
+
+// One token at (pos, token) through the resident launch with its time stamps switched on: per workgroup 16 stamps per
+// layer (four per phase: entered, input staged, multiplied, reduced) and 8 for the output matrix, in ticks of the
+// constant 100 MHz clock.  The caches are left as any forward pass at that position leaves them.
+SLAI_EXPORT int slai_llama2_trace_token(slai_llama2 *m, uint32_t pos, uint32_t token, uint64_t *out, size_t capacity, uint32_t *n_workgroups,
+                                        uint32_t *stamps_per_workgroup) {
+    if (!m || !out || !n_workgroups || !stamps_per_workgroup) return SLAI_E_ARG;
+    slai_ctx *ctx = m->ctx;
+    if (!m->persistent.ready) return set_error(ctx, SLAI_E_STATE, "slai_llama2_trace_token: this model does not take the resident launch");
+    if (pos >= m->config.seq_len || token >= m->config.vocab_size) return set_error(ctx, SLAI_E_ARG, "slai_llama2_trace_token: position or token out of range");
+    const uint32_t stride = 16 * m->config.n_layers + 8, grid = m->persistent.grid;
+    const size_t n = (size_t)grid * stride;
+    if (capacity < n) return set_error(ctx, SLAI_E_SHAPE, "slai_llama2_trace_token: need room for " + std::to_string(n) + " stamps");
+    slai_buffer *buf = nullptr;
+    TRY(slai_buffer_create(ctx, n * 8, SLAI_DT_U8, STORAGE | COPY_SRC, &buf));
+    DecodeState ds{(int)pos, (int)token, 0, 0};
+    int rc = slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds);
+    m->persistent.params.trace = (uint64_t *)buf->dptr;
+    if (!rc) rc = m->enqueue_persistent(0);
+    m->persistent.params.trace = nullptr;
+    if (!rc) rc = slai_synchronize(ctx);
+    if (!rc) rc = handoff_check(ctx);
+    if (!rc) rc = slai_read_buffer(ctx, buf, 0, out, n * 8);
+    slai_buffer_destroy(ctx, buf);
+    *n_workgroups = grid; *stamps_per_workgroup = stride;
+    return rc;
 }
 
 SLAI_EXPORT int slai_llama2_get_config(const slai_llama2 *m, slai_llama2_config *out) {

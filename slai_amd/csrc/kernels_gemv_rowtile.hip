@@ -19,77 +19,13 @@
 #include "common.h"
 #include "attention_fast.h"
 #include "device_util.h"
+#include "gemv_operands.h"
 #include "quant_tiled.h"
 
 namespace slai {
 namespace {
 
-typedef const float __attribute__((address_space(4))) cfloat;   // constant address space: scalar loads
-
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-__device__ __forceinline__ float gelu_f(float x) {
-    const float GELU_COEF_A = 0.044715f, SQRT_2_OVER_PI = 0.7978846f;   // ops/unary.rs:81-85
-    return 0.5f * x * (1.0f + tanhf(SQRT_2_OVER_PI * x * (1.0f + GELU_COEF_A * x * x)));
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-    return v;
-}
-
-typedef float fx16 __attribute__((ext_vector_type(16)));
-typedef const fx16 __attribute__((address_space(4))) cfx16;
-
-// Activations of one super-block, wave-uniform, fetched through the scalar cache one stage ahead of their use.
-struct ScalarX {
-    cfloat *x;   // 256 activations
-    cfloat *s;   // 16 sums of 16 consecutive activations
-    struct St { fx16 a, b; };
-    template <int I1, int I2> __device__ __forceinline__ St stage() const {
-        return St{*(cfx16 *)(x + 16 * I1), *(cfx16 *)(x + 16 * I2)};
-    }
-    // acc += sum_b byte_b(w) * x[16*I_SLOT + 4*W + b].  The conversions are spelled out because the compiler
-    // otherwise extracts bytes 1..3 with a bit-field instruction first.
-    template <int SLOT, int W> __device__ __forceinline__ float fma4(const St &st, uint32_t w, float acc) const {
-        float t0, t1, t2, t3;
-        asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(t0) : "v"(w));
-        asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(t1) : "v"(w));
-        asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(t2) : "v"(w));
-        asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(t3) : "v"(w));
-        const fx16 &c = SLOT ? st.b : st.a;
-        acc = fmaf(t0, c[4 * W], acc);
-        acc = fmaf(t1, c[4 * W + 1], acc);
-        acc = fmaf(t2, c[4 * W + 2], acc);
-        acc = fmaf(t3, c[4 * W + 3], acc);
-        return acc;
-    }
-    __device__ __forceinline__ float sum16(int i) const { return s[i]; }
-};
-
-// Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product.
-template <int T, int N> struct UnitLoader {
-    static constexpr int DEPTH = 1;               // stages requested ahead of the one being multiplied
-    static constexpr int LEAD = 1;                // stages requested before the dot product starts (>= DEPTH)
-    using F = Tiled<T>;
-    const uint8_t *unit[N];                       // + lane * 16 already applied
-    const uint8_t *tailp[N];
-    typename F::Data *d[N];
-    uint16_t *t[N];
-    template <int P> __device__ __forceinline__ void piece() const {
-#pragma unroll
-        for (int n = 0; n < N; ++n) d[n]->p[P] = ld128(unit[n] + (size_t)P * 1024);
-    }
-    __device__ __forceinline__ void tail() const {
-#pragma unroll
-        for (int n = 0; n < N; ++n) *t[n] = ld16(tailp[n]);
-    }
-};
+using namespace lanes;
 
 // The body for one block format.  `partial` = [DUAL?2:1][NW][64] floats, `red` = [NW] floats.
 template <int T, bool DUAL, bool PREP>
@@ -118,7 +54,7 @@ __device__ __forceinline__ void tile_body(const GemvRowtileParams &p, const Gemv
     uint16_t dt = 0, et = 0;
     uint32_t cb = wave;
     constexpr int NM = DUAL ? 2 : 1;
-    UnitLoader<T, NM> ld;
+    UnitLoader<T, NM, 1> ld;
     auto point = [&]() {                                      // aim the loader at super-block cb of this tile
         const size_t off = ((size_t)tile * p.ncb + cb) * unit_bytes;
         ld.unit[0] = seg.W + off + lane * 16; ld.tailp[0] = seg.W + off + (size_t)F::PT * 1024 + lane * 2; ld.d[0] = &d; ld.t[0] = &dt;

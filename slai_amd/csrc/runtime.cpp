@@ -90,6 +90,7 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->tiled_layout = env_int("SLAI_TILED", 1) != 0;
     ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
     ctx->fuse_qkv_attention = env_int("SLAI_FUSE_QKV_ATTN", 1) != 0;
+    ctx->persistent = env_int("SLAI_PERSISTENT", 0) != 0;
     *out = ctx;
     return SLAI_OK;
 }
@@ -446,8 +447,9 @@ int handoff_check(slai_ctx *ctx) {
     uint32_t flag = 0;
     SLAI_HIP_TRY(ctx, hipMemcpy(&flag, ctx->handoff_counters + (size_t)ctx->handoff_heads * 32, sizeof flag, hipMemcpyDeviceToHost));
     if (flag) {
-        // reported once: the slot is cleared so that later, healthy calls are not failed for an old time-out
-        (void)hipMemset(ctx->handoff_counters + (size_t)ctx->handoff_heads * 32, 0, sizeof flag);
+        // reported once: the slot is cleared so that later, healthy calls are not failed for an old time-out, and so are
+        // the per-head counters, which a launch that gave up may have left anywhere
+        (void)hipMemset(ctx->handoff_counters, 0, ((size_t)ctx->handoff_heads * 32 + 32) * sizeof(uint32_t));
         return set_error(ctx, SLAI_E_HIP, "q/k/v -> attention hand-off timed out inside a launch; results are invalid");
     }
     return SLAI_OK;

@@ -533,6 +533,19 @@ class Llama2:
                                                            seed, out.ctypes.data, C.byref(ms)))
         return out, ms.value
 
+    def decode_form(self):
+        """0: one launch per step of the layer loop, 1: the whole layer stack in one resident launch per token."""
+        return int(self.b.L.slai_llama2_decode_form(self.h))
+
+    def trace_token(self, pos, token):
+        """In-kernel time stamps of one token through the resident launch: uint64 [workgroups, 16 * n_layers + 8], ticks of
+        the 100 MHz clock (see slai_llama2_trace_token)."""
+        grid, stride = C.c_uint32(), C.c_uint32()
+        cap = 4096 * (16 * self.config.n_layers + 8)
+        out = np.zeros(cap, dtype=np.uint64)
+        self.b.check(self.b.L.slai_llama2_trace_token(self.h, pos, token, out.ctypes.data, cap, C.byref(grid), C.byref(stride)))
+        return out[:grid.value * stride.value].reshape(grid.value, stride.value)
+
     def prefill_path(self):
         """2: matrix-core GEMM, 1: per-token workgroups over shared weights, 0: the token-by-token loop."""
         return int(self.b.L.slai_llama2_prefill_supported(self.h))
