@@ -93,9 +93,8 @@ __device__ __forceinline__ void flow_probe(const float *probe, Flow &f) {
 template <int N>
 __device__ __forceinline__ void flow_acquire(const float *base, uint32_t off0, uint32_t stride, uint32_t nlive, u32x4 (&v)[N], Flow &f) {
     static_assert(N == 4 || N == 12, "four or twelve pieces");
-    const uint64_t base_bits = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)base >> 32)) << 32) |
-                               __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)base);
-    const uint32_t st = __builtin_amdgcn_readfirstlane(stride);
+    const uint64_t base_bits = join_words(uniform_word((uint32_t)(uintptr_t)base), uniform_word((uint32_t)((uintptr_t)base >> 32)));
+    const uint32_t st = uniform_word(stride);
 #pragma unroll
     for (int k = 0; k < N; ++k) v[k] = u32x4{0, 0, 0, 0};
     uint64_t deadline = 0;
@@ -398,9 +397,8 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
         // this layer's description comes out of LDS field by field, as wave-uniform values, where it is used; the next
         // one's is requested now and parked in LDS at the end of the layer
         const uint32_t *lw = layer_words[l & 1u];
-#define LPTR(T, field) ((T)(uintptr_t)((uint64_t)__builtin_amdgcn_readfirstlane(lw[offsetof(PersistentLayer, field) / 4]) | \
-                                       ((uint64_t)__builtin_amdgcn_readfirstlane(lw[offsetof(PersistentLayer, field) / 4 + 1]) << 32)))
-#define LINT(field) ((int)__builtin_amdgcn_readfirstlane(lw[offsetof(PersistentLayer, field) / 4]))
+#define LPTR(T, field) ((T)(uintptr_t)join_words(uniform_word(lw[offsetof(PersistentLayer, field) / 4]), uniform_word(lw[offsetof(PersistentLayer, field) / 4 + 1])))
+#define LINT(field) ((int)uniform_word(lw[offsetof(PersistentLayer, field) / 4]))
         uint32_t next_word = 0;
         if (threadIdx.x < LWORDS && l + 1 < p.n_layers) next_word = reinterpret_cast<const uint32_t *>(p.layers + l + 1)[threadIdx.x];
         uint64_t *tl = trace ? trace + 16 * l : nullptr;
