@@ -68,6 +68,27 @@ struct ScalarX {
         return acc;
     }
     __device__ __forceinline__ float sum16(int i) const { return s[i]; }
+    // Eight 4-bit weights of one word at once, without converting them: a nibble n left in the low bits of a 16-bit half
+    // is the half-precision subnormal n * 2^-24 (in bits 4..7: 16 n * 2^-24), and v_fma_mix_f32 multiplies such a half
+    // by the f32 activation into an f32 sum.  Low nibbles (chunk I1) go to `lo`, high nibbles (chunk I2) to `hi`, in the
+    // element order of fma4, so `lo` ends as 2^-24 and `hi` as 2^-20 times what fma4 gives -- exactly, powers of two
+    // commute with every rounding here -- and the caller folds the factors into the block scale.
+    static constexpr bool NIBBLE_MIX = true;
+    template <int HALF> static __device__ __forceinline__ float mix(uint32_t halves, float xs, float acc) {
+        float o;
+        if constexpr (HALF == 0) asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(o) : "v"(halves), "s"(xs), "v"(acc));
+        else asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(o) : "v"(halves), "s"(xs), "v"(acc));
+        return o;
+    }
+    template <int W> __device__ __forceinline__ void nib8(const St &st, uint32_t w, float &lo, float &hi) const {
+        const uint32_t b02l = w & 0x000F000Fu, b02h = w & 0x00F000F0u;      // bytes 0 and 2
+        const uint32_t t = w >> 8;
+        const uint32_t b13l = t & 0x000F000Fu, b13h = t & 0x00F000F0u;      // bytes 1 and 3
+        lo = mix<0>(b02l, st.a[4 * W], lo);     hi = mix<0>(b02h, st.b[4 * W], hi);
+        lo = mix<0>(b13l, st.a[4 * W + 1], lo); hi = mix<0>(b13h, st.b[4 * W + 1], hi);
+        lo = mix<1>(b02l, st.a[4 * W + 2], lo); hi = mix<1>(b02h, st.b[4 * W + 2], hi);
+        lo = mix<1>(b13l, st.a[4 * W + 3], lo); hi = mix<1>(b13h, st.b[4 * W + 3], hi);
+    }
 };
 
 // Activations of a super-block held in 16 registers of a 16-lane DPP row.
@@ -79,6 +100,7 @@ struct DevX {
     // Written as assembly: the compiler forms DPP operands only on two-address encodings, which an FMA
     // does not have before register allocation, and it would otherwise hoist all 256 conversions of a
     // super-block ahead of the FMAs and run out of registers.
+    static constexpr bool NIBBLE_MIX = false;
     template <int I1, int I2> struct St {};                   // activations are register resident: a stage is a tag
     template <int I1, int I2> __device__ __forceinline__ St<I1, I2> stage() const { return {}; }
     template <int SLOT, int W, int I1, int I2> __device__ __forceinline__ float fma4(St<I1, I2>, uint32_t w, float acc) const {

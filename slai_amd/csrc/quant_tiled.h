@@ -221,12 +221,20 @@ template <> struct Tiled<T_Q4_K> {
         constexpr int J = K / 2, H = K % 2;
         for (int n = 0; n < N; ++n) {
             const U4 &q = d[n]->p[1 + K];
-            stage_dot(x, st, and4(q, 0x0F0F0F0Fu), and4(shr4(q, 4), 0x0F0F0F0Fu), a.slo[n], a.shi[n]);
+            // (operands that take the nibbles unconverted leave slo scaled by 2^-24 and shi by 2^-20: the 16 is taken
+            // out of the high sub-block's scale here, the 2^-24 out of the block scale in dotn)
+            if constexpr (X::NIBBLE_MIX) {
+                x.template nib8<0>(st, q.x, a.slo[n], a.shi[n]); x.template nib8<1>(st, q.y, a.slo[n], a.shi[n]);
+                x.template nib8<2>(st, q.z, a.slo[n], a.shi[n]); x.template nib8<3>(st, q.w, a.slo[n], a.shi[n]);
+            } else {
+                stage_dot(x, st, and4(q, 0x0F0F0F0Fu), and4(shr4(q, 4), 0x0F0F0F0Fu), a.slo[n], a.shi[n]);
+            }
             if (H == 1) {
                 const uint32_t scw = J < 2 ? a.sc_lo[n] : a.sc_hi[n];
                 constexpr int sh = (J & 1) * 16;
+                constexpr float hi_factor = X::NIBBLE_MIX ? 0.0625f : 1.0f;
                 a.accd[n] = fmaf((float)((scw >> sh) & 0xffu), a.slo[n], a.accd[n]);
-                a.accd[n] = fmaf((float)((scw >> (sh + 8)) & 0xffu), a.shi[n], a.accd[n]);
+                a.accd[n] = fmaf((float)((scw >> (sh + 8)) & 0xffu) * hi_factor, a.shi[n], a.accd[n]);
                 a.slo[n] = 0.0f; a.shi[n] = 0.0f;
             }
         }
@@ -270,7 +278,8 @@ template <> struct Tiled<T_Q4_K> {
         }
         const auto st0 = x.template stage<c1(0), c2(0)>();
         stages<0, N>(d, x, st0, a, ld);
-        for (int n = 0; n < N; ++n) out[n] = dd[n] * a.accd[n] - dmin[n] * accm[n];
+        constexpr float unit = X::NIBBLE_MIX ? 16777216.0f : 1.0f;             // accd is in units of 2^-24 there
+        for (int n = 0; n < N; ++n) out[n] = (dd[n] * unit) * a.accd[n] - dmin[n] * accm[n];
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
         const Data *dp[1] = {&d};
