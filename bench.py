@@ -109,10 +109,18 @@ def counter_probe(backend):
                       "gemv_launch_us": round(ms * 1000, 2)}))
 
 
+EAGER = False        # --eager: launch from the host instead of replaying a HIP graph (for runs under the kernel tracer)
+
+
 def graph_time_us(backend, enqueue, n_launches, reps=20):
     """Mean time per launch of `enqueue` (which issues n_launches kernels) captured in a HIP graph and replayed."""
     enqueue()                                   # eager once: sizes scratch buffers outside the capture
     backend.synchronize()
+    if EAGER:
+        backend.timer_begin()
+        for _ in range(reps):
+            enqueue()
+        return backend.timer_end() * 1000.0 / (reps * n_launches)
     backend.graph_begin_capture()
     enqueue()
     g = backend.graph_end_capture()
@@ -135,6 +143,15 @@ def sweep(backend):
     ctxt = LlmContext(backend)
     names = {2: "Q4_0", 12: "Q4_K", 13: "Q5_K", 14: "Q6_K", 8: "Q8_0"}
     rows = []
+    if EAGER:
+        # under a profiler: a plain copy of known size first (64 MiB read, 64 MiB written per launch), against which
+        # the byte counters of the other kernels are scaled
+        n = 16 * 1024 * 1024
+        ca, cb = GpuTensor(backend, n), GpuTensor(backend, n)
+        for _ in range(16):
+            ctxt.copy(ca, cb)
+        backend.synchronize()
+        ca.destroy(); cb.destroy()
     for (nrows, ncols) in ((4096, 4096), (11008, 4096)):
         for t in (2, 12, 13, 14, 8):
             base = synth.normal_quantized(4242 + t, t, nrows, ncols, 0.02)
@@ -319,12 +336,15 @@ def main():
     ap.add_argument("--no-side", action="store_true", help="only the headline decode (no sampled decode, prompt chunks, config 5)")
     ap.add_argument("--probe", action="store_true", help="counter probe: copy kernel + dominant GEMV only")
     ap.add_argument("--sweep", action="store_true", help="per-format GEMV sweep and long-context attention instead of the decode run")
+    ap.add_argument("--eager", action="store_true", help="with --sweep: launch from the host, no HIP graph (the kernel tracer cannot follow graph launches here)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the decode path on ONE GPU (batch-1 decode does not shard usefully); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
     if args.probe or args.sweep:
+        global EAGER
+        EAGER = args.eager
         from slai_amd.runtime import Backend
         backend = Backend(0)
         if args.probe:

@@ -347,7 +347,6 @@ hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p, const GemvBat
         p.seg[i].ntiles = (p.seg[i].nrows + 63) / 64;
         tiles += p.seg[i].ntiles;
         if (p.seg[i].flags & GEMV_SILU_GATE) dual = true;
-        if ((p.seg[i].flags & GEMV_SILU_GATE) && t == T_Q8_0) return hipErrorInvalidValue;
     }
     for (int i = 0; i < p.nseg; ++i)
         if (dual != ((p.seg[i].flags & GEMV_SILU_GATE) != 0)) return hipErrorInvalidValue;
@@ -366,7 +365,7 @@ hipError_t launch_gemv_rowtile(slai_ctx *ctx, GemvRowtileParams p, const GemvBat
     switch (tt) {
     case T_Q4_K: return dual ? go<T_Q4_K, true>(p, tiles, NT, smem, st, bt) : go<T_Q4_K, false>(p, tiles, NT, smem, st, bt);
     case T_Q6_K: return dual ? go<T_Q6_K, true>(p, tiles, NT, smem, st, bt) : go<T_Q6_K, false>(p, tiles, NT, smem, st, bt);
-    case T_Q8_0: return go<T_Q8_0, false>(p, tiles, NT, smem, st, bt);
+    case T_Q8_0: return dual ? go<T_Q8_0, true>(p, tiles, NT, smem, st, bt) : go<T_Q8_0, false>(p, tiles, NT, smem, st, bt);
     case T_Q4_0: return dual ? go<T_Q4_0, true>(p, tiles, NT, smem, st, bt) : go<T_Q4_0, false>(p, tiles, NT, smem, st, bt);
     case T_Q5_K: return dual ? go<T_Q5_K, true>(p, tiles, NT, smem, st, bt) : go<T_Q5_K, false>(p, tiles, NT, smem, st, bt);
     default: return dual ? go<0, true>(p, tiles, NT, smem, st, bt) : go<0, false>(p, tiles, NT, smem, st, bt);

@@ -391,7 +391,7 @@ bool gemv_is_rowtile(const slai_ctx *ctx, const slai_qmat *m) {
 }
 
 bool gemv_gated_is_rowtile(const slai_ctx *ctx, const slai_qmat *gate, const slai_qmat *up) {
-    return gemv_is_rowtile(ctx, gate) && gemv_is_rowtile(ctx, up) && gate->type == up->type && gate->type != T_Q8_0;
+    return gemv_is_rowtile(ctx, gate) && gemv_is_rowtile(ctx, up) && gate->type == up->type;
 }
 
 // Grows one of the context's scratch blocks.  The block it replaces stays allocated until the context goes: graphs
@@ -468,7 +468,7 @@ int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunc
         const slai_qmat *m = c.m[i], *m2 = c.m2[i];
         rowtile = m && m->tiled && m->rows_log2 == 6 && m->ncols == m0->ncols && m->ncb <= 64 &&
                   (!m2 || (m2->tiled && m2->rows_log2 == 6 && m2->type == m->type && m2->ncols == m->ncols && m2->nrows == m->nrows)) &&
-                  (((c.flags[i] & GEMV_SILU_GATE) != 0) == (m2 != nullptr)) && !(m2 && m->type == T_Q8_0) &&
+                  (((c.flags[i] & GEMV_SILU_GATE) != 0) == (m2 != nullptr)) &&
                   (((c.flags[i] ^ c.flags[0]) & GEMV_SILU_GATE) == 0);
     }
     for (int i = 1; i < c.nseg && rowtile; ++i)

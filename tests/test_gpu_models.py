@@ -174,7 +174,7 @@ def test_generate_works_as_the_first_call_on_a_fresh_context():
 @pytest.mark.parametrize("wtype", [8, 2, 13, 14], ids=["q8_0", "q4_0", "q5_k", "q6_k"])
 def test_llama_tiled_layouts_every_format(backend, wtype):
     """Widths that take the tiled layouts (multiples of 256) in every format that has them, MHA, fp16 cache: logits and
-    greedy ids against the oracle (a gated Q8_0 pair takes the 16-row-tile kernel, the others the 64-row-tile one)."""
+    greedy ids against the oracle."""
     data = gw.llama_gguf(dim=512, hidden_dim=1536, n_layers=3, n_heads=8, n_kv_heads=8, vocab=2048, seq_len=128, wtype=wtype, seed=77,
                          std=0.05, norm_random=True)
     check_llama(backend, data, [5, 1000, 2047, 9, 77, 3], 40, kv_f16=True, check_logit_steps=12)
