@@ -23,7 +23,10 @@
  * ggml layouts + hand-computable blocks + brute force over get_scale_min_k4),
  * the GGUF reader (the reference's own dummy.gguf fixture), rms_norm / softmax /
  * silu / gelu / layernorm / attention / rope (closed forms, torch CPU library
- * routines, invariants), argmax (numpy), whole forward (independent numpy twin).
+ * routines, invariants), argmax (numpy), whole forward (independent numpy twin,
+ * and the `transformers` library's LlamaForCausalLM / Qwen2ForCausalLM /
+ * GPT2LMHeadModel on CPU in float32 with the same seeded weights: logits to
+ * 1e-4 of the largest logit and 32 greedy ids, tests/test_oracle_models_hf.py).
  */
 #include <math.h>
 #include <stdint.h>
