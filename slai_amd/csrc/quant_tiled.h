@@ -26,6 +26,7 @@
 // Block arithmetic follows crates/slai/src/quantization.rs (BlockQ4K :322-379,
 // get_scale_min_k4 :381-389, BlockQ6K :204-244, BlockQ8_0 :29-42).
 #pragma once
+#include <type_traits>
 #include "quant_formats.h"
 
 namespace slai {
@@ -207,6 +208,11 @@ template <class X, class S> SLAI_HD void stage_dot(const X &x, const S &st, cons
     a1 = x.template fma4<0, 3>(st, q1.w, a1); a2 = x.template fma4<1, 3>(st, q2.w, a2);
 }
 
+// Whether an activation operand multiplies 4-bit weights unconverted (its nib8; see ScalarX): operands that do not say
+// so do not.
+template <class X, class = void> struct takes_nibbles : std::false_type {};
+template <class X> struct takes_nibbles<X, std::void_t<decltype(X::NIBBLE_MIX)>> : std::bool_constant<X::NIBBLE_MIX> {};
+
 template <int T> struct Tiled;
 
 template <> struct Tiled<T_Q4_K> {
@@ -223,7 +229,7 @@ template <> struct Tiled<T_Q4_K> {
             const U4 &q = d[n]->p[1 + K];
             // (operands that take the nibbles unconverted leave slo scaled by 2^-24 and shi by 2^-20: the 16 is taken
             // out of the high sub-block's scale here, the 2^-24 out of the block scale in dotn)
-            if constexpr (X::NIBBLE_MIX) {
+            if constexpr (takes_nibbles<X>::value) {
                 x.template nib8<0>(st, q.x, a.slo[n], a.shi[n]); x.template nib8<1>(st, q.y, a.slo[n], a.shi[n]);
                 x.template nib8<2>(st, q.z, a.slo[n], a.shi[n]); x.template nib8<3>(st, q.w, a.slo[n], a.shi[n]);
             } else {
@@ -232,7 +238,7 @@ template <> struct Tiled<T_Q4_K> {
             if (H == 1) {
                 const uint32_t scw = J < 2 ? a.sc_lo[n] : a.sc_hi[n];
                 constexpr int sh = (J & 1) * 16;
-                constexpr float hi_factor = X::NIBBLE_MIX ? 0.0625f : 1.0f;
+                constexpr float hi_factor = takes_nibbles<X>::value ? 0.0625f : 1.0f;
                 a.accd[n] = fmaf((float)((scw >> sh) & 0xffu), a.slo[n], a.accd[n]);
                 a.accd[n] = fmaf((float)((scw >> (sh + 8)) & 0xffu) * hi_factor, a.shi[n], a.accd[n]);
                 a.slo[n] = 0.0f; a.shi[n] = 0.0f;
@@ -278,7 +284,7 @@ template <> struct Tiled<T_Q4_K> {
         }
         const auto st0 = x.template stage<c1(0), c2(0)>();
         stages<0, N>(d, x, st0, a, ld);
-        constexpr float unit = X::NIBBLE_MIX ? 16777216.0f : 1.0f;             // accd is in units of 2^-24 there
+        constexpr float unit = takes_nibbles<X>::value ? 16777216.0f : 1.0f;             // accd is in units of 2^-24 there
         for (int n = 0; n < N; ++n) out[n] = (dd[n] * unit) * a.accd[n] - dmin[n] * accm[n];
     }
     template <class X> SLAI_HD static float dot(const Data &d, uint16_t tail, const X &x) {
