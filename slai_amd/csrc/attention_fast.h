@@ -149,14 +149,14 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
     {
         const uint32_t t = t0 + tid / KL;
         // the fresh row comes from LDS later; lanes without a position read a valid address and are masked
-        const uint32_t tc = (t < t1 && !(own_new && t == pos)) ? t : t0;
+        const uint32_t tc = (t < t1 && !(own_new && t == pos)) ? t : min(t0, pos);
         const CT *kp = kc + (size_t)tc * a.kv_dim + hoff + sub * EPL;
 #pragma unroll
         for (int j = 0; j < EPL / 8; ++j) kv0[j] = Vec8<F16>::load_raw(kp + 8 * j);
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
             const uint32_t tv = t0 + wpos + u * PW + vgl;
-            const uint32_t tvc = (tv < t1 && !(own_new && tv == pos)) ? tv : t0;
+            const uint32_t tvc = (tv < t1 && !(own_new && tv == pos)) ? tv : min(t0, pos);
             vv0[u] = Vec8<F16>::load_raw(vc + (size_t)tvc * a.kv_dim + hoff + ve);
         }
     }
@@ -209,14 +209,14 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
         typename Vec8<F16>::Raw nxt[EPL / 8] = {}, nxtv[NU] = {};
         if (tb + NT / KL < t1) {                               // (uniform) there is a next pass
             const uint32_t tn = t + NT / KL;
-            const uint32_t tnc = (tn < t1 && !(own_new && tn == pos)) ? tn : t0;
+            const uint32_t tnc = (tn < t1 && !(own_new && tn == pos)) ? tn : min(t0, pos);
             const CT *kp = kc + (size_t)tnc * a.kv_dim + hoff + sub * EPL;
 #pragma unroll
             for (int j = 0; j < EPL / 8; ++j) nxt[j] = Vec8<F16>::load_raw(kp + 8 * j);
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
                 const uint32_t tv = tb + NT / KL + wpos + u * PW + vgl;
-                const uint32_t tvc = (tv < t1 && !(own_new && tv == pos)) ? tv : t0;
+                const uint32_t tvc = (tv < t1 && !(own_new && tv == pos)) ? tv : min(t0, pos);
                 nxtv[u] = Vec8<F16>::load_raw(vc + (size_t)tvc * a.kv_dim + hoff + ve);
             }
         }
