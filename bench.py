@@ -37,10 +37,21 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes one launch of the dominant kernel moves: rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch (two counter
-# runs of `bench.py --probe`), each scaled by what the same counter reads for the 64 MiB copy kernel of that probe.
-# The summary of those runs is kept under profiles/.
-DOMINANT_KERNEL_TRAFFIC_BYTES = 51385751
+TRAFFIC_PROFILE = os.path.join("profiles", "gate_up_gemv_q4k_hbm_counters.md")
+
+
+def dominant_kernel_traffic():
+    """HBM bytes one launch of the dominant kernel moves, read from the committed counter summary (rocprofv3 FETCH_SIZE +
+    WRITE_SIZE per dispatch of `bench.py --probe`, each scaled by what the same counter reads for the probe's 64 MiB copy
+    kernel): the bold `= **N B**` figure of that file, or None when the file is not there."""
+    import re
+    try:
+        m = re.search(r"=\s*\*\*(\d+) B\*\*", open(os.path.join(ROOT, TRAFFIC_PROFILE)).read())
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
 CFG = dict(dim=4096, hidden_dim=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000)
 
 
@@ -426,7 +437,7 @@ def main():
             roof = dict(bound="hbm", kernel="gemv_rowtile_kernel<Q4_K, dual> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096); the launch with q/k/v and the "
                                             "attention is longer per token but cannot be launched alone through the operator API",
                         achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
-                        traffic=DOMINANT_KERNEL_TRAFFIC_BYTES, traffic_source="profiles/gate_up_gemv_q4k_hbm_counters.md",
+                        traffic=dominant_kernel_traffic(), traffic_source=TRAFFIC_PROFILE,
                         launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
         log("dominant kernel: %s us/launch, %.1f GB/s" % (roof["launch_us"], roof["achieved"]))
     c5 = None
