@@ -43,6 +43,23 @@ def test_persistent_small_model_vs_oracle(kv_f16):
         b.close()
 
 
+def test_persistent_small_model_behind_large_allocations():
+    """The small model again, loaded after 5 GB of other allocations in steps of 640 MB: its buffers then lie at
+    addresses whose lower 32 bits are spread over the whole range, bit 31 included (the first version of the kernel
+    rebuilt pointers from two words with the lower one sign-extended, which only such addresses expose)."""
+    from slai_amd.runtime import GpuTensor
+    b = backend_with(True)
+    try:
+        pads = [GpuTensor(b, 160 * 1024 * 1024) for _ in range(8)]
+        data = gw.llama_gguf(dim=1024, hidden_dim=2816, n_layers=3, n_heads=8, n_kv_heads=8, vocab=2000, seq_len=256, wtype=12, v_type=14,
+                             out_type=14, embd_type=12, seed=73, std=0.05, norm_random=True)
+        check_llama(b, data, [5, 1000, 1999, 9, 77, 3], 24, kv_f16=True, check_logit_steps=6)
+        for t in pads:
+            t.destroy()
+    finally:
+        b.close()
+
+
 def test_persistent_matches_launch_per_step_form():
     """The same model through both forms on the device: ids identical over 48 steps, logits within 1e-3."""
     from slai_amd.runtime import Gguf, Llama2
