@@ -69,6 +69,30 @@ def token_bytes(cfg, weight_bytes, pos_lo, pos_hi, kv_bytes=2):
     return weight_bytes + kv_read + kv_write
 
 
+BLOCK_BYTES = {12: (144, 256), 14: (210, 256), 8: (34, 32), 13: (176, 256), 2: (18, 32)}      # ggml type: bytes per block, weights per block
+
+
+def packed_bytes(ggml_type, nrows, ncols):
+    b, w = BLOCK_BYTES[ggml_type]
+    return nrows * ncols // w * b
+
+
+def step_bytes(cfg, pos, kv_bytes=2):
+    """Algorithmic HBM bytes of one launch of each step of a layer (and of the output matrix) in the headline model: packed
+    weights + the vectors read and written (+ the cache rows 0..pos and the new row for the launch that holds the attention)."""
+    d, h, v = cfg["dim"], cfg["hidden_dim"], cfg["vocab"]
+    kv_dim = d * cfg["n_kv_heads"] // cfg["n_heads"]
+    vec = 4 * d + 4 * d // 16                                   # a weighted activation vector and its sums of 16
+    return {
+        "llama2 qkv + attention": packed_bytes(12, d, d) + packed_bytes(12, kv_dim, d) + packed_bytes(14, kv_dim, d) + 4 * d + vec
+                                  + 2 * (pos + 1) * kv_dim * kv_bytes + 4 * d,
+        "llama2 attn_output": packed_bytes(12, d, d) + 4 * d + 8 * d + vec,
+        "llama2 ffn gate/up": 2 * packed_bytes(12, h, d) + 4 * d + vec + 4 * h,
+        "llama2 ffn_down": packed_bytes(12, d, h) + 4 * h + 8 * d + vec,
+        "llama2 output": packed_bytes(14, v, d) + 4 * d + vec + 4 * v,
+    }
+
+
 def measure_dominant_kernel(backend, reps=20):
     """Mean launch duration of the fused gate/up GEMV (Q4_K, 11008x4096 twice) over distinct copies, launched the way
     the decode loop launches it: 64-row-tile layout, activations in the prepared form left by the preceding GEMV."""
@@ -401,6 +425,18 @@ def main():
     tb = token_bytes(cfg, model.weight_bytes(), pos0, pos0 + K - 1)
     log("decode: %.3f ms/token (events), wall %.3f ms/token, %.1f tok/s, %.2f GB/token -> %.1f GB/s"
         % (ms_per_step, wall * 1000 / K, tok_s, tb / 1e9, tb / ms_per_step / 1e6))
+    steps = None
+    if form == 0 and not args.no_roofline:
+        # every launch of a token, timed with an event after each (launched from the host, 8 tokens at the middle position)
+        mid = pos0 + K // 2
+        sb = step_bytes(cfg, mid)
+        steps = []
+        for name, us, per, alone in model.time_steps(mid, int(toks[K // 2 - 1]), reps=8):
+            e = dict(step=name, us_per_launch=round(alone, 2), launches_per_token=per, us_between_events_in_a_token=round(us, 2))
+            if name in sb:
+                e.update(algorithmic_bytes=int(sb[name]), gbs=round(sb[name] / alone / 1e3, 1), frac=round(sb[name] / alone / 1e3 / HBM_PEAK_GBS, 4))
+            steps.append(e)
+        log("steps (each alone, one launch per layer back to back): " + "; ".join("%s %.2f us x %d" % (e["step"], e["us_per_launch"], e["launches_per_token"]) for e in steps))
     sampled = prompt_chunks = None
     if not args.no_side:
         # the same K positions with the chat's sampler (temperature 0.7, top-p 0.95) picked on the device: reported beside
@@ -434,11 +470,21 @@ def main():
         else:
             kms, kalgo = measure_dominant_kernel(backend)
             ach = kalgo / (kms * 1e-3) / 1e9
-            roof = dict(bound="hbm", kernel="gemv_rowtile_kernel<Q4_K, dual> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096); the launch with q/k/v and the "
-                                            "attention is longer per token but cannot be launched alone through the operator API",
-                        achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
-                        traffic=dominant_kernel_traffic(), traffic_source=TRAFFIC_PROFILE,
-                        launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
+            gate_up = dict(kernel="gemv_rowtile_kernel<Q4_K, gated pair> (RMSNorm + gate/up GEMV + SiLU, 2x 11008x4096), alone over 8 rotating weight copies",
+                           achieved=round(ach, 1), frac=round(ach / HBM_PEAK_GBS, 4), traffic=dominant_kernel_traffic(), traffic_source=TRAFFIC_PROFILE,
+                           launch_us=round(kms * 1000, 2), algorithmic_bytes=kalgo)
+            top = max((e for e in steps if "algorithmic_bytes" in e), key=lambda e: e["us_per_launch"] * e["launches_per_token"]) if steps else None
+            if top and top["step"] == "llama2 qkv + attention":
+                # the launch that takes the largest share of a token: q/k/v projections and the attention in one kernel.  It
+                # is not an operator of its own: slai_llama2_time_steps launches it alone, layer after layer.
+                roof = dict(bound="hbm", kernel="qkv_attention_kernel (RMSNorm + q/k/v GEMV, RoPE, cache write, attention; 32 launches per token)",
+                            achieved=top["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=top["frac"], traffic=None,
+                            launch_us=top["us_per_launch"], algorithmic_bytes=top["algorithmic_bytes"],
+                            how="its 32 launches of a token (one per layer, each layer's own weights and cache) back to back from the host at position %d, "
+                                "HIP events before the first and after the last, 8 repetitions" % (pos0 + K // 2),
+                            second_kernel=gate_up)
+            else:
+                roof = dict(bound="hbm", peak=HBM_PEAK_GBS, unit="GB/s", **gate_up)
         log("dominant kernel: %s us/launch, %.1f GB/s" % (roof["launch_us"], roof["achieved"]))
     c5 = None
     if not args.no_side:
@@ -468,7 +514,7 @@ def main():
         "token_bytes": int(tb), "hbm_gbs": round(tb / ms_per_step / 1e6, 1),
         "hbm_roofline_frac": round(tb / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
         "roofline_tok_s": round(HBM_PEAK_GBS * 1e9 / tb, 1),
-        "sampled_decode": sampled, "prompt_chunks": prompt_chunks, "config5": c5,
+        "steps": steps, "sampled_decode": sampled, "prompt_chunks": prompt_chunks, "config5": c5,
         "roofline": roof, "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

@@ -352,6 +352,16 @@ int slai_llama2_decode_form(const slai_llama2 *m);
  * projection): entered, input staged, multiplied, reduced -- then 8 for the output matrix.  Zero = phase not taken. */
 int slai_llama2_trace_token(slai_llama2 *m, uint32_t pos, uint32_t token, uint64_t *out, size_t capacity, uint32_t *n_workgroups,
                             uint32_t *stamps_per_workgroup);
+/* Measurement aid without a reference counterpart (the reference times whole forwards, slai-bench/src/main.rs:184-247):
+ * one token at (pos, token) through the launch-per-step form, launched from the host `reps` times with an event after
+ * every launch.  Returns, per step name in order of first appearance (`names`: newline separated, e.g. "llama2 qkv +
+ * attention"), the mean time from the end of the launch before it to the end of the step's launch in microseconds, and
+ * how many times the step occurs per token.  The intervals include the event markers (a few microseconds each), so their
+ * sum is above the time of a token replayed from a graph; `alone_us` is each step's launches alone, one per layer back to
+ * back with events only before the first and after the last: the figure to set against a profiler's kernel duration.
+ * SLAI_E_STATE for a model that takes the resident launch. */
+int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t token, uint32_t reps, char *names, size_t names_len, float *mean_us,
+                           float *alone_us, uint32_t *per_token, uint32_t capacity, uint32_t *n_steps);
 /* Device access for set-up and inspection: layer l's caches ([kv_dim x seq_len]) and the state vectors. */
 int slai_llama2_kv_buffers(slai_llama2 *m, uint32_t layer, slai_buffer **key_cache, slai_buffer **value_cache);
 int slai_llama2_logits_buffer(slai_llama2 *m, slai_buffer **logits);

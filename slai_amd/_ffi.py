@@ -142,6 +142,7 @@ SIGNATURES = {
     "slai_gpt2_check_gguf": (i32, [vp, C.c_char_p, sz]),
     "slai_llama2_decode_form": (i32, [vp]),
     "slai_llama2_trace_token": (i32, [vp, u32, u32, vp, sz, P(u32), P(u32)]),
+    "slai_llama2_time_steps": (i32, [vp, u32, u32, u32, vp, sz, vp, vp, vp, u32, P(u32)]),
     "slai_llama2_destroy": (None, [vp]),
     "slai_llama2_get_config": (i32, [vp, P(Llama2Config)]),
     "slai_llama2_weight_bytes": (sz, [vp]),

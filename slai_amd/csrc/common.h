@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <map>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "slai_hip.h"
@@ -85,6 +86,10 @@ struct slai_ctx {
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
     // SLAI_PERSISTENT=0: never the one-launch-per-token form of the Llama-2 layer stack
     bool persistent = true;
+    // When set, every launch of a decode step is followed by an event recorded under the step's name
+    // (slai_llama2_time_steps); null otherwise.
+    std::vector<std::pair<const char *, hipEvent_t>> *step_marks = nullptr;
+    const char *only_step = nullptr;         // when set, launches of decode steps with another name are skipped (step timing)
     bool use_graph = true;  // SLAI_NO_GRAPH=1 replays the token sequence eagerly (profilers that cannot trace graph launches)
 };
 
@@ -273,6 +278,7 @@ bool gemv_gated_is_rowtile(const slai_ctx *ctx, const slai_qmat *gate, const sla
 // qkv_attention_fusable).
 struct AttnLaunch;
 int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunch *fused_attn = nullptr);
+int step_mark(slai_ctx *ctx, const char *name);        // records an event under `name` when step timing is on
 bool qkv_attention_fusable(const slai_ctx *ctx, const slai_qmat *v, const slai_qmat *k, const slai_qmat *q, const AttnLaunch &a);
 int handoff_reserve(slai_ctx *ctx, uint32_t n_heads);   // not during graph capture
 int handoff_check(slai_ctx *ctx);                        // after a synchronize: error if a hand-off ever timed out

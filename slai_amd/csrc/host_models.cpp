@@ -477,7 +477,11 @@ int slai_llama2::enqueue_fused(int sampler) {
     float *x = (float *)s.x.buf->dptr, *xb = (float *)s.xb.buf->dptr, *hb = (float *)s.hb.buf->dptr, *hb2 = (float *)s.hb2.buf->dptr;
     float *q = (float *)s.q.buf->dptr, *kcol = (float *)s.kcol.buf->dptr, *vcol = (float *)s.vcol.buf->dptr;
     const uint32_t dim = config.dim, kvd = kv_dim();
-    SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, &ds->token, nullptr, nullptr, dim, x));
+    const auto wanted = [&](const char *name) { return !ctx->only_step || strcmp(ctx->only_step, name) == 0; };
+    if (wanted("embedding row")) {
+        SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, &ds->token, nullptr, nullptr, dim, x));
+        TRY(step_mark(ctx, "embedding row"));
+    }
     // When the GEMV that writes x can leave a norm-weighted copy for the 64-row-tile GEMV that reads it next, that
     // consumer skips its own staging of the activations.
     float *xw = (float *)s.xw.buf->dptr;
@@ -525,10 +529,11 @@ int slai_llama2::enqueue_fused(int sampler) {
                 }
             }
         }
-        if (!attention_done) {
+        if (!attention_done && wanted("llama2 attention")) {
             hipError_t e = launch_attention(ctx->stream, a);
             if (e == hipErrorInvalidValue) return set_error(ctx, SLAI_E_SHAPE, "attention: unsupported head size or context length");
             SLAI_HIP_TRY(ctx, e);
+            TRY(step_mark(ctx, "llama2 attention"));
         }
         // ---- attention output projection, residual in the epilogue
         {
@@ -561,7 +566,10 @@ int slai_llama2::enqueue_fused(int sampler) {
                 c.prepared = prepared;
                 TRY(gemv_call(ctx, c, "llama2 ffn gate/up"));
             }
-            SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, config.hidden_dim, 1}, VecView{hb2, config.hidden_dim, 1}));
+            if (wanted("llama2 silu")) {
+                SLAI_HIP_TRY(ctx, launch_silu(ctx->stream, VecView{hb, config.hidden_dim, 1}, VecView{hb2, config.hidden_dim, 1}));
+                TRY(step_mark(ctx, "llama2 silu"));
+            }
         }
         // ---- down projection, residual in the epilogue
         {
@@ -907,6 +915,83 @@ SLAI_EXPORT int slai_llama2_trace_token(slai_llama2 *m, uint32_t pos, uint32_t t
     slai_buffer_destroy(ctx, buf);
     *n_workgroups = grid; *stamps_per_workgroup = stride;
     return rc;
+}
+
+// One token through the launch-per-step form, launched from the host `reps` times at the same position, with an event
+// after every launch: mean time from the end of the launch before to the end of each launch, by step name in order of
+// first appearance (`names`: newline separated), and how often the step occurs per token.
+SLAI_EXPORT int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t token, uint32_t reps, char *names, size_t names_len, float *mean_us,
+                                       float *alone_us, uint32_t *per_token, uint32_t capacity, uint32_t *n_steps) {
+    if (!m || !names || !mean_us || !alone_us || !per_token || !n_steps || reps == 0) return SLAI_E_ARG;
+    slai_ctx *ctx = m->ctx;
+    if (m->persistent.ready) return set_error(ctx, SLAI_E_STATE, "slai_llama2_time_steps: this model takes the resident launch, which has no steps to time");
+    if (pos >= m->config.seq_len || token >= m->config.vocab_size) return set_error(ctx, SLAI_E_ARG, "slai_llama2_time_steps: position or token out of range");
+    if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_llama2_time_steps: not during graph capture");
+    DecodeState ds{(int)pos, (int)token, 0, 0};
+    TRY(slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds));
+    TRY(m->enqueue_fused(0));                                   // untimed: sizes scratch, warms the caches
+    TRY(slai_synchronize(ctx));
+    std::vector<std::pair<const char *, hipEvent_t>> marks;
+    marks.reserve((size_t)reps * (5 * m->config.n_layers + 4));
+    ctx->step_marks = &marks;
+    int rc = SLAI_OK;
+    for (uint32_t r = 0; r < reps && !rc; ++r) {
+        rc = step_mark(ctx, nullptr);                           // where the token starts
+        if (!rc) rc = m->enqueue_fused(0);
+    }
+    ctx->step_marks = nullptr;
+    if (!rc) rc = slai_synchronize(ctx);
+    if (!rc) rc = handoff_check(ctx);
+    std::vector<const char *> order;
+    std::vector<double> total;
+    std::vector<uint32_t> count;
+    for (size_t i = 1; i < marks.size() && !rc; ++i) {
+        if (!marks[i].first) continue;                          // a token's start: nothing was launched before it
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, marks[i - 1].second, marks[i].second) != hipSuccess) { rc = set_error(ctx, SLAI_E_HIP, "slai_llama2_time_steps: event time"); break; }
+        size_t k = 0;
+        while (k < order.size() && strcmp(order[k], marks[i].first) != 0) ++k;
+        if (k == order.size()) { order.push_back(marks[i].first); total.push_back(0.0); count.push_back(0); }
+        total[k] += ms; ++count[k];
+    }
+    for (auto &mk : marks) (void)hipEventDestroy(mk.second);
+    if (rc) return rc;
+    if (order.size() > capacity) return set_error(ctx, SLAI_E_SHAPE, "slai_llama2_time_steps: more steps than room for them");
+    std::string joined;
+    for (size_t k = 0; k < order.size(); ++k) {
+        mean_us[k] = (float)(total[k] * 1000.0 / count[k]);
+        per_token[k] = count[k] / reps;
+        joined += order[k];
+        joined += '\n';
+    }
+    if (joined.size() + 1 > names_len) return set_error(ctx, SLAI_E_SHAPE, "slai_llama2_time_steps: the names do not fit");
+    memcpy(names, joined.c_str(), joined.size() + 1);
+    *n_steps = (uint32_t)order.size();
+    // each step alone: only its launches (one per layer: every layer's own weights, so nothing stays cached from launch to
+    // launch), back to back, an event before the first and after the last
+    hipEvent_t e0, e1;
+    SLAI_HIP_TRY(ctx, hipEventCreate(&e0));
+    SLAI_HIP_TRY(ctx, hipEventCreate(&e1));
+    for (size_t k = 0; k < order.size() && !rc; ++k) {
+        ctx->only_step = order[k];
+        rc = m->enqueue_fused(0);                               // untimed
+        if (!rc && hipEventRecord(e0, ctx->stream) != hipSuccess) rc = SLAI_E_HIP;
+        for (uint32_t r = 0; r < reps && !rc; ++r) rc = m->enqueue_fused(0);
+        if (!rc && hipEventRecord(e1, ctx->stream) != hipSuccess) rc = SLAI_E_HIP;
+        ctx->only_step = nullptr;
+        if (!rc) rc = slai_synchronize(ctx);
+        float ms = 0.0f;
+        if (!rc && hipEventElapsedTime(&ms, e0, e1) != hipSuccess) rc = SLAI_E_HIP;
+        alone_us[k] = ms * 1000.0f / (float)(reps * (per_token[k] ? per_token[k] : 1));
+    }
+    ctx->only_step = nullptr;
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    if (rc == SLAI_E_HIP) return set_error(ctx, SLAI_E_HIP, "slai_llama2_time_steps: event");
+    if (rc) return rc;
+    // leave the state a whole forward at this position leaves
+    TRY(m->enqueue_fused(0));
+    TRY(slai_synchronize(ctx));
+    return handoff_check(ctx);
 }
 
 SLAI_EXPORT int slai_llama2_get_config(const slai_llama2 *m, slai_llama2_config *out) {

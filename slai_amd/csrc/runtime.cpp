@@ -459,7 +459,23 @@ int sampler_scratch_reserve(slai_ctx *ctx, size_t floats) {
     return scratch_grow(ctx, &ctx->sampler_scratch, &ctx->sampler_scratch_floats, floats, "sampler scratch");
 }
 
+int step_mark(slai_ctx *ctx, const char *name) {
+    if (!ctx->step_marks) return SLAI_OK;
+    hipEvent_t e;
+    SLAI_HIP_TRY(ctx, hipEventCreate(&e));
+    ctx->step_marks->emplace_back(name, e);
+    SLAI_HIP_TRY(ctx, hipEventRecord(e, ctx->stream));
+    return SLAI_OK;
+}
+
+static int gemv_call_impl(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunch *fused_attn);
 int gemv_call(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunch *fused_attn) {
+    if (ctx->only_step && strcmp(ctx->only_step, who) != 0) return SLAI_OK;
+    if (int rc = gemv_call_impl(ctx, c, who, fused_attn)) return rc;
+    return step_mark(ctx, who);
+}
+
+static int gemv_call_impl(slai_ctx *ctx, const GemvCall &c, const char *who, const AttnLaunch *fused_attn) {
     const slai_qmat *m0 = c.m[0];
     if (!m0 || c.nseg < 1 || c.nseg > 3) return set_error(ctx, SLAI_E_ARG, std::string(who) + ": bad GEMV call");
     // 64-row tiles: wave-uniform activations, formats may differ between the segments

@@ -546,6 +546,20 @@ class Llama2:
         self.b.check(self.b.L.slai_llama2_trace_token(self.h, pos, token, out.ctypes.data, cap, C.byref(grid), C.byref(stride)))
         return out[:grid.value * stride.value].reshape(grid.value, stride.value)
 
+    def time_steps(self, pos, token, reps=8):
+        """[(step name, microseconds per launch inside a token with an event after every launch, launches per token,
+        microseconds per launch of the step alone)] of the launch-per-step form (see slai_llama2_time_steps)."""
+        cap = 32
+        names = C.create_string_buffer(4096)
+        us = np.zeros(cap, np.float32)
+        alone = np.zeros(cap, np.float32)
+        per = np.zeros(cap, np.uint32)
+        n = C.c_uint32()
+        self.b.check(self.b.L.slai_llama2_time_steps(self.h, pos, token, reps, C.cast(names, C.c_void_p), 4096, us.ctypes.data, alone.ctypes.data,
+                                                     per.ctypes.data, cap, C.byref(n)))
+        labels = names.value.decode().split("\n")[:n.value]
+        return [(labels[i], float(us[i]), int(per[i]), float(alone[i])) for i in range(n.value)]
+
     def prefill_path(self):
         """2: matrix-core GEMM, 1: per-token workgroups over shared weights, 0: the token-by-token loop."""
         return int(self.b.L.slai_llama2_prefill_supported(self.h))

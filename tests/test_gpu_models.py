@@ -295,3 +295,22 @@ def test_device_against_the_transformers_library_directly(backend):
             assert np.array_equal(ids, lib_ids), what
             dm.destroy()
         gg.close()
+
+
+def test_time_steps_names_every_launch_of_a_token(backend):
+    """slai_llama2_time_steps: the launch-per-step form of a 3-layer model reports each of its steps with the number of
+    launches per token and a positive time; the logits afterwards are those of an ordinary forward at that position."""
+    from slai_amd.runtime import Gguf, Llama2
+    data = gw.llama_gguf(dim=512, hidden_dim=1536, n_layers=3, n_heads=4, n_kv_heads=4, vocab=1024, seq_len=64, wtype=12, seed=9, std=0.05)
+    g = Gguf(data)
+    m = Llama2(backend, g, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+    toks, _ = m.generate(np.array([1, 2, 3], np.int32), 8)
+    ref = m.forward_logits(8, int(toks[7]))
+    steps = m.time_steps(8, int(toks[7]), reps=4)
+    names = [s[0] for s in steps]
+    assert names[0] == "embedding row" and names[-1] == "llama2 output", names
+    per = {s[0]: s[2] for s in steps}
+    assert per["llama2 attn_output"] == 3 and per["llama2 ffn gate/up"] == 3 and per["llama2 ffn_down"] == 3 and per["llama2 output"] == 1, per
+    assert all(s[1] > 0.0 and s[3] > 0.0 for s in steps), steps
+    assert np.array_equal(m.forward_logits(8, int(toks[7])), ref)
+    m.destroy(); g.close()
