@@ -18,6 +18,7 @@ struct slai_buffer {
     uint32_t usage = 0;
     void *host_staging = nullptr;  // pinned, when created with SLAI_USAGE_MAP_READ
     uint32_t shape[4] = {0, 0, 0, 0};  // set for buffers handed out by a slai_tensor_cache (its key)
+    bool idle_in_cache = false;        // back in its cache and not handed out: a second reclaim is an error
 };
 
 struct slai_qmat {

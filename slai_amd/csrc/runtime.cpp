@@ -234,11 +234,13 @@ SLAI_EXPORT int slai_tensor_cache_get_or_insert(slai_ctx *ctx, slai_tensor_cache
     if (it != c->tensors.end() && !it->second.empty()) {
         *out = it->second.back();
         it->second.pop_back();
+        (*out)->idle_in_cache = false;
         return SLAI_OK;
     }
     static const size_t esz[] = {4, 2, 1, 4};
     uint64_t n = 1;
     for (int i = 0; i < 4; ++i) {
+        if (shape[i] == 0) return set_error(ctx, SLAI_E_SHAPE, "slai_tensor_cache_get_or_insert: a dimension of size zero");
         n *= shape[i];
         if (n > (uint64_t)1 << 40) return set_error(ctx, SLAI_E_SHAPE, "slai_tensor_cache_get_or_insert: shape too large");
     }
@@ -253,6 +255,9 @@ SLAI_EXPORT int slai_tensor_cache_get_or_insert(slai_ctx *ctx, slai_tensor_cache
 SLAI_EXPORT int slai_tensor_cache_reclaim(slai_ctx *ctx, slai_tensor_cache *c, slai_buffer *b) {
     if (!ctx || !c || !b) return SLAI_E_ARG;
     if (!b->shape[0]) return set_error(ctx, SLAI_E_ARG, "slai_tensor_cache_reclaim: not a cached tensor");
+    // (the reference cannot give a tensor back twice: dropping its handle is what gives it back)
+    if (b->idle_in_cache) return set_error(ctx, SLAI_E_STATE, "slai_tensor_cache_reclaim: this tensor is already back in its cache");
+    b->idle_in_cache = true;
     slai_tensor_key key{b->dtype, {b->shape[0], b->shape[1], b->shape[2], b->shape[3]}, b->usage};
     c->tensors[key].push_back(b);
     return SLAI_OK;

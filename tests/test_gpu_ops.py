@@ -254,7 +254,12 @@ def test_submission_bracket_and_graph_replay_of_an_op_sequence(backend, oracle_l
     assert again.read().shape == (hid,)                                                  # contents are the last holder's
     other = cache.get_or_insert(hid, 2)                                                  # another shape: a miss, a new zeroed buffer
     assert cache.idle() == 3 and not other.read().any()
+    handle = again.h
     cache.reclaim(again); cache.reclaim(other)
+    assert backend.L.slai_tensor_cache_reclaim(backend.h, cache.h, handle) != 0        # already back: refused, not pooled twice
+    assert cache.idle() == 5
+    with pytest.raises(Exception):
+        cache.get_or_insert(0)                                                           # a dimension of size zero
     cache.clear()
     assert cache.idle() == 0
     cache.destroy()
