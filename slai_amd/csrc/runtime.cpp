@@ -91,6 +91,9 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
     ctx->fuse_qkv_attention = env_int("SLAI_FUSE_QKV_ATTN", 1) != 0;
     ctx->persistent = env_int("SLAI_PERSISTENT", 0) != 0;
+    if (ctx->persistent)
+        fprintf(stderr, "slai: SLAI_PERSISTENT=1 -- the one-launch-per-token decode kernel has not run on a device since its pointer "
+                        "handling was corrected; earlier builds of it ended in GPU memory faults on models beyond a few MB\n");
     *out = ctx;
     return SLAI_OK;
 }
