@@ -20,8 +20,8 @@ Also measured here:
     configuration 1 in full on one thread (the reference's CPU path is single-threaded) and on all
     cores, and a bounded sample of the headline shapes (depth 2 and 6, a few tokens) extrapolated to
     32 layers.  A reported baseline, not the target.
-  * config5: the long-context configuration (Q8_0, cache pre-filled to 4000 positions), attention and
-    GEMV rates apart.
+  * config1, config3, config5: the other decode configurations through the same C ABI (tiny Llama and the
+    GPT-2-small shape in full; the long-context one with attention and GEMV rates apart).
 """
 import argparse
 import math
@@ -358,6 +358,60 @@ def config5_block(backend, seed, n_steps=96):
                 decode_form=form)
 
 
+def small_config_blocks(backend, seed):
+    """BASELINE configurations 1 (tiny Llama, Q8_0, 16 prompt ids + 128 tokens) and 3 (GPT-2-small shape, Q8_0, 32 prompt
+    ids + 256 tokens) through the C ABI: tok/s over the generated tokens of the device-resident greedy loop, the prompt
+    fed token by token as the reference does (chat_llama2.rs:105-158), second run timed (the first captures the graph)."""
+    from slai_amd import _ffi
+    from slai_amd import gguf_writer as gw
+    from slai_amd.runtime import Gguf, Gpt2, Llama2
+    out = {}
+    for name, make, cls, vocab, n_prompt, n_tokens in (
+            ("config1", lambda: gw.tiny_llama_gguf(seed=seed), lambda g: Llama2(backend, g, _ffi.MODEL_LLAMA, _ffi.KV_F32), 32000, 16, 128),
+            ("config3", lambda: gw.gpt2_gguf(seed=seed), lambda g: Gpt2(backend, g), 50257, 32, 256)):
+        data = make()
+        g = Gguf(data)
+        m = cls(g)
+        prompt = np.random.Generator(np.random.PCG64(seed)).integers(0, vocab, n_prompt).astype(np.int32)
+        m.generate(prompt, n_prompt + 8)                                        # untimed: graph capture, first touch
+        first, _ = m.generate(prompt, n_prompt - 1)                             # the prompt, untimed (caches only)
+        seq = np.concatenate([prompt, np.zeros(1, np.int32)])
+        _, ms = m.generate(seq, n_tokens, start_pos=n_prompt - 1)               # timed: the generated tokens
+        wbytes = m.weight_bytes()
+        m.destroy(); g.close(); del data
+        out[name] = dict(tok_s=round(1000.0 * n_tokens / ms, 1), ms_per_step=round(ms / n_tokens, 4), tokens=n_tokens, prompt=n_prompt,
+                         weight_bytes=int(wbytes), hbm_gbs=round(wbytes / (ms / n_tokens) / 1e6, 1))
+    out["config1"]["workload"] = "tiny Llama-2: dim 288, 6 layers, 6 heads, FFN 768, vocab 32000, Q8_0, f32 cache"
+    out["config3"]["workload"] = "GPT-2-small shape: dim 768, 12 layers, 12 heads, FFN 3072, vocab 50257, context 1024, Q8_0"
+    return out
+
+
+def bench_line(K, W, ms_per_step, tb, n_layers, distinct_layers, pos0, seq_len, form, step_times=None, sampled=None, prompt_chunks=None,
+               config5=None, small=None, roofline=None, cpu=None):
+    """The one JSON line of the benchmark as a dict (no device needed to build it)."""
+    tok_s = 1000.0 / ms_per_step
+    small = small or {}
+    return {
+        "metric": "decode tok/s & % of HBM roofline, Llama-2-7B-shape Q4_K, batch 1",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": int(K), "warmup": int(W),
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic: seeded N(0,0.02) weights quantized with ggml's reference algorithm "
+                                "(%d layers generated, the rest are row-rotated copies in distinct memory), seeded prompt ids"
+                                % distinct_layers,
+        "config": {"workload": "BASELINE config 4: Llama-2-7B-shape greedy decode, dim 4096, %d layers, 32 heads, FFN 11008, "
+                               "vocab 32000, Q4_K weights (Q6_K v-proj/output), fp16 KV; 64 prompt positions processed untimed, "
+                               "%d token(s) decoded untimed, then %d tokens timed at positions %d..%d"
+                               % (n_layers, W, K, pos0, pos0 + K - 1), "batch": 1, "kv_dtype": "f16", "context": seq_len,
+                   "decode_form": "one resident launch per token" if form else "one launch per step"},
+        "token_bytes": int(tb), "hbm_gbs": round(tb / ms_per_step / 1e6, 1),
+        "hbm_roofline_frac": round(tb / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
+        "roofline_tok_s": round(HBM_PEAK_GBS * 1e9 / tb, 1),
+        "step_times": step_times, "sampled_decode": sampled, "prompt_chunks": prompt_chunks,
+        "config1": small.get("config1"), "config3": small.get("config3"), "config5": config5,
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -486,8 +540,11 @@ def main():
             else:
                 roof = dict(bound="hbm", peak=HBM_PEAK_GBS, unit="GB/s", **gate_up)
         log("dominant kernel: %s us/launch, %.1f GB/s" % (roof["launch_us"], roof["achieved"]))
-    c5 = None
+    c5 = small = None
     if not args.no_side:
+        small = small_config_blocks(backend, args.seed)
+        log("config 1: %.1f tok/s (%.4f ms/token); config 3: %.1f tok/s (%.4f ms/token)"
+            % (small["config1"]["tok_s"], small["config1"]["ms_per_step"], small["config3"]["tok_s"], small["config3"]["ms_per_step"]))
         c5 = config5_block(backend, args.seed)
         log("config 5: %.1f tok/s (%.3f ms/token); attention %.2f us/layer = %.1f GB/s; GEMV %.1f GB/s"
             % (c5["tok_s"], c5["ms_per_step"], c5["attention"]["us_per_layer"], c5["attention"]["gbs"], c5["gemv"]["gbs"]))
@@ -499,24 +556,8 @@ def main():
         cpu = cpu_baseline(args.seed)
         log("cpu baseline: %.3f tok/s on %d threads (%.1f s); config 1 in full: %s" % (cpu["value"], cpu["cores"], time.perf_counter() - t0, cpu["config1"]))
 
-    out = {
-        "metric": "decode tok/s & % of HBM roofline, Llama-2-7B-shape Q4_K, batch 1",
-        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic: seeded N(0,0.02) weights quantized with ggml's reference algorithm "
-                                "(%d layers generated, the rest are row-rotated copies in distinct memory), seeded prompt ids"
-                                % min(args.distinct_layers, cfg["n_layers"]),
-        "config": {"workload": "BASELINE config 4: Llama-2-7B-shape greedy decode, dim 4096, %d layers, 32 heads, FFN 11008, "
-                               "vocab 32000, Q4_K weights (Q6_K v-proj/output), fp16 KV; 64 prompt positions processed untimed, "
-                               "%d token(s) decoded untimed, then %d tokens timed at positions %d..%d"
-                               % (cfg["n_layers"], W, K, pos0, pos0 + K - 1), "batch": 1, "kv_dtype": "f16", "context": seq_len,
-                   "decode_form": "one resident launch per token" if form else "one launch per step"},
-        "token_bytes": int(tb), "hbm_gbs": round(tb / ms_per_step / 1e6, 1),
-        "hbm_roofline_frac": round(tb / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
-        "roofline_tok_s": round(HBM_PEAK_GBS * 1e9 / tb, 1),
-        "steps": steps, "sampled_decode": sampled, "prompt_chunks": prompt_chunks, "config5": c5,
-        "roofline": roof, "cpu_baseline": cpu,
-    }
+    out = bench_line(K, W, ms_per_step, tb, cfg["n_layers"], min(args.distinct_layers, cfg["n_layers"]), pos0, seq_len, form, step_times=steps,
+                     sampled=sampled, prompt_chunks=prompt_chunks, config5=c5, small=small, roofline=roof, cpu=cpu)
     print(json.dumps(out), flush=True)
 
 

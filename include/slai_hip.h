@@ -108,8 +108,14 @@ void *slai_buffer_device_ptr(const slai_buffer *buf);
  *   get_or_insert (:162-188)  an idle buffer with this key (contents as its last holder left them) or a new zero-filled
  *                             one; a hit allocates nothing and is legal during graph capture, a miss is SLAI_E_STATE there
  *   reclaim (:118-124,199-203, what dropping a `CachedTensor` does)  back into the pool under its key
- *   clear (:195-197; the chat calls it once per token, chat_llama2.rs:174)  frees the idle buffers
+ *   clear (:195-197; the chat calls it once per token, chat_llama2.rs:174)  frees the idle buffers; SLAI_E_STATE during
+ *                             a capture.  A buffer that was handed out while a graph was being captured may be named by that
+ *                             graph, so clear / destroy keep its memory until the context is destroyed (the pool forgets it)
+ *   destroy                   clear + the cache itself; inside a capture nothing is synchronised or freed (the idle buffers
+ *                             are kept until the context is destroyed) and the capture goes on
  *   idle  number of buffers in the pool.
+ * slai_buffer_destroy refuses (message in slai_last_error, nothing freed) a buffer that sits idle in a cache, and inside a
+ * capture keeps the buffer's memory until the context is destroyed.
  * The models of this library do not use it: `Llama2State` preallocates every activation (transformer.rs:47-140). */
 int slai_tensor_cache_create(slai_ctx *ctx, slai_tensor_cache **out);
 void slai_tensor_cache_destroy(slai_ctx *ctx, slai_tensor_cache *cache);
@@ -344,7 +350,7 @@ uint32_t slai_llama2_prefill_fp32_repeats(const slai_llama2 *m);
 /* Which form the per-token loop of this model takes: 0 = one launch per step of `Llama2::launch` (transformer.rs:316-381;
  * four to five per layer), 1 = the whole layer stack and the output matrix in one resident launch per token (widths of
  * 1024 .. 4096 in steps of 1024, as many cache heads as query heads of size 128, contexts up to 1024, Q4_K / Q5_K / Q6_K
- * mixes; SLAI_PERSISTENT=0 at slai_ctx_create switches it off).  Results are the same to within summation order. */
+ * mixes; off unless the context was created with SLAI_PERSISTENT=1).  Results are the same to within summation order. */
 int slai_llama2_decode_form(const slai_llama2 *m);
 /* Measurement aid without a reference counterpart (profilers see the resident launch as one kernel): runs one token at
  * (pos, token) with in-kernel time stamps and returns them, n_workgroups x stamps_per_workgroup 64-bit ticks of the

@@ -19,6 +19,7 @@ struct slai_buffer {
     void *host_staging = nullptr;  // pinned, when created with SLAI_USAGE_MAP_READ
     uint32_t shape[4] = {0, 0, 0, 0};  // set for buffers handed out by a slai_tensor_cache (its key)
     bool idle_in_cache = false;        // back in its cache and not handed out: a second reclaim is an error
+    bool captured = false;             // handed out by its cache during a graph capture: a graph may name it, so it is never freed before the context
 };
 
 struct slai_qmat {
@@ -84,9 +85,10 @@ struct slai_ctx {
     // Scratch blocks that a larger one has replaced.  Captured graphs (and launches already queued) hold the old
     // addresses, so a block is only freed with the context.
     std::vector<void *> retired_scratch;
+    std::vector<slai_buffer *> retired_buffers;   // cached tensors a captured graph may name, and buffers destroyed inside a capture
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
-    // SLAI_PERSISTENT=0: never the one-launch-per-token form of the Llama-2 layer stack
-    bool persistent = true;
+    // SLAI_PERSISTENT=1: the one-launch-per-token form of the Llama-2 layer stack where a model's shapes allow it (off by default)
+    bool persistent = false;
     // When set, every launch of a decode step is followed by an event recorded under the step's name
     // (slai_llama2_time_steps); null otherwise.
     std::vector<std::pair<const char *, hipEvent_t>> *step_marks = nullptr;

@@ -98,6 +98,12 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     return SLAI_OK;
 }
 
+static void buffer_free(slai_buffer *b) {
+    if (b->dptr) (void)hipFree(b->dptr);
+    if (b->host_staging) (void)hipHostFree(b->host_staging);
+    delete b;
+}
+
 SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
@@ -108,6 +114,7 @@ SLAI_EXPORT void slai_ctx_destroy(slai_ctx *ctx) {
     if (ctx->sampler_scratch) (void)hipFree(ctx->sampler_scratch);
     if (ctx->handoff_counters) (void)hipFree(ctx->handoff_counters);
     for (void *p : ctx->retired_scratch) (void)hipFree(p);
+    for (slai_buffer *b : ctx->retired_buffers) buffer_free(b);
     if (ctx->timer0) (void)hipEventDestroy(ctx->timer0);
     if (ctx->timer1) (void)hipEventDestroy(ctx->timer1);
     (void)hipStreamDestroy(ctx->stream);
@@ -160,10 +167,18 @@ SLAI_EXPORT int slai_buffer_create(slai_ctx *ctx, size_t bytes, int dtype, uint3
 
 SLAI_EXPORT void slai_buffer_destroy(slai_ctx *ctx, slai_buffer *b) {
     if (!b) return;
+    if (b->idle_in_cache) {
+        // its cache still lists it and would hand the freed memory to the next get_or_insert: the cache frees it (clear / destroy)
+        if (ctx) set_error(ctx, SLAI_E_STATE, "slai_buffer_destroy: the buffer sits idle in a tensor cache; clear or destroy the cache instead");
+        return;
+    }
+    if (ctx && ctx->capturing) {
+        // no synchronisation and no free inside a capture: the buffer is kept until the context goes
+        ctx->retired_buffers.push_back(b);
+        return;
+    }
     if (ctx) (void)hipStreamSynchronize(ctx->stream);
-    if (b->dptr) (void)hipFree(b->dptr);
-    if (b->host_staging) (void)hipHostFree(b->host_staging);
-    delete b;
+    buffer_free(b);
 }
 SLAI_EXPORT size_t slai_buffer_size(const slai_buffer *b) { return b ? b->bytes : 0; }
 SLAI_EXPORT void *slai_buffer_device_ptr(const slai_buffer *b) { return b ? b->dptr : nullptr; }
@@ -212,17 +227,29 @@ SLAI_EXPORT int slai_tensor_cache_create(slai_ctx *ctx, slai_tensor_cache **out)
     return SLAI_OK;
 }
 // `TensorCache::clear` (tensor_cache.rs:195-197): idle tensors are freed; those handed out stay with their holders.
+// A tensor that was handed out while a graph was being captured may be named by that graph for as long as the graph
+// lives, so its memory is not freed here: it is retired and goes with the context (as grown scratch blocks do).
+static void cache_release(slai_ctx *ctx, slai_tensor_cache *c, bool may_free) {
+    bool synced = false;
+    for (auto &kv : c->tensors)
+        for (slai_buffer *b : kv.second) {
+            b->idle_in_cache = false;
+            if (!may_free || b->captured) { ctx->retired_buffers.push_back(b); continue; }
+            if (!synced) { (void)hipStreamSynchronize(ctx->stream); synced = true; }
+            buffer_free(b);
+        }
+    c->tensors.clear();
+}
 SLAI_EXPORT int slai_tensor_cache_clear(slai_ctx *ctx, slai_tensor_cache *c) {
     if (!ctx || !c) return SLAI_E_ARG;
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_tensor_cache_clear during graph capture");
-    for (auto &kv : c->tensors)
-        for (slai_buffer *b : kv.second) slai_buffer_destroy(ctx, b);
-    c->tensors.clear();
+    cache_release(ctx, c, true);
     return SLAI_OK;
 }
+// Inside a capture nothing is synchronised or freed and the capture goes on: the idle tensors are retired.
 SLAI_EXPORT void slai_tensor_cache_destroy(slai_ctx *ctx, slai_tensor_cache *c) {
     if (!c) return;
-    if (ctx) { ctx->capturing = false; slai_tensor_cache_clear(ctx, c); }
+    if (ctx) cache_release(ctx, c, !ctx->capturing);
     delete c;
 }
 // `TensorCache::get_or_insert` (tensor_cache.rs:162-188) with the insert closure of context.rs:107-127: an idle tensor of
@@ -238,6 +265,7 @@ SLAI_EXPORT int slai_tensor_cache_get_or_insert(slai_ctx *ctx, slai_tensor_cache
         *out = it->second.back();
         it->second.pop_back();
         (*out)->idle_in_cache = false;
+        if (ctx->capturing) (*out)->captured = true;
         return SLAI_OK;
     }
     static const size_t esz[] = {4, 2, 1, 4};

@@ -265,3 +265,48 @@ def test_submission_bracket_and_graph_replay_of_an_op_sequence(backend, oracle_l
     cache.destroy()
     for o in (gate, up, down, gx0, gw, cfg, gx):
         o.destroy()
+
+
+def test_tensor_cache_lifetime_rules(backend):
+    """What keeps a pooled tensor's memory valid: an idle tensor cannot be destroyed behind its cache's back; a tensor
+    handed out during a graph capture is retired, not freed, by `clear` (the graph that names it replays correctly
+    afterwards); `clear` is refused inside a capture; destroying a cache inside a capture leaves the capture running."""
+    import ctypes as C
+    from slai_amd.runtime import GpuTensor, LlmContext, TensorCache
+    ctxt = LlmContext(backend)
+    cache = TensorCache(backend)
+    n = 4096
+    t = cache.get_or_insert(n)
+    handle = t.h
+    cache.reclaim(t)
+    backend.L.slai_buffer_destroy(backend.h, handle)                      # refused: the cache still lists it
+    assert b"idle in a tensor cache" in backend.L.slai_last_error(backend.h)
+    assert cache.idle() == 1
+    src = GpuTensor.vector(backend, rnd(11, n))
+    dst = GpuTensor(backend, n)
+    backend.graph_begin_capture()
+    tmp = cache.get_or_insert(n)                                          # a hit: legal inside a capture
+    assert tmp.h.value == handle.value
+    ctxt.copy(src, tmp)
+    ctxt.copy(tmp, dst)
+    assert backend.L.slai_tensor_cache_clear(backend.h, cache.h) == _ffi.E_STATE
+    side = TensorCache(backend)
+    side.destroy()                                                        # nothing synchronised, the capture goes on
+    g = backend.graph_end_capture()
+    cache.reclaim(tmp)
+    cache.clear()                                                         # the graph still names tmp: retired, not freed
+    assert cache.idle() == 0
+    junk = [GpuTensor.vector(backend, np.full(n, 7.0, np.float32)) for _ in range(8)]   # would land on freed memory
+    for rep in range(3):
+        vals = rnd(20 + rep, n)
+        src.write(vals)
+        dst.write(np.zeros(n, np.float32))
+        backend.synchronize()
+        backend.graph_launch(g)
+        backend.synchronize()
+        assert np.array_equal(dst.read(), vals), rep
+        assert all(np.all(j.read() == 7.0) for j in junk)
+    backend.graph_destroy(g)
+    cache.destroy()
+    for o in junk + [src, dst]:
+        o.destroy()
