@@ -392,31 +392,33 @@ hipError_t attention_static_setup(int device);
 
 
 // ---- the whole layer stack of a Llama-2 token in one resident launch (kernels_decode_persistent.hip) ----------------------
-struct PersistentLayer {                 // one per layer, in device memory
-    const uint8_t *wq, *wk, *wv;         // 64-row tiles; K-quant formats tq / tk / tv
-    const uint8_t *wo;                   // 16-row tiles, Q4_K or Q6_K (to)
-    const uint8_t *wgate, *wup;          // 64-row tiles, both Q4_K (tg)
-    const uint8_t *wdown;                // 16-row tiles, Q4_K or Q6_K (td)
-    const float *attn_norm, *ffn_norm;
-    const float *bq, *bk, *bv;           // optional biases
-    void *kcache, *vcache;               // [seq_len][dim]
-    int tq, tk, tv, to, tg, td;
+// A matrix, vector or cache as the kernel sees it: address and size in bytes.  Every access of the kernel to it goes
+// through a buffer descriptor built from the pair, so the hardware checks it against the size.
+struct ResidentBuf { const void *ptr; uint32_t bytes; uint32_t type; };   // type: block format of a weight matrix, else 0
+struct PersistentLayer {                 // one per layer, in device memory (16 bytes per entry)
+    ResidentBuf wq, wk, wv;              // 64-row tiles; K-quant formats
+    ResidentBuf wo;                      // 16-row tiles, Q4_K or Q6_K
+    ResidentBuf wgate, wup;              // 64-row tiles, both Q4_K
+    ResidentBuf wdown;                   // 16-row tiles, Q4_K or Q6_K
+    ResidentBuf attn_norm, ffn_norm;     // dim floats
+    ResidentBuf bq, bk, bv;              // optional biases (ptr null: none)
+    ResidentBuf kcache, vcache;          // [seq_len][dim]
 };
 struct PersistentParams {
     const PersistentLayer *layers;
     uint32_t n_layers, dim, hidden, n_heads, seq_len, vocab;
+    uint32_t qkv_units, gu_rows;         // the decomposition (resident_plan.h: plan::Shape)
     float eps;
     int rope_variant; float rope_base; const float *rope_theta;
     int kv_f16;
-    const uint8_t *wout; int tout; const float *out_norm;     // output matrix (64-row tiles) and the final norm
+    ResidentBuf wout; ResidentBuf out_norm;     // output matrix (64-row tiles) and the final norm
     const float *x;                      // the embedding row of the token (written by the launch before this one)
     float *logits;
     const uint32_t *pos_ptr;
-    // hand-off buffers, filled with FLOW_EMPTY before every launch: xa [(n_layers + 1) x dim] (layer inputs; row 0 unused),
-    // xb, xm [n_layers x dim] (attention output, residual after the attention), hb [n_layers x hidden]
-    float *xa, *xb, *xm, *hb;
-    float *slots; uint32_t slot_stride;  // per-workgroup staging of the normalised input of a 64-row-tile phase
-    float *q, *kcol, *vcol;              // q / k / v of the current layer (handed over inside one XCD)
+    // hand-off buffers, filled with FLOW_EMPTY before every launch (layout: resident_plan.h, plan::flow_*)
+    float *flow;
+    float *slots;                        // per-workgroup staging of the normalised input of a 64-row-unit phase
+    float *q, *kcol, *vcol;              // q / k / v of the current layer (handed over inside one die)
     uint32_t *counters;                  // one 128-byte line per head
     uint32_t *abort_flag;                // set when a reader gave up
     uint64_t *trace;                     // optional: per workgroup 16 * n_layers + 8 time stamps (100 MHz clock); null = none

@@ -18,12 +18,7 @@ template <int BYTES> __device__ __forceinline__ void touch_kernel_arguments() {
     asm volatile("" : : "s"(w));
 }
 
-// A 64-bit value from two 32-bit words.  The words are taken as unsigned on purpose: the lane-broadcast builtins return
-// `int`, and an int with bit 31 set, widened on its way into a 64-bit "or", fills the upper word with ones -- a pointer
-// rebuilt that way is wrong for every address whose lower word is 0x80000000 or above.
-__host__ __device__ constexpr uint64_t join_words(uint32_t lo, uint32_t hi) { return ((uint64_t)hi << 32) | (uint64_t)lo; }
-static_assert(join_words(0x80000000u, 0x7fu) == 0x0000007f80000000ull, "the lower word must not be sign-extended");
-static_assert(join_words((uint32_t)(int)0xffffffffu, 0u) == 0x00000000ffffffffull, "an int -1 as lower word stays 32 bits wide");
+// A lane-broadcast word as an unsigned value (the builtin returns `int`; see join_words in resident_plan.h).
 __device__ __forceinline__ uint32_t uniform_word(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
 // ---- data exchanged between workgroups of one running kernel ---------------------------------------------------------

@@ -7,8 +7,10 @@
 #include "host_gguf.h"
 #include "llm_context.h"
 #include "quant_formats.h"
+#include "resident_plan.h"
 
 #include <algorithm>
+#include <cstdio>
 #include <cstring>
 #include <memory>
 
@@ -174,6 +176,7 @@ struct slai_llama2 {
     // The layer stack as ONE resident launch per token (kernels_decode_persistent.hip), for the models it covers.
     struct {
         bool ready = false;
+        mutable const char *why_not = nullptr;   // set when the context asked for the form and the model does not take it
         uint32_t grid = 0;
         PersistentParams params{};
         slai_buffer *layers = nullptr, *flow = nullptr, *slots = nullptr;
@@ -335,6 +338,8 @@ int slai_llama2::load(const slai_gguf *gg) {
     TRY(ensure_attn_scratch(ctx, attention_scratch_floats(config.n_q_heads, head_size(), attn_splits)));
     TRY(loop_init(ctx, loop, config.seq_len + 1));
     TRY(persistent_setup());
+    if (ctx->persistent && !persistent.ready)
+        fprintf(stderr, "slai: SLAI_PERSISTENT=1, but this model keeps one launch per step: %s\n", persistent.why_not ? persistent.why_not : "unknown");
     return slai_synchronize(ctx);
 }
 
@@ -344,68 +349,75 @@ int slai_llama2::load(const slai_gguf *gg) {
 // residual in 16-row tiles of Q4_K or Q6_K.  Everything else keeps the launch-per-step form.
 bool slai_llama2::persistent_supported() const {
     const uint32_t dim = config.dim, hid = config.hidden_dim, nh = config.n_q_heads;
-    if (!ctx->persistent || !ctx->fuse_qkv_attention || !ctx->rowtile_gemv || !ctx->handoff_counters || nh > ctx->handoff_heads) return false;
+    if (!ctx->persistent) return false;
+    const auto no = [&](const char *why) { persistent.why_not = why; return false; };
+    if (!ctx->fuse_qkv_attention) return no("workgroups are not placed on the dies round robin (or SLAI_FUSE_QKV_ATTN=0)");
+    if (!ctx->rowtile_gemv || !ctx->handoff_counters || nh > ctx->handoff_heads) return no("64-row tiles or the hand-off counters are switched off");
     if (config.n_kv_heads != nh || head_size() != 128 || nh % 8 || dim % 1024 || dim > 4096 || hid % 256 || hid / 256 > 64 || attn_splits != 1 || config.seq_len > 1024)
-        return false;
+        return no("shape: needs as many cache heads as query heads of size 128 (a multiple of 8), a width of 1024 .. 4096, an FFN width in super-blocks, a context of at most 1024");
     const auto kquant = [](int t) { return t == T_Q4_K || t == T_Q5_K || t == T_Q6_K; };
     const auto proj = [&](const slai_qmat *m, uint32_t cols) {
         return m->tiled && m->rows_log2 == 4 && (m->type == T_Q4_K || m->type == T_Q6_K) && m->ncb == cols / 256 && m->ngroups == (cols / 256 + 3) / 4 && m->ngroups <= 16;
     };
     for (const Llama2LayerWeights &w : weights.layers) {
         for (const slai_qmat *m : {w.attn_q, w.attn_k, w.attn_v})
-            if (!gemv_is_rowtile(ctx, m) || !kquant(m->type) || m->ncb != dim / 256) return false;
-        if (!gemv_is_rowtile(ctx, w.ffn_gate) || !gemv_is_rowtile(ctx, w.ffn_up) || w.ffn_gate->type != T_Q4_K || w.ffn_up->type != T_Q4_K) return false;
-        if (!proj(w.attn_output, dim) || !proj(w.ffn_down, hid)) return false;
+            if (!gemv_is_rowtile(ctx, m) || !kquant(m->type) || m->ncb != dim / 256) return no("q / k / v are not K-quants in 64-row tiles");
+        if (!gemv_is_rowtile(ctx, w.ffn_gate) || !gemv_is_rowtile(ctx, w.ffn_up) || w.ffn_gate->type != T_Q4_K || w.ffn_up->type != T_Q4_K)
+            return no("gate / up are not Q4_K in 64-row tiles");
+        if (!proj(w.attn_output, dim) || !proj(w.ffn_down, hid)) return no("the projections into the residual are not Q4_K / Q6_K in 16-row tiles");
     }
-    return gemv_is_rowtile(ctx, weights.output) && kquant(weights.output->type) && weights.output->ncb == dim / 256;
+    if (!(gemv_is_rowtile(ctx, weights.output) && kquant(weights.output->type) && weights.output->ncb == dim / 256)) return no("the output matrix is not a K-quant in 64-row tiles");
+    return true;
 }
 
+// Leaves persistent.ready set when the model takes the resident launch; otherwise persistent.why_not says why not (when
+// the context asked for the form at all).
 int slai_llama2::persistent_setup() {
     if (!persistent_supported()) return SLAI_OK;
+    const auto no = [&](const char *why) { persistent.why_not = why; return SLAI_OK; };
     const uint32_t dim = config.dim, hid = config.hidden_dim, nh = config.n_q_heads, nl = config.n_layers;
     PersistentParams &p = persistent.params;
     p.n_layers = nl; p.dim = dim; p.hidden = hid; p.n_heads = nh; p.seq_len = config.seq_len; p.vocab = config.vocab_size;
     p.eps = config.rms_norm_eps; p.rope_variant = rope_variant(); p.rope_base = config.rope_base_freq;
     p.rope_theta = (const float *)state.rope_theta.buf->dptr;
     p.kv_f16 = kv_dtype == SLAI_KV_F16;
-    p.wout = weights.output->dptr; p.tout = weights.output->type; p.out_norm = (const float *)weights.output_norm.buf->dptr;
+    // every matrix, vector and cache goes to the kernel with its size: the kernel reads them through buffer descriptors
+    bool fits = true;
+    const auto mat = [&](const slai_qmat *m) { if (m->bytes > 0xffffffffull) fits = false; return ResidentBuf{m->dptr, (uint32_t)m->bytes, (uint32_t)m->type}; };
+    const auto vec = [&](const GpuTensor &t) { return t.buf ? ResidentBuf{t.buf->dptr, (uint32_t)t.buf->bytes, 0u} : ResidentBuf{nullptr, 0u, 0u}; };
+    p.wout = mat(weights.output); p.out_norm = vec(weights.output_norm);
     p.x = (const float *)state.x.buf->dptr; p.logits = (float *)state.logits.buf->dptr;
     p.pos_ptr = (const uint32_t *)&((DecodeState *)loop.state->dptr)->pos;
     p.q = (float *)state.q.buf->dptr; p.kcol = (float *)state.kcol.buf->dptr; p.vcol = (float *)state.vcol.buf->dptr;
     p.counters = ctx->handoff_counters; p.abort_flag = ctx->handoff_counters + (size_t)ctx->handoff_heads * 32;
     // the device must keep the whole grid resident: every compute unit one workgroup, and enough of them for every role
     uint32_t resident = 0;
-    if (persistent_capacity(p, ctx->device, &resident) != hipSuccess) return SLAI_OK;
-    const uint32_t need = std::max(std::max(7 * nh, dim / 16), hid / 64);
+    p.qkv_units = 6; p.gu_rows = 64;                                  // (the occupancy query only needs the widths)
+    if (persistent_capacity(p, ctx->device, &resident) != hipSuccess) return no("the occupancy query for the kernel failed");
     hipDeviceProp_t prop;
     SLAI_HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
     const uint32_t grid = std::min(resident, (uint32_t)prop.multiProcessorCount) / 8 * 8;
-    if (grid < need) return SLAI_OK;
+    const plan::Shape sh = plan::make_shape(dim, hid, nh, nl, config.vocab_size, config.seq_len, grid);
+    if (!plan::shape_ok(sh)) return no("the device keeps too few workgroups of the kernel resident for this shape");
+    p.qkv_units = sh.qkv_units; p.gu_rows = sh.gu_rows;
     std::vector<PersistentLayer> host(nl);
     for (uint32_t l = 0; l < nl; ++l) {
         const Llama2LayerWeights &w = weights.layers[l];
         PersistentLayer &d = host[l];
-        d.wq = w.attn_q->dptr; d.wk = w.attn_k->dptr; d.wv = w.attn_v->dptr; d.tq = w.attn_q->type; d.tk = w.attn_k->type; d.tv = w.attn_v->type;
-        d.wo = w.attn_output->dptr; d.to = w.attn_output->type;
-        d.wgate = w.ffn_gate->dptr; d.wup = w.ffn_up->dptr; d.tg = w.ffn_gate->type;
-        d.wdown = w.ffn_down->dptr; d.td = w.ffn_down->type;
-        d.attn_norm = (const float *)w.attn_norm.buf->dptr; d.ffn_norm = (const float *)w.ffn_norm.buf->dptr;
-        d.bq = w.attn_q_bias.buf ? (const float *)w.attn_q_bias.buf->dptr : nullptr;
-        d.bk = w.attn_k_bias.buf ? (const float *)w.attn_k_bias.buf->dptr : nullptr;
-        d.bv = w.attn_v_bias.buf ? (const float *)w.attn_v_bias.buf->dptr : nullptr;
-        d.kcache = state.key_cache[l].buf->dptr; d.vcache = state.value_cache[l].buf->dptr;
+        d.wq = mat(w.attn_q); d.wk = mat(w.attn_k); d.wv = mat(w.attn_v); d.wo = mat(w.attn_output);
+        d.wgate = mat(w.ffn_gate); d.wup = mat(w.ffn_up); d.wdown = mat(w.ffn_down);
+        d.attn_norm = vec(w.attn_norm); d.ffn_norm = vec(w.ffn_norm);
+        d.bq = vec(w.attn_q_bias); d.bk = vec(w.attn_k_bias); d.bv = vec(w.attn_v_bias);
+        d.kcache = vec(state.key_cache[l]); d.vcache = vec(state.value_cache[l]);
     }
+    if (!fits) return no("a matrix beyond 4 GiB");
     TRY(slai_buffer_create(ctx, host.size() * sizeof(PersistentLayer), SLAI_DT_U8, STORAGE | COPY_DST, &persistent.layers));
     TRY(slai_write_buffer(ctx, persistent.layers, 0, host.data(), host.size() * sizeof(PersistentLayer)));
-    persistent.flow_bytes = ((size_t)(3 * nl + 1) * dim + (size_t)nl * hid) * sizeof(float);
+    persistent.flow_bytes = (size_t)plan::flow_floats(sh) * sizeof(float);
     TRY(slai_buffer_create(ctx, persistent.flow_bytes, SLAI_DT_F32, STORAGE, &persistent.flow));
-    p.slot_stride = dim + dim / 16 + 16;
-    TRY(slai_buffer_create(ctx, (size_t)grid * p.slot_stride * sizeof(float), SLAI_DT_F32, STORAGE, &persistent.slots));
+    TRY(slai_buffer_create(ctx, (size_t)plan::slot_floats(sh) * sizeof(float), SLAI_DT_F32, STORAGE, &persistent.slots));
     p.layers = (const PersistentLayer *)persistent.layers->dptr;
-    p.xa = (float *)persistent.flow->dptr;
-    p.xb = p.xa + (size_t)(nl + 1) * dim;
-    p.xm = p.xb + (size_t)nl * dim;
-    p.hb = p.xm + (size_t)nl * dim;
+    p.flow = (float *)persistent.flow->dptr;
     p.slots = (float *)persistent.slots->dptr;
     persistent.grid = grid;
     persistent.ready = true;

@@ -9,29 +9,37 @@
 //     before the launch (one buffer per layer and vector, so nothing is ever reused inside a launch);
 //   * a consumer repeats its agent-scope load of a piece until no element of it is empty -- the data is its own flag, so
 //     a hand-off is one store and one load deep, with no counter or barrier round trip in between;
-//   * the waves that multiply request ALL the weights of their next unit first and only then wait: the weights travel
+//   * the waves that multiply request the weights of their next unit first and only then wait: the weights travel
 //     while the activations are still being produced.  Loads retire in issue order, so the waiting is done by other waves
 //     of the workgroup ("stagers", which hold no outstanding weight requests) and handed over through LDS or through a
 //     per-workgroup slot that the multiplying waves read with scalar loads.
 // The arithmetic is that of the separate kernels (kernels_gemv_rowtile.hip, kernels_gemv_tiled.hip, attention_fast.h):
 // 64-row tiles with wave-uniform activations for q/k/v, gate/up and the output matrix, 16-row tiles with DPP-broadcast
-// activations for the two projections that add into the residual, one workgroup per head for the attention.
+// activations for the two projections that add into the residual, one workgroup per head for the attention.  Work is
+// cut into units of equal size rather than whole tiles (resident_plan.h): a unit of a 64-row-tile matrix is any run of up
+// to 64 rows, so that every compute unit streams the same number of bytes in a phase.
+//
+// Where things are: every offset the kernel forms comes from resident_plan.h, which a host program walks for every
+// (workgroup, wave, lane, layer) against the sizes of the allocations.  Weights, norm vectors and hand-off vectors are
+// read through buffer descriptors that carry those sizes, so an access outside of them reads zero (or is dropped)
+// instead of faulting.
 //
 // Every wait is bounded.  A reader that gives up sets a flag the host turns into an error, and from then on no reader of
-// the launch waits again, so a launch always ends.  The grid is exactly as large as the device can keep resident.
+// the launch waits again, so a launch always ends.  The grid is never larger than what the device keeps resident.
 #include "common.h"
 #include "attention_fast.h"
 #include <cstddef>
 #include "device_util.h"
 #include "gemv_operands.h"
 #include "quant_tiled.h"
+#include "resident_plan.h"
 
 namespace slai {
 namespace {
 
 using namespace lanes;
 
-constexpr int PNT = 1024, PNW = 16;                 // threads and waves of a workgroup
+constexpr int PNT = plan::WG_THREADS, PNW = plan::WG_WAVES;   // threads and waves of a workgroup
 
 // The thread index as a value the compiler cannot follow: what a phase derives from it (lane offsets, addresses) is then
 // computed inside the phase instead of being kept alive across the whole layer loop, where it would not fit the registers.
@@ -46,6 +54,62 @@ __device__ __forceinline__ int phase_tid() {
 __device__ __forceinline__ void stamp(uint64_t *row, uint32_t k) {
     if (row && threadIdx.x == 0) row[k] = wall_clock64();
 }
+
+// ---- memory seen through buffer descriptors ------------------------------------------------------------------------------
+// A descriptor holds the address and the size in bytes of one matrix or vector; loads and stores name a byte offset, and
+// the hardware compares it with the size: outside of it a load returns zero and a store is dropped.
+using Rsrc = __amdgpu_buffer_rsrc_t;
+typedef uint32_t u32x4b __attribute__((ext_vector_type(4)));
+constexpr int RSRC_WORD3 = 0x00020000;                        // untyped 32-bit data, no swizzle
+constexpr int AUX_PLAIN = 0;
+constexpr int AUX_FLOW = (int)0x80000010u;                    // agent scope (sc1): not served by a cache of this die; never merged or hoisted
+struct DevBuf {                                               // wave-uniform
+    Rsrc rs;
+    const void *ptr;
+    uint32_t bytes;
+    int type;
+};
+__device__ __forceinline__ Rsrc make_rsrc(const void *p, uint32_t bytes) { return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), (short)0, (int)bytes, RSRC_WORD3); }
+__device__ __forceinline__ DevBuf dev_buf(const void *p, uint32_t bytes, int type = 0) { return DevBuf{make_rsrc(p, bytes), p, bytes, type}; }
+__device__ __forceinline__ DevBuf dev_buf(const ResidentBuf &b) { return dev_buf(b.ptr, b.bytes, (int)b.type); }
+// entry `word` (in 32-bit words) of the layer description parked in LDS, as wave-uniform values
+__device__ __forceinline__ DevBuf layer_buf(const uint32_t *lw, uint32_t word) {
+    const uint64_t bits = join_words(uniform_word(lw[word]), uniform_word(lw[word + 1]));
+    return dev_buf((const void *)(uintptr_t)bits, uniform_word(lw[word + 2]), (int)uniform_word(lw[word + 3]));
+}
+#define LAYER_BUF(lw, field) layer_buf(lw, (uint32_t)(offsetof(PersistentLayer, field) / 4))
+static_assert(sizeof(ResidentBuf) == 16 && offsetof(ResidentBuf, ptr) == 0 && offsetof(ResidentBuf, bytes) == 8 && offsetof(ResidentBuf, type) == 12, "layer_buf reads these words");
+
+template <int AUX> __device__ __forceinline__ u32x4 buf_load16(Rsrc rs, uint32_t off, uint32_t soff = 0) {
+    const u32x4b v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, (int)soff, AUX);
+    return u32x4{v.x, v.y, v.z, v.w};
+}
+__device__ __forceinline__ float4 as_float4(u32x4 v) { return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)); }
+// one float of a hand-off vector, at agent scope
+__device__ __forceinline__ void flow_put(Rsrc rs, uint32_t index, float v) { __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rs, (int)(index * 4u), 0, AUX_FLOW); }
+
+// Issues the 16-byte pieces of one unit (of both matrices of a gated pair) on request of the dot product, through the
+// matrices' descriptors.  voff: byte offset of this lane's 16 bytes of piece 0; piece P lies P * 1024 further.
+template <int T, int N, int LD> struct BufUnitLoader {
+    static constexpr int DEPTH = LD;
+    static constexpr int LEAD = LD;
+    using F = Tiled<T>;
+    Rsrc rs[N];
+    uint32_t voff[N], toff[N];
+    typename F::Data *d[N];
+    uint16_t *t[N];
+    template <int P> __device__ __forceinline__ void piece() const {
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+            const u32x4b v = __builtin_amdgcn_raw_buffer_load_b128(rs[n], (int)voff[n], P * 1024, AUX_PLAIN);
+            d[n]->p[P] = U4{v.x, v.y, v.z, v.w};
+        }
+    }
+    __device__ __forceinline__ void tail() const {
+#pragma unroll
+        for (int n = 0; n < N; ++n) *t[n] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs[n], (int)toff[n], 0, AUX_PLAIN);
+    }
+};
 
 // ---- waiting for data -------------------------------------------------------------------------------------------------
 constexpr uint64_t FLOW_WAIT_TICKS = 2u * 1000u * 1000u;      // 20 ms of the 100 MHz clock: what a reader waits before it gives up (a token takes about 1)
@@ -68,56 +132,30 @@ __device__ __forceinline__ void flow_backoff(Flow &f, uint64_t &deadline) {
     }
 }
 
-// Waits until the 16 bytes at `probe` (one address for the whole wave: one request per round) are no longer empty.  A
-// wave that arrives long before its input is produced polls this one piece only; the pieces it actually needs are
-// fetched afterwards, when most of them are there.
-__device__ __forceinline__ void flow_probe(const float *probe, Flow &f) {
+// Waits until piece `piece` (16 bytes; one address for the whole wave: one request per round) of the hand-off vector is
+// no longer empty.  A wave that arrives long before its input is produced polls this one piece only; the pieces it
+// actually needs are fetched afterwards, when most of them are there.
+__device__ __forceinline__ void flow_probe(Rsrc x, uint32_t piece, Flow &f) {
     uint64_t deadline = 0;
     while (!f.dead) {
-        const u32x4 v = flow_load16(probe);
+        const u32x4 v = buf_load16<AUX_FLOW>(x, piece * 16u);
         if (!__any(flow_empty(v))) break;
         flow_backoff(f, deadline);
     }
 }
 
-// N (4 or 12) pieces of 16 bytes per lane, each once none of its words is empty: piece k of a lane sits `off0 + k * stride`
-// bytes into the vector at `base` and is requested when k < nlive.  One round trip for all of them, repeated by the whole
-// wave while any is incomplete (after a time-out the values are whatever was there; pieces not requested stay zero).
-// Everything between the first request and the arrival of the last result is ONE assembly block: the compiler does not
-// know that a register named by an earlier block is still being filled, and has been seen to copy such registers before
-// a wait placed in a later block.  Inside the block the loads run under an execution mask (no lane asks for a piece it
-// does not need) and the offset register is stepped by the stride.
-#define SLAI_FLOW_PIECE(K)                                                                                   \
-    "v_cmp_lt_u32 vcc, " #K ", %[nl]\n\ts_and_b64 exec, %[sv], vcc\n\t"                                      \
-    "global_load_dwordx4 %[v" #K "], %[t], %[base] sc1\n\ts_mov_b64 exec, %[sv]\n\tv_add_u32 %[t], %[st], %[t]\n\t"
+// N (4 or 12) pieces of 16 bytes per lane, each once none of its words is empty: piece k of a lane is piece number
+// first + k * step of the vector and is wanted when k < nlive.  One round trip for all of them, repeated by the whole
+// wave while any is incomplete (after a time-out the values are whatever was there).  A lane asks for the pieces it does
+// not want at `spare` (a piece of the vector that exists for every lane) and ignores what comes back, so that the
+// requests need no execution mask.
 template <int N>
-__device__ __forceinline__ void flow_acquire(const float *base, uint32_t off0, uint32_t stride, uint32_t nlive, u32x4 (&v)[N], Flow &f) {
+__device__ __forceinline__ void flow_acquire(Rsrc x, uint32_t first, uint32_t step, uint32_t nlive, uint32_t spare, u32x4 (&v)[N], Flow &f) {
     static_assert(N == 4 || N == 12, "four or twelve pieces");
-    const uint64_t base_bits = join_words(uniform_word((uint32_t)(uintptr_t)base), uniform_word((uint32_t)((uintptr_t)base >> 32)));
-    const uint32_t st = uniform_word(stride);
-#pragma unroll
-    for (int k = 0; k < N; ++k) v[k] = u32x4{0, 0, 0, 0};
     uint64_t deadline = 0;
     for (;;) {
-        uint64_t saved;
-        uint32_t t;
-        if constexpr (N == 4) {
-            asm volatile("s_mov_b64 %[sv], exec\n\tv_mov_b32 %[t], %[off0]\n\t"
-                         SLAI_FLOW_PIECE(0) SLAI_FLOW_PIECE(1) SLAI_FLOW_PIECE(2) SLAI_FLOW_PIECE(3)
-                         "s_waitcnt vmcnt(0)"
-                         : [v0] "+v"(v[0]), [v1] "+v"(v[1]), [v2] "+v"(v[2]), [v3] "+v"(v[3]), [sv] "=&s"(saved), [t] "=&v"(t)
-                         : [base] "s"(base_bits), [off0] "v"(off0), [st] "s"(st), [nl] "v"(nlive)
-                         : "memory", "vcc", "scc");
-        } else {
-            asm volatile("s_mov_b64 %[sv], exec\n\tv_mov_b32 %[t], %[off0]\n\t"
-                         SLAI_FLOW_PIECE(0) SLAI_FLOW_PIECE(1) SLAI_FLOW_PIECE(2) SLAI_FLOW_PIECE(3) SLAI_FLOW_PIECE(4) SLAI_FLOW_PIECE(5)
-                         SLAI_FLOW_PIECE(6) SLAI_FLOW_PIECE(7) SLAI_FLOW_PIECE(8) SLAI_FLOW_PIECE(9) SLAI_FLOW_PIECE(10) SLAI_FLOW_PIECE(11)
-                         "s_waitcnt vmcnt(0)"
-                         : [v0] "+v"(v[0]), [v1] "+v"(v[1]), [v2] "+v"(v[2]), [v3] "+v"(v[3]), [v4] "+v"(v[4]), [v5] "+v"(v[5]), [v6] "+v"(v[6]),
-                           [v7] "+v"(v[7]), [v8] "+v"(v[8]), [v9] "+v"(v[9]), [v10] "+v"(v[10]), [v11] "+v"(v[11]), [sv] "=&s"(saved), [t] "=&v"(t)
-                         : [base] "s"(base_bits), [off0] "v"(off0), [st] "s"(st), [nl] "v"(nlive)
-                         : "memory", "vcc", "scc");
-        }
+#pragma unroll
+        for (int k = 0; k < N; ++k) v[k] = buf_load16<AUX_FLOW>(x, ((uint32_t)k < nlive ? first + (uint32_t)k * step : spare) * 16u);
         bool hole = false;
 #pragma unroll
         for (int k = 0; k < N; ++k) hole = hole || ((uint32_t)k < nlive && flow_empty(v[k]));
@@ -125,13 +163,12 @@ __device__ __forceinline__ void flow_acquire(const float *base, uint32_t off0, u
         flow_backoff(f, deadline);
     }
 }
-#undef SLAI_FLOW_PIECE
 
-// ---- a 64-row tile (q / k / v, gate + up, output matrix) -----------------------------------------------------------------
+// ---- a unit of up to 64 rows of a 64-row-tile matrix (q / k / v, gate + up, output matrix) -------------------------------
 struct TileIn {
-    const float *x;           // the input vector (n floats)
-    bool flow;                // written by this launch: read with flow_acquire16; else ordinary memory from before the launch
-    const float *norm_w;      // RMSNorm weights
+    Rsrc x;                   // the input vector (n floats)
+    bool flow;                // written by this launch: read with flow_acquire; else ordinary memory from before the launch
+    Rsrc norm_w;              // RMSNorm weights (n floats)
     uint32_t n;               // columns
     float eps;
 };
@@ -140,32 +177,31 @@ struct TileIn {
 // red[0..3]: the last four waves of the workgroup, up to four 16-byte pieces per lane (n <= 4096).  rms_norm.slang:48-67;
 // the scale is applied to the finished dot product.
 __device__ __forceinline__ void stage_tile_input(const TileIn &in, float *slot, float *red, Flow &f) {
-    const int tid = phase_tid(), lane = tid & 63, wave = tid >> 6;
-    const uint32_t l = tid - (PNW - 4) * 64;                       // 0 .. 255
+    const uint32_t tid = (uint32_t)phase_tid(), lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l = plan::stage64_lane(tid);                  // 0 .. 255
     uint32_t idx[4];
     bool live[4];
     float4 w[4];
     uint32_t nlive = 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {                                   // the norm weights first: they depend on nothing
-        idx[k] = l + 256 * k;
-        live[k] = idx[k] < in.n / 4;
+        idx[k] = plan::stage64_piece(l, k);
+        live[k] = plan::stage64_live(l, k, in.n);
         nlive += live[k] ? 1u : 0u;
-        w[k] = *reinterpret_cast<const float4 *>(in.norm_w + 4 * (live[k] ? idx[k] : l));
+        w[k] = as_float4(buf_load16<AUX_PLAIN>(in.norm_w, (live[k] ? idx[k] : l) * 16u));
     }
     u32x4 raw[4];
     if (in.flow) {
-        const uint32_t first = 64u * (uint32_t)(wave - (PNW - 4));       // the first piece of this wave's share
-        flow_probe(in.x + 4 * (size_t)(first < in.n / 4 ? first : 0), f);
-        flow_acquire<4>(in.x, l * 16u, 256u * 16u, nlive, raw, f);
+        flow_probe(in.x, plan::stage64_probe(wave, in.n), f);
+        flow_acquire<4>(in.x, l, 256u, nlive, l, raw, f);
     } else {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) raw[k] = *reinterpret_cast<const u32x4 *>(in.x + 4 * (live[k] ? idx[k] : l));
+        for (int k = 0; k < 4; ++k) raw[k] = buf_load16<AUX_PLAIN>(in.x, (live[k] ? idx[k] : l) * 16u);
     }
     float ss = 0.0f;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        float4 v = make_float4(__uint_as_float(raw[k].x), __uint_as_float(raw[k].y), __uint_as_float(raw[k].z), __uint_as_float(raw[k].w));
+        float4 v = as_float4(raw[k]);
         if (!live[k]) v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
         v.x *= w[k].x; v.y *= w[k].y; v.z *= w[k].z; v.w *= w[k].w;
@@ -178,15 +214,16 @@ __device__ __forceinline__ void stage_tile_input(const TileIn &in, float *slot, 
         }
     }
     ss = wave_sum(ss);
-    if (lane == 0) red[wave - (PNW - 4)] = ss;
+    if (lane == 0) red[wave - (PNW - plan::STAGERS64)] = ss;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");               // the slot is in L2 before the barrier lets the readers go
 }
 
-// One tile: rows tile*64 .. +63 of W (and W2) times the staged input; returns, in threads 0..63, the finished value of the
-// thread's row (scaled; gate/up combined with SiLU when DUAL).  `stage`: false when the slot still holds this input.
+// One unit: rows unit.row0 .. + unit.nrows - 1 of W (and W2) times the staged input; returns, in threads 0 .. nrows - 1,
+// the finished value of row unit.row0 + thread (scaled; gate/up combined with SiLU when DUAL).  `stage`: false when the
+// slot still holds this input.
 // smem: partial[2][16][64], red[2][4] (red alternates between calls so that a fast wave cannot overwrite it early).
 template <int T, bool DUAL>
-__device__ __forceinline__ float tile64_phase(const uint8_t *W, const uint8_t *W2, uint32_t tile, uint32_t ncb, const TileIn &in, bool stage,
+__device__ __forceinline__ float tile64_phase(const DevBuf &W, const DevBuf &W2, const plan::RowUnit unit, uint32_t ncb, const TileIn &in, bool stage,
                                               float *slot, float *partial, float *red, Flow &f, uint64_t *tr) {
     using F = Tiled<T>;
     const int tid = phase_tid(), lane = tid & 63;
@@ -194,16 +231,18 @@ __device__ __forceinline__ float tile64_phase(const uint8_t *W, const uint8_t *W
     constexpr uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
     constexpr int NM = DUAL ? 2 : 1;
     const bool has_unit = (uint32_t)wave < ncb;
-    const bool stager = wave >= PNW - 4;
+    const bool stager = wave >= PNW - (int)plan::STAGERS64;
     typename F::Data d, e;
     uint16_t dt = 0, et = 0;
     // As much of the unit as the registers hold without spilling is requested before the wait (a spill of a requested
     // piece would make the wave wait for it before the barrier); the rest follows while the first stages are multiplied.
-    UnitLoader<T, NM, DUAL ? 4 : (F::PT > 9 ? 6 : 8)> ld;
+    BufUnitLoader<T, NM, DUAL ? 4 : (F::PT > 9 ? 6 : 8)> ld;
     auto request = [&]() {
-        const size_t off = ((size_t)tile * ncb + wave) * unit_bytes;
-        ld.unit[0] = W + off + lane * 16; ld.tailp[0] = W + off + (size_t)F::PT * 1024 + lane * 2; ld.d[0] = &d; ld.t[0] = &dt;
-        if constexpr (DUAL) { ld.unit[1] = W2 + off + lane * 16; ld.tailp[1] = W2 + off + (size_t)F::PT * 1024 + lane * 2; ld.d[1] = &e; ld.t[1] = &et; }
+        const uint32_t row = unit.row0 + plan::umin((uint32_t)lane, unit.nrows - 1);     // lanes past the unit repeat its last row
+        const uint32_t voff = plan::tile64_piece0(row, (uint32_t)wave, ncb, unit_bytes);
+        const uint32_t toff = plan::tile64_tail(row, (uint32_t)wave, ncb, unit_bytes, F::PT);
+        ld.rs[0] = W.rs; ld.voff[0] = voff; ld.toff[0] = toff; ld.d[0] = &d; ld.t[0] = &dt;
+        if constexpr (DUAL) { ld.rs[1] = W2.rs; ld.voff[1] = voff; ld.toff[1] = toff; ld.d[1] = &e; ld.t[1] = &et; }
         F::lead(ld);
     };
     stamp(tr, 0);
@@ -223,7 +262,7 @@ __device__ __forceinline__ float tile64_phase(const uint8_t *W, const uint8_t *W
         uint64_t slot_bits = (uint64_t)(uintptr_t)slot;
         asm volatile("" : "+s"(slot_bits) : : "memory");
         cfloat *xsc = (cfloat *)slot_bits;
-        ScalarX X{xsc + (size_t)wave * 256, xsc + in.n + (size_t)wave * 16};
+        ScalarX X{xsc + plan::slot_x((uint32_t)wave), xsc + in.n + (size_t)wave * 16};
         const typename F::Data *dp[NM];
         uint16_t tails[NM];
         float o2[NM];
@@ -255,24 +294,25 @@ __device__ __forceinline__ float tile64_phase(const uint8_t *W, const uint8_t *W
 }
 
 // ---- a 16-row tile (attention output projection, down projection) -------------------------------------------------------
-// Rows tile*16 .. +15 of W times the n-vector at `x` (written by this launch); returns the row's dot product in threads
+// Rows tile*16 .. +15 of W times the n-vector `x` (written by this launch); returns the row's dot product in threads
 // 0..15.  Waves 0 .. ngroups-1 multiply (one unit of 16 rows x 4 super-blocks each), the others fetch the vector into xs.
 template <int T>
-__device__ __forceinline__ float tile16_phase(const uint8_t *W, uint32_t tile, uint32_t ncb, uint32_t ngroups, const float *x, uint32_t n, float *xs,
+__device__ __forceinline__ float tile16_phase(const DevBuf &W, uint32_t tile, uint32_t ncb, uint32_t ngroups, Rsrc x, uint32_t n, float *xs,
                                               float *partial, Flow &f, uint64_t *tr) {
     using F = Tiled<T>;
     const int tid = phase_tid(), lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
     const bool has_unit = (uint32_t)wave < ngroups;
-    const uint32_t first_stager = ngroups < 12 ? ngroups : 12;
+    const uint32_t first_stager = plan::stage16_first(ngroups);
     const bool stager = (uint32_t)wave >= first_stager;
     typename F::Data d;
     uint16_t dt = 0;
-    UnitLoader<T, 1, (F::PT > 9 ? 6 : 8)> ld;
+    BufUnitLoader<T, 1, (F::PT > 9 ? 6 : 8)> ld;
     auto request = [&]() {
-        const size_t off = ((size_t)tile * ngroups + wave) * unit_bytes;
-        ld.unit[0] = W + off + lane * 16; ld.tailp[0] = W + off + (size_t)F::PT * 1024 + lane * 2; ld.d[0] = &d; ld.t[0] = &dt;
+        ld.rs[0] = W.rs; ld.d[0] = &d; ld.t[0] = &dt;
+        ld.voff[0] = plan::tile16_piece0(tile, (uint32_t)wave, ngroups, unit_bytes, (uint32_t)lane);
+        ld.toff[0] = plan::tile16_tail(tile, (uint32_t)wave, ngroups, unit_bytes, F::PT, (uint32_t)lane);
         F::lead(ld);
     };
     stamp(tr, 0);
@@ -280,27 +320,25 @@ __device__ __forceinline__ float tile16_phase(const uint8_t *W, uint32_t tile, u
         if (has_unit) request();
     } else {
         // lane l of the nl stager lanes takes pieces l, l + nl, ...: four per round trip, or twelve when there are many
-        const uint32_t nl = (PNW - first_stager) * 64, l = tid - first_stager * 64;
+        const uint32_t nl = plan::stage16_lanes(ngroups), l = (uint32_t)tid - first_stager * 64u;
         const uint32_t chunks = n / 4;
-        {
-            const uint32_t first = (uint32_t)(wave - first_stager) * 64;            // the wave's first piece (if it has one)
-            flow_probe(x + 4 * (size_t)(first < chunks ? first : 0), f);
-        }
-        if (chunks > 4 * nl) {
-            const uint32_t trips = (chunks + 12 * nl - 1) / (12 * nl);
+        flow_probe(x, plan::stage16_probe((uint32_t)wave, ngroups, chunks), f);
+        const uint32_t spare = (uint32_t)lane;                                   // (chunks >= 64: n >= 256)
+        if (plan::stage16_per_trip(chunks, nl) == 12u) {
+            const uint32_t trips = plan::stage16_trips(chunks, nl);
             for (uint32_t j = 0; j < trips; ++j) {                     // whole waves call the acquire
-                const uint32_t i0 = 12 * j * nl + l;
-                const uint32_t nlive = i0 < chunks ? min(12u, (chunks - i0 + nl - 1) / nl) : 0u;
+                const uint32_t i0 = plan::stage16_first_piece(l, nl, j, 12u);
+                const uint32_t nlive = plan::stage16_nlive(i0, nl, chunks, 12u);
                 u32x4 raw[12];
-                flow_acquire<12>(x, i0 * 16u, nl * 16u, nlive, raw, f);
+                flow_acquire<12>(x, i0, nl, nlive, spare, raw, f);
 #pragma unroll
                 for (int k = 0; k < 12; ++k)
                     if ((uint32_t)k < nlive) *reinterpret_cast<u32x4 *>(xs + 4 * (size_t)(i0 + k * nl)) = raw[k];
             }
         } else {
-            const uint32_t nlive = l < chunks ? min(4u, (chunks - l + nl - 1) / nl) : 0u;
+            const uint32_t nlive = plan::stage16_nlive(l, nl, chunks, 4u);
             u32x4 raw[4];
-            flow_acquire<4>(x, l * 16u, nl * 16u, nlive, raw, f);
+            flow_acquire<4>(x, l, nl, nlive, spare, raw, f);
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 if ((uint32_t)k < nlive) *reinterpret_cast<u32x4 *>(xs + 4 * (size_t)(l + k * nl)) = raw[k];
@@ -343,25 +381,26 @@ __device__ __forceinline__ float tile16_phase(const uint8_t *W, uint32_t tile, u
 }
 
 template <bool DUAL>
-__device__ __forceinline__ float tile64_any(int type, const uint8_t *W, const uint8_t *W2, uint32_t tile, uint32_t ncb, const TileIn &in, bool stage,
+__device__ __forceinline__ float tile64_any(const DevBuf &W, const DevBuf &W2, const plan::RowUnit unit, uint32_t ncb, const TileIn &in, bool stage,
                                             float *slot, float *partial, float *red, Flow &f, uint64_t *tr) {
-    switch (type) {                                                // uniform over the workgroup
-    case T_Q6_K: if constexpr (!DUAL) return tile64_phase<T_Q6_K, false>(W, W2, tile, ncb, in, stage, slot, partial, red, f, tr); else return 0.0f;
-    case T_Q5_K: if constexpr (!DUAL) return tile64_phase<T_Q5_K, false>(W, W2, tile, ncb, in, stage, slot, partial, red, f, tr); else return 0.0f;
-    default: return tile64_phase<T_Q4_K, DUAL>(W, W2, tile, ncb, in, stage, slot, partial, red, f, tr);
+    switch (W.type) {                                              // uniform over the workgroup
+    case T_Q6_K: if constexpr (!DUAL) return tile64_phase<T_Q6_K, false>(W, W2, unit, ncb, in, stage, slot, partial, red, f, tr); else return 0.0f;
+    case T_Q5_K: if constexpr (!DUAL) return tile64_phase<T_Q5_K, false>(W, W2, unit, ncb, in, stage, slot, partial, red, f, tr); else return 0.0f;
+    default: return tile64_phase<T_Q4_K, DUAL>(W, W2, unit, ncb, in, stage, slot, partial, red, f, tr);
     }
 }
-__device__ __forceinline__ float tile16_any(int type, const uint8_t *W, uint32_t tile, uint32_t ncb, uint32_t ngroups, const float *x, uint32_t n, float *xs,
+__device__ __forceinline__ float tile16_any(const DevBuf &W, uint32_t tile, uint32_t ncb, uint32_t ngroups, Rsrc x, uint32_t n, float *xs,
                                             float *partial, Flow &f, uint64_t *tr) {
-    if (type == T_Q6_K) return tile16_phase<T_Q6_K>(W, tile, ncb, ngroups, x, n, xs, partial, f, tr);
+    if (W.type == T_Q6_K) return tile16_phase<T_Q6_K>(W, tile, ncb, ngroups, x, n, xs, partial, f, tr);
     return tile16_phase<T_Q4_K>(W, tile, ncb, ngroups, x, n, xs, partial, f, tr);
 }
 
+__device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
+    return plan::Shape{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, gridDim.x, p.qkv_units, p.gu_rows};
+}
+
 // ---- the kernel ------------------------------------------------------------------------------------------------------------
-// Workgroup roles.  q/k/v: workgroup i < 6 * n_heads takes tile (i / 8) % 6 of head (i % 8) + 8 * (i / 48) (two tiles each
-// of v, k, q: the six tiles of a head run on one XCD, like the attention workgroup a0 + h of that head, a0 = 6 * n_heads;
-// their hand-off goes through that XCD's L2, see kernels_gemv_rowtile.hip).  Projections: workgroup b takes rows 16b .. 16b+15
-// and keeps their residual values from layer to layer.  gate/up: workgroup b takes rows 64b .. 64b+63.
+// Workgroup roles: resident_plan.h (plan::qkv_unit, attention_head, gu_unit, proj_tiles, out_tiles).
 template <bool F16>
 __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const PersistentParams p) {
     extern __shared__ __align__(16) float smem[];
@@ -369,68 +408,69 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
     // The description of the current layer and of the next one.  Read from memory at the moment of use, its lines (which
     // the weight stream has long pushed out of L2) would cost a round trip to memory each, one after the other.
     constexpr int LWORDS = sizeof(PersistentLayer) / 4;
+    static_assert(LWORDS <= PNT && sizeof(PersistentLayer) == 14 * sizeof(ResidentBuf), "one thread per word; fourteen entries");
     __shared__ uint32_t layer_words[2][LWORDS];
-    float *partial = smem;                                         // [2][16][64]
-    float *red = smem + 2 * PNW * 64;                              // [2][4]
-    float *xs = red + 8;                                           // [max(dim, hidden)]
+    float *partial = smem + plan::lds_partial();                   // [2][16][64]
+    float *red = smem + plan::lds_red();                           // [2][4]
+    float *xs = smem + plan::lds_xs();                             // [max(dim, hidden)]
     touch_kernel_arguments<sizeof(PersistentParams)>();
     const uint32_t b = blockIdx.x;
     // A launch after one in which a reader gave up does nothing: the host has not looked yet (it queues many tokens), and
     // every further token would only wait out the same time limits.
     if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
     Flow f{p.abort_flag, false};
+    const plan::Shape sh = shape_of(p);
     const uint32_t dim = p.dim, hid = p.hidden, nh = p.n_heads;
     const uint32_t ncb = dim / 256, ncb_h = hid / 256, ng_o = ncb / 4, ng_d = (ncb_h + 3) / 4;
-    const uint32_t a0 = 6 * nh;
-    float *slot = p.slots + (size_t)b * p.slot_stride;
+    float *slot = p.slots + plan::slot_of(sh, b);
     // time stamps: 16 per layer (4 per phase: entered, input staged, multiplied, reduced), then 4 for the output matrix and the end
-    uint64_t *trace = p.trace ? p.trace + (size_t)b * (16 * p.n_layers + 8) : nullptr;
+    uint64_t *trace = p.trace ? p.trace + plan::trace_row(sh, b) : nullptr;
     uint32_t phase = 0;                                            // parity picks the red[] half
     // the residual value of row 16b + tid: the embedding row the launch before this one left in p.x
     float xres = 0.0f;
-    if (b < dim / 16 && threadIdx.x < 16) xres = p.x[16 * b + threadIdx.x];
+    if (b < plan::proj_tiles(sh) && threadIdx.x < 16) xres = p.x[16 * b + threadIdx.x];
     if (threadIdx.x == 0) wg_dead = 0;
-    if (threadIdx.x < LWORDS && p.n_layers) layer_words[0][threadIdx.x] = reinterpret_cast<const uint32_t *>(p.layers)[threadIdx.x];
+    if (threadIdx.x < LWORDS) layer_words[0][threadIdx.x] = reinterpret_cast<const uint32_t *>(p.layers)[threadIdx.x];
     __syncthreads();
 
     for (uint32_t l = 0; l < p.n_layers; ++l) {
-        // this layer's description comes out of LDS field by field, as wave-uniform values, where it is used; the next
+        // this layer's description comes out of LDS entry by entry, as wave-uniform values, where it is used; the next
         // one's is requested now and parked in LDS at the end of the layer
         const uint32_t *lw = layer_words[l & 1u];
-#define LPTR(T, field) ((T)(uintptr_t)join_words(uniform_word(lw[offsetof(PersistentLayer, field) / 4]), uniform_word(lw[offsetof(PersistentLayer, field) / 4 + 1])))
-#define LINT(field) ((int)uniform_word(lw[offsetof(PersistentLayer, field) / 4]))
         uint32_t next_word = 0;
         if (threadIdx.x < LWORDS && l + 1 < p.n_layers) next_word = reinterpret_cast<const uint32_t *>(p.layers + l + 1)[threadIdx.x];
         uint64_t *tl = trace ? trace + 16 * l : nullptr;
-        float *xa = p.xa + (size_t)l * dim, *xb = p.xb + (size_t)l * dim, *xm = p.xm + (size_t)l * dim, *hb = p.hb + (size_t)l * hid;
+        // the hand-off vectors of this layer, each behind a descriptor of its own size
+        const Rsrc xa = make_rsrc(p.flow + plan::flow_xa(sh, l), dim * 4u), xb = make_rsrc(p.flow + plan::flow_xb(sh, l), dim * 4u);
+        const Rsrc xm = make_rsrc(p.flow + plan::flow_xm(sh, l), dim * 4u), hb = make_rsrc(p.flow + plan::flow_hb(sh, l), hid * 4u);
+        const Rsrc xnext = make_rsrc(p.flow + plan::flow_xa(sh, l + 1), dim * 4u);
         // ---- q / k / v and the attention ---------------------------------------------------------------------------
-        if (b < a0) {
-            const uint32_t j = b >> 3, t = j % 6, h = (b & 7u) + 8u * (j / 6);
-            const int s = (int)(t >> 1);                           // 0: v, 1: k, 2: q
-            const uint32_t tile = 2 * h + (t & 1u);
-            const uint8_t *W = s == 0 ? LPTR(const uint8_t *, wv) : (s == 1 ? LPTR(const uint8_t *, wk) : LPTR(const uint8_t *, wq));
-            const int type = s == 0 ? LINT(tv) : (s == 1 ? LINT(tk) : LINT(tq));
-            float *out = s == 0 ? p.vcol : (s == 1 ? p.kcol : p.q);
-            const TileIn in{l == 0 ? p.x : xa, l != 0, LPTR(const float *, attn_norm), dim, p.eps};
-            const float o = tile64_any<false>(type, W, nullptr, tile, ncb, in, true, slot, partial, red + 4 * (phase & 1u), f, tl);
+        if (b < plan::qkv_workgroups(sh)) {
+            const plan::RowUnit u = plan::qkv_unit(sh, b);
+            const uint32_t h = plan::qkv_head(sh, b);
+            const DevBuf W = u.seg == 0 ? LAYER_BUF(lw, wv) : (u.seg == 1 ? LAYER_BUF(lw, wk) : LAYER_BUF(lw, wq));
+            float *out = u.seg == 0 ? p.vcol : (u.seg == 1 ? p.kcol : p.q);
+            const TileIn in{l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, LAYER_BUF(lw, attn_norm).rs, dim, p.eps};
+            const float o = tile64_any<false>(W, W, u, ncb, in, true, slot, partial, red + 4 * (phase & 1u), f, tl);
             const uint32_t tid = phase_tid();
             if (tid < 64) {
-                flow_store(out + (size_t)tile * 64 + tid, o);
+                if (tid < u.nrows) flow_store(out + u.row0 + tid, o);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                if (tid == 0) __hip_atomic_fetch_add(p.counters + (size_t)h * 32, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (tid == 0) __hip_atomic_fetch_add(p.counters + plan::counter_word(h), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
             ++phase;
-        } else if (b < a0 + nh) {
-            const uint32_t h = b - a0;
+        } else if (plan::is_attention_workgroup(sh, b)) {
+            const uint32_t h = plan::attention_head(sh, b);
             AttnLaunch a{};
             a.q = p.q; a.knew = p.kcol; a.vnew = p.vcol;
-            a.kcache = LPTR(void *, kcache); a.vcache = LPTR(void *, vcache); a.kv_f16 = F16;
+            a.kcache = const_cast<void *>(LAYER_BUF(lw, kcache).ptr); a.vcache = const_cast<void *>(LAYER_BUF(lw, vcache).ptr); a.kv_f16 = F16;
             a.n_heads = nh; a.kv_mul = 1; a.head_size = 128; a.kv_dim = dim; a.seq_len = p.seq_len;
             a.pos_ptr = p.pos_ptr;
-            a.qbias = LPTR(const float *, bq); a.kbias = LPTR(const float *, bk); a.vbias = LPTR(const float *, bv);
+            a.qbias = (const float *)LAYER_BUF(lw, bq).ptr; a.kbias = (const float *)LAYER_BUF(lw, bk).ptr; a.vbias = (const float *)LAYER_BUF(lw, bv).ptr;
             a.rope_variant = p.rope_variant; a.rope_base = p.rope_base; a.rope_theta = p.rope_theta;
-            a.out = xb; a.scratch = nullptr; a.n_splits = 1;
-            uint32_t *counter = p.counters + (size_t)h * 32;
+            a.out = p.flow + plan::flow_xb(sh, l); a.scratch = nullptr; a.n_splits = 1;
+            uint32_t *counter = p.counters + plan::counter_word(h);
+            const uint32_t need = p.qkv_units;
             const uint32_t tid = phase_tid();
             stamp(tl, 0);
             attn::attn_fast_body<F16, PNT, 128, true, true, 8, true>(a, h, 0u, tid, [&]() {
@@ -442,7 +482,7 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
                         // a read-modify-write that returns the value executes in the L2 the producers' atomics went to
                         const uint32_t zero = 0;
                         asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=&v"(seen) : "v"(counter), "v"(zero) : "memory");
-                        if (seen >= 6u) break;
+                        if (seen >= need) break;
                         if ((++spins & 15u) == 0) {
                             const uint64_t now = wall_clock64();
                             if (deadline == 0) deadline = now + FLOW_WAIT_TICKS;
@@ -451,6 +491,7 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
                     }
                     if (gave_up) { wg_dead = 1; __hip_atomic_store(f.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
                     *counter = 0u;                                 // for the next layer; nobody else touches it until then
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 }
                 __syncthreads();
                 asm volatile("" ::: "memory");
@@ -459,42 +500,41 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
             stamp(tl, 3);
         }
         // ---- attention output projection into the residual ---------------------------------------------------------
-        if (b < dim / 16) {
-            const float o = tile16_any(LINT(to), LPTR(const uint8_t *, wo), b, ncb, ng_o, xb, dim, xs, partial, f, tl ? tl + 4 : nullptr);
+        if (b < plan::proj_tiles(sh)) {
+            const float o = tile16_any(LAYER_BUF(lw, wo), b, ncb, ng_o, xb, dim, xs, partial, f, tl ? tl + 4 : nullptr);
             const uint32_t tid = phase_tid();
-            if (tid < 16) { xres += o; flow_store(xm + 16 * b + tid, xres); }          // transformer.rs:352-355
+            if (tid < 16) { xres += o; flow_put(xm, 16 * b + tid, xres); }             // transformer.rs:352-355
         }
         // ---- RMSNorm + gate / up + SiLU ---------------------------------------------------------------------------------
-        if (b < hid / 64) {
-            const TileIn in{xm, true, LPTR(const float *, ffn_norm), dim, p.eps};
-            const float o = tile64_any<true>(LINT(tg), LPTR(const uint8_t *, wgate), LPTR(const uint8_t *, wup), b, ncb, in, true, slot, partial, red + 4 * (phase & 1u), f, tl ? tl + 8 : nullptr);
-            if (phase_tid() < 64) flow_store(hb + 64 * b + phase_tid(), o);
+        if (b < plan::gu_units(sh)) {
+            const plan::RowUnit u = plan::gu_unit(sh, b);
+            const TileIn in{xm, true, LAYER_BUF(lw, ffn_norm).rs, dim, p.eps};
+            const float o = tile64_any<true>(LAYER_BUF(lw, wgate), LAYER_BUF(lw, wup), u, ncb, in, true, slot, partial, red + 4 * (phase & 1u), f, tl ? tl + 8 : nullptr);
+            const uint32_t tid = phase_tid();
+            if (tid < u.nrows) flow_put(hb, u.row0 + tid, o);
             ++phase;
         }
         // ---- down projection into the residual ----------------------------------------------------------------------------
-        if (b < dim / 16) {
-            const float o = tile16_any(LINT(td), LPTR(const uint8_t *, wdown), b, ncb_h, ng_d, hb, hid, xs, partial, f, tl ? tl + 12 : nullptr);
-            float *next = p.xa + (size_t)(l + 1) * dim;
+        if (b < plan::proj_tiles(sh)) {
+            const float o = tile16_any(LAYER_BUF(lw, wdown), b, ncb_h, ng_d, hb, hid, xs, partial, f, tl ? tl + 12 : nullptr);
             const uint32_t tid = phase_tid();
-            if (tid < 16) { xres += o; flow_store(next + 16 * b + tid, xres); }      // transformer.rs:362-365
+            if (tid < 16) { xres += o; flow_put(xnext, 16 * b + tid, xres); }          // transformer.rs:362-365
         }
         if (threadIdx.x < LWORDS) layer_words[(l + 1) & 1u][threadIdx.x] = next_word;
         lds_barrier();
-#undef LPTR
-#undef LINT
     }
     // ---- final RMSNorm and the output matrix: tiles b, b + grid, ... -------------------------------------------------------
     {
-        const uint32_t ntiles = (p.vocab + 63) / 64;
-        const float *xl = p.n_layers ? p.xa + (size_t)p.n_layers * dim : p.x;
-        const TileIn in{xl, p.n_layers != 0, p.out_norm, dim, p.eps};
+        const uint32_t ntiles = plan::out_tiles(sh);
+        const TileIn in{make_rsrc(p.flow + plan::flow_xa(sh, p.n_layers), dim * 4u), true, dev_buf(p.out_norm).rs, dim, p.eps};
+        const DevBuf wout = dev_buf(p.wout);
         bool first = true;
         const uint32_t par = phase & 1u;                            // the input is staged once: its sum of squares stays where it is
         for (uint32_t tile = b; tile < ntiles; tile += gridDim.x) {
-            const float o = tile64_any<false>(p.tout, p.wout, nullptr, tile, ncb, in, first, slot, partial, red + 4 * par, f, first && trace ? trace + 16 * p.n_layers : nullptr);
+            const plan::RowUnit u{0u, tile * 64u, plan::umin(64u, p.vocab - tile * 64u)};
+            const float o = tile64_any<false>(wout, wout, u, ncb, in, first, slot, partial, red + 4 * par, f, first && trace ? trace + 16 * p.n_layers : nullptr);
             const uint32_t tid = phase_tid();
-            const uint32_t row = tile * 64 + tid;
-            if (tid < 64 && row < p.vocab) p.logits[row] = o;
+            if (tid < u.nrows) p.logits[u.row0 + tid] = o;
             first = false;
             lds_barrier();                                         // partial[] is reused by the next tile
         }
@@ -511,7 +551,8 @@ __global__ void flow_fill_kernel(u32x4 *buf, size_t n16) {
 }  // namespace
 
 size_t persistent_smem_bytes(const PersistentParams &p) {
-    return ((size_t)2 * PNW * 64 + 8 + (p.dim > p.hidden ? p.dim : p.hidden)) * sizeof(float);
+    const plan::Shape s{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, 0, p.qkv_units, p.gu_rows};
+    return (size_t)plan::lds_floats(s) * sizeof(float);
 }
 
 // How many workgroups of the kernel the device keeps resident at once (0: it cannot run at all).
@@ -538,6 +579,8 @@ hipError_t launch_flow_fill(hipStream_t s, void *buf, size_t bytes) {
 }
 
 hipError_t launch_decode_persistent(hipStream_t s, const PersistentParams &p, uint32_t grid) {
+    const plan::Shape sh{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, grid, p.qkv_units, p.gu_rows};
+    if (!plan::shape_ok(sh)) return hipErrorInvalidValue;          // the index arithmetic of the kernel assumes these
     const size_t smem = persistent_smem_bytes(p);
     if (p.kv_f16) llama_decode_persistent_kernel<true><<<grid, PNT, smem, s>>>(p);
     else llama_decode_persistent_kernel<false><<<grid, PNT, smem, s>>>(p);

@@ -1,0 +1,160 @@
+// Who does what, and where every access lands, in the resident decode kernel (kernels_decode_persistent.hip): the roles
+// of the workgroups in each phase of a layer, the byte offsets of the weights a lane requests, the pieces of a hand-off
+// vector a staging lane fetches, the rows of the hand-off buffers, the per-workgroup slots, counters and trace rows.
+//
+// Everything here is plain integer arithmetic that compiles for the device and for the host: the kernel forms its
+// addresses with these functions and nothing else, and a host program (tests/native/resident_bounds.cpp) walks every
+// (workgroup, wave, lane, layer) of a launch through the same functions and checks each access against the allocation
+// the loader makes for it.
+#pragma once
+#include "quant_tiled.h"
+
+namespace slai {
+
+// A 64-bit value from two 32-bit words.  The words are taken as unsigned on purpose: the lane-broadcast builtins return
+// `int`, and an int with bit 31 set, widened on its way into a 64-bit "or", fills the upper word with ones -- a pointer
+// rebuilt that way is wrong for every address whose lower word is 0x80000000 or above.
+SLAI_HD constexpr uint64_t join_words(uint32_t lo, uint32_t hi) { return ((uint64_t)hi << 32) | (uint64_t)lo; }
+static_assert(join_words(0x80000000u, 0x7fu) == 0x0000007f80000000ull, "the lower word must not be sign-extended");
+static_assert(join_words((uint32_t)(int)0xffffffffu, 0u) == 0x00000000ffffffffull, "an int -1 as lower word stays 32 bits wide");
+
+namespace plan {
+
+constexpr uint32_t WG_THREADS = 1024, WG_WAVES = 16;
+constexpr uint32_t STAGERS64 = 4;          // waves that stage the input of a 64-row-unit phase (the last four)
+constexpr uint32_t MAX_MULT16 = 12;        // waves that multiply in a 16-row-tile phase before the others only stage
+
+struct Shape {
+    uint32_t dim, hidden, n_heads, n_layers, vocab, seq_len;
+    uint32_t grid;            // workgroups of the launch (all resident)
+    uint32_t qkv_units;       // units per head in the q / k / v phase: 6 (two 64-row units per matrix) or 7 (v in three)
+    uint32_t gu_rows;         // rows per unit of the gate / up phase, at most 64
+};
+
+SLAI_HD uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
+SLAI_HD uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
+// The decomposition a launch of `grid` workgroups uses for a model: v in three units per head when the grid has room for
+// seven units and the attention workgroup of every head; gate / up rows spread evenly over the grid.
+SLAI_HD Shape make_shape(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32_t n_layers, uint32_t vocab, uint32_t seq_len, uint32_t grid) {
+    Shape s{dim, hidden, n_heads, n_layers, vocab, seq_len, grid, 6u, 64u};
+    if (8u * n_heads <= grid) s.qkv_units = 7;
+    s.gu_rows = umin(64u, umax(1u, (hidden + grid - 1) / grid));
+    return s;
+}
+
+// ---- supported shapes: what the kernel's index arithmetic assumes -------------------------------------------------------
+SLAI_HD bool shape_ok(const Shape &s) {
+    if (s.n_heads == 0 || s.n_heads % 8 || s.dim != s.n_heads * 128) return false;            // heads of 128, eight dies
+    if (s.dim % 1024 || s.dim > 4096) return false;                                            // four staging pieces per lane at most
+    if (s.hidden % 256 || s.hidden / 256 > 64) return false;                                   // sixteen multiplying waves x four super-blocks
+    if (s.grid % 8 || s.grid > 1024) return false;
+    if ((s.qkv_units != 6 && s.qkv_units != 7) || (s.qkv_units + 1) * s.n_heads > s.grid) return false;
+    if (s.dim / 16 > s.grid) return false;                                                     // one 16-row tile of the projections each
+    if (s.gu_rows == 0 || s.gu_rows > 64 || (s.hidden + s.gu_rows - 1) / s.gu_rows > s.grid) return false;
+    if (s.seq_len == 0 || s.seq_len > 1024 || s.n_layers == 0 || s.vocab == 0) return false;
+    return true;
+}
+
+// ---- hand-off buffers: one allocation of flow_floats() floats ------------------------------------------------------------
+// xa [(n_layers + 1) x dim]: the input of layer l (row 0 unused: layer 0 reads the embedding row); row n_layers feeds
+// the output matrix.  xb, xm [n_layers x dim]: attention output, residual after the attention.  hb [n_layers x hidden].
+SLAI_HD uint64_t flow_floats(const Shape &s) { return (uint64_t)(3 * s.n_layers + 1) * s.dim + (uint64_t)s.n_layers * s.hidden; }
+SLAI_HD uint64_t flow_xa(const Shape &s, uint32_t l) { return (uint64_t)l * s.dim; }
+SLAI_HD uint64_t flow_xb(const Shape &s, uint32_t l) { return (uint64_t)(s.n_layers + 1) * s.dim + (uint64_t)l * s.dim; }
+SLAI_HD uint64_t flow_xm(const Shape &s, uint32_t l) { return (uint64_t)(2 * s.n_layers + 1) * s.dim + (uint64_t)l * s.dim; }
+SLAI_HD uint64_t flow_hb(const Shape &s, uint32_t l) { return (uint64_t)(3 * s.n_layers + 1) * s.dim + (uint64_t)l * s.hidden; }
+
+// ---- per-workgroup slot (the staged input of a 64-row-unit phase, read back with scalar loads) ---------------------------
+SLAI_HD uint32_t slot_stride(const Shape &s) { return s.dim + s.dim / 16 + 16; }             // floats
+SLAI_HD uint64_t slot_floats(const Shape &s) { return (uint64_t)s.grid * slot_stride(s); }
+SLAI_HD uint64_t slot_of(const Shape &s, uint32_t b) { return (uint64_t)b * slot_stride(s); }
+// a multiplying wave reads 256 activations and 16 sums of its super-block from the slot
+SLAI_HD uint32_t slot_x(uint32_t cb) { return cb * 256; }
+SLAI_HD uint32_t slot_sums(const Shape &s, uint32_t cb) { return s.dim + cb * 16; }
+
+// ---- dynamic LDS of a workgroup, in floats: partial[2][16][64] | red[2][4] | xs[max(dim, hidden)] -----------------------
+SLAI_HD uint32_t lds_partial() { return 0; }
+SLAI_HD uint32_t lds_red() { return 2 * WG_WAVES * 64; }
+SLAI_HD uint32_t lds_xs() { return lds_red() + 8; }
+SLAI_HD uint32_t lds_floats(const Shape &s) { return lds_xs() + umax(s.dim, s.hidden); }
+
+// ---- counters of the q / k / v -> attention hand-off: one 128-byte line per head, then the flag of a wait that gave up ---
+SLAI_HD uint32_t counter_word(uint32_t head) { return head * 32; }
+
+// ---- time stamps: per workgroup 16 per layer (four per phase) and 8 for the output matrix -------------------------------
+SLAI_HD uint32_t trace_stride(const Shape &s) { return 16 * s.n_layers + 8; }
+SLAI_HD uint64_t trace_row(const Shape &s, uint32_t b) { return (uint64_t)b * trace_stride(s); }
+
+// ---- roles ----------------------------------------------------------------------------------------------------------------
+// A unit of a 64-row-unit phase: rows [row0, row0 + nrows) of matrix `seg`, nrows <= 64, lane i of every wave owns row
+// row0 + i (lanes past nrows repeat the last row and their results are dropped); wave w owns super-block w.
+struct RowUnit { uint32_t seg, row0, nrows; };
+
+// q / k / v (segments 0: v, 1: k, 2: q): workgroup i < qkv_units * n_heads takes unit (i / 8) % qkv_units of head
+// (i % 8) + 8 * (i / (8 * qkv_units)), so that all units of a head, and the head's attention workgroup
+// qkv_workgroups + head, run on die i % 8 (their hand-off goes through that die's L2).
+SLAI_HD uint32_t qkv_workgroups(const Shape &s) { return s.qkv_units * s.n_heads; }
+SLAI_HD uint32_t qkv_head(const Shape &s, uint32_t b) { return (b & 7u) + 8u * ((b >> 3) / s.qkv_units); }
+SLAI_HD RowUnit qkv_unit(const Shape &s, uint32_t b) {
+    const uint32_t t = (b >> 3) % s.qkv_units, head = qkv_head(s, b);
+    const uint32_t nv = s.qkv_units - 4;                      // units of v: 2 or 3; k and q two each
+    uint32_t seg, part, parts;
+    if (t < nv) { seg = 0; part = t; parts = nv; }
+    else if (t < nv + 2) { seg = 1; part = t - nv; parts = 2; }
+    else { seg = 2; part = t - nv - 2; parts = 2; }
+    const uint32_t lo = 128u * part / parts, hi = 128u * (part + 1) / parts;
+    return RowUnit{seg, head * 128u + lo, hi - lo};
+}
+SLAI_HD bool is_attention_workgroup(const Shape &s, uint32_t b) { return b >= qkv_workgroups(s) && b < qkv_workgroups(s) + s.n_heads; }
+SLAI_HD uint32_t attention_head(const Shape &s, uint32_t b) { return b - qkv_workgroups(s); }
+
+// gate / up: workgroup b < gu_units takes rows [b * gu_rows, ...) of both matrices
+SLAI_HD uint32_t gu_units(const Shape &s) { return (s.hidden + s.gu_rows - 1) / s.gu_rows; }
+SLAI_HD RowUnit gu_unit(const Shape &s, uint32_t b) { return RowUnit{0u, b * s.gu_rows, umin(s.gu_rows, s.hidden - b * s.gu_rows)}; }
+
+// the two projections into the residual: workgroup b < dim / 16 takes rows 16 b .. 16 b + 15 and keeps their residual
+SLAI_HD uint32_t proj_tiles(const Shape &s) { return s.dim / 16; }
+
+// output matrix: 64-row tiles b, b + grid, ...
+SLAI_HD uint32_t out_tiles(const Shape &s) { return (s.vocab + 63) / 64; }
+
+// ---- weights: byte offsets inside one matrix, all below 2^32 (checked at load time) --------------------------------------
+// 64-row tiles (quant_tiled.h, ROWS = 64, KQ = 1): the 16 bytes of piece P of (row, super-block cb) sit at
+// tile64_piece0 + P * 1024, the 2-byte tail (Q6_K) at tile64_tail.
+SLAI_HD uint32_t tile64_piece0(uint32_t row, uint32_t cb, uint32_t ncb, uint32_t unit_bytes) { return ((row >> 6) * ncb + cb) * unit_bytes + (row & 63u) * 16u; }
+SLAI_HD uint32_t tile64_tail(uint32_t row, uint32_t cb, uint32_t ncb, uint32_t unit_bytes, uint32_t pieces) {
+    return ((row >> 6) * ncb + cb) * unit_bytes + pieces * 1024u + (row & 63u) * 2u;
+}
+// 16-row tiles (ROWS = 16, KQ = 4): lane = 16 * kq + row; column group g of tile t
+SLAI_HD uint32_t tile16_piece0(uint32_t tile, uint32_t g, uint32_t ngroups, uint32_t unit_bytes, uint32_t lane) { return (tile * ngroups + g) * unit_bytes + lane * 16u; }
+SLAI_HD uint32_t tile16_tail(uint32_t tile, uint32_t g, uint32_t ngroups, uint32_t unit_bytes, uint32_t pieces, uint32_t lane) {
+    return (tile * ngroups + g) * unit_bytes + pieces * 1024u + lane * 2u;
+}
+SLAI_HD uint32_t unit_bytes_of(int type) { return tiled_pieces(type) * 1024u + tiled_tail(type); }
+
+// ---- staging the input of a 64-row-unit phase: the last four waves, lane l = 0 .. 255 of them, piece l + 256 k, k < 4 -------
+SLAI_HD uint32_t stage64_lane(uint32_t tid) { return tid - (WG_WAVES - STAGERS64) * 64u; }
+SLAI_HD uint32_t stage64_piece(uint32_t l, uint32_t k) { return l + 256u * k; }                // index of a 16-byte piece (4 floats)
+SLAI_HD bool stage64_live(uint32_t l, uint32_t k, uint32_t n) { return stage64_piece(l, k) < n / 4; }
+// the piece a stager wave polls before it fetches its share (its own first piece, or piece 0 when it has none)
+SLAI_HD uint32_t stage64_probe(uint32_t wave, uint32_t n) {
+    const uint32_t first = 64u * (wave - (WG_WAVES - STAGERS64));
+    return first < n / 4 ? first : 0u;
+}
+
+// ---- staging the input of a 16-row-tile phase into LDS: waves first_stager .. 15 --------------------------------------------
+SLAI_HD uint32_t stage16_first(uint32_t ngroups) { return umin(ngroups, MAX_MULT16); }
+SLAI_HD uint32_t stage16_lanes(uint32_t ngroups) { return (WG_WAVES - stage16_first(ngroups)) * 64u; }
+// lane l of the nl staging lanes takes pieces l, l + nl, ...; `per_trip` (4 or 12) of them per round trip
+SLAI_HD uint32_t stage16_per_trip(uint32_t chunks, uint32_t nl) { return chunks > 4 * nl ? 12u : 4u; }
+SLAI_HD uint32_t stage16_trips(uint32_t chunks, uint32_t nl) { const uint32_t pt = stage16_per_trip(chunks, nl); return (chunks + pt * nl - 1) / (pt * nl); }
+SLAI_HD uint32_t stage16_first_piece(uint32_t l, uint32_t nl, uint32_t trip, uint32_t per_trip) { return per_trip * trip * nl + l; }
+SLAI_HD uint32_t stage16_nlive(uint32_t i0, uint32_t nl, uint32_t chunks, uint32_t per_trip) { return i0 < chunks ? umin(per_trip, (chunks - i0 + nl - 1) / nl) : 0u; }
+SLAI_HD uint32_t stage16_probe(uint32_t wave, uint32_t ngroups, uint32_t chunks) {
+    const uint32_t first = (wave - stage16_first(ngroups)) * 64u;
+    return first < chunks ? first : 0u;
+}
+
+}  // namespace plan
+}  // namespace slai

@@ -91,9 +91,6 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
     ctx->fuse_qkv_attention = env_int("SLAI_FUSE_QKV_ATTN", 1) != 0;
     ctx->persistent = env_int("SLAI_PERSISTENT", 0) != 0;
-    if (ctx->persistent)
-        fprintf(stderr, "slai: SLAI_PERSISTENT=1 -- the one-launch-per-token decode kernel has not run on a device since its pointer "
-                        "handling was corrected; earlier builds of it ended in GPU memory faults on models beyond a few MB\n");
     *out = ctx;
     return SLAI_OK;
 }
@@ -467,11 +464,11 @@ int handoff_reserve(slai_ctx *ctx, uint32_t n_heads) {
     SLAI_HIP_TRY(ctx, hipMalloc((void **)&ctx->handoff_counters, bytes));
     // The hand-off relies on workgroup i running on XCD i mod 8 (workgroups with equal i mod 8 then share an L2):
     // look before relying on it, and keep separate launches on a device that places workgroups differently.
-    uint32_t where[192];
-    SLAI_HIP_TRY(ctx, launch_xcd_of_workgroup(ctx->stream, ctx->handoff_counters, 192));
+    uint32_t where[256];
+    SLAI_HIP_TRY(ctx, launch_xcd_of_workgroup(ctx->stream, ctx->handoff_counters, 256));
     SLAI_HIP_TRY(ctx, hipMemcpyAsync(where, ctx->handoff_counters, sizeof where, hipMemcpyDeviceToHost, ctx->stream));
     SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    for (uint32_t i = 8; i < 192; ++i)
+    for (uint32_t i = 8; i < 256; ++i)
         if (where[i] != where[i % 8]) ctx->fuse_qkv_attention = false;
     SLAI_HIP_TRY(ctx, hipMemsetAsync(ctx->handoff_counters, 0, bytes, ctx->stream));
     SLAI_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));

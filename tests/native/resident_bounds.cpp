@@ -1,0 +1,272 @@
+// Host walk of every address the resident decode kernel (slai_amd/csrc/kernels_decode_persistent.hip) forms, through
+// the same functions the kernel calls (slai_amd/csrc/resident_plan.h), against the sizes of the allocations the loader
+// makes (`slai_llama2::persistent_setup`, slai_qmat_create_layout).  Compiled by tests/test_resident_plan.py with g++.
+//
+// rb_audit walks, for every workgroup, wave and lane of a launch and every layer:
+//   * the weight pieces and tails a lane requests in each phase, against the matrix's bytes;
+//   * the pieces of a hand-off vector a staging lane fetches (and the one it polls, and its spare piece), against the
+//     vector, and the words it writes into the slot / into LDS, against the slot / the LDS block; what the multiplying
+//     waves read back from there;
+//   * the rows a workgroup writes into the hand-off vectors, q / k / v, the logits; counters, trace rows, the layer table;
+//   * coverage: every output row of every matrix is produced exactly once per layer and every piece of an input vector is
+//     staged exactly once per workgroup and phase;
+//   * the 64-bit addresses: each buffer gets a fake base whose lower word lies below or above 0x80000000; the address is
+//     rebuilt from its two words the way the kernel does and every access must fall inside [base, base + bytes).
+// With `sign_extending_join` the lower word is widened as a signed int (the defect an earlier form of the kernel had):
+// the audit must then report violations for bases at or above 0x80000000 in the lower word.
+#include "quant_formats.h"
+#include "quant_tiled.h"
+#include "resident_plan.h"
+
+#include <cstdio>
+#include <string>
+#include <vector>
+
+using namespace slai;
+
+namespace {
+
+struct Region { const char *name; uint64_t base, bytes; };
+
+struct Audit {
+    bool sign_ext = false;
+    uint64_t violations = 0, checks = 0;
+    std::string first;
+    uint64_t rebuilt(uint64_t base) const {
+        const uint32_t lo = (uint32_t)base, hi = (uint32_t)(base >> 32);
+        if (sign_ext) return ((uint64_t)hi << 32) | (uint64_t)(int64_t)(int32_t)lo;     // what `(uint64_t)readfirstlane(lo)` did
+        return join_words(lo, hi);
+    }
+    // an access of `size` bytes at byte offset `off` of region r
+    void touch(const Region &r, uint64_t off, uint64_t size, const char *what, uint32_t b, uint32_t wave, uint32_t lane, uint32_t layer) {
+        ++checks;
+        const uint64_t addr = rebuilt(r.base) + off;
+        if (off + size > r.bytes || addr < r.base || addr + size > r.base + r.bytes) {
+            if (!violations++) {
+                char msg[320];
+                snprintf(msg, sizeof msg, "%s: %s offset %llu + %llu beyond %llu bytes (address %#llx, base %#llx) at workgroup %u wave %u lane %u layer %u",
+                         r.name, what, (unsigned long long)off, (unsigned long long)size, (unsigned long long)r.bytes, (unsigned long long)addr,
+                         (unsigned long long)r.base, b, wave, lane, layer);
+                first = msg;
+            }
+        }
+    }
+    void fail(const std::string &msg) { if (!violations++) first = msg; }
+};
+
+size_t matrix_bytes(int type, uint32_t nrows, uint32_t ncols, uint32_t rows_log2) { return tiled_bytes(tiled_geom(type, nrows, ncols, rows_log2)); }
+
+// the weight requests of one lane for a unit of a 64-row-tile matrix
+void walk_tile64(Audit &a, const Region &w, int type, const plan::RowUnit &u, uint32_t ncb, uint32_t b, uint32_t layer, std::vector<uint32_t> *row_count) {
+    const uint32_t ub = plan::unit_bytes_of(type), pt = tiled_pieces(type);
+    for (uint32_t wave = 0; wave < plan::WG_WAVES; ++wave) {
+        if (wave >= ncb) continue;
+        for (uint32_t lane = 0; lane < 64; ++lane) {
+            const uint32_t row = u.row0 + plan::umin(lane, u.nrows - 1);
+            const uint32_t voff = plan::tile64_piece0(row, wave, ncb, ub);
+            for (uint32_t p = 0; p < pt; ++p) a.touch(w, (uint64_t)voff + p * 1024u, 16, "weight piece", b, wave, lane, layer);
+            if (tiled_tail(type)) a.touch(w, plan::tile64_tail(row, wave, ncb, ub, pt), 2, "weight tail", b, wave, lane, layer);
+        }
+    }
+    if (row_count)
+        for (uint32_t i = 0; i < u.nrows; ++i) {
+            if (u.row0 + i >= row_count->size()) { a.fail("a unit names a row past its matrix"); return; }
+            ++(*row_count)[u.row0 + i];
+        }
+}
+
+// staging of an n-vector into the workgroup's slot by the last four waves, and what the multiplying waves read back
+void walk_stage64(Audit &a, const plan::Shape &s, const Region &x, const Region &norm, const Region &slots, uint32_t n, uint32_t ncb, uint32_t b, uint32_t layer) {
+    std::vector<uint32_t> seen(n / 4, 0);
+    const uint64_t slot0 = plan::slot_of(s, b) * 4;
+    for (uint32_t wave = plan::WG_WAVES - plan::STAGERS64; wave < plan::WG_WAVES; ++wave) {
+        a.touch(x, (uint64_t)plan::stage64_probe(wave, n) * 16, 16, "probe", b, wave, 0, layer);
+        for (uint32_t lane = 0; lane < 64; ++lane) {
+            const uint32_t tid = wave * 64 + lane, l = plan::stage64_lane(tid);
+            a.touch(x, (uint64_t)l * 16, 16, "spare piece", b, wave, lane, layer);
+            for (uint32_t k = 0; k < 4; ++k) {
+                const uint32_t idx = plan::stage64_piece(l, k);
+                const bool live = plan::stage64_live(l, k, n);
+                a.touch(norm, (uint64_t)(live ? idx : l) * 16, 16, "norm weights", b, wave, lane, layer);
+                if (!live) continue;
+                a.touch(x, (uint64_t)idx * 16, 16, "input piece", b, wave, lane, layer);
+                a.touch(slots, slot0 + (uint64_t)idx * 16, 16, "slot values", b, wave, lane, layer);
+                if ((lane & 3) == 0) a.touch(slots, slot0 + ((uint64_t)n + (idx >> 2)) * 4, 4, "slot sums", b, wave, lane, layer);
+                if (idx < seen.size()) ++seen[idx];
+            }
+        }
+    }
+    for (uint32_t i = 0; i < seen.size(); ++i)
+        if (seen[i] != 1) { a.fail("64-row-unit staging: a piece of the input is staged " + std::to_string(seen[i]) + " times"); break; }
+    if ((uint64_t)n + n / 16 > plan::slot_stride(s)) a.fail("the slot is smaller than the staged input");
+    for (uint32_t wave = 0; wave < plan::WG_WAVES && wave < ncb; ++wave) {
+        a.touch(slots, slot0 + (uint64_t)plan::slot_x(wave) * 4, 256 * 4, "slot read (activations)", b, wave, 0, layer);
+        a.touch(slots, slot0 + ((uint64_t)n + wave * 16) * 4, 16 * 4, "slot read (sums)", b, wave, 0, layer);
+        if (plan::slot_x(wave) + 256 > n) a.fail("a multiplying wave reads activations past the input");
+    }
+}
+
+// a 16-row tile phase: weights of the multiplying waves, staging of the n-vector into LDS by the others
+void walk_tile16(Audit &a, const plan::Shape &s, const Region &w, int type, uint32_t tile, uint32_t ncb, uint32_t ngroups, const Region &x, uint32_t n, uint32_t b,
+                 uint32_t layer) {
+    const uint32_t ub = plan::unit_bytes_of(type), pt = tiled_pieces(type);
+    const Region lds{"LDS xs", 0x10000u, (uint64_t)(plan::lds_floats(s) - plan::lds_xs()) * 4};
+    for (uint32_t wave = 0; wave < plan::WG_WAVES && wave < ngroups; ++wave)
+        for (uint32_t lane = 0; lane < 64; ++lane) {
+            const uint32_t voff = plan::tile16_piece0(tile, wave, ngroups, ub, lane);
+            for (uint32_t p = 0; p < pt; ++p) a.touch(w, (uint64_t)voff + p * 1024u, 16, "weight piece (16-row tile)", b, wave, lane, layer);
+            if (tiled_tail(type)) a.touch(w, plan::tile16_tail(tile, wave, ngroups, ub, pt, lane), 2, "weight tail (16-row tile)", b, wave, lane, layer);
+            const uint32_t cb = wave * 4 + (lane >> 4);
+            if (cb < ncb)
+                for (uint32_t i = 0; i < 16; ++i) a.touch(lds, ((uint64_t)cb * 256 + 16 * i + (lane & 15)) * 4, 4, "LDS read", b, wave, lane, layer);
+        }
+    if (ngroups > plan::WG_WAVES) { a.fail("more column groups than waves"); return; }
+    const uint32_t first = plan::stage16_first(ngroups), nl = plan::stage16_lanes(ngroups), chunks = n / 4;
+    if (nl == 0) { a.fail("a 16-row-tile phase without staging waves"); return; }
+    std::vector<uint32_t> seen(chunks, 0);
+    const uint32_t per = plan::stage16_per_trip(chunks, nl), trips = plan::stage16_trips(chunks, nl);
+    for (uint32_t wave = first; wave < plan::WG_WAVES; ++wave) {
+        a.touch(x, (uint64_t)plan::stage16_probe(wave, ngroups, chunks) * 16, 16, "probe", b, wave, 0, layer);
+        for (uint32_t lane = 0; lane < 64; ++lane) {
+            const uint32_t l = wave * 64 + lane - first * 64;
+            a.touch(x, (uint64_t)lane * 16, 16, "spare piece", b, wave, lane, layer);
+            for (uint32_t j = 0; j < trips; ++j) {
+                const uint32_t i0 = plan::stage16_first_piece(l, nl, j, per), nlive = plan::stage16_nlive(i0, nl, chunks, per);
+                for (uint32_t k = 0; k < nlive; ++k) {
+                    const uint32_t piece = i0 + k * nl;
+                    a.touch(x, (uint64_t)piece * 16, 16, "input piece", b, wave, lane, layer);
+                    a.touch(lds, (uint64_t)piece * 16, 16, "LDS write", b, wave, lane, layer);
+                    if (piece < chunks) ++seen[piece];
+                }
+            }
+        }
+    }
+    for (uint32_t i = 0; i < chunks; ++i)
+        if (seen[i] != 1) { a.fail("16-row-tile staging: a piece of the input is staged " + std::to_string(seen[i]) + " times"); break; }
+}
+
+}  // namespace
+
+extern "C" {
+
+// types: block formats of q, k, v, attention output, gate/up, down, output matrix.  handoff_heads: lines of the counter
+// block (the runtime reserves max(n_heads, 256)).  high_bases: fake addresses with bit 31 of the lower word set.
+// Returns the number of violations; `msg` receives the first one, `checked` the number of accesses looked at.
+unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32_t n_layers, uint32_t vocab, uint32_t seq_len, uint32_t grid,
+                            int tq, int tk, int tv, int to, int tg, int td, int tout, uint32_t handoff_heads, int kv_bytes, int high_bases,
+                            int sign_extending_join, char *msg, size_t msg_len, unsigned long long *checked) {
+    Audit a;
+    a.sign_ext = sign_extending_join != 0;
+    const plan::Shape s = plan::make_shape(dim, hidden, n_heads, n_layers, vocab, seq_len, grid);
+    if (!plan::shape_ok(s)) a.fail("plan::shape_ok refuses the shape");
+    else {
+        // fake placement: 4 GiB apart, lower word 0x10000000 or 0x90000000 (+ a region-specific stagger)
+        uint64_t next = high_bases ? 0x0000007f90000000ull : 0x0000007f10000000ull;
+        const auto place = [&](const char *name, uint64_t bytes) { Region r{name, next, bytes}; next += 0x100000000ull + 0x01000000ull; return r; };
+        const uint32_t ncb = dim / 256, ncb_h = hidden / 256, ng_o = ncb / 4, ng_d = (ncb_h + 3) / 4;
+        const Region wq = place("wq", matrix_bytes(tq, dim, dim, 6)), wk = place("wk", matrix_bytes(tk, dim, dim, 6)), wv = place("wv", matrix_bytes(tv, dim, dim, 6));
+        const Region wo = place("wo", matrix_bytes(to, dim, dim, 4)), wg = place("wgate", matrix_bytes(tg, hidden, dim, 6)), wu = place("wup", matrix_bytes(tg, hidden, dim, 6));
+        const Region wd = place("wdown", matrix_bytes(td, dim, hidden, 4)), wout = place("wout", matrix_bytes(tout, vocab, dim, 6));
+        const Region norm = place("norm vector", (uint64_t)dim * 4), xemb = place("embedding row", (uint64_t)dim * 4);
+        const Region flow = place("hand-off buffers", plan::flow_floats(s) * 4), slots = place("slots", plan::slot_floats(s) * 4);
+        const Region qv = place("q / k / v vector", (uint64_t)dim * 4), logits = place("logits", (uint64_t)vocab * 4);
+        const Region counters = place("counters", ((uint64_t)handoff_heads * 32 + 32) * 4);
+        const Region trace = place("trace", (uint64_t)grid * plan::trace_stride(s) * 8);
+        const Region layers = place("layer table", (uint64_t)n_layers * 14 * 16);
+        const Region cache = place("cache", (uint64_t)seq_len * dim * kv_bytes);
+        if ((wd.bytes | wout.bytes | wg.bytes) > 0xffffffffull) a.fail("a matrix beyond 4 GiB");
+        // the four tile16 checks below assume what the loader checks: 16-row tiles with ceil(ncb / 4) groups
+        if (tiled_geom(to, dim, dim, 4).ngroups != ng_o || tiled_geom(td, dim, hidden, 4).ngroups != ng_d) a.fail("group count of a projection differs from the kernel's");
+        for (uint32_t l = 0; l < n_layers && a.violations < 8; ++l) {
+            std::vector<uint32_t> rows_q(dim, 0), rows_k(dim, 0), rows_v(dim, 0), rows_h(hidden, 0), rows_o(dim, 0), rows_d(dim, 0);
+            std::vector<uint32_t> heads_attended(n_heads, 0), units_of_head(n_heads, 0);
+            // a hand-off vector of this layer as a region of its own size, placed inside the allocation
+            const auto vec = [&](const char *name, uint64_t first_float, uint64_t n) {
+                a.touch(flow, first_float * 4, n * 4, "hand-off row", 0, 0, 0, l);
+                return Region{name, flow.base + first_float * 4, n * 4};
+            };
+            const Region xa = vec("xa", plan::flow_xa(s, l), dim), xb = vec("xb", plan::flow_xb(s, l), dim), xm = vec("xm", plan::flow_xm(s, l), dim);
+            const Region hb = vec("hb", plan::flow_hb(s, l), hidden), xnext = vec("xa (next)", plan::flow_xa(s, l + 1), dim);
+            for (uint32_t b = 0; b < grid; ++b) {
+                for (uint32_t tid = 0; tid < 14 * 4 && l + 1 < n_layers; ++tid) a.touch(layers, ((uint64_t)(l + 1) * 14 * 4 + tid) * 4, 4, "layer table word", b, 0, tid, l);
+                for (uint32_t ph = 0; ph < 4; ++ph)
+                    for (uint32_t k = 0; k < 4; ++k) a.touch(trace, (plan::trace_row(s, b) + 16 * l + 4 * ph + k) * 8, 8, "time stamp", b, 0, 0, l);
+                if (b < plan::qkv_workgroups(s)) {
+                    const plan::RowUnit u = plan::qkv_unit(s, b);
+                    const uint32_t h = plan::qkv_head(s, b);
+                    if (u.nrows == 0 || u.nrows > 64 || h >= n_heads || b % 8 != h % 8) { a.fail("q / k / v role"); continue; }
+                    if (u.row0 / 128 != h || (u.row0 + u.nrows - 1) / 128 != h) a.fail("a q / k / v unit leaves its head");
+                    ++units_of_head[h];
+                    walk_tile64(a, u.seg == 0 ? wv : (u.seg == 1 ? wk : wq), u.seg == 0 ? tv : (u.seg == 1 ? tk : tq), u, ncb, b, l, u.seg == 0 ? &rows_v : (u.seg == 1 ? &rows_k : &rows_q));
+                    walk_stage64(a, s, l == 0 ? xemb : xa, norm, slots, dim, ncb, b, l);
+                    for (uint32_t t = 0; t < u.nrows; ++t) a.touch(qv, (uint64_t)(u.row0 + t) * 4, 4, "q / k / v store", b, 0, t, l);
+                    a.touch(counters, (uint64_t)plan::counter_word(h) * 4, 4, "counter", b, 0, 0, l);
+                } else if (plan::is_attention_workgroup(s, b)) {
+                    const uint32_t h = plan::attention_head(s, b);
+                    if (h >= n_heads || b % 8 != h % 8) { a.fail("attention role"); continue; }
+                    ++heads_attended[h];
+                    a.touch(counters, (uint64_t)plan::counter_word(h) * 4, 4, "counter", b, 0, 0, l);
+                    for (uint32_t t = 0; t < 128; ++t) {
+                        a.touch(qv, ((uint64_t)h * 128 + t) * 4, 4, "q / k / v load", b, 0, t, l);
+                        a.touch(xb, ((uint64_t)h * 128 + t) * 4, 4, "attention output", b, 0, t, l);
+                        a.touch(cache, ((uint64_t)(seq_len - 1) * dim + h * 128 + t) * kv_bytes, kv_bytes, "cache row", b, 0, t, l);
+                    }
+                }
+                a.touch(counters, (uint64_t)handoff_heads * 32 * 4, 4, "abort flag", b, 0, 0, l);
+                if (b < plan::proj_tiles(s)) {
+                    if (l == 0) for (uint32_t t = 0; t < 16; ++t) a.touch(xemb, ((uint64_t)16 * b + t) * 4, 4, "residual load", b, 0, t, l);
+                    walk_tile16(a, s, wo, to, b, ncb, ng_o, xb, dim, b, l);
+                    walk_tile16(a, s, wd, td, b, ncb_h, ng_d, hb, hidden, b, l);
+                    for (uint32_t t = 0; t < 16; ++t) {
+                        a.touch(xm, ((uint64_t)16 * b + t) * 4, 4, "xm store", b, 0, t, l);
+                        a.touch(xnext, ((uint64_t)16 * b + t) * 4, 4, "xa store", b, 0, t, l);
+                        ++rows_o[16 * b + t]; ++rows_d[16 * b + t];
+                    }
+                }
+                if (b < plan::gu_units(s)) {
+                    const plan::RowUnit u = plan::gu_unit(s, b);
+                    if (u.nrows == 0 || u.nrows > 64) { a.fail("gate / up role"); continue; }
+                    walk_tile64(a, wg, tg, u, ncb, b, l, &rows_h);
+                    walk_tile64(a, wu, tg, u, ncb, b, l, nullptr);
+                    walk_stage64(a, s, xm, norm, slots, dim, ncb, b, l);
+                    for (uint32_t t = 0; t < u.nrows; ++t) a.touch(hb, (uint64_t)(u.row0 + t) * 4, 4, "hb store", b, 0, t, l);
+                }
+            }
+            const auto once = [&](const std::vector<uint32_t> &v, const char *what) {
+                for (size_t i = 0; i < v.size(); ++i)
+                    if (v[i] != 1) { a.fail(std::string(what) + ": row " + std::to_string(i) + " is produced " + std::to_string(v[i]) + " times in layer " + std::to_string(l)); return; }
+            };
+            once(rows_q, "q"); once(rows_k, "k"); once(rows_v, "v"); once(rows_h, "gate / up"); once(rows_o, "attention output projection"); once(rows_d, "down projection");
+            once(heads_attended, "attention");
+            for (uint32_t h = 0; h < n_heads; ++h)
+                if (units_of_head[h] != s.qkv_units) a.fail("a head's counter would not reach its target");
+        }
+        // the output matrix
+        std::vector<uint32_t> rows_l(vocab, 0);
+        const Region xlast{"xa (last)", flow.base + plan::flow_xa(s, n_layers) * 4, (uint64_t)dim * 4};
+        for (uint32_t b = 0; b < grid && a.violations < 8; ++b) {
+            bool first = true;
+            for (uint32_t tile = b; tile < plan::out_tiles(s); tile += grid) {
+                const plan::RowUnit u{0u, tile * 64u, plan::umin(64u, vocab - tile * 64u)};
+                walk_tile64(a, wout, tout, u, ncb, b, n_layers, &rows_l);
+                if (first) walk_stage64(a, s, xlast, norm, slots, dim, ncb, b, n_layers);
+                first = false;
+                for (uint32_t t = 0; t < u.nrows; ++t) a.touch(logits, (uint64_t)(u.row0 + t) * 4, 4, "logits store", b, 0, t, n_layers);
+            }
+            for (uint32_t k = 0; k < 5; ++k) a.touch(trace, (plan::trace_row(s, b) + 16 * n_layers + k) * 8, 8, "time stamp (output)", b, 0, 0, n_layers);
+        }
+        for (size_t i = 0; i < rows_l.size(); ++i)
+            if (rows_l[i] != 1) { a.fail("logits: row " + std::to_string(i) + " is produced " + std::to_string(rows_l[i]) + " times"); break; }
+    }
+    if (msg && msg_len) snprintf(msg, msg_len, "%s", a.first.c_str());
+    if (checked) *checked = a.checks;
+    return a.violations;
+}
+
+// the decomposition plan::make_shape picks (for the test's report)
+void rb_shape(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32_t grid, uint32_t *qkv_units, uint32_t *gu_rows, uint32_t *gu_units) {
+    const plan::Shape s = plan::make_shape(dim, hidden, n_heads, 1, 64, 64, grid);
+    *qkv_units = s.qkv_units; *gu_rows = s.gu_rows; *gu_units = plan::gu_units(s);
+}
+
+}  // extern "C"

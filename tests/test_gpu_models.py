@@ -22,7 +22,7 @@ def oracle_llama(data, gpu_semantics=1, neox=0, kv_f16=0, name=b"llama"):
 
 
 def check_llama(backend, data, prompt, n_steps, kv_f16=False, model_type=_ffi.MODEL_LLAMA, neox=0, name=b"llama",
-                check_logit_steps=8, tol=LOGIT_TOL):
+                check_logit_steps=8, tol=LOGIT_TOL, decode_form=None):
     from slai_amd.runtime import Gguf, Llama2
     g, om = oracle_llama(data, 1, neox, int(kv_f16), name)
     L = g.L
@@ -37,6 +37,8 @@ def check_llama(backend, data, prompt, n_steps, kv_f16=False, model_type=_ffi.MO
     # step-by-step logits, reference op order (fused=0) and fused kernels (fused=1), fed the oracle's tokens
     for fused in (False, True):
         m = Llama2(backend, gg, model_type, kv)
+        if decode_form is not None:
+            assert m.decode_form() == decode_form      # the form under test is the one the model took
         tok = int(prompt[0])
         for pos in range(min(check_logit_steps, n_steps)):
             logits = m.forward_logits(pos, tok, fused=fused)
