@@ -119,109 +119,68 @@ struct Flow {
     bool dead;                // wave-uniform: this wave no longer waits
 };
 
-// One round of a failed wait: sleep a little, look at the clock and at the flag.  `deadline` is 0 until the first failure.
-__device__ __forceinline__ void flow_backoff(Flow &f, uint64_t &deadline) {
-    __builtin_amdgcn_s_sleep(8);
+// One round of a failed wait.  A round is a round trip to memory (about a microsecond), so the clock is looked at every
+// 16th and the flag of the launch every 64th round only: neither may add a dependent memory access to every poll.
+__device__ __forceinline__ void flow_backoff(Flow &f, uint64_t &deadline, uint32_t &rounds) {
+    ++rounds;
+    if ((rounds & 15u) != 0) return;
     const uint64_t now = wall_clock64();
     if (deadline == 0) deadline = now + FLOW_WAIT_TICKS;
     if (now > deadline) {
         f.dead = true;
         if ((phase_tid() & 63) == 0) __hip_atomic_store(f.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else if (__hip_atomic_load(f.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+    } else if ((rounds & 63u) == 0 && __hip_atomic_load(f.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
         f.dead = true;
     }
 }
 
-// Waits until piece `piece` (16 bytes; one address for the whole wave: one request per round) of the hand-off vector is
-// no longer empty.  A wave that arrives long before its input is produced polls this one piece only; the pieces it
-// actually needs are fetched afterwards, when most of them are there.
-__device__ __forceinline__ void flow_probe(Rsrc x, uint32_t piece, Flow &f) {
+// The 16 bytes of piece `piece` of a hand-off vector for every lane of the wave, once no word of any lane's piece is
+// empty: one request per lane and round, repeated by the whole wave (after a time-out the values are whatever was there).
+__device__ __forceinline__ u32x4 flow_take(Rsrc x, uint32_t piece, Flow &f) {
     uint64_t deadline = 0;
-    while (!f.dead) {
+    uint32_t rounds = 0;
+    for (;;) {
         const u32x4 v = buf_load16<AUX_FLOW>(x, piece * 16u);
-        if (!__any(flow_empty(v))) break;
-        flow_backoff(f, deadline);
+        if (!__any(flow_empty(v)) || f.dead) return v;
+        flow_backoff(f, deadline, rounds);
     }
 }
-
-// N (4 or 12) pieces of 16 bytes per lane, each once none of its words is empty: piece k of a lane is piece number
-// first + k * step of the vector and is wanted when k < nlive.  One round trip for all of them, repeated by the whole
-// wave while any is incomplete (after a time-out the values are whatever was there).  A lane asks for the pieces it does
-// not want at `spare` (a piece of the vector that exists for every lane) and ignores what comes back, so that the
-// requests need no execution mask.
-template <int N>
-__device__ __forceinline__ void flow_acquire(Rsrc x, uint32_t first, uint32_t step, uint32_t nlive, uint32_t spare, u32x4 (&v)[N], Flow &f) {
-    static_assert(N == 4 || N == 12, "four or twelve pieces");
+// Sixteen floats per lane, 16 apart from float `first` on (the register layout of DevX), under the same rule.
+__device__ __forceinline__ void flow_take_strided(Rsrc x, uint32_t first, float (&out)[16], Flow &f) {
     uint64_t deadline = 0;
+    uint32_t rounds = 0;
     for (;;) {
+        uint32_t u[16];
 #pragma unroll
-        for (int k = 0; k < N; ++k) v[k] = buf_load16<AUX_FLOW>(x, ((uint32_t)k < nlive ? first + (uint32_t)k * step : spare) * 16u);
+        for (int i = 0; i < 16; ++i) u[i] = __builtin_amdgcn_raw_buffer_load_b32(x, (int)((first + 16u * i) * 4u), 0, AUX_FLOW);
         bool hole = false;
 #pragma unroll
-        for (int k = 0; k < N; ++k) hole = hole || ((uint32_t)k < nlive && flow_empty(v[k]));
-        if (!__any(hole) || f.dead) break;
-        flow_backoff(f, deadline);
+        for (int i = 0; i < 16; ++i) hole = hole || u[i] == FLOW_EMPTY;
+        if (!__any(hole) || f.dead) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) out[i] = __uint_as_float(u[i]);
+            return;
+        }
+        flow_backoff(f, deadline, rounds);
     }
 }
 
 // ---- a unit of up to 64 rows of a 64-row-tile matrix (q / k / v, gate + up, output matrix) -------------------------------
 struct TileIn {
     Rsrc x;                   // the input vector (n floats)
-    bool flow;                // written by this launch: read with flow_acquire; else ordinary memory from before the launch
+    bool flow;                // written by this launch: read with flow_take; else ordinary memory from before the launch
     Rsrc norm_w;              // RMSNorm weights (n floats)
     uint32_t n;               // columns
     float eps;
 };
 
-// Stages the normalised-but-unscaled input (x * w, then the n/16 sums of 16) into `slot` and the sum of squares into
-// red[0..3]: the last four waves of the workgroup, up to four 16-byte pieces per lane (n <= 4096).  rms_norm.slang:48-67;
-// the scale is applied to the finished dot product.
-__device__ __forceinline__ void stage_tile_input(const TileIn &in, float *slot, float *red, Flow &f) {
-    const uint32_t tid = (uint32_t)phase_tid(), lane = tid & 63u, wave = tid >> 6;
-    const uint32_t l = plan::stage64_lane(tid);                  // 0 .. 255
-    uint32_t idx[4];
-    bool live[4];
-    float4 w[4];
-    uint32_t nlive = 0;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {                                   // the norm weights first: they depend on nothing
-        idx[k] = plan::stage64_piece(l, k);
-        live[k] = plan::stage64_live(l, k, in.n);
-        nlive += live[k] ? 1u : 0u;
-        w[k] = as_float4(buf_load16<AUX_PLAIN>(in.norm_w, (live[k] ? idx[k] : l) * 16u));
-    }
-    u32x4 raw[4];
-    if (in.flow) {
-        flow_probe(in.x, plan::stage64_probe(wave, in.n), f);
-        flow_acquire<4>(in.x, l, 256u, nlive, l, raw, f);
-    } else {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) raw[k] = buf_load16<AUX_PLAIN>(in.x, (live[k] ? idx[k] : l) * 16u);
-    }
-    float ss = 0.0f;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        float4 v = as_float4(raw[k]);
-        if (!live[k]) v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
-        v.x *= w[k].x; v.y *= w[k].y; v.z *= w[k].z; v.w *= w[k].w;
-        float s4 = (v.x + v.y) + (v.z + v.w);
-        s4 += __shfl_xor(s4, 1, 64);
-        s4 += __shfl_xor(s4, 2, 64);                               // lanes 4q..4q+3 hold 16 consecutive activations
-        if (live[k]) {
-            *reinterpret_cast<float4 *>(slot + 4 * idx[k]) = v;
-            if ((lane & 3) == 0) slot[in.n + (idx[k] >> 2)] = s4;
-        }
-    }
-    ss = wave_sum(ss);
-    if (lane == 0) red[wave - (PNW - plan::STAGERS64)] = ss;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");               // the slot is in L2 before the barrier lets the readers go
-}
-
-// One unit: rows unit.row0 .. + unit.nrows - 1 of W (and W2) times the staged input; returns, in threads 0 .. nrows - 1,
-// the finished value of row unit.row0 + thread (scaled; gate/up combined with SiLU when DUAL).  `stage`: false when the
-// slot still holds this input.
-// smem: partial[2][16][64], red[2][4] (red alternates between calls so that a fast wave cannot overwrite it early).
+// One unit: rows unit.row0 .. + unit.nrows - 1 of W (and W2) times the RMS-normalised input; returns, in threads
+// 0 .. nrows - 1, the finished value of row unit.row0 + thread (scaled; gate/up combined with SiLU when DUAL).
+// Wave w owns super-block w and is on its own until the partial sums meet: it requests its weights, then waits for the
+// 256 input values of its super-block (one 16-byte piece per lane), leaves x * w and the sums of 16 in its part of the
+// workgroup's slot (rms_norm.slang:48-67; the scale is applied to the finished dot product) and reads them back as
+// scalar operands.  `stage`: false when the slot still holds this input.
+// smem: partial[2][16][64], red[2][16] (red alternates between calls so that a fast wave cannot overwrite it early).
 template <int T, bool DUAL>
 __device__ __forceinline__ float tile64_phase(const DevBuf &W, const DevBuf &W2, const plan::RowUnit unit, uint32_t ncb, const TileIn &in, bool stage,
                                               float *slot, float *partial, float *red, Flow &f, uint64_t *tr) {
@@ -231,31 +190,40 @@ __device__ __forceinline__ float tile64_phase(const DevBuf &W, const DevBuf &W2,
     constexpr uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
     constexpr int NM = DUAL ? 2 : 1;
     const bool has_unit = (uint32_t)wave < ncb;
-    const bool stager = wave >= PNW - (int)plan::STAGERS64;
-    typename F::Data d, e;
-    uint16_t dt = 0, et = 0;
-    // As much of the unit as the registers hold without spilling is requested before the wait (a spill of a requested
-    // piece would make the wave wait for it before the barrier); the rest follows while the first stages are multiplied.
-    BufUnitLoader<T, NM, DUAL ? 4 : (F::PT > 9 ? 6 : 8)> ld;
-    auto request = [&]() {
-        const uint32_t row = unit.row0 + plan::umin((uint32_t)lane, unit.nrows - 1);     // lanes past the unit repeat its last row
-        const uint32_t voff = plan::tile64_piece0(row, (uint32_t)wave, ncb, unit_bytes);
-        const uint32_t toff = plan::tile64_tail(row, (uint32_t)wave, ncb, unit_bytes, F::PT);
-        ld.rs[0] = W.rs; ld.voff[0] = voff; ld.toff[0] = toff; ld.d[0] = &d; ld.t[0] = &dt;
-        if constexpr (DUAL) { ld.rs[1] = W2.rs; ld.voff[1] = voff; ld.toff[1] = toff; ld.d[1] = &e; ld.t[1] = &et; }
-        F::lead(ld);
-    };
-    stamp(tr, 0);
-    if (stager && stage) {                                        // (either role, never both: the registers hold one at a time)
-        stage_tile_input(in, slot, red, f);
-        if (has_unit) request();
-    } else if (has_unit) {
-        request();
-    }
-    lds_barrier();
-    stamp(tr, 1);
     float v = 0.0f, v2 = 0.0f;
+    stamp(tr, 0);
     if (has_unit) {
+        typename F::Data d, e;
+        uint16_t dt = 0, et = 0;
+        // As much of the unit as the registers hold without spilling is requested before the wait; the rest follows
+        // while the first stages are multiplied.
+        BufUnitLoader<T, NM, DUAL ? 4 : (F::PT > 9 ? 6 : 8)> ld;
+        {
+            const uint32_t row = unit.row0 + plan::umin((uint32_t)lane, unit.nrows - 1);     // lanes past the unit repeat its last row
+            const uint32_t voff = plan::tile64_piece0(row, (uint32_t)wave, ncb, unit_bytes);
+            const uint32_t toff = plan::tile64_tail(row, (uint32_t)wave, ncb, unit_bytes, F::PT);
+            ld.rs[0] = W.rs; ld.voff[0] = voff; ld.toff[0] = toff; ld.d[0] = &d; ld.t[0] = &dt;
+            if constexpr (DUAL) { ld.rs[1] = W2.rs; ld.voff[1] = voff; ld.toff[1] = toff; ld.d[1] = &e; ld.t[1] = &et; }
+            F::lead(ld);
+        }
+        if (stage) {
+            const uint32_t piece = plan::wave_piece((uint32_t)wave, (uint32_t)lane);
+            const float4 w = as_float4(buf_load16<AUX_PLAIN>(in.norm_w, piece * 16u));
+            // (loads retire in issue order: the first answer comes after the weights requested above, which have
+            // had the whole previous phase to travel)
+            float4 x = as_float4(in.flow ? flow_take(in.x, piece, f) : buf_load16<AUX_PLAIN>(in.x, piece * 16u));
+            float ss = fmaf(x.x, x.x, fmaf(x.y, x.y, fmaf(x.z, x.z, x.w * x.w)));
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+            x.x *= w.x; x.y *= w.y; x.z *= w.z; x.w *= w.w;
+            float s4 = (x.x + x.y) + (x.z + x.w);
+            s4 += __shfl_xor(s4, 1, 64);
+            s4 += __shfl_xor(s4, 2, 64);                               // lanes 4q..4q+3 hold 16 consecutive activations
+            *reinterpret_cast<float4 *>(slot + 4 * piece) = x;
+            if ((lane & 3) == 0) slot[in.n + (piece >> 2)] = s4;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // the wave's part of the slot is in L2
+        }
+        stamp(tr, 1);
         // The slot was rewritten with vector stores; the scalar cache may still hold what it held before.  Drop that,
         // and hand the compiler the pointer only now: loads through the constant address space move freely otherwise.
         asm volatile("s_dcache_inv\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
@@ -279,9 +247,9 @@ __device__ __forceinline__ float tile64_phase(const DevBuf &W, const DevBuf &W2,
     stamp(tr, 3);
     float o = 0.0f;
     if (tid < 64) {
-        const float t = (red[0] + red[1]) + (red[2] + red[3]);
+        float t = 0.0f;
+        for (uint32_t w = 0; w < ncb; ++w) { t += red[w]; o += partial[w * 64 + tid]; }
         const float scale = 1.0f / sqrtf(t / (float)in.n + in.eps);
-        for (uint32_t w = 0; w < ncb; ++w) o += partial[w * 64 + tid];
         o *= scale;
         if constexpr (DUAL) {
             float up = 0.0f;
@@ -295,66 +263,31 @@ __device__ __forceinline__ float tile64_phase(const DevBuf &W, const DevBuf &W2,
 
 // ---- a 16-row tile (attention output projection, down projection) -------------------------------------------------------
 // Rows tile*16 .. +15 of W times the n-vector `x` (written by this launch); returns the row's dot product in threads
-// 0..15.  Waves 0 .. ngroups-1 multiply (one unit of 16 rows x 4 super-blocks each), the others fetch the vector into xs.
+// 0..15.  Waves 0 .. ngroups-1 multiply (one unit of 16 rows x 4 super-blocks each): each requests its weights, then
+// waits for the 1024 input values of its four super-blocks, 16 per lane, straight into the registers they are used from.
 template <int T>
-__device__ __forceinline__ float tile16_phase(const DevBuf &W, uint32_t tile, uint32_t ncb, uint32_t ngroups, Rsrc x, uint32_t n, float *xs,
-                                              float *partial, Flow &f, uint64_t *tr) {
+__device__ __forceinline__ float tile16_phase(const DevBuf &W, uint32_t tile, uint32_t ncb, uint32_t ngroups, Rsrc x, float *partial, Flow &f, uint64_t *tr) {
     using F = Tiled<T>;
     const int tid = phase_tid(), lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
     const bool has_unit = (uint32_t)wave < ngroups;
-    const uint32_t first_stager = plan::stage16_first(ngroups);
-    const bool stager = (uint32_t)wave >= first_stager;
-    typename F::Data d;
-    uint16_t dt = 0;
-    BufUnitLoader<T, 1, (F::PT > 9 ? 6 : 8)> ld;
-    auto request = [&]() {
+    float v = 0.0f;
+    stamp(tr, 0);
+    if (has_unit) {
+        typename F::Data d;
+        uint16_t dt = 0;
+        BufUnitLoader<T, 1, (F::PT > 9 ? 6 : 8)> ld;
         ld.rs[0] = W.rs; ld.d[0] = &d; ld.t[0] = &dt;
         ld.voff[0] = plan::tile16_piece0(tile, (uint32_t)wave, ngroups, unit_bytes, (uint32_t)lane);
         ld.toff[0] = plan::tile16_tail(tile, (uint32_t)wave, ngroups, unit_bytes, F::PT, (uint32_t)lane);
         F::lead(ld);
-    };
-    stamp(tr, 0);
-    if (!stager) {
-        if (has_unit) request();
-    } else {
-        // lane l of the nl stager lanes takes pieces l, l + nl, ...: four per round trip, or twelve when there are many
-        const uint32_t nl = plan::stage16_lanes(ngroups), l = (uint32_t)tid - first_stager * 64u;
-        const uint32_t chunks = n / 4;
-        flow_probe(x, plan::stage16_probe((uint32_t)wave, ngroups, chunks), f);
-        const uint32_t spare = (uint32_t)lane;                                   // (chunks >= 64: n >= 256)
-        if (plan::stage16_per_trip(chunks, nl) == 12u) {
-            const uint32_t trips = plan::stage16_trips(chunks, nl);
-            for (uint32_t j = 0; j < trips; ++j) {                     // whole waves call the acquire
-                const uint32_t i0 = plan::stage16_first_piece(l, nl, j, 12u);
-                const uint32_t nlive = plan::stage16_nlive(i0, nl, chunks, 12u);
-                u32x4 raw[12];
-                flow_acquire<12>(x, i0, nl, nlive, spare, raw, f);
-#pragma unroll
-                for (int k = 0; k < 12; ++k)
-                    if ((uint32_t)k < nlive) *reinterpret_cast<u32x4 *>(xs + 4 * (size_t)(i0 + k * nl)) = raw[k];
-            }
-        } else {
-            const uint32_t nlive = plan::stage16_nlive(l, nl, chunks, 4u);
-            u32x4 raw[4];
-            flow_acquire<4>(x, l, nl, nlive, spare, raw, f);
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if ((uint32_t)k < nlive) *reinterpret_cast<u32x4 *>(xs + 4 * (size_t)(l + k * nl)) = raw[k];
-        }
-        if (has_unit) request();
-    }
-    lds_barrier();
-    stamp(tr, 1);
-    float v = 0.0f;
-    if (has_unit) {
-        const int kq = lane >> 4, lane16 = lane & 15;
-        const uint32_t cb = (uint32_t)wave * 4 + kq;
-        const bool valid = cb < ncb;
+        const bool valid = plan::tile16_cb((uint32_t)wave, (uint32_t)lane) < ncb;
         DevX X;
+        flow_take_strided(x, plan::tile16_x0((uint32_t)wave, (uint32_t)lane, ncb), X.x, f);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) X.x[i] = valid ? xs[(size_t)cb * 256 + 16 * i + lane16] : 0.0f;
+        for (int i = 0; i < 16; ++i) X.x[i] = valid ? X.x[i] : 0.0f;
+        stamp(tr, 1);
         if constexpr (T == T_Q6_K) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) X.s[i] = row16_sum(X.x[i]);
@@ -389,10 +322,9 @@ __device__ __forceinline__ float tile64_any(const DevBuf &W, const DevBuf &W2, c
     default: return tile64_phase<T_Q4_K, DUAL>(W, W2, unit, ncb, in, stage, slot, partial, red, f, tr);
     }
 }
-__device__ __forceinline__ float tile16_any(const DevBuf &W, uint32_t tile, uint32_t ncb, uint32_t ngroups, Rsrc x, uint32_t n, float *xs,
-                                            float *partial, Flow &f, uint64_t *tr) {
-    if (W.type == T_Q6_K) return tile16_phase<T_Q6_K>(W, tile, ncb, ngroups, x, n, xs, partial, f, tr);
-    return tile16_phase<T_Q4_K>(W, tile, ncb, ngroups, x, n, xs, partial, f, tr);
+__device__ __forceinline__ float tile16_any(const DevBuf &W, uint32_t tile, uint32_t ncb, uint32_t ngroups, Rsrc x, float *partial, Flow &f, uint64_t *tr) {
+    if (W.type == T_Q6_K) return tile16_phase<T_Q6_K>(W, tile, ncb, ngroups, x, partial, f, tr);
+    return tile16_phase<T_Q4_K>(W, tile, ncb, ngroups, x, partial, f, tr);
 }
 
 __device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
@@ -410,9 +342,12 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
     constexpr int LWORDS = sizeof(PersistentLayer) / 4;
     static_assert(LWORDS <= PNT && sizeof(PersistentLayer) == 14 * sizeof(ResidentBuf), "one thread per word; fourteen entries");
     __shared__ uint32_t layer_words[2][LWORDS];
-    float *partial = smem + plan::lds_partial();                   // [2][16][64]
-    float *red = smem + plan::lds_red();                           // [2][4]
-    float *xs = smem + plan::lds_xs();                             // [max(dim, hidden)]
+    // Two sets of partial[2][16][64] | red[16], taken in turn by the phases of this workgroup: a wave that is done with a
+    // phase goes on to the next one (there is one barrier per phase, before its reduction) while wave 0 may still be
+    // reducing the one before, but it cannot get further ahead than that.
+    float *const lds_sets = smem;
+#define PHASE_PARTIAL (lds_sets + plan::lds_set(phase & 1u) + plan::lds_partial())
+#define PHASE_RED (lds_sets + plan::lds_set(phase & 1u) + plan::lds_red())
     touch_kernel_arguments<sizeof(PersistentParams)>();
     const uint32_t b = blockIdx.x;
     // A launch after one in which a reader gave up does nothing: the host has not looked yet (it queues many tokens), and
@@ -425,7 +360,7 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
     float *slot = p.slots + plan::slot_of(sh, b);
     // time stamps: 16 per layer (4 per phase: entered, input staged, multiplied, reduced), then 4 for the output matrix and the end
     uint64_t *trace = p.trace ? p.trace + plan::trace_row(sh, b) : nullptr;
-    uint32_t phase = 0;                                            // parity picks the red[] half
+    uint32_t phase = 0;                                            // phases this workgroup has run: parity picks the LDS set
     // the residual value of row 16b + tid: the embedding row the launch before this one left in p.x
     float xres = 0.0f;
     if (b < plan::proj_tiles(sh) && threadIdx.x < 16) xres = p.x[16 * b + threadIdx.x];
@@ -451,7 +386,7 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
             const DevBuf W = u.seg == 0 ? LAYER_BUF(lw, wv) : (u.seg == 1 ? LAYER_BUF(lw, wk) : LAYER_BUF(lw, wq));
             float *out = u.seg == 0 ? p.vcol : (u.seg == 1 ? p.kcol : p.q);
             const TileIn in{l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, LAYER_BUF(lw, attn_norm).rs, dim, p.eps};
-            const float o = tile64_any<false>(W, W, u, ncb, in, true, slot, partial, red + 4 * (phase & 1u), f, tl);
+            const float o = tile64_any<false>(W, W, u, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tl);
             const uint32_t tid = phase_tid();
             if (tid < 64) {
                 if (tid < u.nrows) flow_store(out + u.row0 + tid, o);
@@ -501,24 +436,26 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
         }
         // ---- attention output projection into the residual ---------------------------------------------------------
         if (b < plan::proj_tiles(sh)) {
-            const float o = tile16_any(LAYER_BUF(lw, wo), b, ncb, ng_o, xb, dim, xs, partial, f, tl ? tl + 4 : nullptr);
+            const float o = tile16_any(LAYER_BUF(lw, wo), b, ncb, ng_o, xb, PHASE_PARTIAL, f, tl ? tl + 4 : nullptr);
             const uint32_t tid = phase_tid();
             if (tid < 16) { xres += o; flow_put(xm, 16 * b + tid, xres); }             // transformer.rs:352-355
+            ++phase;
         }
         // ---- RMSNorm + gate / up + SiLU ---------------------------------------------------------------------------------
         if (b < plan::gu_units(sh)) {
             const plan::RowUnit u = plan::gu_unit(sh, b);
             const TileIn in{xm, true, LAYER_BUF(lw, ffn_norm).rs, dim, p.eps};
-            const float o = tile64_any<true>(LAYER_BUF(lw, wgate), LAYER_BUF(lw, wup), u, ncb, in, true, slot, partial, red + 4 * (phase & 1u), f, tl ? tl + 8 : nullptr);
+            const float o = tile64_any<true>(LAYER_BUF(lw, wgate), LAYER_BUF(lw, wup), u, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tl ? tl + 8 : nullptr);
             const uint32_t tid = phase_tid();
             if (tid < u.nrows) flow_put(hb, u.row0 + tid, o);
             ++phase;
         }
         // ---- down projection into the residual ----------------------------------------------------------------------------
         if (b < plan::proj_tiles(sh)) {
-            const float o = tile16_any(LAYER_BUF(lw, wdown), b, ncb_h, ng_d, hb, hid, xs, partial, f, tl ? tl + 12 : nullptr);
+            const float o = tile16_any(LAYER_BUF(lw, wdown), b, ncb_h, ng_d, hb, PHASE_PARTIAL, f, tl ? tl + 12 : nullptr);
             const uint32_t tid = phase_tid();
             if (tid < 16) { xres += o; flow_put(xnext, 16 * b + tid, xres); }          // transformer.rs:362-365
+            ++phase;
         }
         if (threadIdx.x < LWORDS) layer_words[(l + 1) & 1u][threadIdx.x] = next_word;
         lds_barrier();
@@ -529,10 +466,10 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
         const TileIn in{make_rsrc(p.flow + plan::flow_xa(sh, p.n_layers), dim * 4u), true, dev_buf(p.out_norm).rs, dim, p.eps};
         const DevBuf wout = dev_buf(p.wout);
         bool first = true;
-        const uint32_t par = phase & 1u;                            // the input is staged once: its sum of squares stays where it is
+        // (the input is staged once: its sums of squares stay in this set, and a barrier separates the tiles)
         for (uint32_t tile = b; tile < ntiles; tile += gridDim.x) {
             const plan::RowUnit u{0u, tile * 64u, plan::umin(64u, p.vocab - tile * 64u)};
-            const float o = tile64_any<false>(wout, wout, u, ncb, in, first, slot, partial, red + 4 * par, f, first && trace ? trace + 16 * p.n_layers : nullptr);
+            const float o = tile64_any<false>(wout, wout, u, ncb, in, first, slot, PHASE_PARTIAL, PHASE_RED, f, first && trace ? trace + 16 * p.n_layers : nullptr);
             const uint32_t tid = phase_tid();
             if (tid < u.nrows) p.logits[u.row0 + tid] = o;
             first = false;
@@ -541,6 +478,9 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
         stamp(trace ? trace + 16 * p.n_layers : nullptr, 4);
     }
 }
+
+#undef PHASE_PARTIAL
+#undef PHASE_RED
 
 // Fills the hand-off buffers of a launch with FLOW_EMPTY (16 bytes per thread and step).
 __global__ void flow_fill_kernel(u32x4 *buf, size_t n16) {

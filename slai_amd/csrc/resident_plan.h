@@ -21,8 +21,6 @@ static_assert(join_words((uint32_t)(int)0xffffffffu, 0u) == 0x00000000fffffffful
 namespace plan {
 
 constexpr uint32_t WG_THREADS = 1024, WG_WAVES = 16;
-constexpr uint32_t STAGERS64 = 4;          // waves that stage the input of a 64-row-unit phase (the last four)
-constexpr uint32_t MAX_MULT16 = 12;        // waves that multiply in a 16-row-tile phase before the others only stage
 
 struct Shape {
     uint32_t dim, hidden, n_heads, n_layers, vocab, seq_len;
@@ -46,8 +44,8 @@ SLAI_HD Shape make_shape(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32
 // ---- supported shapes: what the kernel's index arithmetic assumes -------------------------------------------------------
 SLAI_HD bool shape_ok(const Shape &s) {
     if (s.n_heads == 0 || s.n_heads % 8 || s.dim != s.n_heads * 128) return false;            // heads of 128, eight dies
-    if (s.dim % 1024 || s.dim > 4096) return false;                                            // four staging pieces per lane at most
-    if (s.hidden % 256 || s.hidden / 256 > 64) return false;                                   // sixteen multiplying waves x four super-blocks
+    if (s.dim % 1024 || s.dim > 4096) return false;                                            // one wave per super-block of the input
+    if (s.hidden % 256 || s.hidden / 256 > 64) return false;                                   // sixteen waves x four super-blocks in the down projection
     if (s.grid % 8 || s.grid > 1024) return false;
     if ((s.qkv_units != 6 && s.qkv_units != 7) || (s.qkv_units + 1) * s.n_heads > s.grid) return false;
     if (s.dim / 16 > s.grid) return false;                                                     // one 16-row tile of the projections each
@@ -73,11 +71,11 @@ SLAI_HD uint64_t slot_of(const Shape &s, uint32_t b) { return (uint64_t)b * slot
 SLAI_HD uint32_t slot_x(uint32_t cb) { return cb * 256; }
 SLAI_HD uint32_t slot_sums(const Shape &s, uint32_t cb) { return s.dim + cb * 16; }
 
-// ---- dynamic LDS of a workgroup, in floats: partial[2][16][64] | red[2][4] | xs[max(dim, hidden)] -----------------------
+// ---- dynamic LDS of a workgroup, in floats: two sets of partial[2][16][64] | red[16], used by its phases in turn -----------
 SLAI_HD uint32_t lds_partial() { return 0; }
 SLAI_HD uint32_t lds_red() { return 2 * WG_WAVES * 64; }
-SLAI_HD uint32_t lds_xs() { return lds_red() + 8; }
-SLAI_HD uint32_t lds_floats(const Shape &s) { return lds_xs() + umax(s.dim, s.hidden); }
+SLAI_HD uint32_t lds_set(uint32_t parity) { return parity * (lds_red() + WG_WAVES); }
+SLAI_HD uint32_t lds_floats(const Shape &) { return 2 * (lds_red() + WG_WAVES); }
 
 // ---- counters of the q / k / v -> attention hand-off: one 128-byte line per head, then the flag of a wait that gave up ---
 SLAI_HD uint32_t counter_word(uint32_t head) { return head * 32; }
@@ -133,28 +131,14 @@ SLAI_HD uint32_t tile16_tail(uint32_t tile, uint32_t g, uint32_t ngroups, uint32
 }
 SLAI_HD uint32_t unit_bytes_of(int type) { return tiled_pieces(type) * 1024u + tiled_tail(type); }
 
-// ---- staging the input of a 64-row-unit phase: the last four waves, lane l = 0 .. 255 of them, piece l + 256 k, k < 4 -------
-SLAI_HD uint32_t stage64_lane(uint32_t tid) { return tid - (WG_WAVES - STAGERS64) * 64u; }
-SLAI_HD uint32_t stage64_piece(uint32_t l, uint32_t k) { return l + 256u * k; }                // index of a 16-byte piece (4 floats)
-SLAI_HD bool stage64_live(uint32_t l, uint32_t k, uint32_t n) { return stage64_piece(l, k) < n / 4; }
-// the piece a stager wave polls before it fetches its share (its own first piece, or piece 0 when it has none)
-SLAI_HD uint32_t stage64_probe(uint32_t wave, uint32_t n) {
-    const uint32_t first = 64u * (wave - (WG_WAVES - STAGERS64));
-    return first < n / 4 ? first : 0u;
-}
+// ---- the input of a 64-row-unit phase: wave w (< ncb) fetches the 256 values of super-block w, 16 bytes per lane, and ------
+// leaves them (weighted) and their sums of 16 in its part of the workgroup's slot
+SLAI_HD uint32_t wave_piece(uint32_t wave, uint32_t lane) { return wave * 64u + lane; }          // index of a 16-byte piece (4 floats)
 
-// ---- staging the input of a 16-row-tile phase into LDS: waves first_stager .. 15 --------------------------------------------
-SLAI_HD uint32_t stage16_first(uint32_t ngroups) { return umin(ngroups, MAX_MULT16); }
-SLAI_HD uint32_t stage16_lanes(uint32_t ngroups) { return (WG_WAVES - stage16_first(ngroups)) * 64u; }
-// lane l of the nl staging lanes takes pieces l, l + nl, ...; `per_trip` (4 or 12) of them per round trip
-SLAI_HD uint32_t stage16_per_trip(uint32_t chunks, uint32_t nl) { return chunks > 4 * nl ? 12u : 4u; }
-SLAI_HD uint32_t stage16_trips(uint32_t chunks, uint32_t nl) { const uint32_t pt = stage16_per_trip(chunks, nl); return (chunks + pt * nl - 1) / (pt * nl); }
-SLAI_HD uint32_t stage16_first_piece(uint32_t l, uint32_t nl, uint32_t trip, uint32_t per_trip) { return per_trip * trip * nl + l; }
-SLAI_HD uint32_t stage16_nlive(uint32_t i0, uint32_t nl, uint32_t chunks, uint32_t per_trip) { return i0 < chunks ? umin(per_trip, (chunks - i0 + nl - 1) / nl) : 0u; }
-SLAI_HD uint32_t stage16_probe(uint32_t wave, uint32_t ngroups, uint32_t chunks) {
-    const uint32_t first = (wave - stage16_first(ngroups)) * 64u;
-    return first < chunks ? first : 0u;
-}
+// ---- the input of a 16-row-tile phase: lane (kq, j) of wave g holds x[cb * 256 + 16 i + j], i < 16, cb = 4 g + kq ---------
+SLAI_HD uint32_t tile16_cb(uint32_t wave, uint32_t lane) { return wave * 4u + (lane >> 4); }
+// first float of the lane's sixteen (lanes whose super-block does not exist read super-block 0 and drop it)
+SLAI_HD uint32_t tile16_x0(uint32_t wave, uint32_t lane, uint32_t ncb) { const uint32_t cb = tile16_cb(wave, lane); return (cb < ncb ? cb : 0u) * 256u + (lane & 15u); }
 
 }  // namespace plan
 }  // namespace slai

@@ -4,9 +4,8 @@
 //
 // rb_audit walks, for every workgroup, wave and lane of a launch and every layer:
 //   * the weight pieces and tails a lane requests in each phase, against the matrix's bytes;
-//   * the pieces of a hand-off vector a staging lane fetches (and the one it polls, and its spare piece), against the
-//     vector, and the words it writes into the slot / into LDS, against the slot / the LDS block; what the multiplying
-//     waves read back from there;
+//   * the piece of a hand-off vector a lane fetches, against the vector, and the words it writes into the workgroup's
+//     slot, against the slot; what the wave reads back from there;
 //   * the rows a workgroup writes into the hand-off vectors, q / k / v, the logits; counters, trace rows, the layer table;
 //   * coverage: every output row of every matrix is produced exactly once per layer and every piece of an input vector is
 //     staged exactly once per workgroup and phase;
@@ -75,74 +74,54 @@ void walk_tile64(Audit &a, const Region &w, int type, const plan::RowUnit &u, ui
         }
 }
 
-// staging of an n-vector into the workgroup's slot by the last four waves, and what the multiplying waves read back
+// the input of a 64-row-unit phase: wave w < ncb fetches piece w * 64 + lane of the n-vector and of the norm weights,
+// leaves the weighted values and their sums of 16 in the workgroup's slot, and reads its part of the slot back
 void walk_stage64(Audit &a, const plan::Shape &s, const Region &x, const Region &norm, const Region &slots, uint32_t n, uint32_t ncb, uint32_t b, uint32_t layer) {
     std::vector<uint32_t> seen(n / 4, 0);
     const uint64_t slot0 = plan::slot_of(s, b) * 4;
-    for (uint32_t wave = plan::WG_WAVES - plan::STAGERS64; wave < plan::WG_WAVES; ++wave) {
-        a.touch(x, (uint64_t)plan::stage64_probe(wave, n) * 16, 16, "probe", b, wave, 0, layer);
-        for (uint32_t lane = 0; lane < 64; ++lane) {
-            const uint32_t tid = wave * 64 + lane, l = plan::stage64_lane(tid);
-            a.touch(x, (uint64_t)l * 16, 16, "spare piece", b, wave, lane, layer);
-            for (uint32_t k = 0; k < 4; ++k) {
-                const uint32_t idx = plan::stage64_piece(l, k);
-                const bool live = plan::stage64_live(l, k, n);
-                a.touch(norm, (uint64_t)(live ? idx : l) * 16, 16, "norm weights", b, wave, lane, layer);
-                if (!live) continue;
-                a.touch(x, (uint64_t)idx * 16, 16, "input piece", b, wave, lane, layer);
-                a.touch(slots, slot0 + (uint64_t)idx * 16, 16, "slot values", b, wave, lane, layer);
-                if ((lane & 3) == 0) a.touch(slots, slot0 + ((uint64_t)n + (idx >> 2)) * 4, 4, "slot sums", b, wave, lane, layer);
-                if (idx < seen.size()) ++seen[idx];
-            }
-        }
-    }
-    for (uint32_t i = 0; i < seen.size(); ++i)
-        if (seen[i] != 1) { a.fail("64-row-unit staging: a piece of the input is staged " + std::to_string(seen[i]) + " times"); break; }
-    if ((uint64_t)n + n / 16 > plan::slot_stride(s)) a.fail("the slot is smaller than the staged input");
     for (uint32_t wave = 0; wave < plan::WG_WAVES && wave < ncb; ++wave) {
+        for (uint32_t lane = 0; lane < 64; ++lane) {
+            const uint32_t piece = plan::wave_piece(wave, lane);
+            a.touch(norm, (uint64_t)piece * 16, 16, "norm weights", b, wave, lane, layer);
+            a.touch(x, (uint64_t)piece * 16, 16, "input piece", b, wave, lane, layer);
+            a.touch(slots, slot0 + (uint64_t)piece * 16, 16, "slot values", b, wave, lane, layer);
+            if ((lane & 3) == 0) a.touch(slots, slot0 + ((uint64_t)n + (piece >> 2)) * 4, 4, "slot sums", b, wave, lane, layer);
+            if (piece < seen.size()) ++seen[piece];
+            // what the wave reads back must be what the wave wrote
+            if (piece * 4 < plan::slot_x(wave) || piece * 4 + 4 > plan::slot_x(wave) + 256) a.fail("a wave stages values outside the part of the slot it reads");
+        }
         a.touch(slots, slot0 + (uint64_t)plan::slot_x(wave) * 4, 256 * 4, "slot read (activations)", b, wave, 0, layer);
         a.touch(slots, slot0 + ((uint64_t)n + wave * 16) * 4, 16 * 4, "slot read (sums)", b, wave, 0, layer);
         if (plan::slot_x(wave) + 256 > n) a.fail("a multiplying wave reads activations past the input");
     }
+    for (uint32_t i = 0; i < seen.size(); ++i)
+        if (seen[i] != 1) { a.fail("64-row-unit phase: a piece of the input is staged " + std::to_string(seen[i]) + " times"); break; }
+    if ((uint64_t)n + n / 16 > plan::slot_stride(s)) a.fail("the slot is smaller than the staged input");
+    if ((uint64_t)plan::lds_set(1) + plan::lds_red() + plan::WG_WAVES > plan::lds_floats(s) || ncb > plan::WG_WAVES) a.fail("LDS block smaller than what the phases index");
 }
 
-// a 16-row tile phase: weights of the multiplying waves, staging of the n-vector into LDS by the others
+// a 16-row tile phase: weights of the multiplying waves and the sixteen floats of the n-vector each of their lanes takes
 void walk_tile16(Audit &a, const plan::Shape &s, const Region &w, int type, uint32_t tile, uint32_t ncb, uint32_t ngroups, const Region &x, uint32_t n, uint32_t b,
                  uint32_t layer) {
+    (void)s;
     const uint32_t ub = plan::unit_bytes_of(type), pt = tiled_pieces(type);
-    const Region lds{"LDS xs", 0x10000u, (uint64_t)(plan::lds_floats(s) - plan::lds_xs()) * 4};
-    for (uint32_t wave = 0; wave < plan::WG_WAVES && wave < ngroups; ++wave)
+    if (ngroups > plan::WG_WAVES) { a.fail("more column groups than waves"); return; }
+    std::vector<uint32_t> seen(n, 0);
+    for (uint32_t wave = 0; wave < ngroups; ++wave)
         for (uint32_t lane = 0; lane < 64; ++lane) {
             const uint32_t voff = plan::tile16_piece0(tile, wave, ngroups, ub, lane);
             for (uint32_t p = 0; p < pt; ++p) a.touch(w, (uint64_t)voff + p * 1024u, 16, "weight piece (16-row tile)", b, wave, lane, layer);
             if (tiled_tail(type)) a.touch(w, plan::tile16_tail(tile, wave, ngroups, ub, pt, lane), 2, "weight tail (16-row tile)", b, wave, lane, layer);
-            const uint32_t cb = wave * 4 + (lane >> 4);
-            if (cb < ncb)
-                for (uint32_t i = 0; i < 16; ++i) a.touch(lds, ((uint64_t)cb * 256 + 16 * i + (lane & 15)) * 4, 4, "LDS read", b, wave, lane, layer);
-        }
-    if (ngroups > plan::WG_WAVES) { a.fail("more column groups than waves"); return; }
-    const uint32_t first = plan::stage16_first(ngroups), nl = plan::stage16_lanes(ngroups), chunks = n / 4;
-    if (nl == 0) { a.fail("a 16-row-tile phase without staging waves"); return; }
-    std::vector<uint32_t> seen(chunks, 0);
-    const uint32_t per = plan::stage16_per_trip(chunks, nl), trips = plan::stage16_trips(chunks, nl);
-    for (uint32_t wave = first; wave < plan::WG_WAVES; ++wave) {
-        a.touch(x, (uint64_t)plan::stage16_probe(wave, ngroups, chunks) * 16, 16, "probe", b, wave, 0, layer);
-        for (uint32_t lane = 0; lane < 64; ++lane) {
-            const uint32_t l = wave * 64 + lane - first * 64;
-            a.touch(x, (uint64_t)lane * 16, 16, "spare piece", b, wave, lane, layer);
-            for (uint32_t j = 0; j < trips; ++j) {
-                const uint32_t i0 = plan::stage16_first_piece(l, nl, j, per), nlive = plan::stage16_nlive(i0, nl, chunks, per);
-                for (uint32_t k = 0; k < nlive; ++k) {
-                    const uint32_t piece = i0 + k * nl;
-                    a.touch(x, (uint64_t)piece * 16, 16, "input piece", b, wave, lane, layer);
-                    a.touch(lds, (uint64_t)piece * 16, 16, "LDS write", b, wave, lane, layer);
-                    if (piece < chunks) ++seen[piece];
-                }
+            const uint32_t x0 = plan::tile16_x0(wave, lane, ncb);
+            const bool valid = plan::tile16_cb(wave, lane) < ncb;
+            for (uint32_t i = 0; i < 16; ++i) {
+                a.touch(x, ((uint64_t)x0 + 16 * i) * 4, 4, "input value (16-row tile)", b, wave, lane, layer);
+                if (valid && x0 + 16 * i < n && (lane & 15u) == (x0 & 15u) && lane < 64) ++seen[x0 + 16 * i];
             }
         }
-    }
-    for (uint32_t i = 0; i < chunks; ++i)
-        if (seen[i] != 1) { a.fail("16-row-tile staging: a piece of the input is staged " + std::to_string(seen[i]) + " times"); break; }
+    // every value of the input reaches exactly the 16-lane rows that multiply its super-block: once per such row = once here
+    for (uint32_t i = 0; i < n; ++i)
+        if (seen[i] != 1) { a.fail("16-row-tile phase: input value " + std::to_string(i) + " is taken " + std::to_string(seen[i]) + " times"); break; }
 }
 
 }  // namespace
