@@ -396,9 +396,10 @@ int slai_llama2::persistent_setup() {
     if (persistent_capacity(p, ctx->device, &resident) != hipSuccess) return no("the occupancy query for the kernel failed");
     hipDeviceProp_t prop;
     SLAI_HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
-    const uint32_t grid = std::min(resident, (uint32_t)prop.multiProcessorCount) / 8 * 8;
-    const plan::Shape sh = plan::make_shape(dim, hid, nh, nl, config.vocab_size, config.seq_len, grid);
-    if (!plan::shape_ok(sh)) return no("the device keeps too few workgroups of the kernel resident for this shape");
+    const plan::Shape sh = plan::make_shape(dim, hid, nh, nl, config.vocab_size, config.seq_len);
+    const uint32_t grid = sh.grid;                                    // one workgroup per compute unit at most, all resident
+    if (grid > std::min(resident, (uint32_t)prop.multiProcessorCount)) return no("the device keeps too few workgroups of the kernel resident for this shape");
+    if (!plan::shape_ok(sh)) return no("shape: the FFN width does not spread evenly over one workgroup per 16 rows of the model width");
     p.qkv_units = sh.qkv_units; p.gu_rows = sh.gu_rows;
     std::vector<PersistentLayer> host(nl);
     for (uint32_t l = 0; l < nl; ++l) {

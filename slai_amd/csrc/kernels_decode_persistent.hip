@@ -41,18 +41,40 @@ using namespace lanes;
 
 constexpr int PNT = plan::WG_THREADS, PNW = plan::WG_WAVES;   // threads and waves of a workgroup
 
-// The thread index as a value the compiler cannot follow: what a phase derives from it (lane offsets, addresses) is then
-// computed inside the phase instead of being kept alive across the whole layer loop, where it would not fit the registers.
-__device__ __forceinline__ int phase_tid() {
-    int t = threadIdx.x;
-    asm volatile("" : "+v"(t));
-    return t;
+// Who a thread is: the wave index is a wave-uniform value handed down from the top of the kernel, the lane index is
+// recomputed where it is needed.  The thread index itself must not live in a vector register across the layer loop: it
+// gets spilled there, and a reload of it behind the weights requested ahead waits for all of them.
+__device__ __forceinline__ uint32_t lane_id() {
+    uint32_t l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));      // (volatile: recomputed at every use, never kept)
+    return l;
+}
+
+// A wave-uniform value as one the compiler cannot follow: what is derived from it (comparisons, conversions) is computed
+// where it is used instead of once before the layer loop -- hoisted, a flag or a converted constant lives in a vector
+// register across the whole loop, is spilled there, and its reload waits behind the weights requested ahead.
+__device__ __forceinline__ uint32_t fresh(uint32_t v) {
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
+// Lane exchanges inside the phases.  The library forms (__shfl_xor) derive their lane index once, the compiler then keeps
+// every `lane ^ mask` alive across the whole layer loop -- in spilled registers, and a reload of one behind the weights
+// requested ahead waits for all of them.  These recompute the index where it is used.
+__device__ __forceinline__ float lane_xor(float v, int mask) {
+    const int l = (int)lane_id();
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((l ^ mask) & 63) << 2, __builtin_bit_cast(int, v)));
+}
+__device__ __forceinline__ float wave_total(float v) {            // the sum over the wave, in every lane
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += lane_xor(v, m);
+    return v;
 }
 
 // Optional time stamps (the constant 100 MHz clock) for a per-phase time line of every workgroup: profilers see one long
 // kernel.  `row` is null unless the host asked for a trace.
-__device__ __forceinline__ void stamp(uint64_t *row, uint32_t k) {
-    if (row && threadIdx.x == 0) row[k] = wall_clock64();
+__device__ __forceinline__ void stamp(uint64_t *row, uint32_t k, uint32_t wave) {
+    if (row && fresh(wave) == 0 && lane_id() == 0) row[k] = wall_clock64();
 }
 
 // ---- memory seen through buffer descriptors ------------------------------------------------------------------------------
@@ -128,7 +150,7 @@ __device__ __forceinline__ void flow_backoff(Flow &f, uint64_t &deadline, uint32
     if (deadline == 0) deadline = now + FLOW_WAIT_TICKS;
     if (now > deadline) {
         f.dead = true;
-        if ((phase_tid() & 63) == 0) __hip_atomic_store(f.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane_id() == 0) __hip_atomic_store(f.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else if ((rounds & 63u) == 0 && __hip_atomic_load(f.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
         f.dead = true;
     }
@@ -165,6 +187,56 @@ __device__ __forceinline__ void flow_take_strided(Rsrc x, uint32_t first, float 
     }
 }
 
+// ---- weights on their way ---------------------------------------------------------------------------------------------------
+// A phase's multiply cannot start before its input exists, but its weights do not depend on anything: each wave asks
+// for the unit of its NEXT phase as soon as the registers of the current one are free (right after its dot product,
+// before the partial sums are reduced and handed over), so the weights travel while the hand-off is waited for.
+struct Unit {                 // the 16-byte pieces a wave requested ahead (which ones depends on the block format)
+    U4 a[13], b[9];           // first matrix / second matrix of a gated pair
+    uint16_t ta;              // 2-byte tail of the first matrix (Q6_K)
+};
+struct Req {                  // where the wave's unit lies: kept from the request to the multiply, which asks for the rest
+    Rsrc rs[2];
+    uint32_t voff, toff;
+};
+// Every piece (and the tail) of a single matrix's unit: the block format only decides how many pieces there are, so the
+// request needs no code per format (the registers of a Unit hold the largest).
+// (The fences keep the requests where they are written: moved up into the multiply before them, they would need its
+// registers as well.)
+__device__ __forceinline__ void request_fence() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+__device__ __forceinline__ void request_all(Unit &u, const Req &r, int type) {
+    const uint32_t pt = tiled_pieces(type);
+    request_fence();
+    u = Unit{};                                                  // (nothing of an earlier unit stays alive in the registers)
+#pragma unroll
+    for (int P = 0; P < 13; ++P) {
+        if ((uint32_t)P < pt) {
+            const u32x4b v = __builtin_amdgcn_raw_buffer_load_b128(r.rs[0], (int)r.voff, P * 1024, AUX_PLAIN);
+            u.a[P] = U4{v.x, v.y, v.z, v.w};
+        }
+    }
+    if (tiled_tail(type)) u.ta = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r.rs[0], (int)r.toff, 0, AUX_PLAIN);
+    request_fence();
+}
+// A gated pair of Q4_K matrices: the header and the first GATED_LEAD stages of both (8: everything); the multiply asks
+// for the rest.
+constexpr int GATED_LEAD = 8;
+__device__ __forceinline__ void request_gated(Unit &u, const Req &r) {
+    u = Unit{};
+    request_fence();
+#pragma unroll
+    for (int P = 0; P <= GATED_LEAD; ++P) {
+        const u32x4b v = __builtin_amdgcn_raw_buffer_load_b128(r.rs[0], (int)r.voff, P * 1024, AUX_PLAIN);
+        const u32x4b w = __builtin_amdgcn_raw_buffer_load_b128(r.rs[1], (int)r.voff, P * 1024, AUX_PLAIN);
+        u.a[P] = U4{v.x, v.y, v.z, v.w};
+        u.b[P] = U4{w.x, w.y, w.z, w.w};
+    }
+    request_fence();
+}
+
 // ---- a unit of up to 64 rows of a 64-row-tile matrix (q / k / v, gate + up, output matrix) -------------------------------
 struct TileIn {
     Rsrc x;                   // the input vector (n floats)
@@ -174,56 +246,50 @@ struct TileIn {
     float eps;
 };
 
-// One unit: rows unit.row0 .. + unit.nrows - 1 of W (and W2) times the RMS-normalised input; returns, in threads
-// 0 .. nrows - 1, the finished value of row unit.row0 + thread (scaled; gate/up combined with SiLU when DUAL).
-// Wave w owns super-block w and is on its own until the partial sums meet: it requests its weights, then waits for the
-// 256 input values of its super-block (one 16-byte piece per lane), leaves x * w and the sums of 16 in its part of the
-// workgroup's slot (rms_norm.slang:48-67; the scale is applied to the finished dot product) and reads them back as
-// scalar operands.  `stage`: false when the slot still holds this input.
-// smem: partial[2][16][64], red[2][16] (red alternates between calls so that a fast wave cannot overwrite it early).
+// Rows unit.row0 .. + unit.nrows - 1 of W (and W2), super-block `wave`: lane i owns row unit.row0 + i (lanes past the
+// unit repeat its last row and their results are dropped).
+template <bool DUAL>
+__device__ __forceinline__ void request64(Unit &u, Req &r, const DevBuf &W, const DevBuf &W2, const plan::RowUnit unit, uint32_t ncb, uint32_t wave_) {
+    const uint32_t lane = lane_id(), wave = fresh(wave_);
+    if (wave >= ncb) { u = Unit{}; return; }
+    const uint32_t unit_bytes = plan::unit_bytes_of(W.type);
+    const uint32_t row = plan::unit_row(unit, lane);
+    r.rs[0] = W.rs; r.rs[1] = W2.rs;
+    r.voff = plan::tile64_piece0(row, wave, ncb, unit_bytes);
+    r.toff = plan::tile64_tail(row, wave, ncb, unit_bytes, tiled_pieces(W.type));
+    if constexpr (DUAL) request_gated(u, r);
+    else request_all(u, r, W.type);
+}
+
+// The multiply of a requested unit: wave w waits for the 256 input values of super-block w (one 16-byte piece per lane),
+// leaves x * w and the sums of 16 in its part of the workgroup's slot (rms_norm.slang:48-67; the scale is applied to the
+// finished dot product), reads them back as scalar operands, multiplies, and leaves its partial sums in LDS.  `stage`:
+// false when the slot still holds this input.  partial[2][16][64], red[16].
 template <int T, bool DUAL>
-__device__ __forceinline__ float tile64_phase(const DevBuf &W, const DevBuf &W2, const plan::RowUnit unit, uint32_t ncb, const TileIn &in, bool stage,
-                                              float *slot, float *partial, float *red, Flow &f, uint64_t *tr) {
+__device__ __forceinline__ void mult64(const Unit &u, const Req &r, uint32_t ncb, const TileIn &in, bool stage, float *slot, float *partial, float *red, Flow &f,
+                                       uint64_t *tr, const uint32_t wave_) {
     using F = Tiled<T>;
-    const int tid = phase_tid(), lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    constexpr uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
+    const int lane = (int)lane_id();
+    const uint32_t wave = fresh(wave_);
     constexpr int NM = DUAL ? 2 : 1;
-    const bool has_unit = (uint32_t)wave < ncb;
     float v = 0.0f, v2 = 0.0f;
-    stamp(tr, 0);
-    if (has_unit) {
-        typename F::Data d, e;
-        uint16_t dt = 0, et = 0;
-        // As much of the unit as the registers hold without spilling is requested before the wait; the rest follows
-        // while the first stages are multiplied.
-        BufUnitLoader<T, NM, DUAL ? 4 : (F::PT > 9 ? 6 : 8)> ld;
-        {
-            const uint32_t row = unit.row0 + plan::umin((uint32_t)lane, unit.nrows - 1);     // lanes past the unit repeat its last row
-            const uint32_t voff = plan::tile64_piece0(row, (uint32_t)wave, ncb, unit_bytes);
-            const uint32_t toff = plan::tile64_tail(row, (uint32_t)wave, ncb, unit_bytes, F::PT);
-            ld.rs[0] = W.rs; ld.voff[0] = voff; ld.toff[0] = toff; ld.d[0] = &d; ld.t[0] = &dt;
-            if constexpr (DUAL) { ld.rs[1] = W2.rs; ld.voff[1] = voff; ld.toff[1] = toff; ld.d[1] = &e; ld.t[1] = &et; }
-            F::lead(ld);
-        }
+    if ((uint32_t)wave < ncb) {
         if (stage) {
             const uint32_t piece = plan::wave_piece((uint32_t)wave, (uint32_t)lane);
             const float4 w = as_float4(buf_load16<AUX_PLAIN>(in.norm_w, piece * 16u));
-            // (loads retire in issue order: the first answer comes after the weights requested above, which have
-            // had the whole previous phase to travel)
             float4 x = as_float4(in.flow ? flow_take(in.x, piece, f) : buf_load16<AUX_PLAIN>(in.x, piece * 16u));
             float ss = fmaf(x.x, x.x, fmaf(x.y, x.y, fmaf(x.z, x.z, x.w * x.w)));
-            ss = wave_sum(ss);
+            ss = wave_total(ss);
             if (lane == 0) red[wave] = ss;
             x.x *= w.x; x.y *= w.y; x.z *= w.z; x.w *= w.w;
             float s4 = (x.x + x.y) + (x.z + x.w);
-            s4 += __shfl_xor(s4, 1, 64);
-            s4 += __shfl_xor(s4, 2, 64);                               // lanes 4q..4q+3 hold 16 consecutive activations
+            s4 += lane_xor(s4, 1);
+            s4 += lane_xor(s4, 2);                                     // lanes 4q..4q+3 hold 16 consecutive activations
             *reinterpret_cast<float4 *>(slot + 4 * piece) = x;
             if ((lane & 3) == 0) slot[in.n + (piece >> 2)] = s4;
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // the wave's part of the slot is in L2
         }
-        stamp(tr, 1);
+        stamp(tr, 1, wave);
         // The slot was rewritten with vector stores; the scalar cache may still hold what it held before.  Drop that,
         // and hand the compiler the pointer only now: loads through the constant address space move freely otherwise.
         asm volatile("s_dcache_inv\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
@@ -231,25 +297,47 @@ __device__ __forceinline__ float tile64_phase(const DevBuf &W, const DevBuf &W2,
         asm volatile("" : "+s"(slot_bits) : : "memory");
         cfloat *xsc = (cfloat *)slot_bits;
         ScalarX X{xsc + plan::slot_x((uint32_t)wave), xsc + in.n + (size_t)wave * 16};
+        typename F::Data d, e;
+#pragma unroll
+        for (int i = 0; i < F::PT; ++i) d.p[i] = u.a[i];
+        if constexpr (DUAL) {
+#pragma unroll
+            for (int i = 0; i < F::PT; ++i) e.p[i] = u.b[i];
+        }
+        uint16_t dt = u.ta, et = 0;
         const typename F::Data *dp[NM];
         uint16_t tails[NM];
         float o2[NM];
         dp[0] = &d; tails[0] = dt;
-        if constexpr (DUAL) { dp[1] = &e; tails[1] = et; }
-        F::template dotn<NM>(dp, tails, X, o2, ld);
+        if constexpr (DUAL) {
+            dp[1] = &e; tails[1] = et;
+            BufUnitLoader<T, 2, GATED_LEAD> ld;                        // asks for the pieces that were not requested ahead
+            ld.rs[0] = r.rs[0]; ld.voff[0] = r.voff; ld.toff[0] = r.toff; ld.d[0] = &d; ld.t[0] = &dt;
+            ld.rs[1] = r.rs[1]; ld.voff[1] = r.voff; ld.toff[1] = r.toff; ld.d[1] = &e; ld.t[1] = &et;
+            F::template dotn<2>(dp, tails, X, o2, ld);
+        } else {
+            F::template dotn<1>(dp, tails, X, o2);                   // the whole unit was requested ahead
+        }
         v = o2[0];
         if constexpr (DUAL) v2 = o2[1];
     }
-    stamp(tr, 2);
+    stamp(tr, 2, wave);
     partial[wave * 64 + lane] = v;
     if constexpr (DUAL) partial[(PNW + wave) * 64 + lane] = v2;
+}
+
+// After the barrier: thread i < 64 of the workgroup adds up row i of the unit (scaled; gate / up combined with SiLU).
+template <bool DUAL>
+__device__ __forceinline__ float finish64(uint32_t ncb, const TileIn &in, const float *partial, const float *red, uint64_t *tr, uint32_t wave_) {
+    const uint32_t wave = fresh(wave_);
     lds_barrier();
-    stamp(tr, 3);
+    stamp(tr, 3, wave);
+    const int tid = (int)(wave * 64u + lane_id());
     float o = 0.0f;
     if (tid < 64) {
         float t = 0.0f;
         for (uint32_t w = 0; w < ncb; ++w) { t += red[w]; o += partial[w * 64 + tid]; }
-        const float scale = 1.0f / sqrtf(t / (float)in.n + in.eps);
+        const float scale = 1.0f / sqrtf(t / (float)fresh(in.n) + in.eps);
         o *= scale;
         if constexpr (DUAL) {
             float up = 0.0f;
@@ -261,33 +349,43 @@ __device__ __forceinline__ float tile64_phase(const DevBuf &W, const DevBuf &W2,
     return o;
 }
 
-// ---- a 16-row tile (attention output projection, down projection) -------------------------------------------------------
-// Rows tile*16 .. +15 of W times the n-vector `x` (written by this launch); returns the row's dot product in threads
-// 0..15.  Waves 0 .. ngroups-1 multiply (one unit of 16 rows x 4 super-blocks each): each requests its weights, then
-// waits for the 1024 input values of its four super-blocks, 16 per lane, straight into the registers they are used from.
+// ---- 16-row tiles (attention output projection, down projection) ---------------------------------------------------------
+// Rows tile*16 .. +15 of W times an n-vector written by this launch, plus the residual.  A tile takes `ngroups` waves (one
+// unit of 16 rows x 4 super-blocks each); a workgroup runs up to two tiles side by side (plan::Tiles16): waves
+// k * ngroups .. (k + 1) * ngroups - 1 multiply tile k.  Each wave waits for the 1024 input values of its four
+// super-blocks, 16 per lane, straight into the registers they are used from.
+__device__ __forceinline__ void request16(Unit &u, Req &r, const DevBuf &W, const plan::Tiles16 t, uint32_t ngroups, uint32_t wave_) {
+    const uint32_t lane = lane_id(), wave = fresh(wave_);
+    if (wave >= ngroups * t.n) { u = Unit{}; return; }
+    const uint32_t unit_bytes = plan::unit_bytes_of(W.type);
+    const uint32_t k = wave / ngroups, g = wave - k * ngroups;
+    r.rs[0] = W.rs; r.rs[1] = W.rs;
+    r.voff = plan::tile16_piece0(plan::tiles16_tile(t, k), g, ngroups, unit_bytes, lane);
+    r.toff = plan::tile16_tail(plan::tiles16_tile(t, k), g, ngroups, unit_bytes, tiled_pieces(W.type), lane);
+    request_all(u, r, W.type);
+}
+// `res`: the vector the result is added to (complete long before this phase).  Thread i < 16 * t.n receives, in `residual`,
+// element 16 * tile + i % 16 of it: asked for first, so that it is there when the reduction needs it.
 template <int T>
-__device__ __forceinline__ float tile16_phase(const DevBuf &W, uint32_t tile, uint32_t ncb, uint32_t ngroups, Rsrc x, float *partial, Flow &f, uint64_t *tr) {
+__device__ __forceinline__ void mult16(const Unit &u, const plan::Tiles16 t, uint32_t ncb, uint32_t ngroups, Rsrc x, Rsrc res, bool res_flow, float &residual, float *partial,
+                                       Flow &f, uint64_t *tr, const uint32_t wave_) {
     using F = Tiled<T>;
-    const int tid = phase_tid(), lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    constexpr uint32_t unit_bytes = F::PT * 1024 + (F::TAIL ? 128 : 0);
-    const bool has_unit = (uint32_t)wave < ngroups;
+    const int lane = (int)lane_id();
+    const uint32_t wave = fresh(wave_);
     float v = 0.0f;
-    stamp(tr, 0);
-    if (has_unit) {
-        typename F::Data d;
-        uint16_t dt = 0;
-        BufUnitLoader<T, 1, (F::PT > 9 ? 6 : 8)> ld;
-        ld.rs[0] = W.rs; ld.d[0] = &d; ld.t[0] = &dt;
-        ld.voff[0] = plan::tile16_piece0(tile, (uint32_t)wave, ngroups, unit_bytes, (uint32_t)lane);
-        ld.toff[0] = plan::tile16_tail(tile, (uint32_t)wave, ngroups, unit_bytes, F::PT, (uint32_t)lane);
-        F::lead(ld);
-        const bool valid = plan::tile16_cb((uint32_t)wave, (uint32_t)lane) < ncb;
+    residual = 0.0f;
+    if (wave == 0 && (uint32_t)lane < 16u * t.n) {
+        const uint32_t off = (plan::tiles16_row(t, (uint32_t)lane)) * 4u;
+        residual = __uint_as_float(res_flow ? __builtin_amdgcn_raw_buffer_load_b32(res, (int)off, 0, AUX_FLOW) : __builtin_amdgcn_raw_buffer_load_b32(res, (int)off, 0, AUX_PLAIN));
+    }
+    if (wave < ngroups * t.n) {
+        const uint32_t g = wave % ngroups;
+        const bool valid = plan::tile16_cb(g, (uint32_t)lane) < ncb;
         DevX X;
-        flow_take_strided(x, plan::tile16_x0((uint32_t)wave, (uint32_t)lane, ncb), X.x, f);
+        flow_take_strided(x, plan::tile16_x0(g, (uint32_t)lane, ncb), X.x, f);
 #pragma unroll
         for (int i = 0; i < 16; ++i) X.x[i] = valid ? X.x[i] : 0.0f;
-        stamp(tr, 1);
+        stamp(tr, 1, wave);
         if constexpr (T == T_Q6_K) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) X.s[i] = row16_sum(X.x[i]);
@@ -295,36 +393,49 @@ __device__ __forceinline__ float tile16_phase(const DevBuf &W, uint32_t tile, ui
 #pragma unroll
             for (int i = 0; i < 16; i += 2) { X.s[i] = row16_sum(X.x[i] + X.x[i + 1]); X.s[i + 1] = 0.0f; }
         }
+        typename F::Data d;
+#pragma unroll
+        for (int i = 0; i < F::PT; ++i) d.p[i] = u.a[i];
+        uint16_t dt = u.ta;
         const typename F::Data *dp[1] = {&d};
         uint16_t tails[1] = {dt};
         float o1[1];
-        F::template dotn<1>(dp, tails, X, o1, ld);
+        F::template dotn<1>(dp, tails, X, o1);                       // the whole unit was requested ahead
         v = o1[0];
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);                                // across the four super-blocks of the wave
+        v += lane_xor(v, 16);
+        v += lane_xor(v, 32);                                      // across the four super-blocks of the wave
     }
-    stamp(tr, 2);
+    stamp(tr, 2, wave);
     if (lane < 16) partial[wave * 64 + lane] = v;
+}
+// After the barrier: thread i < 16 * t.n holds the dot product of row plan::tiles16_row(t, i).
+__device__ __forceinline__ float finish16(const plan::Tiles16 t, uint32_t ngroups, const float *partial, uint64_t *tr, uint32_t wave_) {
+    const uint32_t wave = fresh(wave_);
     lds_barrier();
-    stamp(tr, 3);
+    stamp(tr, 3, wave);
+    const uint32_t tid = wave * 64u + lane_id();
     float o = 0.0f;
-    if (tid < 16)
-        for (uint32_t w = 0; w < ngroups; ++w) o += partial[w * 64 + tid];
+    if (tid < 16u * t.n) {
+        const uint32_t k = tid >> 4, j = tid & 15u;
+        for (uint32_t w = 0; w < ngroups; ++w) o += partial[(k * ngroups + w) * 64 + j];
+    }
     return o;
 }
 
+// the block format is uniform over the workgroup
 template <bool DUAL>
-__device__ __forceinline__ float tile64_any(const DevBuf &W, const DevBuf &W2, const plan::RowUnit unit, uint32_t ncb, const TileIn &in, bool stage,
-                                            float *slot, float *partial, float *red, Flow &f, uint64_t *tr) {
-    switch (W.type) {                                              // uniform over the workgroup
-    case T_Q6_K: if constexpr (!DUAL) return tile64_phase<T_Q6_K, false>(W, W2, unit, ncb, in, stage, slot, partial, red, f, tr); else return 0.0f;
-    case T_Q5_K: if constexpr (!DUAL) return tile64_phase<T_Q5_K, false>(W, W2, unit, ncb, in, stage, slot, partial, red, f, tr); else return 0.0f;
-    default: return tile64_phase<T_Q4_K, DUAL>(W, W2, unit, ncb, in, stage, slot, partial, red, f, tr);
+__device__ __forceinline__ void mult64_any(int type, const Unit &u, const Req &r, uint32_t ncb, const TileIn &in, bool stage, float *slot, float *partial, float *red,
+                                           Flow &f, uint64_t *tr, uint32_t wave) {
+    switch (type) {
+    case T_Q6_K: if constexpr (!DUAL) mult64<T_Q6_K, false>(u, r, ncb, in, stage, slot, partial, red, f, tr, wave); break;
+    case T_Q5_K: if constexpr (!DUAL) mult64<T_Q5_K, false>(u, r, ncb, in, stage, slot, partial, red, f, tr, wave); break;
+    default: mult64<T_Q4_K, DUAL>(u, r, ncb, in, stage, slot, partial, red, f, tr, wave); break;
     }
 }
-__device__ __forceinline__ float tile16_any(const DevBuf &W, uint32_t tile, uint32_t ncb, uint32_t ngroups, Rsrc x, float *partial, Flow &f, uint64_t *tr) {
-    if (W.type == T_Q6_K) return tile16_phase<T_Q6_K>(W, tile, ncb, ngroups, x, partial, f, tr);
-    return tile16_phase<T_Q4_K>(W, tile, ncb, ngroups, x, partial, f, tr);
+__device__ __forceinline__ void mult16_any(int type, const Unit &u, const plan::Tiles16 t, uint32_t ncb, uint32_t ngroups, Rsrc x, Rsrc res, bool res_flow, float &residual,
+                                           float *partial, Flow &f, uint64_t *tr, uint32_t wave) {
+    if (type == T_Q6_K) mult16<T_Q6_K>(u, t, ncb, ngroups, x, res, res_flow, residual, partial, f, tr, wave);
+    else mult16<T_Q4_K>(u, t, ncb, ngroups, x, res, res_flow, residual, partial, f, tr, wave);
 }
 
 __device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
@@ -332,69 +443,77 @@ __device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------------------------------
-// Workgroup roles: resident_plan.h (plan::qkv_unit, attention_head, gu_unit, proj_tiles, out_tiles).
-template <bool F16>
-__global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const PersistentParams p) {
-    extern __shared__ __align__(16) float smem[];
-    __shared__ uint32_t wg_dead;                                   // the attention hand-off of this workgroup timed out
-    // The description of the current layer and of the next one.  Read from memory at the moment of use, its lines (which
-    // the weight stream has long pushed out of L2) would cost a round trip to memory each, one after the other.
+// Workgroup roles: resident_plan.h (plan::qkv_unit, attention_head, gu_unit, proj_tiles, out_tiles).  The body exists
+// twice, for the workgroups that run a head's attention in the first phase of a layer (ATTN) and for those that multiply
+// a q / k / v unit there (or nothing): the attention needs nearly all registers, and only a body of its own shows the
+// compiler that no unit requested ahead is ever alive across it.
+template <bool F16, bool ATTN>
+__device__ __forceinline__ void decode_token(const PersistentParams &p, float *smem, uint32_t &wg_dead, uint32_t (&layer_words)[2][sizeof(PersistentLayer) / 4],
+                                             const uint32_t wave) {
     constexpr int LWORDS = sizeof(PersistentLayer) / 4;
-    static_assert(LWORDS <= PNT && sizeof(PersistentLayer) == 14 * sizeof(ResidentBuf), "one thread per word; fourteen entries");
-    __shared__ uint32_t layer_words[2][LWORDS];
     // Two sets of partial[2][16][64] | red[16], taken in turn by the phases of this workgroup: a wave that is done with a
     // phase goes on to the next one (there is one barrier per phase, before its reduction) while wave 0 may still be
     // reducing the one before, but it cannot get further ahead than that.
     float *const lds_sets = smem;
 #define PHASE_PARTIAL (lds_sets + plan::lds_set(phase & 1u) + plan::lds_partial())
 #define PHASE_RED (lds_sets + plan::lds_set(phase & 1u) + plan::lds_red())
-    touch_kernel_arguments<sizeof(PersistentParams)>();
     const uint32_t b = blockIdx.x;
-    // A launch after one in which a reader gave up does nothing: the host has not looked yet (it queues many tokens), and
-    // every further token would only wait out the same time limits.
-    if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
     Flow f{p.abort_flag, false};
     const plan::Shape sh = shape_of(p);
     const uint32_t dim = p.dim, hid = p.hidden, nh = p.n_heads;
     const uint32_t ncb = dim / 256, ncb_h = hid / 256, ng_o = ncb / 4, ng_d = (ncb_h + 3) / 4;
     float *slot = p.slots + plan::slot_of(sh, b);
-    // time stamps: 16 per layer (4 per phase: entered, input staged, multiplied, reduced), then 4 for the output matrix and the end
+    // time stamps: 16 per layer (4 per phase: entered, input there, multiplied, reduced), then 4 for the output matrix and the end
     uint64_t *trace = p.trace ? p.trace + plan::trace_row(sh, b) : nullptr;
     uint32_t phase = 0;                                            // phases this workgroup has run: parity picks the LDS set
-    // the residual value of row 16b + tid: the embedding row the launch before this one left in p.x
-    float xres = 0.0f;
-    if (b < plan::proj_tiles(sh) && threadIdx.x < 16) xres = p.x[16 * b + threadIdx.x];
-    if (threadIdx.x == 0) wg_dead = 0;
-    if (threadIdx.x < LWORDS) layer_words[0][threadIdx.x] = reinterpret_cast<const uint32_t *>(p.layers)[threadIdx.x];
-    __syncthreads();
+    // Every workgroup has a role in every phase (plan::shape_ok: the grid is exactly the 16-row tiles of the projections
+    // = seven q / k / v units and one attention per head = the units of gate / up), so the request for the next phase's
+    // weights always has a place: right after the multiply of the phase before it.
+    const plan::RowUnit qkv_u = ATTN ? plan::run_unit(0u, 0u, 1u) : plan::qkv_unit(sh, b);
+    const plan::RowUnit gu_u = plan::gu_unit(sh, b);
+    const uint32_t ntiles_out = plan::out_tiles(sh);
+    const DevBuf wout = dev_buf(p.wout);
+    const plan::Tiles16 wo_t = plan::wo_tiles(sh, b), down_t = plan::down_tiles(sh, b);
+
+    Unit unit;                                                     // the weights requested ahead for this workgroup's next phase
+    Req req;
+    int unit_type = 0;                                             // its block format
+    const auto qkv_matrix = [&](const uint32_t *lw) { return qkv_u.seg == 0 ? LAYER_BUF(lw, wv) : (qkv_u.seg == 1 ? LAYER_BUF(lw, wk) : LAYER_BUF(lw, wq)); };
+    if constexpr (!ATTN) {
+        const DevBuf W = qkv_matrix(layer_words[0]);
+        request64<false>(unit, req, W, W, qkv_u, ncb, wave);
+        unit_type = W.type;
+    }
 
     for (uint32_t l = 0; l < p.n_layers; ++l) {
         // this layer's description comes out of LDS entry by entry, as wave-uniform values, where it is used; the next
-        // one's is requested now and parked in LDS at the end of the layer
+        // one's is requested now and parked in LDS after the first phase
         const uint32_t *lw = layer_words[l & 1u];
+        const bool last = l + 1 == p.n_layers;
         uint32_t next_word = 0;
-        if (threadIdx.x < LWORDS && l + 1 < p.n_layers) next_word = reinterpret_cast<const uint32_t *>(p.layers + l + 1)[threadIdx.x];
+        if (wave == 0 && lane_id() < LWORDS && !last) next_word = reinterpret_cast<const uint32_t *>(p.layers + l + 1)[lane_id()];
         uint64_t *tl = trace ? trace + 16 * l : nullptr;
         // the hand-off vectors of this layer, each behind a descriptor of its own size
         const Rsrc xa = make_rsrc(p.flow + plan::flow_xa(sh, l), dim * 4u), xb = make_rsrc(p.flow + plan::flow_xb(sh, l), dim * 4u);
         const Rsrc xm = make_rsrc(p.flow + plan::flow_xm(sh, l), dim * 4u), hb = make_rsrc(p.flow + plan::flow_hb(sh, l), hid * 4u);
         const Rsrc xnext = make_rsrc(p.flow + plan::flow_xa(sh, l + 1), dim * 4u);
-        // ---- q / k / v and the attention ---------------------------------------------------------------------------
-        if (b < plan::qkv_workgroups(sh)) {
-            const plan::RowUnit u = plan::qkv_unit(sh, b);
+        // ---- q / k / v, or the attention ------------------------------------------------------------------------------
+        if constexpr (!ATTN) {
             const uint32_t h = plan::qkv_head(sh, b);
-            const DevBuf W = u.seg == 0 ? LAYER_BUF(lw, wv) : (u.seg == 1 ? LAYER_BUF(lw, wk) : LAYER_BUF(lw, wq));
-            float *out = u.seg == 0 ? p.vcol : (u.seg == 1 ? p.kcol : p.q);
+            float *out = qkv_u.seg == 0 ? p.vcol : (qkv_u.seg == 1 ? p.kcol : p.q);
             const TileIn in{l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, LAYER_BUF(lw, attn_norm).rs, dim, p.eps};
-            const float o = tile64_any<false>(W, W, u, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tl);
-            const uint32_t tid = phase_tid();
+            stamp(tl, 0, wave);
+            mult64_any<false>(unit_type, unit, req, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tl, wave);
+            { const DevBuf W = LAYER_BUF(lw, wo); request16(unit, req, W, wo_t, ng_o, wave); unit_type = W.type; }
+            const float o = finish64<false>(ncb, in, PHASE_PARTIAL, PHASE_RED, tl, wave);
+            const uint32_t tid = wave * 64u + lane_id();
             if (tid < 64) {
-                if (tid < u.nrows) flow_store(out + u.row0 + tid, o);
+                if (tid < qkv_u.nrows) flow_store(out + plan::unit_row(qkv_u, tid), o);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 if (tid == 0) __hip_atomic_fetch_add(p.counters + plan::counter_word(h), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
             ++phase;
-        } else if (plan::is_attention_workgroup(sh, b)) {
+        } else {
             const uint32_t h = plan::attention_head(sh, b);
             AttnLaunch a{};
             a.q = p.q; a.knew = p.kcol; a.vnew = p.vcol;
@@ -406,8 +525,8 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
             a.out = p.flow + plan::flow_xb(sh, l); a.scratch = nullptr; a.n_splits = 1;
             uint32_t *counter = p.counters + plan::counter_word(h);
             const uint32_t need = p.qkv_units;
-            const uint32_t tid = phase_tid();
-            stamp(tl, 0);
+            const uint32_t tid = wave * 64u + lane_id();
+            stamp(tl, 0, wave);
             attn::attn_fast_body<F16, PNT, 128, true, true, 8, true>(a, h, 0u, tid, [&]() {
                 if (tid == 0) {
                     uint32_t seen = 0, spins = 0;
@@ -432,51 +551,101 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
                 asm volatile("" ::: "memory");
             });
             if (wg_dead) f.dead = true;
-            stamp(tl, 3);
+            stamp(tl, 3, wave);
+            // (only now: the attention needs the registers; these workgroups have no tile of the output projection)
+            { const DevBuf W = LAYER_BUF(lw, wgate); request64<true>(unit, req, W, LAYER_BUF(lw, wup), gu_u, ncb, wave); unit_type = W.type; }
         }
-        // ---- attention output projection into the residual ---------------------------------------------------------
-        if (b < plan::proj_tiles(sh)) {
-            const float o = tile16_any(LAYER_BUF(lw, wo), b, ncb, ng_o, xb, PHASE_PARTIAL, f, tl ? tl + 4 : nullptr);
-            const uint32_t tid = phase_tid();
-            if (tid < 16) { xres += o; flow_put(xm, 16 * b + tid, xres); }             // transformer.rs:352-355
+        // The next layer's description has arrived by now; nobody reads the slot it goes to any more (the layer before
+        // this one is over for every wave that got here), and a phase barrier lies between this and its first reader.
+        if (wave == 0 && lane_id() < LWORDS && !last) layer_words[(l + 1) & 1u][lane_id()] = next_word;
+        // ---- attention output projection into the residual (the workgroups that multiplied q / k / v) ------------------
+        if constexpr (!ATTN) {
+            uint64_t *tp = tl ? tl + 4 : nullptr;
+            float residual;
+            stamp(tp, 0, wave);
+            mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, PHASE_PARTIAL, f, tp, wave);
+            { const DevBuf W = LAYER_BUF(lw, wgate); request64<true>(unit, req, W, LAYER_BUF(lw, wup), gu_u, ncb, wave); unit_type = W.type; }
+            const float o = finish16(wo_t, ng_o, PHASE_PARTIAL, tp, wave);
+            const uint32_t tid = wave * 64u + lane_id();
+            if (tid < 16u * wo_t.n) flow_put(xm, plan::tiles16_row(wo_t, tid), residual + o);     // transformer.rs:352-355
             ++phase;
         }
         // ---- RMSNorm + gate / up + SiLU ---------------------------------------------------------------------------------
-        if (b < plan::gu_units(sh)) {
-            const plan::RowUnit u = plan::gu_unit(sh, b);
+        {
+            uint64_t *tp = tl ? tl + 8 : nullptr;
             const TileIn in{xm, true, LAYER_BUF(lw, ffn_norm).rs, dim, p.eps};
-            const float o = tile64_any<true>(LAYER_BUF(lw, wgate), LAYER_BUF(lw, wup), u, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tl ? tl + 8 : nullptr);
-            const uint32_t tid = phase_tid();
-            if (tid < u.nrows) flow_put(hb, u.row0 + tid, o);
+            stamp(tp, 0, wave);
+            mult64_any<true>(unit_type, unit, req, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tp, wave);
+            { const DevBuf W = LAYER_BUF(lw, wdown); request16(unit, req, W, down_t, ng_d, wave); unit_type = W.type; }
+            const float o = finish64<true>(ncb, in, PHASE_PARTIAL, PHASE_RED, tp, wave);
+            const uint32_t tid = wave * 64u + lane_id();
+            if (tid < gu_u.nrows) flow_put(hb, gu_u.row0 + tid, o);
             ++phase;
         }
         // ---- down projection into the residual ----------------------------------------------------------------------------
-        if (b < plan::proj_tiles(sh)) {
-            const float o = tile16_any(LAYER_BUF(lw, wdown), b, ncb_h, ng_d, hb, PHASE_PARTIAL, f, tl ? tl + 12 : nullptr);
-            const uint32_t tid = phase_tid();
-            if (tid < 16) { xres += o; flow_put(xnext, 16 * b + tid, xres); }          // transformer.rs:362-365
+        {
+            uint64_t *tp = tl ? tl + 12 : nullptr;
+            float residual;
+            stamp(tp, 0, wave);
+            mult16_any(unit_type, unit, down_t, ncb_h, ng_d, hb, xm, true, residual, PHASE_PARTIAL, f, tp, wave);
+            // what this workgroup multiplies next: its q / k / v unit of the next layer, or its first tile of the output matrix
+            if (last) {
+                if (b < ntiles_out) request64<false>(unit, req, wout, wout, plan::run_unit(0u, b * 64u, plan::umin(64u, p.vocab - b * 64u)), ncb, wave);
+                unit_type = wout.type;
+            } else if constexpr (!ATTN) {
+                const DevBuf W = qkv_matrix(layer_words[(l + 1) & 1u]);
+                request64<false>(unit, req, W, W, qkv_u, ncb, wave);
+                unit_type = W.type;
+            }
+            const float o = finish16(down_t, ng_d, PHASE_PARTIAL, tp, wave);
+            const uint32_t tid = wave * 64u + lane_id();
+            if (tid < 16u * down_t.n) flow_put(xnext, plan::tiles16_row(down_t, tid), residual + o);    // transformer.rs:362-365
             ++phase;
         }
-        if (threadIdx.x < LWORDS) layer_words[(l + 1) & 1u][threadIdx.x] = next_word;
-        lds_barrier();
     }
     // ---- final RMSNorm and the output matrix: tiles b, b + grid, ... -------------------------------------------------------
     {
-        const uint32_t ntiles = plan::out_tiles(sh);
         const TileIn in{make_rsrc(p.flow + plan::flow_xa(sh, p.n_layers), dim * 4u), true, dev_buf(p.out_norm).rs, dim, p.eps};
-        const DevBuf wout = dev_buf(p.wout);
+        uint64_t *to = trace ? trace + 16 * p.n_layers : nullptr;
         bool first = true;
-        // (the input is staged once: its sums of squares stay in this set, and a barrier separates the tiles)
-        for (uint32_t tile = b; tile < ntiles; tile += gridDim.x) {
-            const plan::RowUnit u{0u, tile * 64u, plan::umin(64u, p.vocab - tile * 64u)};
-            const float o = tile64_any<false>(wout, wout, u, ncb, in, first, slot, PHASE_PARTIAL, PHASE_RED, f, first && trace ? trace + 16 * p.n_layers : nullptr);
-            const uint32_t tid = phase_tid();
+        // (the input is staged once: its sums of squares stay in this LDS set, and a barrier separates the tiles)
+        for (uint32_t tile = b; tile < ntiles_out; tile += gridDim.x) {
+            const plan::RowUnit u = plan::run_unit(0u, tile * 64u, plan::umin(64u, p.vocab - tile * 64u));
+            uint64_t *tp = first ? to : nullptr;
+            stamp(tp, 0, wave);
+            mult64_any<false>(wout.type, unit, req, ncb, in, first, slot, PHASE_PARTIAL, PHASE_RED, f, tp, wave);
+            const uint32_t next = tile + gridDim.x;
+            if (next < ntiles_out) request64<false>(unit, req, wout, wout, plan::run_unit(0u, next * 64u, plan::umin(64u, p.vocab - next * 64u)), ncb, wave);
+            const float o = finish64<false>(ncb, in, PHASE_PARTIAL, PHASE_RED, tp, wave);
+            const uint32_t tid = wave * 64u + lane_id();
             if (tid < u.nrows) p.logits[u.row0 + tid] = o;
             first = false;
             lds_barrier();                                         // partial[] is reused by the next tile
         }
-        stamp(trace ? trace + 16 * p.n_layers : nullptr, 4);
+        stamp(to, 4, wave);
     }
+}
+
+// The description of the current layer and of the next one is parked in LDS.  Read from memory at the moment of use, its
+// lines (which the weight stream has long pushed out of L2) would cost a round trip to memory each, one after the other.
+template <bool F16>
+__global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const PersistentParams p) {
+    extern __shared__ __align__(16) float smem[];
+    __shared__ uint32_t wg_dead;                                   // the attention hand-off of this workgroup timed out
+    constexpr int LWORDS = sizeof(PersistentLayer) / 4;
+    static_assert(LWORDS <= 64 && sizeof(PersistentLayer) == 14 * sizeof(ResidentBuf), "one thread per word; fourteen entries");
+    __shared__ uint32_t layer_words[2][LWORDS];
+    touch_kernel_arguments<sizeof(PersistentParams)>();
+    // A launch after one in which a reader gave up does nothing: the host has not looked yet (it queues many tokens), and
+    // every further token would only wait out the same time limits.
+    if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
+    if (threadIdx.x == 0) wg_dead = 0;
+    if (threadIdx.x < LWORDS) layer_words[0][threadIdx.x] = reinterpret_cast<const uint32_t *>(p.layers)[threadIdx.x];
+    __syncthreads();
+    const plan::Shape sh{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, gridDim.x, p.qkv_units, p.gu_rows};
+    const uint32_t wave = uniform_word(threadIdx.x >> 6);
+    if (plan::is_attention_workgroup(sh, blockIdx.x)) decode_token<F16, true>(p, smem, wg_dead, layer_words, wave);
+    else decode_token<F16, false>(p, smem, wg_dead, layer_words, wave);
 }
 
 #undef PHASE_PARTIAL

@@ -25,31 +25,30 @@ constexpr uint32_t WG_THREADS = 1024, WG_WAVES = 16;
 struct Shape {
     uint32_t dim, hidden, n_heads, n_layers, vocab, seq_len;
     uint32_t grid;            // workgroups of the launch (all resident)
-    uint32_t qkv_units;       // units per head in the q / k / v phase: 6 (two 64-row units per matrix) or 7 (v in three)
+    uint32_t qkv_units;       // units per head in the q / k / v phase: 7 (v in three, k and q in two each)
     uint32_t gu_rows;         // rows per unit of the gate / up phase, at most 64
+    uint32_t neox;            // rotary pairs are (i, i + 64) of a head (NeoX) instead of (2i, 2i + 1)
 };
 
 SLAI_HD uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
 SLAI_HD uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
 
-// The decomposition a launch of `grid` workgroups uses for a model: v in three units per head when the grid has room for
-// seven units and the attention workgroup of every head; gate / up rows spread evenly over the grid.
-SLAI_HD Shape make_shape(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32_t n_layers, uint32_t vocab, uint32_t seq_len, uint32_t grid) {
-    Shape s{dim, hidden, n_heads, n_layers, vocab, seq_len, grid, 6u, 64u};
-    if (8u * n_heads <= grid) s.qkv_units = 7;
-    s.gu_rows = umin(64u, umax(1u, (hidden + grid - 1) / grid));
+// The decomposition of a model: the grid is the number of 16-row tiles of the two projections into the residual (dim / 16
+// = 8 per head), which is also seven q / k / v units (v in three, k and q in two each) plus the attention workgroup of
+// every head, and the gate / up rows are spread evenly over it -- every workgroup has a role in every phase of a layer.
+SLAI_HD Shape make_shape(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32_t n_layers, uint32_t vocab, uint32_t seq_len, uint32_t neox = 0) {
+    Shape s{dim, hidden, n_heads, n_layers, vocab, seq_len, dim / 16u, 7u, 64u, neox};
+    s.gu_rows = s.grid ? umin(64u, umax(1u, (hidden + s.grid - 1) / s.grid)) : 0u;
     return s;
 }
 
 // ---- supported shapes: what the kernel's index arithmetic assumes -------------------------------------------------------
 SLAI_HD bool shape_ok(const Shape &s) {
     if (s.n_heads == 0 || s.n_heads % 8 || s.dim != s.n_heads * 128) return false;            // heads of 128, eight dies
-    if (s.dim % 1024 || s.dim > 4096) return false;                                            // one wave per super-block of the input
+    if (s.dim % 1024 || s.dim > 4096) return false;                                            // one wave per super-block of the input; two tiles of the output projection side by side
     if (s.hidden % 256 || s.hidden / 256 > 64) return false;                                   // sixteen waves x four super-blocks in the down projection
-    if (s.grid % 8 || s.grid > 1024) return false;
-    if ((s.qkv_units != 6 && s.qkv_units != 7) || (s.qkv_units + 1) * s.n_heads > s.grid) return false;
-    if (s.dim / 16 > s.grid) return false;                                                     // one 16-row tile of the projections each
-    if (s.gu_rows == 0 || s.gu_rows > 64 || (s.hidden + s.gu_rows - 1) / s.gu_rows > s.grid) return false;
+    if (s.grid != s.dim / 16 || s.qkv_units != 7 || (s.qkv_units + 1) * s.n_heads != s.grid) return false;   // a role for every workgroup in the first two phases
+    if (s.gu_rows == 0 || s.gu_rows > 64 || (s.hidden + s.gu_rows - 1) / s.gu_rows != s.grid) return false;  // ... and in gate / up
     if (s.seq_len == 0 || s.seq_len > 1024 || s.n_layers == 0 || s.vocab == 0) return false;
     return true;
 }
@@ -78,41 +77,68 @@ SLAI_HD uint32_t lds_set(uint32_t parity) { return parity * (lds_red() + WG_WAVE
 SLAI_HD uint32_t lds_floats(const Shape &) { return 2 * (lds_red() + WG_WAVES); }
 
 // ---- counters of the q / k / v -> attention hand-off: one 128-byte line per head, then the flag of a wait that gave up ---
-SLAI_HD uint32_t counter_word(uint32_t head) { return head * 32; }
+SLAI_HD uint32_t counter_word(uint32_t head, uint32_t which = 0) { return head * 32 + which; }
 
 // ---- time stamps: per workgroup 16 per layer (four per phase) and 8 for the output matrix -------------------------------
 SLAI_HD uint32_t trace_stride(const Shape &s) { return 16 * s.n_layers + 8; }
 SLAI_HD uint64_t trace_row(const Shape &s, uint32_t b) { return (uint64_t)b * trace_stride(s); }
 
 // ---- roles ----------------------------------------------------------------------------------------------------------------
-// A unit of a 64-row-unit phase: rows [row0, row0 + nrows) of matrix `seg`, nrows <= 64, lane i of every wave owns row
-// row0 + i (lanes past nrows repeat the last row and their results are dropped); wave w owns super-block w.
-struct RowUnit { uint32_t seg, row0, nrows; };
+// A unit of a 64-row-unit phase: up to 64 rows of matrix `seg`; lane i of every wave owns row unit_row(u, i) (lanes past
+// nrows repeat the last row and their results are dropped); wave w owns super-block w.  The rows are one run
+// [row0, row0 + nrows), or two: lanes below `split` take row0 + i, the others row1 + (i - split).
+struct RowUnit { uint32_t seg, row0, nrows, split, row1; };
+SLAI_HD RowUnit run_unit(uint32_t seg, uint32_t row0, uint32_t nrows) { return RowUnit{seg, row0, nrows, nrows, 0u}; }
+SLAI_HD uint32_t unit_row(const RowUnit &u, uint32_t lane) {
+    const uint32_t i = umin(lane, u.nrows - 1);
+    return i < u.split ? u.row0 + i : u.row1 + (i - u.split);
+}
 
-// q / k / v (segments 0: v, 1: k, 2: q): workgroup i < qkv_units * n_heads takes unit (i / 8) % qkv_units of head
-// (i % 8) + 8 * (i / (8 * qkv_units)), so that all units of a head, and the head's attention workgroup
-// qkv_workgroups + head, run on die i % 8 (their hand-off goes through that die's L2).
+// q / k / v (segments 0: v, 1: k, 2: q): workgroup i < 7 * n_heads takes unit (i / 8) % 7 of head (i % 8) + 8 * (i / 56),
+// so that all units of a head, and the head's attention workgroup qkv_workgroups + head, run on die i % 8 (their hand-off
+// goes through that die's L2).  v is cut into three runs of rows.  q and k are cut in two halves that hold complete rotary
+// pairs, because the workgroup that multiplies a unit also rotates it: rows 0..63 / 64..127 of the head for adjacent
+// pairs, rows {0..31, 64..95} / {32..63, 96..127} for NeoX pairs -- the partner of lane i is lane i ^ 1, or i ^ 32.
 SLAI_HD uint32_t qkv_workgroups(const Shape &s) { return s.qkv_units * s.n_heads; }
 SLAI_HD uint32_t qkv_head(const Shape &s, uint32_t b) { return (b & 7u) + 8u * ((b >> 3) / s.qkv_units); }
 SLAI_HD RowUnit qkv_unit(const Shape &s, uint32_t b) {
     const uint32_t t = (b >> 3) % s.qkv_units, head = qkv_head(s, b);
-    const uint32_t nv = s.qkv_units - 4;                      // units of v: 2 or 3; k and q two each
-    uint32_t seg, part, parts;
-    if (t < nv) { seg = 0; part = t; parts = nv; }
-    else if (t < nv + 2) { seg = 1; part = t - nv; parts = 2; }
-    else { seg = 2; part = t - nv - 2; parts = 2; }
-    const uint32_t lo = 128u * part / parts, hi = 128u * (part + 1) / parts;
-    return RowUnit{seg, head * 128u + lo, hi - lo};
+    const uint32_t nv = s.qkv_units - 4;                      // units of v: 3; k and q two each
+    if (t < nv) {
+        const uint32_t lo = 128u * t / nv, hi = 128u * (t + 1) / nv;
+        return run_unit(0u, head * 128u + lo, hi - lo);
+    }
+    const uint32_t seg = t < nv + 2 ? 1u : 2u, part = (t - nv) & 1u;
+    if (s.neox) return RowUnit{seg, head * 128u + 32u * part, 64u, 32u, head * 128u + 64u + 32u * part};
+    return run_unit(seg, head * 128u + 64u * part, 64u);
 }
+// which counter of the head a unit bumps when its rows are stored: 0 (q: the attention can start) or 1 (k and v: the
+// newest position can be added); and how many bumps the attention waits for
+SLAI_HD uint32_t qkv_counter(const RowUnit &u) { return u.seg == 2 ? 0u : 1u; }
+SLAI_HD uint32_t q_units(const Shape &) { return 2u; }
+SLAI_HD uint32_t kv_units(const Shape &s) { return s.qkv_units - 2u; }
 SLAI_HD bool is_attention_workgroup(const Shape &s, uint32_t b) { return b >= qkv_workgroups(s) && b < qkv_workgroups(s) + s.n_heads; }
 SLAI_HD uint32_t attention_head(const Shape &s, uint32_t b) { return b - qkv_workgroups(s); }
 
 // gate / up: workgroup b < gu_units takes rows [b * gu_rows, ...) of both matrices
 SLAI_HD uint32_t gu_units(const Shape &s) { return (s.hidden + s.gu_rows - 1) / s.gu_rows; }
-SLAI_HD RowUnit gu_unit(const Shape &s, uint32_t b) { return RowUnit{0u, b * s.gu_rows, umin(s.gu_rows, s.hidden - b * s.gu_rows)}; }
+SLAI_HD RowUnit gu_unit(const Shape &s, uint32_t b) { return run_unit(0u, b * s.gu_rows, umin(s.gu_rows, s.hidden - b * s.gu_rows)); }
 
-// the two projections into the residual: workgroup b < dim / 16 takes rows 16 b .. 16 b + 15 and keeps their residual
+// The two projections into the residual, in 16-row tiles (dim / 16 of them = the grid).  Down projection: workgroup b
+// takes tile b.  Attention output projection: the workgroups that run a head's attention have just finished when it
+// starts, so they take no tile; the q / k / v workgroup b takes tile b, and the one with a head's last q unit also the
+// tile 7 * n_heads + head, side by side on other waves.
+struct Tiles16 { uint32_t n, tile0, tile1; };      // (two named fields: an indexed pair would live in memory on the device)
+SLAI_HD uint32_t tiles16_tile(const Tiles16 &t, uint32_t k) { return k == 0 ? t.tile0 : t.tile1; }
 SLAI_HD uint32_t proj_tiles(const Shape &s) { return s.dim / 16; }
+SLAI_HD Tiles16 down_tiles(const Shape &, uint32_t b) { return Tiles16{1u, b, b}; }
+SLAI_HD Tiles16 wo_tiles(const Shape &s, uint32_t b) {
+    if (b >= qkv_workgroups(s)) return Tiles16{0u, 0u, 0u};
+    if ((b >> 3) % s.qkv_units == s.qkv_units - 1) return Tiles16{2u, b, qkv_workgroups(s) + qkv_head(s, b)};
+    return Tiles16{1u, b, b};
+}
+// the row thread i < 16 * t.n of the workgroup finishes
+SLAI_HD uint32_t tiles16_row(const Tiles16 &t, uint32_t i) { return 16u * tiles16_tile(t, (i >> 4) & 1u) + (i & 15u); }
 
 // output matrix: 64-row tiles b, b + grid, ...
 SLAI_HD uint32_t out_tiles(const Shape &s) { return (s.vocab + 63) / 64; }

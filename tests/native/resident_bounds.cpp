@@ -61,7 +61,7 @@ void walk_tile64(Audit &a, const Region &w, int type, const plan::RowUnit &u, ui
     for (uint32_t wave = 0; wave < plan::WG_WAVES; ++wave) {
         if (wave >= ncb) continue;
         for (uint32_t lane = 0; lane < 64; ++lane) {
-            const uint32_t row = u.row0 + plan::umin(lane, u.nrows - 1);
+            const uint32_t row = plan::unit_row(u, lane);
             const uint32_t voff = plan::tile64_piece0(row, wave, ncb, ub);
             for (uint32_t p = 0; p < pt; ++p) a.touch(w, (uint64_t)voff + p * 1024u, 16, "weight piece", b, wave, lane, layer);
             if (tiled_tail(type)) a.touch(w, plan::tile64_tail(row, wave, ncb, ub, pt), 2, "weight tail", b, wave, lane, layer);
@@ -69,8 +69,8 @@ void walk_tile64(Audit &a, const Region &w, int type, const plan::RowUnit &u, ui
     }
     if (row_count)
         for (uint32_t i = 0; i < u.nrows; ++i) {
-            if (u.row0 + i >= row_count->size()) { a.fail("a unit names a row past its matrix"); return; }
-            ++(*row_count)[u.row0 + i];
+            if (plan::unit_row(u, i) >= row_count->size()) { a.fail("a unit names a row past its matrix"); return; }
+            ++(*row_count)[plan::unit_row(u, i)];
         }
 }
 
@@ -100,28 +100,40 @@ void walk_stage64(Audit &a, const plan::Shape &s, const Region &x, const Region 
     if ((uint64_t)plan::lds_set(1) + plan::lds_red() + plan::WG_WAVES > plan::lds_floats(s) || ncb > plan::WG_WAVES) a.fail("LDS block smaller than what the phases index");
 }
 
-// a 16-row tile phase: weights of the multiplying waves and the sixteen floats of the n-vector each of their lanes takes
-void walk_tile16(Audit &a, const plan::Shape &s, const Region &w, int type, uint32_t tile, uint32_t ncb, uint32_t ngroups, const Region &x, uint32_t n, uint32_t b,
-                 uint32_t layer) {
-    (void)s;
+// a 16-row tile phase: the weights of the multiplying waves (tile k of the workgroup on waves k * ngroups ..), the sixteen
+// floats of the n-vector each of their lanes takes, the residual values and the rows written; `rows` counts the latter
+void walk_tile16(Audit &a, const Region &w, int type, const plan::Tiles16 &t, uint32_t ncb, uint32_t ngroups, const Region &x, uint32_t n, const Region &res,
+                 const Region &out, std::vector<uint32_t> &rows, uint32_t b, uint32_t layer) {
     const uint32_t ub = plan::unit_bytes_of(type), pt = tiled_pieces(type);
-    if (ngroups > plan::WG_WAVES) { a.fail("more column groups than waves"); return; }
-    std::vector<uint32_t> seen(n, 0);
-    for (uint32_t wave = 0; wave < ngroups; ++wave)
-        for (uint32_t lane = 0; lane < 64; ++lane) {
-            const uint32_t voff = plan::tile16_piece0(tile, wave, ngroups, ub, lane);
-            for (uint32_t p = 0; p < pt; ++p) a.touch(w, (uint64_t)voff + p * 1024u, 16, "weight piece (16-row tile)", b, wave, lane, layer);
-            if (tiled_tail(type)) a.touch(w, plan::tile16_tail(tile, wave, ngroups, ub, pt, lane), 2, "weight tail (16-row tile)", b, wave, lane, layer);
-            const uint32_t x0 = plan::tile16_x0(wave, lane, ncb);
-            const bool valid = plan::tile16_cb(wave, lane) < ncb;
-            for (uint32_t i = 0; i < 16; ++i) {
-                a.touch(x, ((uint64_t)x0 + 16 * i) * 4, 4, "input value (16-row tile)", b, wave, lane, layer);
-                if (valid && x0 + 16 * i < n && (lane & 15u) == (x0 & 15u) && lane < 64) ++seen[x0 + 16 * i];
+    if (t.n > 2 || ngroups * t.n > plan::WG_WAVES) { a.fail("more column groups than waves"); return; }
+    for (uint32_t k = 0; k < t.n; ++k) {
+        std::vector<uint32_t> seen(n, 0);
+        for (uint32_t wave = k * ngroups; wave < (k + 1) * ngroups; ++wave) {
+            const uint32_t g = wave % ngroups;
+            if (wave / ngroups != k) a.fail("wave to tile mapping");
+            for (uint32_t lane = 0; lane < 64; ++lane) {
+                const uint32_t voff = plan::tile16_piece0(plan::tiles16_tile(t, k), g, ngroups, ub, lane);
+                for (uint32_t p = 0; p < pt; ++p) a.touch(w, (uint64_t)voff + p * 1024u, 16, "weight piece (16-row tile)", b, wave, lane, layer);
+                if (tiled_tail(type)) a.touch(w, plan::tile16_tail(plan::tiles16_tile(t, k), g, ngroups, ub, pt, lane), 2, "weight tail (16-row tile)", b, wave, lane, layer);
+                const uint32_t x0 = plan::tile16_x0(g, lane, ncb);
+                const bool valid = plan::tile16_cb(g, lane) < ncb;
+                for (uint32_t i = 0; i < 16; ++i) {
+                    a.touch(x, ((uint64_t)x0 + 16 * i) * 4, 4, "input value (16-row tile)", b, wave, lane, layer);
+                    if (valid && x0 + 16 * i < n && lane < 16 * (64 / 16)) ++seen[x0 + 16 * i];
+                }
+                a.touch(out, 0, 0, "", b, wave, lane, layer);
             }
         }
-    // every value of the input reaches exactly the 16-lane rows that multiply its super-block: once per such row = once here
-    for (uint32_t i = 0; i < n; ++i)
-        if (seen[i] != 1) { a.fail("16-row-tile phase: input value " + std::to_string(i) + " is taken " + std::to_string(seen[i]) + " times"); break; }
+        // every value of the input reaches the 16-lane row that multiplies its super-block exactly once per tile
+        for (uint32_t i = 0; i < n; ++i)
+            if (seen[i] != 1) { a.fail("16-row-tile phase: input value " + std::to_string(i) + " is taken " + std::to_string(seen[i]) + " times"); break; }
+    }
+    for (uint32_t i = 0; i < 16 * t.n; ++i) {                   // thread i of the workgroup: residual in, row out
+        const uint32_t row = plan::tiles16_row(t, i);
+        a.touch(res, (uint64_t)row * 4, 4, "residual load", b, 0, i, layer);
+        a.touch(out, (uint64_t)row * 4, 4, "projection store", b, 0, i, layer);
+        if (row < rows.size()) ++rows[row];
+    }
 }
 
 }  // namespace
@@ -136,7 +148,9 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                             int sign_extending_join, char *msg, size_t msg_len, unsigned long long *checked) {
     Audit a;
     a.sign_ext = sign_extending_join != 0;
-    const plan::Shape s = plan::make_shape(dim, hidden, n_heads, n_layers, vocab, seq_len, grid);
+    plan::Shape s = plan::make_shape(dim, hidden, n_heads, n_layers, vocab, seq_len);
+    if (grid) s.grid = grid;                                  // (a grid other than the plan's own must be refused)
+    grid = s.grid;
     if (!plan::shape_ok(s)) a.fail("plan::shape_ok refuses the shape");
     else {
         // fake placement: 4 GiB apart, lower word 0x10000000 or 0x90000000 (+ a region-specific stagger)
@@ -174,11 +188,11 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                     const plan::RowUnit u = plan::qkv_unit(s, b);
                     const uint32_t h = plan::qkv_head(s, b);
                     if (u.nrows == 0 || u.nrows > 64 || h >= n_heads || b % 8 != h % 8) { a.fail("q / k / v role"); continue; }
-                    if (u.row0 / 128 != h || (u.row0 + u.nrows - 1) / 128 != h) a.fail("a q / k / v unit leaves its head");
+                    if (plan::unit_row(u, 0) / 128 != h || plan::unit_row(u, u.nrows - 1) / 128 != h) a.fail("a q / k / v unit leaves its head");
                     ++units_of_head[h];
                     walk_tile64(a, u.seg == 0 ? wv : (u.seg == 1 ? wk : wq), u.seg == 0 ? tv : (u.seg == 1 ? tk : tq), u, ncb, b, l, u.seg == 0 ? &rows_v : (u.seg == 1 ? &rows_k : &rows_q));
                     walk_stage64(a, s, l == 0 ? xemb : xa, norm, slots, dim, ncb, b, l);
-                    for (uint32_t t = 0; t < u.nrows; ++t) a.touch(qv, (uint64_t)(u.row0 + t) * 4, 4, "q / k / v store", b, 0, t, l);
+                    for (uint32_t t = 0; t < u.nrows; ++t) a.touch(qv, (uint64_t)plan::unit_row(u, t) * 4, 4, "q / k / v store", b, 0, t, l);
                     a.touch(counters, (uint64_t)plan::counter_word(h) * 4, 4, "counter", b, 0, 0, l);
                 } else if (plan::is_attention_workgroup(s, b)) {
                     const uint32_t h = plan::attention_head(s, b);
@@ -192,15 +206,11 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                     }
                 }
                 a.touch(counters, (uint64_t)handoff_heads * 32 * 4, 4, "abort flag", b, 0, 0, l);
-                if (b < plan::proj_tiles(s)) {
-                    if (l == 0) for (uint32_t t = 0; t < 16; ++t) a.touch(xemb, ((uint64_t)16 * b + t) * 4, 4, "residual load", b, 0, t, l);
-                    walk_tile16(a, s, wo, to, b, ncb, ng_o, xb, dim, b, l);
-                    walk_tile16(a, s, wd, td, b, ncb_h, ng_d, hb, hidden, b, l);
-                    for (uint32_t t = 0; t < 16; ++t) {
-                        a.touch(xm, ((uint64_t)16 * b + t) * 4, 4, "xm store", b, 0, t, l);
-                        a.touch(xnext, ((uint64_t)16 * b + t) * 4, 4, "xa store", b, 0, t, l);
-                        ++rows_o[16 * b + t]; ++rows_d[16 * b + t];
-                    }
+                {
+                    const plan::Tiles16 wt = plan::wo_tiles(s, b), dt = plan::down_tiles(s, b);
+                    if (plan::is_attention_workgroup(s, b) != (wt.n == 0)) a.fail("exactly the attention workgroups take no tile of the output projection");
+                    walk_tile16(a, wo, to, wt, ncb, ng_o, xb, dim, l == 0 ? xemb : xa, xm, rows_o, b, l);
+                    walk_tile16(a, wd, td, dt, ncb_h, ng_d, hb, hidden, xm, xnext, rows_d, b, l);
                 }
                 if (b < plan::gu_units(s)) {
                     const plan::RowUnit u = plan::gu_unit(s, b);
@@ -226,7 +236,7 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
         for (uint32_t b = 0; b < grid && a.violations < 8; ++b) {
             bool first = true;
             for (uint32_t tile = b; tile < plan::out_tiles(s); tile += grid) {
-                const plan::RowUnit u{0u, tile * 64u, plan::umin(64u, vocab - tile * 64u)};
+                const plan::RowUnit u = plan::run_unit(0u, tile * 64u, plan::umin(64u, vocab - tile * 64u));
                 walk_tile64(a, wout, tout, u, ncb, b, n_layers, &rows_l);
                 if (first) walk_stage64(a, s, xlast, norm, slots, dim, ncb, b, n_layers);
                 first = false;
@@ -242,10 +252,11 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
     return a.violations;
 }
 
-// the decomposition plan::make_shape picks (for the test's report)
-void rb_shape(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32_t grid, uint32_t *qkv_units, uint32_t *gu_rows, uint32_t *gu_units) {
-    const plan::Shape s = plan::make_shape(dim, hidden, n_heads, 1, 64, 64, grid);
-    *qkv_units = s.qkv_units; *gu_rows = s.gu_rows; *gu_units = plan::gu_units(s);
+// the decomposition plan::make_shape picks: grid, rows per gate / up unit, number of gate / up units
+void rb_shape(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32_t grid, uint32_t *qkv_units /* receives the grid */, uint32_t *gu_rows, uint32_t *gu_units) {
+    const plan::Shape s = plan::make_shape(dim, hidden, n_heads, 1, 64, 64);
+    (void)grid;
+    *qkv_units = s.grid; *gu_rows = s.gu_rows; *gu_units = plan::gu_units(s);
 }
 
 }  // extern "C"
