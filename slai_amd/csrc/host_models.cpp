@@ -396,7 +396,7 @@ int slai_llama2::persistent_setup() {
     if (persistent_capacity(p, ctx->device, &resident) != hipSuccess) return no("the occupancy query for the kernel failed");
     hipDeviceProp_t prop;
     SLAI_HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
-    const plan::Shape sh = plan::make_shape(dim, hid, nh, nl, config.vocab_size, config.seq_len);
+    const plan::Shape sh = plan::make_shape(dim, hid, nh, nl, config.vocab_size, config.seq_len, rope_variant() == SLAI_ROPE_NEOX ? 1u : 0u);
     const uint32_t grid = sh.grid;                                    // one workgroup per compute unit at most, all resident
     if (grid > std::min(resident, (uint32_t)prop.multiProcessorCount)) return no("the device keeps too few workgroups of the kernel resident for this shape");
     if (!plan::shape_ok(sh)) return no("shape: the FFN width does not spread evenly over one workgroup per 16 rows of the model width");

@@ -438,8 +438,203 @@ __device__ __forceinline__ void mult16_any(int type, const Unit &u, const plan::
     else mult16<T_Q4_K>(u, t, ncb, ngroups, x, res, res_flow, residual, partial, f, tr, wave);
 }
 
+// ---- the attention of one head (transformer.rs:342-350: RoPE, cache write, scores, softmax, weighted values) ------------
+// The workgroups that multiply q, k and v also add the bias, rotate, and write the cache row (rotate_and_store); what is
+// left here is the part that needs the whole head.  Everything that depends on the position only -- the cached keys and
+// values of up to ATT_PRE passes, all of them for the first 384 positions of an f16 cache -- is requested before the
+// query exists.  Every wave runs a softmax of its own over the positions it owns; the newest position, whose key and
+// value are produced in this launch, joins when the waves are merged.
+template <bool F16> struct AttPass {
+    static constexpr int KP = F16 ? 2 : 4, VP = F16 ? 1 : 2;    // 16-byte pieces of a lane's sixteen key / eight value elements
+    U4 k[KP], v[2][VP];
+};
+template <bool F16> __device__ __forceinline__ void att_decode8(const U4 *r, float (&o)[8]) {
+    if constexpr (F16) {
+        const uint32_t u[4] = {r[0].x, r[0].y, r[0].z, r[0].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { o[2 * i] = attn::h2f((uint16_t)(u[i] & 0xffffu)); o[2 * i + 1] = attn::h2f((uint16_t)(u[i] >> 16)); }
+    } else {
+        o[0] = __uint_as_float(r[0].x); o[1] = __uint_as_float(r[0].y); o[2] = __uint_as_float(r[0].z); o[3] = __uint_as_float(r[0].w);
+        o[4] = __uint_as_float(r[1].x); o[5] = __uint_as_float(r[1].y); o[6] = __uint_as_float(r[1].z); o[7] = __uint_as_float(r[1].w);
+    }
+}
+__device__ __forceinline__ U4 as_u4(u32x4 v) { return U4{v.x, v.y, v.z, v.w}; }
+
+template <bool F16> struct Attention {
+    using P = AttPass<F16>;
+    static constexpr uint32_t ES = F16 ? 2 : 4;                 // bytes of a cache element
+    static constexpr int ATT_PRE = F16 ? 3 : 1;                 // passes requested before the query is waited for
+    const plan::Shape &sh;
+    Rsrc kc, vc;              // the layer's caches
+    uint32_t head, T;         // T: cached positions (= the position of this token)
+    uint32_t wave;
+    float m, lsum, o[8];      // this wave's running maximum and sum, this lane's eight outputs
+
+    __device__ __forceinline__ void request(P &ps, uint32_t tb) const {
+        const uint32_t lane = lane_id();
+        // lanes without a position read position 0: a valid address (there is at least one cached position when any pass runs)
+        const uint32_t t = plan::att_k_pos(tb, wave, lane);
+        const uint32_t koff = plan::cache_elem(sh, t < T ? t : 0u, plan::att_k_elem(head, lane)) * ES;
+#pragma unroll
+        for (int j = 0; j < P::KP; ++j) ps.k[j] = as_u4(buf_load16<AUX_PLAIN>(kc, koff + 16u * j));
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const uint32_t tv = plan::att_v_pos(tb, wave, u, lane);
+            const uint32_t voff = plan::cache_elem(sh, tv < T ? tv : 0u, plan::att_v_elem(head, lane)) * ES;
+#pragma unroll
+            for (int j = 0; j < P::VP; ++j) ps.v[u][j] = as_u4(buf_load16<AUX_PLAIN>(vc, voff + 16u * j));
+        }
+    }
+    // scores of this wave's eight positions of the pass, softmax update, weighted values (cpu.rs:505-560 in one sweep)
+    __device__ __forceinline__ void consume(const P &ps, uint32_t tb, const float (&qr)[16]) {
+        const uint32_t lane = lane_id();
+        const bool live = plan::att_k_pos(tb, wave, lane) < T;
+        float part = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            float kv[8];
+            att_decode8<F16>(ps.k + j * (P::KP / 2), kv);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) part = fmaf(qr[8 * j + q], kv[q], part);
+        }
+        part += lane_xor(part, 1);
+        part += lane_xor(part, 2);
+        part += lane_xor(part, 4);
+        const float sc = live ? part / sqrtf(128.0f) : -FLT_MAX;             // cpu.rs:521
+        float mx = sc;
+#pragma unroll
+        for (int msk = 32; msk >= 8; msk >>= 1) mx = fmaxf(mx, lane_xor(mx, msk));
+        const float mn = fmaxf(m, mx);
+        const float resc = expf(m - mn);                        // 0 on the first live pass, 1 while nothing was live
+        const float pr = live ? expf(sc - mn) : 0.0f;
+        lsum = fmaf(lsum, resc, (lane & 7u) == 0 ? pr : 0.0f);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) o[q] *= resc;
+        m = mn;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            // the weight of position u * 4 + lane / 16 of this wave's eight: held by the eight lanes that scored it
+            const int src = (int)(8u * (u * 4u + lane / 16u));
+            const float pw = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src << 2, __builtin_bit_cast(int, pr)));
+            float vv[8];
+            att_decode8<F16>(ps.v[u], vv);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) o[q] = fmaf(pw, vv[q], o[q]);
+        }
+    }
+};
+
+// lds: [16 waves][128] partial outputs, then the waves' maxima and sums.  q / knew / vnew: this layer's hand-off vectors
+// (dim floats each); out: the attention output vector.
+template <bool F16>
+__device__ __forceinline__ void attend(const plan::Shape &sh, uint32_t head, uint32_t pos, Rsrc kc, Rsrc vc, Rsrc q, Rsrc knew, Rsrc vnew, Rsrc out,
+                                       float *lds, Flow &f, uint64_t *tl, uint32_t wave) {
+    using A = Attention<F16>;
+    using P = typename A::P;
+    float *sacc = lds, *smax = lds + PNW * 128, *ssum = smax + PNW;
+    A at{sh, kc, vc, head, pos, wave, -FLT_MAX, 0.0f, {0, 0, 0, 0, 0, 0, 0, 0}};
+    P pre[A::ATT_PRE], cur;
+#pragma unroll
+    for (int i = 0; i < A::ATT_PRE; ++i) {
+        pre[i] = P{};
+        if (i * plan::ATT_PASS < pos) at.request(pre[i], i * plan::ATT_PASS);
+    }
+    cur = P{};
+    if (A::ATT_PRE * plan::ATT_PASS < pos) at.request(cur, A::ATT_PRE * plan::ATT_PASS);
+    // the query: sixteen elements per lane, as soon as all of them are there
+    float qr[16];
+    {
+        const uint32_t first = plan::att_k_elem(head, lane_id());
+        uint64_t deadline = 0;
+        uint32_t rounds = 0;
+        for (;;) {
+            u32x4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = buf_load16<AUX_FLOW>(q, (first + 4u * j) * 4u);
+            const bool hole = flow_empty(v[0]) || flow_empty(v[1]) || flow_empty(v[2]) || flow_empty(v[3]);
+            if (!__any(hole) || f.dead) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { qr[4 * j] = __uint_as_float(v[j].x); qr[4 * j + 1] = __uint_as_float(v[j].y); qr[4 * j + 2] = __uint_as_float(v[j].z); qr[4 * j + 3] = __uint_as_float(v[j].w); }
+                break;
+            }
+            flow_backoff(f, deadline, rounds);
+        }
+    }
+    stamp(tl, 1, wave);
+#pragma unroll
+    for (int i = 0; i < A::ATT_PRE; ++i)
+        if (i * plan::ATT_PASS < pos) at.consume(pre[i], i * plan::ATT_PASS, qr);
+    for (uint32_t tb = A::ATT_PRE * plan::ATT_PASS; tb < pos; tb += plan::ATT_PASS) {
+        P nxt = P{};
+        if (tb + plan::ATT_PASS < pos) at.request(nxt, tb + plan::ATT_PASS);
+        at.consume(cur, tb, qr);
+        cur = nxt;
+    }
+    // this wave's (maximum, sum, outputs): lanes 16 apart hold the same elements of different positions
+    at.lsum = wave_total(at.lsum);
+#pragma unroll
+    for (int msk = 16; msk < 64; msk <<= 1) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) at.o[e] += lane_xor(at.o[e], msk);
+    }
+    const uint32_t lane = lane_id();
+    if (lane < 16) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sacc[wave * 128 + lane * 8 + e] = at.o[e];
+    }
+    if (lane == 0) { smax[wave] = at.m; ssum[wave] = at.lsum; }
+    stamp(tl, 2, wave);
+    // the newest position: its score like a cached one's (waves 0 and 1, whose threads merge), its value per element
+    float snew = 0.0f, vn = 0.0f;
+    if (wave < 2) {
+        const uint32_t first = plan::att_k_elem(head, lane);
+        uint64_t deadline = 0;
+        uint32_t rounds = 0;
+        u32x4 v[4];
+        uint32_t w;
+        for (;;) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = buf_load16<AUX_FLOW>(knew, (first + 4u * j) * 4u);
+            w = __builtin_amdgcn_raw_buffer_load_b32(vnew, (int)((head * 128u + wave * 64u + lane) * 4u), 0, AUX_FLOW);
+            const bool hole = flow_empty(v[0]) || flow_empty(v[1]) || flow_empty(v[2]) || flow_empty(v[3]) || w == FLOW_EMPTY;
+            if (!__any(hole) || f.dead) break;
+            flow_backoff(f, deadline, rounds);
+        }
+        using C = attn::KV<F16>;                                // (what the cache row holds: rounded to its element type)
+        float part = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            part = fmaf(qr[4 * j], C::round(__uint_as_float(v[j].x)), part);
+            part = fmaf(qr[4 * j + 1], C::round(__uint_as_float(v[j].y)), part);
+            part = fmaf(qr[4 * j + 2], C::round(__uint_as_float(v[j].z)), part);
+            part = fmaf(qr[4 * j + 3], C::round(__uint_as_float(v[j].w)), part);
+        }
+        part += lane_xor(part, 1);
+        part += lane_xor(part, 2);
+        part += lane_xor(part, 4);
+        snew = part / sqrtf(128.0f);
+        vn = C::round(__uint_as_float(w));
+    }
+    lds_barrier();
+    if (wave < 2) {
+        const uint32_t e = wave * 64u + lane;
+        float M = snew;
+#pragma unroll
+        for (int w = 0; w < PNW; ++w) M = fmaxf(M, smax[w]);
+        const float fn = expf(snew - M);
+        float r = vn * fn, l = fn;
+#pragma unroll
+        for (int w = 0; w < PNW; ++w) {
+            const float fw = expf(smax[w] - M);                 // a wave that saw no position has sum 0 and outputs 0
+            r = fmaf(sacc[w * 128 + e], fw, r);
+            l = fmaf(ssum[w], fw, l);
+        }
+        flow_put(out, head * 128u + e, r / l);
+    }
+}
+
 __device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
-    return plan::Shape{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, gridDim.x, p.qkv_units, p.gu_rows};
+    return plan::Shape{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, gridDim.x, p.qkv_units, p.gu_rows, p.rope_variant == SLAI_ROPE_NEOX ? 1u : 0u};
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------------------------------
@@ -448,7 +643,7 @@ __device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
 // a q / k / v unit there (or nothing): the attention needs nearly all registers, and only a body of its own shows the
 // compiler that no unit requested ahead is ever alive across it.
 template <bool F16, bool ATTN>
-__device__ __forceinline__ void decode_token(const PersistentParams &p, float *smem, uint32_t &wg_dead, uint32_t (&layer_words)[2][sizeof(PersistentLayer) / 4],
+__device__ __forceinline__ void decode_token(const PersistentParams &p, float *smem, float (&rope_cs)[2][64], uint32_t (&layer_words)[2][sizeof(PersistentLayer) / 4],
                                              const uint32_t wave) {
     constexpr int LWORDS = sizeof(PersistentLayer) / 4;
     // Two sets of partial[2][16][64] | red[16], taken in turn by the phases of this workgroup: a wave that is done with a
@@ -475,6 +670,21 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
     const DevBuf wout = dev_buf(p.wout);
     const plan::Tiles16 wo_t = plan::wo_tiles(sh, b), down_t = plan::down_tiles(sh, b);
 
+    const uint32_t pos = *p.pos_ptr;
+    // The rotation of this lane's row of a q or k unit depends on the position only: cosine and sine are computed once
+    // (rope.slang:36-39: the angle depends on (2 * i) mod head_size for both pairings; the frequencies come from a table
+    // built once with the same powf) and kept in LDS, where reading them waits for no weights.
+    if constexpr (!ATTN) {
+        if (wave == 0 && qkv_u.seg != 0 && p.rope_variant >= 0) {
+            const uint32_t lane = lane_id(), e = plan::unit_row(qkv_u, lane) & 127u;
+            const uint32_t i = p.rope_variant == SLAI_ROPE_NEOX ? (e & 63u) : (e >> 1);
+            const float theta = p.rope_theta ? p.rope_theta[i] : powf(p.rope_base, -(float)((2 * i) % 128u) / 128.0f);
+            float sn, c;
+            sincosf((float)pos * theta, &sn, &c);
+            rope_cs[0][lane] = c; rope_cs[1][lane] = sn;
+        }
+    }
+
     Unit unit;                                                     // the weights requested ahead for this workgroup's next phase
     Req req;
     int unit_type = 0;                                             // its block format
@@ -499,59 +709,48 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
         const Rsrc xnext = make_rsrc(p.flow + plan::flow_xa(sh, l + 1), dim * 4u);
         // ---- q / k / v, or the attention ------------------------------------------------------------------------------
         if constexpr (!ATTN) {
-            const uint32_t h = plan::qkv_head(sh, b);
-            float *out = qkv_u.seg == 0 ? p.vcol : (qkv_u.seg == 1 ? p.kcol : p.q);
             const TileIn in{l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, LAYER_BUF(lw, attn_norm).rs, dim, p.eps};
             stamp(tl, 0, wave);
+            // the bias of this lane's row (zero from an empty descriptor when the model has none): asked for now, behind
+            // this phase's weights -- after the next request it would wait for the next phase's
+            const uint32_t row = plan::unit_row(qkv_u, lane_id());
+            const DevBuf bias = qkv_u.seg == 0 ? LAYER_BUF(lw, bv) : (qkv_u.seg == 1 ? LAYER_BUF(lw, bk) : LAYER_BUF(lw, bq));
+            float bias_v = 0.0f;
+            if (fresh(wave) == 0) bias_v = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(bias.rs, (int)(row * 4u), 0, AUX_PLAIN));
             mult64_any<false>(unit_type, unit, req, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tl, wave);
             { const DevBuf W = LAYER_BUF(lw, wo); request16(unit, req, W, wo_t, ng_o, wave); unit_type = W.type; }
             const float o = finish64<false>(ncb, in, PHASE_PARTIAL, PHASE_RED, tl, wave);
-            const uint32_t tid = wave * 64u + lane_id();
-            if (tid < 64) {
-                if (tid < qkv_u.nrows) flow_store(out + plan::unit_row(qkv_u, tid), o);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                if (tid == 0) __hip_atomic_fetch_add(p.counters + plan::counter_word(h), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (fresh(wave) == 0) {
+                // RoPE (rope.slang:27-84) with the partner of the pair in a neighbouring lane, the row into the cache for the
+                // tokens to come, and the value itself to this token's attention.  Stores only: none of this waits for the
+                // weights just requested.
+                const uint32_t lane = lane_id();
+                float val = o + bias_v;
+                if (qkv_u.seg != 0 && p.rope_variant >= 0) {
+                    const bool neox = p.rope_variant == SLAI_ROPE_NEOX;
+                    const float other = lane_xor(val, neox ? 32 : 1);
+                    const bool first = neox ? lane < 32u : (lane & 1u) == 0;
+                    const float c = rope_cs[0][lane], sn = rope_cs[1][lane];
+                    val = first ? c * val - sn * other : sn * other + c * val;
+                }
+                if (lane < qkv_u.nrows) {
+                    flow_put(make_rsrc(p.flow + plan::flow_qkv(sh, l, qkv_u.seg), dim * 4u), row, val);
+                    if (qkv_u.seg != 2) {
+                        const DevBuf cache = qkv_u.seg == 0 ? LAYER_BUF(lw, vcache) : LAYER_BUF(lw, kcache);
+                        const uint32_t at = plan::cache_elem(sh, pos, row);
+                        if constexpr (F16) __builtin_amdgcn_raw_buffer_store_b16(attn::f2h(val), cache.rs, (int)(at * 2u), 0, AUX_PLAIN);
+                        else __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), cache.rs, (int)(at * 4u), 0, AUX_PLAIN);
+                    }
+                }
             }
             ++phase;
         } else {
             const uint32_t h = plan::attention_head(sh, b);
-            AttnLaunch a{};
-            a.q = p.q; a.knew = p.kcol; a.vnew = p.vcol;
-            a.kcache = const_cast<void *>(LAYER_BUF(lw, kcache).ptr); a.vcache = const_cast<void *>(LAYER_BUF(lw, vcache).ptr); a.kv_f16 = F16;
-            a.n_heads = nh; a.kv_mul = 1; a.head_size = 128; a.kv_dim = dim; a.seq_len = p.seq_len;
-            a.pos_ptr = p.pos_ptr;
-            a.qbias = (const float *)LAYER_BUF(lw, bq).ptr; a.kbias = (const float *)LAYER_BUF(lw, bk).ptr; a.vbias = (const float *)LAYER_BUF(lw, bv).ptr;
-            a.rope_variant = p.rope_variant; a.rope_base = p.rope_base; a.rope_theta = p.rope_theta;
-            a.out = p.flow + plan::flow_xb(sh, l); a.scratch = nullptr; a.n_splits = 1;
-            uint32_t *counter = p.counters + plan::counter_word(h);
-            const uint32_t need = p.qkv_units;
-            const uint32_t tid = wave * 64u + lane_id();
             stamp(tl, 0, wave);
-            attn::attn_fast_body<F16, PNT, 128, true, true, 8, true>(a, h, 0u, tid, [&]() {
-                if (tid == 0) {
-                    uint32_t seen = 0, spins = 0;
-                    uint64_t deadline = 0;
-                    bool gave_up = f.dead;                         // (f.dead: uniform over the workgroup here)
-                    while (!gave_up) {
-                        // a read-modify-write that returns the value executes in the L2 the producers' atomics went to
-                        const uint32_t zero = 0;
-                        asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=&v"(seen) : "v"(counter), "v"(zero) : "memory");
-                        if (seen >= need) break;
-                        if ((++spins & 15u) == 0) {
-                            const uint64_t now = wall_clock64();
-                            if (deadline == 0) deadline = now + FLOW_WAIT_TICKS;
-                            gave_up = now > deadline || __hip_atomic_load(f.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
-                        }
-                    }
-                    if (gave_up) { wg_dead = 1; __hip_atomic_store(f.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-                    *counter = 0u;                                 // for the next layer; nobody else touches it until then
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                }
-                __syncthreads();
-                asm volatile("" ::: "memory");
-            });
-            if (wg_dead) f.dead = true;
+            attend<F16>(sh, h, pos, LAYER_BUF(lw, kcache).rs, LAYER_BUF(lw, vcache).rs, make_rsrc(p.flow + plan::flow_qkv(sh, l, 2), dim * 4u),
+                        make_rsrc(p.flow + plan::flow_qkv(sh, l, 1), dim * 4u), make_rsrc(p.flow + plan::flow_qkv(sh, l, 0), dim * 4u), xb, PHASE_PARTIAL, f, tl, wave);
             stamp(tl, 3, wave);
+            ++phase;
             // (only now: the attention needs the registers; these workgroups have no tile of the output projection)
             { const DevBuf W = LAYER_BUF(lw, wgate); request64<true>(unit, req, W, LAYER_BUF(lw, wup), gu_u, ncb, wave); unit_type = W.type; }
         }
@@ -631,7 +830,7 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
 template <bool F16>
 __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const PersistentParams p) {
     extern __shared__ __align__(16) float smem[];
-    __shared__ uint32_t wg_dead;                                   // the attention hand-off of this workgroup timed out
+    __shared__ float rope_cs[2][64];                               // cosine | sine of the rotation of wave 0's rows (q and k units)
     constexpr int LWORDS = sizeof(PersistentLayer) / 4;
     static_assert(LWORDS <= 64 && sizeof(PersistentLayer) == 14 * sizeof(ResidentBuf), "one thread per word; fourteen entries");
     __shared__ uint32_t layer_words[2][LWORDS];
@@ -639,13 +838,12 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
     // A launch after one in which a reader gave up does nothing: the host has not looked yet (it queues many tokens), and
     // every further token would only wait out the same time limits.
     if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
-    if (threadIdx.x == 0) wg_dead = 0;
     if (threadIdx.x < LWORDS) layer_words[0][threadIdx.x] = reinterpret_cast<const uint32_t *>(p.layers)[threadIdx.x];
     __syncthreads();
-    const plan::Shape sh{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, gridDim.x, p.qkv_units, p.gu_rows};
+    const plan::Shape sh = shape_of(p);
     const uint32_t wave = uniform_word(threadIdx.x >> 6);
-    if (plan::is_attention_workgroup(sh, blockIdx.x)) decode_token<F16, true>(p, smem, wg_dead, layer_words, wave);
-    else decode_token<F16, false>(p, smem, wg_dead, layer_words, wave);
+    if (plan::is_attention_workgroup(sh, blockIdx.x)) decode_token<F16, true>(p, smem, rope_cs, layer_words, wave);
+    else decode_token<F16, false>(p, smem, rope_cs, layer_words, wave);
 }
 
 #undef PHASE_PARTIAL
@@ -660,7 +858,7 @@ __global__ void flow_fill_kernel(u32x4 *buf, size_t n16) {
 }  // namespace
 
 size_t persistent_smem_bytes(const PersistentParams &p) {
-    const plan::Shape s{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, 0, p.qkv_units, p.gu_rows};
+    const plan::Shape s{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, 0, p.qkv_units, p.gu_rows, 0};
     return (size_t)plan::lds_floats(s) * sizeof(float);
 }
 

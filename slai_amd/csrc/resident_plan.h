@@ -56,11 +56,13 @@ SLAI_HD bool shape_ok(const Shape &s) {
 // ---- hand-off buffers: one allocation of flow_floats() floats ------------------------------------------------------------
 // xa [(n_layers + 1) x dim]: the input of layer l (row 0 unused: layer 0 reads the embedding row); row n_layers feeds
 // the output matrix.  xb, xm [n_layers x dim]: attention output, residual after the attention.  hb [n_layers x hidden].
-SLAI_HD uint64_t flow_floats(const Shape &s) { return (uint64_t)(3 * s.n_layers + 1) * s.dim + (uint64_t)s.n_layers * s.hidden; }
+SLAI_HD uint64_t flow_floats(const Shape &s) { return (uint64_t)(6 * s.n_layers + 1) * s.dim + (uint64_t)s.n_layers * s.hidden; }
 SLAI_HD uint64_t flow_xa(const Shape &s, uint32_t l) { return (uint64_t)l * s.dim; }
 SLAI_HD uint64_t flow_xb(const Shape &s, uint32_t l) { return (uint64_t)(s.n_layers + 1) * s.dim + (uint64_t)l * s.dim; }
 SLAI_HD uint64_t flow_xm(const Shape &s, uint32_t l) { return (uint64_t)(2 * s.n_layers + 1) * s.dim + (uint64_t)l * s.dim; }
-SLAI_HD uint64_t flow_hb(const Shape &s, uint32_t l) { return (uint64_t)(3 * s.n_layers + 1) * s.dim + (uint64_t)l * s.hidden; }
+// the rotated query, and the newest key (rotated) and value as the attention of this very token reads them (seg: 0 v, 1 k, 2 q)
+SLAI_HD uint64_t flow_qkv(const Shape &s, uint32_t l, uint32_t seg) { return (uint64_t)((3 + seg) * s.n_layers + 1) * s.dim + (uint64_t)l * s.dim; }
+SLAI_HD uint64_t flow_hb(const Shape &s, uint32_t l) { return (uint64_t)(6 * s.n_layers + 1) * s.dim + (uint64_t)l * s.hidden; }
 
 // ---- per-workgroup slot (the staged input of a 64-row-unit phase, read back with scalar loads) ---------------------------
 SLAI_HD uint32_t slot_stride(const Shape &s) { return s.dim + s.dim / 16 + 16; }             // floats
@@ -73,10 +75,20 @@ SLAI_HD uint32_t slot_sums(const Shape &s, uint32_t cb) { return s.dim + cb * 16
 // ---- dynamic LDS of a workgroup, in floats: two sets of partial[2][16][64] | red[16], used by its phases in turn -----------
 SLAI_HD uint32_t lds_partial() { return 0; }
 SLAI_HD uint32_t lds_red() { return 2 * WG_WAVES * 64; }
-SLAI_HD uint32_t lds_set(uint32_t parity) { return parity * (lds_red() + WG_WAVES); }
-SLAI_HD uint32_t lds_floats(const Shape &) { return 2 * (lds_red() + WG_WAVES); }
+SLAI_HD uint32_t lds_set(uint32_t parity) { return parity * (lds_red() + 2 * WG_WAVES); }
+SLAI_HD uint32_t lds_floats(const Shape &) { return 2 * (lds_red() + 2 * WG_WAVES); }
 
-// ---- counters of the q / k / v -> attention hand-off: one 128-byte line per head, then the flag of a wait that gave up ---
+// ---- the attention of a head over the cached positions: eight lanes per position for the scores (sixteen elements
+// each), sixteen lanes per position for the values (eight elements each); a pass is 128 positions, eight per wave --------
+constexpr uint32_t ATT_PASS = 128;
+SLAI_HD uint32_t att_k_pos(uint32_t tb, uint32_t wave, uint32_t lane) { return tb + wave * 8 + lane / 8; }
+SLAI_HD uint32_t att_k_elem(uint32_t head, uint32_t lane) { return head * 128 + (lane & 7u) * 16; }
+SLAI_HD uint32_t att_v_pos(uint32_t tb, uint32_t wave, uint32_t u, uint32_t lane) { return tb + wave * 8 + u * 4 + lane / 16; }
+SLAI_HD uint32_t att_v_elem(uint32_t head, uint32_t lane) { return head * 128 + (lane & 15u) * 8; }
+// element e of position t of a cache [seq_len x dim] (times the element size: below 4 GiB, shape_ok bounds seq_len and dim)
+SLAI_HD uint32_t cache_elem(const Shape &s, uint32_t t, uint32_t e) { return t * s.dim + e; }
+// the control block: one 128-byte line per head (counters of the launches that hand q / k / v over per step), then the
+// flag of a wait that gave up
 SLAI_HD uint32_t counter_word(uint32_t head, uint32_t which = 0) { return head * 32 + which; }
 
 // ---- time stamps: per workgroup 16 per layer (four per phase) and 8 for the output matrix -------------------------------
@@ -112,11 +124,6 @@ SLAI_HD RowUnit qkv_unit(const Shape &s, uint32_t b) {
     if (s.neox) return RowUnit{seg, head * 128u + 32u * part, 64u, 32u, head * 128u + 64u + 32u * part};
     return run_unit(seg, head * 128u + 64u * part, 64u);
 }
-// which counter of the head a unit bumps when its rows are stored: 0 (q: the attention can start) or 1 (k and v: the
-// newest position can be added); and how many bumps the attention waits for
-SLAI_HD uint32_t qkv_counter(const RowUnit &u) { return u.seg == 2 ? 0u : 1u; }
-SLAI_HD uint32_t q_units(const Shape &) { return 2u; }
-SLAI_HD uint32_t kv_units(const Shape &s) { return s.qkv_units - 2u; }
 SLAI_HD bool is_attention_workgroup(const Shape &s, uint32_t b) { return b >= qkv_workgroups(s) && b < qkv_workgroups(s) + s.n_heads; }
 SLAI_HD uint32_t attention_head(const Shape &s, uint32_t b) { return b - qkv_workgroups(s); }
 

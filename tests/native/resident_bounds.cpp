@@ -145,10 +145,10 @@ extern "C" {
 // Returns the number of violations; `msg` receives the first one, `checked` the number of accesses looked at.
 unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uint32_t n_layers, uint32_t vocab, uint32_t seq_len, uint32_t grid,
                             int tq, int tk, int tv, int to, int tg, int td, int tout, uint32_t handoff_heads, int kv_bytes, int high_bases,
-                            int sign_extending_join, char *msg, size_t msg_len, unsigned long long *checked) {
+                            int sign_extending_join, int neox, char *msg, size_t msg_len, unsigned long long *checked) {
     Audit a;
     a.sign_ext = sign_extending_join != 0;
-    plan::Shape s = plan::make_shape(dim, hidden, n_heads, n_layers, vocab, seq_len);
+    plan::Shape s = plan::make_shape(dim, hidden, n_heads, n_layers, vocab, seq_len, neox ? 1u : 0u);
     if (grid) s.grid = grid;                                  // (a grid other than the plan's own must be refused)
     grid = s.grid;
     if (!plan::shape_ok(s)) a.fail("plan::shape_ok refuses the shape");
@@ -162,7 +162,7 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
         const Region wd = place("wdown", matrix_bytes(td, dim, hidden, 4)), wout = place("wout", matrix_bytes(tout, vocab, dim, 6));
         const Region norm = place("norm vector", (uint64_t)dim * 4), xemb = place("embedding row", (uint64_t)dim * 4);
         const Region flow = place("hand-off buffers", plan::flow_floats(s) * 4), slots = place("slots", plan::slot_floats(s) * 4);
-        const Region qv = place("q / k / v vector", (uint64_t)dim * 4), logits = place("logits", (uint64_t)vocab * 4);
+        const Region bias = place("bias vector", (uint64_t)dim * 4), logits = place("logits", (uint64_t)vocab * 4);
         const Region counters = place("counters", ((uint64_t)handoff_heads * 32 + 32) * 4);
         const Region trace = place("trace", (uint64_t)grid * plan::trace_stride(s) * 8);
         const Region layers = place("layer table", (uint64_t)n_layers * 14 * 16);
@@ -180,6 +180,7 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
             };
             const Region xa = vec("xa", plan::flow_xa(s, l), dim), xb = vec("xb", plan::flow_xb(s, l), dim), xm = vec("xm", plan::flow_xm(s, l), dim);
             const Region hb = vec("hb", plan::flow_hb(s, l), hidden), xnext = vec("xa (next)", plan::flow_xa(s, l + 1), dim);
+            const Region vnew = vec("newest value", plan::flow_qkv(s, l, 0), dim), knew = vec("newest key", plan::flow_qkv(s, l, 1), dim), qvec = vec("query", plan::flow_qkv(s, l, 2), dim);
             for (uint32_t b = 0; b < grid; ++b) {
                 for (uint32_t tid = 0; tid < 14 * 4 && l + 1 < n_layers; ++tid) a.touch(layers, ((uint64_t)(l + 1) * 14 * 4 + tid) * 4, 4, "layer table word", b, 0, tid, l);
                 for (uint32_t ph = 0; ph < 4; ++ph)
@@ -192,17 +193,54 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                     ++units_of_head[h];
                     walk_tile64(a, u.seg == 0 ? wv : (u.seg == 1 ? wk : wq), u.seg == 0 ? tv : (u.seg == 1 ? tk : tq), u, ncb, b, l, u.seg == 0 ? &rows_v : (u.seg == 1 ? &rows_k : &rows_q));
                     walk_stage64(a, s, l == 0 ? xemb : xa, norm, slots, dim, ncb, b, l);
-                    for (uint32_t t = 0; t < u.nrows; ++t) a.touch(qv, (uint64_t)plan::unit_row(u, t) * 4, 4, "q / k / v store", b, 0, t, l);
-                    a.touch(counters, (uint64_t)plan::counter_word(h) * 4, 4, "counter", b, 0, 0, l);
+                    // wave 0: lane t adds the bias of its row, rotates with a partner lane of the same unit, and stores
+                    const Region &hand = u.seg == 0 ? vnew : (u.seg == 1 ? knew : qvec);
+                    for (uint32_t t = 0; t < 64; ++t) {
+                        const uint32_t row = plan::unit_row(u, t);
+                        a.touch(bias, (uint64_t)row * 4, 4, "bias load", b, 0, t, l);
+                        if (t >= u.nrows) continue;
+                        a.touch(hand, (uint64_t)row * 4, 4, "q / k / v store", b, 0, t, l);
+                        if (u.seg != 2) a.touch(cache, (uint64_t)plan::cache_elem(s, seq_len - 1, row) * kv_bytes, kv_bytes, "cache row store", b, 0, t, l);
+                        if (u.seg != 0) {
+                            // the partner of a rotary pair: element e ^ 1 (adjacent pairs) or e ^ 64 (NeoX) of the head, held
+                            // by lane t ^ 1 or t ^ 32 of the same unit
+                            const uint32_t partner = plan::unit_row(u, s.neox ? t ^ 32u : t ^ 1u);
+                            if (partner != (s.neox ? row ^ 64u : row ^ 1u) || (s.neox ? t ^ 32u : t ^ 1u) >= u.nrows) a.fail("a rotary pair is split over units");
+                        }
+                    }
                 } else if (plan::is_attention_workgroup(s, b)) {
                     const uint32_t h = plan::attention_head(s, b);
                     if (h >= n_heads || b % 8 != h % 8) { a.fail("attention role"); continue; }
                     ++heads_attended[h];
-                    a.touch(counters, (uint64_t)plan::counter_word(h) * 4, 4, "counter", b, 0, 0, l);
+                    // cached positions: every pass of the deepest context, every wave and lane; per position, each element of
+                    // the head's key once (eight lanes of sixteen) and of its value once (sixteen lanes of eight)
+                    const uint32_t T = seq_len - 1;
+                    std::vector<uint32_t> kseen((size_t)T * 128, 0), vseen((size_t)T * 128, 0);
+                    for (uint32_t tb = 0; tb < T; tb += plan::ATT_PASS)
+                        for (uint32_t wave = 0; wave < plan::WG_WAVES; ++wave)
+                            for (uint32_t lane = 0; lane < 64; ++lane) {
+                                const uint32_t t = plan::att_k_pos(tb, wave, lane), e = plan::att_k_elem(h, lane);
+                                a.touch(cache, (uint64_t)plan::cache_elem(s, t < T ? t : 0, e) * kv_bytes, 16 * kv_bytes, "cached key", b, wave, lane, l);
+                                if (e / 128 != h || e % 16) a.fail("key elements of another head");
+                                if (t < T) for (uint32_t i = 0; i < 16; ++i) ++kseen[(size_t)t * 128 + e % 128 + i];
+                                for (uint32_t uu = 0; uu < 2; ++uu) {
+                                    const uint32_t tv = plan::att_v_pos(tb, wave, uu, lane), ev = plan::att_v_elem(h, lane);
+                                    a.touch(cache, (uint64_t)plan::cache_elem(s, tv < T ? tv : 0, ev) * kv_bytes, 8 * kv_bytes, "cached value", b, wave, lane, l);
+                                    if (ev / 128 != h) a.fail("value elements of another head");
+                                    if (tv < T) for (uint32_t i = 0; i < 8; ++i) ++vseen[(size_t)tv * 128 + ev % 128 + i];
+                                    // the weight of that position comes from lane 8 * (position within the wave's eight)
+                                    if (plan::att_k_pos(tb, wave, 8 * (uu * 4 + lane / 16)) != tv) a.fail("value lane takes the weight of another position");
+                                }
+                            }
+                    for (size_t i = 0; i < kseen.size(); ++i)
+                        if (kseen[i] != 1 || vseen[i] != 1) { a.fail("attention: an element of a cached position is read " + std::to_string(kseen[i]) + " / " + std::to_string(vseen[i]) + " times"); break; }
+                    for (uint32_t lane = 0; lane < 64; ++lane) {
+                        a.touch(qvec, (uint64_t)plan::att_k_elem(h, lane) * 4, 64, "query", b, 0, lane, l);
+                        a.touch(knew, (uint64_t)plan::att_k_elem(h, lane) * 4, 64, "newest key", b, 0, lane, l);
+                    }
                     for (uint32_t t = 0; t < 128; ++t) {
-                        a.touch(qv, ((uint64_t)h * 128 + t) * 4, 4, "q / k / v load", b, 0, t, l);
-                        a.touch(xb, ((uint64_t)h * 128 + t) * 4, 4, "attention output", b, 0, t, l);
-                        a.touch(cache, ((uint64_t)(seq_len - 1) * dim + h * 128 + t) * kv_bytes, kv_bytes, "cache row", b, 0, t, l);
+                        a.touch(vnew, ((uint64_t)h * 128 + t) * 4, 4, "newest value", b, t / 64, t % 64, l);
+                        a.touch(xb, ((uint64_t)h * 128 + t) * 4, 4, "attention output", b, t / 64, t % 64, l);
                     }
                 }
                 a.touch(counters, (uint64_t)handoff_heads * 32 * 4, 4, "abort flag", b, 0, 0, l);

@@ -39,6 +39,30 @@ def test_persistent_small_model_vs_oracle(kv_f16):
         b.close()
 
 
+def test_persistent_long_context_vs_oracle():
+    """600 steps on the small model: the attention asks for the first 384 cached positions before the query exists and
+    walks the rest in passes of 128 with one pass in flight; positions 384, 385, 512, 513 are where those paths change."""
+    b = backend_with(True)
+    try:
+        data = gw.llama_gguf(dim=1024, hidden_dim=3072, n_layers=2, n_heads=8, n_kv_heads=8, vocab=2000, seq_len=640, wtype=12, v_type=14,
+                             out_type=14, embd_type=12, seed=77, std=0.05, norm_random=True)
+        check_llama(b, data, [5, 1000, 1999], 600, kv_f16=True, check_logit_steps=4, decode_form=1)
+    finally:
+        b.close()
+
+
+def test_persistent_qwen2_bias_and_neox_pairs():
+    """The Qwen2 variant in the resident form: q / k / v biases and NeoX rotary pairs (i, i + 64), which the workgroups that
+    multiply q and k rotate themselves (their units hold rows {0..31, 64..95} / {32..63, 96..127} of a head)."""
+    b = backend_with(True)
+    try:
+        data = gw.llama_gguf(dim=1024, hidden_dim=3072, n_layers=3, n_heads=8, n_kv_heads=8, vocab=2000, seq_len=256, wtype=12, v_type=14,
+                             out_type=14, embd_type=12, seed=75, std=0.05, arch="qwen2", bias=True, norm_random=True, rope_base=1000000.0, rms_eps=1e-6)
+        check_llama(b, data, [5, 1000, 1999, 9], 40, kv_f16=True, model_type=_ffi.MODEL_QWEN2, neox=1, name=b"qwen2", check_logit_steps=12, decode_form=1)
+    finally:
+        b.close()
+
+
 def test_persistent_small_model_behind_large_allocations():
     """The small model again, loaded after 5 GB of other allocations in steps of 640 MB: its buffers then lie at
     addresses whose lower 32 bits are spread over the whole range, bit 31 included (the first version of the kernel

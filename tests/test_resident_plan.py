@@ -21,15 +21,15 @@ def rb(tmp_path_factory):
                            os.path.join(HERE, "native", "resident_bounds.cpp"), "-o", out])
     L = C.CDLL(out)
     L.rb_audit.restype = C.c_ulonglong
-    L.rb_audit.argtypes = [C.c_uint32] * 7 + [C.c_int] * 7 + [C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_ulonglong)]
+    L.rb_audit.argtypes = [C.c_uint32] * 7 + [C.c_int] * 7 + [C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_ulonglong)]
     L.rb_shape.argtypes = [C.c_uint32] * 4 + [C.POINTER(C.c_uint32)] * 3
     return L
 
 
-def audit(rb, dim, hidden, n_heads, n_layers, vocab, seq_len, grid=0, types=(Q4_K, Q4_K, Q6_K, Q4_K, Q4_K, Q4_K, Q6_K), kv_bytes=2, high=0, sign_ext=0):
+def audit(rb, dim, hidden, n_heads, n_layers, vocab, seq_len, grid=0, types=(Q4_K, Q4_K, Q6_K, Q4_K, Q4_K, Q4_K, Q6_K), kv_bytes=2, high=0, sign_ext=0, neox=0):
     msg = C.create_string_buffer(400)
     checked = C.c_ulonglong()
-    bad = rb.rb_audit(dim, hidden, n_heads, n_layers, vocab, seq_len, grid, *types, max(n_heads, 256), kv_bytes, high, sign_ext, msg, 400, C.byref(checked))
+    bad = rb.rb_audit(dim, hidden, n_heads, n_layers, vocab, seq_len, grid, *types, max(n_heads, 256), kv_bytes, high, sign_ext, neox, msg, 400, C.byref(checked))
     return bad, msg.value.decode(), checked.value
 
 
@@ -40,6 +40,7 @@ SHAPES = {
     "dim 2048": dict(dim=2048, hidden=5632, n_heads=16, n_layers=4, vocab=4096, seq_len=512),
     "7B width, 2 layers": dict(dim=4096, hidden=11008, n_heads=32, n_layers=2, vocab=32000, seq_len=128),
     "config 4": dict(dim=4096, hidden=11008, n_heads=32, n_layers=32, vocab=32000, seq_len=512),
+    "NeoX rotary pairs": dict(dim=2048, hidden=5632, n_heads=16, n_layers=2, vocab=4096, seq_len=300, neox=1),
     "wide FFN (12 column groups in the down projection)": dict(dim=3072, hidden=12288, n_heads=24, n_layers=2, vocab=1000, seq_len=64, types=(Q5_K, Q4_K, Q4_K, Q6_K, Q4_K, Q4_K, Q4_K)),
 }
 
