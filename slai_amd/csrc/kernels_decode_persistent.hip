@@ -31,6 +31,7 @@
 #include <cstddef>
 #include "device_util.h"
 #include "gemv_operands.h"
+#include "mfma_q4k.h"
 #include "quant_tiled.h"
 #include "resident_plan.h"
 
@@ -167,10 +168,34 @@ __device__ __forceinline__ u32x4 flow_take(Rsrc x, uint32_t piece, Flow &f) {
         flow_backoff(f, deadline, rounds);
     }
 }
+// Four pieces per lane (piece0 + 64 k: the same lane's piece of four consecutive super-blocks; k >= n is not asked for
+// and comes back as zeros), under the same rule.
+__device__ __forceinline__ void flow_take4(Rsrc x, uint32_t piece0, uint32_t n, u32x4 (&out)[4], Flow &f) {
+    uint64_t deadline = 0;
+    uint32_t rounds = 0;
+    for (;;) {
+        bool hole = false;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            out[k] = u32x4{0u, 0u, 0u, 0u};
+            if ((uint32_t)k < n) { out[k] = buf_load16<AUX_FLOW>(x, (piece0 + 64u * k) * 16u); hole = hole || flow_empty(out[k]); }
+        }
+        if (!__any(hole) || f.dead) return;
+        flow_backoff(f, deadline, rounds);
+    }
+}
 // Sixteen floats per lane, 16 apart from float `first` on (the register layout of DevX), under the same rule.
 __device__ __forceinline__ void flow_take_strided(Rsrc x, uint32_t first, float (&out)[16], Flow &f) {
     uint64_t deadline = 0;
     uint32_t rounds = 0;
+    // While the vector is not there yet, one word per lane is asked for instead of sixteen -- a different one of the
+    // sixteen in each lane of a row, so that the wave as a whole looks at every run of 16 floats it will take: every
+    // wave of the device polls at this point, and sixteen times the requests would slow down the very stores waited for.
+    for (;;) {
+        const uint32_t w = __builtin_amdgcn_raw_buffer_load_b32(x, (int)((first + 16u * (lane_id() & 15u)) * 4u), 0, AUX_FLOW);
+        if (!__any(w == FLOW_EMPTY) || f.dead) break;
+        flow_backoff(f, deadline, rounds);
+    }
     for (;;) {
         uint32_t u[16];
 #pragma unroll
@@ -266,14 +291,44 @@ __device__ __forceinline__ void request64(Unit &u, Req &r, const DevBuf &W, cons
 // finished dot product), reads them back as scalar operands, multiplies, and leaves its partial sums in LDS.  `stage`:
 // false when the slot still holds this input.  partial[2][16][64], red[16].
 template <int T, bool DUAL>
-__device__ __forceinline__ void mult64(const Unit &u, const Req &r, uint32_t ncb, const TileIn &in, bool stage, float *slot, float *partial, float *red, Flow &f,
+__device__ __forceinline__ void mult64(const Unit &u, const Req &r, uint32_t ncb, const TileIn &in, bool stage, float *slot, char *lds, float *partial, float *red, Flow &f,
                                        uint64_t *tr, const uint32_t wave_) {
     using F = Tiled<T>;
     const int lane = (int)lane_id();
     const uint32_t wave = fresh(wave_);
     constexpr int NM = DUAL ? 2 : 1;
     float v = 0.0f, v2 = 0.0f;
-    if ((uint32_t)wave < ncb) {
+    if constexpr (T == T_Q4_K) {
+        // on the matrix cores (mfma_q4k.h): the wave stages its super-block in LDS, for itself alone
+        if ((uint32_t)wave < ncb) {
+            char *sb = lds + plan::lds_mq_sb(wave, 0);
+            if (stage) {
+                const uint32_t piece = plan::wave_piece((uint32_t)wave, (uint32_t)lane);
+                const float4 w = as_float4(buf_load16<AUX_PLAIN>(in.norm_w, piece * 16u));
+                float4 x = as_float4(in.flow ? flow_take(in.x, piece, f) : buf_load16<AUX_PLAIN>(in.x, piece * 16u));
+                float ss = fmaf(x.x, x.x, fmaf(x.y, x.y, fmaf(x.z, x.z, x.w * x.w)));
+                ss = wave_total(ss);
+                if (lane == 0) red[wave] = ss;
+                x.x *= w.x; x.y *= w.y; x.z *= w.z; x.w *= w.w;
+                mq::stage_superblock(x, sb);
+            }
+            stamp(tr, 1, wave);
+            typename F::Data d, e;
+#pragma unroll
+            for (int i = 0; i < F::PT; ++i) d.p[i] = u.a[i];
+            if constexpr (DUAL) {
+#pragma unroll
+                for (int i = 0; i < F::PT; ++i) e.p[i] = u.b[i];
+            }
+            const typename F::Data *dp[NM];
+            float o2[NM];
+            dp[0] = &d;
+            if constexpr (DUAL) dp[1] = &e;
+            mq::dot_q4k<NM>(dp, sb, lds + plan::lds_mq_zero(), lds + plan::lds_mq_cs(wave), o2);
+            v = o2[0];
+            if constexpr (DUAL) v2 = o2[1];
+        }
+    } else if ((uint32_t)wave < ncb) {
         if (stage) {
             const uint32_t piece = plan::wave_piece((uint32_t)wave, (uint32_t)lane);
             const float4 w = as_float4(buf_load16<AUX_PLAIN>(in.norm_w, piece * 16u));
@@ -367,8 +422,8 @@ __device__ __forceinline__ void request16(Unit &u, Req &r, const DevBuf &W, cons
 // `res`: the vector the result is added to (complete long before this phase).  Thread i < 16 * t.n receives, in `residual`,
 // element 16 * tile + i % 16 of it: asked for first, so that it is there when the reduction needs it.
 template <int T>
-__device__ __forceinline__ void mult16(const Unit &u, const plan::Tiles16 t, uint32_t ncb, uint32_t ngroups, Rsrc x, Rsrc res, bool res_flow, float &residual, float *partial,
-                                       Flow &f, uint64_t *tr, const uint32_t wave_) {
+__device__ __forceinline__ void mult16(const Unit &u, const plan::Tiles16 t, uint32_t ncb, uint32_t ngroups, Rsrc x, Rsrc res, bool res_flow, float &residual, char *lds,
+                                       float *partial, Flow &f, uint64_t *tr, const uint32_t wave_) {
     using F = Tiled<T>;
     const int lane = (int)lane_id();
     const uint32_t wave = fresh(wave_);
@@ -378,7 +433,27 @@ __device__ __forceinline__ void mult16(const Unit &u, const plan::Tiles16 t, uin
         const uint32_t off = (plan::tiles16_row(t, (uint32_t)lane)) * 4u;
         residual = __uint_as_float(res_flow ? __builtin_amdgcn_raw_buffer_load_b32(res, (int)off, 0, AUX_FLOW) : __builtin_amdgcn_raw_buffer_load_b32(res, (int)off, 0, AUX_PLAIN));
     }
-    if (wave < ngroups * t.n) {
+    if constexpr (T == T_Q4_K) {
+        // on the matrix cores (mfma_q4k.h): the wave stages its four super-blocks in LDS, for itself alone
+        if (wave < ngroups * t.n) {
+            const uint32_t g = wave % ngroups;
+            const uint32_t n = plan::umin(4u, ncb - plan::tile16_sb(g, 0));
+            u32x4 xv[4];
+            flow_take4(x, plan::tile16_piece(g, 0, (uint32_t)lane), n, xv, f);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) mq::stage_superblock(as_float4(xv[k]), lds + plan::lds_mq_sb(wave, k));
+            stamp(tr, 1, wave);
+            typename F::Data d;
+#pragma unroll
+            for (int i = 0; i < F::PT; ++i) d.p[i] = u.a[i];
+            const typename F::Data *dp[1] = {&d};
+            float o1[1];
+            mq::dot_q4k<1>(dp, lds + plan::lds_mq_sb(wave, (uint32_t)lane >> 4), lds + plan::lds_mq_zero(), lds + plan::lds_mq_cs(wave), o1);
+            v = o1[0];
+            v += lane_xor(v, 16);
+            v += lane_xor(v, 32);                                  // across the four super-blocks of the wave
+        }
+    } else if (wave < ngroups * t.n) {
         const uint32_t g = wave % ngroups;
         const bool valid = plan::tile16_cb(g, (uint32_t)lane) < ncb;
         DevX X;
@@ -424,18 +499,18 @@ __device__ __forceinline__ float finish16(const plan::Tiles16 t, uint32_t ngroup
 
 // the block format is uniform over the workgroup
 template <bool DUAL>
-__device__ __forceinline__ void mult64_any(int type, const Unit &u, const Req &r, uint32_t ncb, const TileIn &in, bool stage, float *slot, float *partial, float *red,
+__device__ __forceinline__ void mult64_any(int type, const Unit &u, const Req &r, uint32_t ncb, const TileIn &in, bool stage, float *slot, char *lds, float *partial, float *red,
                                            Flow &f, uint64_t *tr, uint32_t wave) {
     switch (type) {
-    case T_Q6_K: if constexpr (!DUAL) mult64<T_Q6_K, false>(u, r, ncb, in, stage, slot, partial, red, f, tr, wave); break;
-    case T_Q5_K: if constexpr (!DUAL) mult64<T_Q5_K, false>(u, r, ncb, in, stage, slot, partial, red, f, tr, wave); break;
-    default: mult64<T_Q4_K, DUAL>(u, r, ncb, in, stage, slot, partial, red, f, tr, wave); break;
+    case T_Q6_K: if constexpr (!DUAL) mult64<T_Q6_K, false>(u, r, ncb, in, stage, slot, lds, partial, red, f, tr, wave); break;
+    case T_Q5_K: if constexpr (!DUAL) mult64<T_Q5_K, false>(u, r, ncb, in, stage, slot, lds, partial, red, f, tr, wave); break;
+    default: mult64<T_Q4_K, DUAL>(u, r, ncb, in, stage, slot, lds, partial, red, f, tr, wave); break;
     }
 }
 __device__ __forceinline__ void mult16_any(int type, const Unit &u, const plan::Tiles16 t, uint32_t ncb, uint32_t ngroups, Rsrc x, Rsrc res, bool res_flow, float &residual,
-                                           float *partial, Flow &f, uint64_t *tr, uint32_t wave) {
-    if (type == T_Q6_K) mult16<T_Q6_K>(u, t, ncb, ngroups, x, res, res_flow, residual, partial, f, tr, wave);
-    else mult16<T_Q4_K>(u, t, ncb, ngroups, x, res, res_flow, residual, partial, f, tr, wave);
+                                           char *lds, float *partial, Flow &f, uint64_t *tr, uint32_t wave) {
+    if (type == T_Q6_K) mult16<T_Q6_K>(u, t, ncb, ngroups, x, res, res_flow, residual, lds, partial, f, tr, wave);
+    else mult16<T_Q4_K>(u, t, ncb, ngroups, x, res, res_flow, residual, lds, partial, f, tr, wave);
 }
 
 // ---- the attention of one head (transformer.rs:342-350: RoPE, cache write, scores, softmax, weighted values) ------------
@@ -633,6 +708,23 @@ __device__ __forceinline__ void attend(const plan::Shape &sh, uint32_t head, uin
     }
 }
 
+// A wave's unit of a 16-row tile parked in LDS and taken back: the attention needs the registers in between.
+__device__ __forceinline__ void park_unit(const Unit &u, float *lds, int type, uint32_t wave) {
+    const uint32_t lane = lane_id(), pt = tiled_pieces(type);
+#pragma unroll
+    for (int P = 0; P < (int)plan::PARK_PIECES; ++P)
+        if ((uint32_t)P < pt) *reinterpret_cast<U4 *>(lds + plan::lds_park_piece(wave, P, lane)) = u.a[P];
+    reinterpret_cast<uint32_t *>(lds)[plan::lds_park_tail(wave, lane)] = u.ta;
+}
+__device__ __forceinline__ void unpark_unit(Unit &u, const float *lds, int type, uint32_t wave) {
+    const uint32_t lane = lane_id(), pt = tiled_pieces(type);
+    u = Unit{};
+#pragma unroll
+    for (int P = 0; P < (int)plan::PARK_PIECES; ++P)
+        if ((uint32_t)P < pt) u.a[P] = *reinterpret_cast<const U4 *>(lds + plan::lds_park_piece(wave, P, lane));
+    u.ta = (uint16_t)reinterpret_cast<const uint32_t *>(lds)[plan::lds_park_tail(wave, lane)];
+}
+
 __device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
     return plan::Shape{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, gridDim.x, p.qkv_units, p.gu_rows, p.rope_variant == SLAI_ROPE_NEOX ? 1u : 0u};
 }
@@ -650,6 +742,7 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
     // phase goes on to the next one (there is one barrier per phase, before its reduction) while wave 0 may still be
     // reducing the one before, but it cannot get further ahead than that.
     float *const lds_sets = smem;
+    char *const lds = reinterpret_cast<char *>(smem);
 #define PHASE_PARTIAL (lds_sets + plan::lds_set(phase & 1u) + plan::lds_partial())
 #define PHASE_RED (lds_sets + plan::lds_set(phase & 1u) + plan::lds_red())
     const uint32_t b = blockIdx.x;
@@ -689,11 +782,22 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
     Req req;
     int unit_type = 0;                                             // its block format
     const auto qkv_matrix = [&](const uint32_t *lw) { return qkv_u.seg == 0 ? LAYER_BUF(lw, wv) : (qkv_u.seg == 1 ? LAYER_BUF(lw, wk) : LAYER_BUF(lw, wq)); };
-    if constexpr (!ATTN) {
-        const DevBuf W = qkv_matrix(layer_words[0]);
-        request64<false>(unit, req, W, W, qkv_u, ncb, wave);
-        unit_type = W.type;
-    }
+    // Which weights a wave asks for next (a wave without a part in a 16-row-tile phase gets to the request after it at once).
+    const auto ask_wo = [&](const uint32_t *lw) { const DevBuf W = LAYER_BUF(lw, wo); request16(unit, req, W, wo_t, ng_o, wave); unit_type = W.type; };
+    const auto ask_gate_up = [&](const uint32_t *lw) { const DevBuf W = LAYER_BUF(lw, wgate); request64<true>(unit, req, W, LAYER_BUF(lw, wup), gu_u, ncb, wave); unit_type = W.type; };
+    const auto ask_down = [&](const uint32_t *lw) { const DevBuf W = LAYER_BUF(lw, wdown); request16(unit, req, W, down_t, ng_d, wave); unit_type = W.type; };
+    // what this workgroup multiplies after a layer: its q / k / v unit of the next one, or its first tile of the output matrix
+    const auto ask_next = [&](const uint32_t *lw_next, bool last) {
+        if (last) {
+            if (b < ntiles_out) request64<false>(unit, req, wout, wout, plan::run_unit(0u, b * 64u, plan::umin(64u, p.vocab - b * 64u)), ncb, wave);
+            unit_type = wout.type;
+        } else if constexpr (!ATTN) {
+            const DevBuf W = qkv_matrix(lw_next);
+            request64<false>(unit, req, W, W, qkv_u, ncb, wave);
+            unit_type = W.type;
+        }
+    };
+    if constexpr (!ATTN) ask_next(layer_words[0], false);
 
     for (uint32_t l = 0; l < p.n_layers; ++l) {
         // this layer's description comes out of LDS entry by entry, as wave-uniform values, where it is used; the next
@@ -702,6 +806,12 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
         const bool last = l + 1 == p.n_layers;
         uint32_t next_word = 0;
         if (wave == 0 && lane_id() < LWORDS && !last) next_word = reinterpret_cast<const uint32_t *>(p.layers + l + 1)[lane_id()];
+        // Parked once wave 0 has waited for its memory requests anyway.  Nobody reads the slot it goes to any more (its
+        // last reader was the gate / up phase of the layer before this one, two barriers ago), and a phase barrier lies
+        // between this and its first reader.
+        const auto park_next_layer = [&]() {
+            if (wave == 0 && lane_id() < LWORDS && !last) layer_words[(l + 1) & 1u][lane_id()] = next_word;
+        };
         uint64_t *tl = trace ? trace + 16 * l : nullptr;
         // the hand-off vectors of this layer, each behind a descriptor of its own size
         const Rsrc xa = make_rsrc(p.flow + plan::flow_xa(sh, l), dim * 4u), xb = make_rsrc(p.flow + plan::flow_xb(sh, l), dim * 4u);
@@ -717,8 +827,9 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
             const DevBuf bias = qkv_u.seg == 0 ? LAYER_BUF(lw, bv) : (qkv_u.seg == 1 ? LAYER_BUF(lw, bk) : LAYER_BUF(lw, bq));
             float bias_v = 0.0f;
             if (fresh(wave) == 0) bias_v = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(bias.rs, (int)(row * 4u), 0, AUX_PLAIN));
-            mult64_any<false>(unit_type, unit, req, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tl, wave);
-            { const DevBuf W = LAYER_BUF(lw, wo); request16(unit, req, W, wo_t, ng_o, wave); unit_type = W.type; }
+            mult64_any<false>(unit_type, unit, req, ncb, in, true, slot, lds, PHASE_PARTIAL, PHASE_RED, f, tl, wave);
+            park_next_layer();
+            ask_wo(lw);
             const float o = finish64<false>(ncb, in, PHASE_PARTIAL, PHASE_RED, tl, wave);
             if (fresh(wave) == 0) {
                 // RoPE (rope.slang:27-84) with the partner of the pair in a neighbouring lane, the row into the cache for the
@@ -747,23 +858,30 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
         } else {
             const uint32_t h = plan::attention_head(sh, b);
             stamp(tl, 0, wave);
+            // This workgroup's tile of the output projection: fetched now, while the query is being computed elsewhere,
+            // and parked in LDS -- the attention needs the registers, and asked for after it the tile would arrive late.
+            if (wave < ng_o) {
+                ask_wo(lw);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                park_unit(unit, smem, unit_type, wave);
+            }
+            park_next_layer();
             attend<F16>(sh, h, pos, LAYER_BUF(lw, kcache).rs, LAYER_BUF(lw, vcache).rs, make_rsrc(p.flow + plan::flow_qkv(sh, l, 2), dim * 4u),
                         make_rsrc(p.flow + plan::flow_qkv(sh, l, 1), dim * 4u), make_rsrc(p.flow + plan::flow_qkv(sh, l, 0), dim * 4u), xb, PHASE_PARTIAL, f, tl, wave);
             stamp(tl, 3, wave);
             ++phase;
-            // (only now: the attention needs the registers; these workgroups have no tile of the output projection)
-            { const DevBuf W = LAYER_BUF(lw, wgate); request64<true>(unit, req, W, LAYER_BUF(lw, wup), gu_u, ncb, wave); unit_type = W.type; }
+            if (wave < ng_o) unpark_unit(unit, smem, unit_type, wave); else unit = Unit{};
         }
-        // The next layer's description has arrived by now; nobody reads the slot it goes to any more (the layer before
-        // this one is over for every wave that got here), and a phase barrier lies between this and its first reader.
-        if (wave == 0 && lane_id() < LWORDS && !last) layer_words[(l + 1) & 1u][lane_id()] = next_word;
-        // ---- attention output projection into the residual (the workgroups that multiplied q / k / v) ------------------
-        if constexpr (!ATTN) {
+        // ---- attention output projection into the residual ---------------------------------------------------------------
+        {
             uint64_t *tp = tl ? tl + 4 : nullptr;
             float residual;
             stamp(tp, 0, wave);
-            mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, PHASE_PARTIAL, f, tp, wave);
-            { const DevBuf W = LAYER_BUF(lw, wgate); request64<true>(unit, req, W, LAYER_BUF(lw, wup), gu_u, ncb, wave); unit_type = W.type; }
+            // (one branch for the multiply and the request after it: the other waves hold their gate / up unit across this
+            // phase, and only so does the compiler see that these waves' registers hold nothing but the tile)
+            residual = 0.0f;
+            if (wave < ng_o) mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, lds, PHASE_PARTIAL, f, tp, wave);
+            ask_gate_up(lw);                                        // (the waves without a part in the tile: at once)
             const float o = finish16(wo_t, ng_o, PHASE_PARTIAL, tp, wave);
             const uint32_t tid = wave * 64u + lane_id();
             if (tid < 16u * wo_t.n) flow_put(xm, plan::tiles16_row(wo_t, tid), residual + o);     // transformer.rs:352-355
@@ -774,8 +892,8 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
             uint64_t *tp = tl ? tl + 8 : nullptr;
             const TileIn in{xm, true, LAYER_BUF(lw, ffn_norm).rs, dim, p.eps};
             stamp(tp, 0, wave);
-            mult64_any<true>(unit_type, unit, req, ncb, in, true, slot, PHASE_PARTIAL, PHASE_RED, f, tp, wave);
-            { const DevBuf W = LAYER_BUF(lw, wdown); request16(unit, req, W, down_t, ng_d, wave); unit_type = W.type; }
+            mult64_any<true>(unit_type, unit, req, ncb, in, true, slot, lds, PHASE_PARTIAL, PHASE_RED, f, tp, wave);
+            ask_down(lw);
             const float o = finish64<true>(ncb, in, PHASE_PARTIAL, PHASE_RED, tp, wave);
             const uint32_t tid = wave * 64u + lane_id();
             if (tid < gu_u.nrows) flow_put(hb, gu_u.row0 + tid, o);
@@ -786,16 +904,9 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
             uint64_t *tp = tl ? tl + 12 : nullptr;
             float residual;
             stamp(tp, 0, wave);
-            mult16_any(unit_type, unit, down_t, ncb_h, ng_d, hb, xm, true, residual, PHASE_PARTIAL, f, tp, wave);
-            // what this workgroup multiplies next: its q / k / v unit of the next layer, or its first tile of the output matrix
-            if (last) {
-                if (b < ntiles_out) request64<false>(unit, req, wout, wout, plan::run_unit(0u, b * 64u, plan::umin(64u, p.vocab - b * 64u)), ncb, wave);
-                unit_type = wout.type;
-            } else if constexpr (!ATTN) {
-                const DevBuf W = qkv_matrix(layer_words[(l + 1) & 1u]);
-                request64<false>(unit, req, W, W, qkv_u, ncb, wave);
-                unit_type = W.type;
-            }
+            residual = 0.0f;
+            if (wave < ng_d) mult16_any(unit_type, unit, down_t, ncb_h, ng_d, hb, xm, true, residual, lds, PHASE_PARTIAL, f, tp, wave);
+            ask_next(layer_words[(l + 1) & 1u], last);
             const float o = finish16(down_t, ng_d, PHASE_PARTIAL, tp, wave);
             const uint32_t tid = wave * 64u + lane_id();
             if (tid < 16u * down_t.n) flow_put(xnext, plan::tiles16_row(down_t, tid), residual + o);    // transformer.rs:362-365
@@ -812,7 +923,7 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
             const plan::RowUnit u = plan::run_unit(0u, tile * 64u, plan::umin(64u, p.vocab - tile * 64u));
             uint64_t *tp = first ? to : nullptr;
             stamp(tp, 0, wave);
-            mult64_any<false>(wout.type, unit, req, ncb, in, first, slot, PHASE_PARTIAL, PHASE_RED, f, tp, wave);
+            mult64_any<false>(wout.type, unit, req, ncb, in, first, slot, lds, PHASE_PARTIAL, PHASE_RED, f, tp, wave);
             const uint32_t next = tile + gridDim.x;
             if (next < ntiles_out) request64<false>(unit, req, wout, wout, plan::run_unit(0u, next * 64u, plan::umin(64u, p.vocab - next * 64u)), ncb, wave);
             const float o = finish64<false>(ncb, in, PHASE_PARTIAL, PHASE_RED, tp, wave);
@@ -839,6 +950,7 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
     // every further token would only wait out the same time limits.
     if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
     if (threadIdx.x < LWORDS) layer_words[0][threadIdx.x] = reinterpret_cast<const uint32_t *>(p.layers)[threadIdx.x];
+    if (threadIdx.x < plan::MQ_ZERO_BYTES / 4) reinterpret_cast<uint32_t *>(smem)[plan::lds_mq_zero() / 4 + threadIdx.x] = 0u;   // the zeros of mfma_q4k.h
     __syncthreads();
     const plan::Shape sh = shape_of(p);
     const uint32_t wave = uniform_word(threadIdx.x >> 6);

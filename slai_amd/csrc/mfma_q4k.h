@@ -1,0 +1,160 @@
+// Q4_K rows times an f32 vector on the matrix cores, for the row-per-lane tiled layout (quant_tiled.h).
+//
+// A lane owns one row of one 256-column super-block: nine 16-byte pieces, the header and 128 bytes of 4-bit values.  The
+// dot product of such a row with 256 activations costs the vector unit about 2.3 instructions per weight (extract, convert,
+// multiply-add); a layer's weights arrive faster than that.  v_mfma_f32_16x16x32_f16 takes eight f16 per lane and operand
+// and multiplies a 16 x 32 by a 32 x 16 matrix in the time of four vector instructions, and two facts make it usable here
+// without moving a weight between lanes:
+//
+//   * a 4-bit value n masked in place -- (w & 0x000f000f), ((w >> 8) & 0x000f000f), and the high nibbles through
+//     0x00f000f0 -- IS a pair of f16 numbers: the subnormals n * 2^-24 (16 n * 2^-24 for a high nibble).  The matrix cores
+//     take subnormal inputs exactly, so the operand costs 5/8 of an instruction per weight and nothing is rounded;
+//   * the instruction's A operand wants, from lane (g, r) = (lane / 16, lane % 16), eight values of row r and "k group" g.
+//     The 64 lanes of a wave hold 64 different (row, super-block) pairs, not 16 rows with four k groups each -- but if the
+//     B operand of k group g is non-zero in column g only, column g of the result is the dot product of the lanes of group
+//     g alone: C[r][g] = (eight weights of lane (g, r)) . (their eight activations).  Columns g and 4 + g carry the high
+//     and low halves of the activations, columns 8 + g and 12 + g the same for the steps that take the high nibbles, so
+//     one accumulator holds the two sub-blocks (scales) of a 64-column quarter apart.
+//
+// Activations: x * 2^k = hi + lo with hi, lo in f16 (22 bits of x; 2^k, per super-block, brings the largest magnitude to
+// [2^14, 2^15)), staged once per super-block in LDS in the order the masks above deliver the weights: 32 steps of
+// (8 hi | 8 lo).  A lane reads its operand from the block of its super-block if its column is one of the two that are live
+// in the step, and from a block of zeros otherwise; the choice is in the base address, the step in the immediate offset.
+// The products n * hi and n * lo are exact in f32 and the matrix cores accumulate in f32, so the result differs from the
+// f32 multiply-add chain of the vector path by accumulation order and by the 2^-22 of the split only.
+//
+// After the eight steps of a quarter the accumulator (rows 4 q .. 4 q + 3 of column c in lane (q, c)) goes through LDS to
+// the lanes that own the rows, which apply the sub-block scales as before (quantization.rs:322-389).
+#pragma once
+#include "quant_tiled.h"
+
+namespace slai {
+namespace mq {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t w32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t w32x2 __attribute__((ext_vector_type(2)));
+
+// ---- LDS layout, in bytes --------------------------------------------------------------------------------------------------
+// One staged super-block: 32 steps x (8 hi | 8 lo) f16, then eight sums of 32 activations (f32) and 2^-k.
+constexpr uint32_t SB_STEPS = 32, SB_STEP_BYTES = 32, SB_B_BYTES = SB_STEPS * SB_STEP_BYTES;
+constexpr uint32_t SB_SUMS = SB_B_BYTES, SB_INV = SB_B_BYTES + 32, SB_BYTES = SB_B_BYTES + 64;
+// the accumulator of one matrix on its way to the lanes that own the rows: [16 columns][16 rows] f32
+constexpr uint32_t CS_BYTES = 16 * 16 * 4;
+SLAI_HD uint32_t step_of(uint32_t K, uint32_t h, uint32_t nib) { return K * 4 + h * 2 + nib; }   // piece 1 + K, words (x, y) | (z, w), low | high nibbles
+
+__device__ __forceinline__ uint32_t lane_now() {
+    uint32_t l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+__device__ __forceinline__ float xor_lane(float v, int mask) {
+    const int l = (int)lane_now();
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((l ^ mask) & 63) << 2, __builtin_bit_cast(int, v)));
+}
+__device__ __forceinline__ uint32_t pack_f16(_Float16 a, _Float16 b) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+}
+
+// Stages the 256 activations of one super-block: lane i of the wave holds elements 4 i .. 4 i + 3 in `x`.  `sb`: the
+// super-block's block in LDS (SB_BYTES, 16-byte aligned).  Element e = 64 J + 32 nib + 16 H + 8 h + i' belongs to step
+// (K = 2 J + H, h, nib), at position [0, 2, 1, 3, 4, 6, 5, 7]^-1 (i') of its eight: the order in which the masks deliver the
+// weights of bytes 8 h .. 8 h + 7 of piece 1 + K.
+__device__ __forceinline__ void stage_superblock(float4 x, char *sb) {
+    const uint32_t i = lane_now();
+    float s = (x.x + x.y) + (x.z + x.w);
+    s += xor_lane(s, 1); s += xor_lane(s, 2); s += xor_lane(s, 4);                  // the 32 activations of a sub-block: 8 lanes
+    float mx = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, xor_lane(mx, m));
+    uint32_t E = (__float_as_uint(mx) >> 23) & 0xffu;                            // biased exponent of the largest magnitude
+    E = E < 30u ? 30u : E;
+    const float up = __uint_as_float((268u - E) << 23), down = __uint_as_float((E - 14u) << 23);   // 2^k, 2^-k: k = 14 - (E - 127)
+    const float a = x.x * up, b = x.y * up, c = x.z * up, d = x.w * up;
+    const _Float16 ha = (_Float16)a, hb = (_Float16)b, hc = (_Float16)c, hd = (_Float16)d;
+    const _Float16 la = (_Float16)(a - (float)ha), lb = (_Float16)(b - (float)hb), lc = (_Float16)(c - (float)hc), ld = (_Float16)(d - (float)hd);
+    const uint32_t J = i >> 4, nib = (i >> 3) & 1u, H = (i >> 2) & 1u, h = (i >> 1) & 1u;
+    char *blk = sb + step_of(2 * J + H, h, nib) * SB_STEP_BYTES + (i & 1u) * 8u;
+    *reinterpret_cast<w32x2 *>(blk) = w32x2{pack_f16(ha, hc), pack_f16(hb, hd)};
+    *reinterpret_cast<w32x2 *>(blk + 16) = w32x2{pack_f16(la, lc), pack_f16(lb, ld)};
+    if ((i & 7u) == 0) reinterpret_cast<float *>(sb + SB_SUMS)[i >> 3] = s;
+    if (i == 0) *reinterpret_cast<float *>(sb + SB_INV) = down;
+}
+
+// The dot products of this lane's row of N matrices (the same row and super-block of each: a gated pair shares the
+// activations) with the staged super-block `sb`.  `zeros`: SB_B_BYTES of zeros; `cs`: N * CS_BYTES for this wave alone.
+// Every lane of the wave takes part, whatever its row holds.
+template <int N>
+__device__ __forceinline__ void dot_q4k(const Tiled<T_Q4_K>::Data *const *d, const char *sb, const char *zeros, char *cs, float *out) {
+    const uint32_t lane = lane_now(), g = lane >> 4, col = lane & 15u;
+    // low-nibble steps live in columns g (hi half of x) and 4 + g (lo half); high-nibble steps in 8 + g and 12 + g
+    const char *b_even = col == g ? sb : (col == 4u + g ? sb + 16 : zeros);
+    const char *b_odd = col == 8u + g ? sb : (col == 12u + g ? sb + 16 : zeros);
+    float acc[N], accm[N], dd[N], dmin[N];
+    uint32_t sc_lo[N], sc_hi[N];
+    const f32x4 s0 = *reinterpret_cast<const f32x4 *>(sb + SB_SUMS), s1 = *reinterpret_cast<const f32x4 *>(sb + SB_SUMS + 16);
+    const float down = *reinterpret_cast<const float *>(sb + SB_INV);
+    const float sums[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+        const U4 &hd = d[n]->p[0];
+        dd[n] = scale_f16((uint16_t)(hd.x & 0xffffu)); dmin[n] = scale_f16((uint16_t)(hd.x >> 16));
+        // all eight 6-bit scales / mins at once (quantization.rs:381-389 applied bytewise)
+        sc_lo[n] = hd.y & 0x3f3f3f3fu;
+        sc_hi[n] = (hd.w & 0x0f0f0f0fu) | (((hd.y >> 6) & 0x03030303u) << 4);
+        const uint32_t m_lo = hd.z & 0x3f3f3f3fu;
+        const uint32_t m_hi = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
+        float am = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) am = fmaf((float)(((s < 4 ? m_lo : m_hi) >> (8 * (s & 3))) & 0xffu), sums[s], am);
+        accm[n] = am; acc[n] = 0.0f;
+    }
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {
+        f32x4 c[N];
+        __builtin_amdgcn_sched_barrier(0);                         // (the operand reads of a quarter stay in it: 32 registers, not 128)
+#pragma unroll
+        for (int n = 0; n < N; ++n) c[n] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int H = 0; H < 2; ++H) {
+            constexpr uint32_t LO = 0x000f000fu, HI = 0x00f000f0u;
+            const int K = 2 * J + H;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const half8 be = __builtin_bit_cast(half8, *reinterpret_cast<const w32x4 *>(b_even + step_of(K, h, 0) * SB_STEP_BYTES));
+                const half8 bo = __builtin_bit_cast(half8, *reinterpret_cast<const w32x4 *>(b_odd + step_of(K, h, 1) * SB_STEP_BYTES));
+#pragma unroll
+                for (int n = 0; n < N; ++n) {
+                    const U4 &q = d[n]->p[1 + K];
+                    const uint32_t w0 = h ? q.z : q.x, w1 = h ? q.w : q.y;
+                    const uint32_t v0 = w0 >> 8, v1 = w1 >> 8;
+                    const half8 ae = __builtin_bit_cast(half8, w32x4{w0 & LO, v0 & LO, w1 & LO, v1 & LO});
+                    const half8 ao = __builtin_bit_cast(half8, w32x4{w0 & HI, v0 & HI, w1 & HI, v1 & HI});
+                    c[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ae, be, c[n], 0, 0, 0);
+                    c[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ao, bo, c[n], 0, 0, 0);
+                }
+            }
+        }
+        // lane (q, col) holds rows 4 q .. 4 q + 3 of column col; lane (g, r) wants row r of columns g, 4 + g, 8 + g, 12 + g
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+            float *t = reinterpret_cast<float *>(cs + n * CS_BYTES);
+            asm volatile("" ::: "memory");
+            *reinterpret_cast<f32x4 *>(t + col * 16u + 4u * g) = c[n];
+            asm volatile("" ::: "memory");
+            const float even = t[g * 16u + col] + t[(4u + g) * 16u + col];
+            const float odd = t[(8u + g) * 16u + col] + t[(12u + g) * 16u + col];
+            asm volatile("" ::: "memory");
+            const uint32_t scw = J < 2 ? sc_lo[n] : sc_hi[n];
+            const int sh = (J & 1) * 16;
+            acc[n] = fmaf((float)((scw >> sh) & 0xffu), even, acc[n]);
+            acc[n] = fmaf((float)((scw >> (sh + 8)) & 0xffu) * 0.0625f, odd, acc[n]);      // (high nibbles were taken as 16 n)
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < N; ++n) out[n] = (dd[n] * 16777216.0f * down) * acc[n] - dmin[n] * accm[n];
+}
+
+}  // namespace mq
+}  // namespace slai
