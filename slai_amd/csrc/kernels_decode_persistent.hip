@@ -157,11 +157,25 @@ __device__ __forceinline__ void flow_backoff(Flow &f, uint64_t &deadline, uint32
     }
 }
 
+// Every wave of the device waits for its input at some point, most of them for many microseconds, and a request for a
+// hand-off vector is served by memory itself: what the waiting waves ask for competes with the weights.  So a wave first
+// watches a single word -- every lane the same one: one request of one line per round -- and only when that word is there
+// asks for its whole part, which the other producers have then written as well or are about to.
+__device__ __forceinline__ void flow_watch(Rsrc x, uint32_t word, Flow &f) {
+    uint64_t deadline = 0;
+    uint32_t rounds = 0;
+    for (;;) {
+        const uint32_t w = __builtin_amdgcn_raw_buffer_load_b32(x, (int)(word * 4u), 0, AUX_FLOW);
+        if (w != FLOW_EMPTY || f.dead) return;
+        flow_backoff(f, deadline, rounds);
+    }
+}
 // The 16 bytes of piece `piece` of a hand-off vector for every lane of the wave, once no word of any lane's piece is
 // empty: one request per lane and round, repeated by the whole wave (after a time-out the values are whatever was there).
 __device__ __forceinline__ u32x4 flow_take(Rsrc x, uint32_t piece, Flow &f) {
     uint64_t deadline = 0;
     uint32_t rounds = 0;
+    flow_watch(x, uniform_word(piece) * 4u + 255u, f);           // the last word of the wave's 64 pieces
     for (;;) {
         const u32x4 v = buf_load16<AUX_FLOW>(x, piece * 16u);
         if (!__any(flow_empty(v)) || f.dead) return v;
@@ -173,6 +187,7 @@ __device__ __forceinline__ u32x4 flow_take(Rsrc x, uint32_t piece, Flow &f) {
 __device__ __forceinline__ void flow_take4(Rsrc x, uint32_t piece0, uint32_t n, u32x4 (&out)[4], Flow &f) {
     uint64_t deadline = 0;
     uint32_t rounds = 0;
+    flow_watch(x, (uniform_word(piece0) + 64u * (n - 1u)) * 4u + 255u, f);
     for (;;) {
         bool hole = false;
 #pragma unroll
@@ -188,14 +203,7 @@ __device__ __forceinline__ void flow_take4(Rsrc x, uint32_t piece0, uint32_t n, 
 __device__ __forceinline__ void flow_take_strided(Rsrc x, uint32_t first, float (&out)[16], Flow &f) {
     uint64_t deadline = 0;
     uint32_t rounds = 0;
-    // While the vector is not there yet, one word per lane is asked for instead of sixteen -- a different one of the
-    // sixteen in each lane of a row, so that the wave as a whole looks at every run of 16 floats it will take: every
-    // wave of the device polls at this point, and sixteen times the requests would slow down the very stores waited for.
-    for (;;) {
-        const uint32_t w = __builtin_amdgcn_raw_buffer_load_b32(x, (int)((first + 16u * (lane_id() & 15u)) * 4u), 0, AUX_FLOW);
-        if (!__any(w == FLOW_EMPTY) || f.dead) break;
-        flow_backoff(f, deadline, rounds);
-    }
+    flow_watch(x, uniform_word(first) + 255u, f);
     for (;;) {
         uint32_t u[16];
 #pragma unroll
@@ -441,7 +449,7 @@ __device__ __forceinline__ void mult16(const Unit &u, const plan::Tiles16 t, uin
             u32x4 xv[4];
             flow_take4(x, plan::tile16_piece(g, 0, (uint32_t)lane), n, xv, f);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) mq::stage_superblock(as_float4(xv[k]), lds + plan::lds_mq_sb(wave, k));
+            for (int k = 0; k < 4; ++k) mq::stage_superblock(as_float4(xv[k]), lds + plan::lds_mq_sb(wave, k));   // (past the end: zeros)
             stamp(tr, 1, wave);
             typename F::Data d;
 #pragma unroll
@@ -622,6 +630,7 @@ __device__ __forceinline__ void attend(const plan::Shape &sh, uint32_t head, uin
         const uint32_t first = plan::att_k_elem(head, lane_id());
         uint64_t deadline = 0;
         uint32_t rounds = 0;
+        flow_watch(q, head * 128u + 127u, f);
         for (;;) {
             u32x4 v[4];
 #pragma unroll
@@ -881,10 +890,13 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
             // phase, and only so does the compiler see that these waves' registers hold nothing but the tile)
             residual = 0.0f;
             if (wave < ng_o) mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, lds, PHASE_PARTIAL, f, tp, wave);
-            ask_gate_up(lw);                                        // (the waves without a part in the tile: at once)
+            // The waves without a part in the tile ask at once -- except where the attention has only just ended: there the
+            // tile's waves are still polling, behind everything this compute unit has asked for.
+            if (!ATTN || wave < ng_o) ask_gate_up(lw);
             const float o = finish16(wo_t, ng_o, PHASE_PARTIAL, tp, wave);
             const uint32_t tid = wave * 64u + lane_id();
             if (tid < 16u * wo_t.n) flow_put(xm, plan::tiles16_row(wo_t, tid), residual + o);     // transformer.rs:352-355
+            if (ATTN && wave >= ng_o) ask_gate_up(lw);
             ++phase;
         }
         // ---- RMSNorm + gate / up + SiLU ---------------------------------------------------------------------------------

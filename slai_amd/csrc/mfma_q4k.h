@@ -83,7 +83,7 @@ __device__ __forceinline__ void stage_superblock(float4 x, char *sb) {
 }
 
 // The dot products of this lane's row of N matrices (the same row and super-block of each: a gated pair shares the
-// activations) with the staged super-block `sb`.  `zeros`: SB_B_BYTES of zeros; `cs`: N * CS_BYTES for this wave alone.
+// activations) with the staged super-block `sb`.  `zeros`: SB_BYTES of zeros (a lane without a super-block may name it as `sb`); `cs`: N * CS_BYTES for this wave alone.
 // Every lane of the wave takes part, whatever its row holds.
 template <int N>
 __device__ __forceinline__ void dot_q4k(const Tiled<T_Q4_K>::Data *const *d, const char *sb, const char *zeros, char *cs, float *out) {
