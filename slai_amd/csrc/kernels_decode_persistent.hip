@@ -67,9 +67,11 @@ __device__ __forceinline__ float lane_xor(float v, int mask) {
     return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((l ^ mask) & 63) << 2, __builtin_bit_cast(int, v)));
 }
 __device__ __forceinline__ float wave_total(float v) {            // the sum over the wave, in every lane
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += lane_xor(v, m);
-    return v;
+    v += mq::dpp<mq::DPP_XOR1>(v); v += mq::dpp<mq::DPP_XOR2>(v); v += mq::dpp<mq::DPP_HALF_MIRROR>(v); v += mq::dpp<mq::DPP_MIRROR>(v);
+    const int b = __builtin_bit_cast(int, v);                   // every lane of a row of 16 holds the row's sum
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
 }
 
 // Optional time stamps (the constant 100 MHz clock) for a per-phase time line of every workgroup: profilers see one long

@@ -49,9 +49,25 @@ __device__ __forceinline__ uint32_t lane_now() {
     asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
     return l;
 }
-__device__ __forceinline__ float xor_lane(float v, int mask) {
-    const int l = (int)lane_now();
-    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((l ^ mask) & 63) << 2, __builtin_bit_cast(int, v)));
+// Lane exchanges as operand modifiers (no LDS round trip, no lane index): within quads, half rows (8 lanes) and rows (16).
+template <int CTRL> __device__ __forceinline__ float dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E;               // quad_perm [1,0,3,2], [2,3,0,1]
+constexpr int DPP_HALF_MIRROR = 0x141, DPP_MIRROR = 0x140;    // lane i <-> 7 - i of its half row, 15 - i of its row
+// sum over the 8 lanes of a half row, in all of them
+__device__ __forceinline__ float sum8(float v) {
+    v += dpp<DPP_XOR1>(v); v += dpp<DPP_XOR2>(v); v += dpp<DPP_HALF_MIRROR>(v);
+    return v;
+}
+// the largest of a non-negative value's bit patterns over the wave, as a wave-uniform word
+__device__ __forceinline__ uint32_t max64_bits(float v) {
+    v = fmaxf(v, dpp<DPP_XOR1>(v)); v = fmaxf(v, dpp<DPP_XOR2>(v)); v = fmaxf(v, dpp<DPP_HALF_MIRROR>(v)); v = fmaxf(v, dpp<DPP_MIRROR>(v));
+    const int b = __builtin_bit_cast(int, v);
+    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane(b, 0), r1 = (uint32_t)__builtin_amdgcn_readlane(b, 16);
+    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane(b, 32), r3 = (uint32_t)__builtin_amdgcn_readlane(b, 48);
+    const uint32_t a = r0 > r1 ? r0 : r1, c = r2 > r3 ? r2 : r3;
+    return a > c ? a : c;
 }
 __device__ __forceinline__ uint32_t pack_f16(_Float16 a, _Float16 b) {
     return (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
@@ -63,12 +79,9 @@ __device__ __forceinline__ uint32_t pack_f16(_Float16 a, _Float16 b) {
 // weights of bytes 8 h .. 8 h + 7 of piece 1 + K.
 __device__ __forceinline__ void stage_superblock(float4 x, char *sb) {
     const uint32_t i = lane_now();
-    float s = (x.x + x.y) + (x.z + x.w);
-    s += xor_lane(s, 1); s += xor_lane(s, 2); s += xor_lane(s, 4);                  // the 32 activations of a sub-block: 8 lanes
-    float mx = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, xor_lane(mx, m));
-    uint32_t E = (__float_as_uint(mx) >> 23) & 0xffu;                            // biased exponent of the largest magnitude
+    const float s = sum8((x.x + x.y) + (x.z + x.w));                           // the 32 activations of a sub-block: 8 lanes
+    const float mx = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
+    uint32_t E = (max64_bits(mx) >> 23) & 0xffu;                                // biased exponent of the largest magnitude
     E = E < 30u ? 30u : E;
     const float up = __uint_as_float((268u - E) << 23), down = __uint_as_float((E - 14u) << 23);   // 2^k, 2^-k: k = 14 - (E - 127)
     const float a = x.x * up, b = x.y * up, c = x.z * up, d = x.w * up;
