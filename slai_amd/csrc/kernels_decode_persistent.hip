@@ -719,23 +719,6 @@ __device__ __forceinline__ void attend(const plan::Shape &sh, uint32_t head, uin
     }
 }
 
-// A wave's unit of a 16-row tile parked in LDS and taken back: the attention needs the registers in between.
-__device__ __forceinline__ void park_unit(const Unit &u, float *lds, int type, uint32_t wave) {
-    const uint32_t lane = lane_id(), pt = tiled_pieces(type);
-#pragma unroll
-    for (int P = 0; P < (int)plan::PARK_PIECES; ++P)
-        if ((uint32_t)P < pt) *reinterpret_cast<U4 *>(lds + plan::lds_park_piece(wave, P, lane)) = u.a[P];
-    reinterpret_cast<uint32_t *>(lds)[plan::lds_park_tail(wave, lane)] = u.ta;
-}
-__device__ __forceinline__ void unpark_unit(Unit &u, const float *lds, int type, uint32_t wave) {
-    const uint32_t lane = lane_id(), pt = tiled_pieces(type);
-    u = Unit{};
-#pragma unroll
-    for (int P = 0; P < (int)plan::PARK_PIECES; ++P)
-        if ((uint32_t)P < pt) u.a[P] = *reinterpret_cast<const U4 *>(lds + plan::lds_park_piece(wave, P, lane));
-    u.ta = (uint16_t)reinterpret_cast<const uint32_t *>(lds)[plan::lds_park_tail(wave, lane)];
-}
-
 __device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
     return plan::Shape{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, gridDim.x, p.qkv_units, p.gu_rows, p.rope_variant == SLAI_ROPE_NEOX ? 1u : 0u};
 }
@@ -869,36 +852,24 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
         } else {
             const uint32_t h = plan::attention_head(sh, b);
             stamp(tl, 0, wave);
-            // This workgroup's tile of the output projection: fetched now, while the query is being computed elsewhere,
-            // and parked in LDS -- the attention needs the registers, and asked for after it the tile would arrive late.
-            if (wave < ng_o) {
-                ask_wo(lw);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                park_unit(unit, smem, unit_type, wave);
-            }
             park_next_layer();
             attend<F16>(sh, h, pos, LAYER_BUF(lw, kcache).rs, LAYER_BUF(lw, vcache).rs, make_rsrc(p.flow + plan::flow_qkv(sh, l, 2), dim * 4u),
                         make_rsrc(p.flow + plan::flow_qkv(sh, l, 1), dim * 4u), make_rsrc(p.flow + plan::flow_qkv(sh, l, 0), dim * 4u), xb, PHASE_PARTIAL, f, tl, wave);
             stamp(tl, 3, wave);
             ++phase;
-            if (wave < ng_o) unpark_unit(unit, smem, unit_type, wave); else unit = Unit{};
+            // (only now: the attention needs the registers; these workgroups have no tile of the output projection)
+            ask_gate_up(lw);
         }
-        // ---- attention output projection into the residual ---------------------------------------------------------------
-        {
+        // ---- attention output projection into the residual (the workgroups that multiplied q / k / v) ------------------
+        if constexpr (!ATTN) {
             uint64_t *tp = tl ? tl + 4 : nullptr;
             float residual;
             stamp(tp, 0, wave);
-            // (one branch for the multiply and the request after it: the other waves hold their gate / up unit across this
-            // phase, and only so does the compiler see that these waves' registers hold nothing but the tile)
-            residual = 0.0f;
-            if (wave < ng_o) mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, lds, PHASE_PARTIAL, f, tp, wave);
-            // The waves without a part in the tile ask at once -- except where the attention has only just ended: there the
-            // tile's waves are still polling, behind everything this compute unit has asked for.
-            if (!ATTN || wave < ng_o) ask_gate_up(lw);
+            mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, lds, PHASE_PARTIAL, f, tp, wave);
+            ask_gate_up(lw);                                        // (the waves without a part in the tiles: at once)
             const float o = finish16(wo_t, ng_o, PHASE_PARTIAL, tp, wave);
             const uint32_t tid = wave * 64u + lane_id();
             if (tid < 16u * wo_t.n) flow_put(xm, plan::tiles16_row(wo_t, tid), residual + o);     // transformer.rs:352-355
-            if (ATTN && wave >= ng_o) ask_gate_up(lw);
             ++phase;
         }
         // ---- RMSNorm + gate / up + SiLU ---------------------------------------------------------------------------------
@@ -919,7 +890,7 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
             float residual;
             stamp(tp, 0, wave);
             residual = 0.0f;
-            if (wave < ng_d) mult16_any(unit_type, unit, down_t, ncb_h, ng_d, hb, xm, true, residual, lds, PHASE_PARTIAL, f, tp, wave);
+            mult16_any(unit_type, unit, down_t, ncb_h, ng_d, hb, xm, true, residual, lds, PHASE_PARTIAL, f, tp, wave);
             ask_next(layer_words[(l + 1) & 1u], last);
             const float o = finish16(down_t, ng_d, PHASE_PARTIAL, tp, wave);
             const uint32_t tid = wave * 64u + lane_id();

@@ -85,15 +85,6 @@ SLAI_HD uint32_t lds_mq_wave(uint32_t wave) { return lds_mq_zero() + MQ_ZERO_BYT
 SLAI_HD uint32_t lds_mq_sb(uint32_t wave, uint32_t k) { return lds_mq_wave(wave) + k * MQ_SB_BYTES; }
 SLAI_HD uint32_t lds_mq_cs(uint32_t wave) { return lds_mq_wave(wave) + 4 * MQ_SB_BYTES; }
 SLAI_HD uint32_t lds_bytes(const Shape &) { return lds_mq_wave(WG_WAVES); }
-// ... and, in the same bytes, the weights of one 16-row tile parked while the registers are needed for something else (up
-// to four waves' units of thirteen 16-byte pieces per lane and a 2-byte tail, kept as a word): [wave][piece][lane], then
-// [wave][lane].  They lie in the blocks of waves 4 and up, which stage nothing between the parking and the taking back
-// (those waves have no part in the 16-row-tile phase that follows).
-constexpr uint32_t PARK_WAVES = 4, PARK_PIECES = 13;
-SLAI_HD uint32_t lds_park() { return lds_mq_wave(PARK_WAVES) / 4; }                                     // in floats
-SLAI_HD uint32_t lds_park_piece(uint32_t wave, uint32_t piece, uint32_t lane) { return lds_park() + ((wave * PARK_PIECES + piece) * 64 + lane) * 4; }
-SLAI_HD uint32_t lds_park_tail(uint32_t wave, uint32_t lane) { return lds_park() + PARK_WAVES * PARK_PIECES * 64 * 4 + wave * 64 + lane; }
-SLAI_HD uint32_t lds_park_end() { return lds_park() + PARK_WAVES * PARK_PIECES * 64 * 4 + PARK_WAVES * 64; }
 SLAI_HD uint32_t lds_floats(const Shape &s) { return lds_bytes(s) / 4; }
 
 // ---- the attention of a head over the cached positions: eight lanes per position for the scores (sixteen elements
@@ -149,13 +140,19 @@ SLAI_HD uint32_t attention_head(const Shape &s, uint32_t b) { return b - qkv_wor
 SLAI_HD uint32_t gu_units(const Shape &s) { return (s.hidden + s.gu_rows - 1) / s.gu_rows; }
 SLAI_HD RowUnit gu_unit(const Shape &s, uint32_t b) { return run_unit(0u, b * s.gu_rows, umin(s.gu_rows, s.hidden - b * s.gu_rows)); }
 
-// The two projections into the residual, in 16-row tiles (dim / 16 of them = the grid): workgroup b takes tile b of
-// both.  (A workgroup may take two tiles side by side on other waves; no shape does at present.)
+// The two projections into the residual, in 16-row tiles (dim / 16 of them = the grid).  Down projection: workgroup b
+// takes tile b.  Attention output projection: the workgroups that run a head's attention have just finished when it
+// starts and hold none of its weights, so they take no tile; the q / k / v workgroup b takes tile b, and the one with a
+// head's last q unit also the tile 7 * n_heads + head, side by side on other waves.
 struct Tiles16 { uint32_t n, tile0, tile1; };      // (two named fields: an indexed pair would live in memory on the device)
 SLAI_HD uint32_t tiles16_tile(const Tiles16 &t, uint32_t k) { return k == 0 ? t.tile0 : t.tile1; }
 SLAI_HD uint32_t proj_tiles(const Shape &s) { return s.dim / 16; }
 SLAI_HD Tiles16 down_tiles(const Shape &, uint32_t b) { return Tiles16{1u, b, b}; }
-SLAI_HD Tiles16 wo_tiles(const Shape &, uint32_t b) { return Tiles16{1u, b, b}; }
+SLAI_HD Tiles16 wo_tiles(const Shape &s, uint32_t b) {
+    if (b >= qkv_workgroups(s)) return Tiles16{0u, 0u, 0u};
+    if ((b >> 3) % s.qkv_units == s.qkv_units - 1) return Tiles16{2u, b, qkv_workgroups(s) + qkv_head(s, b)};
+    return Tiles16{1u, b, b};
+}
 // the row thread i < 16 * t.n of the workgroup finishes
 SLAI_HD uint32_t tiles16_row(const Tiles16 &t, uint32_t i) { return 16u * tiles16_tile(t, (i >> 4) & 1u) + (i & 15u); }
 

@@ -97,19 +97,7 @@ void walk_stage64(Audit &a, const plan::Shape &s, const Region &x, const Region 
     for (uint32_t i = 0; i < seen.size(); ++i)
         if (seen[i] != 1) { a.fail("64-row-unit phase: a piece of the input is staged " + std::to_string(seen[i]) + " times"); break; }
     if ((uint64_t)n + n / 16 > plan::slot_stride(s)) a.fail("the slot is smaller than the staged input");
-    if ((uint64_t)plan::lds_set(1) + plan::lds_red() + 2 * plan::WG_WAVES > plan::lds_park() || ncb > plan::WG_WAVES) a.fail("LDS block smaller than what the phases index");
-    // the parked tile of the attention workgroups: ncb / 4 waves of up to thirteen pieces and a tail word per lane
-    if (plan::lds_mq_zero() < (plan::lds_set(1) + plan::lds_red() + 2 * plan::WG_WAVES) * 4 || plan::lds_mq_zero() % 16 || plan::lds_mq_sb(0, 0) % 16 || plan::MQ_SB_BYTES % 16
-        || plan::lds_mq_cs(plan::WG_WAVES - 1) + 2 * plan::MQ_CS_BYTES > plan::lds_bytes(s) || plan::lds_mq_sb(0, 0) < plan::lds_mq_zero() + plan::MQ_ZERO_BYTES)
-        a.fail("the LDS blocks of the matrix-core phases overlap or are misaligned");
-    if (plan::lds_bytes(s) > 160 * 1024) a.fail("more LDS than a compute unit has");
-    if (ncb / 4 > plan::PARK_WAVES || plan::lds_park() % 4 || plan::lds_park() * 4 < plan::lds_mq_wave(plan::PARK_WAVES) || plan::lds_park_end() > plan::lds_floats(s))
-        a.fail("more waves park a tile than there is room for");
-    for (uint32_t w = 0; w < ncb / 4; ++w)
-        for (uint32_t lane = 0; lane < 64; ++lane) {
-            if ((uint64_t)plan::lds_park_piece(w, plan::PARK_PIECES - 1, lane) + 4 > plan::lds_park_tail(0, 0) || plan::lds_park_piece(w, 0, lane) % 4) a.fail("parked pieces overlap the tails");
-            if (plan::lds_park_tail(w, lane) >= plan::lds_floats(s)) a.fail("parked tail beyond the LDS block");
-        }
+    if (ncb > plan::WG_WAVES) a.fail("more super-blocks than waves");
 }
 
 // a 16-row tile phase: the weights of the multiplying waves (tile k of the workgroup on waves k * ngroups ..), the sixteen
@@ -267,6 +255,7 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                 a.touch(counters, (uint64_t)handoff_heads * 32 * 4, 4, "abort flag", b, 0, 0, l);
                 {
                     const plan::Tiles16 wt = plan::wo_tiles(s, b), dt = plan::down_tiles(s, b);
+                    if (plan::is_attention_workgroup(s, b) != (wt.n == 0)) a.fail("exactly the attention workgroups take no tile of the output projection");
                     walk_tile16(a, wo, to, wt, ncb, ng_o, xb, dim, l == 0 ? xemb : xa, xm, rows_o, b, l);
                     walk_tile16(a, wd, td, dt, ncb_h, ng_d, hb, hidden, xm, xnext, rows_d, b, l);
                 }
