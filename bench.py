@@ -38,6 +38,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 TRAFFIC_PROFILE = os.path.join("profiles", "gate_up_gemv_q4k_hbm_counters.md")
+RESIDENT_TRAFFIC_PROFILE = os.path.join("profiles", "resident_decode_llama2_7b_q4k_hbm_counters.md")
 
 
 def dominant_kernel_traffic():
@@ -47,6 +48,16 @@ def dominant_kernel_traffic():
     import re
     try:
         m = re.search(r"=\s*\*\*(\d+) B\*\*", open(os.path.join(ROOT, TRAFFIC_PROFILE)).read())
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def resident_kernel_traffic():
+    """The same for the resident launch of a whole token (`bench.py --probe-resident` under the counters)."""
+    import re
+    try:
+        m = re.search(r"=\s*\*\*(\d+) B\*\*", open(os.path.join(ROOT, RESIDENT_TRAFFIC_PROFILE)).read())
         return int(m.group(1)) if m else None
     except OSError:
         return None
@@ -142,6 +153,36 @@ def counter_probe(backend):
     print(json.dumps({"probe": "copy kernel 67108864 B read + 67108864 B written per launch (64 launches); "
                                "gate/up GEMV %d algorithmic bytes per launch" % algo,
                       "gemv_launch_us": round(ms * 1000, 2)}))
+
+
+def counter_probe_resident(backend, seed, pos=192, reps=8):
+    """For hardware-counter runs of the resident launch: 64 launches of the copy kernel of known size, then the
+    configuration-4 model (all 32 layers), 64 prompt positions through the chunked pass, and `reps` + 3 tokens at one
+    position launched from the host (embedding row, emptying of the hand-off buffers, the resident launch), nothing else."""
+    from slai_amd import _ffi
+    from slai_amd import gguf_writer as gw
+    from slai_amd.runtime import Gguf, GpuTensor, Llama2, LlmContext
+    n = 16 * 1024 * 1024
+    a = GpuTensor(backend, n)
+    b = GpuTensor(backend, n)
+    ctxt = LlmContext(backend)
+    for _ in range(64):
+        ctxt.copy(a, b)
+    backend.synchronize()
+    a.destroy(); b.destroy()
+    data = gw.llama_gguf(dim=CFG["dim"], hidden_dim=CFG["hidden_dim"], n_layers=CFG["n_layers"], n_heads=CFG["n_heads"], n_kv_heads=CFG["n_kv_heads"],
+                         vocab=CFG["vocab"], seq_len=512, wtype=12, v_type=14, out_type=14, embd_type=12, seed=seed, distinct_layers=4)
+    g = Gguf(data)
+    m = Llama2(backend, g, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+    assert m.decode_form() == 1, "the model did not take the resident launch"
+    prompt = np.random.Generator(np.random.PCG64(seed)).integers(0, CFG["vocab"], pos).astype(np.int32)
+    m.prefill(prompt, 0, 0)
+    steps = m.time_steps(pos, 17, reps=reps)
+    tb = token_bytes(CFG, m.weight_bytes(), pos, pos)
+    m.destroy(); g.close()
+    print(json.dumps({"probe": "copy kernel 67108864 B read + 67108864 B written per launch (64 launches); resident launch of a token at position %d, "
+                               "%d algorithmic bytes per launch (%d launches)" % (pos, tb, reps + 3),
+                      "launches_us": {name: round(us, 2) for name, us, _, _ in steps}}))
 
 
 EAGER = False        # --eager: launch from the host instead of replaying a HIP graph (for runs under the kernel tracer)
@@ -424,6 +465,7 @@ def main():
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-side", action="store_true", help="only the headline decode (no sampled decode, prompt chunks, config 5)")
     ap.add_argument("--probe", action="store_true", help="counter probe: copy kernel + dominant GEMV only")
+    ap.add_argument("--probe-resident", action="store_true", help="counter probe: copy kernel + the resident launch of a few tokens only")
     ap.add_argument("--sweep", action="store_true", help="per-format GEMV sweep and long-context attention instead of the decode run")
     ap.add_argument("--eager", action="store_true", help="with --sweep: launch from the host, no HIP graph (the kernel tracer cannot follow graph launches here)")
     args = ap.parse_args()
@@ -431,13 +473,13 @@ def main():
         print("bench.py: this build runs the decode path on ONE GPU (batch-1 decode does not shard usefully); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    if args.probe or args.sweep:
+    if args.probe or args.probe_resident or args.sweep:
         global EAGER
         EAGER = args.eager
         from slai_amd.runtime import Backend
         backend = Backend(0)
-        if args.probe:
-            counter_probe(backend)
+        if args.probe or args.probe_resident:
+            counter_probe_resident(backend, args.seed) if args.probe_resident else counter_probe(backend)
         else:
             sweep(backend)
         backend.close()
@@ -480,6 +522,15 @@ def main():
     log("decode: %.3f ms/token (events), wall %.3f ms/token, %.1f tok/s, %.2f GB/token -> %.1f GB/s"
         % (ms_per_step, wall * 1000 / K, tok_s, tb / 1e9, tb / ms_per_step / 1e6))
     steps = None
+    resident_us = None
+    if form == 1 and not args.no_roofline:
+        # the launches of a token with an event after each (launched from the host, 8 tokens at the middle position): the
+        # embedding row, the emptying of the hand-off buffers, the resident launch of the layer stack and the output matrix
+        mid = pos0 + K // 2
+        steps = [dict(step=name, us_per_launch=round(us, 2), launches_per_token=per, us_between_events_in_a_token=round(us, 2))
+                 for name, us, per, _ in model.time_steps(mid, int(toks[K // 2 - 1]), reps=8)]
+        resident_us = next(e["us_per_launch"] for e in steps if e["step"] == "llama2 resident token")
+        log("launches of a token: " + "; ".join("%s %.2f us" % (e["step"], e["us_per_launch"]) for e in steps))
     if form == 0 and not args.no_roofline:
         # every launch of a token, timed with an event after each (launched from the host, 8 tokens at the middle position)
         mid = pos0 + K // 2
@@ -513,14 +564,13 @@ def main():
     roof = None
     if not args.no_roofline:
         if form == 1:
-            # the resident launch is the token: embedding gather, buffer fill and the pick (three small launches) are the
-            # only other kernels and are part of the measured time, so this is a lower bound of the launch's own rate
-            ach = tb / (ms_per_step * 1e-3) / 1e9
-            roof = dict(bound="hbm", kernel="llama_decode_persistent_kernel (all 32 layers: RMSNorm + q/k/v, RoPE + attention, output projection, "
+            # the resident launch is nearly the whole token: its bytes are the token's bytes less the embedding row
+            ach = tb / (resident_us * 1e-6) / 1e9
+            roof = dict(bound="hbm", kernel="llama_decode_persistent_kernel (all 32 layers: RMSNorm + q/k/v + RoPE + cache write, attention, output projection, "
                                             "RMSNorm + gate/up + SiLU, down projection; final norm + output matrix): one launch per token",
-                        achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4), traffic=None,
-                        launch_us=round(ms_per_step * 1000, 2), algorithmic_bytes=int(tb),
-                        how="token bytes over the mean time per token of the timed loop (HIP events on the library's stream)")
+                        achieved=round(ach, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4), traffic=resident_kernel_traffic(),
+                        traffic_source=RESIDENT_TRAFFIC_PROFILE, launch_us=resident_us, algorithmic_bytes=int(tb),
+                        how="HIP events on the library's stream before and after the launch, 8 tokens at position %d launched from the host" % (pos0 + K // 2))
         else:
             kms, kalgo = measure_dominant_kernel(backend)
             ach = kalgo / (kms * 1e-3) / 1e9

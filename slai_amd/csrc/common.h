@@ -87,8 +87,8 @@ struct slai_ctx {
     std::vector<void *> retired_scratch;
     std::vector<slai_buffer *> retired_buffers;   // cached tensors a captured graph may name, and buffers destroyed inside a capture
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
-    // SLAI_PERSISTENT=1: the one-launch-per-token form of the Llama-2 layer stack where a model's shapes allow it (off by default)
-    bool persistent = false;
+    // the one-launch-per-token form of the Llama-2 layer stack where a model's shapes allow it (SLAI_PERSISTENT=0 switches it off)
+    bool persistent = true;
     // When set, every launch of a decode step is followed by an event recorded under the step's name
     // (slai_llama2_time_steps); null otherwise.
     std::vector<std::pair<const char *, hipEvent_t>> *step_marks = nullptr;

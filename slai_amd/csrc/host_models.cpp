@@ -11,6 +11,7 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 
@@ -338,8 +339,10 @@ int slai_llama2::load(const slai_gguf *gg) {
     TRY(ensure_attn_scratch(ctx, attention_scratch_floats(config.n_q_heads, head_size(), attn_splits)));
     TRY(loop_init(ctx, loop, config.seq_len + 1));
     TRY(persistent_setup());
-    if (ctx->persistent && !persistent.ready)
-        fprintf(stderr, "slai: SLAI_PERSISTENT=1, but this model keeps one launch per step: %s\n", persistent.why_not ? persistent.why_not : "unknown");
+    // (said only to a caller who asked for the form by name: most models simply have other shapes)
+    const char *asked = getenv("SLAI_PERSISTENT");
+    if (asked && ctx->persistent && !persistent.ready)
+        fprintf(stderr, "slai: SLAI_PERSISTENT=%s, but this model keeps one launch per step: %s\n", asked, persistent.why_not ? persistent.why_not : "unknown");
     return slai_synchronize(ctx);
 }
 
@@ -430,8 +433,11 @@ int slai_llama2::enqueue_persistent(int sampler) {
     Llama2State &s = state;
     DecodeState *ds = (DecodeState *)loop.state->dptr;
     SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, &ds->token, nullptr, nullptr, config.dim, (float *)s.x.buf->dptr));
+    TRY(step_mark(ctx, "embedding row"));
     SLAI_HIP_TRY(ctx, launch_flow_fill(ctx->stream, persistent.flow->dptr, persistent.flow_bytes));
+    TRY(step_mark(ctx, "hand-off buffers emptied"));
     SLAI_HIP_TRY(ctx, launch_decode_persistent(ctx->stream, persistent.params, persistent.grid));
+    TRY(step_mark(ctx, "llama2 resident token"));
     if (sampler == 1)
         SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, nullptr, ds,
                                         (const int *)loop.prompt->dptr, (int *)loop.out_tokens->dptr));
@@ -930,19 +936,19 @@ SLAI_EXPORT int slai_llama2_trace_token(slai_llama2 *m, uint32_t pos, uint32_t t
     return rc;
 }
 
-// One token through the launch-per-step form, launched from the host `reps` times at the same position, with an event
-// after every launch: mean time from the end of the launch before to the end of each launch, by step name in order of
+// One token, launched from the host `reps` times at the same position, with an event after every launch (the resident
+// form: the embedding row, the emptying of the hand-off buffers and the one launch of the layer stack): mean time from the end of the launch before to the end of each launch, by step name in order of
 // first appearance (`names`: newline separated), and how often the step occurs per token.
 SLAI_EXPORT int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t token, uint32_t reps, char *names, size_t names_len, float *mean_us,
                                        float *alone_us, uint32_t *per_token, uint32_t capacity, uint32_t *n_steps) {
     if (!m || !names || !mean_us || !alone_us || !per_token || !n_steps || reps == 0) return SLAI_E_ARG;
     slai_ctx *ctx = m->ctx;
-    if (m->persistent.ready) return set_error(ctx, SLAI_E_STATE, "slai_llama2_time_steps: this model takes the resident launch, which has no steps to time");
     if (pos >= m->config.seq_len || token >= m->config.vocab_size) return set_error(ctx, SLAI_E_ARG, "slai_llama2_time_steps: position or token out of range");
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_llama2_time_steps: not during graph capture");
     DecodeState ds{(int)pos, (int)token, 0, 0};
     TRY(slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds));
-    TRY(m->enqueue_fused(0));                                   // untimed: sizes scratch, warms the caches
+    const auto enqueue = [&]() { return m->persistent.ready ? m->enqueue_persistent(0) : m->enqueue_fused(0); };
+    TRY(enqueue());                                             // untimed: sizes scratch, warms the caches
     TRY(slai_synchronize(ctx));
     std::vector<std::pair<const char *, hipEvent_t>> marks;
     marks.reserve((size_t)reps * (5 * m->config.n_layers + 4));
@@ -950,7 +956,7 @@ SLAI_EXPORT int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t to
     int rc = SLAI_OK;
     for (uint32_t r = 0; r < reps && !rc; ++r) {
         rc = step_mark(ctx, nullptr);                           // where the token starts
-        if (!rc) rc = m->enqueue_fused(0);
+        if (!rc) rc = enqueue();
     }
     ctx->step_marks = nullptr;
     if (!rc) rc = slai_synchronize(ctx);
@@ -986,6 +992,7 @@ SLAI_EXPORT int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t to
     SLAI_HIP_TRY(ctx, hipEventCreate(&e0));
     SLAI_HIP_TRY(ctx, hipEventCreate(&e1));
     for (size_t k = 0; k < order.size() && !rc; ++k) {
+        if (m->persistent.ready) { alone_us[k] = mean_us[k]; continue; }     // (a resident launch needs the buffers emptied before it: never alone)
         ctx->only_step = order[k];
         rc = m->enqueue_fused(0);                               // untimed
         if (!rc && hipEventRecord(e0, ctx->stream) != hipSuccess) rc = SLAI_E_HIP;
@@ -1002,7 +1009,7 @@ SLAI_EXPORT int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t to
     if (rc == SLAI_E_HIP) return set_error(ctx, SLAI_E_HIP, "slai_llama2_time_steps: event");
     if (rc) return rc;
     // leave the state a whole forward at this position leaves
-    TRY(m->enqueue_fused(0));
+    TRY(enqueue());
     TRY(slai_synchronize(ctx));
     return handoff_check(ctx);
 }

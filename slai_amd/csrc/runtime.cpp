@@ -90,7 +90,7 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->tiled_layout = env_int("SLAI_TILED", 1) != 0;
     ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
     ctx->fuse_qkv_attention = env_int("SLAI_FUSE_QKV_ATTN", 1) != 0;
-    ctx->persistent = env_int("SLAI_PERSISTENT", 0) != 0;
+    ctx->persistent = env_int("SLAI_PERSISTENT", 1) != 0;
     *out = ctx;
     return SLAI_OK;
 }

@@ -86,18 +86,33 @@ def fused_vs_op_sequence(backend, data, prompt, n_steps, kv_fill=None, start_pos
 CONFIG4_PROMPT, CONFIG4_TOKENS = 64, 256     # "Prompt is 64 seeded token ids; greedy decode of 256 tokens"
 
 
-def took_the_fused_qkv_attention_launch(m, pos, token):
-    """Whether the model's decode sequence runs q/k/v + attention as the one launch the headline figure is quoted on
-    (`qkv_attention_kernel`): slai_llama2_time_steps names every launch of a token."""
+def backend_of_form(resident):
+    """A context whose Llama-2 models take the resident launch where their shapes allow it (the default), or never."""
+    import os
+    from slai_amd.runtime import Backend
+    os.environ["SLAI_PERSISTENT"] = "1" if resident else "0"
+    try:
+        return Backend(0)
+    finally:
+        del os.environ["SLAI_PERSISTENT"]
+
+
+def took_the_launches_the_metric_is_quoted_on(m, pos, token, resident):
+    """Whether the model's decode sequence is the one the headline figure is quoted on: the whole layer stack in one
+    resident launch per token (`llama_decode_persistent_kernel`), or, with that form switched off, q/k/v + attention as one
+    launch per layer (`qkv_attention_kernel`).  slai_llama2_time_steps names every launch of a token."""
     names = [s[0] for s in m.time_steps(pos, token, reps=1)]
-    return "llama2 qkv + attention" in names and "llama2 attention" not in names and "llama2 qkv" not in names
+    if resident:
+        return m.decode_form() == 1 and "llama2 resident token" in names and not any("attention" in n or "qkv" in n for n in names)
+    return m.decode_form() == 0 and "llama2 qkv + attention" in names and "llama2 attention" not in names and "llama2 qkv" not in names
 
 
-def test_config4_depth2_vs_oracle_at_the_metric_positions(backend):
+@pytest.mark.parametrize("resident", [True, False], ids=["one resident launch per token", "one launch per step"])
+def test_config4_depth2_vs_oracle_at_the_metric_positions(resident):
     """Configuration 4's layer shapes (dim 4096, 32 heads of 128, FFN 11008, vocab 32000, Q4_K with Q6_K v-proj and output,
     fp16 cache) at depth 2 against the oracle over ALL the positions the metric is quoted on: 64 seeded prompt ids + 256
-    greedy tokens = positions 0 .. 319, which takes the fused q/k/v + attention launch through its second and third pass
-    over the cache (128 positions per pass).  Ids identical (chat_llama2.rs:105-158 loop, cpu.rs:488-539 attention);
+    greedy tokens = positions 0 .. 319, which takes the attention through its second and third pass over the cache (128
+    positions per pass), in both launch forms.  Ids identical (chat_llama2.rs:105-158 loop, cpu.rs:488-539 attention);
     logits within the bar at the pass boundaries and at both ends, through the fused kernels one token at a time."""
     from slai_amd.runtime import Gguf, Llama2
     data = gw.llama_gguf(dim=4096, hidden_dim=11008, n_layers=2, n_heads=32, n_kv_heads=32, vocab=32000, seq_len=512, wtype=12, v_type=14,
@@ -111,39 +126,49 @@ def test_config4_depth2_vs_oracle_at_the_metric_positions(backend):
     ref_tokens = np.zeros(n, np.int32); ref_logits = np.zeros((n, 32000), np.float32)
     print("config 4 depth 2: oracle run", flush=True)
     assert L.slo_llama2_generate(om, prompt.ctypes.data, prompt.size, 0, n, -1, ref_tokens.ctypes.data, ref_logits.ctypes.data) == n
-    gg = Gguf(data)
-    m = Llama2(backend, gg, _ffi.MODEL_LLAMA, _ffi.KV_F16)
-    assert m.decode_form() == 0
-    print("config 4 depth 2: device run", flush=True)
-    got, _ = m.generate(prompt, n)
-    assert np.array_equal(got, ref_tokens), (np.flatnonzero(got != ref_tokens)[:4].tolist(), got.tolist(), ref_tokens.tolist())
-    assert took_the_fused_qkv_attention_launch(m, 5, int(prompt[5]))
-    # the caches hold the whole run: the logits of any position can be recomputed in place
-    worst = 0.0
-    for pos in (0, 1, 63, 64, 126, 127, 128, 129, 191, 192, 255, 256, 257, 318, 319):
-        tok = int(prompt[pos]) if pos < CONFIG4_PROMPT else int(ref_tokens[pos - 1])
-        for fused in (True, False):
-            err = rel_err(m.forward_logits(pos, tok, fused=fused), ref_logits[pos])
-            worst = max(worst, err)
-            assert err < LOGIT_TOL, (pos, fused, err)
-    print("config 4 depth 2, positions 0..319: worst logits rel err %.2e" % worst)
-    m.destroy(); gg.close(); L.slo_llama2_free(om); g.close()
+    backend = backend_of_form(resident)
+    try:
+        gg = Gguf(data)
+        m = Llama2(backend, gg, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+        assert m.decode_form() == int(resident)
+        print("config 4 depth 2: device run", flush=True)
+        got, _ = m.generate(prompt, n)
+        assert np.array_equal(got, ref_tokens), (np.flatnonzero(got != ref_tokens)[:4].tolist(), got.tolist(), ref_tokens.tolist())
+        assert took_the_launches_the_metric_is_quoted_on(m, 5, int(prompt[5]), resident)
+        # the caches hold the whole run: the logits of any position can be recomputed in place
+        worst = 0.0
+        for pos in (0, 1, 63, 64, 126, 127, 128, 129, 191, 192, 255, 256, 257, 318, 319):
+            tok = int(prompt[pos]) if pos < CONFIG4_PROMPT else int(ref_tokens[pos - 1])
+            for fused in (True, False):
+                err = rel_err(m.forward_logits(pos, tok, fused=fused), ref_logits[pos])
+                worst = max(worst, err)
+                assert err < LOGIT_TOL, (pos, fused, err)
+        print("config 4 depth 2, positions 0..319: worst logits rel err %.2e" % worst)
+        m.destroy(); gg.close()
+    finally:
+        backend.close()
+    L.slo_llama2_free(om); g.close()
 
 
-def test_config4_llama7b_q4k_full_depth(backend):
+@pytest.mark.parametrize("resident", [True, False], ids=["one resident launch per token", "one launch per step"])
+def test_config4_llama7b_q4k_full_depth(resident):
     """Llama-2-7B shape at its full 32 layers (Q4_K, Q6_K v-proj / output, fp16 cache, context 512) over the metric's own
-    run: 64 prompt ids + 256 greedy tokens (positions 0 .. 319) from the decode graph equal those of the op-by-op
-    sequence, and the graph is the one with the fused q/k/v + attention launch."""
+    run: 64 prompt ids + 256 greedy tokens (positions 0 .. 319) from the decode loop equal those of the op-by-op
+    sequence, and the loop is made of the launches the headline figure is quoted on, in both launch forms."""
     from slai_amd.runtime import Gguf, Llama2
     data = gw.llama_gguf(dim=4096, hidden_dim=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000, seq_len=512, wtype=12, v_type=14,
                          out_type=14, embd_type=12, seed=1234, distinct_layers=4)
     prompt = np.random.Generator(np.random.PCG64(1234)).integers(0, 32000, CONFIG4_PROMPT)
-    gg = Gguf(data)
-    probe = Llama2(backend, gg, _ffi.MODEL_LLAMA, _ffi.KV_F16)
-    assert probe.decode_form() == 0 and took_the_fused_qkv_attention_launch(probe, 0, int(prompt[0]))
-    probe.destroy(); gg.close()
-    worst, ms = fused_vs_op_sequence(backend, data, prompt, CONFIG4_PROMPT + CONFIG4_TOKENS)
-    print("config 4 at 32 layers, positions 0..319: worst logits rel err %.2e, %.3f ms/token" % (worst, ms))
+    backend = backend_of_form(resident)
+    try:
+        gg = Gguf(data)
+        probe = Llama2(backend, gg, _ffi.MODEL_LLAMA, _ffi.KV_F16)
+        assert took_the_launches_the_metric_is_quoted_on(probe, 0, int(prompt[0]), resident)
+        probe.destroy(); gg.close()
+        worst, ms = fused_vs_op_sequence(backend, data, prompt, CONFIG4_PROMPT + CONFIG4_TOKENS)
+        print("config 4 at 32 layers, positions 0..319: worst logits rel err %.2e, %.3f ms/token" % (worst, ms))
+    finally:
+        backend.close()
 
 
 def seeded_kv(seed, layer, n_pos, kv_dim):
