@@ -201,27 +201,6 @@ __device__ __forceinline__ void flow_take4(Rsrc x, uint32_t piece0, uint32_t n, 
         flow_backoff(f, deadline, rounds);
     }
 }
-// Sixteen floats per lane, 16 apart from float `first` on (the register layout of DevX), under the same rule.
-__device__ __forceinline__ void flow_take_strided(Rsrc x, uint32_t first, float (&out)[16], Flow &f) {
-    uint64_t deadline = 0;
-    uint32_t rounds = 0;
-    flow_watch(x, uniform_word(first) + 255u, f);
-    for (;;) {
-        uint32_t u[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) u[i] = __builtin_amdgcn_raw_buffer_load_b32(x, (int)((first + 16u * i) * 4u), 0, AUX_FLOW);
-        bool hole = false;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) hole = hole || u[i] == FLOW_EMPTY;
-        if (!__any(hole) || f.dead) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) out[i] = __uint_as_float(u[i]);
-            return;
-        }
-        flow_backoff(f, deadline, rounds);
-    }
-}
-
 // ---- weights on their way ---------------------------------------------------------------------------------------------------
 // A phase's multiply cannot start before its input exists, but its weights do not depend on anything: each wave asks
 // for the unit of its NEXT phase as soon as the registers of the current one are free (right after its dot product,
@@ -308,7 +287,7 @@ __device__ __forceinline__ void mult64(const Unit &u, const Req &r, uint32_t ncb
     const uint32_t wave = fresh(wave_);
     constexpr int NM = DUAL ? 2 : 1;
     float v = 0.0f, v2 = 0.0f;
-    if constexpr (T == T_Q4_K) {
+    if constexpr (T == T_Q4_K || T == T_Q6_K) {
         // on the matrix cores (mfma_q4k.h): the wave stages its super-block in LDS, for itself alone
         if ((uint32_t)wave < ncb) {
             char *sb = lds + plan::lds_mq_sb(wave, 0);
@@ -320,7 +299,7 @@ __device__ __forceinline__ void mult64(const Unit &u, const Req &r, uint32_t ncb
                 ss = wave_total(ss);
                 if (lane == 0) red[wave] = ss;
                 x.x *= w.x; x.y *= w.y; x.z *= w.z; x.w *= w.w;
-                mq::stage_superblock(x, sb);
+                mq::stage_superblock<T>(x, sb);
             }
             stamp(tr, 1, wave);
             typename F::Data d, e;
@@ -330,13 +309,18 @@ __device__ __forceinline__ void mult64(const Unit &u, const Req &r, uint32_t ncb
 #pragma unroll
                 for (int i = 0; i < F::PT; ++i) e.p[i] = u.b[i];
             }
-            const typename F::Data *dp[NM];
-            float o2[NM];
-            dp[0] = &d;
-            if constexpr (DUAL) dp[1] = &e;
-            mq::dot_q4k<NM>(dp, sb, lds + plan::lds_mq_zero(), lds + plan::lds_mq_cs(wave), o2);
-            v = o2[0];
-            if constexpr (DUAL) v2 = o2[1];
+            if constexpr (T == T_Q6_K) {
+                static_assert(!DUAL, "gated pairs are Q4_K");
+                v = mq::dot_q6k(d, u.ta, sb, lds + plan::lds_mq_zero(), lds + plan::lds_mq_cs(wave));
+            } else {
+                const typename F::Data *dp[NM];
+                float o2[NM];
+                dp[0] = &d;
+                if constexpr (DUAL) dp[1] = &e;
+                mq::dot_q4k<NM>(dp, sb, lds + plan::lds_mq_zero(), lds + plan::lds_mq_cs(wave), o2);
+                v = o2[0];
+                if constexpr (DUAL) v2 = o2[1];
+            }
         }
     } else if ((uint32_t)wave < ncb) {
         if (stage) {
@@ -443,50 +427,28 @@ __device__ __forceinline__ void mult16(const Unit &u, const plan::Tiles16 t, uin
         const uint32_t off = (plan::tiles16_row(t, (uint32_t)lane)) * 4u;
         residual = __uint_as_float(res_flow ? __builtin_amdgcn_raw_buffer_load_b32(res, (int)off, 0, AUX_FLOW) : __builtin_amdgcn_raw_buffer_load_b32(res, (int)off, 0, AUX_PLAIN));
     }
-    if constexpr (T == T_Q4_K) {
-        // on the matrix cores (mfma_q4k.h): the wave stages its four super-blocks in LDS, for itself alone
-        if (wave < ngroups * t.n) {
-            const uint32_t g = wave % ngroups;
-            const uint32_t n = plan::umin(4u, ncb - plan::tile16_sb(g, 0));
-            u32x4 xv[4];
-            flow_take4(x, plan::tile16_piece(g, 0, (uint32_t)lane), n, xv, f);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) mq::stage_superblock(as_float4(xv[k]), lds + plan::lds_mq_sb(wave, k));   // (past the end: zeros)
-            stamp(tr, 1, wave);
-            typename F::Data d;
-#pragma unroll
-            for (int i = 0; i < F::PT; ++i) d.p[i] = u.a[i];
-            const typename F::Data *dp[1] = {&d};
-            float o1[1];
-            mq::dot_q4k<1>(dp, lds + plan::lds_mq_sb(wave, (uint32_t)lane >> 4), lds + plan::lds_mq_zero(), lds + plan::lds_mq_cs(wave), o1);
-            v = o1[0];
-            v += lane_xor(v, 16);
-            v += lane_xor(v, 32);                                  // across the four super-blocks of the wave
-        }
-    } else if (wave < ngroups * t.n) {
+    // on the matrix cores (mfma_q4k.h): the wave stages its four super-blocks in LDS, for itself alone
+    static_assert(T == T_Q4_K || T == T_Q6_K, "the projections into the residual are Q4_K or Q6_K");
+    if (wave < ngroups * t.n) {
         const uint32_t g = wave % ngroups;
-        const bool valid = plan::tile16_cb(g, (uint32_t)lane) < ncb;
-        DevX X;
-        flow_take_strided(x, plan::tile16_x0(g, (uint32_t)lane, ncb), X.x, f);
+        const uint32_t n = plan::umin(4u, ncb - plan::tile16_sb(g, 0));
+        u32x4 xv[4];
+        flow_take4(x, plan::tile16_piece(g, 0, (uint32_t)lane), n, xv, f);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) X.x[i] = valid ? X.x[i] : 0.0f;
+        for (int k = 0; k < 4; ++k) mq::stage_superblock<T>(as_float4(xv[k]), lds + plan::lds_mq_sb(wave, k));   // (past the end: zeros)
         stamp(tr, 1, wave);
-        if constexpr (T == T_Q6_K) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) X.s[i] = row16_sum(X.x[i]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 16; i += 2) { X.s[i] = row16_sum(X.x[i] + X.x[i + 1]); X.s[i + 1] = 0.0f; }
-        }
         typename F::Data d;
 #pragma unroll
         for (int i = 0; i < F::PT; ++i) d.p[i] = u.a[i];
-        uint16_t dt = u.ta;
-        const typename F::Data *dp[1] = {&d};
-        uint16_t tails[1] = {dt};
-        float o1[1];
-        F::template dotn<1>(dp, tails, X, o1);                       // the whole unit was requested ahead
-        v = o1[0];
+        const char *sb = lds + plan::lds_mq_sb(wave, (uint32_t)lane >> 4);
+        if constexpr (T == T_Q6_K) {
+            v = mq::dot_q6k(d, u.ta, sb, lds + plan::lds_mq_zero(), lds + plan::lds_mq_cs(wave));
+        } else {
+            const typename F::Data *dp[1] = {&d};
+            float o1[1];
+            mq::dot_q4k<1>(dp, sb, lds + plan::lds_mq_zero(), lds + plan::lds_mq_cs(wave), o1);
+            v = o1[0];
+        }
         v += lane_xor(v, 16);
         v += lane_xor(v, 32);                                      // across the four super-blocks of the wave
     }

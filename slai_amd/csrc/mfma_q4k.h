@@ -37,12 +37,15 @@ typedef uint32_t w32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t w32x2 __attribute__((ext_vector_type(2)));
 
 // ---- LDS layout, in bytes --------------------------------------------------------------------------------------------------
-// One staged super-block: 32 steps x (8 hi | 8 lo) f16, then eight sums of 32 activations (f32) and 2^-k.
+// One staged super-block: 32 steps x (8 hi | 8 lo) f16, then the sums of its activations (eight of 32 for Q4_K, sixteen of
+// 16 for Q6_K; f32) and 2^-k.
 constexpr uint32_t SB_STEPS = 32, SB_STEP_BYTES = 32, SB_B_BYTES = SB_STEPS * SB_STEP_BYTES;
-constexpr uint32_t SB_SUMS = SB_B_BYTES, SB_INV = SB_B_BYTES + 32, SB_BYTES = SB_B_BYTES + 64;
+constexpr uint32_t SB_SUMS = SB_B_BYTES, SB_INV = SB_B_BYTES + 64, SB_BYTES = SB_B_BYTES + 80;
 // the accumulator of one matrix on its way to the lanes that own the rows: [16 columns][16 rows] f32
 constexpr uint32_t CS_BYTES = 16 * 16 * 4;
-SLAI_HD uint32_t step_of(uint32_t K, uint32_t h, uint32_t nib) { return K * 4 + h * 2 + nib; }   // piece 1 + K, words (x, y) | (z, w), low | high nibbles
+SLAI_HD uint32_t step_of(uint32_t K, uint32_t h, uint32_t nib) { return K * 4 + h * 2 + nib; }   // Q4_K: piece 1 + K, words (x, y) | (z, w), low | high nibbles
+// Q6_K: 128-half I, l-range M (l = 16 M ..), quadrant r, words (x, y) | (z, w): the sixteen weights of scale 8 I + 2 r + M in two steps
+SLAI_HD uint32_t step_of_q6k(uint32_t I, uint32_t M, uint32_t r, uint32_t h) { return ((I * 2 + M) * 4 + r) * 2 + h; }
 
 __device__ __forceinline__ uint32_t lane_now() {
     uint32_t l;
@@ -74,12 +77,14 @@ __device__ __forceinline__ uint32_t pack_f16(_Float16 a, _Float16 b) {
 }
 
 // Stages the 256 activations of one super-block: lane i of the wave holds elements 4 i .. 4 i + 3 in `x`.  `sb`: the
-// super-block's block in LDS (SB_BYTES, 16-byte aligned).  Element e = 64 J + 32 nib + 16 H + 8 h + i' belongs to step
-// (K = 2 J + H, h, nib), at position [0, 2, 1, 3, 4, 6, 5, 7]^-1 (i') of its eight: the order in which the masks deliver the
-// weights of bytes 8 h .. 8 h + 7 of piece 1 + K.
+// super-block's block in LDS (SB_BYTES, 16-byte aligned).  Q4_K: element e = 64 J + 32 nib + 16 H + 8 h + i' belongs to
+// step (K = 2 J + H, h, nib); Q6_K: e = 128 I + 32 r + 16 M + 8 h + i' to step (I, M, r, h).  In both it stands at position
+// [0, 2, 1, 3, 4, 6, 5, 7]^-1 (i') of the step's eight: the order in which the masks deliver the weights of bytes
+// 8 h .. 8 h + 7 of a piece.
+template <int T>
 __device__ __forceinline__ void stage_superblock(float4 x, char *sb) {
+    static_assert(T == T_Q4_K || T == T_Q6_K, "formats with a matrix-core path");
     const uint32_t i = lane_now();
-    const float s = sum8((x.x + x.y) + (x.z + x.w));                           // the 32 activations of a sub-block: 8 lanes
     const float mx = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
     uint32_t E = (max64_bits(mx) >> 23) & 0xffu;                                // biased exponent of the largest magnitude
     E = E < 30u ? 30u : E;
@@ -87,11 +92,20 @@ __device__ __forceinline__ void stage_superblock(float4 x, char *sb) {
     const float a = x.x * up, b = x.y * up, c = x.z * up, d = x.w * up;
     const _Float16 ha = (_Float16)a, hb = (_Float16)b, hc = (_Float16)c, hd = (_Float16)d;
     const _Float16 la = (_Float16)(a - (float)ha), lb = (_Float16)(b - (float)hb), lc = (_Float16)(c - (float)hc), ld = (_Float16)(d - (float)hd);
-    const uint32_t J = i >> 4, nib = (i >> 3) & 1u, H = (i >> 2) & 1u, h = (i >> 1) & 1u;
-    char *blk = sb + step_of(2 * J + H, h, nib) * SB_STEP_BYTES + (i & 1u) * 8u;
+    uint32_t step;
+    if constexpr (T == T_Q4_K) {
+        const float s = sum8((x.x + x.y) + (x.z + x.w));                       // the 32 activations of a sub-block: 8 lanes
+        if ((i & 7u) == 0) reinterpret_cast<float *>(sb + SB_SUMS)[i >> 3] = s;
+        step = step_of(2 * (i >> 4) + ((i >> 2) & 1u), (i >> 1) & 1u, (i >> 3) & 1u);
+    } else {
+        float s = (x.x + x.y) + (x.z + x.w);                                   // the 16 activations of a scale: 4 lanes
+        s += dpp<DPP_XOR1>(s); s += dpp<DPP_XOR2>(s);
+        if ((i & 3u) == 0) reinterpret_cast<float *>(sb + SB_SUMS)[i >> 2] = s;
+        step = step_of_q6k(i >> 5, (i >> 2) & 1u, (i >> 3) & 3u, (i >> 1) & 1u);
+    }
+    char *blk = sb + step * SB_STEP_BYTES + (i & 1u) * 8u;
     *reinterpret_cast<w32x2 *>(blk) = w32x2{pack_f16(ha, hc), pack_f16(hb, hd)};
     *reinterpret_cast<w32x2 *>(blk + 16) = w32x2{pack_f16(la, lc), pack_f16(lb, ld)};
-    if ((i & 7u) == 0) reinterpret_cast<float *>(sb + SB_SUMS)[i >> 3] = s;
     if (i == 0) *reinterpret_cast<float *>(sb + SB_INV) = down;
 }
 
@@ -167,6 +181,77 @@ __device__ __forceinline__ void dot_q4k(const Tiled<T_Q4_K>::Data *const *d, con
     }
 #pragma unroll
     for (int n = 0; n < N; ++n) out[n] = (dd[n] * 16777216.0f * down) * acc[n] - dmin[n] * accm[n];
+}
+
+// The same for a Q6_K row (quantization.rs:204-244): value = d * scale * (q - 32), q = low 4 bits | high 2 bits << 4.  The six
+// bits of a weight are put together in place -- (ql & 0x000f000f) | ((qh << 4) & 0x00300030) and its relatives -- into the
+// subnormal q * 2^-24 (16 q * 2^-24 for the weights whose low bits are a high nibble); the sixteen weights of a scale
+// are two steps, two scales share an accumulator (columns g, 4 + g and 8 + g, 12 + g), and the -32 goes through the
+// sums of the activations.  `tail`: d.
+__device__ __forceinline__ float dot_q6k(const Tiled<T_Q6_K>::Data &d, uint16_t tail, const char *sb, const char *zeros, char *cs) {
+    const uint32_t lane = lane_now(), g = lane >> 4, col = lane & 15u;
+    const char *b_even = col == g ? sb : (col == 4u + g ? sb + 16 : zeros);
+    const char *b_odd = col == 8u + g ? sb : (col == 12u + g ? sb + 16 : zeros);
+    const float down = *reinterpret_cast<const float *>(sb + SB_INV);
+    const U4 scp = d.p[12];
+    const auto scale = [scp](int I, int M, int r) {              // scales[8 I + 2 r + M]
+        const uint32_t w = r < 2 ? (I == 0 ? scp.x : scp.z) : (I == 0 ? scp.y : scp.w);
+        return (float)(int8_t)((w >> (8 * (M + 2 * (r & 1)))) & 0xff);
+    };
+    float acc = 0.0f, c32 = 0.0f;
+#pragma unroll
+    for (int IM = 0; IM < 4; ++IM) {
+        const int I = IM / 2, M = IM % 2;
+        const U4 &ql0 = d.p[4 * I + M], &ql32 = d.p[4 * I + 2 + M], &qh = d.p[8 + 2 * I + M];
+#pragma unroll
+        for (int rp = 0; rp < 2; ++rp) {                         // quadrants 2 rp (low bits in ql0) and 2 rp + 1 (in ql32)
+            const uint32_t mlo = rp ? 0x00f000f0u : 0x000f000fu, mhi = rp ? 0x03000300u : 0x00300030u;
+            __builtin_amdgcn_sched_barrier(0);
+            f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                __builtin_amdgcn_sched_barrier(0);
+                // the high bits of quadrant r of bytes (0, 2) | (1, 3), moved next to the low bits: r even <- bits 0-1 | 4-5 of
+                // the byte, r odd <- bits 2-3 | 6-7.  (One quadrant after the other: fewer values alive at a time.)
+                const uint32_t h0 = h ? qh.z : qh.x, h1 = h ? qh.w : qh.y;
+                {
+                    const uint32_t a0 = h ? ql0.z : ql0.x, a1 = h ? ql0.w : ql0.y;
+                    const half8 ae = __builtin_bit_cast(half8, w32x4{((h0 << 4) & mhi) | (a0 & mlo), ((h0 >> 4) & mhi) | ((a0 >> 8) & mlo),
+                                                                      ((h1 << 4) & mhi) | (a1 & mlo), ((h1 >> 4) & mhi) | ((a1 >> 8) & mlo)});
+                    const half8 be = __builtin_bit_cast(half8, *reinterpret_cast<const w32x4 *>(b_even + step_of_q6k(I, M, 2 * rp, h) * SB_STEP_BYTES));
+                    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(ae, be, c, 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                {
+                    const uint32_t b0 = h ? ql32.z : ql32.x, b1 = h ? ql32.w : ql32.y;
+                    const half8 ao = __builtin_bit_cast(half8, w32x4{((h0 << 2) & mhi) | (b0 & mlo), ((h0 >> 6) & mhi) | ((b0 >> 8) & mlo),
+                                                                      ((h1 << 2) & mhi) | (b1 & mlo), ((h1 >> 6) & mhi) | ((b1 >> 8) & mlo)});
+                    const half8 bo = __builtin_bit_cast(half8, *reinterpret_cast<const w32x4 *>(b_odd + step_of_q6k(I, M, 2 * rp + 1, h) * SB_STEP_BYTES));
+                    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(ao, bo, c, 0, 0, 0);
+                }
+            }
+            float *t = reinterpret_cast<float *>(cs);
+            asm volatile("" ::: "memory");
+            *reinterpret_cast<f32x4 *>(t + col * 16u + 4u * g) = c;
+            asm volatile("" ::: "memory");
+            const float even = t[g * 16u + col] + t[(4u + g) * 16u + col];
+            const float odd = t[(8u + g) * 16u + col] + t[(12u + g) * 16u + col];
+            asm volatile("" ::: "memory");
+            const float f = rp ? 0.0625f : 1.0f;                 // (the weights of quadrants 2 and 3 were taken as 16 q)
+            acc = fmaf(scale(I, M, 2 * rp) * f, even, acc);
+            acc = fmaf(scale(I, M, 2 * rp + 1) * f, odd, acc);
+        }
+    }
+    // (the -32 of every weight last, when the registers of the weights are free)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const f32x4 s4 = *reinterpret_cast<const f32x4 *>(sb + SB_SUMS + 16 * q);      // sums 4 q .. 4 q + 3: I = q / 2, r = 2 (q % 2) + {0, 0, 1, 1}, M = {0, 1, 0, 1}
+        const int I = q / 2, r0 = 2 * (q % 2);
+        c32 = fmaf(scale(I, 0, r0), s4.x, c32); c32 = fmaf(scale(I, 1, r0), s4.y, c32);
+        c32 = fmaf(scale(I, 0, r0 + 1), s4.z, c32); c32 = fmaf(scale(I, 1, r0 + 1), s4.w, c32);
+    }
+    return scale_f16(tail) * (16777216.0f * down * acc - 32.0f * c32);
 }
 
 }  // namespace mq
