@@ -88,6 +88,7 @@ typedef uint32_t u32x4b __attribute__((ext_vector_type(4)));
 constexpr int RSRC_WORD3 = 0x00020000;                        // untyped 32-bit data, no swizzle
 constexpr int AUX_PLAIN = 0;
 constexpr int AUX_FLOW = (int)0x80000010u;                    // agent scope (sc1): not served by a cache of this die; never merged or hoisted
+constexpr int AUX_ONCE = (int)0x80000000u;                    // through the caches like any load, but never merged or hoisted
 struct DevBuf {                                               // wave-uniform
     Rsrc rs;
     const void *ptr;
@@ -178,6 +179,15 @@ __device__ __forceinline__ u32x4 flow_take(Rsrc x, uint32_t piece, Flow &f) {
     uint64_t deadline = 0;
     uint32_t rounds = 0;
     flow_watch(x, uniform_word(piece) * 4u + 255u, f);           // the last word of the wave's 64 pieces
+    // Every workgroup takes the whole vector: asked of memory 256 times over, that is what a hand-off costs.  The first
+    // request therefore goes through the die's L2 like any load, and the workgroups of a die share one fetch.  A line
+    // that was cached before its producer wrote it shows empty words (a word only ever changes from empty to its value,
+    // and no line survives from an earlier launch: the caches are invalidated when a kernel starts), and then the
+    // requests go to memory as before.
+    {
+        const u32x4 v = buf_load16<AUX_ONCE>(x, piece * 16u);
+        if (!__any(flow_empty(v))) return v;
+    }
     for (;;) {
         const u32x4 v = buf_load16<AUX_FLOW>(x, piece * 16u);
         if (!__any(flow_empty(v)) || f.dead) return v;
@@ -190,6 +200,15 @@ __device__ __forceinline__ void flow_take4(Rsrc x, uint32_t piece0, uint32_t n, 
     uint64_t deadline = 0;
     uint32_t rounds = 0;
     flow_watch(x, (uniform_word(piece0) + 64u * (n - 1u)) * 4u + 255u, f);
+    {                                                             // (through the die's L2 first: see flow_take)
+        bool hole = false;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            out[k] = u32x4{0u, 0u, 0u, 0u};
+            if ((uint32_t)k < n) { out[k] = buf_load16<AUX_ONCE>(x, (piece0 + 64u * k) * 16u); hole = hole || flow_empty(out[k]); }
+        }
+        if (!__any(hole)) return;
+    }
     for (;;) {
         bool hole = false;
 #pragma unroll
