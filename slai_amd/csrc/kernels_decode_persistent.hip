@@ -7,17 +7,17 @@
 // where they are and hand the vectors over themselves:
 //   * a producer writes its slice of the vector with agent-scope stores into a buffer that was filled with FLOW_EMPTY
 //     before the launch (one buffer per layer and vector, so nothing is ever reused inside a launch);
-//   * a consumer repeats its agent-scope load of a piece until no element of it is empty -- the data is its own flag, so
-//     a hand-off is one store and one load deep, with no counter or barrier round trip in between;
-//   * the waves that multiply request the weights of their next unit first and only then wait: the weights travel
-//     while the activations are still being produced.  Loads retire in issue order, so the waiting is done by other waves
-//     of the workgroup ("stagers", which hold no outstanding weight requests) and handed over through LDS or through a
-//     per-workgroup slot that the multiplying waves read with scalar loads.
-// The arithmetic is that of the separate kernels (kernels_gemv_rowtile.hip, kernels_gemv_tiled.hip, attention_fast.h):
-// 64-row tiles with wave-uniform activations for q/k/v, gate/up and the output matrix, 16-row tiles with DPP-broadcast
-// activations for the two projections that add into the residual, one workgroup per head for the attention.  Work is
-// cut into units of equal size rather than whole tiles (resident_plan.h): a unit of a 64-row-tile matrix is any run of up
-// to 64 rows, so that every compute unit streams the same number of bytes in a phase.
+//   * a consumer watches one word of the vector until it is there, then repeats its load of its whole part until no
+//     element of it is empty -- the data is its own flag: no counter, no fence, no barrier round trip;
+//   * a wave asks for the weights of its NEXT phase as soon as the registers of the current one are free, right after its
+//     dot product: the weights travel while the hand-off is waited for.  Loads retire in issue order, so a wave's poll
+//     waits behind its own requests: every wave waits for its own input itself, with the unit it multiplies next asked
+//     for one phase earlier (and nothing may be spilled: a scratch reload waits behind the requested weights too).
+// The workgroups that multiply q, k and v also add the bias, rotate, and write the cache row; the attention of a head is
+// one workgroup that asks for the cached rows before the query exists.  Q4_K and Q6_K dot products run on the matrix
+// cores (mfma_q4k.h), Q5_K on the vector unit with wave-uniform activations (kernels_gemv_rowtile.hip's arithmetic).
+// Work is cut into units of equal size rather than whole tiles (resident_plan.h): a unit of a 64-row-tile matrix is any
+// run of up to 64 rows, so that every compute unit streams the same number of bytes in a phase.
 //
 // Where things are: every offset the kernel forms comes from resident_plan.h, which a host program walks for every
 // (workgroup, wave, lane, layer) against the sizes of the allocations.  Weights, norm vectors and hand-off vectors are

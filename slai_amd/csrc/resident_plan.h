@@ -1,6 +1,7 @@
 // Who does what, and where every access lands, in the resident decode kernel (kernels_decode_persistent.hip): the roles
 // of the workgroups in each phase of a layer, the byte offsets of the weights a lane requests, the pieces of a hand-off
-// vector a staging lane fetches, the rows of the hand-off buffers, the per-workgroup slots, counters and trace rows.
+// vector a lane takes, the rows of the hand-off buffers and of the caches, the blocks of LDS, the per-workgroup slots and
+// trace rows.
 //
 // Everything here is plain integer arithmetic that compiles for the device and for the host: the kernel forms its
 // addresses with these functions and nothing else, and a host program (tests/native/resident_bounds.cpp) walks every
