@@ -185,6 +185,41 @@ def counter_probe_resident(backend, seed, pos=192, reps=8):
                       "launches_us": {name: round(us, 2) for name, us, _, _ in steps}}))
 
 
+def counter_probe_gqa(backend, seed, pos=4047, n_caches=10, rounds=4):
+    """For hardware-counter runs of the attention of a grouped-query model: 64 launches of the copy kernel of known size,
+    then the attention operator on a Qwen2-7B-shaped layer (28 query heads on 4 kv heads of 128, fp16 cache, context 4096)
+    at position `pos`, over `n_caches` distinct cache pairs, launched from the host.  SLAI_GQA_ON_DIE=0 in the environment
+    gives the plain workgroup order for comparison."""
+    from slai_amd import _ffi
+    from slai_amd.runtime import GpuTensor, LlmContext
+    n = 16 * 1024 * 1024
+    a = GpuTensor(backend, n)
+    b = GpuTensor(backend, n)
+    ctxt = LlmContext(backend)
+    for _ in range(64):
+        ctxt.copy(a, b)
+    backend.synchronize()
+    a.destroy(); b.destroy()
+    nh, nkv, hs, seq_len = 28, 4, 128, 4096
+    kv_dim = nkv * hs
+    rng = np.random.Generator(np.random.PCG64(seed))
+    caches = [(GpuTensor(backend, kv_dim, seq_len, _ffi.DT_F16, data=rng.standard_normal((seq_len, kv_dim), dtype=np.float32).astype(np.float16)),
+               GpuTensor(backend, kv_dim, seq_len, _ffi.DT_F16, data=rng.standard_normal((seq_len, kv_dim), dtype=np.float32).astype(np.float16))) for _ in range(n_caches)]
+    params = _ffi.AttnParams(seq_len, kv_dim, nh // nkv, nh, hs, pos, (0, 0))
+    gparams = GpuTensor.scalar(backend, params)
+    gq = GpuTensor.vector(backend, rng.standard_normal(nh * hs, dtype=np.float32))
+    gatt, gxb = GpuTensor(backend, seq_len, nh), GpuTensor(backend, nh * hs)
+    backend.timer_begin()
+    for _ in range(rounds):
+        for kc, vc in caches:
+            ctxt.attention(params, gparams, gq, kc, vc, gatt, gxb)
+    us = backend.timer_end() * 1000.0 / (rounds * n_caches)
+    print(json.dumps({"probe": "copy kernel 67108864 B read + 67108864 B written per launch (64 launches); attention of 28 query heads on 4 kv heads of 128 "
+                               "at position %d, fp16 cache: %d algorithmic bytes per call (%d calls over %d cache pairs)"
+                               % (pos, 2 * (pos + 1) * kv_dim * 2, rounds * n_caches, n_caches),
+                      "us_per_call": round(us, 2), "on_die": os.environ.get("SLAI_GQA_ON_DIE", "1")}))
+
+
 EAGER = False        # --eager: launch from the host instead of replaying a HIP graph (for runs under the kernel tracer)
 
 
@@ -466,6 +501,7 @@ def main():
     ap.add_argument("--no-side", action="store_true", help="only the headline decode (no sampled decode, prompt chunks, config 5)")
     ap.add_argument("--probe", action="store_true", help="counter probe: copy kernel + dominant GEMV only")
     ap.add_argument("--probe-resident", action="store_true", help="counter probe: copy kernel + the resident launch of a few tokens only")
+    ap.add_argument("--probe-gqa", action="store_true", help="counter probe: copy kernel + the attention of a grouped-query layer only")
     ap.add_argument("--sweep", action="store_true", help="per-format GEMV sweep and long-context attention instead of the decode run")
     ap.add_argument("--eager", action="store_true", help="with --sweep: launch from the host, no HIP graph (the kernel tracer cannot follow graph launches here)")
     args = ap.parse_args()
@@ -473,12 +509,14 @@ def main():
         print("bench.py: this build runs the decode path on ONE GPU (batch-1 decode does not shard usefully); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    if args.probe or args.probe_resident or args.sweep:
+    if args.probe or args.probe_resident or args.probe_gqa or args.sweep:
         global EAGER
         EAGER = args.eager
         from slai_amd.runtime import Backend
         backend = Backend(0)
-        if args.probe or args.probe_resident:
+        if args.probe_gqa:
+            counter_probe_gqa(backend, args.seed)
+        elif args.probe or args.probe_resident:
             counter_probe_resident(backend, args.seed) if args.probe_resident else counter_probe(backend)
         else:
             sweep(backend)

@@ -14,6 +14,7 @@
 // In the model path the kernel also performs RoPE (rope.slang:27-84) on q and on the fresh key
 // and writes the fresh key/value into the cache, so Q/K/V leave the projection GEMV exactly once.
 #include "common.h"
+#include <cstdlib>
 #include "device_util.h"
 #include "attention_fast.h"
 #include "quant_formats.h"
@@ -171,10 +172,28 @@ __global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_
 }
 
 // ---- the fast form (attention_fast.h) as a kernel of its own: grid = (n_heads, n_splits), block = NT
+// Grouped-query models (`grouped`: a one-dimensional grid): the kv_mul query heads of a kv head read the same cache rows
+// (batched_multiquery_attention.rs:48-98 serves them from one product).  Workgroup b of a launch runs on die b mod 8, and
+// a die's workgroups share its L2, so the workgroups of one (kv head, split) are given indices 8 apart: they run at the
+// same time on one die, the rows come from memory once, and the other kv_mul - 1 workgroups find them in that L2.
+//   b = (key mod 8) + 8 * (j + kv_mul * (key / 8)),  key = kv head + n_kv_heads * split,  j = query head within the group
 template <bool F16, int NT, int HS, bool SINGLE>
-__global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t max_split_len) {
+__global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t max_split_len, uint32_t grouped) {
     touch_kernel_arguments<sizeof(AttnLaunch) + 8>();
-    attn_fast_body<F16, NT, HS, SINGLE, false>(a, blockIdx.x, SINGLE ? 0u : blockIdx.y, threadIdx.x, []() {});
+    uint32_t h = blockIdx.x, split = SINGLE ? 0u : blockIdx.y;
+    if (grouped) {
+        const uint32_t b = blockIdx.x, slot = b >> 3, j = slot % a.kv_mul, key = (b & 7u) + 8u * (slot / a.kv_mul);
+        const uint32_t n_kv = a.n_heads / a.kv_mul;
+        if (key >= n_kv * a.n_splits) return;                    // (the grid is rounded up to whole dies)
+        h = (key % n_kv) * a.kv_mul + j;
+        split = key / n_kv;
+    }
+    attn_fast_body<F16, NT, HS, SINGLE, false>(a, h, split, threadIdx.x, []() {});
+}
+// the size of that grid
+static uint32_t grouped_grid(const AttnLaunch &a) {
+    const uint32_t keys = (a.n_heads / a.kv_mul) * a.n_splits;
+    return 8u * a.kv_mul * ((keys + 7u) / 8u);
 }
 
 // A chunk of tokens whose keys and values are already in the caches: grid = (n_heads, tokens), whole context in one
@@ -282,16 +301,19 @@ size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n
 hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
     if (a.head_size > MAX_HS || a.head_size % 2 || a.head_size / 2 > ATT_THREADS || a.n_splits == 0 || a.n_splits > 64) return hipErrorInvalidValue;
     const uint32_t max_split_len = (a.seq_len + a.n_splits - 1) / a.n_splits;
-    dim3 grid(a.n_heads, a.n_splits);
     const bool fast = (a.head_size == 64 || a.head_size == 128) && a.kv_dim % 8 == 0;
+    // (SLAI_GQA_ON_DIE=0: one workgroup per (query head, split) in plain order, for comparisons)
+    static const bool on_die = [] { const char *e = getenv("SLAI_GQA_ON_DIE"); return !(e && e[0] == '0'); }();
+    const uint32_t grouped = fast && on_die && a.kv_mul > 1 && a.n_heads % a.kv_mul == 0 ? 1u : 0u;
+    dim3 grid(grouped ? grouped_grid(a) : a.n_heads, grouped ? 1u : a.n_splits);
     const size_t smem = fast ? 0 : (size_t)max_split_len * sizeof(float);   // the general kernel keeps its scores in LDS
     if (smem > 48 * 1024) return hipErrorInvalidValue;
     if (fast && a.n_splits == 1) {
-        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 512, 128, true><<<grid, 512, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 512, 128, true><<<grid, 512, smem, s>>>(a, max_split_len); }
-        else { if (a.kv_f16) attn_fast_kernel<true, 512, 64, true><<<grid, 512, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 512, 64, true><<<grid, 512, smem, s>>>(a, max_split_len); }
+        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 512, 128, true><<<grid, 512, smem, s>>>(a, max_split_len, grouped); else attn_fast_kernel<false, 512, 128, true><<<grid, 512, smem, s>>>(a, max_split_len, grouped); }
+        else { if (a.kv_f16) attn_fast_kernel<true, 512, 64, true><<<grid, 512, smem, s>>>(a, max_split_len, grouped); else attn_fast_kernel<false, 512, 64, true><<<grid, 512, smem, s>>>(a, max_split_len, grouped); }
     } else if (fast) {
-        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 256, 128, false><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 128, false><<<grid, 256, smem, s>>>(a, max_split_len); }
-        else { if (a.kv_f16) attn_fast_kernel<true, 256, 64, false><<<grid, 256, smem, s>>>(a, max_split_len); else attn_fast_kernel<false, 256, 64, false><<<grid, 256, smem, s>>>(a, max_split_len); }
+        if (a.head_size == 128) { if (a.kv_f16) attn_fast_kernel<true, 256, 128, false><<<grid, 256, smem, s>>>(a, max_split_len, grouped); else attn_fast_kernel<false, 256, 128, false><<<grid, 256, smem, s>>>(a, max_split_len, grouped); }
+        else { if (a.kv_f16) attn_fast_kernel<true, 256, 64, false><<<grid, 256, smem, s>>>(a, max_split_len, grouped); else attn_fast_kernel<false, 256, 64, false><<<grid, 256, smem, s>>>(a, max_split_len, grouped); }
     } else if (a.kv_f16) attn_kernel<true><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
     else attn_kernel<false><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
     hipError_t e = hipGetLastError();

@@ -128,6 +128,11 @@ def test_argmax_first_maximum(backend):
                                  # long contexts take the split (flash-decoding) form with a combine pass
                                  dict(n_heads=32, kv_mul=1, hs=128, seq=4096, pos=4000),
                                  dict(n_heads=8, kv_mul=4, hs=64, seq=2048, pos=1029),
+                                 # grouped-query shapes whose workgroups are laid out by (kv head, split) over the dies: a
+                                 # Qwen2-7B layer (28 / 4) split and unsplit, and a key count that does not fill the dies
+                                 dict(n_heads=28, kv_mul=7, hs=128, seq=4096, pos=4047),
+                                 dict(n_heads=28, kv_mul=7, hs=128, seq=512, pos=200),
+                                 dict(n_heads=24, kv_mul=2, hs=64, seq=3072, pos=2500),
                                  dict(n_heads=6, kv_mul=1, hs=48, seq=1536, pos=700),
                                  dict(n_heads=4, kv_mul=1, hs=128, seq=2048, pos=5)])
 @pytest.mark.parametrize("f16", [False, True])
