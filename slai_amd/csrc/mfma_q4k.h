@@ -110,7 +110,7 @@ __device__ __forceinline__ void stage_superblock(float4 x, char *sb) {
 }
 
 // The dot products of this lane's row of N matrices (the same row and super-block of each: a gated pair shares the
-// activations) with the staged super-block `sb`.  `zeros`: SB_BYTES of zeros (a lane without a super-block may name it as `sb`); `cs`: N * CS_BYTES for this wave alone.
+// activations) with the staged super-block `sb`.  `zeros`: SB_BYTES of zeros (a lane without a super-block may name it as `sb`); `cs`: 2 N * CS_BYTES for this wave alone.
 // Every lane of the wave takes part, whatever its row holds.
 template <int N>
 __device__ __forceinline__ void dot_q4k(const Tiled<T_Q4_K>::Data *const *d, const char *sb, const char *zeros, char *cs, float *out) {
@@ -137,47 +137,73 @@ __device__ __forceinline__ void dot_q4k(const Tiled<T_Q4_K>::Data *const *d, con
         for (int s = 0; s < 8; ++s) am = fmaf((float)(((s < 4 ? m_lo : m_hi) >> (8 * (s & 3))) & 0xffu), sums[s], am);
         accm[n] = am; acc[n] = 0.0f;
     }
+    // Latencies are hidden by hand (four waves per SIMD do not hide them): the operands of step pair i + 1 are read from LDS
+    // before the products of pair i are issued, and the accumulator of quarter J comes back from LDS -- transposed to the
+    // lanes that own the rows -- while quarter J + 1 is multiplied (two blocks per matrix, used in turn).
+    constexpr uint32_t LO = 0x000f000fu, HI = 0x00f000f0u;
+    const auto read_b = [&](int it, half8 &be, half8 &bo) {     // step pair `it`: piece 1 + it / 2, words (x, y) | (z, w)
+        be = __builtin_bit_cast(half8, *reinterpret_cast<const w32x4 *>(b_even + step_of(it >> 1, it & 1, 0) * SB_STEP_BYTES));
+        bo = __builtin_bit_cast(half8, *reinterpret_cast<const w32x4 *>(b_odd + step_of(it >> 1, it & 1, 1) * SB_STEP_BYTES));
+    };
+    // lane (q, col) holds rows 4 q .. 4 q + 3 of column col; lane (g, r) wants row r of columns g, 4 + g, 8 + g, 12 + g
+    const auto cs_of = [&](int n, int J) { return reinterpret_cast<float *>(cs + (n * 2 + (J & 1)) * CS_BYTES); };
+    const auto take_back = [&](int J, float (&back)[N][4]) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+            const float *t = cs_of(n, J);
+            back[n][0] = t[g * 16u + col]; back[n][1] = t[(4u + g) * 16u + col];
+            back[n][2] = t[(8u + g) * 16u + col]; back[n][3] = t[(12u + g) * 16u + col];
+        }
+    };
+    const auto add_back = [&](int J, const float (&back)[N][4]) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+            const uint32_t scw = J < 2 ? sc_lo[n] : sc_hi[n];
+            const int sh = (J & 1) * 16;
+            acc[n] = fmaf((float)((scw >> sh) & 0xffu), back[n][0] + back[n][1], acc[n]);
+            acc[n] = fmaf((float)((scw >> (sh + 8)) & 0xffu) * 0.0625f, back[n][2] + back[n][3], acc[n]);   // (high nibbles were taken as 16 n)
+        }
+    };
+    half8 be, bo;
+    read_b(0, be, bo);
 #pragma unroll
     for (int J = 0; J < 4; ++J) {
         f32x4 c[N];
-        __builtin_amdgcn_sched_barrier(0);                         // (the operand reads of a quarter stay in it: 32 registers, not 128)
+        float back[N][4];
+        __builtin_amdgcn_sched_barrier(0);
+        if (J > 0) take_back(J - 1, back);                        // (asked for now, used after this quarter's products)
 #pragma unroll
         for (int n = 0; n < N; ++n) c[n] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int H = 0; H < 2; ++H) {
-            constexpr uint32_t LO = 0x000f000fu, HI = 0x00f000f0u;
-            const int K = 2 * J + H;
+        for (int i4 = 0; i4 < 4; ++i4) {
+            const int it = 4 * J + i4, K = it >> 1, h = it & 1;
+            half8 be_next = be, bo_next = bo;
+            if (it + 1 < 16) read_b(it + 1, be_next, bo_next);
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const half8 be = __builtin_bit_cast(half8, *reinterpret_cast<const w32x4 *>(b_even + step_of(K, h, 0) * SB_STEP_BYTES));
-                const half8 bo = __builtin_bit_cast(half8, *reinterpret_cast<const w32x4 *>(b_odd + step_of(K, h, 1) * SB_STEP_BYTES));
-#pragma unroll
-                for (int n = 0; n < N; ++n) {
-                    const U4 &q = d[n]->p[1 + K];
-                    const uint32_t w0 = h ? q.z : q.x, w1 = h ? q.w : q.y;
-                    const uint32_t v0 = w0 >> 8, v1 = w1 >> 8;
-                    const half8 ae = __builtin_bit_cast(half8, w32x4{w0 & LO, v0 & LO, w1 & LO, v1 & LO});
-                    const half8 ao = __builtin_bit_cast(half8, w32x4{w0 & HI, v0 & HI, w1 & HI, v1 & HI});
-                    c[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ae, be, c[n], 0, 0, 0);
-                    c[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ao, bo, c[n], 0, 0, 0);
-                }
+            for (int n = 0; n < N; ++n) {
+                const U4 &q = d[n]->p[1 + K];
+                const uint32_t w0 = h ? q.z : q.x, w1 = h ? q.w : q.y;
+                const uint32_t v0 = w0 >> 8, v1 = w1 >> 8;
+                const half8 ae = __builtin_bit_cast(half8, w32x4{w0 & LO, v0 & LO, w1 & LO, v1 & LO});
+                const half8 ao = __builtin_bit_cast(half8, w32x4{w0 & HI, v0 & HI, w1 & HI, v1 & HI});
+                c[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ae, be, c[n], 0, 0, 0);
+                c[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ao, bo, c[n], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            be = be_next; bo = bo_next;
         }
-        // lane (q, col) holds rows 4 q .. 4 q + 3 of column col; lane (g, r) wants row r of columns g, 4 + g, 8 + g, 12 + g
 #pragma unroll
         for (int n = 0; n < N; ++n) {
-            float *t = reinterpret_cast<float *>(cs + n * CS_BYTES);
             asm volatile("" ::: "memory");
-            *reinterpret_cast<f32x4 *>(t + col * 16u + 4u * g) = c[n];
+            *reinterpret_cast<f32x4 *>(cs_of(n, J) + col * 16u + 4u * g) = c[n];
             asm volatile("" ::: "memory");
-            const float even = t[g * 16u + col] + t[(4u + g) * 16u + col];
-            const float odd = t[(8u + g) * 16u + col] + t[(12u + g) * 16u + col];
-            asm volatile("" ::: "memory");
-            const uint32_t scw = J < 2 ? sc_lo[n] : sc_hi[n];
-            const int sh = (J & 1) * 16;
-            acc[n] = fmaf((float)((scw >> sh) & 0xffu), even, acc[n]);
-            acc[n] = fmaf((float)((scw >> (sh + 8)) & 0xffu) * 0.0625f, odd, acc[n]);      // (high nibbles were taken as 16 n)
         }
+        if (J > 0) add_back(J - 1, back);
+    }
+    {
+        float back[N][4];
+        take_back(3, back);
+        add_back(3, back);
     }
 #pragma unroll
     for (int n = 0; n < N; ++n) out[n] = (dd[n] * 16777216.0f * down) * acc[n] - dmin[n] * accm[n];

@@ -80,7 +80,7 @@ SLAI_HD uint32_t lds_set(uint32_t parity) { return parity * (lds_red() + 2 * WG_
 // ... then, for the Q4_K phases on the matrix cores (mfma_q4k.h): a block of zeros, and per wave the staged activations
 // of up to four super-blocks and room for the accumulators of two matrices on their way to the lanes that own the rows
 constexpr uint32_t MQ_SB_BYTES = 1024 + 80, MQ_ZERO_BYTES = MQ_SB_BYTES, MQ_CS_BYTES = 1024;   // (zeros: a whole staged super-block of them)
-constexpr uint32_t MQ_WAVE_BYTES = 4 * MQ_SB_BYTES + 2 * MQ_CS_BYTES;
+constexpr uint32_t MQ_WAVE_BYTES = 4 * MQ_SB_BYTES + 4 * MQ_CS_BYTES;   // (two accumulator blocks per matrix of a gated pair)
 SLAI_HD uint32_t lds_mq_zero() { return 2 * (lds_red() + 2 * WG_WAVES) * 4; }                          // bytes from here on
 SLAI_HD uint32_t lds_mq_wave(uint32_t wave) { return lds_mq_zero() + MQ_ZERO_BYTES + wave * MQ_WAVE_BYTES; }
 SLAI_HD uint32_t lds_mq_sb(uint32_t wave, uint32_t k) { return lds_mq_wave(wave) + k * MQ_SB_BYTES; }
