@@ -415,11 +415,10 @@ struct PersistentParams {
     const float *x;                      // the embedding row of the token (written by the launch before this one)
     float *logits;
     const uint32_t *pos_ptr;
-    // hand-off buffers, filled with FLOW_EMPTY before every launch (layout: resident_plan.h, plan::flow_*)
+    // hand-off buffers, filled with FLOW_EMPTY before every launch (layout: resident_plan.h, plan::flow_*): the vectors that
+    // cross workgroups, q and the newest k and v among them
     float *flow;
     float *slots;                        // per-workgroup staging of the normalised input of a 64-row-unit phase
-    float *q, *kcol, *vcol;              // q / k / v of the current layer (handed over inside one die)
-    uint32_t *counters;                  // one 128-byte line per head
     uint32_t *abort_flag;                // set when a reader gave up
     uint64_t *trace;                     // optional: per workgroup 16 * n_layers + 8 time stamps (100 MHz clock); null = none
 };

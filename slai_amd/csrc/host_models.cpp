@@ -391,8 +391,7 @@ int slai_llama2::persistent_setup() {
     p.wout = mat(weights.output); p.out_norm = vec(weights.output_norm);
     p.x = (const float *)state.x.buf->dptr; p.logits = (float *)state.logits.buf->dptr;
     p.pos_ptr = (const uint32_t *)&((DecodeState *)loop.state->dptr)->pos;
-    p.q = (float *)state.q.buf->dptr; p.kcol = (float *)state.kcol.buf->dptr; p.vcol = (float *)state.vcol.buf->dptr;
-    p.counters = ctx->handoff_counters; p.abort_flag = ctx->handoff_counters + (size_t)ctx->handoff_heads * 32;
+    p.abort_flag = ctx->handoff_counters + (size_t)ctx->handoff_heads * 32;
     // the device must keep the whole grid resident: every compute unit one workgroup, and enough of them for every role
     uint32_t resident = 0;
     p.qkv_units = 6; p.gu_rows = 64;                                  // (the occupancy query only needs the widths)

@@ -100,7 +100,7 @@ def _f32(a):
 def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, wtype, seed=1234,
                std=0.02, rope_base=10000.0, rms_eps=1e-5, out_type=None, v_type=None, embd_type=None,
                with_output=True, arch="llama", bias=False, norm_random=False, distinct_layers=None, tokenizer=None,
-               ffn_norm_scale=1.0, tensor_hook=None):
+               ffn_norm_scale=1.0, tensor_hook=None, tensor_types=None):
     """Synthetic Llama-2-shape model file (uint8 numpy array).
 
     Weights are seeded std*N(0,1) quantized to `wtype` (`v_type` for attn_v, `out_type` for
@@ -158,6 +158,8 @@ def llama_gguf(dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab, seq_len, w
         shapes = [("attn_q", dim, dim, wtype), ("attn_k", kv_dim, dim, wtype), ("attn_v", kv_dim, dim, v_type),
                   ("attn_output", dim, dim, wtype), ("ffn_gate", hidden_dim, dim, wtype),
                   ("ffn_up", hidden_dim, dim, wtype), ("ffn_down", dim, hidden_dim, wtype)]
+        if tensor_types:     # e.g. {"ffn_down": 14}: the mixes of real K-quant files (Q6_K down / v in half of the layers)
+            shapes = [(nm, nr, nc, tensor_types.get(nm, t)) for nm, nr, nc, t in shapes]
         w.add_tensor(p + "attn_norm.weight", [dim], 0, norm_vec(dim))
         for nm, nr, nc, t in shapes:
             if src is None:

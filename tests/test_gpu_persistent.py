@@ -39,14 +39,30 @@ def test_persistent_small_model_vs_oracle(kv_f16):
         b.close()
 
 
-def test_persistent_long_context_vs_oracle():
-    """600 steps on the small model: the attention asks for the first 384 cached positions before the query exists and
-    walks the rest in passes of 128 with one pass in flight; positions 384, 385, 512, 513 are where those paths change."""
+@pytest.mark.parametrize("kv_f16", [True, False])
+def test_persistent_long_context_vs_oracle(kv_f16):
+    """600 steps on the small model: the attention asks for the first 384 cached positions (f16 cache; 128 with an f32
+    cache) before the query exists and walks the rest in passes of 128 with one pass in flight; positions 128, 129, 384,
+    385, 512, 513 are where those paths change."""
     b = backend_with(True)
     try:
         data = gw.llama_gguf(dim=1024, hidden_dim=3072, n_layers=2, n_heads=8, n_kv_heads=8, vocab=2000, seq_len=640, wtype=12, v_type=14,
                              out_type=14, embd_type=12, seed=77, std=0.05, norm_random=True)
-        check_llama(b, data, [5, 1000, 1999], 600, kv_f16=True, check_logit_steps=4, decode_form=1)
+        check_llama(b, data, [5, 1000, 1999], 600, kv_f16=kv_f16, check_logit_steps=4, decode_form=1)
+    finally:
+        b.close()
+
+
+def test_persistent_other_kquant_mixes():
+    """The block formats the resident launch takes besides the headline mix: Q6_K in the two projections into the residual
+    (16-row tiles on the matrix cores), Q5_K q and k (the vector-unit path with wave-uniform activations), Q6_K q, f32 cache."""
+    b = backend_with(True)
+    try:
+        for seed, types, kv_f16 in ((81, {"attn_output": 14, "ffn_down": 14}, True), (82, {"attn_q": 13, "attn_k": 13, "ffn_down": 14}, False),
+                                    (83, {"attn_q": 14, "attn_output": 14}, True)):
+            data = gw.llama_gguf(dim=1024, hidden_dim=3072, n_layers=2, n_heads=8, n_kv_heads=8, vocab=1500, seq_len=320, wtype=12, v_type=14,
+                                 out_type=12, embd_type=12, seed=seed, std=0.05, norm_random=True, tensor_types=types)
+            check_llama(b, data, [5, 1000, 1499, 9], 24, kv_f16=kv_f16, check_logit_steps=6, decode_form=1)
     finally:
         b.close()
 
