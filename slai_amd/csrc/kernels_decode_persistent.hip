@@ -184,13 +184,12 @@ __device__ __forceinline__ u32x4 flow_take(Rsrc x, uint32_t piece, Flow &f) {
     // that was cached before its producer wrote it shows empty words (a word only ever changes from empty to its value,
     // and no line survives from an earlier launch: the caches are invalidated when a kernel starts), and then the
     // requests go to memory as before.
-    {
-        const u32x4 v = buf_load16<AUX_ONCE>(x, piece * 16u);
-        if (!__any(flow_empty(v))) return v;
-    }
+    u32x4 v = buf_load16<AUX_ONCE>(x, piece * 16u);
+    // only the lanes whose piece shows an empty word ask again: what the late producers wrote, not the whole part
     for (;;) {
-        const u32x4 v = buf_load16<AUX_FLOW>(x, piece * 16u);
-        if (!__any(flow_empty(v)) || f.dead) return v;
+        const bool hole = flow_empty(v);
+        if (!__any(hole) || f.dead) return v;
+        if (hole) v = buf_load16<AUX_FLOW>(x, piece * 16u);
         flow_backoff(f, deadline, rounds);
     }
 }
@@ -200,23 +199,19 @@ __device__ __forceinline__ void flow_take4(Rsrc x, uint32_t piece0, uint32_t n, 
     uint64_t deadline = 0;
     uint32_t rounds = 0;
     flow_watch(x, (uniform_word(piece0) + 64u * (n - 1u)) * 4u + 255u, f);
-    {                                                             // (through the die's L2 first: see flow_take)
-        bool hole = false;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            out[k] = u32x4{0u, 0u, 0u, 0u};
-            if ((uint32_t)k < n) { out[k] = buf_load16<AUX_ONCE>(x, (piece0 + 64u * k) * 16u); hole = hole || flow_empty(out[k]); }
-        }
-        if (!__any(hole)) return;
+    for (int k = 0; k < 4; ++k) {                                 // (through the die's L2 first: see flow_take)
+        out[k] = u32x4{0u, 0u, 0u, 0u};
+        if ((uint32_t)k < n) out[k] = buf_load16<AUX_ONCE>(x, (piece0 + 64u * k) * 16u);
     }
     for (;;) {
         bool hole = false;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            out[k] = u32x4{0u, 0u, 0u, 0u};
-            if ((uint32_t)k < n) { out[k] = buf_load16<AUX_FLOW>(x, (piece0 + 64u * k) * 16u); hole = hole || flow_empty(out[k]); }
-        }
+        for (int k = 0; k < 4; ++k) hole = hole || flow_empty(out[k]);
         if (!__any(hole) || f.dead) return;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)                               // (a piece past n is zeros: never empty)
+            if (flow_empty(out[k])) out[k] = buf_load16<AUX_FLOW>(x, (piece0 + 64u * k) * 16u);
         flow_backoff(f, deadline, rounds);
     }
 }
