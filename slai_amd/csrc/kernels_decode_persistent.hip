@@ -521,6 +521,8 @@ template <bool F16> __device__ __forceinline__ void att_decode8(const U4 *r, flo
 }
 __device__ __forceinline__ U4 as_u4(u32x4 v) { return U4{v.x, v.y, v.z, v.w}; }
 
+constexpr int DPP_ROW_ROR8 = 0x128;                           // lane i of a row of 16 takes lane (i + 8) % 16
+
 template <bool F16> struct Attention {
     using P = AttPass<F16>;
     static constexpr uint32_t ES = F16 ? 2 : 4;                 // bytes of a cache element
@@ -558,13 +560,13 @@ template <bool F16> struct Attention {
 #pragma unroll
             for (int q = 0; q < 8; ++q) part = fmaf(qr[8 * j + q], kv[q], part);
         }
-        part += lane_xor(part, 1);
-        part += lane_xor(part, 2);
-        part += lane_xor(part, 4);
+        part = mq::sum8(part);                                   // over the eight lanes of the position
         const float sc = live ? part / sqrtf(128.0f) : -FLT_MAX;             // cpu.rs:521
-        float mx = sc;
-#pragma unroll
-        for (int msk = 32; msk >= 8; msk >>= 1) mx = fmaxf(mx, lane_xor(mx, msk));
+        // the largest of the wave's eight scores: the row's two positions, then the four rows
+        const float mrow = fmaxf(sc, mq::dpp<mq::DPP_MIRROR>(sc));
+        const int mb = __builtin_bit_cast(int, mrow);
+        const float mx = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 0)), __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 16))),
+                               fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 32)), __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 48))));
         const float mn = fmaxf(m, mx);
         const float resc = expf(m - mn);                        // 0 on the first live pass, 1 while nothing was live
         const float pr = live ? expf(sc - mn) : 0.0f;
@@ -572,15 +574,17 @@ template <bool F16> struct Attention {
 #pragma unroll
         for (int q = 0; q < 8; ++q) o[q] *= resc;
         m = mn;
+        // The weights of the row's two positions (plan::att_v_pos: value lanes of row r take positions 2 r and 2 r + 1):
+        // lanes 0-7 of the row scored the first, lanes 8-15 the second.
+        const float other = mq::dpp<DPP_ROW_ROR8>(pr);
+        const bool second = (lane & 8u) != 0;
+        const float pw[2] = {second ? other : pr, second ? pr : other};
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            // the weight of position u * 4 + lane / 16 of this wave's eight: held by the eight lanes that scored it
-            const int src = (int)(8u * (u * 4u + lane / 16u));
-            const float pw = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src << 2, __builtin_bit_cast(int, pr)));
             float vv[8];
             att_decode8<F16>(ps.v[u], vv);
 #pragma unroll
-            for (int q = 0; q < 8; ++q) o[q] = fmaf(pw, vv[q], o[q]);
+            for (int q = 0; q < 8; ++q) o[q] = fmaf(pw[u], vv[q], o[q]);
         }
     }
 };
@@ -632,17 +636,25 @@ __device__ __forceinline__ void attend(const plan::Shape &sh, uint32_t head, uin
         at.consume(cur, tb, qr);
         cur = nxt;
     }
-    // this wave's (maximum, sum, outputs): lanes 16 apart hold the same elements of different positions
+    // This wave's (maximum, sum, outputs): lanes 16 apart hold the same elements of different positions.  Two registers
+    // are added across the halves of the wave with one exchange (lanes 0-31 keep the first's sum, lanes 32-63 the
+    // second's), then the same across neighbouring rows: row r of s0 / s1 ends with element [0, 2, 1, 3][r] / that + 4.
     at.lsum = wave_total(at.lsum);
-#pragma unroll
-    for (int msk = 16; msk < 64; msk <<= 1) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) at.o[e] += lane_xor(at.o[e], msk);
-    }
+    const auto across_halves = [](float a, float b) {
+        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+        return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    };
+    const auto across_rows = [](float a, float b) {
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+        return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    };
+    const float s0 = across_rows(across_halves(at.o[0], at.o[1]), across_halves(at.o[2], at.o[3]));
+    const float s1 = across_rows(across_halves(at.o[4], at.o[5]), across_halves(at.o[6], at.o[7]));
     const uint32_t lane = lane_id();
-    if (lane < 16) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sacc[wave * 128 + lane * 8 + e] = at.o[e];
+    {
+        const uint32_t row = lane >> 4, e = ((row & 1u) << 1) | (row >> 1);
+        sacc[wave * 128 + (lane & 15u) * 8 + e] = s0;
+        sacc[wave * 128 + (lane & 15u) * 8 + e + 4] = s1;
     }
     if (lane == 0) { smax[wave] = at.m; ssum[wave] = at.lsum; }
     stamp(tl, 2, wave);

@@ -89,11 +89,12 @@ SLAI_HD uint32_t lds_bytes(const Shape &) { return lds_mq_wave(WG_WAVES); }
 SLAI_HD uint32_t lds_floats(const Shape &s) { return lds_bytes(s) / 4; }
 
 // ---- the attention of a head over the cached positions: eight lanes per position for the scores (sixteen elements
-// each), sixteen lanes per position for the values (eight elements each); a pass is 128 positions, eight per wave --------
+// each), sixteen lanes per position for the values (eight elements each: the two positions the row of 16 lanes scored);
+// a pass is 128 positions, eight per wave ---------------------------------------------------------------------------------
 constexpr uint32_t ATT_PASS = 128;
 SLAI_HD uint32_t att_k_pos(uint32_t tb, uint32_t wave, uint32_t lane) { return tb + wave * 8 + lane / 8; }
 SLAI_HD uint32_t att_k_elem(uint32_t head, uint32_t lane) { return head * 128 + (lane & 7u) * 16; }
-SLAI_HD uint32_t att_v_pos(uint32_t tb, uint32_t wave, uint32_t u, uint32_t lane) { return tb + wave * 8 + u * 4 + lane / 16; }
+SLAI_HD uint32_t att_v_pos(uint32_t tb, uint32_t wave, uint32_t u, uint32_t lane) { return tb + wave * 8 + 2 * (lane / 16) + u; }
 SLAI_HD uint32_t att_v_elem(uint32_t head, uint32_t lane) { return head * 128 + (lane & 15u) * 8; }
 // element e of position t of a cache [seq_len x dim] (times the element size: below 4 GiB, shape_ok bounds seq_len and dim)
 SLAI_HD uint32_t cache_elem(const Shape &s, uint32_t t, uint32_t e) { return t * s.dim + e; }

@@ -237,8 +237,8 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                                     a.touch(cache, (uint64_t)plan::cache_elem(s, tv < T ? tv : 0, ev) * kv_bytes, 8 * kv_bytes, "cached value", b, wave, lane, l);
                                     if (ev / 128 != h) a.fail("value elements of another head");
                                     if (tv < T) for (uint32_t i = 0; i < 8; ++i) ++vseen[(size_t)tv * 128 + ev % 128 + i];
-                                    // the weight of that position comes from lane 8 * (position within the wave's eight)
-                                    if (plan::att_k_pos(tb, wave, 8 * (uu * 4 + lane / 16)) != tv) a.fail("value lane takes the weight of another position");
+                                    // the weight of that position comes from the half of the lane's own row of 16 that scored it
+                                    if (plan::att_k_pos(tb, wave, 16 * (lane / 16) + 8 * uu) != tv) a.fail("value lane takes the weight of another position");
                                 }
                             }
                     for (size_t i = 0; i < kseen.size(); ++i)
