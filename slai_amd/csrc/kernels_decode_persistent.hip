@@ -589,6 +589,23 @@ template <bool F16> struct Attention {
     }
 };
 
+// The products of the newest position's score this lane owns: lane (i, jj) = (lane % 8, lane / 8 % 4) holds elements
+// 16 i + 4 jj .. + 3 of the key in `kn` (and sixteen of the query in qr).
+template <bool F16> __device__ __forceinline__ float att_new_score(const float (&qr)[16], u32x4 kn) {
+    using C = attn::KV<F16>;                                    // (what the cache row holds: rounded to its element type)
+    const uint32_t jj = (lane_id() >> 3) & 3u;
+    float part = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float d = qr[4 * j] * C::round(__uint_as_float(kn.x));
+        d = fmaf(qr[4 * j + 1], C::round(__uint_as_float(kn.y)), d);
+        d = fmaf(qr[4 * j + 2], C::round(__uint_as_float(kn.z)), d);
+        d = fmaf(qr[4 * j + 3], C::round(__uint_as_float(kn.w)), d);
+        part = jj == (uint32_t)j ? d : part;
+    }
+    return part;
+}
+
 // lds: [16 waves][128] partial outputs, then the waves' maxima and sums.  q / knew / vnew: this layer's hand-off vectors
 // (dim floats each); out: the attention output vector.
 template <bool F16>
@@ -606,21 +623,35 @@ __device__ __forceinline__ void attend(const plan::Shape &sh, uint32_t head, uin
     }
     cur = P{};
     if (A::ATT_PRE * plan::ATT_PASS < pos) at.request(cur, A::ATT_PRE * plan::ATT_PASS);
-    // the query: sixteen elements per lane, as soon as all of them are there
+    // The query: sixteen elements per lane, as soon as all of them are there.  Waves 0 and 1, whose threads merge, ask for
+    // the newest key and value in the same rounds: the key is produced at about the same time as the query, the value
+    // often is, and what is complete then costs no round trip after the passes.
     float qr[16];
+    // (The newest key: lane (i, jj) = (lane % 8, lane / 8 % 4) asks for elements 16 i + 4 jj .. + 3 only, a quarter of what
+    // it holds of the query, and the products are summed over 32 lanes.)
+    const uint32_t kn_first = plan::att_k_elem(head, lane_id()) + 4u * ((lane_id() >> 3) & 3u);
+    float snew_part = 0.0f;
+    uint32_t vnw = FLOW_EMPTY;
+    bool kv_hole = true;
     {
         const uint32_t first = plan::att_k_elem(head, lane_id());
         uint64_t deadline = 0;
         uint32_t rounds = 0;
         flow_watch(q, head * 128u + 127u, f);
         for (;;) {
-            u32x4 v[4];
+            u32x4 v[4], kn = u32x4{FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY};
 #pragma unroll
             for (int j = 0; j < 4; ++j) v[j] = buf_load16<AUX_FLOW>(q, (first + 4u * j) * 4u);
+            if (fresh(wave) < 2) {
+                kn = buf_load16<AUX_FLOW>(knew, kn_first * 4u);
+                vnw = __builtin_amdgcn_raw_buffer_load_b32(vnew, (int)((head * 128u + fresh(wave) * 64u + lane_id()) * 4u), 0, AUX_FLOW);
+            }
             const bool hole = flow_empty(v[0]) || flow_empty(v[1]) || flow_empty(v[2]) || flow_empty(v[3]);
             if (!__any(hole) || f.dead) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) { qr[4 * j] = __uint_as_float(v[j].x); qr[4 * j + 1] = __uint_as_float(v[j].y); qr[4 * j + 2] = __uint_as_float(v[j].z); qr[4 * j + 3] = __uint_as_float(v[j].w); }
+                kv_hole = __any(flow_empty(kn) || vnw == FLOW_EMPTY);
+                if (!kv_hole) snew_part = att_new_score<F16>(qr, kn);
                 break;
             }
             flow_backoff(f, deadline, rounds);
@@ -661,48 +692,44 @@ __device__ __forceinline__ void attend(const plan::Shape &sh, uint32_t head, uin
     // the newest position: its score like a cached one's (waves 0 and 1, whose threads merge), its value per element
     float snew = 0.0f, vn = 0.0f;
     if (wave < 2) {
-        const uint32_t first = plan::att_k_elem(head, lane);
         uint64_t deadline = 0;
         uint32_t rounds = 0;
-        u32x4 v[4];
-        uint32_t w;
-        for (;;) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = buf_load16<AUX_FLOW>(knew, (first + 4u * j) * 4u);
-            w = __builtin_amdgcn_raw_buffer_load_b32(vnew, (int)((head * 128u + wave * 64u + lane) * 4u), 0, AUX_FLOW);
-            const bool hole = flow_empty(v[0]) || flow_empty(v[1]) || flow_empty(v[2]) || flow_empty(v[3]) || w == FLOW_EMPTY;
-            if (!__any(hole) || f.dead) break;
-            flow_backoff(f, deadline, rounds);
+        while (kv_hole) {                                         // (not complete in the round that brought the query)
+            const u32x4 kn = buf_load16<AUX_FLOW>(knew, kn_first * 4u);
+            vnw = __builtin_amdgcn_raw_buffer_load_b32(vnew, (int)((head * 128u + wave * 64u + lane) * 4u), 0, AUX_FLOW);
+            kv_hole = __any(flow_empty(kn) || vnw == FLOW_EMPTY) && !f.dead;
+            if (kv_hole) flow_backoff(f, deadline, rounds);
+            else snew_part = att_new_score<F16>(qr, kn);
         }
         using C = attn::KV<F16>;                                // (what the cache row holds: rounded to its element type)
-        float part = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            part = fmaf(qr[4 * j], C::round(__uint_as_float(v[j].x)), part);
-            part = fmaf(qr[4 * j + 1], C::round(__uint_as_float(v[j].y)), part);
-            part = fmaf(qr[4 * j + 2], C::round(__uint_as_float(v[j].z)), part);
-            part = fmaf(qr[4 * j + 3], C::round(__uint_as_float(v[j].w)), part);
+        float part = mq::sum8(snew_part);                        // over i, then over jj: the two half rows, then the neighbouring row
+        part += mq::dpp<mq::DPP_MIRROR>(part);
+        {
+            const auto rr = __builtin_amdgcn_permlane16_swap(__float_as_uint(part), __float_as_uint(part), false, false);   // [row 0, row 0, row 2, row 2], [row 1, row 1, row 3, row 3]
+            part = __uint_as_float(rr[0]) + __uint_as_float(rr[1]);
         }
-        part += lane_xor(part, 1);
-        part += lane_xor(part, 2);
-        part += lane_xor(part, 4);
         snew = part / sqrtf(128.0f);
-        vn = C::round(__uint_as_float(w));
+        vn = C::round(__uint_as_float(vnw));
     }
     lds_barrier();
     if (wave < 2) {
+        // Lane i of every row of 16 takes wave i's maximum and sum: one exponential per lane instead of sixteen per
+        // thread; the factors then reach the threads as scalar operands.
         const uint32_t e = wave * 64u + lane;
-        float M = snew;
-#pragma unroll
-        for (int w = 0; w < PNW; ++w) M = fmaxf(M, smax[w]);
+        const float mw = smax[lane & 15u];
+        float M = fmaxf(mw, mq::dpp<mq::DPP_XOR1>(mw));
+        M = fmaxf(M, mq::dpp<mq::DPP_XOR2>(M)); M = fmaxf(M, mq::dpp<mq::DPP_HALF_MIRROR>(M)); M = fmaxf(M, mq::dpp<mq::DPP_MIRROR>(M));
+        M = fmaxf(M, snew);
+        const float fw = expf(mw - M);                          // a wave that saw no position has sum 0 and outputs 0
+        float lw = ssum[lane & 15u] * fw;
+        lw = mq::sum8(lw);
+        lw += mq::dpp<mq::DPP_MIRROR>(lw);
         const float fn = expf(snew - M);
-        float r = vn * fn, l = fn;
+        float r = vn * fn;
+        const float l = lw + fn;
+        const int fb = __builtin_bit_cast(int, fw);
 #pragma unroll
-        for (int w = 0; w < PNW; ++w) {
-            const float fw = expf(smax[w] - M);                 // a wave that saw no position has sum 0 and outputs 0
-            r = fmaf(sacc[w * 128 + e], fw, r);
-            l = fmaf(ssum[w], fw, l);
-        }
+        for (int w = 0; w < PNW; ++w) r = fmaf(sacc[w * 128 + e], __builtin_bit_cast(float, __builtin_amdgcn_readlane(fb, w)), r);
         flow_put(out, head * 128u + e, r / l);
     }
 }
