@@ -95,8 +95,7 @@ struct DeviceLoop {           // device-resident state of the greedy loop
     slai_buffer *prompt = nullptr;      // int32[capacity]
     slai_buffer *out_tokens = nullptr;  // int32[capacity]
     uint32_t capacity = 0;
-    slai_graph *graph = nullptr;        // one token with the greedy pick
-    slai_graph *graph_sampled = nullptr;  // one token with the temperature / top-p pick
+    slai_graph *graph[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};   // one token, [launch form][greedy pick | temperature / top-p pick]
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 };
 int loop_init(slai_ctx *ctx, DeviceLoop &L, uint32_t capacity) {
@@ -109,8 +108,9 @@ int loop_init(slai_ctx *ctx, DeviceLoop &L, uint32_t capacity) {
     return SLAI_OK;
 }
 void loop_destroy(slai_ctx *ctx, DeviceLoop &L) {
-    if (L.graph) slai_graph_destroy(ctx, L.graph);
-    if (L.graph_sampled) slai_graph_destroy(ctx, L.graph_sampled);
+    for (auto &form : L.graph)
+        for (slai_graph *g : form)
+            if (g) slai_graph_destroy(ctx, g);
     if (L.state) slai_buffer_destroy(ctx, L.state);
     if (L.prompt) slai_buffer_destroy(ctx, L.prompt);
     if (L.out_tokens) slai_buffer_destroy(ctx, L.out_tokens);
@@ -172,7 +172,8 @@ struct slai_llama2 {
 
     int load(const slai_gguf *g);
     int launch(LlmContext &ctxt, const slai_attn_params &attn_params, uint32_t pos);   // transformer.rs:316-381
-    int enqueue_fused(int sampler);   // 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state
+    int enqueue_fused(int sampler, int form = 0);   // sampler 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state; form 1: the resident launch
+    int form_at(uint32_t pos) const;               // the launch form of the token at `pos`
 
     // The layer stack as ONE resident launch per token (kernels_decode_persistent.hip), for the models it covers.
     struct {
@@ -347,17 +348,18 @@ int slai_llama2::load(const slai_gguf *gg) {
 }
 
 // The resident launch covers the shapes of the headline configuration and its smaller relatives: as many cache heads as
-// query heads of size 128, a width of 1024 .. 4096 in steps of 1024, a context one workgroup per head can walk, q / k / v,
-// gate / up and the output matrix in 64-row tiles of K-quants (gate and up both Q4_K), the two projections into the
-// residual in 16-row tiles of Q4_K or Q6_K.  Everything else keeps the launch-per-step form.
+// query heads of size 128, a width of 1024 .. 4096 in steps of 1024, q / k / v, gate / up and the output matrix in 64-row
+// tiles of K-quants (gate and up both Q4_K), the two projections into the residual in 16-row tiles of Q4_K or Q6_K.
+// Everything else keeps the launch-per-step form, and so do the tokens of these models beyond the position up to which
+// one workgroup per head walks the cache fast enough (form_at).
 bool slai_llama2::persistent_supported() const {
     const uint32_t dim = config.dim, hid = config.hidden_dim, nh = config.n_q_heads;
     if (!ctx->persistent) return false;
     const auto no = [&](const char *why) { persistent.why_not = why; return false; };
     if (!ctx->fuse_qkv_attention) return no("workgroups are not placed on the dies round robin (or SLAI_FUSE_QKV_ATTN=0)");
     if (!ctx->rowtile_gemv || !ctx->handoff_counters || nh > ctx->handoff_heads) return no("64-row tiles or the hand-off counters are switched off");
-    if (config.n_kv_heads != nh || head_size() != 128 || nh % 8 || dim % 1024 || dim > 4096 || hid % 256 || hid / 256 > 64 || attn_splits != 1 || config.seq_len > 1024)
-        return no("shape: needs as many cache heads as query heads of size 128 (a multiple of 8), a width of 1024 .. 4096, an FFN width in super-blocks, a context of at most 1024");
+    if (config.n_kv_heads != nh || head_size() != 128 || nh % 8 || dim % 1024 || dim > 4096 || hid % 256 || hid / 256 > 64)
+        return no("shape: needs as many cache heads as query heads of size 128 (a multiple of 8), a width of 1024 .. 4096, an FFN width in super-blocks");
     const auto kquant = [](int t) { return t == T_Q4_K || t == T_Q5_K || t == T_Q6_K; };
     const auto proj = [&](const slai_qmat *m, uint32_t cols) {
         return m->tiled && m->rows_log2 == 4 && (m->type == T_Q4_K || m->type == T_Q6_K) && m->ncb == cols / 256 && m->ngroups == (cols / 256 + 3) / 4 && m->ngroups <= 16;
@@ -488,8 +490,13 @@ int slai_llama2::launch(LlmContext &ctxt, const slai_attn_params &attn_params, u
 // in device memory, so the sequence can be captured once and replayed for every token:
 //   embedding-row gather | per layer: [RMSNorm+QKV GEMV] [RoPE+cache write+attention] [Wo GEMV+residual]
 //   [RMSNorm+gate/up GEMV+SiLU] [down GEMV+residual] | [RMSNorm+logits GEMV] [argmax + loop state]
-int slai_llama2::enqueue_fused(int sampler) {
-    if (persistent.ready) return enqueue_persistent(sampler);
+// The resident launch walks a head's cached positions with one workgroup, at the rate one compute unit reads memory;
+// the launch-per-step form spreads them over the device.  Up to ctx->resident_max_pos positions the resident launch is
+// the faster one, beyond it the steps are: the form is chosen per token (both keep the same caches and loop state).
+int slai_llama2::form_at(uint32_t pos) const { return persistent.ready && pos < ctx->resident_max_pos ? 1 : 0; }
+
+int slai_llama2::enqueue_fused(int sampler, int form) {
+    if (form == 1) return persistent.ready ? enqueue_persistent(sampler) : set_error(ctx, SLAI_E_STATE, "this model does not take the resident launch");
     Llama2State &s = state;
     DecodeState *ds = (DecodeState *)loop.state->dptr;
     float *x = (float *)s.x.buf->dptr, *xb = (float *)s.xb.buf->dptr, *hb = (float *)s.hb.buf->dptr, *hb2 = (float *)s.hb2.buf->dptr;
@@ -946,7 +953,7 @@ SLAI_EXPORT int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t to
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_llama2_time_steps: not during graph capture");
     DecodeState ds{(int)pos, (int)token, 0, 0};
     TRY(slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds));
-    const auto enqueue = [&]() { return m->persistent.ready ? m->enqueue_persistent(0) : m->enqueue_fused(0); };
+    const auto enqueue = [&]() { return m->enqueue_fused(0, m->persistent.ready ? 1 : 0); };
     TRY(enqueue());                                             // untimed: sizes scratch, warms the caches
     TRY(slai_synchronize(ctx));
     std::vector<std::pair<const char *, hipEvent_t>> marks;
@@ -993,9 +1000,9 @@ SLAI_EXPORT int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t to
     for (size_t k = 0; k < order.size() && !rc; ++k) {
         if (m->persistent.ready) { alone_us[k] = mean_us[k]; continue; }     // (a resident launch needs the buffers emptied before it: never alone)
         ctx->only_step = order[k];
-        rc = m->enqueue_fused(0);                               // untimed
+        rc = m->enqueue_fused(0, 0);                            // untimed
         if (!rc && hipEventRecord(e0, ctx->stream) != hipSuccess) rc = SLAI_E_HIP;
-        for (uint32_t r = 0; r < reps && !rc; ++r) rc = m->enqueue_fused(0);
+        for (uint32_t r = 0; r < reps && !rc; ++r) rc = m->enqueue_fused(0, 0);
         if (!rc && hipEventRecord(e1, ctx->stream) != hipSuccess) rc = SLAI_E_HIP;
         ctx->only_step = nullptr;
         if (!rc) rc = slai_synchronize(ctx);
@@ -1049,7 +1056,7 @@ SLAI_EXPORT int slai_llama2_forward_logits(slai_llama2 *m, uint32_t pos, uint32_
     } else {
         DecodeState ds{(int)pos, (int)token, 0, 0};
         TRY(slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds));
-        TRY(m->enqueue_fused(false));
+        TRY(m->enqueue_fused(0, m->form_at(pos)));
     }
     TRY(slai_synchronize(ctx));                                          // :219
     TRY(handoff_check(ctx));
@@ -1077,17 +1084,19 @@ static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_le
     TRY(slai_write_buffer(ctx, L.prompt, 0, prompt, (size_t)n_prompt * 4));
     if (!ctx->use_graph) {
         SLAI_HIP_TRY(ctx, hipEventRecord(L.ev0, ctx->stream));
-        for (uint32_t i = 0; i < n_steps; ++i) TRY(m->enqueue_fused(mode));
+        for (uint32_t i = 0; i < n_steps; ++i) TRY(m->enqueue_fused(mode, m->form_at(start_pos + i)));
         SLAI_HIP_TRY(ctx, hipEventRecord(L.ev1, ctx->stream));
         TRY(slai_synchronize(ctx));
         TRY(handoff_check(ctx));
         if (elapsed_ms) SLAI_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, L.ev0, L.ev1));
         return slai_read_buffer(ctx, L.out_tokens, 0, out_tokens, (size_t)n_steps * 4);
     }
-    slai_graph *&graph = sampling ? L.graph_sampled : L.graph;
-    if (!graph) {
+    // one captured token per launch form the run needs (the form depends on the position: Model::form_at)
+    for (uint32_t i = 0; i < n_steps; ++i) {
+        slai_graph *&graph = L.graph[m->form_at(start_pos + i)][sampling ? 1 : 0];
+        if (graph) continue;
         TRY(slai_graph_begin_capture(ctx));
-        int rc = m->enqueue_fused(mode);
+        int rc = m->enqueue_fused(mode, m->form_at(start_pos + i));
         slai_graph *g = nullptr;
         int rc2 = slai_graph_end_capture(ctx, &g);
         if (rc) { if (g) slai_graph_destroy(ctx, g); return rc; }
@@ -1095,7 +1104,7 @@ static int generate_impl(Model *m, slai_ctx *ctx, DeviceLoop &L, uint32_t seq_le
         graph = g;
     }
     SLAI_HIP_TRY(ctx, hipEventRecord(L.ev0, ctx->stream));
-    for (uint32_t i = 0; i < n_steps; ++i) TRY(slai_graph_launch(ctx, graph));         // chat_llama2.rs:109 loop
+    for (uint32_t i = 0; i < n_steps; ++i) TRY(slai_graph_launch(ctx, L.graph[m->form_at(start_pos + i)][sampling ? 1 : 0]));   // chat_llama2.rs:109 loop
     SLAI_HIP_TRY(ctx, hipEventRecord(L.ev1, ctx->stream));
     TRY(slai_synchronize(ctx));
     TRY(handoff_check(ctx));
@@ -1219,7 +1228,8 @@ struct slai_gpt2 {
     uint32_t attn_splits = 1;
 
     int load(const slai_gguf *g);
-    int enqueue_fused(int sampler);   // 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state
+    int enqueue_fused(int sampler, int form = 0);   // 0: stop at the logits, 1: greedy pick + loop state, 2: temperature / top-p pick + loop state (one form only)
+    int form_at(uint32_t) const { return 0; }
 
     // Prompt tokens in chunks of up to 32 on the matrix cores (see slai_llama2::enqueue_chunk_gemm); row-major x and qkv,
     // quad-major xn (normalised rows, then the attention output) and h.
@@ -1342,7 +1352,7 @@ int slai_gpt2::load(const slai_gguf *gg) {
 }
 
 // gpt2/cpu.rs:224-383 as fused kernels (LayerNorm eps 1e-5: ops/layernorm.rs:105)
-int slai_gpt2::enqueue_fused(int sampler) {
+int slai_gpt2::enqueue_fused(int sampler, int) {
     DecodeState *ds = (DecodeState *)loop.state->dptr;
     const uint32_t E = params.n_embd;
     float *x = (float *)layer_input.buf->dptr, *att_out = (float *)curr_768.buf->dptr, *qkv = (float *)curr_2304.buf->dptr,

@@ -50,7 +50,7 @@ SLAI_HD bool shape_ok(const Shape &s) {
     if (s.hidden % 256 || s.hidden / 256 > 64) return false;                                   // sixteen waves x four super-blocks in the down projection
     if (s.grid != s.dim / 16 || s.qkv_units != 7 || (s.qkv_units + 1) * s.n_heads != s.grid) return false;   // a role for every workgroup in the first two phases
     if (s.gu_rows == 0 || s.gu_rows > 64 || (s.hidden + s.gu_rows - 1) / s.gu_rows != s.grid) return false;  // ... and in gate / up
-    if (s.seq_len == 0 || s.seq_len > 1024 || s.n_layers == 0 || s.vocab == 0) return false;
+    if (s.seq_len == 0 || s.seq_len > 65536 || s.n_layers == 0 || s.vocab == 0) return false;     // (a cache stays far below 4 GiB: cache_elem)
     return true;
 }
 

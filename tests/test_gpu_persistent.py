@@ -16,13 +16,16 @@ from test_gpu_models import check_llama
 pytestmark = pytest.mark.gpu
 
 
-def backend_with(persistent):
+def backend_with(persistent, resident_max_pos=None):
     from slai_amd.runtime import Backend
     os.environ["SLAI_PERSISTENT"] = "1" if persistent else "0"
+    if resident_max_pos is not None:
+        os.environ["SLAI_RESIDENT_MAX_POS"] = str(resident_max_pos)
     try:
         return Backend(0)
     finally:
         del os.environ["SLAI_PERSISTENT"]
+        os.environ.pop("SLAI_RESIDENT_MAX_POS", None)
 
 
 @pytest.mark.parametrize("kv_f16", [True, False])
@@ -49,6 +52,20 @@ def test_persistent_long_context_vs_oracle(kv_f16):
         data = gw.llama_gguf(dim=1024, hidden_dim=3072, n_layers=2, n_heads=8, n_kv_heads=8, vocab=2000, seq_len=640, wtype=12, v_type=14,
                              out_type=14, embd_type=12, seed=77, std=0.05, norm_random=True)
         check_llama(b, data, [5, 1000, 1999], 600, kv_f16=kv_f16, check_logit_steps=4, decode_form=1)
+    finally:
+        b.close()
+
+
+@pytest.mark.parametrize("kv_f16", [True, False])
+def test_launch_form_changes_with_the_position(kv_f16):
+    """A model with a context of 2048 takes the resident launch for its first positions and one launch per step beyond
+    (here from position 21 on, so that the prompt, the step-by-step logits and the generated ids all cross the change):
+    both forms keep the same caches and loop state, and the ids and logits follow the oracle's throughout."""
+    b = backend_with(True, resident_max_pos=21)
+    try:
+        data = gw.llama_gguf(dim=1024, hidden_dim=3072, n_layers=2, n_heads=8, n_kv_heads=8, vocab=2000, seq_len=2048, wtype=12, v_type=14,
+                             out_type=14, embd_type=12, seed=91, std=0.05, norm_random=True)
+        check_llama(b, data, [5, 1000, 1999, 9, 77, 3, 8, 21], 40, kv_f16=kv_f16, check_logit_steps=30, decode_form=1)
     finally:
         b.close()
 

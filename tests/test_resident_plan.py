@@ -40,6 +40,7 @@ SHAPES = {
     "dim 2048": dict(dim=2048, hidden=5632, n_heads=16, n_layers=4, vocab=4096, seq_len=512),
     "7B width, 2 layers": dict(dim=4096, hidden=11008, n_heads=32, n_layers=2, vocab=32000, seq_len=128),
     "config 4": dict(dim=4096, hidden=11008, n_heads=32, n_layers=32, vocab=32000, seq_len=512),
+    "7B width, context 4096, f32 cache": dict(dim=4096, hidden=11008, n_heads=32, n_layers=2, vocab=32000, seq_len=4096, kv_bytes=4),
     "NeoX rotary pairs": dict(dim=2048, hidden=5632, n_heads=16, n_layers=2, vocab=4096, seq_len=300, neox=1),
     "wide FFN (12 column groups in the down projection)": dict(dim=3072, hidden=12288, n_heads=24, n_layers=2, vocab=1000, seq_len=64, types=(Q5_K, Q4_K, Q4_K, Q6_K, Q4_K, Q4_K, Q4_K)),
 }
@@ -68,7 +69,7 @@ def test_the_decomposition_gives_every_workgroup_a_role_in_every_phase(rb):
 
 
 def test_unsupported_shapes_are_refused(rb):
-    for kw in (dict(dim=4096, hidden=11008, n_heads=32, n_layers=2, vocab=32000, seq_len=2048),      # context beyond one workgroup per head
+    for kw in (dict(dim=4096, hidden=11008, n_heads=32, n_layers=2, vocab=32000, seq_len=100000),    # context beyond what the plan admits
                dict(dim=5120, hidden=13824, n_heads=40, n_layers=2, vocab=32000, seq_len=512),       # width beyond four staging pieces per lane
                dict(dim=3072, hidden=4096, n_heads=24, n_layers=2, vocab=100, seq_len=64),           # 192 workgroups: units of 22 rows cover 4096 rows with 187
                dict(dim=1024, hidden=2800, n_heads=8, n_layers=2, vocab=100, seq_len=64)):            # FFN width not in super-blocks
