@@ -63,18 +63,24 @@ __device__ __forceinline__ float sum8(float v) {
     v += dpp<DPP_XOR1>(v); v += dpp<DPP_XOR2>(v); v += dpp<DPP_HALF_MIRROR>(v);
     return v;
 }
-// the largest of a non-negative value's bit patterns over the wave, as a wave-uniform word
+// max(m, the word of the lane CTRL names), unsigned: zero, what a lane without a source reads, is neutral, so the exchange
+// folds into the instruction (and an integer maximum needs no canonical operands, as a float one does)
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_umax(uint32_t m) {
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, CTRL, 0xf, 0xf, true);
+    return m > o ? m : o;
+}
+// the largest of a non-negative value's bit patterns over the wave, as a wave-uniform word (such patterns order like the values)
 __device__ __forceinline__ uint32_t max64_bits(float v) {
-    v = fmaxf(v, dpp<DPP_XOR1>(v)); v = fmaxf(v, dpp<DPP_XOR2>(v)); v = fmaxf(v, dpp<DPP_HALF_MIRROR>(v)); v = fmaxf(v, dpp<DPP_MIRROR>(v));
-    const int b = __builtin_bit_cast(int, v);
+    uint32_t m = __builtin_bit_cast(uint32_t, v);
+    m = dpp_umax<DPP_XOR1>(m); m = dpp_umax<DPP_XOR2>(m); m = dpp_umax<DPP_HALF_MIRROR>(m); m = dpp_umax<DPP_MIRROR>(m);
+    const int b = (int)m;
     const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane(b, 0), r1 = (uint32_t)__builtin_amdgcn_readlane(b, 16);
     const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane(b, 32), r3 = (uint32_t)__builtin_amdgcn_readlane(b, 48);
     const uint32_t a = r0 > r1 ? r0 : r1, c = r2 > r3 ? r2 : r3;
     return a > c ? a : c;
 }
-__device__ __forceinline__ uint32_t pack_f16(_Float16 a, _Float16 b) {
-    return (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
-}
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_f16(_Float16 a, _Float16 b) { return __builtin_bit_cast(uint32_t, half2v{a, b}); }
 
 // Stages the 256 activations of one super-block: lane i of the wave holds elements 4 i .. 4 i + 3 in `x`.  `sb`: the
 // super-block's block in LDS (SB_BYTES, 16-byte aligned).  Q4_K: element e = 64 J + 32 nib + 16 H + 8 h + i' belongs to
