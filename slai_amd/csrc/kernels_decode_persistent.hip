@@ -7,8 +7,9 @@
 // where they are and hand the vectors over themselves:
 //   * a producer writes its slice of the vector with agent-scope stores into a buffer that was filled with FLOW_EMPTY
 //     before the launch (one buffer per layer and vector, so nothing is ever reused inside a launch);
-//   * a consumer watches one word of the vector until it is there, then repeats its load of its whole part until no
-//     element of it is empty -- the data is its own flag: no counter, no fence, no barrier round trip;
+//   * a consumer watches one word of the vector until it is there, then asks for its whole part, and the lanes that see
+//     an empty word in theirs ask again until none does -- the data is its own flag: no counter, no fence, no barrier
+//     round trip;
 //   * a wave asks for the weights of its NEXT phase as soon as the registers of the current one are free, right after its
 //     dot product: the weights travel while the hand-off is waited for.  Loads retire in issue order, so a wave's poll
 //     waits behind its own requests: every wave waits for its own input itself, with the unit it multiplies next asked
