@@ -89,7 +89,7 @@ struct slai_ctx {
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
     // the one-launch-per-token form of the Llama-2 layer stack where a model's shapes allow it (SLAI_PERSISTENT=0 switches it off)
     bool persistent = true;
-    uint32_t resident_max_pos = 1536;   // tokens at positions below this take the resident launch (where the model has one): SLAI_RESIDENT_MAX_POS
+    uint32_t resident_max_pos = 2176;   // tokens at positions below this take the resident launch (where the model has one): SLAI_RESIDENT_MAX_POS
     // When set, every launch of a decode step is followed by an event recorded under the step's name
     // (slai_llama2_time_steps); null otherwise.
     std::vector<std::pair<const char *, hipEvent_t>> *step_marks = nullptr;
@@ -426,6 +426,8 @@ struct PersistentParams {
 size_t persistent_smem_bytes(const PersistentParams &p);
 hipError_t persistent_capacity(const PersistentParams &p, int device, uint32_t *resident);
 hipError_t launch_flow_fill(hipStream_t s, void *buf, size_t bytes);
-hipError_t launch_decode_persistent(hipStream_t s, const PersistentParams &p, uint32_t grid);
+// far: the variant for a position beyond resident_far_from(kv_f16), whose unit workgroups touch the far cache rows into L2
+hipError_t launch_decode_persistent(hipStream_t s, const PersistentParams &p, uint32_t grid, bool far);
+uint32_t resident_far_from(bool kv_f16);
 
 }  // namespace slai

@@ -95,7 +95,7 @@ struct DeviceLoop {           // device-resident state of the greedy loop
     slai_buffer *prompt = nullptr;      // int32[capacity]
     slai_buffer *out_tokens = nullptr;  // int32[capacity]
     uint32_t capacity = 0;
-    slai_graph *graph[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};   // one token, [launch form][greedy pick | temperature / top-p pick]
+    slai_graph *graph[3][2] = {{nullptr, nullptr}, {nullptr, nullptr}, {nullptr, nullptr}};   // one token, [launch form][greedy pick | temperature / top-p pick]
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 };
 int loop_init(slai_ctx *ctx, DeviceLoop &L, uint32_t capacity) {
@@ -186,7 +186,7 @@ struct slai_llama2 {
     } persistent;
     bool persistent_supported() const;
     int persistent_setup();
-    int enqueue_persistent(int sampler);
+    int enqueue_persistent(int sampler, bool far);
 
     // Prompt tokens in chunks: every weight matrix is read once per chunk instead of once per token.
     PromptChunkState chunk;
@@ -430,14 +430,14 @@ int slai_llama2::persistent_setup() {
 }
 
 // embedding row | hand-off buffers emptied | the layer stack and the output matrix | pick
-int slai_llama2::enqueue_persistent(int sampler) {
+int slai_llama2::enqueue_persistent(int sampler, bool far) {
     Llama2State &s = state;
     DecodeState *ds = (DecodeState *)loop.state->dptr;
     SLAI_HIP_TRY(ctx, launch_embed(ctx->stream, weights.token_embd, &ds->token, nullptr, nullptr, config.dim, (float *)s.x.buf->dptr));
     TRY(step_mark(ctx, "embedding row"));
     SLAI_HIP_TRY(ctx, launch_flow_fill(ctx->stream, persistent.flow->dptr, persistent.flow_bytes));
     TRY(step_mark(ctx, "hand-off buffers emptied"));
-    SLAI_HIP_TRY(ctx, launch_decode_persistent(ctx->stream, persistent.params, persistent.grid));
+    SLAI_HIP_TRY(ctx, launch_decode_persistent(ctx->stream, persistent.params, persistent.grid, far));
     TRY(step_mark(ctx, "llama2 resident token"));
     if (sampler == 1)
         SLAI_HIP_TRY(ctx, launch_argmax(ctx->stream, (const float *)s.logits.buf->dptr, config.vocab_size, nullptr, ds,
@@ -493,10 +493,16 @@ int slai_llama2::launch(LlmContext &ctxt, const slai_attn_params &attn_params, u
 // The resident launch walks a head's cached positions with one workgroup, at the rate one compute unit reads memory;
 // the launch-per-step form spreads them over the device.  Up to ctx->resident_max_pos positions the resident launch is
 // the faster one, beyond it the steps are: the form is chosen per token (both keep the same caches and loop state).
-int slai_llama2::form_at(uint32_t pos) const { return persistent.ready && pos < ctx->resident_max_pos ? 1 : 0; }
+// (Forms: 0 one launch per step, 1 the resident launch, 2 the resident launch whose unit workgroups also bring the cache
+// rows beyond the ones the attention asks for ahead into the die's L2 -- a kernel of its own, so that the short contexts do
+// not carry that code.)
+int slai_llama2::form_at(uint32_t pos) const {
+    if (!persistent.ready || pos >= ctx->resident_max_pos) return 0;
+    return pos > resident_far_from(kv_dtype == SLAI_KV_F16) ? 2 : 1;
+}
 
 int slai_llama2::enqueue_fused(int sampler, int form) {
-    if (form == 1) return persistent.ready ? enqueue_persistent(sampler) : set_error(ctx, SLAI_E_STATE, "this model does not take the resident launch");
+    if (form != 0) return persistent.ready ? enqueue_persistent(sampler, form == 2) : set_error(ctx, SLAI_E_STATE, "this model does not take the resident launch");
     Llama2State &s = state;
     DecodeState *ds = (DecodeState *)loop.state->dptr;
     float *x = (float *)s.x.buf->dptr, *xb = (float *)s.xb.buf->dptr, *hb = (float *)s.hb.buf->dptr, *hb2 = (float *)s.hb2.buf->dptr;
@@ -932,7 +938,7 @@ SLAI_EXPORT int slai_llama2_trace_token(slai_llama2 *m, uint32_t pos, uint32_t t
     DecodeState ds{(int)pos, (int)token, 0, 0};
     int rc = slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds);
     m->persistent.params.trace = (uint64_t *)buf->dptr;
-    if (!rc) rc = m->enqueue_persistent(0);
+    if (!rc) rc = m->enqueue_persistent(0, pos > resident_far_from(m->kv_dtype == SLAI_KV_F16));
     m->persistent.params.trace = nullptr;
     if (!rc) rc = slai_synchronize(ctx);
     if (!rc) rc = handoff_check(ctx);
@@ -953,7 +959,7 @@ SLAI_EXPORT int slai_llama2_time_steps(slai_llama2 *m, uint32_t pos, uint32_t to
     if (ctx->capturing) return set_error(ctx, SLAI_E_STATE, "slai_llama2_time_steps: not during graph capture");
     DecodeState ds{(int)pos, (int)token, 0, 0};
     TRY(slai_write_buffer(ctx, m->loop.state, 0, &ds, sizeof ds));
-    const auto enqueue = [&]() { return m->enqueue_fused(0, m->persistent.ready ? 1 : 0); };
+    const auto enqueue = [&]() { return m->enqueue_fused(0, m->persistent.ready ? (pos > resident_far_from(m->kv_dtype == SLAI_KV_F16) ? 2 : 1) : 0); };
     TRY(enqueue());                                             // untimed: sizes scratch, warms the caches
     TRY(slai_synchronize(ctx));
     std::vector<std::pair<const char *, hipEvent_t>> marks;

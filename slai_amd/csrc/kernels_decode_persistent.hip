@@ -739,12 +739,28 @@ __device__ __forceinline__ plan::Shape shape_of(const PersistentParams &p) {
     return plan::Shape{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, gridDim.x, p.qkv_units, p.gu_rows, p.rope_variant == SLAI_ROPE_NEOX ? 1u : 0u};
 }
 
+// A long context (plan::att_ahead): the head's attention walks the cached rows beyond the ones it asked for ahead at the
+// rate one compute unit reads memory.  The seven workgroups of the head's units sit on the same die and wait for the
+// attention's result anyway: their tile waves touch one word of every line of those rows, so that the attention finds
+// them in the die's L2.
+__device__ __forceinline__ void touch_far_rows(const plan::Shape &sh, uint32_t b, uint32_t pos, bool f16, uint32_t tile_waves, Rsrc kc, Rsrc vc, uint32_t wave_) {
+    const uint32_t wave = fresh(wave_), n = plan::touch_count(pos, f16);
+    if (wave >= tile_waves || n == 0) return;
+    const uint32_t head = plan::qkv_head(sh, b), t = (b >> 3) % sh.qkv_units;
+    uint32_t any = 0;
+    for (uint32_t w = plan::touch_first(t, tile_waves, wave, lane_id()); w < n; w += plan::touch_stride(sh, tile_waves)) {
+        const int off = (int)plan::touch_byte(sh, w, head, f16);
+        any |= plan::touch_is_value(w, f16) ? __builtin_amdgcn_raw_buffer_load_b32(vc, off, 0, AUX_PLAIN) : __builtin_amdgcn_raw_buffer_load_b32(kc, off, 0, AUX_PLAIN);
+    }
+    asm volatile("" : : "v"(any));                                  // (the words are not used: the requests are the point)
+}
+
 // ---- the kernel ------------------------------------------------------------------------------------------------------------
 // Workgroup roles: resident_plan.h (plan::qkv_unit, attention_head, gu_unit, proj_tiles, out_tiles).  The body exists
 // twice, for the workgroups that run a head's attention in the first phase of a layer (ATTN) and for those that multiply
 // a q / k / v unit there (or nothing): the attention needs nearly all registers, and only a body of its own shows the
 // compiler that no unit requested ahead is ever alive across it.
-template <bool F16, bool ATTN>
+template <bool F16, bool ATTN, bool FAR>
 __device__ __forceinline__ void decode_token(const PersistentParams &p, float *smem, float (&rope_cs)[2][64], uint32_t (&layer_words)[2][sizeof(PersistentLayer) / 4],
                                              const uint32_t wave) {
     constexpr int LWORDS = sizeof(PersistentLayer) / 4;
@@ -881,6 +897,16 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
             uint64_t *tp = tl ? tl + 4 : nullptr;
             float residual;
             stamp(tp, 0, wave);
+            // A long context: the head's attention walks the cached rows beyond the ones it asked for ahead at the rate one
+            // compute unit reads memory.  The seven workgroups of the head's units sit on the same die and wait here anyway:
+            // their tile waves touch one word of every line of those rows, so that the attention finds them in the die's L2.
+            static_assert((Attention<F16>::ATT_PRE + 1) * plan::ATT_PASS == plan::att_ahead(F16), "what the attention requests before the query");
+            if constexpr (FAR) {
+                // (only in the kernel the host launches for long contexts: the short ones, which the throughput is quoted on,
+                // should not carry this code and its registers)
+                const DevBuf kc = LAYER_BUF(lw, kcache), vc = LAYER_BUF(lw, vcache);
+                touch_far_rows(sh, b, pos, F16, ng_o, kc.rs, vc.rs, wave);
+            }
             mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, lds, PHASE_PARTIAL, f, tp, wave);
             ask_gate_up(lw);                                        // (the waves without a part in the tiles: at once)
             const float o = finish16(wo_t, ng_o, PHASE_PARTIAL, tp, wave);
@@ -939,7 +965,8 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
 
 // The description of the current layer and of the next one is parked in LDS.  Read from memory at the moment of use, its
 // lines (which the weight stream has long pushed out of L2) would cost a round trip to memory each, one after the other.
-template <bool F16>
+// FAR: the variant for positions beyond plan::att_ahead (touch_far_rows); the host picks it per token.
+template <bool F16, bool FAR>
 __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const PersistentParams p) {
     extern __shared__ __align__(16) float smem[];
     __shared__ float rope_cs[2][64];                               // cosine | sine of the rotation of wave 0's rows (q and k units)
@@ -955,8 +982,8 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
     __syncthreads();
     const plan::Shape sh = shape_of(p);
     const uint32_t wave = uniform_word(threadIdx.x >> 6);
-    if (plan::is_attention_workgroup(sh, blockIdx.x)) decode_token<F16, true>(p, smem, rope_cs, layer_words, wave);
-    else decode_token<F16, false>(p, smem, rope_cs, layer_words, wave);
+    if (plan::is_attention_workgroup(sh, blockIdx.x)) decode_token<F16, true, false>(p, smem, rope_cs, layer_words, wave);
+    else decode_token<F16, false, FAR>(p, smem, rope_cs, layer_words, wave);
 }
 
 #undef PHASE_PARTIAL
@@ -979,8 +1006,10 @@ size_t persistent_smem_bytes(const PersistentParams &p) {
 hipError_t persistent_capacity(const PersistentParams &p, int device, uint32_t *resident) {
     *resident = 0;
     const size_t smem = persistent_smem_bytes(p);
-    const void *fn = p.kv_f16 ? (const void *)llama_decode_persistent_kernel<true> : (const void *)llama_decode_persistent_kernel<false>;
+    const void *fn = p.kv_f16 ? (const void *)llama_decode_persistent_kernel<true, false> : (const void *)llama_decode_persistent_kernel<false, false>;
+    const void *far = p.kv_f16 ? (const void *)llama_decode_persistent_kernel<true, true> : (const void *)llama_decode_persistent_kernel<false, true>;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e == hipSuccess) e = hipFuncSetAttribute(far, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     int per_cu = 0;
     e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, PNT, smem);
@@ -992,18 +1021,20 @@ hipError_t persistent_capacity(const PersistentParams &p, int device, uint32_t *
     return hipSuccess;
 }
 
+uint32_t resident_far_from(bool kv_f16) { return plan::att_ahead(kv_f16); }
+
 hipError_t launch_flow_fill(hipStream_t s, void *buf, size_t bytes) {
     if (bytes % 16 || (uintptr_t)buf % 16) return hipErrorInvalidValue;
     flow_fill_kernel<<<64, 1024, 0, s>>>((u32x4 *)buf, bytes / 16);
     return hipGetLastError();
 }
 
-hipError_t launch_decode_persistent(hipStream_t s, const PersistentParams &p, uint32_t grid) {
+hipError_t launch_decode_persistent(hipStream_t s, const PersistentParams &p, uint32_t grid, bool far) {
     const plan::Shape sh{p.dim, p.hidden, p.n_heads, p.n_layers, p.vocab, p.seq_len, grid, p.qkv_units, p.gu_rows};
     if (!plan::shape_ok(sh)) return hipErrorInvalidValue;          // the index arithmetic of the kernel assumes these
     const size_t smem = persistent_smem_bytes(p);
-    if (p.kv_f16) llama_decode_persistent_kernel<true><<<grid, PNT, smem, s>>>(p);
-    else llama_decode_persistent_kernel<false><<<grid, PNT, smem, s>>>(p);
+    if (p.kv_f16) { if (far) llama_decode_persistent_kernel<true, true><<<grid, PNT, smem, s>>>(p); else llama_decode_persistent_kernel<true, false><<<grid, PNT, smem, s>>>(p); }
+    else { if (far) llama_decode_persistent_kernel<false, true><<<grid, PNT, smem, s>>>(p); else llama_decode_persistent_kernel<false, false><<<grid, PNT, smem, s>>>(p); }
     return hipGetLastError();
 }
 

@@ -98,6 +98,22 @@ SLAI_HD uint32_t att_v_pos(uint32_t tb, uint32_t wave, uint32_t u, uint32_t lane
 SLAI_HD uint32_t att_v_elem(uint32_t head, uint32_t lane) { return head * 128 + (lane & 15u) * 8; }
 // element e of position t of a cache [seq_len x dim] (times the element size: below 4 GiB, shape_ok bounds seq_len and dim)
 SLAI_HD uint32_t cache_elem(const Shape &s, uint32_t t, uint32_t e) { return t * s.dim + e; }
+// The attention asks for the first att_ahead() cached positions before the query exists; the rows beyond them it walks at
+// the rate one compute unit reads memory.  The workgroups of the head's q / k / v units (same die) therefore touch one
+// word of every 128-byte line of those rows while they wait for the attention's result, so that the attention finds them
+// in the die's L2.  Touch number w of a head: row att_ahead + w / (2 lines_per_row), key | value, line w % lines_per_row.
+SLAI_HD constexpr uint32_t att_ahead(bool f16) { return (f16 ? 4u : 2u) * ATT_PASS; }
+SLAI_HD uint32_t touch_lines_per_row(uint32_t elem_bytes) { return 128u * elem_bytes / 128u; }
+SLAI_HD uint32_t touch_count(uint32_t pos, bool f16) { const uint32_t a = att_ahead(f16); return pos > a ? (pos - a) * 2u * touch_lines_per_row(f16 ? 2u : 4u) : 0u; }
+SLAI_HD uint32_t touch_row(uint32_t w, bool f16) { return att_ahead(f16) + w / (2u * touch_lines_per_row(f16 ? 2u : 4u)); }
+SLAI_HD bool touch_is_value(uint32_t w, bool f16) { return (w / touch_lines_per_row(f16 ? 2u : 4u)) & 1u; }
+SLAI_HD uint32_t touch_byte(const Shape &s, uint32_t w, uint32_t head, bool f16) {
+    const uint32_t es = f16 ? 2u : 4u;
+    return cache_elem(s, touch_row(w, f16), head * 128u) * es + (w % touch_lines_per_row(es)) * 128u;
+}
+// touches are dealt to the tile waves of the head's unit workgroups: worker (unit t, wave, lane) starts at its index and strides
+SLAI_HD uint32_t touch_first(uint32_t t, uint32_t tile_waves, uint32_t wave, uint32_t lane) { return (t * tile_waves + wave) * 64u + lane; }
+SLAI_HD uint32_t touch_stride(const Shape &s, uint32_t tile_waves) { return s.qkv_units * tile_waves * 64u; }
 // the control block: one 128-byte line per head (counters of the launches that hand q / k / v over per step), then the
 // flag of a wait that gave up
 SLAI_HD uint32_t counter_word(uint32_t head, uint32_t which = 0) { return head * 32 + which; }

@@ -182,6 +182,7 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
         for (uint32_t l = 0; l < n_layers && a.violations < 8; ++l) {
             std::vector<uint32_t> rows_q(dim, 0), rows_k(dim, 0), rows_v(dim, 0), rows_h(hidden, 0), rows_o(dim, 0), rows_d(dim, 0);
             std::vector<uint32_t> heads_attended(n_heads, 0), units_of_head(n_heads, 0);
+            std::vector<std::vector<uint32_t>> touched(n_heads, std::vector<uint32_t>(plan::touch_count(seq_len - 1, kv_bytes == 2), 0));
             // a hand-off vector of this layer as a region of its own size, placed inside the allocation
             const auto vec = [&](const char *name, uint64_t first_float, uint64_t n) {
                 a.touch(flow, first_float * 4, n * 4, "hand-off row", 0, 0, 0, l);
@@ -216,6 +217,21 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                             const uint32_t partner = plan::unit_row(u, s.neox ? t ^ 32u : t ^ 1u);
                             if (partner != (s.neox ? row ^ 64u : row ^ 1u) || (s.neox ? t ^ 32u : t ^ 1u) >= u.nrows) a.fail("a rotary pair is split over units");
                         }
+                    }
+                    // the far cache rows of the head, touched into the die's L2 by the tile waves of its unit workgroups: every
+                    // 128-byte line of every row beyond what the attention asks for ahead, of key and value, exactly once
+                    {
+                        const bool f16 = kv_bytes == 2;
+                        const uint32_t T = seq_len - 1, n = plan::touch_count(T, f16), t = (b >> 3) % s.qkv_units;
+                        for (uint32_t wave = 0; wave < ng_o; ++wave)
+                            for (uint32_t lane = 0; lane < 64; ++lane)
+                                for (uint32_t w = plan::touch_first(t, ng_o, wave, lane); w < n; w += plan::touch_stride(s, ng_o)) {
+                                    const uint32_t byte = plan::touch_byte(s, w, h, f16);
+                                    a.touch(cache, byte, 4, "cache line touched", b, wave, lane, l);
+                                    const uint32_t row = plan::touch_row(w, f16), in_row = byte - plan::cache_elem(s, row, h * 128) * kv_bytes;
+                                    if (row < plan::att_ahead(f16) || row >= T || byte % 128 != 0 || in_row >= 128 * kv_bytes) a.fail("a touch outside the head's far cache rows");
+                                    ++touched[h][(size_t)w];
+                                }
                     }
                 } else if (plan::is_attention_workgroup(s, b)) {
                     const uint32_t h = plan::attention_head(s, b);
@@ -268,6 +284,9 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                     for (uint32_t t = 0; t < u.nrows; ++t) a.touch(hb, (uint64_t)(u.row0 + t) * 4, 4, "hb store", b, 0, t, l);
                 }
             }
+            for (uint32_t h = 0; h < n_heads; ++h)
+                for (size_t w = 0; w < touched[h].size(); ++w)
+                    if (touched[h][w] != 1) { a.fail("far cache rows of head " + std::to_string(h) + ": line " + std::to_string(w) + " is touched " + std::to_string(touched[h][w]) + " times"); h = n_heads; break; }
             const auto once = [&](const std::vector<uint32_t> &v, const char *what) {
                 for (size_t i = 0; i < v.size(); ++i)
                     if (v[i] != 1) { a.fail(std::string(what) + ": row " + std::to_string(i) + " is produced " + std::to_string(v[i]) + " times in layer " + std::to_string(l)); return; }

@@ -46,7 +46,8 @@ def test_persistent_small_model_vs_oracle(kv_f16):
 def test_persistent_long_context_vs_oracle(kv_f16):
     """600 steps on the small model: the attention asks for the first 384 cached positions (f16 cache; 128 with an f32
     cache) before the query exists and walks the rest in passes of 128 with one pass in flight; positions 128, 129, 384,
-    385, 512, 513 are where those paths change."""
+    385, 512, 513 are where those paths change.  Beyond position 512 (256 with an f32 cache) the host launches the
+    variant of the kernel whose unit workgroups touch the far cache rows into the die's L2."""
     b = backend_with(True)
     try:
         data = gw.llama_gguf(dim=1024, hidden_dim=3072, n_layers=2, n_heads=8, n_kv_heads=8, vocab=2000, seq_len=640, wtype=12, v_type=14,
