@@ -87,7 +87,9 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
     using CT = typename C::T;
     constexpr int NW = NT / 64;
     // KL lanes share a position in the score phase (4, or 8 where registers are scarce: half as many elements per lane)
-    constexpr int EPL = HS / KL;                  // elements per lane in the score phase
+    constexpr int EPL = HS / KL;                  // elements per lane in the score phase: piece jj (eight of them) is elements
+                                                  // 8 KL jj + 8 sub .. + 7, so that the KL lanes of a position ask for 16 KL contiguous
+                                                  // bytes (of an f16 cache) in one request, not for 16 bytes each at a stride of 2 EPL
     constexpr int PPW = 64 / KL;                  // positions a wave owns per pass
     constexpr int LPP = HS / 8;                   // lanes per position in the value phase
     __shared__ float sq[HS], sk[HS], sv[HS];
@@ -150,9 +152,9 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
         const uint32_t t = t0 + tid / KL;
         // the fresh row comes from LDS later; lanes without a position read a valid address and are masked
         const uint32_t tc = (t < t1 && !(own_new && t == pos)) ? t : min(t0, pos);
-        const CT *kp = kc + (size_t)tc * a.kv_dim + hoff + sub * EPL;
+        const CT *kp = kc + (size_t)tc * a.kv_dim + hoff + sub * 8;
 #pragma unroll
-        for (int j = 0; j < EPL / 8; ++j) kv0[j] = Vec8<F16>::load_raw(kp + 8 * j);
+        for (int j = 0; j < EPL / 8; ++j) kv0[j] = Vec8<F16>::load_raw(kp + 8 * KL * j);
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
             const uint32_t tv = t0 + wpos + u * PW + vgl;
@@ -198,7 +200,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
     // pass is used. -----------------------------------------------------------------------------------------------
     float qr[EPL];
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) qr[j] = sq[sub * EPL + j];
+    for (int j = 0; j < EPL; ++j) qr[j] = sq[(j / 8) * 8 * KL + sub * 8 + (j % 8)];
     const float root = sqrtf((float)HS);
     float m = -FLT_MAX, lsum = 0.0f;
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -210,9 +212,9 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
         if (tb + NT / KL < t1) {                               // (uniform) there is a next pass
             const uint32_t tn = t + NT / KL;
             const uint32_t tnc = (tn < t1 && !(own_new && tn == pos)) ? tn : min(t0, pos);
-            const CT *kp = kc + (size_t)tnc * a.kv_dim + hoff + sub * EPL;
+            const CT *kp = kc + (size_t)tnc * a.kv_dim + hoff + sub * 8;
 #pragma unroll
-            for (int j = 0; j < EPL / 8; ++j) nxt[j] = Vec8<F16>::load_raw(kp + 8 * j);
+            for (int j = 0; j < EPL / 8; ++j) nxt[j] = Vec8<F16>::load_raw(kp + 8 * KL * j);
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
                 const uint32_t tv = tb + NT / KL + wpos + u * PW + vgl;
@@ -230,7 +232,7 @@ __device__ __forceinline__ void attn_fast_body(const AttnLaunch &a, uint32_t h, 
         }
         if (use_new) {
 #pragma unroll
-            for (int j = 0; j < EPL; ++j) kv[j] = sk[sub * EPL + j];
+            for (int j = 0; j < EPL; ++j) kv[j] = sk[(j / 8) * 8 * KL + sub * 8 + (j % 8)];
         }
         float part = 0.0f;
 #pragma unroll
