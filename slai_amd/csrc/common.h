@@ -359,6 +359,11 @@ struct AttnLaunch {
     float *out;              // [n_heads*head_size]
     float *scratch;          // n_heads*n_splits*(head_size+2) floats when n_splits > 1
     uint32_t n_splits;
+    // When set (n_splits > 1, fast form only): one zeroed 128-byte line of counters per head.  The workgroup of a head's
+    // split that finishes last merges the head's partial results itself and no combine launch follows.  Only for callers
+    // who have verified that workgroup i of a launch runs on die i mod 8 (slai_ctx::fuse_qkv_attention): the partial
+    // results of a head's splits then meet in that die's L2.
+    uint32_t *combine_counters;
 };
 hipError_t launch_attention(hipStream_t s, const AttnLaunch &a);
 // A chunk of `n` consecutive tokens whose keys and values are already in the caches: token b attends from q + b * q_stride

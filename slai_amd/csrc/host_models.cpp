@@ -533,6 +533,8 @@ int slai_llama2::enqueue_fused(int sampler, int form) {
         a.rope_variant = rope_variant(); a.rope_base = config.rope_base_freq;
         a.rope_theta = (const float *)s.rope_theta.buf->dptr;
         a.out = xb; a.scratch = ctx->attn_scratch; a.n_splits = attn_splits;
+        // (split attention: the last split of a head merges them, where the placement of workgroups on the dies was verified)
+        if (ctx->fuse_qkv_attention && ctx->handoff_counters && a.n_heads <= ctx->handoff_heads) a.combine_counters = ctx->handoff_counters;
         bool attention_done = false;
         // ---- RMSNorm + Q/K/V projections: matrices of one format and layout share a launch
         {

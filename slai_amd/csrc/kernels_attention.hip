@@ -177,6 +177,8 @@ __global__ void __launch_bounds__(ATT_THREADS) attn_kernel(AttnLaunch a, uint32_
 // a die's workgroups share its L2, so the workgroups of one (kv head, split) are given indices 8 apart: they run at the
 // same time on one die, the rows come from memory once, and the other kv_mul - 1 workgroups find them in that L2.
 //   b = (key mod 8) + 8 * (j + kv_mul * (key / 8)),  key = kv head + n_kv_heads * split,  j = query head within the group
+__device__ __forceinline__ void combine_head(const float *scratch, float *out, uint32_t hs, uint32_t n_splits, uint32_t h, uint32_t tid, uint32_t nthreads, float *sw);
+
 template <bool F16, int NT, int HS, bool SINGLE>
 __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t max_split_len, uint32_t grouped) {
     touch_kernel_arguments<sizeof(AttnLaunch) + 8>();
@@ -189,6 +191,27 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
         split = key / n_kv;
     }
     attn_fast_body<F16, NT, HS, SINGLE, false>(a, h, split, threadIdx.x, []() {});
+    if constexpr (!SINGLE) {
+        // The last of a head's splits merges them: every workgroup waits until its partial result is in the die's L2
+        // (all splits of the head run on this die: the launcher has checked), then counts itself in with an atomic that
+        // executes there and returns the count; the one that completes it finds every partial result in that L2.
+        if (a.combine_counters) {
+            __shared__ uint32_t last;
+            __shared__ float sw[64];
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                uint32_t *counter = a.combine_counters + (size_t)h * 32;
+                uint32_t seen;
+                const uint32_t one = 1;
+                asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=&v"(seen) : "v"(counter), "v"(one) : "memory");
+                last = seen + 1 == a.n_splits ? 1u : 0u;
+                if (last) *counter = 0u;                               // for the next launch; nobody else touches it any more
+            }
+            __syncthreads();
+            if (last) combine_head(a.scratch, a.out, HS, a.n_splits, h, threadIdx.x, NT, sw);
+        }
+    }
 }
 // the size of that grid
 static uint32_t grouped_grid(const AttnLaunch &a) {
@@ -265,9 +288,7 @@ __global__ void rope_theta_kernel(float *out, uint32_t hs, float base) {
 // grid = n_heads, block = 128: merge the per-split (max, sum, unnormalised output) triples.
 // n_splits <= 64: one lane per split computes its weight exp(m_s - M) / L, then every thread
 // accumulates its output elements with independent loads.
-__global__ void __launch_bounds__(128) attn_combine_kernel(const float *scratch, float *out, uint32_t hs, uint32_t n_splits) {
-    __shared__ float sw[64];
-    const uint32_t h = blockIdx.x, tid = threadIdx.x;
+__device__ __forceinline__ void combine_head(const float *scratch, float *out, uint32_t hs, uint32_t n_splits, uint32_t h, uint32_t tid, uint32_t nthreads, float *sw /* [64], LDS */) {
     const float *base = scratch + (size_t)h * n_splits * (hs + 2);
     if (tid < 64) {
         const bool on = tid < n_splits;
@@ -279,12 +300,16 @@ __global__ void __launch_bounds__(128) attn_combine_kernel(const float *scratch,
         sw[tid] = w / L;
     }
     __syncthreads();
-    for (uint32_t e = tid; e < hs; e += blockDim.x) {
+    for (uint32_t e = tid; e < hs; e += nthreads) {
         float acc = 0.0f;
 #pragma unroll 8
         for (uint32_t s = 0; s < n_splits; ++s) acc = fmaf(sw[s], base[(size_t)s * (hs + 2) + e], acc);
         out[(size_t)h * hs + e] = acc;
     }
+}
+__global__ void __launch_bounds__(128) attn_combine_kernel(const float *scratch, float *out, uint32_t hs, uint32_t n_splits) {
+    __shared__ float sw[64];
+    combine_head(scratch, out, hs, n_splits, blockIdx.x, threadIdx.x, blockDim.x, sw);
 }
 
 }  // namespace
@@ -298,7 +323,18 @@ size_t attention_scratch_floats(uint32_t n_heads, uint32_t head_size, uint32_t n
     return n_splits > 1 ? (size_t)n_heads * n_splits * (head_size + 2) : 0;
 }
 
-hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
+hipError_t launch_attention(hipStream_t s, const AttnLaunch &a_in) {
+    AttnLaunch a = a_in;
+    {
+        // The splits of a head merge themselves only in the fast form, and only when all of them run on one die: workgroup
+        // (head, split) of the two-dimensional grid has index head + n_heads * split, a (kv head, split) key of the grouped
+        // grid lands on die (kv head + n_kv_heads * split) mod 8.
+        const bool fast_form = (a.head_size == 64 || a.head_size == 128) && a.kv_dim % 8 == 0;
+        static const bool on_die_env = [] { const char *e = getenv("SLAI_GQA_ON_DIE"); return !(e && e[0] == '0'); }();
+        const bool grouped_form = fast_form && on_die_env && a.kv_mul > 1 && a.n_heads % a.kv_mul == 0;
+        const uint32_t per_die = grouped_form ? a.n_heads / a.kv_mul : a.n_heads;
+        if (a.n_splits <= 1 || !fast_form || per_die % 8 != 0) a.combine_counters = nullptr;
+    }
     if (a.head_size > MAX_HS || a.head_size % 2 || a.head_size / 2 > ATT_THREADS || a.n_splits == 0 || a.n_splits > 64) return hipErrorInvalidValue;
     const uint32_t max_split_len = (a.seq_len + a.n_splits - 1) / a.n_splits;
     const bool fast = (a.head_size == 64 || a.head_size == 128) && a.kv_dim % 8 == 0;
@@ -318,7 +354,7 @@ hipError_t launch_attention(hipStream_t s, const AttnLaunch &a) {
     else attn_kernel<false><<<grid, ATT_THREADS, smem, s>>>(a, max_split_len);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    if (a.n_splits > 1) {
+    if (a.n_splits > 1 && !a.combine_counters) {
         attn_combine_kernel<<<a.n_heads, 128, 0, s>>>(a.scratch, a.out, a.head_size, a.n_splits);
         e = hipGetLastError();
     }
