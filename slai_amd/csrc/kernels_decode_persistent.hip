@@ -140,6 +140,7 @@ template <int T, int N, int LD> struct BufUnitLoader {
 
 // ---- waiting for data -------------------------------------------------------------------------------------------------
 constexpr uint64_t FLOW_WAIT_TICKS = 2u * 1000u * 1000u;      // 20 ms of the 100 MHz clock: what a reader waits before it gives up (a token takes about 1)
+constexpr uint32_t LDS_WAIT_ROUNDS = 1u << 19;                 // rounds of a wait on a word of LDS (about 0.1 us each): far beyond any phase
 
 struct Flow {
     uint32_t *abort_flag;     // device word: non-zero once any reader of the launch has given up
@@ -159,6 +160,30 @@ __device__ __forceinline__ void flow_backoff(Flow &f, uint64_t &deadline, uint32
     } else if ((rounds & 63u) == 0 && __hip_atomic_load(f.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
         f.dead = true;
     }
+}
+
+// A word of LDS that the waves of a workgroup count themselves in on (real LDS instructions: a flat access would return
+// behind the wave's outstanding weight requests).
+typedef __attribute__((address_space(3))) uint32_t LdsWord;
+__device__ __forceinline__ void lds_count_in(LdsWord *c) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");         // what the wave left in LDS comes first
+    if (lane_id() == 0) __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+// Waits until `need` waves have counted themselves in, and clears the word for its next use (which lies behind a
+// workgroup barrier).  Every wave that counts does so unconditionally after waits that are bounded themselves; the
+// rounds here are bounded all the same.
+__device__ __forceinline__ void lds_count_wait(LdsWord *c, uint32_t need, Flow &f) {
+    uint32_t rounds = 0;
+    while (__hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < need) {
+        __builtin_amdgcn_s_sleep(1);
+        if (++rounds > LDS_WAIT_ROUNDS) {
+            f.dead = true;
+            if (lane_id() == 0) __hip_atomic_store(f.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    if (lane_id() == 0) __hip_atomic_store(c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
 // Every wave of the device waits for its input at some point, most of them for many microseconds, and a request for a
@@ -432,7 +457,7 @@ __device__ __forceinline__ void request16(Unit &u, Req &r, const DevBuf &W, cons
 // element 16 * tile + i % 16 of it: asked for first, so that it is there when the reduction needs it.
 template <int T>
 __device__ __forceinline__ void mult16(const Unit &u, const plan::Tiles16 t, uint32_t ncb, uint32_t ngroups, Rsrc x, Rsrc res, bool res_flow, float &residual, char *lds,
-                                       float *partial, Flow &f, uint64_t *tr, const uint32_t wave_) {
+                                       float *partial, LdsWord *arrived, Flow &f, uint64_t *tr, const uint32_t wave_) {
     using F = Tiled<T>;
     const int lane = (int)lane_id();
     const uint32_t wave = fresh(wave_);
@@ -469,17 +494,24 @@ __device__ __forceinline__ void mult16(const Unit &u, const plan::Tiles16 t, uin
     }
     stamp(tr, 2, wave);
     if (lane < 16) partial[wave * 64 + lane] = v;
+    if (wave < ngroups * t.n) lds_count_in(arrived);
 }
-// After the barrier: thread i < 16 * t.n holds the dot product of row plan::tiles16_row(t, i).
-__device__ __forceinline__ float finish16(const plan::Tiles16 t, uint32_t ngroups, const float *partial, uint64_t *tr, uint32_t wave_) {
+// The rows of the tiles are added up by wave 0 (thread i < 16 * t.n: row plan::tiles16_row(t, i)) as soon as the waves that
+// multiplied have left their partial sums -- not behind the workgroup barrier: the other waves ask for the weights of
+// their next phase before they get there, and a compute unit takes its requests at the rate memory answers them (the
+// barrier came 1.3 us after the last product in the attention output projection, 2.3 us in the down projection).  The
+// caller hands the result on, asks for wave 0's own next weights, and only then joins the barrier of the phase.
+__device__ __forceinline__ float finish16(const plan::Tiles16 t, uint32_t ngroups, const float *partial, LdsWord *arrived, Flow &f, uint64_t *tr, uint32_t wave_) {
     const uint32_t wave = fresh(wave_);
-    lds_barrier();
-    stamp(tr, 3, wave);
-    const uint32_t tid = wave * 64u + lane_id();
     float o = 0.0f;
-    if (tid < 16u * t.n) {
-        const uint32_t k = tid >> 4, j = tid & 15u;
-        for (uint32_t w = 0; w < ngroups; ++w) o += partial[(k * ngroups + w) * 64 + j];
+    if (wave == 0 && t.n != 0) {
+        lds_count_wait(arrived, ngroups * t.n, f);
+        stamp(tr, 3, wave);
+        const uint32_t tid = lane_id();
+        if (tid < 16u * t.n) {
+            const uint32_t k = tid >> 4, j = tid & 15u;
+            for (uint32_t w = 0; w < ngroups; ++w) o += partial[(k * ngroups + w) * 64 + j];
+        }
     }
     return o;
 }
@@ -495,9 +527,9 @@ __device__ __forceinline__ void mult64_any(int type, const Unit &u, const Req &r
     }
 }
 __device__ __forceinline__ void mult16_any(int type, const Unit &u, const plan::Tiles16 t, uint32_t ncb, uint32_t ngroups, Rsrc x, Rsrc res, bool res_flow, float &residual,
-                                           char *lds, float *partial, Flow &f, uint64_t *tr, uint32_t wave) {
-    if (type == T_Q6_K) mult16<T_Q6_K>(u, t, ncb, ngroups, x, res, res_flow, residual, lds, partial, f, tr, wave);
-    else mult16<T_Q4_K>(u, t, ncb, ngroups, x, res, res_flow, residual, lds, partial, f, tr, wave);
+                                           char *lds, float *partial, LdsWord *arrived, Flow &f, uint64_t *tr, uint32_t wave) {
+    if (type == T_Q6_K) mult16<T_Q6_K>(u, t, ncb, ngroups, x, res, res_flow, residual, lds, partial, arrived, f, tr, wave);
+    else mult16<T_Q4_K>(u, t, ncb, ngroups, x, res, res_flow, residual, lds, partial, arrived, f, tr, wave);
 }
 
 // ---- the attention of one head (transformer.rs:342-350: RoPE, cache write, scores, softmax, weighted values) ------------
@@ -761,12 +793,12 @@ __device__ __forceinline__ void touch_far_rows(const plan::Shape &sh, uint32_t b
 // a q / k / v unit there (or nothing): the attention needs nearly all registers, and only a body of its own shows the
 // compiler that no unit requested ahead is ever alive across it.
 template <bool F16, bool ATTN, bool FAR>
-__device__ __forceinline__ void decode_token(const PersistentParams &p, float *smem, float (&rope_cs)[2][64], uint32_t (&layer_words)[2][sizeof(PersistentLayer) / 4],
+__device__ __forceinline__ void decode_token(const PersistentParams &p, float *smem, LdsWord *arrived, float (&rope_cs)[2][64], uint32_t (&layer_words)[2][sizeof(PersistentLayer) / 4],
                                              const uint32_t wave) {
     constexpr int LWORDS = sizeof(PersistentLayer) / 4;
     // Two sets of partial[2][16][64] | red[16], taken in turn by the phases of this workgroup: a wave that is done with a
-    // phase goes on to the next one (there is one barrier per phase, before its reduction) while wave 0 may still be
-    // reducing the one before, but it cannot get further ahead than that.
+    // phase goes on to the next one (there is one barrier per phase: before the reduction of a 64-row-unit phase, after
+    // that of a 16-row-tile phase) while wave 0 may still be reducing the one before, but it cannot get further ahead than that.
     float *const lds_sets = smem;
     char *const lds = reinterpret_cast<char *>(smem);
 #define PHASE_PARTIAL (lds_sets + plan::lds_set(phase & 1u) + plan::lds_partial())
@@ -889,10 +921,10 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
                         make_rsrc(p.flow + plan::flow_qkv(sh, l, 1), dim * 4u), make_rsrc(p.flow + plan::flow_qkv(sh, l, 0), dim * 4u), xb, PHASE_PARTIAL, f, tl, wave);
             stamp(tl, 3, wave);
             ++phase;
-            // (only now: the attention needs the registers; these workgroups have no tile of the output projection)
+            // (only now: the attention needs the registers; these workgroups take no tile of the output projection)
             ask_gate_up(lw);
         }
-        // ---- attention output projection into the residual (the workgroups that multiplied q / k / v) ------------------
+        // ---- attention output projection into the residual (two tiles in each workgroup that multiplied q or k; the others pass) ---
         if constexpr (!ATTN) {
             uint64_t *tp = tl ? tl + 4 : nullptr;
             float residual;
@@ -907,11 +939,12 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
                 const DevBuf kc = LAYER_BUF(lw, kcache), vc = LAYER_BUF(lw, vcache);
                 touch_far_rows(sh, b, pos, F16, ng_o, kc.rs, vc.rs, wave);
             }
-            mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, lds, PHASE_PARTIAL, f, tp, wave);
-            ask_gate_up(lw);                                        // (the waves without a part in the tiles: at once)
-            const float o = finish16(wo_t, ng_o, PHASE_PARTIAL, tp, wave);
+            mult16_any(unit_type, unit, wo_t, ncb, ng_o, xb, l == 0 ? make_rsrc(p.x, dim * 4u) : xa, l != 0, residual, lds, PHASE_PARTIAL, arrived, f, tp, wave);
+            const float o = finish16(wo_t, ng_o, PHASE_PARTIAL, arrived, f, tp, wave);               // (wave 0 only; the others go straight on)
             const uint32_t tid = wave * 64u + lane_id();
             if (tid < 16u * wo_t.n) flow_put(xm, plan::tiles16_row(wo_t, tid), residual + o);     // transformer.rs:352-355
+            ask_gate_up(lw);                                        // (the waves without a part in the tiles: at once)
+            lds_barrier();
             ++phase;
         }
         // ---- RMSNorm + gate / up + SiLU ---------------------------------------------------------------------------------
@@ -932,11 +965,12 @@ __device__ __forceinline__ void decode_token(const PersistentParams &p, float *s
             float residual;
             stamp(tp, 0, wave);
             residual = 0.0f;
-            mult16_any(unit_type, unit, down_t, ncb_h, ng_d, hb, xm, true, residual, lds, PHASE_PARTIAL, f, tp, wave);
-            ask_next(layer_words[(l + 1) & 1u], last);
-            const float o = finish16(down_t, ng_d, PHASE_PARTIAL, tp, wave);
+            mult16_any(unit_type, unit, down_t, ncb_h, ng_d, hb, xm, true, residual, lds, PHASE_PARTIAL, arrived, f, tp, wave);
+            const float o = finish16(down_t, ng_d, PHASE_PARTIAL, arrived, f, tp, wave);
             const uint32_t tid = wave * 64u + lane_id();
             if (tid < 16u * down_t.n) flow_put(xnext, plan::tiles16_row(down_t, tid), residual + o);    // transformer.rs:362-365
+            ask_next(layer_words[(l + 1) & 1u], last);
+            lds_barrier();
             ++phase;
         }
     }
@@ -973,17 +1007,20 @@ __global__ void __launch_bounds__(PNT) llama_decode_persistent_kernel(const Pers
     constexpr int LWORDS = sizeof(PersistentLayer) / 4;
     static_assert(LWORDS <= 64 && sizeof(PersistentLayer) == 14 * sizeof(ResidentBuf), "one thread per word; fourteen entries");
     __shared__ uint32_t layer_words[2][LWORDS];
+    __shared__ uint32_t arrived_word;                              // the waves of a 16-row-tile phase count themselves in here (finish16)
     touch_kernel_arguments<sizeof(PersistentParams)>();
     // A launch after one in which a reader gave up does nothing: the host has not looked yet (it queues many tokens), and
     // every further token would only wait out the same time limits.
     if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
     if (threadIdx.x < LWORDS) layer_words[0][threadIdx.x] = reinterpret_cast<const uint32_t *>(p.layers)[threadIdx.x];
+    if (threadIdx.x == 0) arrived_word = 0u;
     if (threadIdx.x < plan::MQ_ZERO_BYTES / 4) reinterpret_cast<uint32_t *>(smem)[plan::lds_mq_zero() / 4 + threadIdx.x] = 0u;   // the zeros of mfma_q4k.h
     __syncthreads();
     const plan::Shape sh = shape_of(p);
     const uint32_t wave = uniform_word(threadIdx.x >> 6);
-    if (plan::is_attention_workgroup(sh, blockIdx.x)) decode_token<F16, true, false>(p, smem, rope_cs, layer_words, wave);
-    else decode_token<F16, false, FAR>(p, smem, rope_cs, layer_words, wave);
+    LdsWord *arrived = (LdsWord *)&arrived_word;
+    if (plan::is_attention_workgroup(sh, blockIdx.x)) decode_token<F16, true, false>(p, smem, arrived, rope_cs, layer_words, wave);
+    else decode_token<F16, false, FAR>(p, smem, arrived, rope_cs, layer_words, wave);
 }
 
 #undef PHASE_PARTIAL

@@ -159,17 +159,19 @@ SLAI_HD uint32_t gu_units(const Shape &s) { return (s.hidden + s.gu_rows - 1) / 
 SLAI_HD RowUnit gu_unit(const Shape &s, uint32_t b) { return run_unit(0u, b * s.gu_rows, umin(s.gu_rows, s.hidden - b * s.gu_rows)); }
 
 // The two projections into the residual, in 16-row tiles (dim / 16 of them = the grid).  Down projection: workgroup b
-// takes tile b.  Attention output projection: the workgroups that run a head's attention have just finished when it
-// starts and hold none of its weights, so they take no tile; the q / k / v workgroup b takes tile b, and the one with a
-// head's last q unit also the tile 7 * n_heads + head, side by side on other waves.
+// takes tile b.  Attention output projection: the workgroups of a head's q and k units take two tiles each, side by side
+// on other waves -- their own, b, and the one of a workgroup that takes none: the head's three v units (which end last in
+// the phase before and have asked for all their gate / up weights by then: their polls for the attention's result would
+// return behind those) and the head's attention workgroup (which has just finished and holds no weights).
 struct Tiles16 { uint32_t n, tile0, tile1; };      // (two named fields: an indexed pair would live in memory on the device)
 SLAI_HD uint32_t tiles16_tile(const Tiles16 &t, uint32_t k) { return k == 0 ? t.tile0 : t.tile1; }
 SLAI_HD uint32_t proj_tiles(const Shape &s) { return s.dim / 16; }
 SLAI_HD Tiles16 down_tiles(const Shape &, uint32_t b) { return Tiles16{1u, b, b}; }
+SLAI_HD bool takes_wo_tiles(const Shape &s, uint32_t b) { return b < qkv_workgroups(s) && (b >> 3) % s.qkv_units >= s.qkv_units - 4; }
 SLAI_HD Tiles16 wo_tiles(const Shape &s, uint32_t b) {
-    if (b >= qkv_workgroups(s)) return Tiles16{0u, 0u, 0u};
-    if ((b >> 3) % s.qkv_units == s.qkv_units - 1) return Tiles16{2u, b, qkv_workgroups(s) + qkv_head(s, b)};
-    return Tiles16{1u, b, b};
+    if (!takes_wo_tiles(s, b)) return Tiles16{0u, 0u, 0u};
+    const uint32_t t = (b >> 3) % s.qkv_units, nv = s.qkv_units - 4, j = t - nv;       // j: which of the head's four q / k units
+    return Tiles16{2u, b, j < nv ? b - 8u * (t - j) : qkv_workgroups(s) + qkv_head(s, b)};    // + v unit j's tile, or the attention's
 }
 // the row thread i < 16 * t.n of the workgroup finishes
 SLAI_HD uint32_t tiles16_row(const Tiles16 &t, uint32_t i) { return 16u * tiles16_tile(t, (i >> 4) & 1u) + (i & 15u); }

@@ -271,7 +271,7 @@ unsigned long long rb_audit(uint32_t dim, uint32_t hidden, uint32_t n_heads, uin
                 a.touch(counters, (uint64_t)handoff_heads * 32 * 4, 4, "abort flag", b, 0, 0, l);
                 {
                     const plan::Tiles16 wt = plan::wo_tiles(s, b), dt = plan::down_tiles(s, b);
-                    if (plan::is_attention_workgroup(s, b) != (wt.n == 0)) a.fail("exactly the attention workgroups take no tile of the output projection");
+if (plan::takes_wo_tiles(s, b) != (wt.n == 2) || (wt.n != 0 && wt.n != 2)) a.fail("the workgroups of the q and k units take two tiles of the output projection each, the others none");
                     walk_tile16(a, wo, to, wt, ncb, ng_o, xb, dim, l == 0 ? xemb : xa, xm, rows_o, b, l);
                     walk_tile16(a, wd, td, dt, ncb_h, ng_d, hb, hidden, xm, xnext, rows_d, b, l);
                 }
