@@ -140,7 +140,7 @@ template <int T, int N, int LD> struct BufUnitLoader {
 
 // ---- waiting for data -------------------------------------------------------------------------------------------------
 constexpr uint64_t FLOW_WAIT_TICKS = 2u * 1000u * 1000u;      // 20 ms of the 100 MHz clock: what a reader waits before it gives up (a token takes about 1)
-constexpr uint32_t LDS_WAIT_ROUNDS = 1u << 19;                 // rounds of a wait on a word of LDS (about 0.1 us each): far beyond any phase
+constexpr uint32_t LDS_WAIT_ROUNDS = 1u << 22;                 // rounds of a wait on a word of LDS (at least 60 ns each: a quarter of a second, beyond every bounded wait of the waves it waits for)
 
 struct Flow {
     uint32_t *abort_flag;     // device word: non-zero once any reader of the launch has given up
