@@ -244,7 +244,8 @@ __device__ __forceinline__ void flow_take4(Rsrc x, uint32_t piece0, uint32_t n, 
 // ---- weights on their way ---------------------------------------------------------------------------------------------------
 // A phase's multiply cannot start before its input exists, but its weights do not depend on anything: each wave asks
 // for the unit of its NEXT phase as soon as the registers of the current one are free (right after its dot product,
-// before the partial sums are reduced and handed over), so the weights travel while the hand-off is waited for.
+// before the partial sums are reduced and handed over -- except wave 0 of a 16-row-tile phase, which adds up and hands the
+// rows on first: finish16), so the weights travel while the hand-off is waited for.
 struct Unit {                 // the 16-byte pieces a wave requested ahead (which ones depends on the block format)
     U4 a[13], b[9];           // first matrix / second matrix of a gated pair
     uint16_t ta;              // 2-byte tail of the first matrix (Q6_K)
