@@ -138,6 +138,19 @@ def test_persistent_matches_launch_per_step_form():
     print("ms/token: per-step launches %.3f, one launch %.3f" % (out[False][2], out[True][2]))
 
 
+def test_persistent_width_3072_vs_oracle():
+    """dim 3072 (24 heads), FFN 12288, 2 layers: twelve super-blocks per row (twelve of the sixteen waves multiply a
+    64-row unit, three waves a 16-row tile of the output projection, twelve one of the down projection) and gate / up units
+    of 64 rows -- the decomposition between the test shapes above and the headline's."""
+    b = backend_with(True)
+    try:
+        data = gw.llama_gguf(dim=3072, hidden_dim=12288, n_layers=2, n_heads=24, n_kv_heads=24, vocab=1000, seq_len=128, wtype=12, v_type=14,
+                             out_type=14, embd_type=12, seed=43, std=0.03, norm_random=True)
+        check_llama(b, data, [5, 999, 77, 3], 24, kv_f16=True, check_logit_steps=8, decode_form=1)
+    finally:
+        b.close()
+
+
 def test_persistent_7b_width_two_layers_vs_oracle():
     """The headline shapes (dim 4096, hidden 11008, 32 heads, vocab 32000) at depth 2 against the oracle."""
     b = backend_with(True)

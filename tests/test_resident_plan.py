@@ -41,6 +41,7 @@ SHAPES = {
     "7B width, 2 layers": dict(dim=4096, hidden=11008, n_heads=32, n_layers=2, vocab=32000, seq_len=128),
     "config 4": dict(dim=4096, hidden=11008, n_heads=32, n_layers=32, vocab=32000, seq_len=512),
     "7B width, context 4096, f32 cache": dict(dim=4096, hidden=11008, n_heads=32, n_layers=2, vocab=32000, seq_len=4096, kv_bytes=4),
+    "dim 3072": dict(dim=3072, hidden=12288, n_heads=24, n_layers=2, vocab=1000, seq_len=128),
     "NeoX rotary pairs": dict(dim=2048, hidden=5632, n_heads=16, n_layers=2, vocab=4096, seq_len=300, neox=1),
     "wide FFN (12 column groups in the down projection)": dict(dim=3072, hidden=12288, n_heads=24, n_layers=2, vocab=1000, seq_len=64, types=(Q5_K, Q4_K, Q4_K, Q6_K, Q4_K, Q4_K, Q4_K)),
 }
