@@ -692,7 +692,6 @@ int slai_llama2::chunk_reserve(uint32_t rows) {
 int slai_llama2::enqueue_chunk(uint32_t pos0, uint32_t n, const int *tokens_dev) {
     PromptChunkState &pc = chunk;
     if (n == 0 || n > pc.rows || pos0 + n > config.seq_len) return set_error(ctx, SLAI_E_ARG, "prompt chunk out of range");
-    Llama2State &s = state;
     const uint32_t dim = config.dim, kvd = kv_dim(), hid = config.hidden_dim, xws = dim + dim / 16;
     float *x = (float *)pc.x.buf->dptr, *xw = (float *)pc.xw.buf->dptr, *xb = (float *)pc.xb.buf->dptr, *q = (float *)pc.q.buf->dptr;
     float *k = (float *)pc.k.buf->dptr, *v = (float *)pc.v.buf->dptr, *hb = (float *)pc.hb.buf->dptr;
