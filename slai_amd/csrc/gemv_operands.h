@@ -132,7 +132,7 @@ template <int T, int N, int LD> struct UnitLoader {
     uint16_t *t[N];
     template <int P> __device__ __forceinline__ void piece() const {
 #pragma unroll
-        for (int n = 0; n < N; ++n) d[n]->p[P] = ld128(unit[n] + (size_t)P * 1024);
+        for (int n = 0; n < N; ++n) d[n]->p[P] = ld128_stream(unit[n] + (size_t)P * 1024);
     }
     __device__ __forceinline__ void tail() const {
 #pragma unroll

@@ -110,6 +110,17 @@ SLAI_HD U4 ld128(const uint8_t *p) {
     U4 v; memcpy(&v, p, 16); return v;
 #endif
 }
+// The same for weights that a kernel reads exactly once: the non-temporal hint keeps them from displacing what the caches
+// are needed for (the vectors handed from launch to launch, or from workgroup to workgroup inside one).
+SLAI_HD U4 ld128_stream(const uint8_t *p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef uint32_t words4 __attribute__((ext_vector_type(4)));
+    const words4 v = __builtin_nontemporal_load(reinterpret_cast<const words4 *>(p));
+    return U4{v.x, v.y, v.z, v.w};
+#else
+    return ld128(p);
+#endif
+}
 SLAI_HD uint32_t byte_of(const U4 &v, int k) {  // byte k (0..15) of a 128-bit value
     uint32_t w = (k < 8) ? ((k < 4) ? v.x : v.y) : ((k < 12) ? v.z : v.w);
     return (w >> (8 * (k & 3))) & 0xffu;
