@@ -176,7 +176,7 @@ template <> struct Deq<T_Q4_0> {          // BlockQ4_0, quantization.rs:47-69: v
 template <int T> __device__ __forceinline__ void load_unit(const uint8_t *unit, int lane, typename Tiled<T>::Data &d, uint16_t &tail) {
     using F = Tiled<T>;
 #pragma unroll
-    for (int P = 0; P < F::PT; ++P) d.p[P] = ld128(unit + (size_t)P * 1024 + lane * 16);
+    for (int P = 0; P < F::PT; ++P) d.p[P] = ld128_stream(unit + (size_t)P * 1024 + lane * 16);
     tail = F::TAIL ? ld16(unit + (size_t)F::PT * 1024 + lane * 2) : (uint16_t)0;
 }
 
