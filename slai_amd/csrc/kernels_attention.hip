@@ -190,7 +190,9 @@ __global__ void __launch_bounds__(NT) attn_fast_kernel(AttnLaunch a, uint32_t ma
         h = (key % n_kv) * a.kv_mul + j;
         split = key / n_kv;
     }
-    attn_fast_body<F16, NT, HS, SINGLE, false>(a, h, split, threadIdx.x, []() {});
+    // (the split form on a model without grouped queries reads every cached row exactly once: non-temporal requests)
+    if (!SINGLE && F16 && a.kv_mul == 1) attn_fast_body<F16, NT, HS, SINGLE, false, 4, false, true>(a, h, split, threadIdx.x, []() {});
+    else attn_fast_body<F16, NT, HS, SINGLE, false>(a, h, split, threadIdx.x, []() {});
     if constexpr (!SINGLE) {
         // The last of a head's splits merges them: every workgroup waits until its partial result is in the die's L2
         // (all splits of the head run on this die: the launcher has checked), then counts itself in with an atomic that
