@@ -351,7 +351,7 @@ uint32_t slai_llama2_prefill_fp32_repeats(const slai_llama2 *m);
  * four to five per layer), 1 = the whole layer stack and the output matrix in one resident launch per token (widths of
  * 1024 .. 4096 in steps of 1024, as many cache heads as query heads of size 128, Q4_K / Q5_K / Q6_K mixes, gate / up in
  * Q4_K; a context created with SLAI_PERSISTENT=0 in the environment never takes it).  The form is chosen per token: a model
- * of form 1 takes the resident launch at positions below SLAI_RESIDENT_MAX_POS (environment, default 2176) and one launch
+ * of form 1 takes the resident launch at positions below SLAI_RESIDENT_MAX_POS (environment, default 2048) and one launch
  * per step beyond, with the same caches and loop state.  Results are the same to within summation order. */
 int slai_llama2_decode_form(const slai_llama2 *m);
 /* Measurement aid without a reference counterpart (profilers see the resident launch as one kernel): runs one token at

@@ -89,7 +89,7 @@ struct slai_ctx {
     hipEvent_t timer0 = nullptr, timer1 = nullptr;
     // the one-launch-per-token form of the Llama-2 layer stack where a model's shapes allow it (SLAI_PERSISTENT=0 switches it off)
     bool persistent = true;
-    uint32_t resident_max_pos = 2176;   // tokens at positions below this take the resident launch (where the model has one): SLAI_RESIDENT_MAX_POS
+    uint32_t resident_max_pos = 2048;   // tokens at positions below this take the resident launch (where the model has one): SLAI_RESIDENT_MAX_POS
     // When set, every launch of a decode step is followed by an event recorded under the step's name
     // (slai_llama2_time_steps); null otherwise.
     std::vector<std::pair<const char *, hipEvent_t>> *step_marks = nullptr;

@@ -91,7 +91,7 @@ SLAI_EXPORT int slai_ctx_create(int device, slai_ctx **out) {
     ctx->rowtile_gemv = env_int("SLAI_ROWTILE", 1) != 0;
     ctx->fuse_qkv_attention = env_int("SLAI_FUSE_QKV_ATTN", 1) != 0;
     ctx->persistent = env_int("SLAI_PERSISTENT", 1) != 0;
-    ctx->resident_max_pos = (uint32_t)std::max(0, env_int("SLAI_RESIDENT_MAX_POS", 2176));
+    ctx->resident_max_pos = (uint32_t)std::max(0, env_int("SLAI_RESIDENT_MAX_POS", 2048));
     *out = ctx;
     return SLAI_OK;
 }
